@@ -1,0 +1,154 @@
+/*
+ * gptq_hip.h -- C ABI of the MI355X (gfx950) GPTQ solve and packed-int4 matmul.
+ *
+ * This is the drop-in boundary: the entry points below are what a binding of the
+ * reference's per-layer solve (jax_gptq/gptq.py) and of its quantized-matmul
+ * custom call (jax_gptq/op.py:46-63, jt.triton_call) would bind.  Each entry
+ * names the reference code it replaces (paths relative to the reference).
+ *
+ * Conventions (all entry points):
+ *   - `stream` is a hipStream_t passed as void*; NULL means the default stream.
+ *   - every pointer except the host tables named below is a DEVICE pointer;
+ *   - matrices are row-major; W is [K, N] with K = input features (contraction
+ *     axis 0) and N = output channels, exactly as in gptq.py:118,136-147;
+ *   - calls only enqueue work on `stream`: no host synchronisation, no device
+ *     allocation.  Scratch memory is passed in by the caller (`ws`, `ws_bytes`);
+ *     the matching `*_workspace_bytes` query gives the required size;
+ *   - return value 0 means success, otherwise a GPTQ_HIP_E* code; nothing throws.
+ *   - thread-safe; no mutable global state.
+ */
+#ifndef GPTQ_HIP_H_
+#define GPTQ_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GPTQ_HIP_ABI_VERSION 1
+
+/* element types of float operands */
+enum { GPTQ_HIP_F32 = 0, GPTQ_HIP_F16 = 1, GPTQ_HIP_BF16 = 2 };
+
+/* status codes */
+enum {
+  GPTQ_HIP_OK = 0,
+  GPTQ_HIP_EINVAL = 1,      /* bad shape / null pointer / unsupported block size */
+  GPTQ_HIP_EDTYPE = 2,      /* unsupported element type */
+  GPTQ_HIP_EWORKSPACE = 3,  /* workspace too small */
+  GPTQ_HIP_ELAUNCH = 4      /* the HIP runtime refused a launch */
+};
+
+int gptq_hip_abi_version(void);
+const char *gptq_hip_error_string(int code);
+
+/* ---- per-column quantisation parameters -------------------------------------
+ * Replaces get_quantize_params / get_col_quantize_params (gptq.py:105-118).
+ * W [K, N] (element type w_dtype, row stride ldw) -> scale[N], zero[N] (fp32).
+ * maxq = 2^bits - 1.  ws: gptq_hip_col_params_workspace_bytes(K, N). */
+size_t gptq_hip_col_params_workspace_bytes(int64_t K, int64_t N);
+int gptq_hip_col_params(void *stream, const void *W, int w_dtype, int64_t K, int64_t N,
+                        int64_t ldw, int bits, float *scale, float *zero, void *ws,
+                        size_t ws_bytes);
+
+/* ---- Hessian ------------------------------------------------------------------
+ * Replaces _accumulate_H_step / accumulate_H (gptq.py:57-103).
+ * gptq_hip_hessian_accumulate adds sum_b X_b^T X_b to the UPPER triangle (128x128
+ * tile granularity) of H [K, K] fp32.  x_ptrs / x_rows are HOST arrays of
+ * n_batches device pointers / row counts; batch b is [x_rows[b], K] row-major,
+ * contiguous.  The running mean of the reference cancels algebraically
+ * (H = sum X^T X / n), so none is kept.
+ * gptq_hip_hessian_finalize multiplies by 1/n_samples and mirrors the upper
+ * triangle into the lower one, giving the full symmetric H the reference returns. */
+int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const int64_t *x_rows,
+                                int n_batches, int x_dtype, int64_t K, float *H);
+int gptq_hip_hessian_finalize(void *stream, float *H, int64_t K, double n_samples);
+
+/* ---- dead features, damping, Cholesky factor of the inverse -----------------------
+ * Replaces _damp_and_invert + _cholesky_inv (gptq.py:155-168, 44-48).
+ * H [K, K] fp32 full symmetric (read; its diagonal is rewritten with the dead-feature
+ * fix and the damping, as the reference's donated buffer is); W [K, N] fp32 (rows
+ * of dead features zeroed in place; may be NULL with N = 0); L [K, K] fp32 out:
+ * lower triangular, L L^T = (H + damping*mean(diag H) I)^-1, upper part zero.
+ * status (device int32[2]): status[0] = 0, or 1 + index of the first 128-block whose
+ * pivot was not positive (L then holds NaN, as the reference's does, gptq.py:166);
+ * status[1] = number of dead features.  fix_dead = 0 skips the dead-feature fix (with
+ * damping = 0 the call is then exactly _cholesky_inv, gptq.py:44-48). */
+size_t gptq_hip_damp_invert_workspace_bytes(int64_t K);
+int gptq_hip_damp_invert(void *stream, float *H, float *W, int64_t K, int64_t N, int64_t ldw,
+                         float damping, int fix_dead, float *L, int32_t *status, void *ws,
+                         size_t ws_bytes);
+
+/* ---- blocked column loop ------------------------------------------------------------
+ * Replaces the loop of gptq() with _process_block and the lazy update
+ * (gptq.py:199-208, 130-153).  W [K, N] fp32 is consumed (overwritten).  L [K, K]
+ * lower factor from gptq_hip_damp_invert.  Outputs (either may be NULL):
+ *   Q      [K, N] dequantised values scale*(q - zero) in element type q_dtype
+ *          (what gptq() returns, gptq.py:208,212);
+ *   codes  [K, N] uint8 integer codes q.
+ * block_size must divide K and be <= 128 (the reference's default is 128).
+ * ws: gptq_hip_solve_workspace_bytes(K, N, block_size). */
+size_t gptq_hip_solve_workspace_bytes(int64_t K, int64_t N, int block_size);
+int gptq_hip_solve(void *stream, float *W, int64_t K, int64_t N, const float *L,
+                   const float *scale, const float *zero, int maxq, int block_size, void *Q,
+                   int q_dtype, uint8_t *codes, void *ws, size_t ws_bytes);
+
+/* One block of the loop: replaces _process_block (gptq.py:130-153).  Wblock points at
+ * the first of the block's block_size rows of W [*, N] (rows of the block are used as
+ * scratch and overwritten); Lblock points at L[start][start] (row stride ldl).  Outputs:
+ * Qblock / codes_block [block_size, N] (either may be NULL) and errors [block_size, N]
+ * fp32, the (w - q) / L_ii rows that the lazy update consumes. */
+int gptq_hip_process_block(void *stream, float *Wblock, int64_t N, const float *Lblock,
+                           int64_t ldl, int block_size, const float *scale, const float *zero,
+                           int maxq, void *Qblock, int q_dtype, uint8_t *codes_block,
+                           float *errors);
+
+/* ---- activation order ---------------------------------------------------------------
+ * Replaces the gathers of _permute / _unpermute (gptq.py:170-180); the argsort itself
+ * stays with the caller.  out[i, :] = in[perm[i], :] for rows; the symmetric form
+ * gathers rows and columns: out[i, j] = in[perm[i], perm[j]].  perm is device int64[K]. */
+int gptq_hip_gather_rows(void *stream, const void *in, void *out, int elem_bytes, int64_t K,
+                         int64_t N, const int64_t *perm);
+int gptq_hip_gather_sym(void *stream, const float *in, float *out, int64_t K, const int64_t *perm);
+
+/* ---- int4 codec -----------------------------------------------------------------------
+ * A tensor is viewed as [outer, axis_len, inner] and packed along the middle axis:
+ * byte[o, j, i] = c[o, 2j, i] | c[o, 2j+1, i] << 4   (gptq.py:237-249, 265-292).
+ * axis_len must be even for pack.  unpack is the inverse (gptq.py:251-263).
+ * codes are taken modulo 256 from elements of code_bytes bytes (1 = uint8, 4 = int32,
+ * 8 = int64). */
+int gptq_hip_pack_int4(void *stream, const void *codes, int code_bytes, int64_t outer,
+                       int64_t axis_len, int64_t inner, uint8_t *packed);
+int gptq_hip_unpack_int4(void *stream, const uint8_t *packed, int64_t outer,
+                         int64_t packed_axis_len, int64_t inner, uint8_t *codes);
+/* pack_matrix (gptq.py:214-228): c = uint8(rint(Q/scale + zero)) then pack along the
+ * middle axis; scale/zero are fp32 and indexed [o, i] (the contraction axis removed). */
+int gptq_hip_quantize_pack(void *stream, const void *Q, int q_dtype, int64_t outer,
+                           int64_t axis_len, int64_t inner, const float *scale,
+                           const float *zero, uint8_t *packed);
+/* unpack_matrix (gptq.py:230-235): out = (code - zero) * scale in element type
+ * zs_dtype (that of zero/scale, which is also the output type, gptq.py:20-22). */
+int gptq_hip_dequant(void *stream, const uint8_t *packed, int64_t outer,
+                     int64_t packed_axis_len, int64_t inner, const void *zero,
+                     const void *scale, int zs_dtype, void *out);
+
+/* ---- packed-int4 matmul ------------------------------------------------------------------
+ * Replaces the jt.triton_call custom call of _quantized_matmul (op.py:19-69) and the two
+ * Triton kernels behind it (kernel.py:17-127, 141-253).
+ * packed [R, C] uint8 holds W [2R, C] (contraction axis 0).  zero/scale [C] of type
+ * zs_dtype.  x [M, Kx] and out of type x_dtype.
+ *   transpose_b = 0: Kx = 2R, out [M, C]  = x @ ((code - zero) * scale)
+ *   transpose_b = 1: Kx = C,  out [M, 2R] = x @ ((code - zero) * scale)^T
+ * fp32 accumulation; the result is rounded to fp16 and then converted to x_dtype, as
+ * op.py:43,66-68 does.  ws: gptq_hip_qmatmul_workspace_bytes(M, R, C, transpose_b). */
+size_t gptq_hip_qmatmul_workspace_bytes(int64_t M, int64_t R, int64_t C, int transpose_b);
+int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
+                     int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype,
+                     int transpose_b, void *out, void *ws, size_t ws_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GPTQ_HIP_H_ */

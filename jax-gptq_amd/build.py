@@ -1,0 +1,70 @@
+"""Builds libgptq_hip.so (gfx950 only) next to the Python package.
+
+    python jax-gptq_amd/build.py [--force]
+
+hipcc cross-compiles without a GPU; the .so is kept in-tree (git-ignored).
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OUT_DIR = os.path.join(HERE, "jax_gptq_amd")
+LIB = os.path.join(OUT_DIR, "libgptq_hip.so")
+SOURCES = ["api.hip", "codec.hip", "gemm_f32.hip", "hessian.hip", "cholinv.hip", "solve.hip",
+           "qmatmul.hip"]
+FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-Wno-unused-result"]
+
+
+def _hipcc():
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if cand and (os.path.sep not in cand or os.path.exists(cand)):
+            return cand
+    return "hipcc"
+
+
+def needs_build():
+    if not os.path.exists(LIB):
+        return True
+    t = os.path.getmtime(LIB)
+    deps = [os.path.join(CSRC, f) for f in os.listdir(CSRC)]
+    deps.append(os.path.join(HERE, "..", "include", "gptq_hip.h"))
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def build(force=False, verbose=True):
+    if not force and not needs_build():
+        return LIB
+    obj_dir = os.path.join(HERE, "build")
+    os.makedirs(obj_dir, exist_ok=True)
+    hipcc = _hipcc()
+    procs = []
+    objs = []
+    for src in SOURCES:
+        obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
+        objs.append(obj)
+        cmd = [hipcc, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
+    failed = False
+    for src, p in procs:
+        out = p.communicate()[0].decode()
+        out = "\n".join(l for l in out.splitlines() if "packed-fp32-ops" not in l)
+        if p.returncode != 0:
+            failed = True
+            sys.stderr.write(f"[build] {src} FAILED\n{out}\n")
+        elif verbose and out.strip():
+            sys.stderr.write(f"[build] {src}:\n{out}\n")
+    if failed:
+        raise RuntimeError("hipcc failed")
+    cmd = [hipcc, "-shared", "--offload-arch=gfx950", "-fPIC", *objs, "-o", LIB]
+    subprocess.check_call(cmd)
+    if verbose:
+        print(f"[build] wrote {LIB}")
+    return LIB
+
+
+if __name__ == "__main__":
+    build(force="--force" in sys.argv)

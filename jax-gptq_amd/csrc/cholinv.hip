@@ -1,0 +1,318 @@
+// Dead-feature fix, damping and the lower Cholesky factor L of the inverse Hessian,
+// L L^T = H^-1, on one device.
+//
+// The reference obtains L in three LAPACK steps (factor, solve against I, factor again,
+// about 8/3 K^3 flop).  Here L is obtained in two (about 2/3 K^3 flop):
+//   1. H = M^T M with M lower triangular ("reverse" Cholesky, processed from the last
+//      128-block upwards so that every trailing update is an X^T X form);
+//   2. L = M^-1, by pairwise merging of inverted diagonal blocks:
+//      inv([[A,0],[C,B]]) = [[A^-1,0],[-B^-1 C A^-1, B^-1]].
+// H^-1 = M^-1 M^-T = L L^T with L lower triangular and a positive diagonal, which is the
+// unique Cholesky factor the reference computes.
+//
+// All O(K^3) work runs on the fp32 MFMA GEMM; only the 128x128 diagonal blocks are
+// factorised and inverted inside one workgroup, in LDS.
+#include "common.h"
+#include "gemm_f32.h"
+
+namespace {
+
+constexpr int NB = 128;
+
+// ---------------------------------------------------------------- diag / damping prep
+// One workgroup.  dead_i = (H_ii == 0) -> H_ii = 1; mean over the fixed diagonal;
+// H_ii += damping * mean.  Writes dead flags and status[1] = number of dead features.
+__global__ __launch_bounds__(1024) void damp_diag_kernel(float *H, int64_t K, float damping,
+                                                         int fix_dead, uint8_t *dead,
+                                                         int32_t *status) {
+#pragma clang fp contract(off)
+  __shared__ float ssum[1024];
+  __shared__ int scnt[1024];
+  const int tid = threadIdx.x;
+  float sum = 0.f;
+  int cnt = 0;
+  for (int64_t i = tid; i < K; i += 1024) {
+    float d = H[i * K + i];
+    const bool is_dead = fix_dead && (d == 0.f);
+    if (is_dead) { d = 1.f; ++cnt; }
+    dead[i] = is_dead ? 1 : 0;
+    sum += d;
+  }
+  ssum[tid] = sum;
+  scnt[tid] = cnt;
+  __syncthreads();
+  for (int s = 512; s > 0; s >>= 1) {
+    if (tid < s) { ssum[tid] += ssum[tid + s]; scnt[tid] += scnt[tid + s]; }
+    __syncthreads();
+  }
+  const float add = (ssum[0] / (float)K) * damping;
+  for (int64_t i = tid; i < K; i += 1024) {
+    float d = H[i * K + i];
+    if (dead[i]) d = 1.f;
+    H[i * K + i] = d + add;
+  }
+  if (tid == 0) { status[0] = 0; status[1] = scnt[0]; }
+}
+
+__global__ __launch_bounds__(256) void zero_dead_rows_kernel(float *W, int64_t N, int64_t ldw,
+                                                             const uint8_t *dead) {
+  const int64_t row = blockIdx.y;
+  if (!dead[row]) return;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < N; c += (int64_t)gridDim.x * 256)
+    W[row * ldw + c] = 0.f;
+}
+
+// A (Kp x Kp, padded with the identity) <- H ; Minv <- 0
+__global__ __launch_bounds__(256) void pad_copy_kernel(const float *H, int64_t K, float *A,
+                                                       float *Minv, int64_t Kp) {
+  const int64_t row = blockIdx.y;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < Kp; c += (int64_t)gridDim.x * 256) {
+    float v;
+    if (row < K && c < K) v = H[row * K + c];
+    else v = (row == c) ? 1.f : 0.f;
+    A[row * Kp + c] = v;
+    Minv[row * Kp + c] = 0.f;
+  }
+}
+
+// L (K x K, ld K) <- lower(Minv[0:K, 0:K]), upper part zero
+__global__ __launch_bounds__(256) void copy_out_kernel(const float *Minv, int64_t Kp, float *L,
+                                                       int64_t K) {
+  const int64_t row = blockIdx.y;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < K; c += (int64_t)gridDim.x * 256)
+    L[row * K + c] = (c <= row) ? Minv[row * Kp + c] : 0.f;
+}
+
+// ---------------------------------------------------------------- 128x128 diagonal block
+// D = A[b,b] (its lower triangle is read).  Finds M_bb lower with M_bb^T M_bb = D by a
+// standard Cholesky of the index-reversed block: G G^T = J D J, M_bb = J G^T J.  Writes
+// M_bb over A[b,b] (upper part zeroed) and M_bb^-1 = J G^-T J into Minv[b,b].
+constexpr int GS = NB + 1;  // LDS row stride
+
+__global__ __launch_bounds__(256) void chol_diag_kernel(float *A, float *Minv, int64_t ld, int b,
+                                                        int32_t *status) {
+  extern __shared__ float smem[];
+  float *G = smem;             // [NB][GS]   factor, lower
+  float *X = smem + NB * GS;   // [NB][GS]   inverse of the factor, lower
+  __shared__ float colbuf[NB];
+  __shared__ int bad;
+  const int tid = threadIdx.x;
+  float *D = A + (int64_t)b * NB * ld + (int64_t)b * NB;
+  float *Dinv = Minv + (int64_t)b * NB * ld + (int64_t)b * NB;
+  if (tid == 0) bad = 0;
+
+  // G[r][c] (r >= c) = D[127-c][127-r]  (lower element of D, since 127-c >= 127-r)
+  for (int idx = tid; idx < NB * NB; idx += 256) {
+    const int i = idx / NB, j = idx % NB;  // element D[i][j], coalesced along j
+    if (i >= j) G[(NB - 1 - j) * GS + (NB - 1 - i)] = D[(int64_t)i * ld + j];
+    X[i * GS + j] = 0.f;
+  }
+  __syncthreads();
+
+  // right-looking Cholesky, 2 barriers per column
+  const int tr = tid >> 4, tc = tid & 15;
+  for (int k = 0; k < NB; ++k) {
+    const float piv = G[k * GS + k];
+    if (tid == 0 && !(piv > 0.f)) bad = 1;
+    const float root = sqrtf(piv);
+    const float rinv = 1.f / root;
+    if (tid < NB && tid > k) colbuf[tid] = G[tid * GS + k] * rinv;
+    __syncthreads();
+    if (tid < NB) {
+      if (tid > k) G[tid * GS + k] = colbuf[tid];
+      else if (tid == k) G[k * GS + k] = root;
+    }
+    for (int r = k + 1 + tr; r < NB; r += 16) {
+      const float lr = colbuf[r];
+      for (int c = k + 1 + tc; c <= r; c += 16) G[r * GS + c] -= lr * colbuf[c];
+    }
+    __syncthreads();
+  }
+
+  // X = G^-1 by rows: X[i][j] = (delta_ij - sum_{k<i} G[i][k] X[k][j]) / G[i][i].
+  // Two threads per column j split the k range (even / odd) and combine by a lane swap.
+  {
+    const int j = tid >> 1, par = tid & 1;
+    for (int i = 0; i < NB; ++i) {
+      float acc = 0.f;
+      if (i > j) {
+        for (int k = j + par; k < i; k += 2) acc += G[i * GS + k] * X[k * GS + j];
+      }
+      acc += __shfl_xor(acc, 1);
+      if (par == 0 && i >= j) X[i * GS + j] = ((i == j ? 1.f : 0.f) - acc) / G[i * GS + i];
+      __syncthreads();
+    }
+  }
+
+  // M_bb[i][j] = G[127-j][127-i], Minv_bb[i][j] = X[127-j][127-i]  (i >= j), zero above
+  for (int idx = tid; idx < NB * NB; idx += 256) {
+    const int i = idx / NB, j = idx % NB;
+    float m = 0.f, x = 0.f;
+    if (i >= j) {
+      m = G[(NB - 1 - j) * GS + (NB - 1 - i)];
+      x = X[(NB - 1 - j) * GS + (NB - 1 - i)];
+    }
+    D[(int64_t)i * ld + j] = m;
+    Dinv[(int64_t)i * ld + j] = x;
+  }
+  if (tid == 0 && bad) atomicMax(status, b + 1);
+}
+
+struct Plan {
+  int64_t K, Kp;
+  float *A, *Minv, *T;
+  uint8_t *dead;
+  size_t bytes;
+};
+
+Plan make_plan(int64_t K, void *ws) {
+  Plan p;
+  p.K = K;
+  p.Kp = round_up64(K, NB);
+  const size_t mat = (size_t)p.Kp * (size_t)p.Kp * sizeof(float);
+  char *base = reinterpret_cast<char *>(ws);
+  p.A = reinterpret_cast<float *>(base);
+  p.Minv = reinterpret_cast<float *>(base + mat);
+  p.T = reinterpret_cast<float *>(base + 2 * mat);
+  p.dead = reinterpret_cast<uint8_t *>(base + 3 * mat);
+  p.bytes = 3 * mat + (size_t)round_up64(K, 256);
+  return p;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t gptq_hip_damp_invert_workspace_bytes(int64_t K) {
+  if (K <= 0) return 0;
+  return make_plan(K, nullptr).bytes;
+}
+
+int gptq_hip_damp_invert(void *stream, float *H, float *W, int64_t K, int64_t N, int64_t ldw,
+                         float damping, int fix_dead, float *L, int32_t *status, void *ws,
+                         size_t ws_bytes) {
+  if (!H || !L || !status || K <= 0 || K > 65535 || N < 0 || (N > 0 && (!W || ldw < N)))
+    return GPTQ_HIP_EINVAL;
+  if (!ws || ws_bytes < gptq_hip_damp_invert_workspace_bytes(K)) return GPTQ_HIP_EWORKSPACE;
+  if ((reinterpret_cast<uintptr_t>(ws) & 15) != 0) return GPTQ_HIP_EINVAL;
+  hipStream_t st = as_stream(stream);
+  const Plan p = make_plan(K, ws);
+  const int64_t Kp = p.Kp;
+  const int nblk = (int)(Kp / NB);
+
+  hipLaunchKernelGGL(damp_diag_kernel, dim3(1), dim3(1024), 0, st, H, K, damping, fix_dead,
+                     p.dead, status);
+  GPTQ_CHECK_LAUNCH();
+  if (N > 0) {
+    unsigned gx = (unsigned)ceil_div64(N, 256);
+    if (gx > 32) gx = 32;
+    hipLaunchKernelGGL(zero_dead_rows_kernel, dim3(gx, (unsigned)K), dim3(256), 0, st, W, N, ldw,
+                       p.dead);
+    GPTQ_CHECK_LAUNCH();
+  }
+  {
+    unsigned gx = (unsigned)ceil_div64(Kp, 256);
+    if (gx > 32) gx = 32;
+    hipLaunchKernelGGL(pad_copy_kernel, dim3(gx, (unsigned)Kp), dim3(256), 0, st, H, K, p.A, p.Minv,
+                       Kp);
+    GPTQ_CHECK_LAUNCH();
+  }
+
+  // ---- step 1: H = M^T M, last block first
+  const size_t diag_lds = 2 * (size_t)NB * GS * sizeof(float);
+  static_assert(2 * NB * GS * sizeof(float) <= 160 * 1024 - 1024, "diag block must fit LDS");
+  if (hipFuncSetAttribute(reinterpret_cast<const void *>(chol_diag_kernel),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)diag_lds) != hipSuccess)
+    return GPTQ_HIP_ELAUNCH;
+  for (int b = nblk - 1; b >= 0; --b) {
+    hipLaunchKernelGGL(chol_diag_kernel, dim3(1), dim3(256), diag_lds, st, p.A, p.Minv, Kp, b,
+                       status);
+    GPTQ_CHECK_LAUNCH();
+    if (b == 0) break;
+    float *panel = p.A + (int64_t)b * NB * Kp;  // rows of block b, columns 0 .. b*NB
+    // panel <- Minv_bb^T * panel   (in place: every workgroup reads only its own columns)
+    GemmArgs g;
+    g.A = p.Minv + (int64_t)b * NB * Kp + (int64_t)b * NB;
+    g.B = panel;
+    g.C = panel;
+    g.lda = g.ldb = g.ldc = Kp;
+    g.m = NB;
+    g.n = b * NB;
+    g.k = NB;
+    g.alpha = 1.f;
+    g.beta = 0.f;
+    g.a_kmajor = 1;
+    int rc = gptq_gemm_f32(st, g);
+    if (rc) return rc;
+    // A[0:b, 0:b] -= panel^T panel  (lower tiles)
+    GemmArgs s;
+    s.A = panel;
+    s.B = panel;
+    s.C = p.A;
+    s.lda = s.ldb = s.ldc = Kp;
+    s.m = s.n = b * NB;
+    s.k = NB;
+    s.alpha = -1.f;
+    s.beta = 1.f;
+    s.a_kmajor = 1;
+    s.tri = 2;
+    rc = gptq_gemm_f32(st, s);
+    if (rc) return rc;
+  }
+
+  // ---- step 2: L = M^-1 by pairwise merging
+  for (int64_t s = NB; s < Kp; s *= 2) {
+    const int npairs = (int)ceil_div64(Kp, 2 * s);
+    const int64_t pair_stride = 2 * s * (Kp + 1);
+    // T = C * Ainv
+    GemmArgs g;
+    g.A = p.A + s * Kp;             // C of pair 0: rows [s, 2s), cols [0, s)
+    g.B = p.Minv;                   // Ainv of pair 0
+    g.C = p.T + s * Kp;
+    g.lda = g.ldb = g.ldc = Kp;
+    g.m = (int)s;
+    g.n = (int)s;
+    g.k = (int)s;
+    g.alpha = 1.f;
+    g.beta = 0.f;
+    g.a_kmajor = 0;
+    g.kskip = 1;
+    g.batch = npairs;
+    g.strideA = g.strideB = g.strideC = pair_stride;
+    g.m_total = (int)(Kp - s);
+    g.m_step = (int)(2 * s);
+    int rc = gptq_gemm_f32(st, g);
+    if (rc) return rc;
+    // Minv[B rows, A cols] = -Binv * T
+    GemmArgs h;
+    h.A = p.Minv + s * (Kp + 1);    // Binv of pair 0
+    h.B = p.T + s * Kp;
+    h.C = p.Minv + s * Kp;
+    h.lda = h.ldb = h.ldc = Kp;
+    h.m = (int)s;
+    h.n = (int)s;
+    h.k = (int)s;
+    h.alpha = -1.f;
+    h.beta = 0.f;
+    h.a_kmajor = 0;
+    h.kskip = 2;
+    h.batch = npairs;
+    h.strideA = h.strideB = h.strideC = pair_stride;
+    h.m_total = (int)(Kp - s);
+    h.m_step = (int)(2 * s);
+    h.k_total = (int)(Kp - s);
+    h.k_step = (int)(2 * s);
+    rc = gptq_gemm_f32(st, h);
+    if (rc) return rc;
+  }
+
+  {
+    unsigned gx = (unsigned)ceil_div64(K, 256);
+    if (gx > 32) gx = 32;
+    hipLaunchKernelGGL(copy_out_kernel, dim3(gx, (unsigned)K), dim3(256), 0, st, p.Minv, Kp, L, K);
+    GPTQ_CHECK_LAUNCH();
+  }
+  return GPTQ_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,329 @@
+// Per-column quantisation parameters, int4 nibble codec, dequantisation and the row /
+// symmetric gathers of the activation-order option.  All of these are HBM-bound
+// streaming kernels: lanes run along the innermost (contiguous) axis.
+#include "common.h"
+
+namespace {
+
+constexpr int TPB = 256;
+
+// ------------------------------------------------------------------ column min/max
+// stage 1: grid (ceil(N/TPB), S); thread = one column, rows [s*rows_per, ...) -> partial
+template <typename T>
+__global__ __launch_bounds__(TPB) void col_minmax_partial(const T *W, int64_t K, int64_t N,
+                                                          int64_t ldw, int rows_per,
+                                                          float *part /* [S][2][N] */) {
+  const int64_t n = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  if (n >= N) return;
+  const int s = blockIdx.y;
+  const int64_t r0 = (int64_t)s * rows_per;
+  const int64_t r1 = min(K, r0 + (int64_t)rows_per);
+  float mn = INFINITY, mx = -INFINITY;
+  for (int64_t r = r0; r < r1; ++r) {
+    const float v = to_f32(W[r * ldw + n]);
+    mn = fminf(mn, v);
+    mx = fmaxf(mx, v);
+  }
+  part[((int64_t)s * 2 + 0) * N + n] = mn;
+  part[((int64_t)s * 2 + 1) * N + n] = mx;
+}
+
+__global__ __launch_bounds__(TPB) void col_params_finish(const float *part, int S, int64_t N,
+                                                         float maxq, float *scale, float *zero) {
+#pragma clang fp contract(off)
+  const int64_t n = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  if (n >= N) return;
+  float mn = INFINITY, mx = -INFINITY;
+  for (int s = 0; s < S; ++s) {
+    mn = fminf(mn, part[((int64_t)s * 2 + 0) * N + n]);
+    mx = fmaxf(mx, part[((int64_t)s * 2 + 1) * N + n]);
+  }
+  float xmin = fminf(0.f, mn), xmax = fmaxf(0.f, mx);
+  if (xmin == 0.f) xmin = -1.f;
+  if (xmax == 0.f) xmax = 1.f;
+  const float sc = (xmax - xmin) / maxq;
+  scale[n] = sc;
+  zero[n] = rintf(-xmin / sc);
+}
+
+// ------------------------------------------------------------------ nibble codec
+// [outer, axis, inner] views; one thread per packed byte.
+template <typename TC>
+__global__ __launch_bounds__(TPB) void pack_kernel(const TC *codes, int64_t outer, int64_t pa,
+                                                   int64_t inner, uint8_t *packed) {
+  const int64_t total = outer * pa * inner;
+  for (int64_t idx = (int64_t)blockIdx.x * TPB + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * TPB) {
+    const int64_t i = idx % inner, j = (idx / inner) % pa, o = idx / (inner * pa);
+    const int64_t src = (o * (2 * pa) + 2 * j) * inner + i;
+    const uint8_t lo = (uint8_t)codes[src], hi = (uint8_t)codes[src + inner];
+    packed[idx] = (uint8_t)(lo | (uint8_t)(hi << 4));
+  }
+}
+
+__global__ __launch_bounds__(TPB) void unpack_kernel(const uint8_t *packed, int64_t outer,
+                                                     int64_t pa, int64_t inner, uint8_t *codes) {
+  const int64_t total = outer * pa * inner;
+  for (int64_t idx = (int64_t)blockIdx.x * TPB + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * TPB) {
+    const int64_t i = idx % inner, j = (idx / inner) % pa, o = idx / (inner * pa);
+    const uint8_t b = packed[idx];
+    const int64_t dst = (o * (2 * pa) + 2 * j) * inner + i;
+    codes[dst] = b & 0xF;
+    codes[dst + inner] = (b >> 4) & 0xF;
+  }
+}
+
+__device__ __forceinline__ uint8_t code_of(float q, float sc, float z) {
+#pragma clang fp contract(off)
+  float c = rintf(q / sc + z);
+  c = fminf(fmaxf(c, 0.f), 255.f);
+  return (uint8_t)c;
+}
+
+template <typename TQ>
+__global__ __launch_bounds__(TPB) void quantize_pack_kernel(const TQ *Q, int64_t outer, int64_t pa,
+                                                            int64_t inner, const float *scale,
+                                                            const float *zero, uint8_t *packed) {
+  const int64_t total = outer * pa * inner;
+  for (int64_t idx = (int64_t)blockIdx.x * TPB + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * TPB) {
+    const int64_t i = idx % inner, j = (idx / inner) % pa, o = idx / (inner * pa);
+    const int64_t src = (o * (2 * pa) + 2 * j) * inner + i;
+    const float sc = scale[o * inner + i], z = zero[o * inner + i];
+    const uint8_t lo = code_of(to_f32(Q[src]), sc, z);
+    const uint8_t hi = code_of(to_f32(Q[src + inner]), sc, z);
+    packed[idx] = (uint8_t)(lo | (uint8_t)(hi << 4));
+  }
+}
+
+// out = (code - zero) * scale, each operation rounded to the element type T (the
+// reference computes in zero.dtype).
+template <typename T>
+__global__ __launch_bounds__(TPB) void dequant_kernel(const uint8_t *packed, int64_t outer,
+                                                      int64_t pa, int64_t inner, const T *zero,
+                                                      const T *scale, T *out) {
+#pragma clang fp contract(off)
+  const int64_t total = outer * pa * inner;
+  for (int64_t idx = (int64_t)blockIdx.x * TPB + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * TPB) {
+    const int64_t i = idx % inner, j = (idx / inner) % pa, o = idx / (inner * pa);
+    const uint8_t b = packed[idx];
+    const float z = to_f32(zero[o * inner + i]), sc = to_f32(scale[o * inner + i]);
+    const int64_t dst = (o * (2 * pa) + 2 * j) * inner + i;
+    const float d0 = to_f32(from_f32<T>((float)(b & 0xF) - z));
+    const float d1 = to_f32(from_f32<T>((float)((b >> 4) & 0xF) - z));
+    out[dst] = from_f32<T>(d0 * sc);
+    out[dst + inner] = from_f32<T>(d1 * sc);
+  }
+}
+
+// ------------------------------------------------------------------ gathers
+template <typename T>
+__global__ __launch_bounds__(TPB) void gather_rows_kernel(const T *in, T *out, int64_t N,
+                                                          const int64_t *perm) {
+  const int64_t row = blockIdx.y;
+  const int64_t src = perm[row];
+  for (int64_t c = (int64_t)blockIdx.x * TPB + threadIdx.x; c < N; c += (int64_t)gridDim.x * TPB)
+    out[row * N + c] = in[src * N + c];
+}
+
+__global__ __launch_bounds__(TPB) void gather_sym_kernel(const float *in, float *out, int64_t K,
+                                                         const int64_t *perm) {
+  const int64_t row = blockIdx.y;
+  const int64_t src = perm[row];
+  for (int64_t c = (int64_t)blockIdx.x * TPB + threadIdx.x; c < K; c += (int64_t)gridDim.x * TPB)
+    out[row * K + c] = in[src * K + perm[c]];
+}
+
+inline unsigned grid_for(int64_t total) {
+  int64_t g = ceil_div64(total, TPB);
+  if (g > 1 << 20) g = 1 << 20;
+  if (g < 1) g = 1;
+  return (unsigned)g;
+}
+
+inline int minmax_splits(int64_t K) {
+  int64_t s = ceil_div64(K, 64);
+  if (s > 64) s = 64;
+  if (s < 1) s = 1;
+  return (int)s;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t gptq_hip_col_params_workspace_bytes(int64_t K, int64_t N) {
+  if (K <= 0 || N <= 0) return 0;
+  return (size_t)minmax_splits(K) * 2 * (size_t)N * sizeof(float);
+}
+
+int gptq_hip_col_params(void *stream, const void *W, int w_dtype, int64_t K, int64_t N,
+                        int64_t ldw, int bits, float *scale, float *zero, void *ws,
+                        size_t ws_bytes) {
+  if (!W || !scale || !zero || K <= 0 || N <= 0 || ldw < N || bits < 1 || bits > 8)
+    return GPTQ_HIP_EINVAL;
+  if (!ws || ws_bytes < gptq_hip_col_params_workspace_bytes(K, N)) return GPTQ_HIP_EWORKSPACE;
+  const int S = minmax_splits(K);
+  const int rows_per = (int)ceil_div64(K, S);
+  const dim3 grid((unsigned)ceil_div64(N, TPB), (unsigned)S);
+  float *part = reinterpret_cast<float *>(ws);
+  hipStream_t st = as_stream(stream);
+  switch (w_dtype) {
+    case GPTQ_HIP_F32:
+      hipLaunchKernelGGL(col_minmax_partial<float>, grid, dim3(TPB), 0, st,
+                         (const float *)W, K, N, ldw, rows_per, part);
+      break;
+    case GPTQ_HIP_F16:
+      hipLaunchKernelGGL(col_minmax_partial<__half>, grid, dim3(TPB), 0, st,
+                         (const __half *)W, K, N, ldw, rows_per, part);
+      break;
+    case GPTQ_HIP_BF16:
+      hipLaunchKernelGGL(col_minmax_partial<__hip_bfloat16>, grid, dim3(TPB), 0, st,
+                         (const __hip_bfloat16 *)W, K, N, ldw, rows_per, part);
+      break;
+    default:
+      return GPTQ_HIP_EDTYPE;
+  }
+  GPTQ_CHECK_LAUNCH();
+  hipLaunchKernelGGL(col_params_finish, dim3((unsigned)ceil_div64(N, TPB)), dim3(TPB), 0, st, part,
+                     S, N, (float)((1 << bits) - 1), scale, zero);
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
+int gptq_hip_pack_int4(void *stream, const void *codes, int code_bytes, int64_t outer,
+                       int64_t axis_len, int64_t inner, uint8_t *packed) {
+  if (outer < 0 || axis_len < 0 || inner < 0 || (axis_len & 1)) return GPTQ_HIP_EINVAL;
+  const int64_t total = outer * (axis_len / 2) * inner;
+  if (total == 0) return GPTQ_HIP_OK;
+  if (!codes || !packed) return GPTQ_HIP_EINVAL;
+  hipStream_t st = as_stream(stream);
+  if (code_bytes == 1)
+    hipLaunchKernelGGL(pack_kernel<uint8_t>, dim3(grid_for(total)), dim3(TPB), 0, st,
+                       (const uint8_t *)codes, outer, axis_len / 2, inner, packed);
+  else if (code_bytes == 4)
+    hipLaunchKernelGGL(pack_kernel<int32_t>, dim3(grid_for(total)), dim3(TPB), 0, st,
+                       (const int32_t *)codes, outer, axis_len / 2, inner, packed);
+  else if (code_bytes == 8)
+    hipLaunchKernelGGL(pack_kernel<int64_t>, dim3(grid_for(total)), dim3(TPB), 0, st,
+                       (const int64_t *)codes, outer, axis_len / 2, inner, packed);
+  else
+    return GPTQ_HIP_EDTYPE;
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
+int gptq_hip_unpack_int4(void *stream, const uint8_t *packed, int64_t outer,
+                         int64_t packed_axis_len, int64_t inner, uint8_t *codes) {
+  if (outer < 0 || packed_axis_len < 0 || inner < 0) return GPTQ_HIP_EINVAL;
+  const int64_t total = outer * packed_axis_len * inner;
+  if (total == 0) return GPTQ_HIP_OK;
+  if (!codes || !packed) return GPTQ_HIP_EINVAL;
+  hipLaunchKernelGGL(unpack_kernel, dim3(grid_for(total)), dim3(TPB), 0, as_stream(stream), packed,
+                     outer, packed_axis_len, inner, codes);
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
+int gptq_hip_quantize_pack(void *stream, const void *Q, int q_dtype, int64_t outer,
+                           int64_t axis_len, int64_t inner, const float *scale,
+                           const float *zero, uint8_t *packed) {
+  if (outer < 0 || axis_len < 0 || inner < 0 || (axis_len & 1)) return GPTQ_HIP_EINVAL;
+  const int64_t total = outer * (axis_len / 2) * inner;
+  if (total == 0) return GPTQ_HIP_OK;
+  if (!Q || !scale || !zero || !packed) return GPTQ_HIP_EINVAL;
+  hipStream_t st = as_stream(stream);
+  const dim3 grid(grid_for(total)), block(TPB);
+  switch (q_dtype) {
+    case GPTQ_HIP_F32:
+      hipLaunchKernelGGL(quantize_pack_kernel<float>, grid, block, 0, st, (const float *)Q, outer,
+                         axis_len / 2, inner, scale, zero, packed);
+      break;
+    case GPTQ_HIP_F16:
+      hipLaunchKernelGGL(quantize_pack_kernel<__half>, grid, block, 0, st, (const __half *)Q,
+                         outer, axis_len / 2, inner, scale, zero, packed);
+      break;
+    case GPTQ_HIP_BF16:
+      hipLaunchKernelGGL(quantize_pack_kernel<__hip_bfloat16>, grid, block, 0, st,
+                         (const __hip_bfloat16 *)Q, outer, axis_len / 2, inner, scale, zero,
+                         packed);
+      break;
+    default:
+      return GPTQ_HIP_EDTYPE;
+  }
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
+int gptq_hip_dequant(void *stream, const uint8_t *packed, int64_t outer,
+                     int64_t packed_axis_len, int64_t inner, const void *zero,
+                     const void *scale, int zs_dtype, void *out) {
+  if (outer < 0 || packed_axis_len < 0 || inner < 0) return GPTQ_HIP_EINVAL;
+  const int64_t total = outer * packed_axis_len * inner;
+  if (total == 0) return GPTQ_HIP_OK;
+  if (!packed || !zero || !scale || !out) return GPTQ_HIP_EINVAL;
+  hipStream_t st = as_stream(stream);
+  const dim3 grid(grid_for(total)), block(TPB);
+  switch (zs_dtype) {
+    case GPTQ_HIP_F32:
+      hipLaunchKernelGGL(dequant_kernel<float>, grid, block, 0, st, packed, outer, packed_axis_len,
+                         inner, (const float *)zero, (const float *)scale, (float *)out);
+      break;
+    case GPTQ_HIP_F16:
+      hipLaunchKernelGGL(dequant_kernel<__half>, grid, block, 0, st, packed, outer,
+                         packed_axis_len, inner, (const __half *)zero, (const __half *)scale,
+                         (__half *)out);
+      break;
+    case GPTQ_HIP_BF16:
+      hipLaunchKernelGGL(dequant_kernel<__hip_bfloat16>, grid, block, 0, st, packed, outer,
+                         packed_axis_len, inner, (const __hip_bfloat16 *)zero,
+                         (const __hip_bfloat16 *)scale, (__hip_bfloat16 *)out);
+      break;
+    default:
+      return GPTQ_HIP_EDTYPE;
+  }
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
+int gptq_hip_gather_rows(void *stream, const void *in, void *out, int elem_bytes, int64_t K,
+                         int64_t N, const int64_t *perm) {
+  if (K <= 0 || N <= 0) return GPTQ_HIP_OK;
+  if (!in || !out || !perm) return GPTQ_HIP_EINVAL;
+  hipStream_t st = as_stream(stream);
+  unsigned gx = (unsigned)ceil_div64(N, TPB);
+  if (gx > 64) gx = 64;
+  // blockIdx.y carries the row; rows beyond 65535 are handled by row-chunked launches
+  for (int64_t r0 = 0; r0 < K; r0 += 65535) {
+    const unsigned rows = (unsigned)min((int64_t)65535, K - r0);
+    const dim3 grid(gx, rows);
+    if (elem_bytes == 4)
+      hipLaunchKernelGGL(gather_rows_kernel<uint32_t>, grid, dim3(TPB), 0, st,
+                         (const uint32_t *)in, (uint32_t *)out + r0 * N, N, perm + r0);
+    else if (elem_bytes == 2)
+      hipLaunchKernelGGL(gather_rows_kernel<uint16_t>, grid, dim3(TPB), 0, st,
+                         (const uint16_t *)in, (uint16_t *)out + r0 * N, N, perm + r0);
+    else if (elem_bytes == 1)
+      hipLaunchKernelGGL(gather_rows_kernel<uint8_t>, grid, dim3(TPB), 0, st, (const uint8_t *)in,
+                         (uint8_t *)out + r0 * N, N, perm + r0);
+    else
+      return GPTQ_HIP_EDTYPE;
+    GPTQ_CHECK_LAUNCH();
+  }
+  return GPTQ_HIP_OK;
+}
+
+int gptq_hip_gather_sym(void *stream, const float *in, float *out, int64_t K, const int64_t *perm) {
+  if (K <= 0) return GPTQ_HIP_OK;
+  if (!in || !out || !perm || K > 65535) return GPTQ_HIP_EINVAL;
+  unsigned gx = (unsigned)ceil_div64(K, TPB);
+  if (gx > 64) gx = 64;
+  hipLaunchKernelGGL(gather_sym_kernel, dim3(gx, (unsigned)K), dim3(TPB), 0, as_stream(stream), in,
+                     out, K, perm);
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,252 @@
+// fp32 MFMA GEMM for gfx950: C = alpha * op(A) * B + beta * C.
+//
+// One workgroup (4 wavefronts of 64) owns a 128x128 tile of C; each wavefront owns a
+// 64x64 quadrant as 2x2 tiles of v_mfma_f32_32x32x2_f32 (64 accumulator VGPRs).  A and B
+// are staged through LDS in slabs of 16 along k, double buffered: the global loads of
+// slab s+1 are issued before the MFMAs of slab s and written to the other LDS buffer
+// afterwards, so one barrier per slab is enough.
+//
+// LDS layouts are chosen for the MFMA operand fetch (lane l supplies element
+// [l % 32][l / 32] of a 32x2 operand):
+//   k-major operands ([k][idx], row stride 160 floats): the two half-waves read two
+//     consecutive k rows, 32 consecutive floats each, 32 banks apart;
+//   idx-major A ([m][k], row stride 17 floats): consecutive lanes are 17 banks apart.
+#include "gemm_f32.h"
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+namespace {
+
+constexpr int BM = 128, BN = 128, BK = 16, NTHREADS = 256;
+constexpr int LDT = 160;   // k-major LDS row stride (floats)
+constexpr int LDI = 17;    // idx-major LDS row stride (floats)
+constexpr int TILE_FLOATS = BK * LDT;  // 2560 >= BM * LDI (2176)
+
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+  static __device__ __forceinline__ void load(const float *p, float (&v)[4]) {
+    const float4 r = *reinterpret_cast<const float4 *>(p);
+    v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w;
+  }
+};
+template <> struct Vec4<__half> {
+  static __device__ __forceinline__ void load(const __half *p, float (&v)[4]) {
+    const uint2 r = *reinterpret_cast<const uint2 *>(p);
+    const __half2 a = *reinterpret_cast<const __half2 *>(&r.x);
+    const __half2 b = *reinterpret_cast<const __half2 *>(&r.y);
+    const float2 fa = __half22float2(a), fb = __half22float2(b);
+    v[0] = fa.x; v[1] = fa.y; v[2] = fb.x; v[3] = fb.y;
+  }
+};
+template <> struct Vec4<__hip_bfloat16> {
+  static __device__ __forceinline__ void load(const __hip_bfloat16 *p, float (&v)[4]) {
+    const uint2 r = *reinterpret_cast<const uint2 *>(p);
+    v[0] = __uint_as_float(r.x << 16); v[1] = __uint_as_float(r.x & 0xffff0000u);
+    v[2] = __uint_as_float(r.y << 16); v[3] = __uint_as_float(r.y & 0xffff0000u);
+  }
+};
+
+// 4 consecutive elements of a row; `nvalid` of them exist (0..4), the rest read as 0.
+template <typename T>
+__device__ __forceinline__ void load_row4(const T *p, bool fast, int nvalid, float (&v)[4]) {
+  if (fast) {
+    Vec4<T>::load(p, v);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = (e < nvalid) ? to_f32(p[e]) : 0.f;
+  }
+}
+
+template <typename T, bool AK>
+__global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(GemmArgs p) {
+  __shared__ __attribute__((aligned(16))) float As[2][TILE_FLOATS];
+  __shared__ __attribute__((aligned(16))) float Bs[2][TILE_FLOATS];
+
+  int tm, tn;
+  if (p.tri) {
+    const int t = blockIdx.x;
+    int i = (int)((sqrtf(8.f * (float)t + 1.f) - 1.f) * 0.5f);
+    while ((i + 1) * (i + 2) / 2 <= t) ++i;
+    while (i * (i + 1) / 2 > t) --i;
+    const int j = t - i * (i + 1) / 2;  // j <= i
+    if (p.tri == 2) { tm = i; tn = j; } else { tm = j; tn = i; }
+  } else {
+    tn = blockIdx.x;
+    tm = blockIdx.y;
+  }
+  const int z = blockIdx.z;
+  int m_eff = p.m, k_eff = p.k;
+  if (p.m_step) m_eff = min(p.m, p.m_total - z * p.m_step);
+  if (p.k_step) k_eff = min(p.k, p.k_total - z * p.k_step);
+  const int m0 = tm * BM, n0 = tn * BN;
+  if (m0 >= m_eff || n0 >= p.n || k_eff <= 0) return;
+
+  int kb = 0, ke = k_eff;
+  if (p.kskip & 1) kb = min(n0, ke) & ~(BK - 1);
+  if (p.kskip & 2) ke = min(ke, m0 + BM);
+
+  const T *A = reinterpret_cast<const T *>(p.A) + (int64_t)z * p.strideA;
+  const T *B = reinterpret_cast<const T *>(p.B) + (int64_t)z * p.strideB;
+  float *C = p.C + (int64_t)z * p.strideC;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l32 = lane & 31, lhi = lane >> 5;
+
+  const bool a_al = (p.lda % 4 == 0) && ((reinterpret_cast<uintptr_t>(A) % (4 * sizeof(T))) == 0);
+  const bool b_al = (p.ldb % 4 == 0) && ((reinterpret_cast<uintptr_t>(B) % (4 * sizeof(T))) == 0);
+  const bool m_full = (m0 + BM <= m_eff);
+  const bool n_full = (n0 + BN <= p.n);
+
+  float ra[2][4], rb[2][4];
+
+  auto load_tiles = [&](int kt) {
+    const bool k_full = (kt + BK <= ke);
+    if (AK) {
+      const int r = tid >> 5, c4 = (tid & 31) * 4;
+      const bool fast = a_al && m_full && k_full;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int kk = kt + r + 8 * i;
+        int nv = (kk < ke) ? min(4, m_eff - (m0 + c4)) : 0;
+        const T *src = A + (int64_t)kk * p.lda + m0 + c4;
+        load_row4<T>(src, fast, nv, ra[i]);
+      }
+    } else {
+      const int row = tid >> 2, k4 = (tid & 3) * 4;
+      const bool fast = a_al && m_full && k_full;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int mm = m0 + row + 64 * i;
+        int nv = (mm < m_eff) ? min(4, ke - (kt + k4)) : 0;
+        const T *src = A + (int64_t)mm * p.lda + kt + k4;
+        load_row4<T>(src, fast, nv, ra[i]);
+      }
+    }
+    {
+      const int r = tid >> 5, c4 = (tid & 31) * 4;
+      const bool fast = b_al && n_full && k_full;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int kk = kt + r + 8 * i;
+        int nv = (kk < ke) ? min(4, p.n - (n0 + c4)) : 0;
+        const T *src = B + (int64_t)kk * p.ldb + n0 + c4;
+        load_row4<T>(src, fast, nv, rb[i]);
+      }
+    }
+  };
+
+  auto store_tiles = [&](int buf) {
+    if (AK) {
+      const int r = tid >> 5, c4 = (tid & 31) * 4;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        *reinterpret_cast<float4 *>(&As[buf][(r + 8 * i) * LDT + c4]) =
+            make_float4(ra[i][0], ra[i][1], ra[i][2], ra[i][3]);
+    } else {
+      const int row = tid >> 2, k4 = (tid & 3) * 4;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) As[buf][(row + 64 * i) * LDI + k4 + e] = ra[i][e];
+    }
+    {
+      const int r = tid >> 5, c4 = (tid & 31) * 4;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        *reinterpret_cast<float4 *>(&Bs[buf][(r + 8 * i) * LDT + c4]) =
+            make_float4(rb[i][0], rb[i][1], rb[i][2], rb[i][3]);
+    }
+  };
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  int buf = 0;
+  if (kb < ke) {
+    load_tiles(kb);
+    store_tiles(0);
+  }
+  __syncthreads();
+  for (int kt = kb; kt < ke; kt += BK) {
+    const bool more = (kt + BK < ke);
+    if (more) load_tiles(kt + BK);
+    const float *as = As[buf];
+    const float *bs = Bs[buf];
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 2) {
+      const int krow = kk + lhi;
+      float a[2], b[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        a[t] = AK ? as[krow * LDT + wm * 64 + t * 32 + l32]
+                  : as[(wm * 64 + t * 32 + l32) * LDI + krow];
+        b[t] = bs[krow * LDT + wn * 64 + t * 32 + l32];
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (more) store_tiles(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+  }
+
+  const float alpha = p.alpha, beta = p.beta;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = n0 + wn * 64 + j * 32 + l32;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+        if (row < m_eff && col < p.n) {
+          float *dst = C + (int64_t)row * p.ldc + col;
+          float v = alpha * acc[i][j][r];
+          if (beta != 0.f) v += beta * (*dst);
+          *dst = v;
+        }
+      }
+    }
+}
+
+}  // namespace
+
+int gptq_gemm_f32(hipStream_t stream, const GemmArgs &a) {
+  if (a.m <= 0 || a.n <= 0 || a.batch <= 0) return GPTQ_HIP_OK;
+  if (!a.A || !a.B || !a.C) return GPTQ_HIP_EINVAL;
+  dim3 grid;
+  const int tm = (a.m + BM - 1) / BM, tn = (a.n + BN - 1) / BN;
+  if (a.tri) {
+    const int t = tm > tn ? tm : tn;
+    grid = dim3((unsigned)((int64_t)t * (t + 1) / 2), 1, (unsigned)a.batch);
+  } else {
+    grid = dim3((unsigned)tn, (unsigned)tm, (unsigned)a.batch);
+  }
+  if (grid.y > 65535u || grid.z > 65535u) return GPTQ_HIP_EINVAL;
+  const dim3 block(NTHREADS);
+  if (a.in_dtype == GPTQ_HIP_F32) {
+    if (a.a_kmajor)
+      hipLaunchKernelGGL((gemm_f32_kernel<float, true>), grid, block, 0, stream, a);
+    else
+      hipLaunchKernelGGL((gemm_f32_kernel<float, false>), grid, block, 0, stream, a);
+  } else if (a.in_dtype == GPTQ_HIP_F16 && a.a_kmajor) {
+    hipLaunchKernelGGL((gemm_f32_kernel<__half, true>), grid, block, 0, stream, a);
+  } else if (a.in_dtype == GPTQ_HIP_BF16 && a.a_kmajor) {
+    hipLaunchKernelGGL((gemm_f32_kernel<__hip_bfloat16, true>), grid, block, 0, stream, a);
+  } else {
+    return GPTQ_HIP_EDTYPE;
+  }
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}

@@ -1,0 +1,179 @@
+// Blocked GPTQ column loop: quantise block_size rows with error feedback, then push the
+// accumulated error into all remaining rows with one fp32 MFMA GEMM per block.
+//
+// In-block kernel: the N output channels are independent, so one lane owns one channel.
+// The block is walked in sub-blocks of SB rows.  The SB rows of a sub-block and their SB
+// errors live in VGPRs (statically indexed, fully unrolled triangle); the rows of the
+// block below the sub-block are then updated in place in W (they stay L2-resident),
+// coalesced across lanes.  The block of L sits in LDS in its natural layout: every lane
+// reads the same address (LDS broadcast) and the SB factors of one row are consecutive.
+//
+// Every floating-point operation is the IEEE operation the reference writes (true
+// division, round-half-even, separate multiply and subtract) and every element receives
+// its updates in the reference's order, so given the same L and W the block result is
+// bit-identical to a CPU evaluation of gptq.py:136-147.
+#include "common.h"
+#include "gemm_f32.h"
+
+namespace {
+
+constexpr int SOLVE_TPB = 128;
+
+template <int SB, typename TQ>
+__global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
+    float *Wb, int64_t N, const float *Lb, int64_t ldl, int bs, const float *scale,
+    const float *zero, float maxq, TQ *Qb, uint8_t *cb, float *Err) {
+  // Wb, Qb, cb: first row of the block in W, Q, codes; Lb: the block's diagonal corner of L
+#pragma clang fp contract(off)
+  extern __shared__ float Ln[];  // Ln[j * bs + i] = Lb[j][i]
+  const int tid = threadIdx.x;
+  for (int idx = tid; idx < bs * bs; idx += SOLVE_TPB) {
+    const int j = idx / bs, i = idx - j * bs;
+    Ln[idx] = Lb[(int64_t)j * ldl + i];
+  }
+  __syncthreads();
+  const int64_t n = (int64_t)blockIdx.x * SOLVE_TPB + tid;
+  if (n >= N) return;
+  const float sc = scale[n], z = zero[n];
+  float *wcol = Wb + n;
+
+  for (int r0 = 0; r0 < bs; r0 += SB) {
+    float w[SB], e[SB];
+#pragma unroll
+    for (int t = 0; t < SB; ++t) w[t] = wcol[(int64_t)(r0 + t) * N];
+    const float *ld = Ln + r0 * bs + r0;  // diagonal sub-block
+#pragma unroll
+    for (int t = 0; t < SB; ++t) {
+      float x = w[t];
+#pragma unroll
+      for (int u = 0; u < t; ++u) {
+        const float upd = ld[t * bs + u] * e[u];
+        x = x - upd;
+      }
+      float q = rintf(x / sc) + z;
+      q = fminf(fmaxf(q, 0.f), maxq);
+      const float qh = sc * (q - z);
+      e[t] = (x - qh) / ld[t * bs + t];
+      const int64_t o = (int64_t)(r0 + t) * N + n;
+      if (Qb) Qb[o] = from_f32<TQ>(qh);
+      if (cb) cb[o] = (uint8_t)q;
+      Err[(int64_t)(r0 + t) * N + n] = e[t];
+    }
+    // rows of this block below the sub-block
+#pragma unroll 2
+    for (int j = r0 + SB; j < bs; ++j) {
+      float x = wcol[(int64_t)j * N];
+      const float *lr = Ln + j * bs + r0;
+#pragma unroll
+      for (int u = 0; u < SB; ++u) {
+        const float upd = lr[u] * e[u];
+        x = x - upd;
+      }
+      wcol[(int64_t)j * N] = x;
+    }
+  }
+}
+
+template <int SB>
+int launch_block(hipStream_t st, float *W, int64_t N, const float *L, int64_t ldl, int bs,
+                 const float *scale, const float *zero, float maxq, void *Q, int q_dtype,
+                 uint8_t *codes, float *Err) {
+  const dim3 grid((unsigned)ceil_div64(N, SOLVE_TPB)), block(SOLVE_TPB);
+  const size_t lds = (size_t)bs * bs * sizeof(float);
+  switch (q_dtype) {
+    case GPTQ_HIP_F32:
+      hipLaunchKernelGGL((block_quant_kernel<SB, float>), grid, block, lds, st, W, N, L, ldl,
+                         bs, scale, zero, maxq, (float *)Q, codes, Err);
+      break;
+    case GPTQ_HIP_F16:
+      hipLaunchKernelGGL((block_quant_kernel<SB, __half>), grid, block, lds, st, W, N, L, ldl,
+                         bs, scale, zero, maxq, (__half *)Q, codes, Err);
+      break;
+    case GPTQ_HIP_BF16:
+      hipLaunchKernelGGL((block_quant_kernel<SB, __hip_bfloat16>), grid, block, lds, st, W, N, L,
+                         ldl, bs, scale, zero, maxq, (__hip_bfloat16 *)Q, codes, Err);
+      break;
+    default:
+      return GPTQ_HIP_EDTYPE;
+  }
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
+bool block_size_ok(int bs) { return bs >= 1 && bs <= 128; }
+
+int process_block(hipStream_t st, float *Wb, int64_t N, const float *Lb, int64_t ldl, int bs,
+                  const float *scale, const float *zero, int maxq, void *Qb, int q_dtype,
+                  uint8_t *cb, float *Err) {
+#define GPTQ_SB_CASE(SB) \
+  return launch_block<SB>(st, Wb, N, Lb, ldl, bs, scale, zero, (float)maxq, Qb, q_dtype, cb, Err)
+  if (bs % 16 == 0) GPTQ_SB_CASE(16);
+  if (bs % 8 == 0) GPTQ_SB_CASE(8);
+  if (bs % 4 == 0) GPTQ_SB_CASE(4);
+  if (bs % 2 == 0) GPTQ_SB_CASE(2);
+  GPTQ_SB_CASE(1);
+#undef GPTQ_SB_CASE
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t gptq_hip_solve_workspace_bytes(int64_t K, int64_t N, int block_size) {
+  if (K <= 0 || N <= 0 || !block_size_ok(block_size)) return 0;
+  return (size_t)block_size * (size_t)N * sizeof(float);
+}
+
+int gptq_hip_process_block(void *stream, float *Wblock, int64_t N, const float *Lblock,
+                           int64_t ldl, int block_size, const float *scale, const float *zero,
+                           int maxq, void *Qblock, int q_dtype, uint8_t *codes_block,
+                           float *errors) {
+  if (!Wblock || !Lblock || !scale || !zero || !errors || N <= 0 || ldl < block_size)
+    return GPTQ_HIP_EINVAL;
+  if (!block_size_ok(block_size) || maxq < 1 || maxq > 255) return GPTQ_HIP_EINVAL;
+  return process_block(as_stream(stream), Wblock, N, Lblock, ldl, block_size, scale, zero, maxq,
+                       Qblock, q_dtype, codes_block, errors);
+}
+
+int gptq_hip_solve(void *stream, float *W, int64_t K, int64_t N, const float *L,
+                   const float *scale, const float *zero, int maxq, int block_size, void *Q,
+                   int q_dtype, uint8_t *codes, void *ws, size_t ws_bytes) {
+  if (!W || !L || !scale || !zero || K <= 0 || N <= 0 || K > 2147483647LL || N > 2147483647LL)
+    return GPTQ_HIP_EINVAL;
+  if (!block_size_ok(block_size) || K % block_size != 0 || maxq < 1 || maxq > 255)
+    return GPTQ_HIP_EINVAL;
+  if (q_dtype != GPTQ_HIP_F32 && q_dtype != GPTQ_HIP_F16 && q_dtype != GPTQ_HIP_BF16)
+    return GPTQ_HIP_EDTYPE;
+  if (!ws || ws_bytes < gptq_hip_solve_workspace_bytes(K, N, block_size)) return GPTQ_HIP_EWORKSPACE;
+  hipStream_t st = as_stream(stream);
+  float *Err = reinterpret_cast<float *>(ws);
+  const size_t qsz = dtype_size(q_dtype);
+  for (int64_t start = 0; start < K; start += block_size) {
+    void *Qb = Q ? (void *)((char *)Q + (size_t)start * N * qsz) : nullptr;
+    uint8_t *cb = codes ? codes + start * N : nullptr;
+    int rc = process_block(st, W + start * N, N, L + start * K + start, K, block_size, scale, zero,
+                           maxq, Qb, q_dtype, cb, Err);
+    if (rc) return rc;
+    const int64_t end = start + block_size;
+    if (end >= K) break;
+    // W[end:, :] -= L[end:, start:end] @ Err
+    GemmArgs g;
+    g.A = L + end * K + start;
+    g.B = Err;
+    g.C = W + end * N;
+    g.lda = K;
+    g.ldb = N;
+    g.ldc = N;
+    g.m = (int)(K - end);
+    g.n = (int)N;
+    g.k = block_size;
+    g.alpha = -1.f;
+    g.beta = 1.f;
+    g.a_kmajor = 0;
+    rc = gptq_gemm_f32(st, g);
+    if (rc) return rc;
+  }
+  return GPTQ_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,73 @@
+"""ctypes binding of libgptq_hip.so (the C ABI declared in include/gptq_hip.h).
+
+There is no CPU fallback: importing the compute entry points without the built
+library raises, so that a missing HIP extension is never silently papered over.
+"""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libgptq_hip.so")
+
+F32, F16, BF16 = 0, 1, 2
+OK, EINVAL, EDTYPE, EWORKSPACE, ELAUNCH = 0, 1, 2, 3, 4
+
+_vp, _i64, _i32, _f32, _f64, _sz = (ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float,
+                                   ctypes.c_double, ctypes.c_size_t)
+
+# name -> (restype, argtypes); mirrors include/gptq_hip.h one to one
+SIGNATURES = {
+    "gptq_hip_abi_version": (_i32, []),
+    "gptq_hip_error_string": (ctypes.c_char_p, [_i32]),
+    "gptq_hip_col_params_workspace_bytes": (_sz, [_i64, _i64]),
+    "gptq_hip_col_params": (_i32, [_vp, _vp, _i32, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _sz]),
+    "gptq_hip_hessian_accumulate": (_i32, [_vp, _vp, _vp, _i32, _i32, _i64, _vp]),
+    "gptq_hip_hessian_finalize": (_i32, [_vp, _vp, _i64, _f64]),
+    "gptq_hip_damp_invert_workspace_bytes": (_sz, [_i64]),
+    "gptq_hip_damp_invert": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _f32, _i32, _vp, _vp, _vp, _sz]),
+    "gptq_hip_solve_workspace_bytes": (_sz, [_i64, _i64, _i32]),
+    "gptq_hip_solve": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _i32, _i32, _vp, _i32, _vp, _vp, _sz]),
+    "gptq_hip_process_block": (_i32, [_vp, _vp, _i64, _vp, _i64, _i32, _vp, _vp, _i32, _vp, _i32, _vp, _vp]),
+    "gptq_hip_gather_rows": (_i32, [_vp, _vp, _vp, _i32, _i64, _i64, _vp]),
+    "gptq_hip_gather_sym": (_i32, [_vp, _vp, _vp, _i64, _vp]),
+    "gptq_hip_pack_int4": (_i32, [_vp, _vp, _i32, _i64, _i64, _i64, _vp]),
+    "gptq_hip_unpack_int4": (_i32, [_vp, _vp, _i64, _i64, _i64, _vp]),
+    "gptq_hip_quantize_pack": (_i32, [_vp, _vp, _i32, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "gptq_hip_dequant": (_i32, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i32, _vp]),
+    "gptq_hip_qmatmul_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
+    "gptq_hip_qmatmul": (_i32, [_vp, _vp, _i32, _i64, _vp, _i64, _i64, _vp, _vp, _i32, _i32, _vp, _vp, _sz]),
+}
+
+_lib = None
+
+
+def load():
+    """Load the shared library (once) and attach the prototypes."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python jax-gptq_amd/build.py` "
+            "(hipcc, gfx950). There is no CPU fallback.")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    if lib.gptq_hip_abi_version() != 1:
+        raise ImportError("libgptq_hip.so has an unexpected ABI version")
+    _lib = lib
+    return lib
+
+
+def check(code, what):
+    """Map a status code to the exception type the reference raises in that situation."""
+    if code == OK:
+        return
+    msg = f"{what}: {load().gptq_hip_error_string(code).decode()}"
+    if code == EINVAL:
+        raise ValueError(msg)
+    if code == EDTYPE:
+        raise TypeError(msg)
+    raise RuntimeError(msg)

@@ -1,0 +1,415 @@
+"""Host-side mirror of the reference's ``jax_gptq/gptq.py`` on top of the HIP C ABI.
+
+Same names, argument order, defaults, return structure and error behaviour as the
+reference; arrays are ``torch`` tensors on the GPU (torch is used for device memory
+and streams only -- every computation is a kernel of ``libgptq_hip.so``).  NumPy
+arrays and CPU tensors are accepted and moved to the device.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _native as N
+
+__all__ = [
+    "QuantizedMatrix", "quant_matrix_shape", "accumulate_H", "get_quantize_params",
+    "get_col_quantize_params", "gptq", "pack_matrix", "unpack_matrix", "pack_along_axis",
+    "unpack_along_axis", "pack_rowwise", "pack_colwise", "unpack_rowwise", "unpack_colwise",
+]
+
+_DT = {torch.float32: N.F32, torch.float16: N.F16, torch.bfloat16: N.BF16}
+
+
+def _device():
+    if not torch.cuda.is_available():
+        raise RuntimeError("jax_gptq_amd needs a ROCm GPU (gfx950); there is no CPU path")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def _dev(x, dtype=None):
+    """Array-like -> contiguous tensor on the current GPU."""
+    if isinstance(x, torch.Tensor):
+        t = x
+    else:
+        t = torch.from_numpy(np.ascontiguousarray(np.asarray(x)))
+    t = t.to(_device())
+    if dtype is not None and t.dtype != dtype:
+        t = t.to(dtype)
+    return t.contiguous()
+
+
+def _float_dev(x):
+    t = _dev(x)
+    if t.dtype not in _DT:
+        t = t.to(torch.float32)     # integer / fp64 inputs are promoted to fp32, as jnp would
+    return t
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _ws(nbytes):
+    return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=_device())
+
+
+class QuantizedMatrix:
+    """Packed matrix container (reference ``gptq.py:8-22``): ``int_weight`` uint8 with two
+    4-bit codes per byte along ``contraction_axis``, per-channel ``zero`` and ``scale``."""
+
+    def __init__(self, int_weight, zero, scale, contraction_axis=0):
+        self.int_weight = int_weight
+        self.zero = zero
+        self.scale = scale
+        self.contraction_axis = contraction_axis
+
+    @property
+    def shape(self):
+        return quant_matrix_shape(self)
+
+    @property
+    def dtype(self):
+        return self.zero.dtype
+
+    # pytree-style helpers (the reference registers the class as a pytree, gptq.py:24-32)
+    def tree_flatten(self):
+        return (self.int_weight, self.zero, self.scale), self.contraction_axis
+
+    @classmethod
+    def tree_unflatten(cls, contraction_axis, children):
+        return cls(*children, contraction_axis=contraction_axis)
+
+    def to(self, device):
+        return QuantizedMatrix(self.int_weight.to(device), self.zero.to(device),
+                               self.scale.to(device), self.contraction_axis)
+
+
+def quant_matrix_shape(quantized_matrix, bits=4):
+    """Logical shape of a packed matrix (reference ``gptq.py:34-42``)."""
+    mat = quantized_matrix.int_weight
+    ele_width = mat.element_size() * 8 if isinstance(mat, torch.Tensor) else mat.dtype.itemsize * 8
+    shape = list(mat.shape)
+    shape[quantized_matrix.contraction_axis] *= ele_width // bits
+    return tuple(shape)
+
+
+# ------------------------------------------------------------------------------- Hessian
+_MAX_BATCHES_PER_CALL = 1024
+
+
+def _accumulate_H_step(H, running_mean, n_samples, batch):
+    """One batch of the Hessian accumulation (reference ``gptq.py:57-74``).
+
+    The state differs from the reference's in representation, not in meaning: ``H``
+    carries the raw second-moment sum (upper 128x128 tiles) and ``running_mean`` stays
+    zero, so that the reference's closing formula ``H / n + outer(mean, mean)`` still
+    yields ``sum X^T X / n``.
+    """
+    batch = _float_dev(batch)
+    if batch.dim() > 2:
+        batch = batch.reshape(-1, batch.shape[-1])
+    _hessian_accumulate(H, [batch])
+    return H, running_mean, n_samples + batch.shape[0]
+
+
+def _hessian_accumulate(H, batches):
+    lib = N.load()
+    K = H.shape[0]
+    for lo in range(0, len(batches), _MAX_BATCHES_PER_CALL):
+        chunk = batches[lo:lo + _MAX_BATCHES_PER_CALL]
+        dts = {b.dtype for b in chunk}
+        if len(dts) != 1:
+            # one launch table per element type
+            for b in chunk:
+                _hessian_accumulate(H, [b])
+            continue
+        nb = len(chunk)
+        ptrs = (ctypes.c_void_p * nb)(*[b.data_ptr() for b in chunk])
+        rows = (ctypes.c_int64 * nb)(*[b.shape[0] for b in chunk])
+        N.check(lib.gptq_hip_hessian_accumulate(_stream(), ptrs, rows, nb, _DT[chunk[0].dtype], K,
+                                                _ptr(H)), "hessian_accumulate")
+
+
+def accumulate_H(xs, use_fp64=False):
+    """``H = sum_b X_b^T X_b / n`` over a list of calibration batches (``gptq.py:76-103``)."""
+    if use_fp64:
+        raise NotImplementedError("use_fp64=True is not available on the HIP path")
+    lib = N.load()
+    batches = []
+    for x in xs:
+        b = _float_dev(x)
+        if b.dim() > 2:
+            b = b.reshape(-1, b.shape[-1])
+        elif b.dim() == 1:
+            b = b.reshape(1, -1)
+        batches.append(b.contiguous())
+    K = batches[0].shape[-1]
+    for b in batches:
+        if b.shape[-1] != K:
+            raise ValueError("all calibration batches must share the feature dimension")
+    H = torch.zeros((K, K), dtype=torch.float32, device=_device())
+    _hessian_accumulate(H, batches)
+    n = sum(b.shape[0] for b in batches)
+    N.check(lib.gptq_hip_hessian_finalize(_stream(), _ptr(H), K, float(n)), "hessian_finalize")
+    return H
+
+
+# ------------------------------------------------------------------------------- params
+def get_col_quantize_params(weight, bits=4):
+    """Per-output-channel (column) min-max parameters (reference ``gptq.py:105-118``)."""
+    lib = N.load()
+    W = _float_dev(weight)
+    if W.dim() != 2:
+        raise ValueError("get_col_quantize_params expects a 2-D matrix")
+    K, Nc = W.shape
+    scale = torch.empty(Nc, dtype=torch.float32, device=W.device)
+    zero = torch.empty(Nc, dtype=torch.float32, device=W.device)
+    ws = _ws(lib.gptq_hip_col_params_workspace_bytes(K, Nc))
+    N.check(lib.gptq_hip_col_params(_stream(), _ptr(W), _DT[W.dtype], K, Nc, Nc, bits, _ptr(scale),
+                                    _ptr(zero), _ptr(ws), ws.numel()), "col_params")
+    return {"maxq": 2 ** bits - 1, "scale": scale, "zero": zero}
+
+
+def get_quantize_params(weight, bits=4):
+    """Parameters of one channel: min-max over the whole array (``gptq.py:105-116``)."""
+    W = _float_dev(weight).reshape(-1, 1)
+    p = get_col_quantize_params(W, bits=bits)
+    return {"maxq": p["maxq"], "scale": p["scale"].reshape(()), "zero": p["zero"].reshape(())}
+
+
+# ------------------------------------------------------------------------------- factor
+def _damp_invert(W, H, damping, fix_dead=True):
+    lib = N.load()
+    K = H.shape[0]
+    Nc = 0 if W is None else W.shape[1]
+    L = torch.empty((K, K), dtype=torch.float32, device=H.device)
+    status = torch.zeros(2, dtype=torch.int32, device=H.device)
+    ws = _ws(lib.gptq_hip_damp_invert_workspace_bytes(K))
+    N.check(lib.gptq_hip_damp_invert(_stream(), _ptr(H), _ptr(W), K, Nc, Nc, float(damping),
+                                     1 if fix_dead else 0, _ptr(L), _ptr(status), _ptr(ws),
+                                     ws.numel()), "damp_invert")
+    return L, status
+
+
+def _cholesky_inv(mat):
+    """Lower Cholesky factor of ``inv(mat)`` (reference ``gptq.py:44-48``)."""
+    H = _dev(mat, torch.float32).clone()
+    L, _ = _damp_invert(None, H, 0.0, fix_dead=False)
+    return L
+
+
+def _damp_and_invert(W, H, damping):
+    """Dead-feature fix, damping, factor of the inverse (reference ``gptq.py:155-168``).
+    ``W`` and ``H`` are updated in place (the reference donates both)."""
+    L, status = _damp_invert(W, H, damping, fix_dead=True)
+    any_nan = bool(status[0].item() != 0)
+    return W, L, any_nan
+
+
+# ------------------------------------------------------------------------------- act-order
+def _permute(W, H):
+    """Rows of ``W`` and rows/columns of ``H`` in descending ``diag(H)`` order (``gptq.py:170-175``)."""
+    lib = N.load()
+    K, Nc = W.shape
+    perm = torch.argsort(torch.diagonal(H), stable=True).flip(0).contiguous()
+    Wp = torch.empty_like(W)
+    Hp = torch.empty_like(H)
+    N.check(lib.gptq_hip_gather_rows(_stream(), _ptr(W), _ptr(Wp), W.element_size(), K, Nc,
+                                     _ptr(perm)), "gather_rows")
+    N.check(lib.gptq_hip_gather_sym(_stream(), _ptr(H), _ptr(Hp), K, _ptr(perm)), "gather_sym")
+    return Wp, Hp, perm
+
+
+def _unpermute(Q, perm):
+    """Inverse row permutation (reference ``gptq.py:177-180``)."""
+    lib = N.load()
+    K, Nc = Q.shape
+    invperm = torch.argsort(perm, stable=True).contiguous()
+    out = torch.empty_like(Q)
+    N.check(lib.gptq_hip_gather_rows(_stream(), _ptr(Q), _ptr(out), Q.element_size(), K, Nc,
+                                     _ptr(invperm)), "gather_rows")
+    return out
+
+
+# ------------------------------------------------------------------------------- loop
+def _process_block(W, Hinv, start, quantize_params, block_size):
+    """One block of the column loop (reference ``gptq.py:130-153``): returns
+    ``(q_block, errors)``, both ``[block_size, N]`` fp32.  ``W`` is not modified."""
+    lib = N.load()
+    W = _dev(W, torch.float32)
+    Hinv = _dev(Hinv, torch.float32)
+    K, Nc = W.shape
+    if start < 0 or start + block_size > K:
+        raise ValueError("block out of range")
+    blk = W[start:start + block_size].clone()
+    q = torch.empty((block_size, Nc), dtype=torch.float32, device=W.device)
+    err = torch.empty((block_size, Nc), dtype=torch.float32, device=W.device)
+    lblk = Hinv[start:, start:]
+    N.check(lib.gptq_hip_process_block(
+        _stream(), _ptr(blk), Nc, ctypes.c_void_p(lblk.data_ptr()), Hinv.shape[1], block_size,
+        _ptr(_dev(quantize_params["scale"], torch.float32)),
+        _ptr(_dev(quantize_params["zero"], torch.float32)), int(quantize_params["maxq"]),
+        _ptr(q), N.F32, ctypes.c_void_p(0), _ptr(err)), "process_block")
+    return q, err
+
+
+def _solve(W, L, params, block_size, out_dtype, want_codes=False):
+    lib = N.load()
+    K, Nc = W.shape
+    Q = torch.empty((K, Nc), dtype=out_dtype, device=W.device)
+    codes = torch.empty((K, Nc), dtype=torch.uint8, device=W.device) if want_codes else None
+    ws = _ws(lib.gptq_hip_solve_workspace_bytes(K, Nc, block_size))
+    N.check(lib.gptq_hip_solve(_stream(), _ptr(W), K, Nc, _ptr(L), _ptr(params["scale"]),
+                               _ptr(params["zero"]), int(params["maxq"]), block_size, _ptr(Q),
+                               _DT[out_dtype], _ptr(codes), _ptr(ws), ws.numel()), "solve")
+    return Q, codes
+
+
+def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False):
+    """The per-layer GPTQ solve (reference ``gptq.py:182-212``).
+
+    ``W`` is ``[K, N]`` (input features x output channels), ``xs`` a list of calibration
+    batches ``[..., K]``.  Returns ``(Q, params)``: ``Q`` the dequantised matrix in ``W``'s
+    dtype, ``params`` with ``scale`` / ``zero`` (fp32, one per column) and ``maxq``.
+    """
+    if use_fp64:
+        raise NotImplementedError("use_fp64=True is not available on the HIP path")
+    Wt = _float_dev(W)
+    if Wt.dim() != 2:
+        raise ValueError("W must be a 2-D matrix [K, N]")
+    orig_type = Wt.dtype
+    K, Nc = Wt.shape
+    if block_size < 1 or block_size > 128 or K % block_size != 0:
+        raise ValueError(f"block_size={block_size} must divide K={K} and be at most 128")
+    W32 = Wt.to(torch.float32)
+    if W32.data_ptr() == Wt.data_ptr():
+        W32 = W32.clone()              # the loop consumes its working copy
+    quantize_params = get_col_quantize_params(W32)
+    H = accumulate_H(xs, use_fp64=use_fp64)
+    if H.shape[0] != K:
+        raise ValueError(f"calibration feature dim {H.shape[0]} != K={K}")
+
+    perm = None
+    if actorder:
+        W32, H, perm = _permute(W32, H)
+
+    W32, Hinv, any_nan = _damp_and_invert(W32, H, damping)
+    if any_nan:
+        xs_nan = any(bool(torch.isnan(_float_dev(x)).any()) for x in xs)
+        raise ValueError(f"NaN when computing Hinv. Features NaN?: {xs_nan}")
+
+    Q, _ = _solve(W32, Hinv, quantize_params, block_size, orig_type)
+    if perm is not None:
+        Q = _unpermute(Q, perm)
+    return Q, quantize_params
+
+
+# ------------------------------------------------------------------------------- codec
+def _view3(shape, axis):
+    if axis < 0 or axis >= len(shape):
+        raise ValueError(f"Axis {axis} is out of bounds for array of dimension {len(shape)}")
+    outer = int(np.prod(shape[:axis], dtype=np.int64)) if axis > 0 else 1
+    inner = int(np.prod(shape[axis + 1:], dtype=np.int64)) if axis + 1 < len(shape) else 1
+    return outer, int(shape[axis]), inner
+
+
+def pack_along_axis(axis, w):
+    """``byte[j] = c[2j] | c[2j+1] << 4`` along ``axis`` (reference ``gptq.py:237-249, 265-283``)."""
+    lib = N.load()
+    w = _dev(w)
+    if w.dtype not in (torch.uint8, torch.int8, torch.int32, torch.int64):
+        w = w.to(torch.int32)
+    outer, alen, inner = _view3(w.shape, axis)
+    if alen % 2:
+        raise ValueError("the packed axis must have even length")
+    shape = list(w.shape)
+    shape[axis] = alen // 2
+    out = torch.empty(shape, dtype=torch.uint8, device=w.device)
+    N.check(lib.gptq_hip_pack_int4(_stream(), _ptr(w), w.element_size(), outer, alen, inner,
+                                   _ptr(out)), "pack_int4")
+    return out
+
+
+def unpack_along_axis(axis, w):
+    """Inverse of :func:`pack_along_axis` (reference ``gptq.py:251-263, 285-286``)."""
+    lib = N.load()
+    w = _dev(w, torch.uint8)
+    outer, plen, inner = _view3(w.shape, axis)
+    shape = list(w.shape)
+    shape[axis] = plen * 2
+    out = torch.empty(shape, dtype=torch.uint8, device=w.device)
+    N.check(lib.gptq_hip_unpack_int4(_stream(), _ptr(w), outer, plen, inner, _ptr(out)),
+            "unpack_int4")
+    return out
+
+
+def _pack(w_int):
+    assert len(w_int.shape) == 1
+    return pack_along_axis(0, w_int)
+
+
+def _unpack(packed):
+    assert len(packed.shape) == 1
+    return unpack_along_axis(0, packed)
+
+
+def pack_rowwise(w):
+    return pack_along_axis(1, w)
+
+
+def pack_colwise(w):
+    return pack_along_axis(0, w)
+
+
+def unpack_rowwise(w):
+    return unpack_along_axis(1, w)
+
+
+def unpack_colwise(w):
+    return unpack_along_axis(0, w)
+
+
+def pack_matrix(Q, params, contraction_axis=0):
+    """Dequantised floats -> integer codes -> packed container (reference ``gptq.py:214-228``)."""
+    lib = N.load()
+    Qt = _float_dev(Q)
+    scale = _dev(params["scale"])
+    zero = _dev(params["zero"])
+    outer, alen, inner = _view3(Qt.shape, contraction_axis)
+    if alen % 2:
+        raise ValueError("the contraction axis must have even length")
+    if scale.numel() != outer * inner or zero.numel() != outer * inner:
+        raise ValueError("scale/zero must have the shape of Q without the contraction axis")
+    shape = list(Qt.shape)
+    shape[contraction_axis] = alen // 2
+    packed = torch.empty(shape, dtype=torch.uint8, device=Qt.device)
+    N.check(lib.gptq_hip_quantize_pack(
+        _stream(), _ptr(Qt), _DT[Qt.dtype], outer, alen, inner,
+        _ptr(scale.to(torch.float32).contiguous()), _ptr(zero.to(torch.float32).contiguous()),
+        _ptr(packed)), "quantize_pack")
+    return QuantizedMatrix(int_weight=packed, zero=zero, scale=scale,
+                           contraction_axis=contraction_axis)
+
+
+def unpack_matrix(weight):
+    """Dense ``(code - zero) * scale`` in ``zero.dtype`` (reference ``gptq.py:230-235``)."""
+    lib = N.load()
+    iw = _dev(weight.int_weight, torch.uint8)
+    zero = _float_dev(weight.zero)
+    scale = _float_dev(weight.scale).to(zero.dtype)
+    outer, plen, inner = _view3(iw.shape, weight.contraction_axis)
+    if zero.numel() != outer * inner or scale.numel() != outer * inner:
+        raise ValueError("scale/zero must have the shape of the matrix without the contraction axis")
+    shape = list(iw.shape)
+    shape[weight.contraction_axis] = plen * 2
+    out = torch.empty(shape, dtype=zero.dtype, device=iw.device)
+    N.check(lib.gptq_hip_dequant(_stream(), _ptr(iw), outer, plen, inner, _ptr(zero), _ptr(scale),
+                                 _DT[zero.dtype], _ptr(out)), "dequant")
+    return out

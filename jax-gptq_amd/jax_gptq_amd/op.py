@@ -1,0 +1,84 @@
+"""Quantized-matmul operator: host-side mirror of the reference's ``jax_gptq/op.py``.
+
+``quantized_matmul(x, quantized_matrix, transpose_b=False)`` flattens the leading
+dimensions of ``x``, launches the packed-int4 HIP kernel (the counterpart of the
+``jt.triton_call`` at ``op.py:46-63``) and restores the shape.  Like the reference's
+``custom_vjp`` (``op.py:71-81``) it is differentiable with respect to ``x`` only: the
+backward pass is the same operator with ``transpose_b`` flipped.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _native as N
+from .gptq import _DT, _float_dev, _dev, _ptr, _stream, _ws
+
+
+def _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b):
+    lib = N.load()
+    leading_dims = None
+    if x.dim() > 2:
+        leading_dims = x.shape[:-1]
+        x = x.reshape(-1, x.shape[-1])
+    elif x.dim() == 1:
+        raise ValueError("x must have at least 2 dimensions")
+    x = x.contiguous()
+    M, K = x.shape
+    if int_weight.dim() != 2:
+        raise ValueError("quantized_matmul needs a 2-D packed matrix (contraction axis 0)")
+    R, C = int_weight.shape
+    if transpose_b:
+        K2, out_n = C, 2 * R
+    else:
+        K2, out_n = 2 * R, C
+    assert K == K2, f"Inner dim mismatch: {K} != {K2}"
+    if zero.dtype != scale.dtype:
+        scale = scale.to(zero.dtype)
+    out = torch.empty((M, out_n), dtype=x.dtype, device=x.device)
+    ws = _ws(lib.gptq_hip_qmatmul_workspace_bytes(M, R, C, int(transpose_b)))
+    N.check(lib.gptq_hip_qmatmul(_stream(), _ptr(x), _DT[x.dtype], M, _ptr(int_weight), R, C,
+                                 _ptr(zero), _ptr(scale), _DT[zero.dtype], int(transpose_b),
+                                 _ptr(out), _ptr(ws), ws.numel()), "qmatmul")
+    if leading_dims is not None:
+        out = out.reshape(tuple(leading_dims) + (out_n,))
+    return out
+
+
+class _QuantizedMatmulFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, int_weight, zero, scale, transpose_b):
+        ctx.save_for_backward(int_weight, zero, scale)
+        ctx.transpose_b = transpose_b
+        return _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b)
+
+    @staticmethod
+    def backward(ctx, y_bar):
+        int_weight, zero, scale = ctx.saved_tensors
+        x_bar = _quantized_matmul_raw(y_bar.contiguous(), int_weight, zero, scale,
+                                      not ctx.transpose_b)
+        return x_bar, None, None, None, None
+
+
+def _quantized_matmul(x, quantized_matrix, transpose_b):
+    x = _float_dev(x)
+    if getattr(quantized_matrix, "contraction_axis", 0) != 0:
+        raise ValueError("quantized_matmul needs contraction_axis == 0")
+    iw = _dev(quantized_matrix.int_weight, torch.uint8)
+    zero = _float_dev(quantized_matrix.zero)
+    scale = _float_dev(quantized_matrix.scale)
+    if x.requires_grad:
+        return _QuantizedMatmulFn.apply(x, iw, zero, scale, bool(transpose_b))
+    return _quantized_matmul_raw(x, iw, zero, scale, bool(transpose_b))
+
+
+def quantized_matmul(x, quantized_matrix, transpose_b=False):
+    """``x @ dequant(W)`` (``transpose_b``: ``x @ dequant(W).T``), reference ``op.py:11-14``."""
+    return _quantized_matmul(x, quantized_matrix, transpose_b)
+
+
+def qmatmul_fwd(x, quantized_matrix, transpose_b):
+    return _quantized_matmul(x, quantized_matrix, transpose_b), quantized_matrix
+
+
+def qmatmul_bwd(transposed, quantized_matrix, y_bar):
+    return _quantized_matmul(y_bar, quantized_matrix, transpose_b=not transposed), None

@@ -1,0 +1,67 @@
+"""GPU parity of the Hessian accumulation (fp32 MFMA) against the closed form and the oracle."""
+import numpy as np
+import pytest
+
+from helpers import to_np
+from oracle import gptq_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def G():
+    import jax_gptq_amd.gptq as g
+    return g
+
+
+def _closed_form(xs):
+    flat = np.concatenate([np.asarray(x, dtype=np.float64).reshape(-1, x.shape[-1]) for x in xs])
+    return flat.T @ flat / flat.shape[0]
+
+
+# tolerance: fp32 accumulation of n products of O(1) numbers; entries are O(1) after /n
+TOL = 2e-5
+
+
+@pytest.mark.parametrize("rows,K,nb", [(37, 256, 20), (2048, 768, 1), (512, 768, 3), (33, 100, 4),
+                                       (5, 130, 2), (300, 1, 1), (1, 384, 1)])
+def test_accumulate_H_closed_form(G, rows, K, nb):
+    rng = np.random.default_rng(9876)
+    xs = [rng.standard_normal((rows, K)).astype(np.float32) for _ in range(nb)]
+    H = to_np(G.accumulate_H(xs))
+    ref = _closed_form(xs)
+    assert H.shape == (K, K) and H.dtype == np.float32
+    assert np.array_equal(H, H.T)
+    assert np.abs(H - ref).max() < TOL * max(1.0, np.abs(ref).max())
+    orc = O.accumulate_H(xs)
+    assert np.abs(H - orc).max() < 2 * TOL * max(1.0, np.abs(ref).max())
+
+
+def test_accumulate_H_ragged_and_3d_batches(G):
+    rng = np.random.default_rng(1)
+    xs = [rng.standard_normal((3, 11, 96)).astype(np.float32),
+          rng.standard_normal((7, 96)).astype(np.float32) + 2.0,
+          rng.standard_normal((129, 96)).astype(np.float32)]
+    H = to_np(G.accumulate_H(xs))
+    ref = _closed_form(xs)
+    assert np.abs(H - ref).max() < TOL * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("dt", ["float16", "bfloat16"])
+def test_accumulate_H_half_inputs(G, dt):
+    import torch
+    rng = np.random.default_rng(2)
+    tdt = getattr(torch, dt)
+    xs_t = [torch.from_numpy(rng.standard_normal((200, 264)).astype(np.float32)).to(tdt)
+            for _ in range(3)]
+    H = to_np(G.accumulate_H(xs_t))
+    ref = _closed_form([x.float().numpy() for x in xs_t])   # the inputs as rounded
+    assert np.abs(H - ref).max() < TOL * np.abs(ref).max()
+
+
+def test_accumulate_H_zero_feature_is_exact_zero(G):
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((64, 160)).astype(np.float32)
+    x[:, 5] = 0
+    H = to_np(G.accumulate_H([x]))
+    assert np.all(H[5] == 0) and np.all(H[:, 5] == 0)

@@ -1,0 +1,123 @@
+"""GPU parity of the packed-int4 matmul (forward and transposed) against the oracle.
+
+Tolerance (task statement): atol 1e-2, rtol 1e-3 against the fp32 dense product.
+"""
+import numpy as np
+import pytest
+
+from helpers import to_np
+from oracle import gptq_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+ATOL, RTOL = 1e-2, 1e-3
+
+
+@pytest.fixture(scope="module")
+def OP():
+    import jax_gptq_amd.op as op
+    return op
+
+
+def _matrix(seed, K, N, zs_dtype=np.float32):
+    rng = np.random.default_rng(seed)
+    codes = rng.integers(0, 16, (K, N)).astype(np.uint8)
+    scale = rng.uniform(0.001, 0.01, N).astype(zs_dtype)
+    zero = rng.integers(0, 16, N).astype(zs_dtype)
+    return O.QuantizedMatrix(O.pack_colwise(codes), zero, scale)
+
+
+def _check(got, x, qm, transpose):
+    dense = ((O.unpack_colwise(qm.int_weight).astype(np.float64) - qm.zero.astype(np.float64)[None])
+             * qm.scale.astype(np.float64)[None])
+    ref = x.astype(np.float64) @ (dense.T if transpose else dense)
+    got = to_np(got).astype(np.float64)
+    assert got.shape == ref.shape
+    err = np.abs(got - ref)
+    # fp16 rounding of the result (2^-11 relative) is part of the operator's definition
+    tol = ATOL + RTOL * np.abs(ref)
+    assert np.all(err <= tol), f"max err {err.max():.3e} at |ref|={np.abs(ref).flat[err.argmax()]:.3e}"
+
+
+# shapes of the reference's test_kernel.py:13 plus the decode shapes of the benchmark config
+SHAPES = [(137, 909, 256), (32, 1024, 2048), (37, 32000, 5120), (1, 11008, 4096), (16, 4096, 11008),
+          (128, 11008, 4096), (3, 130, 66), (1, 64, 2)]
+
+
+@pytest.mark.parametrize("transpose", [False, True])
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_qmatmul_fp16(OP, M, N, K, transpose):
+    qm = _matrix(M + N + K, K, N, np.float16)
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((M, N if transpose else K)) * (0.05 if transpose else 1.0)).astype(np.float16)
+    got = OP.quantized_matmul(x, qm, transpose_b=transpose)
+    assert to_np(got).dtype == np.float16
+    _check(got, x.astype(np.float32), qm, transpose)
+    ref = O.quantized_matmul(x, qm, transpose_b=transpose)
+    assert np.allclose(to_np(got).astype(np.float32), ref.astype(np.float32), atol=ATOL, rtol=2 * RTOL)
+
+
+@pytest.mark.parametrize("transpose", [False, True])
+@pytest.mark.parametrize("M,N,K", [(137, 909, 256), (32, 1024, 2048), (5, 192, 384)])
+def test_qmatmul_fp32_x_and_params(OP, M, N, K, transpose):
+    qm = _matrix(M * 3 + N, K, N, np.float32)
+    rng = np.random.default_rng(6)
+    x = (rng.standard_normal((M, N if transpose else K)) * (0.05 if transpose else 1.0)).astype(np.float32)
+    got = OP.quantized_matmul(x, qm, transpose_b=transpose)
+    assert to_np(got).dtype == np.float32
+    _check(got, x, qm, transpose)
+
+
+def test_qmatmul_bf16_x(OP):
+    import torch
+    qm = _matrix(77, 512, 384, np.float32)
+    x = torch.randn((9, 512), generator=torch.Generator().manual_seed(0)).to(torch.bfloat16)
+    got = OP.quantized_matmul(x, qm)
+    assert got.dtype == torch.bfloat16
+    dense = O.unpack_matrix(qm)
+    ref = x.float().numpy() @ dense
+    assert np.allclose(to_np(got), ref, atol=3e-2, rtol=1e-2)    # bf16 result: 2^-8 relative
+
+
+def test_qmatmul_leading_dims_and_errors(OP):
+    qm = _matrix(8, 256, 192)
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((2, 3, 5, 256)).astype(np.float32)
+    got = OP.quantized_matmul(x, qm)
+    assert tuple(got.shape) == (2, 3, 5, 192)
+    _check(to_np(got).reshape(-1, 192), x.reshape(-1, 256), qm, False)
+    with pytest.raises(AssertionError):
+        OP.quantized_matmul(x[..., :-2], qm)
+    with pytest.raises(AssertionError):
+        OP.quantized_matmul(x, qm, transpose_b=True)
+
+
+def test_qmatmul_gradient_wrt_x(OP):
+    """custom-VJP counterpart (reference op.py:71-81): grad wrt x is y_bar @ dequant(W)^T."""
+    import torch
+    qm = _matrix(9, 256, 128)
+    dense = O.unpack_matrix(qm)
+    x = torch.randn((6, 256), generator=torch.Generator().manual_seed(1)).cuda().requires_grad_(True)
+    y = OP.quantized_matmul(x, qm)
+    y[3].sum().backward()
+    ref = np.zeros((6, 256), np.float32)
+    ref[3] = dense.sum(axis=1)
+    assert np.allclose(to_np(x.grad), ref, atol=1e-1)      # reference tests.py:186 uses atol 1e-1
+    assert np.allclose(to_np(x.grad), ref, atol=ATOL, rtol=RTOL)
+
+
+def test_qmatmul_after_gptq_matches_dense(OP):
+    """End to end as in the reference's test_kernel.py: solve, pack, multiply."""
+    import jax_gptq_amd.gptq as G
+    rng = np.random.default_rng(4)
+    M, N, K = 137, 909, 256
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    W = rng.standard_normal((K, N)).astype(np.float32)
+    quant_w, params = G.gptq(W, [x])
+    packed = G.pack_matrix(quant_w, params)
+    for transpose in (False, True):
+        inp = rng.standard_normal((M, N)).astype(np.float32) if transpose else x
+        ret = to_np(OP.quantized_matmul(inp, packed, transpose_b=transpose))
+        qw = to_np(quant_w)
+        expected = inp @ (qw.T if transpose else qw)
+        assert np.mean(np.abs(ret - expected)) < 3e-2        # reference test_kernel.py:41
