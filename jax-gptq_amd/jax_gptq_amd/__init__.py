@@ -1,16 +1,11 @@
 """MI355X-native GPTQ per-layer solve and packed-int4 matmul.
 
-Host-side mirror of ``jax_gptq`` (``gptq``, ``accumulate_H``, ``pack_matrix`` /
-``unpack_matrix``, ``QuantizedMatrix``, ``quantized_matmul``) over hand-written HIP
-kernels for gfx950, reached through the C ABI in ``include/gptq_hip.h``.
+Host-side mirror of ``jax_gptq`` over hand-written HIP kernels for gfx950, reached through
+the C ABI in ``include/gptq_hip.h``.  As in the reference, the solve lives in the
+``gptq`` submodule (``from jax_gptq_amd.gptq import gptq, accumulate_H, pack_matrix, ...``)
+and the operator in ``op`` (``from jax_gptq_amd.op import quantized_matmul``).
 """
-from .gptq import (QuantizedMatrix, accumulate_H, get_col_quantize_params, get_quantize_params,
-                   gptq, pack_colwise, pack_matrix, pack_rowwise, quant_matrix_shape,
-                   unpack_colwise, unpack_matrix, unpack_rowwise)
-from .op import quantized_matmul
+from . import gptq, op, utils  # noqa: F401  (submodules, as in the reference's layout)
+from .gptq import QuantizedMatrix
 
-__all__ = [
-    "QuantizedMatrix", "accumulate_H", "get_col_quantize_params", "get_quantize_params", "gptq",
-    "pack_colwise", "pack_matrix", "pack_rowwise", "quant_matrix_shape", "unpack_colwise",
-    "unpack_matrix", "unpack_rowwise", "quantized_matmul",
-]
+__all__ = ["QuantizedMatrix", "gptq", "op", "utils"]

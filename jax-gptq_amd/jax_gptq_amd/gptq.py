@@ -252,10 +252,12 @@ def _process_block(W, Hinv, start, quantize_params, block_size):
     q = torch.empty((block_size, Nc), dtype=torch.float32, device=W.device)
     err = torch.empty((block_size, Nc), dtype=torch.float32, device=W.device)
     lblk = Hinv[start:, start:]
+    # named locals: the tensors must stay alive until the launch has been enqueued
+    scale = _dev(quantize_params["scale"], torch.float32)
+    zero = _dev(quantize_params["zero"], torch.float32)
     N.check(lib.gptq_hip_process_block(
         _stream(), _ptr(blk), Nc, ctypes.c_void_p(lblk.data_ptr()), Hinv.shape[1], block_size,
-        _ptr(_dev(quantize_params["scale"], torch.float32)),
-        _ptr(_dev(quantize_params["zero"], torch.float32)), int(quantize_params["maxq"]),
+        _ptr(scale), _ptr(zero), int(quantize_params["maxq"]),
         _ptr(q), N.F32, ctypes.c_void_p(0), _ptr(err)), "process_block")
     return q, err
 
@@ -390,9 +392,10 @@ def pack_matrix(Q, params, contraction_axis=0):
     shape = list(Qt.shape)
     shape[contraction_axis] = alen // 2
     packed = torch.empty(shape, dtype=torch.uint8, device=Qt.device)
+    scale32 = scale.to(torch.float32).contiguous()     # kept alive across the launch
+    zero32 = zero.to(torch.float32).contiguous()
     N.check(lib.gptq_hip_quantize_pack(
-        _stream(), _ptr(Qt), _DT[Qt.dtype], outer, alen, inner,
-        _ptr(scale.to(torch.float32).contiguous()), _ptr(zero.to(torch.float32).contiguous()),
+        _stream(), _ptr(Qt), _DT[Qt.dtype], outer, alen, inner, _ptr(scale32), _ptr(zero32),
         _ptr(packed)), "quantize_pack")
     return QuantizedMatrix(int_weight=packed, zero=zero, scale=scale,
                            contraction_axis=contraction_axis)
