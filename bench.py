@@ -80,30 +80,44 @@ def one_layer(G, W, xs, timers=None):
     return packed
 
 
-def bench_qmatmul(OP, G, reps=200):
-    """Packed-int4 matmul against the HBM roofline.  The packed weight (22.5 MB) would fit
-    the 256 MB Infinity Cache, so the timed loop rotates over 24 independent copies."""
+def bench_qmatmul(reps=240):
+    """Packed-int4 matmul against the HBM roofline, called through the C ABI with
+    preallocated buffers (the Python operator adds ~10 us of host time per call, which
+    would hide a ~10 us kernel).  The packed weight (22.5 MB) would fit the 256 MB Infinity
+    Cache, so the timed loop rotates over 24 independent copies (540 MB)."""
+    import ctypes
     import torch
+    from jax_gptq_amd import _native
+    lib = _native.load()
     out = []
     g = torch.Generator(device="cuda")
     g.manual_seed(1)
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     for (K, N) in ((4096, 11008), (11008, 4096)):
         copies = 24
-        qms = []
-        for _ in range(copies):
-            iw = torch.randint(0, 256, (K // 2, N), generator=g, device="cuda", dtype=torch.uint8)
-            scale = (0.001 + 0.009 * torch.rand(N, generator=g, device="cuda")).to(torch.float16)
-            zero = torch.randint(0, 16, (N,), generator=g, device="cuda").to(torch.float16)
-            qms.append(G.QuantizedMatrix(iw, zero, scale))
+        iws = [torch.randint(0, 256, (K // 2, N), generator=g, device="cuda", dtype=torch.uint8)
+               for _ in range(copies)]
+        scale = (0.001 + 0.009 * torch.rand(N, generator=g, device="cuda")).to(torch.float16)
+        zero = torch.randint(0, 16, (N,), generator=g, device="cuda").to(torch.float16)
         for M in (1, 16, 128):
             x = torch.randn((M, K), generator=g, device="cuda").to(torch.float16)
+            y = torch.empty((M, N), dtype=torch.float16, device="cuda")
+            ws = torch.zeros(max(lib.gptq_hip_qmatmul_workspace_bytes(M, K // 2, N, 0), 256),
+                             dtype=torch.uint8, device="cuda")
+
+            def call(i):
+                rc = lib.gptq_hip_qmatmul(st, x.data_ptr(), _native.F16, M, iws[i % copies].data_ptr(),
+                                          K // 2, N, zero.data_ptr(), scale.data_ptr(), _native.F16, 0,
+                                          y.data_ptr(), ws.data_ptr(), ws.numel())
+                assert rc == 0, rc
+
             for i in range(copies):
-                OP.quantized_matmul(x, qms[i])
+                call(i)
             torch.cuda.synchronize()
             e0, e1 = _events(2)
             e0.record()
             for i in range(reps):
-                OP.quantized_matmul(x, qms[i % copies])
+                call(i)
             e1.record()
             torch.cuda.synchronize()
             us = e0.elapsed_time(e1) * 1e3 / reps
@@ -159,7 +173,6 @@ def main():
 
     import torch
     import jax_gptq_amd.gptq as G
-    import jax_gptq_amd.op as OP
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
 
@@ -203,7 +216,7 @@ def main():
         "phases_ms": phases,
     }
     if not args.no_qmatmul:
-        qm = bench_qmatmul(OP, G)
+        qm = bench_qmatmul()
         result["qmatmul"] = qm
         m1 = [r for r in qm if r["M"] == 1 and r["K"] == 4096][0]
         result["int4_matmul_hbm_gbps"] = m1["GBps"]

@@ -142,7 +142,10 @@ int gptq_hip_dequant(void *stream, const uint8_t *packed, int64_t outer,
  *   transpose_b = 0: Kx = 2R, out [M, C]  = x @ ((code - zero) * scale)
  *   transpose_b = 1: Kx = C,  out [M, 2R] = x @ ((code - zero) * scale)^T
  * fp32 accumulation; the result is rounded to fp16 and then converted to x_dtype, as
- * op.py:43,66-68 does.  ws: gptq_hip_qmatmul_workspace_bytes(M, R, C, transpose_b). */
+ * op.py:43,66-68 does.  ws: gptq_hip_qmatmul_workspace_bytes(M, R, C, transpose_b) bytes.
+ * The workspace begins with arrival counters of the split-K reduction: it must be
+ * ZERO-FILLED before its first use; every call leaves the counters zero again, so one
+ * buffer can serve any sequence of calls that do not overlap in time. */
 size_t gptq_hip_qmatmul_workspace_bytes(int64_t M, int64_t R, int64_t C, int transpose_b);
 int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
                      int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype,

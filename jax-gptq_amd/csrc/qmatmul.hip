@@ -55,6 +55,323 @@ __global__ __launch_bounds__(TPB) void qmm_bwd_simple(const TX *x, int64_t M, co
   }
 }
 
+// ---------------------------------------------------------------------------- MFMA path
+// Forward, fp16 activations, C % 16 == 0.  One workgroup owns a strip of 256 output
+// channels and a slice of NW * SPW * 16 packed rows (NW wavefronts, SPW MFMA k-steps of 16
+// packed rows each).  A wavefront first issues its (small, L2-resident) activation loads,
+// then ALL its weight loads in one burst (SPW * 4 loads of 16 B per lane), so that the
+// whole matrix is in flight at once; it dequantises in registers as the rows arrive and
+// feeds v_mfma_f32_16x16x32_f16:
+//   A = activations  (lane: row m = l % 16, eight k slots of lane group g = l / 16)
+//   B = weights      (lane: channel 16*(l % 16) + t for t = 0..15, same eight k slots)
+// Lane group g owns the packed rows 16*s + 4*i + g (i = 0..3) of k-step s, i.e. the k slots
+// [2r0, 2r1, 2r0+1, 2r1+1, 2r2, 2r3, 2r2+1, 2r3+1]; both operands are built in that order.
+// Nibbles become fp16 with three VALU operations per four codes: one byte permute and two
+// and-or with 0x6400 (fp16 1024), giving 1024 + code for even k and 1024 + 16*code for odd
+// k.  Odd-k activations enter the MFMA divided by 16 (exact in fp16 but for subnormals), so
+//   acc = sum_k x*code + 1024 * (sum_even x + sum_odd x/16)
+// and with the two activation sums (kept per lane in fp32) the epilogue computes
+//   out = scale * (acc - 1024*(se + so) - zero * (se + 16*so)),  se = sum_even x, so = sum_odd x/16.
+// No LDS or barrier is used before the final cross-wavefront reduction.
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int QSTRIP = 256;    // channels per workgroup
+
+__device__ __forceinline__ uint32_t u4_comp(const uint4 &v, int w) {
+  return w == 0 ? v.x : (w == 1 ? v.y : (w == 2 ? v.z : v.w));
+}
+
+__device__ __forceinline__ void dequant_pair(uint32_t da, uint32_t db, uint32_t sel,
+                                             uint32_t &lo, uint32_t &hi) {
+  // bytes of p: [7:0] = row a, [23:16] = row b.  lo = 1024 + code (even k), hi = 1024 + 16*code
+  // (odd k) as fp16 pairs; the offsets and the factor 16 are undone outside the MFMA.
+  const uint32_t p = __builtin_amdgcn_perm(db, da, sel);
+  lo = (p & 0x000F000Fu) | 0x64006400u;
+  hi = (p & 0x00F000F0u) | 0x64006400u;
+}
+
+// Workspace layout (only touched when the K range is split over S > 1 workgroups):
+//   [counters: QMM_COUNTER_BYTES, one int32 per (m-chunk, strip), zero between calls; the
+//    size is fixed so that no other region of an earlier call can alias a counter]
+//   [x1part:  (m-chunk, strip, split, 2, 16) fp32]   [part: (split, M, C) fp32]
+// The last workgroup to finish a strip (atomic ticket) sums the S partials in split order,
+// so the result does not depend on the arrival order, and resets the counter.
+constexpr int QMM_COUNTER_BYTES = 65536;
+constexpr int QMM_MAX_COUNTERS = QMM_COUNTER_BYTES / 4;
+
+struct QmmWs {
+  int32_t *counters;
+  float *x1part;
+  float *part;
+};
+
+template <int SPW, typename TZ>
+__global__ __launch_bounds__(SPW == 2 ? 1024 : 512) void qmm_fwd_mfma_kernel(
+    const __half *x, int M, int K, const uint8_t *pk, int R, int C, const TZ *zero,
+    const TZ *scale, __half *out, QmmWs ws, int S) {
+  extern __shared__ float red[];   // [wave][mrows][256] partial tiles, then [wave][2][16] x sums
+  __shared__ int s_last;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int nw = blockDim.x >> 6;
+  const int strip = blockIdx.x, split = blockIdx.y, m0 = blockIdx.z * 16;
+  const int mvalid = min(16, M - m0);
+  const int mrows = mvalid <= 4 ? 4 : 16;
+  const int r_wave = (split * nw + wave) * SPW * 16;
+  const int g = lane >> 4, l16 = lane & 15;
+
+  // ---- activation loads (k pairs 2r, 2r+1 of this lane's rows): small, L2 resident
+  uint32_t pr[SPW][4];
+  {
+    const __half *xr = x + (int64_t)(m0 + l16) * K;
+#pragma unroll
+    for (int s = 0; s < SPW; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = r_wave + s * 16 + 4 * i + g;
+        pr[s][i] = (l16 < mvalid && row < R) ? *reinterpret_cast<const uint32_t *>(xr + 2 * row) : 0u;
+      }
+  }
+  // ---- weight loads of this wavefront, all in flight
+  uint4 d[SPW][4];
+  const int col0 = strip * QSTRIP + 16 * l16;
+#pragma unroll
+  for (int s = 0; s < SPW; ++s)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = r_wave + s * 16 + 4 * i + g;
+      d[s][i] = (row < R && col0 < C)
+                    ? *reinterpret_cast<const uint4 *>(pk + (int64_t)row * C + col0)
+                    : make_uint4(0, 0, 0, 0);
+    }
+
+  // A operands: even-k slots hold x, odd-k slots hold x/16 (see above); per-lane fp32 sums of
+  // exactly the fp16 values the MFMA sees, then summed over the four lane groups
+  uint4 av[SPW];
+  float se = 0.f, so = 0.f;
+  const half2_t sixteenth = half2_t{(_Float16)0.0625f, (_Float16)0.0625f};
+#pragma unroll
+  for (int s = 0; s < SPW; ++s) {
+    av[s].x = __builtin_amdgcn_perm(pr[s][1], pr[s][0], 0x05040100u);  // {x[2r0],   x[2r1]}
+    av[s].z = __builtin_amdgcn_perm(pr[s][3], pr[s][2], 0x05040100u);
+    const half2_t o0 =
+        __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(pr[s][1], pr[s][0], 0x07060302u)) * sixteenth;
+    const half2_t o1 =
+        __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(pr[s][3], pr[s][2], 0x07060302u)) * sixteenth;
+    av[s].y = __builtin_bit_cast(uint32_t, o0);   // {x[2r0+1], x[2r1+1]} / 16
+    av[s].w = __builtin_bit_cast(uint32_t, o1);
+    const half2_t e0 = __builtin_bit_cast(half2_t, av[s].x), e1 = __builtin_bit_cast(half2_t, av[s].z);
+    se += ((float)e0[0] + (float)e0[1]) + ((float)e1[0] + (float)e1[1]);
+    so += ((float)o0[0] + (float)o0[1]) + ((float)o1[0] + (float)o1[1]);
+  }
+  se += __shfl_xor(se, 16);
+  se += __shfl_xor(se, 32);
+  so += __shfl_xor(so, 16);
+  so += __shfl_xor(so, 32);
+
+  float *slot = red + (size_t)wave * mrows * QSTRIP;
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    floatx4 acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < SPW; ++s) {
+      const half8_t a = __builtin_bit_cast(half8_t, av[s]);
+#pragma unroll
+      for (int tt = 0; tt < 8; ++tt) {
+        const int t = half * 8 + tt;
+        const int w = t >> 2, tb = t & 3;
+        const uint32_t sel = 0x0c000c00u | ((uint32_t)(4 + tb) << 16) | (uint32_t)tb;
+        uint4 bv;
+        dequant_pair(u4_comp(d[s][0], w), u4_comp(d[s][1], w), sel, bv.x, bv.y);
+        dequant_pair(u4_comp(d[s][2], w), u4_comp(d[s][3], w), sel, bv.z, bv.w);
+        const half8_t b = __builtin_bit_cast(half8_t, bv);
+        acc[tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[tt], 0, 0, 0);
+      }
+    }
+    // acc[tt][r] = tile[m = 4g + r][channel 16*l16 + half*8 + tt]
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = 4 * g + r;
+      if (m < mrows) {
+        float *dst = slot + m * QSTRIP + 16 * l16 + half * 8;
+        *reinterpret_cast<float4 *>(dst) = make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]);
+        *reinterpret_cast<float4 *>(dst + 4) = make_float4(acc[4][r], acc[5][r], acc[6][r], acc[7][r]);
+      }
+    }
+  }
+  float *xs = red + (size_t)nw * mrows * QSTRIP;   // [wave][2][16]
+  if (g == 0) { xs[wave * 32 + l16] = se; xs[wave * 32 + 16 + l16] = so; }
+  __syncthreads();
+
+  // epilogue value of one output from the accumulated tile sum v and the activation sums
+  auto finish = [&](float v, float e, float o, int n) -> __half {
+    const float z = to_f32(zero[n]);
+    return __float2half_rn(to_f32(scale[n]) * ((v - 1024.f * (e + o)) - z * (e + 16.f * o)));
+  };
+  const int n_items = mvalid * QSTRIP;
+  // x sums of this workgroup: [split][2][16] per (m-chunk, strip)
+  const int64_t x1base = (((int64_t)blockIdx.z * gridDim.x + strip) * S) * 32;
+  if (S == 1) {
+    for (int idx = tid; idx < n_items; idx += blockDim.x) {
+      const int m = idx >> 8, c = idx & 255, n = strip * QSTRIP + c;
+      if (n >= C) continue;
+      float v = 0.f, e = 0.f, o = 0.f;
+      for (int w = 0; w < nw; ++w) {
+        v += red[(w * mrows + m) * QSTRIP + c];
+        e += xs[w * 32 + m];
+        o += xs[w * 32 + 16 + m];
+      }
+      out[(int64_t)(m0 + m) * C + n] = finish(v, e, o, n);
+    }
+    return;
+  }
+  for (int idx = tid; idx < n_items; idx += blockDim.x) {
+    const int m = idx >> 8, c = idx & 255, n = strip * QSTRIP + c;
+    if (n >= C) continue;
+    float v = 0.f;
+    for (int w = 0; w < nw; ++w) v += red[(w * mrows + m) * QSTRIP + c];
+    // agent-scope write-through store: visible to every XCD once it has completed
+    __hip_atomic_store(&ws.part[((int64_t)split * M + m0 + m) * C + n], v, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (tid < 32 && (tid & 15) < mvalid) {
+    float x1 = 0.f;
+    for (int w = 0; w < nw; ++w) x1 += xs[w * 32 + tid];
+    __hip_atomic_store(&ws.x1part[x1base + (int64_t)split * 32 + tid], x1, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+  }
+  // Each thread waits for its own write-through stores, then the barrier orders all of them
+  // before the ticket.  (A device-wide fence here would write back / invalidate the whole
+  // L2 of the XCD, which costs tens of microseconds.)
+  __syncthreads();
+  if (tid == 0) {
+    int32_t *ctr = ws.counters + blockIdx.z * gridDim.x + strip;
+    const int ticket = atomicAdd(ctr, 1);
+    s_last = (ticket == S - 1);
+    if (ticket == S - 1)               // every other workgroup of this strip has arrived
+      __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (!s_last) return;
+  // Last workgroup of the strip: sum the S partials in split order.  Loads are agent-scope
+  // (never served from a stale line of this XCD's L2).  Every thread keeps all its outputs
+  // in registers and walks the splits in order, so that the loads of one split (and, through
+  // unrolling, of the next) are in flight together instead of one latency per output.
+  if (tid < 32) {
+    float a = 0.f;
+    for (int sp0 = 0; sp0 < S; sp0 += 8) {
+      float px[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        px[u] = __hip_atomic_load(&ws.x1part[x1base + (int64_t)min(sp0 + u, S - 1) * 32 + tid],
+                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (sp0 + u < S) a += px[u];
+    }
+    xs[tid] = a;     // [0..15] even-k sums, [16..31] odd-k sums, per row m
+  }
+  // n_items <= 4096; the workgroup size is fixed per instantiation (1024 or 512 threads)
+  constexpr int IT = (SPW == 2) ? 4 : 8;
+  float v[IT];
+#pragma unroll
+  for (int it = 0; it < IT; ++it) v[it] = 0.f;
+#pragma unroll 2
+  for (int sp = 0; sp < S; ++sp) {
+    float pv[IT];
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+      const int idx = tid + it * blockDim.x;
+      const int m = idx >> 8, n = strip * QSTRIP + (idx & 255);
+      pv[it] = (idx < n_items && n < C)
+                   ? __hip_atomic_load(&ws.part[((int64_t)sp * M + m0 + m) * C + n],
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                   : 0.f;
+    }
+#pragma unroll
+    for (int it = 0; it < IT; ++it) v[it] += pv[it];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int it = 0; it < IT; ++it) {
+    const int idx = tid + it * blockDim.x;
+    const int m = idx >> 8, n = strip * QSTRIP + (idx & 255);
+    if (idx < n_items && n < C) out[(int64_t)(m0 + m) * C + n] = finish(v[it], xs[m], xs[16 + m], n);
+  }
+}
+
+struct FwdPlan {
+  int nw, spw, S, strips, mch;
+  size_t lds_bytes, counter_bytes, x1_bytes, part_bytes, total_bytes;
+};
+
+FwdPlan fwd_plan(int64_t M, int64_t R, int64_t C) {
+  FwdPlan p;
+  p.strips = (int)ceil_div64(C, QSTRIP);
+  p.mch = (int)ceil_div64(M, 16);
+  // 512 packed rows per workgroup either way: 16 wavefronts x 8 KB (all resident, small
+  // tiles) for M <= 4, 8 wavefronts x 16 KB otherwise
+  if (M <= 4) { p.nw = 16; p.spw = 2; }
+  else { p.nw = 8; p.spw = 4; }
+  p.S = (int)ceil_div64(R, (int64_t)p.nw * p.spw * 16);
+  const int mrows = (M <= 4) ? 4 : 16;
+  p.lds_bytes = ((size_t)p.nw * mrows * QSTRIP + (size_t)p.nw * 32) * sizeof(float);
+  p.counter_bytes = QMM_COUNTER_BYTES;
+  p.x1_bytes = (size_t)round_up64((int64_t)p.strips * p.mch * p.S * 32 * sizeof(float), 256);
+  p.part_bytes = (size_t)p.S * M * C * sizeof(float);
+  p.total_bytes = p.S > 1 ? p.counter_bytes + p.x1_bytes + p.part_bytes : 0;
+  return p;
+}
+
+template <int SPW, typename TZ>
+int launch_fwd_mfma(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, const uint8_t *pk,
+                    int64_t R, int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
+  QmmWs ws;
+  char *base = reinterpret_cast<char *>(wsp);
+  ws.counters = reinterpret_cast<int32_t *>(base);
+  ws.x1part = reinterpret_cast<float *>(base + p.counter_bytes);
+  ws.part = reinterpret_cast<float *>(base + p.counter_bytes + p.x1_bytes);
+  auto kern = qmm_fwd_mfma_kernel<SPW, TZ>;
+  if (p.lds_bytes > 48 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)p.lds_bytes) != hipSuccess)
+    return GPTQ_HIP_ELAUNCH;
+  // at most QMM_MAX_COUNTERS (m-chunk, strip) pairs per launch
+  const int mch_per = QMM_MAX_COUNTERS / p.strips;
+  if (mch_per < 1) return GPTQ_HIP_EINVAL;
+  for (int c0 = 0; c0 < p.mch; c0 += mch_per) {
+    const int nch = min(mch_per, p.mch - c0);
+    const int64_t row0 = (int64_t)c0 * 16;
+    const int64_t rows = min((int64_t)nch * 16, M - row0);
+    const dim3 grid((unsigned)p.strips, (unsigned)p.S, (unsigned)nch);
+    // the kernel sees the sub-problem rows [row0, row0 + rows); launches are stream ordered,
+    // so they can share the workspace
+    hipLaunchKernelGGL(kern, grid, dim3(p.nw * 64), p.lds_bytes, st,
+                       (const __half *)x + row0 * 2 * R, (int)rows, (int)(2 * R), pk, (int)R,
+                       (int)C, (const TZ *)zero, (const TZ *)scale, (__half *)out + row0 * C, ws,
+                       p.S);
+    GPTQ_CHECK_LAUNCH();
+  }
+  return GPTQ_HIP_OK;
+}
+
+template <typename TZ>
+int launch_fwd_mfma_z(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, const uint8_t *pk,
+                      int64_t R, int64_t C, const void *zero, const void *scale, void *out,
+                      void *wsp) {
+  if (p.spw == 2) return launch_fwd_mfma<2, TZ>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
+  return launch_fwd_mfma<4, TZ>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
+}
+
+bool fwd_fast_ok(int x_dtype, int64_t M, int64_t R, int64_t C, const void *x, const uint8_t *pk) {
+  return x_dtype == GPTQ_HIP_F16 && C % 16 == 0 && M >= 1 && M <= 65535 * 16LL &&
+         (reinterpret_cast<uintptr_t>(pk) & 15) == 0 && (reinterpret_cast<uintptr_t>(x) & 3) == 0 &&
+         R < (1LL << 30) && C < (1LL << 30);
+}
+
 template <typename TX, typename TZ>
 int launch_simple(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
                   const void *zero, const void *scale, int transpose_b, void *out) {
@@ -92,18 +409,31 @@ int dispatch_z(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int6
 extern "C" {
 
 size_t gptq_hip_qmatmul_workspace_bytes(int64_t M, int64_t R, int64_t C, int transpose_b) {
-  (void)M; (void)R; (void)C; (void)transpose_b;
-  return 0;
+  if (transpose_b || M <= 0 || R <= 0 || C <= 0) return 0;
+  return fwd_plan(M, R, C).total_bytes;
 }
 
 int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
                      int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype,
                      int transpose_b, void *out, void *ws, size_t ws_bytes) {
-  (void)ws; (void)ws_bytes;
   if (M < 0 || R <= 0 || C <= 0) return GPTQ_HIP_EINVAL;
   if (M == 0) return GPTQ_HIP_OK;
   if (!x || !packed || !zero || !scale || !out) return GPTQ_HIP_EINVAL;
   hipStream_t st = as_stream(stream);
+  if (!transpose_b && fwd_fast_ok(x_dtype, M, R, C, x, packed)) {
+    const FwdPlan p = fwd_plan(M, R, C);
+    if (p.total_bytes && (!ws || ws_bytes < p.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+    switch (zs_dtype) {
+      case GPTQ_HIP_F32:
+        return launch_fwd_mfma_z<float>(st, p, x, M, packed, R, C, zero, scale, out, ws);
+      case GPTQ_HIP_F16:
+        return launch_fwd_mfma_z<__half>(st, p, x, M, packed, R, C, zero, scale, out, ws);
+      case GPTQ_HIP_BF16:
+        return launch_fwd_mfma_z<__hip_bfloat16>(st, p, x, M, packed, R, C, zero, scale, out, ws);
+      default:
+        return GPTQ_HIP_EDTYPE;
+    }
+  }
   switch (x_dtype) {
     case GPTQ_HIP_F32:
       return dispatch_z<float>(st, x, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out);

@@ -7,7 +7,8 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libgptq_hip.so")
+# GPTQ_HIP_LIBRARY selects another build of the same ABI (e.g. an instrumented one)
+LIB_PATH = os.environ.get("GPTQ_HIP_LIBRARY") or os.path.join(HERE, "libgptq_hip.so")
 
 F32, F16, BF16 = 0, 1, 2
 OK, EINVAL, EDTYPE, EWORKSPACE, ELAUNCH = 0, 1, 2, 3, 4

@@ -14,6 +14,21 @@ from . import _native as N
 from .gptq import _DT, _float_dev, _dev, _ptr, _stream, _ws
 
 
+# The matmul workspace starts with split-K arrival counters that must be zero when a call
+# starts; every call leaves them zero again.  One zero-initialised buffer per (device,
+# stream) is therefore kept and only ever grown.
+_WS_CACHE = {}
+
+
+def _qmm_workspace(nbytes, device):
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _WS_CACHE.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+        _WS_CACHE[key] = ws
+    return ws
+
+
 def _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b):
     lib = N.load()
     leading_dims = None
@@ -35,7 +50,7 @@ def _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b):
     if zero.dtype != scale.dtype:
         scale = scale.to(zero.dtype)
     out = torch.empty((M, out_n), dtype=x.dtype, device=x.device)
-    ws = _ws(lib.gptq_hip_qmatmul_workspace_bytes(M, R, C, int(transpose_b)))
+    ws = _qmm_workspace(lib.gptq_hip_qmatmul_workspace_bytes(M, R, C, int(transpose_b)), x.device)
     N.check(lib.gptq_hip_qmatmul(_stream(), _ptr(x), _DT[x.dtype], M, _ptr(int_weight), R, C,
                                  _ptr(zero), _ptr(scale), _DT[zero.dtype], int(transpose_b),
                                  _ptr(out), _ptr(ws), ws.numel()), "qmatmul")
