@@ -195,14 +195,24 @@ def main():
         one_layer(G, W, xs, timers)
     phases = {k: round(sum(v) / len(v), 3) for k, v in timers.items()}
     hess_ms = phases["hessian"]
-    flop_per_launch = 2.0 * ROWS * K_IN * K_IN            # one launch = one calibration batch
-    avg_launch_ms = hess_ms / N_BATCH
-    achieved = flop_per_launch / (avg_launch_ms * 1e-3) * 1e-12
-    roofline = {"kernel": "gemm_f32_kernel (X^T X, upper tiles)", "bound": "mfma",
+    # One launch covers all 128 batches; the phase time also contains the (tiny) slice
+    # reduction, the zero fill of H and the finalisation, which makes the figure conservative.
+    n_tokens = N_BATCH * ROWS
+    flop_per_launch = 2.0 * n_tokens * K_IN * K_IN          # the full GEMM the reference executes
+    tiles = (K_IN + 127) // 128
+    executed_flop = flop_per_launch * (tiles + 1) / (2 * tiles)   # upper 128x128 tiles only
+    achieved = flop_per_launch / (hess_ms * 1e-3) * 1e-12
+    executed = executed_flop / (hess_ms * 1e-3) * 1e-12
+    roofline = {"kernel": "syrk_kernel<float> (X^T X, fp32 MFMA, upper tiles)", "bound": "mfma",
                 "achieved": round(achieved, 2), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None,
-                "flop_per_launch": flop_per_launch, "avg_launch_ms": round(avg_launch_ms, 4),
-                "launches_per_step": N_BATCH}
+                "flop_per_launch": flop_per_launch, "avg_launch_ms": round(hess_ms, 4),
+                "launches_per_step": 1,
+                "executed_tflops": round(executed, 2),
+                "executed_frac": round(executed / FP32_MFMA_PEAK_TFLOPS, 4),
+                "note": "achieved counts the algorithmic 2*n*K^2 flop; the kernel computes only the "
+                        "upper tiles of the symmetric result (executed_*), which is what MFMA "
+                        "utilisation counters see"}
 
     result = {
         "metric": "GPTQ s/layer @4096x11008", "value": round(sec_per_step, 5), "unit": "s/layer",

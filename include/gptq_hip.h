@@ -58,12 +58,17 @@ int gptq_hip_col_params(void *stream, const void *W, int w_dtype, int64_t K, int
  * gptq_hip_hessian_accumulate adds sum_b X_b^T X_b to the UPPER triangle (128x128
  * tile granularity) of H [K, K] fp32.  x_ptrs / x_rows are HOST arrays of
  * n_batches device pointers / row counts; batch b is [x_rows[b], K] row-major,
- * contiguous.  The running mean of the reference cancels algebraically
- * (H = sum X^T X / n), so none is kept.
+ * contiguous.  All batches of one call are reduced in one launch (in registers), so
+ * passing the whole calibration set at once is the fast path; one batch per call
+ * reproduces the reference's streaming use.  The running mean of the reference cancels
+ * algebraically (H = sum X^T X / n), so none is kept.
+ * ws: gptq_hip_hessian_accumulate_workspace_bytes(K) bytes (0 for large K).
  * gptq_hip_hessian_finalize multiplies by 1/n_samples and mirrors the upper
  * triangle into the lower one, giving the full symmetric H the reference returns. */
+size_t gptq_hip_hessian_accumulate_workspace_bytes(int64_t K);
 int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const int64_t *x_rows,
-                                int n_batches, int x_dtype, int64_t K, float *H);
+                                int n_batches, int x_dtype, int64_t K, float *H, void *ws,
+                                size_t ws_bytes);
 int gptq_hip_hessian_finalize(void *stream, float *H, int64_t K, double n_samples);
 
 /* ---- dead features, damping, Cholesky factor of the inverse -----------------------

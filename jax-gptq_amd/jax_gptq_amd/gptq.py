@@ -122,6 +122,7 @@ def _accumulate_H_step(H, running_mean, n_samples, batch):
 def _hessian_accumulate(H, batches):
     lib = N.load()
     K = H.shape[0]
+    ws = _ws(lib.gptq_hip_hessian_accumulate_workspace_bytes(K))
     for lo in range(0, len(batches), _MAX_BATCHES_PER_CALL):
         chunk = batches[lo:lo + _MAX_BATCHES_PER_CALL]
         dts = {b.dtype for b in chunk}
@@ -134,7 +135,8 @@ def _hessian_accumulate(H, batches):
         ptrs = (ctypes.c_void_p * nb)(*[b.data_ptr() for b in chunk])
         rows = (ctypes.c_int64 * nb)(*[b.shape[0] for b in chunk])
         N.check(lib.gptq_hip_hessian_accumulate(_stream(), ptrs, rows, nb, _DT[chunk[0].dtype], K,
-                                                _ptr(H)), "hessian_accumulate")
+                                                _ptr(H), _ptr(ws), ws.numel()),
+                "hessian_accumulate")
 
 
 def accumulate_H(xs, use_fp64=False):
