@@ -101,11 +101,11 @@ int gptq_hip_solve(void *stream, float *W, int64_t K, int64_t N, const float *L,
                    int q_dtype, uint8_t *codes, void *ws, size_t ws_bytes);
 
 /* One block of the loop: replaces _process_block (gptq.py:130-153).  Wblock points at
- * the first of the block's block_size rows of W [*, N] (rows of the block are used as
- * scratch and overwritten); Lblock points at L[start][start] (row stride ldl).  Outputs:
+ * the first of the block's block_size rows of W [*, N] (read only); Lblock points at
+ * L[start][start] (row stride ldl).  Outputs:
  * Qblock / codes_block [block_size, N] (either may be NULL) and errors [block_size, N]
  * fp32, the (w - q) / L_ii rows that the lazy update consumes. */
-int gptq_hip_process_block(void *stream, float *Wblock, int64_t N, const float *Lblock,
+int gptq_hip_process_block(void *stream, const float *Wblock, int64_t N, const float *Lblock,
                            int64_t ldl, int block_size, const float *scale, const float *zero,
                            int maxq, void *Qblock, int q_dtype, uint8_t *codes_block,
                            float *errors);

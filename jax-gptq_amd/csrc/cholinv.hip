@@ -4,20 +4,20 @@
 // The reference obtains L in three LAPACK steps (factor, solve against I, factor again,
 // about 8/3 K^3 flop).  Here L is obtained in two (about 2/3 K^3 flop):
 //   1. H = M^T M with M lower triangular ("reverse" Cholesky, processed from the last
-//      128-block upwards so that every trailing update is an X^T X form);
+//      diagonal block upwards so that every trailing update is an X^T X form);
 //   2. L = M^-1, by pairwise merging of inverted diagonal blocks:
 //      inv([[A,0],[C,B]]) = [[A^-1,0],[-B^-1 C A^-1, B^-1]].
 // H^-1 = M^-1 M^-T = L L^T with L lower triangular and a positive diagonal, which is the
 // unique Cholesky factor the reference computes.
 //
-// All O(K^3) work runs on the fp32 MFMA GEMM; only the 128x128 diagonal blocks are
+// All O(K^3) work runs on the fp32 MFMA GEMM; only the NB x NB diagonal blocks are
 // factorised and inverted inside one workgroup, in LDS.
 #include "common.h"
 #include "gemm_f32.h"
 
 namespace {
 
-constexpr int NB = 128;
+constexpr int NB = 64;
 
 // ---------------------------------------------------------------- diag / damping prep
 // One workgroup.  dead_i = (H_ii == 0) -> H_ii = 1; mean over the fixed diagonal;
@@ -83,79 +83,87 @@ __global__ __launch_bounds__(256) void copy_out_kernel(const float *Minv, int64_
     L[row * K + c] = (c <= row) ? Minv[row * Kp + c] : 0.f;
 }
 
-// ---------------------------------------------------------------- 128x128 diagonal block
+// ---------------------------------------------------------------- NB x NB diagonal block
 // D = A[b,b] (its lower triangle is read).  Finds M_bb lower with M_bb^T M_bb = D by a
 // standard Cholesky of the index-reversed block: G G^T = J D J, M_bb = J G^T J.  Writes
 // M_bb over A[b,b] (upper part zeroed) and M_bb^-1 = J G^-T J into Minv[b,b].
-constexpr int GS = NB + 1;  // LDS row stride
+//
+// One wavefront and no barrier inside the factorisation: lane r keeps row r of G (64
+// VGPRs) and later column r of G^-1; the loops are fully unrolled.  What another lane needs
+// (the scaled pivot column during the factorisation, a row of G during the inversion) goes
+// through LDS and is read back with broadcast reads (every lane the same address, four
+// values per read).  The block is on the critical path of the blocked factorisation
+// (nothing else can run while it does), so latency is what counts here.
+static_assert(NB == 64, "the diagonal kernel maps one matrix row to one lane of a wavefront");
+constexpr int GSTR = NB + 4;   // LDS row stride of G: rows stay 16-byte aligned
 
-__global__ __launch_bounds__(256) void chol_diag_kernel(float *A, float *Minv, int64_t ld, int b,
-                                                        int32_t *status) {
-  extern __shared__ float smem[];
-  float *G = smem;             // [NB][GS]   factor, lower
-  float *X = smem + NB * GS;   // [NB][GS]   inverse of the factor, lower
-  __shared__ float colbuf[NB];
-  __shared__ int bad;
-  const int tid = threadIdx.x;
+__device__ __forceinline__ float lane_bcast(float v, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+__global__ __launch_bounds__(64) void chol_diag_kernel(float *A, float *Minv, int64_t ld, int b,
+                                                       int32_t *status) {
+  __shared__ __attribute__((aligned(16))) float col[NB];
+  __shared__ __attribute__((aligned(16))) float Gs[NB * GSTR];
+  __shared__ float Xs[NB][NB + 1];
+  const int r = threadIdx.x;
   float *D = A + (int64_t)b * NB * ld + (int64_t)b * NB;
   float *Dinv = Minv + (int64_t)b * NB * ld + (int64_t)b * NB;
-  if (tid == 0) bad = 0;
 
-  // G[r][c] (r >= c) = D[127-c][127-r]  (lower element of D, since 127-c >= 127-r)
-  for (int idx = tid; idx < NB * NB; idx += 256) {
-    const int i = idx / NB, j = idx % NB;  // element D[i][j], coalesced along j
-    if (i >= j) G[(NB - 1 - j) * GS + (NB - 1 - i)] = D[(int64_t)i * ld + j];
-    X[i * GS + j] = 0.f;
+  // G[r][c] (c <= r) = D[63-c][63-r]: for fixed c the lanes read one row of D (coalesced)
+  float g[NB];
+#pragma unroll
+  for (int c = 0; c < NB; ++c) {
+    // the upper part of D is never used: read the mirrored (valid) element instead of branching
+    const float v = D[(int64_t)(NB - 1 - c) * ld + (NB - 1 - r)];
+    g[c] = (c <= r) ? v : 0.f;
   }
-  __syncthreads();
 
-  // right-looking Cholesky, 2 barriers per column
-  const int tr = tid >> 4, tc = tid & 15;
+  // ---- Cholesky, right-looking: after step k, g[k] of lane r >= k holds G[r][k]
+  bool bad = false;
+#pragma unroll
   for (int k = 0; k < NB; ++k) {
-    const float piv = G[k * GS + k];
-    if (tid == 0 && !(piv > 0.f)) bad = 1;
+    const float piv = lane_bcast(g[k], k);
+    bad = bad || !(piv > 0.f);
     const float root = sqrtf(piv);
     const float rinv = 1.f / root;
-    if (tid < NB && tid > k) colbuf[tid] = G[tid * GS + k] * rinv;
-    __syncthreads();
-    if (tid < NB) {
-      if (tid > k) G[tid * GS + k] = colbuf[tid];
-      else if (tid == k) G[k * GS + k] = root;
-    }
-    for (int r = k + 1 + tr; r < NB; r += 16) {
-      const float lr = colbuf[r];
-      for (int c = k + 1 + tc; c <= r; c += 16) G[r * GS + c] -= lr * colbuf[c];
-    }
-    __syncthreads();
-  }
-
-  // X = G^-1 by rows: X[i][j] = (delta_ij - sum_{k<i} G[i][k] X[k][j]) / G[i][i].
-  // Two threads per column j split the k range (even / odd) and combine by a lane swap.
-  {
-    const int j = tid >> 1, par = tid & 1;
-    for (int i = 0; i < NB; ++i) {
-      float acc = 0.f;
-      if (i > j) {
-        for (int k = j + par; k < i; k += 2) acc += G[i * GS + k] * X[k * GS + j];
+    const float l = (r == k) ? root : g[k] * rinv;   // lanes r < k hold 0 already
+    g[k] = l;
+    if (k + 1 < NB) {
+      col[r] = l;
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int c = k + 1; c < NB; ++c) {
+        const float lc = col[c];   // G[c][k], same address in every lane
+        g[c] = (c <= r) ? g[c] - l * lc : g[c];
       }
-      acc += __shfl_xor(acc, 1);
-      if (par == 0 && i >= j) X[i * GS + j] = ((i == j ? 1.f : 0.f) - acc) / G[i * GS + i];
-      __syncthreads();
+      __builtin_amdgcn_wave_barrier();
     }
   }
+#pragma unroll
+  for (int c = 0; c < NB; ++c) Gs[r * GSTR + c] = g[c];
+  __syncthreads();
 
-  // M_bb[i][j] = G[127-j][127-i], Minv_bb[i][j] = X[127-j][127-i]  (i >= j), zero above
-  for (int idx = tid; idx < NB * NB; idx += 256) {
-    const int i = idx / NB, j = idx % NB;
-    float m = 0.f, x = 0.f;
-    if (i >= j) {
-      m = G[(NB - 1 - j) * GS + (NB - 1 - i)];
-      x = X[(NB - 1 - j) * GS + (NB - 1 - i)];
-    }
-    D[(int64_t)i * ld + j] = m;
-    Dinv[(int64_t)i * ld + j] = x;
+  // ---- X = G^-1, lane j computes column j: x[i] = (delta_ij - sum_{k<i} G[i][k] x[k]) / G[i][i]
+  float x[NB];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    float acc = (i == r) ? 1.f : 0.f;
+#pragma unroll
+    for (int k = 0; k < i; ++k) acc -= Gs[i * GSTR + k] * x[k];
+    x[i] = acc / Gs[i * GSTR + i];   // x[i] stays 0 for i < j since every term is 0
   }
-  if (tid == 0 && bad) atomicMax(status, b + 1);
+#pragma unroll
+  for (int i = 0; i < NB; ++i) Xs[i][r] = x[i];
+  __syncthreads();
+
+  // M_bb[i][j] = G[63-j][63-i], Minv_bb[i][j] = X[63-j][63-i]  (i >= j), zero above
+  for (int i = 0; i < NB; ++i) {
+    const bool low = (i >= r);
+    D[(int64_t)i * ld + r] = low ? Gs[(NB - 1 - r) * GSTR + (NB - 1 - i)] : 0.f;
+    Dinv[(int64_t)i * ld + r] = low ? Xs[NB - 1 - r][NB - 1 - i] : 0.f;
+  }
+  if (__any(bad) && r == 0) atomicMax(status, b + 1);
 }
 
 struct Plan {
@@ -219,14 +227,8 @@ int gptq_hip_damp_invert(void *stream, float *H, float *W, int64_t K, int64_t N,
   }
 
   // ---- step 1: H = M^T M, last block first
-  const size_t diag_lds = 2 * (size_t)NB * GS * sizeof(float);
-  static_assert(2 * NB * GS * sizeof(float) <= 160 * 1024 - 1024, "diag block must fit LDS");
-  if (hipFuncSetAttribute(reinterpret_cast<const void *>(chol_diag_kernel),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)diag_lds) != hipSuccess)
-    return GPTQ_HIP_ELAUNCH;
   for (int b = nblk - 1; b >= 0; --b) {
-    hipLaunchKernelGGL(chol_diag_kernel, dim3(1), dim3(256), diag_lds, st, p.A, p.Minv, Kp, b,
-                       status);
+    hipLaunchKernelGGL(chol_diag_kernel, dim3(1), dim3(64), 0, st, p.A, p.Minv, Kp, b, status);
     GPTQ_CHECK_LAUNCH();
     if (b == 0) break;
     float *panel = p.A + (int64_t)b * NB * Kp;  // rows of block b, columns 0 .. b*NB

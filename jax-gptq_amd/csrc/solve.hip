@@ -2,11 +2,13 @@
 // accumulated error into all remaining rows with one fp32 MFMA GEMM per block.
 //
 // In-block kernel: the N output channels are independent, so one lane owns one channel.
-// The block is walked in sub-blocks of SB rows.  The SB rows of a sub-block and their SB
-// errors live in VGPRs (statically indexed, fully unrolled triangle); the rows of the
-// block below the sub-block are then updated in place in W (they stay L2-resident),
-// coalesced across lanes.  The block of L sits in LDS in its natural layout: every lane
-// reads the same address (LDS broadcast) and the SB factors of one row are consecutive.
+// A workgroup of 128 lanes first copies its 128 channels of the block's rows and the
+// block's corner of L into LDS (both coalesced), then works out of LDS only.  The block is
+// walked in sub-blocks of SB rows: the SB rows of a sub-block and their SB errors live in
+// VGPRs (statically indexed, fully unrolled triangle); the rows of the block below the
+// sub-block are then updated in the LDS tile (each lane touches only its own column, so
+// there are no bank conflicts and no barriers).  L is read with broadcast reads (every lane
+// the same address) and the SB factors of one row are consecutive.  W itself is not written.
 //
 // Every floating-point operation is the IEEE operation the reference writes (true
 // division, round-half-even, separate multiply and subtract) and every element receives
@@ -21,26 +23,41 @@ constexpr int SOLVE_TPB = 128;
 
 template <int SB, typename TQ>
 __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
-    float *Wb, int64_t N, const float *Lb, int64_t ldl, int bs, const float *scale,
+    const float *Wb, int64_t N, const float *Lb, int64_t ldl, int bs, const float *scale,
     const float *zero, float maxq, TQ *Qb, uint8_t *cb, float *Err) {
   // Wb, Qb, cb: first row of the block in W, Q, codes; Lb: the block's diagonal corner of L
 #pragma clang fp contract(off)
-  extern __shared__ float Ln[];  // Ln[j * bs + i] = Lb[j][i]
+  extern __shared__ float smem[];
+  float *Ln = smem;                 // Ln[j * bs + i] = Lb[j][i]
+  float *Wl = smem + bs * bs;       // Wl[j * SOLVE_TPB + lane] = W[block row j][channel]
   const int tid = threadIdx.x;
   for (int idx = tid; idx < bs * bs; idx += SOLVE_TPB) {
     const int j = idx / bs, i = idx - j * bs;
     Ln[idx] = Lb[(int64_t)j * ldl + i];
   }
-  __syncthreads();
   const int64_t n = (int64_t)blockIdx.x * SOLVE_TPB + tid;
-  if (n >= N) return;
+  const bool live = n < N;
+  float *wcol = Wl + tid;
+  if (live) {
+    const float *src = Wb + n;
+    int j = 0;
+    for (; j + 8 <= bs; j += 8) {     // eight independent loads in flight
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = src[(int64_t)(j + u) * N];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) wcol[(j + u) * SOLVE_TPB] = v[u];
+    }
+    for (; j < bs; ++j) wcol[j * SOLVE_TPB] = src[(int64_t)j * N];
+  }
+  __syncthreads();
+  if (!live) return;
   const float sc = scale[n], z = zero[n];
-  float *wcol = Wb + n;
 
   for (int r0 = 0; r0 < bs; r0 += SB) {
     float w[SB], e[SB];
 #pragma unroll
-    for (int t = 0; t < SB; ++t) w[t] = wcol[(int64_t)(r0 + t) * N];
+    for (int t = 0; t < SB; ++t) w[t] = wcol[(r0 + t) * SOLVE_TPB];
     const float *ld = Ln + r0 * bs + r0;  // diagonal sub-block
 #pragma unroll
     for (int t = 0; t < SB; ++t) {
@@ -57,29 +74,39 @@ __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
       const int64_t o = (int64_t)(r0 + t) * N + n;
       if (Qb) Qb[o] = from_f32<TQ>(qh);
       if (cb) cb[o] = (uint8_t)q;
-      Err[(int64_t)(r0 + t) * N + n] = e[t];
+      Err[o] = e[t];
     }
     // rows of this block below the sub-block
-#pragma unroll 2
+#pragma unroll 4
     for (int j = r0 + SB; j < bs; ++j) {
-      float x = wcol[(int64_t)j * N];
+      float x = wcol[j * SOLVE_TPB];
       const float *lr = Ln + j * bs + r0;
 #pragma unroll
       for (int u = 0; u < SB; ++u) {
         const float upd = lr[u] * e[u];
         x = x - upd;
       }
-      wcol[(int64_t)j * N] = x;
+      wcol[j * SOLVE_TPB] = x;
     }
   }
 }
 
 template <int SB>
-int launch_block(hipStream_t st, float *W, int64_t N, const float *L, int64_t ldl, int bs,
+int launch_block(hipStream_t st, const float *W, int64_t N, const float *L, int64_t ldl, int bs,
                  const float *scale, const float *zero, float maxq, void *Q, int q_dtype,
                  uint8_t *codes, float *Err) {
   const dim3 grid((unsigned)ceil_div64(N, SOLVE_TPB)), block(SOLVE_TPB);
-  const size_t lds = (size_t)bs * bs * sizeof(float);
+  const size_t lds = ((size_t)bs * bs + (size_t)bs * SOLVE_TPB) * sizeof(float);
+  if (lds > 64 * 1024) {
+    // up to 128 KB of the 160 KB LDS of a CU; the limit has to be raised per kernel
+    const void *fn = q_dtype == GPTQ_HIP_F32
+                         ? reinterpret_cast<const void *>(block_quant_kernel<SB, float>)
+                         : (q_dtype == GPTQ_HIP_F16
+                                ? reinterpret_cast<const void *>(block_quant_kernel<SB, __half>)
+                                : reinterpret_cast<const void *>(block_quant_kernel<SB, __hip_bfloat16>));
+    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return GPTQ_HIP_ELAUNCH;
+  }
   switch (q_dtype) {
     case GPTQ_HIP_F32:
       hipLaunchKernelGGL((block_quant_kernel<SB, float>), grid, block, lds, st, W, N, L, ldl,
@@ -102,7 +129,7 @@ int launch_block(hipStream_t st, float *W, int64_t N, const float *L, int64_t ld
 
 bool block_size_ok(int bs) { return bs >= 1 && bs <= 128; }
 
-int process_block(hipStream_t st, float *Wb, int64_t N, const float *Lb, int64_t ldl, int bs,
+int process_block(hipStream_t st, const float *Wb, int64_t N, const float *Lb, int64_t ldl, int bs,
                   const float *scale, const float *zero, int maxq, void *Qb, int q_dtype,
                   uint8_t *cb, float *Err) {
 #define GPTQ_SB_CASE(SB) \
@@ -124,7 +151,7 @@ size_t gptq_hip_solve_workspace_bytes(int64_t K, int64_t N, int block_size) {
   return (size_t)block_size * (size_t)N * sizeof(float);
 }
 
-int gptq_hip_process_block(void *stream, float *Wblock, int64_t N, const float *Lblock,
+int gptq_hip_process_block(void *stream, const float *Wblock, int64_t N, const float *Lblock,
                            int64_t ldl, int block_size, const float *scale, const float *zero,
                            int maxq, void *Qblock, int q_dtype, uint8_t *codes_block,
                            float *errors) {

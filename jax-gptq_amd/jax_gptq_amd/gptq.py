@@ -243,14 +243,14 @@ def _unpermute(Q, perm):
 # ------------------------------------------------------------------------------- loop
 def _process_block(W, Hinv, start, quantize_params, block_size):
     """One block of the column loop (reference ``gptq.py:130-153``): returns
-    ``(q_block, errors)``, both ``[block_size, N]`` fp32.  ``W`` is not modified."""
+    ``(q_block, errors)``, both ``[block_size, N]`` fp32."""
     lib = N.load()
     W = _dev(W, torch.float32)
     Hinv = _dev(Hinv, torch.float32)
     K, Nc = W.shape
     if start < 0 or start + block_size > K:
         raise ValueError("block out of range")
-    blk = W[start:start + block_size].clone()
+    blk = W[start:start + block_size]
     q = torch.empty((block_size, Nc), dtype=torch.float32, device=W.device)
     err = torch.empty((block_size, Nc), dtype=torch.float32, device=W.device)
     lblk = Hinv[start:, start:]
