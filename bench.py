@@ -130,7 +130,7 @@ def bench_qmatmul(reps=240):
     return out
 
 
-def cpu_baseline(sample_batches=4):
+def cpu_baseline(sample_batches=16):
     """The oracle (NumPy/SciPy restatement of the reference) timed on this host's cores on a
     bounded sample of the same workload: the Hessian over `sample_batches` of the 128
     batches (scaled linearly), then the complete factorisation, column loop and packing."""
@@ -167,6 +167,10 @@ def main():
     ap.add_argument("--x-dtype", default="float32", choices=["float32", "float16", "bfloat16"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-qmatmul", action="store_true", help="skip the int4 matmul section")
+    ap.add_argument("--section", default="all", choices=["all", "hessian", "qmatmul", "copy"],
+                    help="profiling aid: run only one part (hessian: X^T X over the 128 batches; "
+                         "qmatmul: the int4 matmul loop; copy: a plain 1 GiB device copy used to "
+                         "calibrate the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (use --gpus 1)")
@@ -176,8 +180,33 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
 
+    if args.section == "copy":
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")      # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(max(1, args.steps)):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"section": "copy", "bytes_read": src.numel() * 4,
+                          "bytes_written": src.numel() * 4, "launches": max(1, args.steps)}))
+        return
+    if args.section == "qmatmul":
+        print(json.dumps({"section": "qmatmul", "qmatmul": bench_qmatmul()}))
+        return
+
     W, xs = make_inputs(K_IN, N_OUT, N_BATCH, ROWS, getattr(torch, args.x_dtype))
     torch.cuda.synchronize()
+    if args.section == "hessian":
+        G.accumulate_H(xs)
+        e0, e1 = _events(2)
+        e0.record()
+        for _ in range(max(1, args.steps)):
+            G.accumulate_H(xs)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / max(1, args.steps)
+        print(json.dumps({"section": "hessian", "ms": round(ms, 3),
+                          "algorithmic_tflops": round(2.0 * N_BATCH * ROWS * K_IN * K_IN / ms * 1e-9, 2)}))
+        return
 
     for _ in range(args.warmup):
         one_layer(G, W, xs)
@@ -205,7 +234,10 @@ def main():
     executed = executed_flop / (hess_ms * 1e-3) * 1e-12
     roofline = {"kernel": "syrk_kernel<float> (X^T X, fp32 MFMA, upper tiles)", "bound": "mfma",
                 "achieved": round(achieved, 2), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
+                # bytes per launch beyond L2 from rocprofv3 FETCH_SIZE + WRITE_SIZE (scaled by what the
+                # counters read for a 1 GiB copy: x2.000 / x1.000), summary kept under profiles/
+                "traffic": 6.48e10,
                 "flop_per_launch": flop_per_launch, "avg_launch_ms": round(hess_ms, 4),
                 "launches_per_step": 1,
                 "executed_tflops": round(executed, 2),
@@ -232,7 +264,7 @@ def main():
         result["int4_matmul_hbm_gbps"] = m1["GBps"]
         result["roofline_qmatmul"] = {"kernel": "qmatmul M=1 4096x11008", "bound": "hbm",
                                       "achieved": m1["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                      "frac": m1["hbm_frac"], "traffic": None}
+                                      "frac": m1["hbm_frac"], "traffic": 2.32e7}
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))

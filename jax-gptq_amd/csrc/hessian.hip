@@ -52,7 +52,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
   __shared__ __attribute__((aligned(16))) float As[2][HBK * HLD];
   __shared__ __attribute__((aligned(16))) float Bs[2][HBK * HLD];
   const int ntiles = p.T * (p.T + 1) / 2;
-  const int rs = blockIdx.x / ntiles, t = blockIdx.x - rs * ntiles;
+  // Workgroup ids are dealt round-robin to the 8 XCDs (each with its own L2).  With a
+  // multiple of 8 row slices, give every XCD its own slices: all tiles of one slice then
+  // run on one XCD and that L2 sees only 1/RS of the rows of X.
+  int rs, t;
+  if ((p.RS & 7) == 0) {
+    const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
+    rs = xcd + 8 * (q / ntiles);
+    t = q % ntiles;
+  } else {
+    rs = blockIdx.x / ntiles;
+    t = blockIdx.x - rs * ntiles;
+  }
   int ti, tj;
   tile_decode(t, ti, tj);
   const int m0 = ti * HB, n0 = tj * HB, K = p.K;
@@ -216,8 +227,8 @@ __global__ __launch_bounds__(256) void syrk_reduce_kernel(float *H, const float 
 int pick_rs(int64_t K) {
   const int64_t T = ceil_div64(K, HB), ntiles = T * (T + 1) / 2;
   int64_t rs = ceil_div64(6144, ntiles);   // about eight waves of workgroups over 768 slots
-  if (rs > H_RSMAX) rs = H_RSMAX;
   if (rs < 1) rs = 1;
+  if (rs > 4) rs = (rs <= 8) ? 8 : H_RSMAX;   // multiples of 8 get the per-XCD slice mapping
   return (int)rs;
 }
 
@@ -299,7 +310,7 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
     a.RS = pick_rs(K);
     // never more slices than 16-row slabs in the largest batch
     const int64_t slabs = ceil_div64(max_rows, HBK);
-    if (a.RS > slabs) a.RS = (int)slabs;
+    while (a.RS > 1 && a.RS > slabs) a.RS = (a.RS > 8) ? 8 : ((a.RS > 4) ? 4 : a.RS - 1);
     a.H = H;
     a.ws = reinterpret_cast<float *>(ws);
     const dim3 grid((unsigned)((int64_t)ntiles * a.RS)), block(256);
