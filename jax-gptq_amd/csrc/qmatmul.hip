@@ -366,6 +366,167 @@ int launch_fwd_mfma_z(hipStream_t st, const FwdPlan &p, const void *x, int64_t M
   return launch_fwd_mfma<4, TZ>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
 }
 
+// ---------------------------------------------------------------------------- large M
+// Forward, fp16 activations, M > 32: a tiled GEMM that dequantises on the way into LDS.
+// Workgroup tile 64 (M) x BN (N) x 64 (k) per stage, 4 wavefronts as 2 x 2, accumulators of
+// v_mfma_f32_16x16x32_f16 in registers for the whole K loop (no split-K, no partials).
+//   A = activations: staged in their natural [m][k] layout (k contiguous = the operand order)
+//   B = weights: every thread loads 16 packed bytes (16 channels of one packed row), turns
+//       each byte into the fp16 pair {code_lo - zero, code_hi - zero} (0x6400 trick, exact for
+//       the integer zero points GPTQ produces) and stores it at Bs[channel][2*row], so that the
+//       operand fetch is again one 16-byte read of 8 consecutive k.
+// Row pitch 72 halves and a skew of 8 words per 16-channel group keep both the transposing
+// stores and the operand reads free of bank conflicts.  scale is applied in the epilogue.
+constexpr int GBM = 64, GBK = 64;
+constexpr int GPITCH = GBK + 8;                 // halves per LDS row
+constexpr int GGROUP = 16 * GPITCH + 16;        // halves per 16-row group (16 = the 8-word skew)
+
+__device__ __forceinline__ int g_off(int row, int k) {   // LDS offset (halves) of element [row][k]
+  return (row >> 4) * GGROUP + (row & 15) * GPITCH + k;
+}
+
+template <int BN, typename TZ>
+__global__ __launch_bounds__(256) void qmm_fwd_gemm_kernel(const __half *x, int M, int K,
+                                                           const uint8_t *pk, int R, int C,
+                                                           const TZ *zero, const TZ *scale,
+                                                           __half *out) {
+  constexpr int A_HALVES = (GBM / 16) * GGROUP;
+  constexpr int B_HALVES = (BN / 16) * GGROUP;
+  constexpr int TN = BN / 32;                   // 16-wide MFMA tiles per wavefront along N
+  constexpr int B_THREADS = 2 * BN;             // threads that stage weights: 32 rows x BN/16 segments
+  __shared__ __attribute__((aligned(16))) _Float16 As[2][A_HALVES];
+  __shared__ __attribute__((aligned(16))) _Float16 Bs[2][B_HALVES];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, g = lane >> 4, l16 = lane & 15;
+  const int n0 = blockIdx.x * BN, m0 = blockIdx.y * GBM;
+
+  // A staging: thread -> row tid/4, 16 halves at k = (tid%4)*16
+  const int a_row = tid >> 2, a_k = (tid & 3) * 16;
+  const bool a_ok = (m0 + a_row) < M;
+  const __half *a_src = x + (int64_t)(m0 + a_row) * K + a_k;
+  // B staging: thread -> packed row tid / (BN/16), 16 channels at (tid % (BN/16)) * 16
+  const int b_row = tid / (BN / 16), b_c = (tid % (BN / 16)) * 16;
+  const bool b_thread = tid < B_THREADS;
+  const bool b_ok = b_thread && (n0 + b_c) < C;
+  const uint8_t *b_src = pk + (int64_t)b_row * C + n0 + b_c;
+  // -(1024 + zero) per staged channel, as fp16 pairs
+  uint32_t zc[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const float z = b_ok ? to_f32(zero[n0 + b_c + i]) : 0.f;
+    const _Float16 h = (_Float16)(-(1024.f + z));
+    zc[i] = __builtin_bit_cast(uint32_t, half2_t{h, h});
+  }
+
+  // Register ring of four stages (named variables, so that they are sure to live in VGPRs):
+  // the loads of stage s + 4 are issued while stage s is being multiplied, so about four
+  // stage times hide the memory latency even with one workgroup per CU.
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  struct Stage { u32x4 a0, a1, b; };
+  // Loads are unconditional (out-of-range lanes read a clamped, valid address and are zeroed
+  // when the stage is written to LDS): a load inside a branch would make the compiler wait
+  // for it at the join and defeat the prefetch.  K % 8 == 0 is guaranteed by the dispatcher.
+  auto load_stage = [&](int k0, Stage &st) __attribute__((always_inline)) {
+    const bool ok0 = a_ok && (k0 + a_k + 8 <= K), ok1 = a_ok && (k0 + a_k + 16 <= K);
+    st.a0 = *reinterpret_cast<const u32x4 *>(ok0 ? a_src + k0 : x);
+    st.a1 = *reinterpret_cast<const u32x4 *>(ok1 ? a_src + k0 + 8 : x);
+    const bool okb = b_ok && ((k0 >> 1) + b_row < R);
+    st.b = *reinterpret_cast<const u32x4 *>(okb ? b_src + (int64_t)(k0 >> 1) * C : pk);
+  };
+  auto store_stage = [&](int buf, int k0, const Stage &st) __attribute__((always_inline)) {
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
+    const bool ok0 = a_ok && (k0 + a_k + 8 <= K), ok1 = a_ok && (k0 + a_k + 16 <= K);
+    *reinterpret_cast<u32x4 *>(&As[buf][g_off(a_row, a_k)]) = ok0 ? st.a0 : zero4;
+    *reinterpret_cast<u32x4 *>(&As[buf][g_off(a_row, a_k + 8)]) = ok1 ? st.a1 : zero4;
+    if (b_thread) {
+      const bool okb = b_ok && ((k0 >> 1) + b_row < R);
+      const u32x4 pbm = okb ? st.b : zero4;
+      const uint32_t w[4] = {pbm[0], pbm[1], pbm[2], pbm[3]};
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const uint32_t b = (w[i >> 2] >> (8 * (i & 3))) & 0xFFu;
+        const uint32_t v = ((b | (b << 12)) & 0x000F000Fu) | 0x64006400u;   // {1024+lo, 1024+hi}
+        const half2_t d = __builtin_bit_cast(half2_t, v) + __builtin_bit_cast(half2_t, zc[i]);
+        *reinterpret_cast<uint32_t *>(&Bs[buf][g_off(b_c + i, 2 * b_row)]) =
+            __builtin_bit_cast(uint32_t, d);
+      }
+    }
+  };
+
+  floatx4 acc[2][TN];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  Stage s0, s1, s2, s3;
+  load_stage(0, s0);
+  load_stage(GBK, s1);
+  load_stage(2 * GBK, s2);
+  load_stage(3 * GBK, s3);
+  int buf = 0;
+  store_stage(0, 0, s0);
+  __syncthreads();
+  // one stage: refill the ring slot that was just consumed, multiply the stage in LDS, write
+  // the next stage to the other LDS buffer
+  auto step = [&](int k0, Stage &refill, const Stage &next) __attribute__((always_inline)) {
+    if (k0 >= K) return;
+    load_stage(k0 + 4 * GBK, refill);
+#pragma unroll
+    for (int ks = 0; ks < GBK; ks += 32) {
+      half8_t a[2], b[TN];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        a[i] = *reinterpret_cast<const half8_t *>(&As[buf][g_off(wm * 32 + i * 16 + l16, ks + 8 * g)]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        b[j] = *reinterpret_cast<const half8_t *>(
+            &Bs[buf][g_off(wn * (BN / 2) + j * 16 + l16, ks + 8 * g)]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (k0 + GBK < K) store_stage(buf ^ 1, k0 + GBK, next);
+    __syncthreads();
+    buf ^= 1;
+  };
+  for (int kb = 0; kb < K; kb += 4 * GBK) {
+    step(kb, s0, s1);
+    step(kb + GBK, s1, s2);
+    step(kb + 2 * GBK, s2, s3);
+    step(kb + 3 * GBK, s3, s0);
+  }
+
+  // acc[i][j][r] = out[m0 + wm*32 + i*16 + 4g + r][n0 + wn*BN/2 + j*16 + l16]
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int n = n0 + wn * (BN / 2) + j * 16 + l16;
+    if (n >= C) continue;
+    const float sc = to_f32(scale[n]);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = m0 + wm * 32 + i * 16 + 4 * g + r;
+        if (m < M) out[(int64_t)m * C + n] = __float2half_rn(sc * acc[i][j][r]);
+      }
+  }
+}
+
+template <typename TZ>
+int launch_fwd_gemm(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
+                    const void *zero, const void *scale, void *out) {
+  const int64_t mt = ceil_div64(M, GBM);
+  if (mt > 65535) return GPTQ_HIP_EINVAL;
+  hipLaunchKernelGGL((qmm_fwd_gemm_kernel<128, TZ>), dim3((unsigned)ceil_div64(C, 128), (unsigned)mt),
+                     dim3(256), 0, st, (const __half *)x, (int)M, (int)(2 * R), pk, (int)R, (int)C,
+                     (const TZ *)zero, (const TZ *)scale, (__half *)out);
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
 bool fwd_fast_ok(int x_dtype, int64_t M, int64_t R, int64_t C, const void *x, const uint8_t *pk) {
   return x_dtype == GPTQ_HIP_F16 && C % 16 == 0 && M >= 1 && M <= 65535 * 16LL &&
          (reinterpret_cast<uintptr_t>(pk) & 15) == 0 && (reinterpret_cast<uintptr_t>(x) & 3) == 0 &&
@@ -420,6 +581,19 @@ int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const 
   if (M == 0) return GPTQ_HIP_OK;
   if (!x || !packed || !zero || !scale || !out) return GPTQ_HIP_EINVAL;
   hipStream_t st = as_stream(stream);
+  // The tiled kernel has no split-K: it needs enough 64 x 128 output tiles to occupy the
+  // chip; otherwise 16-row chunks through the split-K kernel (weights re-read from cache) win.
+  if (!transpose_b && fwd_fast_ok(x_dtype, M, R, C, x, packed) && M > 32 &&
+      ceil_div64(C, 128) * ceil_div64(M, GBM) >= 160 &&
+      (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (2 * R) % 8 == 0) {
+    switch (zs_dtype) {
+      case GPTQ_HIP_F32: return launch_fwd_gemm<float>(st, x, M, packed, R, C, zero, scale, out);
+      case GPTQ_HIP_F16: return launch_fwd_gemm<__half>(st, x, M, packed, R, C, zero, scale, out);
+      case GPTQ_HIP_BF16:
+        return launch_fwd_gemm<__hip_bfloat16>(st, x, M, packed, R, C, zero, scale, out);
+      default: return GPTQ_HIP_EDTYPE;
+    }
+  }
   if (!transpose_b && fwd_fast_ok(x_dtype, M, R, C, x, packed)) {
     const FwdPlan p = fwd_plan(M, R, C);
     if (p.total_bytes && (!ws || ws_bytes < p.total_bytes)) return GPTQ_HIP_EWORKSPACE;

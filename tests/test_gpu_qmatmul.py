@@ -41,7 +41,7 @@ def _check(got, x, qm, transpose):
 
 # shapes of the reference's test_kernel.py:13 plus the decode shapes of the benchmark config
 SHAPES = [(137, 909, 256), (32, 1024, 2048), (37, 32000, 5120), (1, 11008, 4096), (16, 4096, 11008),
-          (128, 11008, 4096), (3, 130, 66), (1, 64, 2)]
+          (128, 11008, 4096), (128, 4096, 11008), (70, 2304, 768), (3, 130, 66), (1, 64, 2)]
 
 
 @pytest.mark.parametrize("transpose", [False, True])
