@@ -111,7 +111,8 @@ __global__ __launch_bounds__(64) void chol_diag_kernel(float *A, float *Minv, in
   float *Dinv = Minv + (int64_t)b * NB * ld + (int64_t)b * NB;
 
   // G[r][c] (c <= r) = D[63-c][63-r]: for fixed c the lanes read one row of D (coalesced)
-  float g[NB];
+  typedef float rowvec __attribute__((ext_vector_type(NB)));   // a vector value, never an alloca
+  rowvec g;
 #pragma unroll
   for (int c = 0; c < NB; ++c) {
     // the upper part of D is never used: read the mirrored (valid) element instead of branching
@@ -135,7 +136,11 @@ __global__ __launch_bounds__(64) void chol_diag_kernel(float *A, float *Minv, in
 #pragma unroll
       for (int c = k + 1; c < NB; ++c) {
         const float lc = col[c];   // G[c][k], same address in every lane
-        g[c] = (c <= r) ? g[c] - l * lc : g[c];
+        float t = (c <= r) ? g[c] - l * lc : g[c];
+        // Pin the update to this step.  Left free, the compiler defers every update until the
+        // element is needed and keeps all broadcast values of all steps alive (2000 registers).
+        asm volatile("" : "+v"(t));
+        g[c] = t;
       }
       __builtin_amdgcn_wave_barrier();
     }
@@ -145,13 +150,15 @@ __global__ __launch_bounds__(64) void chol_diag_kernel(float *A, float *Minv, in
   __syncthreads();
 
   // ---- X = G^-1, lane j computes column j: x[i] = (delta_ij - sum_{k<i} G[i][k] x[k]) / G[i][i]
-  float x[NB];
+  rowvec x;
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
     float acc = (i == r) ? 1.f : 0.f;
 #pragma unroll
     for (int k = 0; k < i; ++k) acc -= Gs[i * GSTR + k] * x[k];
-    x[i] = acc / Gs[i * GSTR + i];   // x[i] stays 0 for i < j since every term is 0
+    float xi = acc / Gs[i * GSTR + i];   // stays 0 for i < j since every term is 0
+    asm volatile("" : "+v"(xi));         // keeps the row reads of later steps from being hoisted
+    x[i] = xi;
   }
 #pragma unroll
   for (int i = 0; i < NB; ++i) Xs[i][r] = x[i];
