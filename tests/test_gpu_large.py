@@ -15,7 +15,7 @@ SHAPES = [
     (4096, 11008, 4),    # LLaMA-7B gate/up projection, the benchmark layer
     (11008, 4096, 4),    # LLaMA-7B down projection
     (7168, 28672, 2),    # OPT-30B fc1
-    (28672, 7168, 4),    # OPT-30B fc2: H is 28672^2 fp32
+    (28672, 7168, 16),   # OPT-30B fc2: H is 28672^2 fp32 (rows >= K keeps H well conditioned)
 ]
 
 
