@@ -30,7 +30,7 @@ extern "C" {
 #define GPTQ_HIP_ABI_VERSION 1
 
 /* element types of float operands */
-enum { GPTQ_HIP_F32 = 0, GPTQ_HIP_F16 = 1, GPTQ_HIP_BF16 = 2 };
+enum { GPTQ_HIP_F32 = 0, GPTQ_HIP_F16 = 1, GPTQ_HIP_BF16 = 2, GPTQ_HIP_F64 = 3 };
 
 /* status codes */
 enum {
@@ -56,35 +56,39 @@ int gptq_hip_col_params(void *stream, const void *W, int w_dtype, int64_t K, int
 /* ---- Hessian ------------------------------------------------------------------
  * Replaces _accumulate_H_step / accumulate_H (gptq.py:57-103).
  * gptq_hip_hessian_accumulate adds sum_b X_b^T X_b to the UPPER triangle (128x128
- * tile granularity) of H [K, K] fp32.  x_ptrs / x_rows are HOST arrays of
+ * tile granularity) of H [K, K], whose element type h_dtype is GPTQ_HIP_F32 or, for the
+ * reference's use_fp64 option (gptq.py:88, 182-187), GPTQ_HIP_F64 (products and sums in
+ * double; the batches may then be fp64 too).  x_ptrs / x_rows are HOST arrays of
  * n_batches device pointers / row counts; batch b is [x_rows[b], K] row-major,
  * contiguous.  All batches of one call are reduced in one launch (in registers), so
  * passing the whole calibration set at once is the fast path; one batch per call
  * reproduces the reference's streaming use.  The running mean of the reference cancels
  * algebraically (H = sum X^T X / n), so none is kept.
- * ws: gptq_hip_hessian_accumulate_workspace_bytes(K) bytes (0 for large K).
+ * ws: gptq_hip_hessian_accumulate_workspace_bytes(K, h_dtype) bytes (0 for large K and for fp64).
  * gptq_hip_hessian_finalize multiplies by 1/n_samples and mirrors the upper
  * triangle into the lower one, giving the full symmetric H the reference returns. */
-size_t gptq_hip_hessian_accumulate_workspace_bytes(int64_t K);
+size_t gptq_hip_hessian_accumulate_workspace_bytes(int64_t K, int h_dtype);
 int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const int64_t *x_rows,
-                                int n_batches, int x_dtype, int64_t K, float *H, void *ws,
-                                size_t ws_bytes);
-int gptq_hip_hessian_finalize(void *stream, float *H, int64_t K, double n_samples);
+                                int n_batches, int x_dtype, int64_t K, void *H, int h_dtype,
+                                void *ws, size_t ws_bytes);
+int gptq_hip_hessian_finalize(void *stream, void *H, int h_dtype, int64_t K, double n_samples);
 
 /* ---- dead features, damping, Cholesky factor of the inverse -----------------------
  * Replaces _damp_and_invert + _cholesky_inv (gptq.py:155-168, 44-48).
- * H [K, K] fp32 full symmetric (read; its diagonal is rewritten with the dead-feature
- * fix and the damping, as the reference's donated buffer is); W [K, N] fp32 (rows
- * of dead features zeroed in place; may be NULL with N = 0); L [K, K] fp32 out:
- * lower triangular, L L^T = (H + damping*mean(diag H) I)^-1, upper part zero.
- * status (device int32[2]): status[0] = 0, or 1 + index of the first 128-block whose
+ * H [K, K] full symmetric, element type h_dtype = GPTQ_HIP_F32 or GPTQ_HIP_F64 (read; its
+ * diagonal is rewritten with the dead-feature fix and the damping, as the reference's
+ * donated buffer is); W [K, N] fp32 (rows of dead features zeroed in place; may be NULL
+ * with N = 0); L [K, K] out, same element type as H: lower triangular,
+ * L L^T = (H + damping*mean(diag H) I)^-1, upper part zero.  L32 (may be NULL) also
+ * receives L rounded to fp32, the cast of gptq.py:197 that feeds the column loop.
+ * status (device int32[2]): status[0] = 0, or 1 + index of the first 64-block whose
  * pivot was not positive (L then holds NaN, as the reference's does, gptq.py:166);
  * status[1] = number of dead features.  fix_dead = 0 skips the dead-feature fix (with
  * damping = 0 the call is then exactly _cholesky_inv, gptq.py:44-48). */
-size_t gptq_hip_damp_invert_workspace_bytes(int64_t K);
-int gptq_hip_damp_invert(void *stream, float *H, float *W, int64_t K, int64_t N, int64_t ldw,
-                         float damping, int fix_dead, float *L, int32_t *status, void *ws,
-                         size_t ws_bytes);
+size_t gptq_hip_damp_invert_workspace_bytes(int64_t K, int h_dtype);
+int gptq_hip_damp_invert(void *stream, void *H, int h_dtype, float *W, int64_t K, int64_t N,
+                         int64_t ldw, double damping, int fix_dead, void *L, float *L32,
+                         int32_t *status, void *ws, size_t ws_bytes);
 
 /* ---- blocked column loop ------------------------------------------------------------
  * Replaces the loop of gptq() with _process_block and the lazy update
@@ -113,10 +117,12 @@ int gptq_hip_process_block(void *stream, const float *Wblock, int64_t N, const f
 /* ---- activation order ---------------------------------------------------------------
  * Replaces the gathers of _permute / _unpermute (gptq.py:170-180); the argsort itself
  * stays with the caller.  out[i, :] = in[perm[i], :] for rows; the symmetric form
- * gathers rows and columns: out[i, j] = in[perm[i], perm[j]].  perm is device int64[K]. */
+ * gathers rows and columns: out[i, j] = in[perm[i], perm[j]].  perm is device int64[K];
+ * elem_bytes is 1, 2, 4 or 8 for rows and 4 or 8 for the symmetric form. */
 int gptq_hip_gather_rows(void *stream, const void *in, void *out, int elem_bytes, int64_t K,
                          int64_t N, const int64_t *perm);
-int gptq_hip_gather_sym(void *stream, const float *in, float *out, int64_t K, const int64_t *perm);
+int gptq_hip_gather_sym(void *stream, const void *in, void *out, int elem_bytes, int64_t K,
+                        const int64_t *perm);
 
 /* ---- int4 codec -----------------------------------------------------------------------
  * A tensor is viewed as [outer, axis_len, inner] and packed along the middle axis:

@@ -10,8 +10,9 @@
 // H^-1 = M^-1 M^-T = L L^T with L lower triangular and a positive diagonal, which is the
 // unique Cholesky factor the reference computes.
 //
-// All O(K^3) work runs on the fp32 MFMA GEMM; only the NB x NB diagonal blocks are
-// factorised and inverted inside one workgroup, in LDS.
+// All O(K^3) work runs on the MFMA GEMM; only the NB x NB diagonal blocks are factorised
+// and inverted by a single wavefront.  Everything is templated on the scalar type R:
+// float is the default path, double the reference's use_fp64 option (gptq.py:182-197).
 #include "common.h"
 #include "gemm_f32.h"
 
@@ -22,19 +23,20 @@ constexpr int NB = 64;
 // ---------------------------------------------------------------- diag / damping prep
 // One workgroup.  dead_i = (H_ii == 0) -> H_ii = 1; mean over the fixed diagonal;
 // H_ii += damping * mean.  Writes dead flags and status[1] = number of dead features.
-__global__ __launch_bounds__(1024) void damp_diag_kernel(float *H, int64_t K, float damping,
+template <typename R>
+__global__ __launch_bounds__(1024) void damp_diag_kernel(R *H, int64_t K, R damping,
                                                          int fix_dead, uint8_t *dead,
                                                          int32_t *status) {
 #pragma clang fp contract(off)
-  __shared__ float ssum[1024];
+  __shared__ R ssum[1024];
   __shared__ int scnt[1024];
   const int tid = threadIdx.x;
-  float sum = 0.f;
+  R sum = 0;
   int cnt = 0;
   for (int64_t i = tid; i < K; i += 1024) {
-    float d = H[i * K + i];
-    const bool is_dead = fix_dead && (d == 0.f);
-    if (is_dead) { d = 1.f; ++cnt; }
+    R d = H[i * K + i];
+    const bool is_dead = fix_dead && (d == R(0));
+    if (is_dead) { d = 1; ++cnt; }
     dead[i] = is_dead ? 1 : 0;
     sum += d;
   }
@@ -45,10 +47,10 @@ __global__ __launch_bounds__(1024) void damp_diag_kernel(float *H, int64_t K, fl
     if (tid < s) { ssum[tid] += ssum[tid + s]; scnt[tid] += scnt[tid + s]; }
     __syncthreads();
   }
-  const float add = (ssum[0] / (float)K) * damping;
+  const R add = (ssum[0] / (R)K) * damping;
   for (int64_t i = tid; i < K; i += 1024) {
-    float d = H[i * K + i];
-    if (dead[i]) d = 1.f;
+    R d = H[i * K + i];
+    if (dead[i]) d = 1;
     H[i * K + i] = d + add;
   }
   if (tid == 0) { status[0] = 0; status[1] = scnt[0]; }
@@ -63,24 +65,29 @@ __global__ __launch_bounds__(256) void zero_dead_rows_kernel(float *W, int64_t N
 }
 
 // A (Kp x Kp, padded with the identity) <- H ; Minv <- 0
-__global__ __launch_bounds__(256) void pad_copy_kernel(const float *H, int64_t K, float *A,
-                                                       float *Minv, int64_t Kp) {
+template <typename R>
+__global__ __launch_bounds__(256) void pad_copy_kernel(const R *H, int64_t K, R *A, R *Minv,
+                                                       int64_t Kp) {
   const int64_t row = blockIdx.y;
   for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < Kp; c += (int64_t)gridDim.x * 256) {
-    float v;
+    R v;
     if (row < K && c < K) v = H[row * K + c];
-    else v = (row == c) ? 1.f : 0.f;
+    else v = (row == c) ? 1 : 0;
     A[row * Kp + c] = v;
-    Minv[row * Kp + c] = 0.f;
+    Minv[row * Kp + c] = 0;
   }
 }
 
-// L (K x K, ld K) <- lower(Minv[0:K, 0:K]), upper part zero
-__global__ __launch_bounds__(256) void copy_out_kernel(const float *Minv, int64_t Kp, float *L,
-                                                       int64_t K) {
+// L (K x K, ld K) <- lower(Minv[0:K, 0:K]), upper part zero; L32, if given, gets the fp32 cast
+template <typename R>
+__global__ __launch_bounds__(256) void copy_out_kernel(const R *Minv, int64_t Kp, R *L,
+                                                       float *L32, int64_t K) {
   const int64_t row = blockIdx.y;
-  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < K; c += (int64_t)gridDim.x * 256)
-    L[row * K + c] = (c <= row) ? Minv[row * Kp + c] : 0.f;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < K; c += (int64_t)gridDim.x * 256) {
+    const R v = (c <= row) ? Minv[row * Kp + c] : R(0);
+    L[row * K + c] = v;
+    if (L32) L32[row * K + c] = (float)v;
+  }
 }
 
 // ---------------------------------------------------------------- NB x NB diagonal block
@@ -100,43 +107,52 @@ constexpr int GSTR = NB + 4;   // LDS row stride of G: rows stay 16-byte aligned
 __device__ __forceinline__ float lane_bcast(float v, int lane) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
+__device__ __forceinline__ double lane_bcast(double v, int lane) {
+  const int2 w = __builtin_bit_cast(int2, v);
+  int2 o;
+  o.x = __builtin_amdgcn_readlane(w.x, lane);
+  o.y = __builtin_amdgcn_readlane(w.y, lane);
+  return __builtin_bit_cast(double, o);
+}
+__device__ __forceinline__ float root_of(float v) { return sqrtf(v); }
+__device__ __forceinline__ double root_of(double v) { return sqrt(v); }
 
-__global__ __launch_bounds__(64) void chol_diag_kernel(float *A, float *Minv, int64_t ld, int b,
+template <typename R>
+__global__ __launch_bounds__(64) void chol_diag_kernel(R *A, R *Minv, int64_t ld, int b,
                                                        int32_t *status) {
-  __shared__ __attribute__((aligned(16))) float col[NB];
-  __shared__ __attribute__((aligned(16))) float Gs[NB * GSTR];
-  __shared__ float Xs[NB][NB + 1];
+  __shared__ __attribute__((aligned(16))) R col[NB];
+  __shared__ __attribute__((aligned(16))) R Gs[NB * GSTR];   // G, later reused for X = G^-1
   const int r = threadIdx.x;
-  float *D = A + (int64_t)b * NB * ld + (int64_t)b * NB;
-  float *Dinv = Minv + (int64_t)b * NB * ld + (int64_t)b * NB;
+  R *D = A + (int64_t)b * NB * ld + (int64_t)b * NB;
+  R *Dinv = Minv + (int64_t)b * NB * ld + (int64_t)b * NB;
 
   // G[r][c] (c <= r) = D[63-c][63-r]: for fixed c the lanes read one row of D (coalesced)
-  typedef float rowvec __attribute__((ext_vector_type(NB)));   // a vector value, never an alloca
+  typedef R rowvec __attribute__((ext_vector_type(NB)));   // a vector value, never an alloca
   rowvec g;
 #pragma unroll
   for (int c = 0; c < NB; ++c) {
     // the upper part of D is never used: read the mirrored (valid) element instead of branching
-    const float v = D[(int64_t)(NB - 1 - c) * ld + (NB - 1 - r)];
-    g[c] = (c <= r) ? v : 0.f;
+    const R v = D[(int64_t)(NB - 1 - c) * ld + (NB - 1 - r)];
+    g[c] = (c <= r) ? v : R(0);
   }
 
   // ---- Cholesky, right-looking: after step k, g[k] of lane r >= k holds G[r][k]
   bool bad = false;
 #pragma unroll
   for (int k = 0; k < NB; ++k) {
-    const float piv = lane_bcast(g[k], k);
-    bad = bad || !(piv > 0.f);
-    const float root = sqrtf(piv);
-    const float rinv = 1.f / root;
-    const float l = (r == k) ? root : g[k] * rinv;   // lanes r < k hold 0 already
+    const R piv = lane_bcast(g[k], k);
+    bad = bad || !(piv > R(0));
+    const R root = root_of(piv);
+    const R rinv = R(1) / root;
+    const R l = (r == k) ? root : g[k] * rinv;   // lanes r < k hold 0 already
     g[k] = l;
     if (k + 1 < NB) {
       col[r] = l;
       __builtin_amdgcn_wave_barrier();
 #pragma unroll
       for (int c = k + 1; c < NB; ++c) {
-        const float lc = col[c];   // G[c][k], same address in every lane
-        float t = (c <= r) ? g[c] - l * lc : g[c];
+        const R lc = col[c];   // G[c][k], same address in every lane
+        R t = (c <= r) ? g[c] - l * lc : g[c];
         // Pin the update to this step.  Left free, the compiler defers every update until the
         // element is needed and keeps all broadcast values of all steps alive (2000 registers).
         asm volatile("" : "+v"(t));
@@ -153,69 +169,59 @@ __global__ __launch_bounds__(64) void chol_diag_kernel(float *A, float *Minv, in
   rowvec x;
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
-    float acc = (i == r) ? 1.f : 0.f;
+    R acc = (i == r) ? 1 : 0;
 #pragma unroll
     for (int k = 0; k < i; ++k) acc -= Gs[i * GSTR + k] * x[k];
-    float xi = acc / Gs[i * GSTR + i];   // stays 0 for i < j since every term is 0
+    R xi = acc / Gs[i * GSTR + i];   // stays 0 for i < j since every term is 0
     asm volatile("" : "+v"(xi));         // keeps the row reads of later steps from being hoisted
     x[i] = xi;
   }
+  // M_bb[i][j] = G[63-j][63-i]  (i >= j), zero above
+  for (int i = 0; i < NB; ++i)
+    D[(int64_t)i * ld + r] = (i >= r) ? Gs[(NB - 1 - r) * GSTR + (NB - 1 - i)] : R(0);
+  __syncthreads();   // G is not needed any more: its LDS holds X from here on
+  constexpr int XSTR = NB + 1;
 #pragma unroll
-  for (int i = 0; i < NB; ++i) Xs[i][r] = x[i];
+  for (int i = 0; i < NB; ++i) Gs[i * XSTR + r] = x[i];
   __syncthreads();
-
-  // M_bb[i][j] = G[63-j][63-i], Minv_bb[i][j] = X[63-j][63-i]  (i >= j), zero above
-  for (int i = 0; i < NB; ++i) {
-    const bool low = (i >= r);
-    D[(int64_t)i * ld + r] = low ? Gs[(NB - 1 - r) * GSTR + (NB - 1 - i)] : 0.f;
-    Dinv[(int64_t)i * ld + r] = low ? Xs[NB - 1 - r][NB - 1 - i] : 0.f;
-  }
+  // Minv_bb[i][j] = X[63-j][63-i]  (i >= j), zero above
+  for (int i = 0; i < NB; ++i)
+    Dinv[(int64_t)i * ld + r] = (i >= r) ? Gs[(NB - 1 - r) * XSTR + (NB - 1 - i)] : R(0);
   if (__any(bad) && r == 0) atomicMax(status, b + 1);
 }
 
+template <typename R>
 struct Plan {
   int64_t K, Kp;
-  float *A, *Minv, *T;
+  R *A, *Minv, *T;
   uint8_t *dead;
   size_t bytes;
 };
 
-Plan make_plan(int64_t K, void *ws) {
-  Plan p;
+template <typename R>
+Plan<R> make_plan(int64_t K, void *ws) {
+  Plan<R> p;
   p.K = K;
   p.Kp = round_up64(K, NB);
-  const size_t mat = (size_t)p.Kp * (size_t)p.Kp * sizeof(float);
+  const size_t mat = (size_t)p.Kp * (size_t)p.Kp * sizeof(R);
   char *base = reinterpret_cast<char *>(ws);
-  p.A = reinterpret_cast<float *>(base);
-  p.Minv = reinterpret_cast<float *>(base + mat);
-  p.T = reinterpret_cast<float *>(base + 2 * mat);
+  p.A = reinterpret_cast<R *>(base);
+  p.Minv = reinterpret_cast<R *>(base + mat);
+  p.T = reinterpret_cast<R *>(base + 2 * mat);
   p.dead = reinterpret_cast<uint8_t *>(base + 3 * mat);
   p.bytes = 3 * mat + (size_t)round_up64(K, 256);
   return p;
 }
 
-}  // namespace
-
-extern "C" {
-
-size_t gptq_hip_damp_invert_workspace_bytes(int64_t K) {
-  if (K <= 0) return 0;
-  return make_plan(K, nullptr).bytes;
-}
-
-int gptq_hip_damp_invert(void *stream, float *H, float *W, int64_t K, int64_t N, int64_t ldw,
-                         float damping, int fix_dead, float *L, int32_t *status, void *ws,
-                         size_t ws_bytes) {
-  if (!H || !L || !status || K <= 0 || K > 65535 || N < 0 || (N > 0 && (!W || ldw < N)))
-    return GPTQ_HIP_EINVAL;
-  if (!ws || ws_bytes < gptq_hip_damp_invert_workspace_bytes(K)) return GPTQ_HIP_EWORKSPACE;
-  if ((reinterpret_cast<uintptr_t>(ws) & 15) != 0) return GPTQ_HIP_EINVAL;
-  hipStream_t st = as_stream(stream);
-  const Plan p = make_plan(K, ws);
+template <typename R>
+int damp_invert(hipStream_t st, R *H, float *W, int64_t K, int64_t N, int64_t ldw, double damping,
+                int fix_dead, R *L, float *L32, int32_t *status, void *ws) {
+  const Plan<R> p = make_plan<R>(K, ws);
   const int64_t Kp = p.Kp;
   const int nblk = (int)(Kp / NB);
+  constexpr int DT = sizeof(R) == 8 ? GPTQ_HIP_F64 : GPTQ_HIP_F32;
 
-  hipLaunchKernelGGL(damp_diag_kernel, dim3(1), dim3(1024), 0, st, H, K, damping, fix_dead,
+  hipLaunchKernelGGL(damp_diag_kernel<R>, dim3(1), dim3(1024), 0, st, H, K, (R)damping, fix_dead,
                      p.dead, status);
   GPTQ_CHECK_LAUNCH();
   if (N > 0) {
@@ -228,17 +234,17 @@ int gptq_hip_damp_invert(void *stream, float *H, float *W, int64_t K, int64_t N,
   {
     unsigned gx = (unsigned)ceil_div64(Kp, 256);
     if (gx > 32) gx = 32;
-    hipLaunchKernelGGL(pad_copy_kernel, dim3(gx, (unsigned)Kp), dim3(256), 0, st, H, K, p.A, p.Minv,
-                       Kp);
+    hipLaunchKernelGGL(pad_copy_kernel<R>, dim3(gx, (unsigned)Kp), dim3(256), 0, st, H, K, p.A,
+                       p.Minv, Kp);
     GPTQ_CHECK_LAUNCH();
   }
 
   // ---- step 1: H = M^T M, last block first
   for (int b = nblk - 1; b >= 0; --b) {
-    hipLaunchKernelGGL(chol_diag_kernel, dim3(1), dim3(64), 0, st, p.A, p.Minv, Kp, b, status);
+    hipLaunchKernelGGL(chol_diag_kernel<R>, dim3(1), dim3(64), 0, st, p.A, p.Minv, Kp, b, status);
     GPTQ_CHECK_LAUNCH();
     if (b == 0) break;
-    float *panel = p.A + (int64_t)b * NB * Kp;  // rows of block b, columns 0 .. b*NB
+    R *panel = p.A + (int64_t)b * NB * Kp;  // rows of block b, columns 0 .. b*NB
     // panel <- Minv_bb^T * panel   (in place: every workgroup reads only its own columns)
     GemmArgs g;
     g.A = p.Minv + (int64_t)b * NB * Kp + (int64_t)b * NB;
@@ -251,7 +257,8 @@ int gptq_hip_damp_invert(void *stream, float *H, float *W, int64_t K, int64_t N,
     g.alpha = 1.f;
     g.beta = 0.f;
     g.a_kmajor = 1;
-    int rc = gptq_gemm_f32(st, g);
+    g.in_dtype = DT;
+    int rc = gptq_gemm(st, g, (R *)nullptr);
     if (rc) return rc;
     // A[0:b, 0:b] -= panel^T panel  (lower tiles)
     GemmArgs s;
@@ -264,8 +271,9 @@ int gptq_hip_damp_invert(void *stream, float *H, float *W, int64_t K, int64_t N,
     s.alpha = -1.f;
     s.beta = 1.f;
     s.a_kmajor = 1;
+    s.in_dtype = DT;
     s.tri = 2;
-    rc = gptq_gemm_f32(st, s);
+    rc = gptq_gemm(st, s, (R *)nullptr);
     if (rc) return rc;
   }
 
@@ -285,12 +293,13 @@ int gptq_hip_damp_invert(void *stream, float *H, float *W, int64_t K, int64_t N,
     g.alpha = 1.f;
     g.beta = 0.f;
     g.a_kmajor = 0;
+    g.in_dtype = DT;
     g.kskip = 1;
     g.batch = npairs;
     g.strideA = g.strideB = g.strideC = pair_stride;
     g.m_total = (int)(Kp - s);
     g.m_step = (int)(2 * s);
-    int rc = gptq_gemm_f32(st, g);
+    int rc = gptq_gemm(st, g, (R *)nullptr);
     if (rc) return rc;
     // Minv[B rows, A cols] = -Binv * T
     GemmArgs h;
@@ -304,6 +313,7 @@ int gptq_hip_damp_invert(void *stream, float *H, float *W, int64_t K, int64_t N,
     h.alpha = -1.f;
     h.beta = 0.f;
     h.a_kmajor = 0;
+    h.in_dtype = DT;
     h.kskip = 2;
     h.batch = npairs;
     h.strideA = h.strideB = h.strideC = pair_stride;
@@ -311,17 +321,44 @@ int gptq_hip_damp_invert(void *stream, float *H, float *W, int64_t K, int64_t N,
     h.m_step = (int)(2 * s);
     h.k_total = (int)(Kp - s);
     h.k_step = (int)(2 * s);
-    rc = gptq_gemm_f32(st, h);
+    rc = gptq_gemm(st, h, (R *)nullptr);
     if (rc) return rc;
   }
 
   {
     unsigned gx = (unsigned)ceil_div64(K, 256);
     if (gx > 32) gx = 32;
-    hipLaunchKernelGGL(copy_out_kernel, dim3(gx, (unsigned)K), dim3(256), 0, st, p.Minv, Kp, L, K);
+    hipLaunchKernelGGL(copy_out_kernel<R>, dim3(gx, (unsigned)K), dim3(256), 0, st, p.Minv, Kp, L,
+                       L32, K);
     GPTQ_CHECK_LAUNCH();
   }
   return GPTQ_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t gptq_hip_damp_invert_workspace_bytes(int64_t K, int h_dtype) {
+  if (K <= 0) return 0;
+  return h_dtype == GPTQ_HIP_F64 ? make_plan<double>(K, nullptr).bytes
+                                 : make_plan<float>(K, nullptr).bytes;
+}
+
+int gptq_hip_damp_invert(void *stream, void *H, int h_dtype, float *W, int64_t K, int64_t N,
+                         int64_t ldw, double damping, int fix_dead, void *L, float *L32,
+                         int32_t *status, void *ws, size_t ws_bytes) {
+  if (!H || !L || !status || K <= 0 || K > 65535 || N < 0 || (N > 0 && (!W || ldw < N)))
+    return GPTQ_HIP_EINVAL;
+  if (h_dtype != GPTQ_HIP_F32 && h_dtype != GPTQ_HIP_F64) return GPTQ_HIP_EDTYPE;
+  if (!ws || ws_bytes < gptq_hip_damp_invert_workspace_bytes(K, h_dtype)) return GPTQ_HIP_EWORKSPACE;
+  if ((reinterpret_cast<uintptr_t>(ws) & 15) != 0) return GPTQ_HIP_EINVAL;
+  hipStream_t st = as_stream(stream);
+  if (h_dtype == GPTQ_HIP_F64)
+    return damp_invert<double>(st, reinterpret_cast<double *>(H), W, K, N, ldw, damping, fix_dead,
+                               reinterpret_cast<double *>(L), L32, status, ws);
+  return damp_invert<float>(st, reinterpret_cast<float *>(H), W, K, N, ldw, damping, fix_dead,
+                            reinterpret_cast<float *>(L), L32, status, ws);
 }
 
 }  // extern "C"

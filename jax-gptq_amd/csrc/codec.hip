@@ -128,7 +128,8 @@ __global__ __launch_bounds__(TPB) void gather_rows_kernel(const T *in, T *out, i
     out[row * N + c] = in[src * N + c];
 }
 
-__global__ __launch_bounds__(TPB) void gather_sym_kernel(const float *in, float *out, int64_t K,
+template <typename T>
+__global__ __launch_bounds__(TPB) void gather_sym_kernel(const T *in, T *out, int64_t K,
                                                          const int64_t *perm) {
   const int64_t row = blockIdx.y;
   const int64_t src = perm[row];
@@ -302,6 +303,9 @@ int gptq_hip_gather_rows(void *stream, const void *in, void *out, int elem_bytes
     if (elem_bytes == 4)
       hipLaunchKernelGGL(gather_rows_kernel<uint32_t>, grid, dim3(TPB), 0, st,
                          (const uint32_t *)in, (uint32_t *)out + r0 * N, N, perm + r0);
+    else if (elem_bytes == 8)
+      hipLaunchKernelGGL(gather_rows_kernel<uint64_t>, grid, dim3(TPB), 0, st,
+                         (const uint64_t *)in, (uint64_t *)out + r0 * N, N, perm + r0);
     else if (elem_bytes == 2)
       hipLaunchKernelGGL(gather_rows_kernel<uint16_t>, grid, dim3(TPB), 0, st,
                          (const uint16_t *)in, (uint16_t *)out + r0 * N, N, perm + r0);
@@ -315,13 +319,21 @@ int gptq_hip_gather_rows(void *stream, const void *in, void *out, int elem_bytes
   return GPTQ_HIP_OK;
 }
 
-int gptq_hip_gather_sym(void *stream, const float *in, float *out, int64_t K, const int64_t *perm) {
+int gptq_hip_gather_sym(void *stream, const void *in, void *out, int elem_bytes, int64_t K,
+                        const int64_t *perm) {
   if (K <= 0) return GPTQ_HIP_OK;
   if (!in || !out || !perm || K > 65535) return GPTQ_HIP_EINVAL;
   unsigned gx = (unsigned)ceil_div64(K, TPB);
   if (gx > 64) gx = 64;
-  hipLaunchKernelGGL(gather_sym_kernel, dim3(gx, (unsigned)K), dim3(TPB), 0, as_stream(stream), in,
-                     out, K, perm);
+  const dim3 grid(gx, (unsigned)K);
+  if (elem_bytes == 4)
+    hipLaunchKernelGGL(gather_sym_kernel<uint32_t>, grid, dim3(TPB), 0, as_stream(stream),
+                       (const uint32_t *)in, (uint32_t *)out, K, perm);
+  else if (elem_bytes == 8)
+    hipLaunchKernelGGL(gather_sym_kernel<uint64_t>, grid, dim3(TPB), 0, as_stream(stream),
+                       (const uint64_t *)in, (uint64_t *)out, K, perm);
+  else
+    return GPTQ_HIP_EDTYPE;
   GPTQ_CHECK_LAUNCH();
   return GPTQ_HIP_OK;
 }

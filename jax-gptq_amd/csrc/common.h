@@ -30,4 +30,6 @@ template <> __device__ __forceinline__ __hip_bfloat16 from_f32<__hip_bfloat16>(f
   return __float2bfloat16(v);
 }
 
-static inline size_t dtype_size(int dt) { return dt == GPTQ_HIP_F32 ? 4 : 2; }
+static inline size_t dtype_size(int dt) {
+  return dt == GPTQ_HIP_F64 ? 8 : (dt == GPTQ_HIP_F32 ? 4 : 2);
+}

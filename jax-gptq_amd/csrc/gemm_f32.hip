@@ -51,7 +51,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(GemmArgs p) {
 
   const T *A = reinterpret_cast<const T *>(p.A) + (int64_t)z * p.strideA;
   const T *B = reinterpret_cast<const T *>(p.B) + (int64_t)z * p.strideB;
-  float *C = p.C + (int64_t)z * p.strideC;
+  float *C = reinterpret_cast<float *>(p.C) + (int64_t)z * p.strideC;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;

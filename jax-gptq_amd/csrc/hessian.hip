@@ -237,8 +237,9 @@ constexpr int TS = 32;
 // Scale the upper tiles by 1/n and mirror them below the diagonal.  One workgroup
 // per 32x32 tile pair (ti <= tj); the transposed copy goes through LDS so that both
 // the read and the mirrored write are coalesced.
-__global__ __launch_bounds__(TS * 8) void finalize_kernel(float *H, int64_t K, float n) {
-  __shared__ float tile[TS][TS + 1];
+template <typename R>
+__global__ __launch_bounds__(TS * 8) void finalize_kernel(R *H, int64_t K, R n) {
+  __shared__ R tile[TS][TS + 1];
   const int t = blockIdx.x;
   int j = (int)((sqrtf(8.f * (float)t + 1.f) - 1.f) * 0.5f);
   while ((j + 1) * (j + 2) / 2 <= t) ++j;
@@ -247,7 +248,7 @@ __global__ __launch_bounds__(TS * 8) void finalize_kernel(float *H, int64_t K, f
   const int tx = threadIdx.x % TS, ty = threadIdx.x / TS;
   for (int r = ty; r < TS; r += 8) {
     const int64_t row = (int64_t)i * TS + r, col = (int64_t)j * TS + tx;
-    float v = 0.f;
+    R v = 0;
     if (row < K && col < K) {
       v = H[row * K + col] / n;
       // inside a diagonal tile only the upper part is authoritative
@@ -267,8 +268,8 @@ __global__ __launch_bounds__(TS * 8) void finalize_kernel(float *H, int64_t K, f
 
 extern "C" {
 
-size_t gptq_hip_hessian_accumulate_workspace_bytes(int64_t K) {
-  if (K <= 0) return 0;
+size_t gptq_hip_hessian_accumulate_workspace_bytes(int64_t K, int h_dtype) {
+  if (K <= 0 || h_dtype != GPTQ_HIP_F32) return 0;
   const int rs = pick_rs(K);
   if (rs == 1) return 0;
   const int64_t T = ceil_div64(K, HB), ntiles = T * (T + 1) / 2;
@@ -276,15 +277,42 @@ size_t gptq_hip_hessian_accumulate_workspace_bytes(int64_t K) {
 }
 
 int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const int64_t *x_rows,
-                                int n_batches, int x_dtype, int64_t K, float *H, void *ws,
-                                size_t ws_bytes) {
-  if (n_batches < 0 || K <= 0 || K > 46000 || !H) return GPTQ_HIP_EINVAL;
-  if (x_dtype != GPTQ_HIP_F32 && x_dtype != GPTQ_HIP_F16 && x_dtype != GPTQ_HIP_BF16)
+                                int n_batches, int x_dtype, int64_t K, void *Hv, int h_dtype,
+                                void *ws, size_t ws_bytes) {
+  if (n_batches < 0 || K <= 0 || K > 46000 || !Hv) return GPTQ_HIP_EINVAL;
+  if (h_dtype != GPTQ_HIP_F32 && h_dtype != GPTQ_HIP_F64) return GPTQ_HIP_EDTYPE;
+  if (x_dtype != GPTQ_HIP_F32 && x_dtype != GPTQ_HIP_F16 && x_dtype != GPTQ_HIP_BF16 &&
+      !(x_dtype == GPTQ_HIP_F64 && h_dtype == GPTQ_HIP_F64))
     return GPTQ_HIP_EDTYPE;
   if (n_batches > 0 && (!x_ptrs || !x_rows)) return GPTQ_HIP_EINVAL;
-  const size_t need = gptq_hip_hessian_accumulate_workspace_bytes(K);
-  if (need && (!ws || ws_bytes < need)) return GPTQ_HIP_EWORKSPACE;
   hipStream_t st = as_stream(stream);
+  if (h_dtype == GPTQ_HIP_F64) {
+    // fp64 accumulation: one X_b^T X_b product per batch on the fp64 MFMA GEMM, upper tiles
+    for (int b = 0; b < n_batches; ++b) {
+      const int64_t rows = x_rows[b];
+      if (rows < 0 || rows > 2147483647LL) return GPTQ_HIP_EINVAL;
+      if (rows == 0) continue;
+      if (!x_ptrs[b]) return GPTQ_HIP_EINVAL;
+      GemmArgs g;
+      g.A = x_ptrs[b];
+      g.B = x_ptrs[b];
+      g.C = Hv;
+      g.lda = g.ldb = g.ldc = K;
+      g.m = g.n = (int)K;
+      g.k = (int)rows;
+      g.alpha = 1.f;
+      g.beta = 1.f;
+      g.a_kmajor = 1;
+      g.in_dtype = x_dtype;
+      g.tri = 1;
+      const int rc = gptq_gemm_f64(st, g);
+      if (rc) return rc;
+    }
+    return GPTQ_HIP_OK;
+  }
+  float *H = reinterpret_cast<float *>(Hv);
+  const size_t need = gptq_hip_hessian_accumulate_workspace_bytes(K, h_dtype);
+  if (need && (!ws || ws_bytes < need)) return GPTQ_HIP_EWORKSPACE;
   const int T = (int)ceil_div64(K, HB);
   const int ntiles = T * (T + 1) / 2;
   int b0 = 0;
@@ -338,11 +366,18 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
   return GPTQ_HIP_OK;
 }
 
-int gptq_hip_hessian_finalize(void *stream, float *H, int64_t K, double n_samples) {
+int gptq_hip_hessian_finalize(void *stream, void *H, int h_dtype, int64_t K, double n_samples) {
   if (!H || K <= 0 || !(n_samples > 0)) return GPTQ_HIP_EINVAL;
   const int64_t T = ceil_div64(K, TS);
-  hipLaunchKernelGGL(finalize_kernel, dim3((unsigned)(T * (T + 1) / 2)), dim3(TS * 8), 0,
-                     as_stream(stream), H, K, (float)n_samples);
+  const dim3 grid((unsigned)(T * (T + 1) / 2)), block(TS * 8);
+  if (h_dtype == GPTQ_HIP_F32)
+    hipLaunchKernelGGL(finalize_kernel<float>, grid, block, 0, as_stream(stream),
+                       reinterpret_cast<float *>(H), K, (float)n_samples);
+  else if (h_dtype == GPTQ_HIP_F64)
+    hipLaunchKernelGGL(finalize_kernel<double>, grid, block, 0, as_stream(stream),
+                       reinterpret_cast<double *>(H), K, n_samples);
+  else
+    return GPTQ_HIP_EDTYPE;
   GPTQ_CHECK_LAUNCH();
   return GPTQ_HIP_OK;
 }

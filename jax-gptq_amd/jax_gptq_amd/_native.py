@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 # GPTQ_HIP_LIBRARY selects another build of the same ABI (e.g. an instrumented one)
 LIB_PATH = os.environ.get("GPTQ_HIP_LIBRARY") or os.path.join(HERE, "libgptq_hip.so")
 
-F32, F16, BF16 = 0, 1, 2
+F32, F16, BF16, F64 = 0, 1, 2, 3
 OK, EINVAL, EDTYPE, EWORKSPACE, ELAUNCH = 0, 1, 2, 3, 4
 
 _vp, _i64, _i32, _f32, _f64, _sz = (ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float,
@@ -22,16 +22,17 @@ SIGNATURES = {
     "gptq_hip_error_string": (ctypes.c_char_p, [_i32]),
     "gptq_hip_col_params_workspace_bytes": (_sz, [_i64, _i64]),
     "gptq_hip_col_params": (_i32, [_vp, _vp, _i32, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _sz]),
-    "gptq_hip_hessian_accumulate_workspace_bytes": (_sz, [_i64]),
-    "gptq_hip_hessian_accumulate": (_i32, [_vp, _vp, _vp, _i32, _i32, _i64, _vp, _vp, _sz]),
-    "gptq_hip_hessian_finalize": (_i32, [_vp, _vp, _i64, _f64]),
-    "gptq_hip_damp_invert_workspace_bytes": (_sz, [_i64]),
-    "gptq_hip_damp_invert": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _f32, _i32, _vp, _vp, _vp, _sz]),
+    "gptq_hip_hessian_accumulate_workspace_bytes": (_sz, [_i64, _i32]),
+    "gptq_hip_hessian_accumulate": (_i32, [_vp, _vp, _vp, _i32, _i32, _i64, _vp, _i32, _vp, _sz]),
+    "gptq_hip_hessian_finalize": (_i32, [_vp, _vp, _i32, _i64, _f64]),
+    "gptq_hip_damp_invert_workspace_bytes": (_sz, [_i64, _i32]),
+    "gptq_hip_damp_invert": (_i32, [_vp, _vp, _i32, _vp, _i64, _i64, _i64, _f64, _i32, _vp, _vp, _vp,
+                                    _vp, _sz]),
     "gptq_hip_solve_workspace_bytes": (_sz, [_i64, _i64, _i32]),
     "gptq_hip_solve": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _i32, _i32, _vp, _i32, _vp, _vp, _sz]),
     "gptq_hip_process_block": (_i32, [_vp, _vp, _i64, _vp, _i64, _i32, _vp, _vp, _i32, _vp, _i32, _vp, _vp]),
     "gptq_hip_gather_rows": (_i32, [_vp, _vp, _vp, _i32, _i64, _i64, _vp]),
-    "gptq_hip_gather_sym": (_i32, [_vp, _vp, _vp, _i64, _vp]),
+    "gptq_hip_gather_sym": (_i32, [_vp, _vp, _vp, _i32, _i64, _vp]),
     "gptq_hip_pack_int4": (_i32, [_vp, _vp, _i32, _i64, _i64, _i64, _vp]),
     "gptq_hip_unpack_int4": (_i32, [_vp, _vp, _i64, _i64, _i64, _vp]),
     "gptq_hip_quantize_pack": (_i32, [_vp, _vp, _i32, _i64, _i64, _i64, _vp, _vp, _vp]),

@@ -21,6 +21,8 @@ __all__ = [
 ]
 
 _DT = {torch.float32: N.F32, torch.float16: N.F16, torch.bfloat16: N.BF16}
+_DT_H = {torch.float32: N.F32, torch.float64: N.F64}       # element types of H and L
+_DT_X64 = {**_DT, torch.float64: N.F64}                    # batches of the fp64 Hessian
 
 
 def _device():
@@ -41,9 +43,9 @@ def _dev(x, dtype=None):
     return t.contiguous()
 
 
-def _float_dev(x):
+def _float_dev(x, keep_fp64=False):
     t = _dev(x)
-    if t.dtype not in _DT:
+    if t.dtype not in _DT and not (keep_fp64 and t.dtype == torch.float64):
         t = t.to(torch.float32)     # integer / fp64 inputs are promoted to fp32, as jnp would
     return t
 
@@ -112,17 +114,17 @@ def _accumulate_H_step(H, running_mean, n_samples, batch):
     zero, so that the reference's closing formula ``H / n + outer(mean, mean)`` still
     yields ``sum X^T X / n``.
     """
-    batch = _float_dev(batch)
+    batch = _float_dev(batch, keep_fp64=(H.dtype == torch.float64))
     if batch.dim() > 2:
         batch = batch.reshape(-1, batch.shape[-1])
-    _hessian_accumulate(H, [batch])
+    _hessian_accumulate(H, [batch.contiguous()])
     return H, running_mean, n_samples + batch.shape[0]
 
 
 def _hessian_accumulate(H, batches):
     lib = N.load()
     K = H.shape[0]
-    ws = _ws(lib.gptq_hip_hessian_accumulate_workspace_bytes(K))
+    ws = _ws(lib.gptq_hip_hessian_accumulate_workspace_bytes(K, _DT_H[H.dtype]))
     for lo in range(0, len(batches), _MAX_BATCHES_PER_CALL):
         chunk = batches[lo:lo + _MAX_BATCHES_PER_CALL]
         dts = {b.dtype for b in chunk}
@@ -134,19 +136,19 @@ def _hessian_accumulate(H, batches):
         nb = len(chunk)
         ptrs = (ctypes.c_void_p * nb)(*[b.data_ptr() for b in chunk])
         rows = (ctypes.c_int64 * nb)(*[b.shape[0] for b in chunk])
-        N.check(lib.gptq_hip_hessian_accumulate(_stream(), ptrs, rows, nb, _DT[chunk[0].dtype], K,
-                                                _ptr(H), _ptr(ws), ws.numel()),
+        N.check(lib.gptq_hip_hessian_accumulate(_stream(), ptrs, rows, nb, _DT_X64[chunk[0].dtype],
+                                                K, _ptr(H), _DT_H[H.dtype], _ptr(ws), ws.numel()),
                 "hessian_accumulate")
 
 
 def accumulate_H(xs, use_fp64=False):
-    """``H = sum_b X_b^T X_b / n`` over a list of calibration batches (``gptq.py:76-103``)."""
-    if use_fp64:
-        raise NotImplementedError("use_fp64=True is not available on the HIP path")
+    """``H = sum_b X_b^T X_b / n`` over a list of calibration batches (``gptq.py:76-103``);
+    fp32, or fp64 products and sums with ``use_fp64`` (``gptq.py:88``)."""
     lib = N.load()
+    hdt = torch.float64 if use_fp64 else torch.float32
     batches = []
     for x in xs:
-        b = _float_dev(x)
+        b = _float_dev(x, keep_fp64=use_fp64)
         if b.dim() > 2:
             b = b.reshape(-1, b.shape[-1])
         elif b.dim() == 1:
@@ -156,10 +158,11 @@ def accumulate_H(xs, use_fp64=False):
     for b in batches:
         if b.shape[-1] != K:
             raise ValueError("all calibration batches must share the feature dimension")
-    H = torch.zeros((K, K), dtype=torch.float32, device=_device())
+    H = torch.zeros((K, K), dtype=hdt, device=_device())
     _hessian_accumulate(H, batches)
     n = sum(b.shape[0] for b in batches)
-    N.check(lib.gptq_hip_hessian_finalize(_stream(), _ptr(H), K, float(n)), "hessian_finalize")
+    N.check(lib.gptq_hip_hessian_finalize(_stream(), _ptr(H), _DT_H[hdt], K, float(n)),
+            "hessian_finalize")
     return H
 
 
@@ -187,30 +190,44 @@ def get_quantize_params(weight, bits=4):
 
 
 # ------------------------------------------------------------------------------- factor
-def _damp_invert(W, H, damping, fix_dead=True):
+def _damp_invert(W, H, damping, fix_dead=True, want_f32=False):
+    """Returns ``(L, L32, status)``: ``L`` in ``H``'s element type; ``L32`` its fp32 rounding when
+    ``H`` is fp64 and ``want_f32`` is set (``L`` itself when ``H`` is fp32)."""
     lib = N.load()
     K = H.shape[0]
     Nc = 0 if W is None else W.shape[1]
-    L = torch.empty((K, K), dtype=torch.float32, device=H.device)
+    L = torch.empty((K, K), dtype=H.dtype, device=H.device)
+    L32 = None
+    if want_f32:
+        L32 = L if H.dtype == torch.float32 else torch.empty((K, K), dtype=torch.float32,
+                                                             device=H.device)
     status = torch.zeros(2, dtype=torch.int32, device=H.device)
-    ws = _ws(lib.gptq_hip_damp_invert_workspace_bytes(K))
-    N.check(lib.gptq_hip_damp_invert(_stream(), _ptr(H), _ptr(W), K, Nc, Nc, float(damping),
-                                     1 if fix_dead else 0, _ptr(L), _ptr(status), _ptr(ws),
-                                     ws.numel()), "damp_invert")
-    return L, status
+    hdt = _DT_H[H.dtype]
+    ws = _ws(lib.gptq_hip_damp_invert_workspace_bytes(K, hdt))
+    N.check(lib.gptq_hip_damp_invert(_stream(), _ptr(H), hdt, _ptr(W), K, Nc, Nc, float(damping),
+                                     1 if fix_dead else 0, _ptr(L),
+                                     _ptr(L32 if H.dtype == torch.float64 else None),
+                                     _ptr(status), _ptr(ws), ws.numel()), "damp_invert")
+    return L, L32, status
+
+
+def _factor_dtype(mat):
+    t = _dev(mat)
+    return t if t.dtype == torch.float64 else t.to(torch.float32)
 
 
 def _cholesky_inv(mat):
-    """Lower Cholesky factor of ``inv(mat)`` (reference ``gptq.py:44-48``)."""
-    H = _dev(mat, torch.float32).clone()
-    L, _ = _damp_invert(None, H, 0.0, fix_dead=False)
+    """Lower Cholesky factor of ``inv(mat)`` (reference ``gptq.py:44-48``), in fp64 for an fp64
+    matrix and in fp32 otherwise."""
+    H = _factor_dtype(mat).clone()
+    L, _, _ = _damp_invert(None, H, 0.0, fix_dead=False)
     return L
 
 
 def _damp_and_invert(W, H, damping):
     """Dead-feature fix, damping, factor of the inverse (reference ``gptq.py:155-168``).
     ``W`` and ``H`` are updated in place (the reference donates both)."""
-    L, status = _damp_invert(W, H, damping, fix_dead=True)
+    L, _, status = _damp_invert(W, H, damping, fix_dead=True)
     any_nan = bool(status[0].item() != 0)
     return W, L, any_nan
 
@@ -225,7 +242,8 @@ def _permute(W, H):
     Hp = torch.empty_like(H)
     N.check(lib.gptq_hip_gather_rows(_stream(), _ptr(W), _ptr(Wp), W.element_size(), K, Nc,
                                      _ptr(perm)), "gather_rows")
-    N.check(lib.gptq_hip_gather_sym(_stream(), _ptr(H), _ptr(Hp), K, _ptr(perm)), "gather_sym")
+    N.check(lib.gptq_hip_gather_sym(_stream(), _ptr(H), _ptr(Hp), H.element_size(), K, _ptr(perm)),
+            "gather_sym")
     return Wp, Hp, perm
 
 
@@ -283,8 +301,6 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False):
     batches ``[..., K]``.  Returns ``(Q, params)``: ``Q`` the dequantised matrix in ``W``'s
     dtype, ``params`` with ``scale`` / ``zero`` (fp32, one per column) and ``maxq``.
     """
-    if use_fp64:
-        raise NotImplementedError("use_fp64=True is not available on the HIP path")
     Wt = _float_dev(W)
     if Wt.dim() != 2:
         raise ValueError("W must be a 2-D matrix [K, N]")
@@ -304,7 +320,9 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False):
     if actorder:
         W32, H, perm = _permute(W32, H)
 
-    W32, Hinv, any_nan = _damp_and_invert(W32, H, damping)
+    # _damp_and_invert (gptq.py:193) and the fp32 cast of the factor (gptq.py:197) in one call
+    _, Hinv, status = _damp_invert(W32, H, damping, fix_dead=True, want_f32=True)
+    any_nan = bool(status[0].item() != 0)
     if any_nan:
         xs_nan = any(bool(torch.isnan(_float_dev(x)).any()) for x in xs)
         raise ValueError(f"NaN when computing Hinv. Features NaN?: {xs_nan}")

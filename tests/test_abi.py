@@ -50,8 +50,11 @@ def test_workspace_queries_are_pure_host_functions():
     lib = _native.load()
     assert lib.gptq_hip_col_params_workspace_bytes(4096, 11008) > 0
     kp = 4096
-    assert lib.gptq_hip_damp_invert_workspace_bytes(4096) >= 3 * kp * kp * 4
-    assert lib.gptq_hip_damp_invert_workspace_bytes(100) >= 3 * 128 * 128 * 4
+    assert lib.gptq_hip_damp_invert_workspace_bytes(4096, _native.F32) >= 3 * kp * kp * 4
+    assert lib.gptq_hip_damp_invert_workspace_bytes(4096, _native.F64) >= 3 * kp * kp * 8
+    assert lib.gptq_hip_damp_invert_workspace_bytes(100, _native.F32) >= 3 * 128 * 128 * 4
+    assert lib.gptq_hip_hessian_accumulate_workspace_bytes(28672, _native.F32) == 0
+    assert lib.gptq_hip_hessian_accumulate_workspace_bytes(256, _native.F64) == 0
     assert lib.gptq_hip_solve_workspace_bytes(4096, 11008, 128) == 128 * 11008 * 4
     assert lib.gptq_hip_solve_workspace_bytes(4096, 11008, 129) == 0
 

@@ -139,6 +139,4 @@ def test_gptq_argument_errors(G):
     with pytest.raises(ValueError):
         G.gptq(W, [X], block_size=48)          # does not divide K
     with pytest.raises(ValueError):
-        G.gptq(W, [X[:, :32]])                 # feature dimension mismatch
-    with pytest.raises(NotImplementedError):
-        G.gptq(W, [X], use_fp64=True)
+        G.gptq(W, [X[:, :32]], block_size=64)  # feature dimension mismatch
