@@ -47,7 +47,10 @@ __device__ __forceinline__ void load4_f64(const T *src, bool fast, int nv, doubl
   }
 }
 
-template <typename T, bool AK>
+// FAST: every tile is full and every 4-element group aligned (checked on the host), so the
+// loads carry no guards: a load inside a branch would make the compiler wait for it at the
+// join, in front of the MFMAs it is meant to overlap with.
+template <typename T, bool AK, bool FAST>
 __global__ __launch_bounds__(NTHREADS) void gemm_f64_kernel(GemmArgs p) {
   __shared__ __attribute__((aligned(16))) double As[2][BK * LDD];
   __shared__ __attribute__((aligned(16))) double Bs[2][BK * LDD];
@@ -99,18 +102,18 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f64_kernel(GemmArgs p) {
       const int r = tid >> 5, c4 = (tid & 31) * 4;
       const int kk = kt + r;
       const int nv = (kk < ke) ? min(4, m_eff - (m0 + c4)) : 0;
-      load4_f64<T>(A + (int64_t)kk * p.lda + m0 + c4, a_al && m_full && k_full, nv, ra);
+      load4_f64<T>(A + (int64_t)kk * p.lda + m0 + c4, FAST || (a_al && m_full && k_full), nv, ra);
     } else {    // A stored [m][k]: 128 m rows x 8 k, four consecutive k per thread
       const int row = tid >> 1, k4 = (tid & 1) * 4;
       const int mm = m0 + row;
       const int nv = (mm < m_eff) ? min(4, ke - (kt + k4)) : 0;
-      load4_f64<T>(A + (int64_t)mm * p.lda + kt + k4, a_al && m_full && k_full, nv, ra);
+      load4_f64<T>(A + (int64_t)mm * p.lda + kt + k4, FAST || (a_al && m_full && k_full), nv, ra);
     }
     {
       const int r = tid >> 5, c4 = (tid & 31) * 4;
       const int kk = kt + r;
       const int nv = (kk < ke) ? min(4, p.n - (n0 + c4)) : 0;
-      load4_f64<T>(B + (int64_t)kk * p.ldb + n0 + c4, b_al && n_full && k_full, nv, rb);
+      load4_f64<T>(B + (int64_t)kk * p.ldb + n0 + c4, FAST || (b_al && n_full && k_full), nv, rb);
     }
   };
 
@@ -191,10 +194,20 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f64_kernel(GemmArgs p) {
 
 template <typename T>
 void launch(hipStream_t stream, dim3 grid, const GemmArgs &a) {
-  if (a.a_kmajor)
-    hipLaunchKernelGGL((gemm_f64_kernel<T, true>), grid, dim3(NTHREADS), 0, stream, a);
-  else
-    hipLaunchKernelGGL((gemm_f64_kernel<T, false>), grid, dim3(NTHREADS), 0, stream, a);
+  const uintptr_t vb = 4 * sizeof(T) < 16 ? 4 * sizeof(T) : 16;
+  const bool fast = a.m % BM == 0 && a.n % BN == 0 && a.k % BK == 0 && a.m_step == 0 &&
+                    a.k_step == 0 && a.lda % 4 == 0 && a.ldb % 4 == 0 &&
+                    reinterpret_cast<uintptr_t>(a.A) % vb == 0 &&
+                    reinterpret_cast<uintptr_t>(a.B) % vb == 0 &&
+                    (a.batch == 1 || (a.strideA % 4 == 0 && a.strideB % 4 == 0));
+  const dim3 block(NTHREADS);
+  if (a.a_kmajor) {
+    if (fast) hipLaunchKernelGGL((gemm_f64_kernel<T, true, true>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((gemm_f64_kernel<T, true, false>), grid, block, 0, stream, a);
+  } else {
+    if (fast) hipLaunchKernelGGL((gemm_f64_kernel<T, false, true>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((gemm_f64_kernel<T, false, false>), grid, block, 0, stream, a);
+  }
 }
 
 }  // namespace
