@@ -1,14 +1,19 @@
 // Blocked GPTQ column loop: quantise block_size rows with error feedback, then push the
 // accumulated error into all remaining rows with one fp32 MFMA GEMM per block.
 //
-// In-block kernel: the N output channels are independent, so one lane owns one channel.
-// A workgroup of 128 lanes first copies its 128 channels of the block's rows and the
-// block's corner of L into LDS (both coalesced), then works out of LDS only.  The block is
-// walked in sub-blocks of SB rows: the SB rows of a sub-block and their SB errors live in
-// VGPRs (statically indexed, fully unrolled triangle); the rows of the block below the
-// sub-block are then updated in the LDS tile (each lane touches only its own column, so
-// there are no bank conflicts and no barriers).  L is read with broadcast reads (every lane
-// the same address) and the SB factors of one row are consecutive.  W itself is not written.
+// In-block kernel: the N output channels are independent, so one lane owns one channel and a
+// workgroup of four wavefronts owns 64 channels.  The workgroup first copies its channels of
+// the block's rows and the block's corner of L into LDS (all loads of a wavefront in flight
+// at once), then works out of LDS only.  The block is walked in sub-blocks of SB rows:
+//   * the SB rows of a sub-block and their SB errors live in VGPRs (statically indexed,
+//     fully unrolled triangle).  This part is a sequential chain per channel; all four
+//     wavefronts evaluate it redundantly (same instructions, same values), which saves a
+//     broadcast of the errors and costs nothing, since they sit on different SIMDs;
+//   * the rows of the block below the sub-block are then updated in the LDS tile, the rows
+//     dealt round-robin to the four wavefronts; one barrier per sub-block.
+// Each lane touches only its own column of the tile (no bank conflicts); L is read with
+// broadcast reads (every lane the same address), the SB factors of one row are consecutive.
+// W itself is not written.
 //
 // Every floating-point operation is the IEEE operation the reference writes (true
 // division, round-half-even, separate multiply and subtract) and every element receives
@@ -19,7 +24,9 @@
 
 namespace {
 
-constexpr int SOLVE_TPB = 128;
+constexpr int SOLVE_CH = 64;               // channels per workgroup (one per lane)
+constexpr int SOLVE_NW = 4;                // wavefronts per workgroup
+constexpr int SOLVE_TPB = SOLVE_CH * SOLVE_NW;
 
 template <int SB, typename TQ>
 __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
@@ -29,35 +36,52 @@ __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
 #pragma clang fp contract(off)
   extern __shared__ float smem[];
   float *Ln = smem;                 // Ln[j * bs + i] = Lb[j][i]
-  float *Wl = smem + bs * bs;       // Wl[j * SOLVE_TPB + lane] = W[block row j][channel]
+  float *Wl = smem + bs * bs;       // Wl[j * SOLVE_CH + lane] = W[block row j][channel]
   const int tid = threadIdx.x;
-  for (int idx = tid; idx < bs * bs; idx += SOLVE_TPB) {
-    const int j = idx / bs, i = idx - j * bs;
-    Ln[idx] = Lb[(int64_t)j * ldl + i];
-  }
-  const int64_t n = (int64_t)blockIdx.x * SOLVE_TPB + tid;
+  const int lane = tid & (SOLVE_CH - 1);
+  const int wave = tid / SOLVE_CH;
+  const int64_t n = (int64_t)blockIdx.x * SOLVE_CH + lane;
   const bool live = n < N;
-  float *wcol = Wl + tid;
-  if (live) {
-    const float *src = Wb + n;
-    int j = 0;
-    for (; j + 8 <= bs; j += 8) {     // eight independent loads in flight
-      float v[8];
+  const int64_t nl = live ? n : N - 1;   // lanes past the edge shadow the last channel, store nothing
+
+  // ---- stage L's corner and the W tile; loads are unconditional (clamped) and batched so
+  //      that a wavefront has 16 of them in flight before it waits
+  {
+    const int total = bs * bs;
+    for (int base = 0; base < total; base += SOLVE_TPB * 16) {
+      float v[16];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = src[(int64_t)(j + u) * N];
+      for (int u = 0; u < 16; ++u) {
+        const int idx = min(base + u * SOLVE_TPB + tid, total - 1);
+        const int j = idx / bs, i = idx - j * bs;
+        v[u] = Lb[(int64_t)j * ldl + i];
+      }
 #pragma unroll
-      for (int u = 0; u < 8; ++u) wcol[(j + u) * SOLVE_TPB] = v[u];
+      for (int u = 0; u < 16; ++u) {
+        const int idx = base + u * SOLVE_TPB + tid;
+        if (idx < total) Ln[idx] = v[u];
+      }
     }
-    for (; j < bs; ++j) wcol[j * SOLVE_TPB] = src[(int64_t)j * N];
+    const float *src = Wb + nl;
+    for (int j0 = wave; j0 < bs; j0 += SOLVE_NW * 16) {
+      float v[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) v[u] = src[(int64_t)min(j0 + SOLVE_NW * u, bs - 1) * N];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int j = j0 + SOLVE_NW * u;
+        if (j < bs) Wl[j * SOLVE_CH + lane] = v[u];
+      }
+    }
   }
+  const float sc = scale[nl], z = zero[nl];
+  float *wcol = Wl + lane;
   __syncthreads();
-  if (!live) return;
-  const float sc = scale[n], z = zero[n];
 
   for (int r0 = 0; r0 < bs; r0 += SB) {
     float w[SB], e[SB];
 #pragma unroll
-    for (int t = 0; t < SB; ++t) w[t] = wcol[(r0 + t) * SOLVE_TPB];
+    for (int t = 0; t < SB; ++t) w[t] = wcol[(r0 + t) * SOLVE_CH];
     const float *ld = Ln + r0 * bs + r0;  // diagonal sub-block
 #pragma unroll
     for (int t = 0; t < SB; ++t) {
@@ -71,23 +95,26 @@ __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
       q = fminf(fmaxf(q, 0.f), maxq);
       const float qh = sc * (q - z);
       e[t] = (x - qh) / ld[t * bs + t];
-      const int64_t o = (int64_t)(r0 + t) * N + n;
-      if (Qb) Qb[o] = from_f32<TQ>(qh);
-      if (cb) cb[o] = (uint8_t)q;
-      Err[o] = e[t];
+      if (live && (t % SOLVE_NW) == wave) {   // the stores of a sub-block are dealt over the wavefronts
+        const int64_t o = (int64_t)(r0 + t) * N + n;
+        if (Qb) Qb[o] = from_f32<TQ>(qh);
+        if (cb) cb[o] = (uint8_t)q;
+        Err[o] = e[t];
+      }
     }
-    // rows of this block below the sub-block
-#pragma unroll 4
-    for (int j = r0 + SB; j < bs; ++j) {
-      float x = wcol[j * SOLVE_TPB];
+    // rows of this block below the sub-block, round-robin over the wavefronts
+#pragma unroll 2
+    for (int j = r0 + SB + wave; j < bs; j += SOLVE_NW) {
+      float x = wcol[j * SOLVE_CH];
       const float *lr = Ln + j * bs + r0;
 #pragma unroll
       for (int u = 0; u < SB; ++u) {
         const float upd = lr[u] * e[u];
         x = x - upd;
       }
-      wcol[j * SOLVE_TPB] = x;
+      wcol[j * SOLVE_CH] = x;
     }
+    __syncthreads();
   }
 }
 
@@ -95,10 +122,10 @@ template <int SB>
 int launch_block(hipStream_t st, const float *W, int64_t N, const float *L, int64_t ldl, int bs,
                  const float *scale, const float *zero, float maxq, void *Q, int q_dtype,
                  uint8_t *codes, float *Err) {
-  const dim3 grid((unsigned)ceil_div64(N, SOLVE_TPB)), block(SOLVE_TPB);
-  const size_t lds = ((size_t)bs * bs + (size_t)bs * SOLVE_TPB) * sizeof(float);
+  const dim3 grid((unsigned)ceil_div64(N, SOLVE_CH)), block(SOLVE_TPB);
+  const size_t lds = ((size_t)bs * bs + (size_t)bs * SOLVE_CH) * sizeof(float);
   if (lds > 64 * 1024) {
-    // up to 128 KB of the 160 KB LDS of a CU; the limit has to be raised per kernel
+    // up to 96 KB of the 160 KB LDS of a CU; the limit has to be raised per kernel
     const void *fn = q_dtype == GPTQ_HIP_F32
                          ? reinterpret_cast<const void *>(block_quant_kernel<SB, float>)
                          : (q_dtype == GPTQ_HIP_F16
