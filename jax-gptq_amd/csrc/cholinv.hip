@@ -96,11 +96,15 @@ __global__ __launch_bounds__(256) void copy_out_kernel(const R *Minv, int64_t Kp
 // M_bb over A[b,b] (upper part zeroed) and M_bb^-1 = J G^-T J into Minv[b,b].
 //
 // One wavefront and no barrier inside the factorisation: lane r keeps row r of G (64
-// VGPRs) and later column r of G^-1; the loops are fully unrolled.  What another lane needs
-// (the scaled pivot column during the factorisation, a row of G during the inversion) goes
-// through LDS and is read back with broadcast reads (every lane the same address, four
-// values per read).  The block is on the critical path of the blocked factorisation
-// (nothing else can run while it does), so latency is what counts here.
+// VGPRs) and later column r of G^-1; the loops are fully unrolled.  During the factorisation
+// the scaled pivot column is handed to the other lanes with v_readlane (lane c's entry
+// becomes a scalar operand of the update of column c), so a step is two instructions per
+// remaining column and touches no memory; during the inversion a row of G is read from LDS
+// with broadcast reads (every lane the same address, four values per read).  The block is
+// on the critical path of the blocked factorisation (nothing else can run while it does),
+// so latency is what counts here.  Entries above the diagonal of G hold garbage while the
+// factorisation runs (masking them would cost a third instruction per element) and are
+// replaced by zeros when G is written out.
 static_assert(NB == 64, "the diagonal kernel maps one matrix row to one lane of a wavefront");
 constexpr int GSTR = NB + 4;   // LDS row stride of G: rows stay 16-byte aligned
 
@@ -114,13 +118,23 @@ __device__ __forceinline__ double lane_bcast(double v, int lane) {
   o.y = __builtin_amdgcn_readlane(w.y, lane);
   return __builtin_bit_cast(double, o);
 }
-__device__ __forceinline__ float root_of(float v) { return sqrtf(v); }
-__device__ __forceinline__ double root_of(double v) { return sqrt(v); }
+// square root of a pivot and its reciprocal
+__device__ __forceinline__ void root_and_inverse(float piv, float &root, float &rinv) {
+  // hardware reciprocal square root (1 ulp) plus one Newton step instead of the long
+  // correctly-rounded sqrt and division sequences: this sits on the per-step latency chain
+  const float y = __builtin_amdgcn_rsqf(piv);
+  rinv = y * fmaf(-0.5f * piv * y, y, 1.5f);
+  root = piv * rinv;
+}
+__device__ __forceinline__ void root_and_inverse(double piv, double &root, double &rinv) {
+  root = sqrt(piv);
+  rinv = 1.0 / root;
+}
 
 template <typename R>
 __global__ __launch_bounds__(64) void chol_diag_kernel(R *A, R *Minv, int64_t ld, int b,
                                                        int32_t *status) {
-  __shared__ __attribute__((aligned(16))) R col[NB];
+  __shared__ __attribute__((aligned(16))) R dinv[NB];   // 1 / G[k][k]
   __shared__ __attribute__((aligned(16))) R Gs[NB * GSTR];   // G, later reused for X = G^-1
   const int r = threadIdx.x;
   R *D = A + (int64_t)b * NB * ld + (int64_t)b * NB;
@@ -131,9 +145,7 @@ __global__ __launch_bounds__(64) void chol_diag_kernel(R *A, R *Minv, int64_t ld
   rowvec g;
 #pragma unroll
   for (int c = 0; c < NB; ++c) {
-    // the upper part of D is never used: read the mirrored (valid) element instead of branching
-    const R v = D[(int64_t)(NB - 1 - c) * ld + (NB - 1 - r)];
-    g[c] = (c <= r) ? v : R(0);
+    g[c] = D[(int64_t)(NB - 1 - c) * ld + (NB - 1 - r)];   // c > r: finite garbage, never used
   }
 
   // ---- Cholesky, right-looking: after step k, g[k] of lane r >= k holds G[r][k]
@@ -142,27 +154,22 @@ __global__ __launch_bounds__(64) void chol_diag_kernel(R *A, R *Minv, int64_t ld
   for (int k = 0; k < NB; ++k) {
     const R piv = lane_bcast(g[k], k);
     bad = bad || !(piv > R(0));
-    const R root = root_of(piv);
-    const R rinv = R(1) / root;
-    const R l = (r == k) ? root : g[k] * rinv;   // lanes r < k hold 0 already
+    R root, rinv;
+    root_and_inverse(piv, root, rinv);
+    const R l = (r == k) ? root : g[k] * rinv;
     g[k] = l;
-    if (k + 1 < NB) {
-      col[r] = l;
-      __builtin_amdgcn_wave_barrier();
+    if (r == k) dinv[k] = rinv;
 #pragma unroll
-      for (int c = k + 1; c < NB; ++c) {
-        const R lc = col[c];   // G[c][k], same address in every lane
-        R t = (c <= r) ? g[c] - l * lc : g[c];
-        // Pin the update to this step.  Left free, the compiler defers every update until the
-        // element is needed and keeps all broadcast values of all steps alive (2000 registers).
-        asm volatile("" : "+v"(t));
-        g[c] = t;
-      }
-      __builtin_amdgcn_wave_barrier();
+    for (int c = k + 1; c < NB; ++c) {
+      R t = g[c] - l * lane_bcast(l, c);   // G[r][c] -= G[r][k] G[c][k]
+      // Pin the update to this step: left free, the compiler may defer every update until the
+      // element is needed and keep the operands of all steps alive.
+      asm volatile("" : "+v"(t));
+      g[c] = t;
     }
   }
 #pragma unroll
-  for (int c = 0; c < NB; ++c) Gs[r * GSTR + c] = g[c];
+  for (int c = 0; c < NB; ++c) Gs[r * GSTR + c] = (c <= r) ? g[c] : R(0);
   __syncthreads();
 
   // ---- X = G^-1, lane j computes column j: x[i] = (delta_ij - sum_{k<i} G[i][k] x[k]) / G[i][i]
@@ -172,7 +179,7 @@ __global__ __launch_bounds__(64) void chol_diag_kernel(R *A, R *Minv, int64_t ld
     R acc = (i == r) ? 1 : 0;
 #pragma unroll
     for (int k = 0; k < i; ++k) acc -= Gs[i * GSTR + k] * x[k];
-    R xi = acc / Gs[i * GSTR + i];   // stays 0 for i < j since every term is 0
+    R xi = acc * dinv[i];   // stays 0 for i < j since every term is 0
     asm volatile("" : "+v"(xi));         // keeps the row reads of later steps from being hoisted
     x[i] = xi;
   }
