@@ -1,5 +1,6 @@
 // Packed-int4 matmul: out = x @ dequant(Wpacked)  (and the transposed form).
 #include "common.h"
+#include <type_traits>
 
 namespace {
 
@@ -372,9 +373,11 @@ int launch_fwd_mfma_z(hipStream_t st, const FwdPlan &p, const void *x, int64_t M
 // v_mfma_f32_16x16x32_f16 in registers for the whole K loop (no split-K, no partials).
 //   A = activations: staged in their natural [m][k] layout (k contiguous = the operand order)
 //   B = weights: every thread loads 16 packed bytes (16 channels of one packed row), turns
-//       each byte into the fp16 pair {code_lo - zero, code_hi - zero} (0x6400 trick, exact for
-//       the integer zero points GPTQ produces) and stores it at Bs[channel][2*row], so that the
-//       operand fetch is again one 16-byte read of 8 consecutive k.
+//       each byte into the fp16 pair {code_lo - zi, code_hi - zi}, zi = rint(zero) (0x6400 trick:
+//       1024 + code plus the constant -(1024 + zi), exact) and stores it at Bs[channel][2*row],
+//       so that the operand fetch is again one 16-byte read of 8 consecutive k.  The fraction
+//       zero - zi (0 for the zero points GPTQ produces) is applied exactly in the epilogue
+//       through the row sums of the activations, which the staging threads keep in fp32.
 // Row pitch 72 halves and a skew of 8 words per 16-channel group keep both the transposing
 // stores and the operand reads free of bank conflicts.  scale is applied in the epilogue.
 constexpr int GBM = 64, GBK = 64;
@@ -409,11 +412,13 @@ __global__ __launch_bounds__(256) void qmm_fwd_gemm_kernel(const __half *x, int 
   const bool b_thread = tid < B_THREADS;
   const bool b_ok = b_thread && (n0 + b_c) < C;
   const uint8_t *b_src = pk + (int64_t)b_row * C + n0 + b_c;
-  // -(1024 + zero) per staged channel, as fp16 pairs
+  __shared__ float rowsum[GBM];
+  float xsum = 0.f;     // sum over k of this thread's share of activation row a_row
+  // -(1024 + rint(zero)) per staged channel, as fp16 pairs
   uint32_t zc[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
-    const float z = b_ok ? to_f32(zero[n0 + b_c + i]) : 0.f;
+    const float z = b_ok ? rintf(to_f32(zero[n0 + b_c + i])) : 0.f;
     const _Float16 h = (_Float16)(-(1024.f + z));
     zc[i] = __builtin_bit_cast(uint32_t, half2_t{h, h});
   }
@@ -436,8 +441,18 @@ __global__ __launch_bounds__(256) void qmm_fwd_gemm_kernel(const __half *x, int 
   auto store_stage = [&](int buf, int k0, const Stage &st) __attribute__((always_inline)) {
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
     const bool ok0 = a_ok && (k0 + a_k + 8 <= K), ok1 = a_ok && (k0 + a_k + 16 <= K);
-    *reinterpret_cast<u32x4 *>(&As[buf][g_off(a_row, a_k)]) = ok0 ? st.a0 : zero4;
-    *reinterpret_cast<u32x4 *>(&As[buf][g_off(a_row, a_k + 8)]) = ok1 ? st.a1 : zero4;
+    const u32x4 va0 = ok0 ? st.a0 : zero4, va1 = ok1 ? st.a1 : zero4;
+    *reinterpret_cast<u32x4 *>(&As[buf][g_off(a_row, a_k)]) = va0;
+    *reinterpret_cast<u32x4 *>(&As[buf][g_off(a_row, a_k + 8)]) = va1;
+    {
+      const half2_t ones = half2_t{(_Float16)1.f, (_Float16)1.f};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t w0 = va0[i], w1 = va1[i];
+        xsum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, w0), ones, xsum, false);
+        xsum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, w1), ones, xsum, false);
+      }
+    }
     if (b_thread) {
       const bool okb = b_ok && ((k0 >> 1) + b_row < R);
       const u32x4 pbm = okb ? st.b : zero4;
@@ -499,18 +514,26 @@ __global__ __launch_bounds__(256) void qmm_fwd_gemm_kernel(const __half *x, int 
     step(kb + 3 * GBK, s3, s0);
   }
 
+  // the four staging threads of a row are neighbouring lanes
+  xsum += __shfl_xor(xsum, 1);
+  xsum += __shfl_xor(xsum, 2);
+  if ((tid & 3) == 0) rowsum[a_row] = xsum;
+  __syncthreads();
   // acc[i][j][r] = out[m0 + wm*32 + i*16 + 4g + r][n0 + wn*BN/2 + j*16 + l16]
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int n = n0 + wn * (BN / 2) + j * 16 + l16;
     if (n >= C) continue;
     const float sc = to_f32(scale[n]);
+    const float z = to_f32(zero[n]);
+    const float zf = z - rintf(z);
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int m = m0 + wm * 32 + i * 16 + 4 * g + r;
-        if (m < M) out[(int64_t)m * C + n] = __float2half_rn(sc * acc[i][j][r]);
+        const int ml = wm * 32 + i * 16 + 4 * g + r;
+        if (m0 + ml < M)
+          out[(int64_t)(m0 + ml) * C + n] = __float2half_rn(sc * (acc[i][j][r] - zf * rowsum[ml]));
       }
   }
 }
@@ -525,6 +548,203 @@ int launch_fwd_gemm(hipStream_t st, const void *x, int64_t M, const uint8_t *pk,
                      (const TZ *)zero, (const TZ *)scale, (__half *)out);
   GPTQ_CHECK_LAUNCH();
   return GPTQ_HIP_OK;
+}
+
+// ---------------------------------------------------------------------------- transposed
+// out[m, 2j + h] = sum_n x[m, n] * scale[n] * (nibble_h(pk[j, n]) - zero[n]): the VJP of the
+// forward product (op.py:71-81, kernel.py:141-253).  The contraction runs along the packed
+// rows, which is the contiguous axis of the packed matrix, so the weights need no transpose
+// on their way into LDS: a thread loads 16 bytes of one packed row (16 consecutive n), turns
+// them into the 16 + 16 fp16 values (code - zero[n]) * scale[n] of output columns 2j and
+// 2j + 1 (byte permute against 0x64 gives 1024 + code, the subtraction of 1024 is exact, one
+// packed fma applies zero and scale) and stores them k-contiguous, which is the operand
+// order.  Same 64 x 128 x 64 tiles, LDS layout, register ring and MFMA loop as the forward
+// kernel; zero and scale of a stage's 64 channels travel in the ring with the weights.
+template <typename TZ> struct ZsRaw;          // 16 consecutive zero / scale values as loaded
+template <> struct ZsRaw<__half> { static constexpr int NV = 2; };
+template <> struct ZsRaw<__hip_bfloat16> { static constexpr int NV = 2; };
+template <> struct ZsRaw<float> { static constexpr int NV = 4; };
+
+typedef uint32_t qu32x4 __attribute__((ext_vector_type(4)));
+
+// the 16 values of v[] as 8 fp16 pairs, negated if NEG
+template <typename TZ, bool NEG>
+__device__ __forceinline__ void zs_to_half2(const qu32x4 *v, half2_t out[8]) {
+  if constexpr (sizeof(TZ) == 4) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      // (the element is copied out first: a bit cast applied directly to a vector element
+      //  reads element 0 whatever the index)
+      const uint32_t wa = v[i >> 1][(2 * i) & 3], wb = v[i >> 1][(2 * i + 1) & 3];
+      const float a = __builtin_bit_cast(float, wa);
+      const float b = __builtin_bit_cast(float, wb);
+      out[i] = NEG ? half2_t{(_Float16)-a, (_Float16)-b} : half2_t{(_Float16)a, (_Float16)b};
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t w = v[i >> 2][i & 3];
+      if constexpr (std::is_same<TZ, __half>::value) {
+        const half2_t h = __builtin_bit_cast(half2_t, w);
+        out[i] = NEG ? -h : h;
+      } else {   // bf16 pair -> fp32 -> fp16
+        const float a = __builtin_bit_cast(float, w << 16);
+        const float b = __builtin_bit_cast(float, w & 0xFFFF0000u);
+        out[i] = NEG ? half2_t{(_Float16)-a, (_Float16)-b} : half2_t{(_Float16)a, (_Float16)b};
+      }
+    }
+  }
+}
+
+template <typename TZ>
+__global__ __launch_bounds__(256) void qmm_bwd_gemm_kernel(const __half *x, int M, const uint8_t *pk,
+                                                           int R, int C, const TZ *zero,
+                                                           const TZ *scale, __half *out) {
+  constexpr int BN = 128;                       // output columns per tile = 64 packed rows
+  constexpr int A_HALVES = (GBM / 16) * GGROUP;
+  constexpr int B_HALVES = (BN / 16) * GGROUP;
+  constexpr int TN = BN / 32;
+  constexpr int NV = ZsRaw<TZ>::NV;
+  __shared__ __attribute__((aligned(16))) _Float16 As[2][A_HALVES];
+  __shared__ __attribute__((aligned(16))) _Float16 Bs[2][B_HALVES];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, g = lane >> 4, l16 = lane & 15;
+  const int j0 = blockIdx.x * (BN / 2), m0 = blockIdx.y * GBM;
+
+  // A staging: thread -> row tid/4, 16 halves at n = (tid%4)*16 of the stage
+  // B staging: thread -> packed row j0 + tid/4, the same 16 channels
+  const int s_row = tid >> 2, s_k = (tid & 3) * 16;
+  const bool a_ok = (m0 + s_row) < M;
+  const bool b_ok = (j0 + s_row) < R;
+  const __half *a_src = x + (int64_t)(m0 + s_row) * C + s_k;
+  const uint8_t *b_src = pk + (int64_t)(j0 + s_row) * C + s_k;
+
+  struct Stage { qu32x4 a0, a1, b; qu32x4 z[NV], s[NV]; };
+  // unconditional, clamped loads (see the forward kernel); C % 16 == 0 is guaranteed
+  auto load_stage = [&](int k0, Stage &st) __attribute__((always_inline)) {
+    const bool in = (k0 + s_k + 16 <= C);
+    const int n = in ? k0 + s_k : 0;
+    st.a0 = *reinterpret_cast<const qu32x4 *>(a_ok && in ? a_src + k0 : x);
+    st.a1 = *reinterpret_cast<const qu32x4 *>(a_ok && in ? a_src + k0 + 8 : x);
+    st.b = *reinterpret_cast<const qu32x4 *>(b_ok && in ? b_src + k0 : pk);
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      st.z[v] = reinterpret_cast<const qu32x4 *>(zero + n)[v];
+      st.s[v] = reinterpret_cast<const qu32x4 *>(scale + n)[v];
+    }
+  };
+  auto store_stage = [&](int buf, int k0, const Stage &st) __attribute__((always_inline)) {
+    const qu32x4 zero4 = {0u, 0u, 0u, 0u};
+    const bool in = (k0 + s_k + 16 <= C);
+    *reinterpret_cast<qu32x4 *>(&As[buf][g_off(s_row, s_k)]) = (a_ok && in) ? st.a0 : zero4;
+    *reinterpret_cast<qu32x4 *>(&As[buf][g_off(s_row, s_k + 8)]) = (a_ok && in) ? st.a1 : zero4;
+    half2_t sc[8], nzs[8];
+    zs_to_half2<TZ, false>(st.s, sc);
+    zs_to_half2<TZ, true>(st.z, nzs);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) nzs[i] = nzs[i] * sc[i];        // -zero * scale
+    const bool okb = b_ok && in;
+    const half2_t k1024 = half2_t{(_Float16)1024.f, (_Float16)1024.f};
+    qu32x4 lo[2], hi[2];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint32_t w = okb ? st.b[q] : 0u;
+      const uint32_t l = w & 0x0F0F0F0Fu, h = (w >> 4) & 0x0F0F0F0Fu;
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const uint32_t sel = e ? 0x04030402u : 0x04010400u;      // bytes (2e, 2e+1) -> 0x64xx pairs
+        const half2_t cl = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, l, sel)) - k1024;
+        const half2_t ch = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, h, sel)) - k1024;
+        const int i = 2 * q + e;                                   // pair index: n = s_k + 2i, 2i+1
+        const half2_t dl = okb ? cl * sc[i] + nzs[i] : half2_t{(_Float16)0.f, (_Float16)0.f};
+        const half2_t dh = okb ? ch * sc[i] + nzs[i] : half2_t{(_Float16)0.f, (_Float16)0.f};
+        lo[i >> 2][i & 3] = __builtin_bit_cast(uint32_t, dl);
+        hi[i >> 2][i & 3] = __builtin_bit_cast(uint32_t, dh);
+      }
+    }
+    *reinterpret_cast<qu32x4 *>(&Bs[buf][g_off(2 * s_row, s_k)]) = lo[0];
+    *reinterpret_cast<qu32x4 *>(&Bs[buf][g_off(2 * s_row, s_k + 8)]) = lo[1];
+    *reinterpret_cast<qu32x4 *>(&Bs[buf][g_off(2 * s_row + 1, s_k)]) = hi[0];
+    *reinterpret_cast<qu32x4 *>(&Bs[buf][g_off(2 * s_row + 1, s_k + 8)]) = hi[1];
+  };
+
+  floatx4 acc[2][TN];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  Stage s0, s1, s2, s3;
+  load_stage(0, s0);
+  load_stage(GBK, s1);
+  load_stage(2 * GBK, s2);
+  load_stage(3 * GBK, s3);
+  int buf = 0;
+  store_stage(0, 0, s0);
+  __syncthreads();
+  auto step = [&](int k0, Stage &refill, const Stage &next) __attribute__((always_inline)) {
+    if (k0 >= C) return;
+    load_stage(k0 + 4 * GBK, refill);
+#pragma unroll
+    for (int ks = 0; ks < GBK; ks += 32) {
+      half8_t a[2], b[TN];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        a[i] = *reinterpret_cast<const half8_t *>(&As[buf][g_off(wm * 32 + i * 16 + l16, ks + 8 * g)]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        b[j] = *reinterpret_cast<const half8_t *>(
+            &Bs[buf][g_off(wn * (BN / 2) + j * 16 + l16, ks + 8 * g)]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (k0 + GBK < C) store_stage(buf ^ 1, k0 + GBK, next);
+    __syncthreads();
+    buf ^= 1;
+  };
+  for (int kb = 0; kb < C; kb += 4 * GBK) {
+    step(kb, s0, s1);
+    step(kb + GBK, s1, s2);
+    step(kb + 2 * GBK, s2, s3);
+    step(kb + 3 * GBK, s3, s0);
+  }
+
+  // acc[i][j][r] = out[m0 + wm*32 + i*16 + 4g + r][2*j0 + wn*64 + j*16 + l16]
+  const int KO = 2 * R;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int c = 2 * j0 + wn * (BN / 2) + j * 16 + l16;
+    if (c >= KO) continue;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = m0 + wm * 32 + i * 16 + 4 * g + r;
+        if (m < M) out[(int64_t)m * KO + c] = __float2half_rn(acc[i][j][r]);
+      }
+  }
+}
+
+template <typename TZ>
+int launch_bwd_gemm(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
+                    const void *zero, const void *scale, void *out) {
+  const int64_t mt = ceil_div64(M, GBM);
+  if (mt > 65535) return GPTQ_HIP_EINVAL;
+  hipLaunchKernelGGL((qmm_bwd_gemm_kernel<TZ>), dim3((unsigned)ceil_div64(R, 64), (unsigned)mt),
+                     dim3(256), 0, st, (const __half *)x, (int)M, pk, (int)R, (int)C,
+                     (const TZ *)zero, (const TZ *)scale, (__half *)out);
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
+bool bwd_fast_ok(int x_dtype, int64_t M, int64_t R, int64_t C, const void *x, const uint8_t *pk,
+                 const void *zero, const void *scale) {
+  return x_dtype == GPTQ_HIP_F16 && C % 16 == 0 && M >= 1 && R < (1LL << 30) && C < (1LL << 30) &&
+         ((reinterpret_cast<uintptr_t>(pk) | reinterpret_cast<uintptr_t>(x) |
+           reinterpret_cast<uintptr_t>(zero) | reinterpret_cast<uintptr_t>(scale)) & 15) == 0;
 }
 
 bool fwd_fast_ok(int x_dtype, int64_t M, int64_t R, int64_t C, const void *x, const uint8_t *pk) {
@@ -591,6 +811,15 @@ int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const 
       case GPTQ_HIP_F16: return launch_fwd_gemm<__half>(st, x, M, packed, R, C, zero, scale, out);
       case GPTQ_HIP_BF16:
         return launch_fwd_gemm<__hip_bfloat16>(st, x, M, packed, R, C, zero, scale, out);
+      default: return GPTQ_HIP_EDTYPE;
+    }
+  }
+  if (transpose_b && bwd_fast_ok(x_dtype, M, R, C, x, packed, zero, scale)) {
+    switch (zs_dtype) {
+      case GPTQ_HIP_F32: return launch_bwd_gemm<float>(st, x, M, packed, R, C, zero, scale, out);
+      case GPTQ_HIP_F16: return launch_bwd_gemm<__half>(st, x, M, packed, R, C, zero, scale, out);
+      case GPTQ_HIP_BF16:
+        return launch_bwd_gemm<__hip_bfloat16>(st, x, M, packed, R, C, zero, scale, out);
       default: return GPTQ_HIP_EDTYPE;
     }
   }

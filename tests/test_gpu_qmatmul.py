@@ -68,6 +68,27 @@ def test_qmatmul_fp32_x_and_params(OP, M, N, K, transpose):
     _check(got, x, qm, transpose)
 
 
+@pytest.mark.parametrize("transpose", [False, True])
+@pytest.mark.parametrize("zs", ["float32", "float16", "bfloat16"])
+@pytest.mark.parametrize("M", [1, 16, 200])
+def test_qmatmul_fractional_zero_points_and_param_dtypes(OP, M, zs, transpose):
+    """Zero points need not be integers (the reference subtracts them in fp32, kernel.py:98);
+    every kernel of the dispatch table (GEMV, chunked, tiled, transposed) has to honour that."""
+    import torch
+    import jax_gptq_amd.gptq as G
+    K, N = 256, 5120
+    rng = np.random.default_rng(M)
+    codes = rng.integers(0, 16, (K, N)).astype(np.uint8)
+    tdt = getattr(torch, zs)
+    scale = torch.from_numpy(rng.uniform(0.001, 0.01, N).astype(np.float32)).to(tdt)
+    zero = torch.from_numpy(rng.uniform(0.0, 15.0, N).astype(np.float32)).to(tdt)
+    qm_ref = O.QuantizedMatrix(O.pack_colwise(codes), zero.float().numpy(), scale.float().numpy())
+    qm = G.QuantizedMatrix(torch.from_numpy(qm_ref.int_weight).cuda(), zero.cuda(), scale.cuda())
+    x = (rng.standard_normal((M, N if transpose else K)) * (0.05 if transpose else 1.0)).astype(np.float16)
+    got = OP.quantized_matmul(x, qm, transpose_b=transpose)
+    _check(got, x.astype(np.float32), qm_ref, transpose)
+
+
 def test_qmatmul_bf16_x(OP):
     import torch
     qm = _matrix(77, 512, 384, np.float32)
