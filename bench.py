@@ -99,15 +99,16 @@ def bench_qmatmul(reps=240):
                for _ in range(copies)]
         scale = (0.001 + 0.009 * torch.rand(N, generator=g, device="cuda")).to(torch.float16)
         zero = torch.randint(0, 16, (N,), generator=g, device="cuda").to(torch.float16)
-        for M in (1, 16, 128):
-            x = torch.randn((M, K), generator=g, device="cuda").to(torch.float16)
-            y = torch.empty((M, N), dtype=torch.float16, device="cuda")
-            ws = torch.zeros(max(lib.gptq_hip_qmatmul_workspace_bytes(M, K // 2, N, 0), 256),
+        # forward at the decode / small-batch sizes, and the transposed (VJP) product at 2048 rows
+        for (M, tr) in ((1, 0), (16, 0), (128, 0), (2048, 0), (2048, 1)):
+            x = torch.randn((M, N if tr else K), generator=g, device="cuda").to(torch.float16)
+            y = torch.empty((M, K if tr else N), dtype=torch.float16, device="cuda")
+            ws = torch.zeros(max(lib.gptq_hip_qmatmul_workspace_bytes(M, K // 2, N, tr), 256),
                              dtype=torch.uint8, device="cuda")
 
             def call(i):
                 rc = lib.gptq_hip_qmatmul(st, x.data_ptr(), _native.F16, M, iws[i % copies].data_ptr(),
-                                          K // 2, N, zero.data_ptr(), scale.data_ptr(), _native.F16, 0,
+                                          K // 2, N, zero.data_ptr(), scale.data_ptr(), _native.F16, tr,
                                           y.data_ptr(), ws.data_ptr(), ws.numel())
                 assert rc == 0, rc
 
@@ -122,7 +123,7 @@ def bench_qmatmul(reps=240):
             torch.cuda.synchronize()
             us = e0.elapsed_time(e1) * 1e3 / reps
             nbytes = K * N // 2 + 2 * N * 2 + M * K * 2 + M * N * 2
-            out.append({"M": M, "K": K, "N": N, "us": round(us, 2),
+            out.append({"M": M, "K": K, "N": N, "transpose_b": tr, "us": round(us, 2),
                         "algorithmic_bytes": nbytes,
                         "GBps": round(nbytes / us * 1e-3, 1),
                         "hbm_frac": round(nbytes / us * 1e-3 / HBM_PEAK_GBS, 4),
