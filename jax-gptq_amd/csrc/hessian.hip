@@ -32,16 +32,47 @@ struct SyrkArgs {
   int K;
   int T;       // tiles per side
   int RS;      // row slices
+  int chunk;   // 16-bit kernel: rows of the concatenated batches per slice (multiple of 64)
   float *H;
   float *ws;   // [RS][tiles][128][128] when RS > 1
 };
 
-__device__ __forceinline__ void tile_decode(int t, int &ti, int &tj) {
-  int j = (int)((sqrtf(8.f * (float)t + 1.f) - 1.f) * 0.5f);
-  while ((j + 1) * (j + 2) / 2 <= t) ++j;
-  while (j * (j + 1) / 2 > t) --j;
-  ti = t - j * (j + 1) / 2;  // ti <= tj : upper triangle
-  tj = j;
+// upper-triangular pair number t -> (i <= j), column by column
+__device__ __forceinline__ void tri_decode(int t, int &i, int &j) {
+  int c = (int)((sqrtf(8.f * (float)t + 1.f) - 1.f) * 0.5f);
+  while ((c + 1) * (c + 2) / 2 <= t) ++c;
+  while (c * (c + 1) / 2 > t) --c;
+  i = t - c * (c + 1) / 2;
+  j = c;
+}
+
+// Tile number -> upper tile (ti <= tj) of a T x T tile grid, in blocks of 8 x 8 tiles:
+// workgroups that run at the same time have neighbouring numbers, so the ~64 of them that
+// share an XCD's L2 work on one block and read 8 + 8 feature panels of X between them instead
+// of nearly all T (consecutive tiles of a plain column order span whole tile columns).
+constexpr int TBLK = 8;
+__device__ __forceinline__ void tile_decode(int t, int T, int &ti, int &tj) {
+  const int nblk = (T + TBLK - 1) / TBLK;
+  for (int bj = 0; bj < nblk; ++bj) {
+    const int wj = min(TBLK, T - TBLK * bj);        // tile columns in this block column
+    const int off = bj * TBLK * wj;                 // tiles in its bj full-height blocks
+    const int cnt = off + wj * (wj + 1) / 2;        // ... plus the diagonal block
+    if (t < cnt) {
+      if (t < off) {
+        const int bi = t / (TBLK * wj), r = t - bi * (TBLK * wj);
+        ti = TBLK * bi + (r % TBLK);
+        tj = TBLK * bj + (r / TBLK);
+      } else {
+        int a, b;
+        tri_decode(t - off, a, b);
+        ti = TBLK * bj + a;
+        tj = TBLK * bj + b;
+      }
+      return;
+    }
+    t -= cnt;
+  }
+  ti = tj = 0;   // not reached for t < T (T + 1) / 2
 }
 
 // FAST: K % 128 == 0, every batch 16-byte aligned with a multiple of 16 rows.  All slabs are
@@ -65,7 +96,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     t = blockIdx.x - rs * ntiles;
   }
   int ti, tj;
-  tile_decode(t, ti, tj);
+  tile_decode(t, p.T, ti, tj);
   const int m0 = ti * HB, n0 = tj * HB, K = p.K;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
@@ -198,13 +229,226 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
   }
 }
 
+// ---------------------------------------------------------------------------- 16-bit inputs
+// X^T X for fp16 / bf16 batches on v_mfma_f32_32x32x16_{f16,bf16}.  The product of two fp16
+// (or two bf16) numbers is exact in fp32 and the instruction accumulates in fp32, so this
+// computes what the fp32 kernel computes from the widened inputs, up to summation order, at
+// the 16-bit matrix rate.  Same ownership as above (upper tile x row slice, accumulators in
+// registers for the whole launch, partial tiles reduced in slice order).
+//
+// Both MFMA operands want, per lane, 8 consecutive rows (k) of ONE feature, while X is stored
+// with the features contiguous.  The transpose happens in registers on the way into LDS: a
+// thread loads an 8-row x 8-feature block (8 loads of 16 bytes), turns it with 32 byte
+// permutes and writes 8 feature rows of 16 bytes.  LDS
+// holds [feature][k] with a pitch of 72 halves, which makes the operand fetch (16 bytes per
+// lane, 32 consecutive features) conflict free.  Slabs are 64 rows, double buffered (72 KiB).
+constexpr int S16_BK = 64;
+constexpr int S16_PITCH = S16_BK + 8;
+constexpr int S16_OP = HB * S16_PITCH;            // halves per operand buffer
+constexpr int S16_LDS_BYTES = 2 * 2 * S16_OP * 2;
+
+typedef uint32_t hu32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Mfma16;
+template <> struct Mfma16<__half> {
+  typedef _Float16 v8 __attribute__((ext_vector_type(8)));
+  static __device__ __forceinline__ floatx16 mma(v8 a, v8 b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mfma16<__hip_bfloat16> {
+  typedef __bf16 v8 __attribute__((ext_vector_type(8)));
+  static __device__ __forceinline__ floatx16 mma(v8 a, v8 b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+// Requires K % 8 == 0 and 16-byte aligned batches (checked on the host).
+template <typename T>
+__global__ __launch_bounds__(256) void syrk16_kernel(SyrkArgs p) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds16[];   // [buffer][A, B][feature][k]
+  typedef typename Mfma16<T>::v8 v8;
+  const int ntiles = p.T * (p.T + 1) / 2;
+  // Slices are taken out of the concatenation of all batches and handed out slice-major: the
+  // workgroups in flight then work on one or two slices (134 MB each for K = 4096 and 16384
+  // rows), which the 256 MB Infinity Cache keeps while the tiles re-read them.
+  const int rs = blockIdx.x / ntiles, t = blockIdx.x - rs * ntiles;
+  int ti, tj;
+  tile_decode(t, p.T, ti, tj);
+  const int m0 = ti * HB, n0 = tj * HB, K = p.K;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
+
+  // staging role: wavefronts 0-1 bring in the ti panel (operand A), 2-3 the tj panel (B).
+  // Block assignment: 16 neighbouring lanes hold 8 row blocks x 2 feature groups.  Their
+  // transposed 16-byte stores then land 4 words apart (row blocks) and 32 banks apart (feature
+  // groups, 8 x 36 words), i.e. on 64 distinct banks; their loads form 128-byte row segments.
+  const int op = tid >> 7, t7 = tid & 127, kb = t7 & 7, fg = t7 >> 3;
+  const int f0 = (op ? n0 : m0) + fg * 8;
+  const bool f_ok = f0 + 8 <= K;
+  const int f0c = f_ok ? f0 : 0;
+  const bool edge_tile = (n0 + HB > K);   // tj >= ti: the only panels that can run past K
+
+  // this slice: global rows [g0, g0 + left); find the batch and row it starts at and count
+  // its slabs (a slab never crosses a batch boundary)
+  int b = 0, kt = 0, left = 0, nslabs = 0;
+  {
+    const int64_t g0 = (int64_t)rs * p.chunk;
+    int64_t base = 0;
+    bool started = false;
+    int rem = 0;
+    for (int bb = 0; bb < p.nb; ++bb) {
+      const int rows = p.rows[bb];
+      if (!started && g0 < base + rows) {
+        started = true;
+        b = bb;
+        kt = (int)(g0 - base);
+        rem = p.chunk;
+      }
+      if (started && rem > 0) {
+        const int from = (bb == b) ? kt : 0;
+        const int take = min(rows - from, rem);
+        nslabs += (take + S16_BK - 1) / S16_BK;
+        left += take;
+        rem -= take;
+      }
+      base += rows;
+    }
+  }
+
+  // A slab in flight: this thread's 8 x 8 block, the number of its rows that exist and whether
+  // the whole slab is full.  Three slabs are kept in flight (a slab is only ~0.2 us of matrix
+  // work, far less than a trip to memory).  Loads are unconditional, from clamped addresses (a
+  // load inside a branch would be waited for at the join); what does not exist is zeroed
+  // before the store to LDS.
+  struct Slab { hu32x4 r[8]; int nvalid; bool full; };
+  auto load_next = [&](Slab &sl) __attribute__((always_inline)) {
+    const bool live = left > 0;
+    const int bb = live ? b : 0;
+    const int rows = p.rows[bb];
+    const uint16_t *X = reinterpret_cast<const uint16_t *>(p.ptr[bb]);
+    const int k0 = live ? kt : 0;
+    const int avail = live ? min(min(S16_BK, rows - k0), left) : 1;
+    const int row0 = k0 + kb * 8, kend = k0 + avail;
+    sl.nvalid = (live && f_ok) ? kend - row0 : 0;
+    sl.full = live && avail == S16_BK && !edge_tile;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int row = min(row0 + r, kend - 1);
+      sl.r[r] = *reinterpret_cast<const hu32x4 *>(X + (int64_t)row * K + f0c);
+    }
+    // advance (scalar selects only)
+    const int nkt = k0 + avail;
+    const bool wrap = nkt >= rows;
+    left = live ? left - avail : 0;
+    kt = live ? (wrap ? 0 : nkt) : kt;
+    b = (live && wrap) ? b + 1 : b;
+  };
+  auto store_slab = [&](Slab &sl, int buf) __attribute__((always_inline)) {
+    if (!sl.full) {     // ragged end of a batch or slice, or features past K (uniform branch)
+      const hu32x4 zero4 = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int r = 0; r < 8; ++r) sl.r[r] = (r < sl.nvalid) ? sl.r[r] : zero4;
+    }
+    uint16_t *dst = lds16 + (buf * 2 + op) * S16_OP + (fg * 8) * S16_PITCH + kb * 8;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;   // high / low halves of two words
+      hu32x4 o;
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const uint32_t w0 = sl.r[2 * m][c >> 1], w1 = sl.r[2 * m + 1][c >> 1];
+        o[m] = __builtin_amdgcn_perm(w1, w0, sel);                // {X[2m][f], X[2m+1][f]}
+      }
+      *reinterpret_cast<hu32x4 *>(dst + c * S16_PITCH) = o;
+    }
+  };
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  Slab s0, s1, s2;
+  load_next(s0);
+  load_next(s1);
+  load_next(s2);
+  int buf = 0;
+  if (nslabs > 0) store_slab(s0, 0);
+  __syncthreads();
+  // one step: refill the ring slot whose slab is already in LDS, multiply the slab in LDS,
+  // stage the next one.  The main loop runs whole triples with no conditions inside (every
+  // early exit would be another path into the loop head on which the compiler has to assume
+  // the worst about loads still in flight); the last one to three slabs follow it.
+  auto step = [&](Slab &refill, Slab &next, bool do_load, bool has_next) __attribute__((always_inline)) {
+    if (do_load) load_next(refill);
+    const uint16_t *as = lds16 + (buf * 2) * S16_OP + (wm * 64 + l32) * S16_PITCH + lhi * 8;
+    const uint16_t *bs = lds16 + (buf * 2 + 1) * S16_OP + (wn * 64 + l32) * S16_PITCH + lhi * 8;
+#pragma unroll
+    for (int ks = 0; ks < S16_BK; ks += 16) {
+      v8 a[2], bq[2];
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        a[q] = *reinterpret_cast<const v8 *>(as + q * 32 * S16_PITCH + ks);
+        bq[q] = *reinterpret_cast<const v8 *>(bs + q * 32 * S16_PITCH + ks);
+      }
+#pragma unroll
+      for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[ii][j] = Mfma16<T>::mma(a[ii], bq[j], acc[ii][j]);
+    }
+    if (has_next) store_slab(next, buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+  };
+  int i = 0;
+  for (; i + 3 < nslabs; i += 3) {
+    step(s0, s1, true, true);
+    step(s1, s2, true, true);
+    step(s2, s0, true, true);
+  }
+  if (i < nslabs) step(s0, s1, false, i + 1 < nslabs);
+  if (i + 1 < nslabs) step(s1, s2, false, i + 2 < nslabs);
+  if (i + 2 < nslabs) step(s2, s0, false, false);
+
+  if (p.RS == 1) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int col = n0 + wn * 64 + j * 32 + l32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+          if (row < K && col < K) p.H[(int64_t)row * K + col] += acc[i][j][r];
+        }
+      }
+  } else {
+    float *dst = p.ws + ((int64_t)rs * ntiles + t) * (HB * HB);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int col = wn * 64 + j * 32 + l32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = wm * 64 + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+          dst[row * HB + col] = acc[i][j][r];
+        }
+      }
+  }
+}
+
 // H tile += sum over the row slices, in slice order
 __global__ __launch_bounds__(256) void syrk_reduce_kernel(float *H, const float *ws, int K, int T,
                                                           int RS) {
   const int ntiles = T * (T + 1) / 2;
   const int t = blockIdx.x;
   int ti, tj;
-  tile_decode(t, ti, tj);
+  tile_decode(t, T, ti, tj);
   const int m0 = ti * HB, n0 = tj * HB;
   for (int e = threadIdx.x; e < HB * HB / 4; e += 256) {
     const int row = e >> 5, c4 = (e & 31) * 4;
@@ -342,6 +586,34 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
     a.H = H;
     a.ws = reinterpret_cast<float *>(ws);
     const dim3 grid((unsigned)((int64_t)ntiles * a.RS)), block(256);
+    // fp16 / bf16 batches: the 16-bit MFMA kernel, if every batch is 16-byte aligned
+    bool mfma16 = (x_dtype == GPTQ_HIP_F16 || x_dtype == GPTQ_HIP_BF16) && K % 8 == 0;
+    for (int i = 0; i < a.nb && mfma16; ++i)
+      mfma16 = (reinterpret_cast<uintptr_t>(a.ptr[i]) & 15) == 0;
+    if (mfma16) {
+      int64_t total_rows = 0;
+      for (int i = 0; i < a.nb; ++i) total_rows += a.rows[i];
+      const int64_t chunk = round_up64(ceil_div64(total_rows, a.RS), S16_BK);
+      if (chunk > 2147483647LL) return GPTQ_HIP_EINVAL;
+      a.chunk = (int)chunk;
+      const void *fn = x_dtype == GPTQ_HIP_F16
+                           ? reinterpret_cast<const void *>(syrk16_kernel<__half>)
+                           : reinterpret_cast<const void *>(syrk16_kernel<__hip_bfloat16>);
+      if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, S16_LDS_BYTES) !=
+          hipSuccess)
+        return GPTQ_HIP_ELAUNCH;
+      if (x_dtype == GPTQ_HIP_F16)
+        hipLaunchKernelGGL(syrk16_kernel<__half>, grid, block, S16_LDS_BYTES, st, a);
+      else
+        hipLaunchKernelGGL(syrk16_kernel<__hip_bfloat16>, grid, block, S16_LDS_BYTES, st, a);
+      GPTQ_CHECK_LAUNCH();
+      if (a.RS > 1) {
+        hipLaunchKernelGGL(syrk_reduce_kernel, dim3((unsigned)ntiles), dim3(256), 0, st, H, a.ws,
+                           (int)K, T, a.RS);
+        GPTQ_CHECK_LAUNCH();
+      }
+      continue;
+    }
     bool fast = (K % HB == 0);
     for (int i = 0; i < a.nb && fast; ++i)
       fast = (a.rows[i] % HBK == 0) && ((reinterpret_cast<uintptr_t>(a.ptr[i]) & 15) == 0);

@@ -59,6 +59,39 @@ def test_accumulate_H_half_inputs(G, dt):
     assert np.abs(H - ref).max() < TOL * np.abs(ref).max()
 
 
+@pytest.mark.parametrize("dt", ["float16", "bfloat16"])
+@pytest.mark.parametrize("rows,K,nb", [(37, 256, 20), (2048, 768, 2), (33, 104, 4), (5, 136, 2),
+                                       (1, 384, 1), (130, 4096, 3), (64, 128, 1), (700, 520, 5)])
+def test_accumulate_H_16bit_mfma_path(G, rows, K, nb, dt):
+    """fp16 / bf16 batches with K % 8 == 0 run on the 16-bit matrix instructions: products of
+    two such numbers are exact in fp32, so the result must agree with the closed form of the
+    widened inputs, and with the fp32 kernel fed the widened inputs, to fp32 summation error."""
+    import torch
+    rng = np.random.default_rng(rows + K)
+    tdt = getattr(torch, dt)
+    xs_t = [torch.from_numpy(rng.standard_normal((rows, K)).astype(np.float32)).to(tdt).cuda()
+            for _ in range(nb)]
+    H = to_np(G.accumulate_H(xs_t))
+    wide = [x.float() for x in xs_t]
+    ref = _closed_form([x.cpu().numpy() for x in wide])
+    assert H.dtype == np.float32 and np.array_equal(H, H.T)
+    assert np.abs(H - ref).max() < TOL * max(1.0, np.abs(ref).max())
+    H32 = to_np(G.accumulate_H(wide))
+    assert np.abs(H - H32).max() < TOL * max(1.0, np.abs(ref).max())
+
+
+def test_accumulate_H_16bit_unaligned_batch_falls_back(G):
+    """A batch that is not 16-byte aligned takes the fp32 kernel; same result."""
+    import torch
+    rng = np.random.default_rng(77)
+    base = torch.from_numpy(rng.standard_normal((64 * 264 + 1,)).astype(np.float32)).to(torch.float16).cuda()
+    x = base[1:].view(64, 264)          # 2-byte aligned only
+    assert x.data_ptr() % 16 != 0
+    H = to_np(G.accumulate_H([x]))
+    ref = _closed_form([x.float().cpu().numpy()])
+    assert np.abs(H - ref).max() < TOL * np.abs(ref).max()
+
+
 def test_accumulate_H_zero_feature_is_exact_zero(G):
     rng = np.random.default_rng(3)
     x = rng.standard_normal((64, 160)).astype(np.float32)
