@@ -88,9 +88,74 @@ class QuantizedMatrix:
     def tree_unflatten(cls, contraction_axis, children):
         return cls(*children, contraction_axis=contraction_axis)
 
-    def to(self, device):
+    def to(self, *args, **kwargs):
+        """Move to a device.  Element-type requests are ignored: a cast of a packed parameter
+        is the identity (reference ``inverse_convert_type``, ``quantize_interpreter.py:556-557``)."""
+        device = kwargs.get("device")
+        for a in args:
+            if isinstance(a, (str, torch.device, int)):
+                device = a
+        if device is None:
+            return self
         return QuantizedMatrix(self.int_weight.to(device), self.zero.to(device),
                                self.scale.to(device), self.contraction_axis)
+
+    # ---- array-like behaviour inside model functions.  A model written for dense weights
+    # (x @ w, F.linear(x, w), w.T @ x, torch.tensordot(w, x, ...)) runs unchanged on packed ones:
+    # torch hands every call that receives a QuantizedMatrix to transform.quantized_torch_function
+    # (the counterpart of the reference's jaxpr re-interpretation, transform.py:59-135).
+    @classmethod
+    def __torch_function__(cls, func, types, args=(), kwargs=None):
+        from . import transform
+        return transform.quantized_torch_function(func, args, kwargs or {})
+
+    def __matmul__(self, other):
+        return torch.matmul(self, other)
+
+    def __rmatmul__(self, other):
+        return torch.matmul(other, self)
+
+    def dim(self):
+        return len(self.shape)
+
+    ndim = property(dim)
+
+    def size(self, i=None):
+        return torch.Size(self.shape) if i is None else self.shape[i]
+
+    def permute(self, *dims):
+        from . import transform
+        if len(dims) == 1 and isinstance(dims[0], (tuple, list)):
+            dims = tuple(dims[0])
+        return transform.permute_quantized(self, dims)
+
+    def transpose(self, dim0, dim1):
+        perm = list(range(self.dim()))
+        perm[dim0], perm[dim1] = perm[dim1], perm[dim0]
+        return self.permute(*perm)
+
+    def t(self):
+        return self.transpose(0, 1) if self.dim() == 2 else self
+
+    @property
+    def T(self):
+        return self.permute(*reversed(range(self.dim())))
+
+    @property
+    def mT(self):
+        return self.transpose(-2, -1)
+
+    def float(self):
+        return self
+
+    half = bfloat16 = double = contiguous = detach = float
+
+    def __getattr__(self, name):
+        # any other tensor method (w.sum(), w.abs(), ...): unpack, then do as written
+        # (reference transform.py:74-79)
+        if name.startswith("_") or name in ("int_weight", "zero", "scale", "contraction_axis"):
+            raise AttributeError(name)
+        return getattr(unpack_matrix(self), name)
 
 
 def quant_matrix_shape(quantized_matrix, bits=4):

@@ -1,0 +1,297 @@
+"""GPU tests of the callers of the hot path: ``quantize`` (sequential calibration driver) and
+``use_quantized`` (inference dispatch).  They restate the reference's behavioural tests
+(``tests.py:46-138, 158-291``) for ``torch`` model functions, and add what pins the driver:
+its result must equal the layer-by-layer chain of ``gptq`` calls written out by hand."""
+import numpy as np
+import pytest
+
+from helpers import to_np
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def T():
+    import torch
+    return torch
+
+
+@pytest.fixture(scope="module")
+def J():
+    import jax_gptq_amd
+    return jax_gptq_amd
+
+
+def _randn(T, seed, *shape, dtype=None):
+    g = T.Generator(device="cuda")
+    g.manual_seed(seed)
+    return T.randn(shape, generator=g, device="cuda", dtype=dtype or T.float32)
+
+
+def test_single(T, J):
+    """reference test_single (tests.py:46-73) + equality with the direct solve."""
+    G = J.gptq
+    w = _randn(T, 0, 256, 64)
+    orig_w = w.clone()
+    xs = [_randn(T, 1 + i, 32, 256) for i in range(4)]
+    f = lambda w, x: x @ w
+    orig_output = f(orig_w, xs[0])
+    quantized = J.quantize(f, w, xs, block_size=16)
+    assert isinstance(quantized, J.QuantizedMatrix)
+    assert tuple(quantized.int_weight.shape) == (128, 64) and quantized.contraction_axis == 0
+    de_quantized = G.unpack_matrix(quantized)
+    Q, p = G.gptq(orig_w.clone(), xs, block_size=16)
+    assert T.equal(de_quantized, Q)                                   # the driver adds nothing
+    assert T.equal(quantized.int_weight, G.pack_matrix(Q, p).int_weight)
+    new_output = f(de_quantized, xs[0])
+    assert float((orig_output - new_output).abs().mean() / orig_output.abs().mean()) < 0.15
+    assert T.equal(w, Q)          # the parameter buffer now holds the quantised values
+
+
+@pytest.mark.parametrize("use_quantized_activations", [True, False])
+def test_three_linear_layers_are_solved_sequentially(T, J, use_quantized_activations):
+    """reference test_hk (tests.py:75-116): three bias-free fp16 linear layers 256 -> 1024 ->
+    1024 -> 1024, 64 batches of 32."""
+    G = J.gptq
+    dims = [256, 1024, 1024, 1024]
+    params = {f"linear_{i}": {"w": (_randn(T, 10 + i, dims[i], dims[i + 1]) / np.sqrt(dims[i])).half()}
+              for i in range(3)}
+    originals = {k: v["w"].clone() for k, v in params.items()}
+    xs = [_randn(T, 100 + i, 32, 256).half() for i in range(64)]
+
+    def f(p, x):
+        for i in range(3):
+            x = x @ p[f"linear_{i}"]["w"]
+        return x
+
+    quantized_params = J.quantize(f, params, xs, use_quantized_activations=use_quantized_activations)
+    # the same chain by hand: layer i is calibrated on what the layers before it produce
+    acts = list(xs)
+    for i in range(3):
+        W = originals[f"linear_{i}"]
+        Q, p = G.gptq(W.clone(), acts)
+        got = quantized_params[f"linear_{i}"]["w"]
+        assert isinstance(got, J.QuantizedMatrix)
+        assert T.equal(got.int_weight, G.pack_matrix(Q, p).int_weight), f"layer {i}"
+        acts = [a @ (Q if use_quantized_activations else W) for a in acts]
+
+    manual_result = xs[0]
+    for i in range(3):
+        manual_result = manual_result @ G.unpack_matrix(quantized_params[f"linear_{i}"]["w"]).half()
+    new_output = J.use_quantized(f)(quantized_params, xs[0])
+    assert T.allclose(manual_result.float(), new_output.float(), atol=3e-3, rtol=0)
+    kernel_output = J.use_quantized(f, use_kernel=True)(quantized_params, xs[0])
+    assert T.allclose(manual_result.float(), kernel_output.float(), atol=3e-2, rtol=1e-2)
+
+
+def test_transform(T, J):
+    """reference test_transform (tests.py:118-138), 1024 x 1024."""
+    G = J.gptq
+    w = _randn(T, 0, 1024, 1024)
+    xs = [_randn(T, i, 32, 1024) for i in range(16)]
+    f = lambda w, x: x @ w
+    quantized_params = J.quantize(f, w, xs, block_size=16)
+    unpacked_matrix = G.unpack_matrix(quantized_params)
+    manual_result = xs[0] @ unpacked_matrix
+    transform_result = J.use_quantized(f)(quantized_params, xs[0])
+    assert T.allclose(manual_result, transform_result, atol=1e-4, rtol=0)
+
+
+@pytest.fixture(scope="module")
+def simple_model(T, J):
+    w = _randn(T, 0, 256, 64)
+    xs = [_randn(T, 1 + i, 32, 256) for i in range(4)]
+    f = lambda w, x: x @ w
+    w_q = J.quantize(f, w.clone(), xs, block_size=4)
+    return f, w, w_q, xs
+
+
+def test_remat(T, J, simple_model):
+    """reference test_remat (tests.py:158-168)."""
+    f, _, w_q, xs = simple_model
+    x = xs[0].half()
+    expected = x.float() @ J.gptq.unpack_matrix(w_q)
+    result = J.use_quantized(f, use_kernel=True, remat_unpack=True)(w_q, x)
+    assert T.allclose(result.float(), expected, atol=0.03, rtol=0)
+
+
+@pytest.mark.parametrize("use_kernel,remat_unpack", [(True, False), (False, True), (False, False)])
+def test_grad(T, J, simple_model, use_kernel, remat_unpack):
+    """reference test_grad (tests.py:170-186): gradient with respect to x through the packed matrix."""
+    _, _, w_q, xs = simple_model
+    f = lambda x, w: (x @ w)[3].sum()
+    unpacked = J.gptq.unpack_matrix(w_q)
+    x = xs[0].clone().requires_grad_(True)
+    J.use_quantized(f, use_kernel=use_kernel, remat_unpack=remat_unpack)(x, w_q).backward()
+    x2 = xs[0].clone().requires_grad_(True)
+    f(x2, unpacked).backward()
+    assert T.allclose(x.grad, x2.grad, atol=1e-1, rtol=0)
+    assert float(x.grad[3].abs().sum()) > 0 and float(x.grad[0].abs().sum()) == 0
+
+
+@pytest.mark.parametrize("w_contract", range(3))
+@pytest.mark.parametrize("x_contract", range(2))
+def test_weird_dots(T, J, w_contract, x_contract):
+    """reference test_weird_dots (tests.py:188-217): a 3-D weight contracted along any axis."""
+    w_shape, x_shape = [47, 768], [32]
+    w_shape.insert(w_contract, 256)
+    x_shape.insert(x_contract, 256)
+    w = _randn(T, 9999, *w_shape)
+    xs = [_randn(T, 10 * i, *x_shape) for i in range(10)]
+    f = lambda w, x: T.tensordot(w, x, dims=([w_contract], [x_contract]))
+    expected_output = f(w.clone(), xs[0])
+    quantized_params = J.quantize(f, w, xs, block_size=16)
+    assert isinstance(quantized_params, J.QuantizedMatrix)
+    assert quantized_params.contraction_axis == w_contract and tuple(quantized_params.shape) == tuple(w_shape)
+    quantized_output = J.use_quantized(f)(quantized_params, xs[0])
+    mean_error = (expected_output - quantized_output).abs().mean()
+    assert float(mean_error / expected_output.abs().mean()) < 0.1
+
+
+def test_conv(T, J):
+    """reference test_conv (tests.py:219-254): a 1x1 convolution is the same product."""
+    import torch.nn.functional as F
+    w = _randn(T, 0, 79, 32)
+    xs = [_randn(T, i, 11, 32, 13) for i in range(1, 20)]
+    matmul_f = lambda w, x: T.tensordot(w, x, dims=([1], [1]))
+    conv_f = lambda w, x: F.conv1d(x, w)
+    quantized_params = J.quantize(matmul_f, w.clone(), xs, block_size=16)
+    quantized_output = J.use_quantized(matmul_f)(quantized_params, xs[0])
+    conv_quantized = J.quantize(conv_f, w.clone()[:, :, None], xs, block_size=16)
+    unpacked_w = J.gptq.unpack_matrix(quantized_params)
+    unpacked_kernel = J.gptq.unpack_matrix(conv_quantized)
+    assert int((unpacked_w != unpacked_kernel[:, :, 0]).sum()) < 10
+    quantized_conv_output = J.use_quantized(conv_f)(conv_quantized, xs[0]).permute(1, 0, 2)
+    assert float((quantized_output - quantized_conv_output).abs().max()) < 1e-4
+
+
+def test_transpose(T, J):
+    """reference test_transpose (tests.py:256-278): the parameter is transposed before use."""
+    w = _randn(T, 9999, 256, 1024)
+    w_copy = w.clone()
+    xs = [_randn(T, i, 256, 32) for i in range(10)]
+    f = lambda w, x: w.T @ x
+    quantized_params = J.quantize(f, w, xs, block_size=16)
+    assert isinstance(quantized_params, J.QuantizedMatrix)
+    assert tuple(quantized_params.shape) == (256, 1024) and quantized_params.contraction_axis == 0
+    quantized_output = J.use_quantized(f)(quantized_params, xs[0])
+    unpacked = J.gptq.unpack_matrix(quantized_params)
+    manual_result = unpacked.T @ xs[0]
+    assert float((unpacked - w_copy).abs().mean()) < 0.15
+    assert T.allclose(manual_result, quantized_output, atol=1e-4)
+    # same codes as solving the [K, N] matrix directly
+    Q, p = J.gptq.gptq(w_copy.clone(), [x.T for x in xs], block_size=16)
+    assert T.equal(unpacked, Q)
+
+
+def test_reuse(T, J, simple_model):
+    """reference test_reuse (tests.py:280-291): other uses of a parameter do not confuse the driver."""
+    _, w, _, xs = simple_model
+
+    def f(w, x):
+        intermediate = w.T       # noqa: F841  (unused on purpose)
+        answer = w.T @ x.T
+        answer = answer + w.sum()
+        return answer
+
+    quantized_params = J.quantize(f, w.clone(), xs, block_size=16)
+    assert isinstance(quantized_params, J.QuantizedMatrix)
+    quantized_output = J.use_quantized(f)(quantized_params, xs[0])
+    dense = J.gptq.unpack_matrix(quantized_params)
+    assert T.allclose(quantized_output, dense.T @ xs[0].T + dense.sum(), atol=1e-3)
+
+
+def test_parameter_used_by_two_products_is_quantized_once(T, J):
+    w = _randn(T, 3, 128, 128)
+    xs = [_randn(T, i, 16, 128) for i in range(4)]
+    f = lambda w, x: (x @ w) @ w
+    q = J.quantize(f, w.clone(), xs, block_size=16)
+    Q, p = J.gptq.gptq(w.clone(), xs, block_size=16)
+    assert T.equal(J.gptq.unpack_matrix(q), Q)
+
+
+def test_other_leaves_pass_through_and_errors(T, J):
+    params = {"w": _randn(T, 0, 64, 32), "b": _randn(T, 1, 32), "n": 3, "unused": _randn(T, 2, 8, 8)}
+    xs = [_randn(T, i, 8, 64) for i in range(3)]
+    f = lambda p, x: (x @ p["w"] + p["b"]) * p["n"]
+    out = J.quantize(f, params, xs, block_size=16)
+    assert isinstance(out["w"], J.QuantizedMatrix)
+    assert out["b"] is params["b"] and out["n"] == 3 and out["unused"] is params["unused"]
+    with pytest.raises(NotImplementedError):
+        J.quantize(lambda p, x: p["w"].T @ p["w"], {"w": _randn(T, 0, 64, 32)}, xs, block_size=16)
+    with pytest.raises(ValueError):
+        J.quantize(f, {"w": _randn(T, 0, 64, 32), "b": params["b"], "n": 1}, xs, block_size=48)
+    with pytest.raises(ZeroDivisionError):
+        J.quantize(lambda p, x: x @ p["w"] / 0 if False else 1 // 0, params, xs)
+
+
+def _gpt2_params(T, d, n_layer, vocab, n_ctx, seed=0):
+    g = T.Generator(device="cuda")
+    g.manual_seed(seed)
+    n = lambda *s: 0.02 * T.randn(s, generator=g, device="cuda")
+    p = {"wte": n(vocab, d), "wpe": n(n_ctx, d), "ln_f": {"g": T.ones(d, device="cuda"), "b": T.zeros(d, device="cuda")},
+         "h": []}
+    for _ in range(n_layer):
+        p["h"].append({
+            "ln_1": {"g": T.ones(d, device="cuda"), "b": T.zeros(d, device="cuda")},
+            "ln_2": {"g": T.ones(d, device="cuda"), "b": T.zeros(d, device="cuda")},
+            "attn": {"c_attn": {"w": n(d, 3 * d), "b": T.zeros(3 * d, device="cuda")},
+                     "c_proj": {"w": n(d, d), "b": T.zeros(d, device="cuda")}},
+            "mlp": {"c_fc": {"w": n(d, 4 * d), "b": T.zeros(4 * d, device="cuda")},
+                    "c_proj": {"w": n(4 * d, d), "b": T.zeros(d, device="cuda")}}})
+    return p
+
+
+def _gpt2(n_head):
+    import torch
+    import torch.nn.functional as F
+
+    def forward(p, tokens):
+        B, S = tokens.shape
+        d = p["wte"].shape[1]
+        x = F.embedding(tokens, p["wte"]) + p["wpe"][:S]
+        mask = torch.ones(S, S, dtype=torch.bool, device=tokens.device).tril()
+        for blk in p["h"]:
+            h = F.layer_norm(x, (d,), blk["ln_1"]["g"], blk["ln_1"]["b"])
+            qkv = h @ blk["attn"]["c_attn"]["w"] + blk["attn"]["c_attn"]["b"]
+            q, k, v = (t.reshape(B, S, n_head, d // n_head).transpose(1, 2) for t in qkv.split(d, dim=-1))
+            att = (q @ k.transpose(-1, -2)) / (d // n_head) ** 0.5
+            att = att.masked_fill(~mask, float("-inf")).softmax(-1)
+            a = (att @ v).transpose(1, 2).reshape(B, S, d)
+            x = x + a @ blk["attn"]["c_proj"]["w"] + blk["attn"]["c_proj"]["b"]
+            h = F.layer_norm(x, (d,), blk["ln_2"]["g"], blk["ln_2"]["b"])
+            h = F.gelu(h @ blk["mlp"]["c_fc"]["w"] + blk["mlp"]["c_fc"]["b"])
+            x = x + h @ blk["mlp"]["c_proj"]["w"] + blk["mlp"]["c_proj"]["b"]
+        x = F.layer_norm(x, (d,), p["ln_f"]["g"], p["ln_f"]["b"])
+        return x @ p["wte"].T          # tied output head
+    return forward
+
+
+def test_gpt2_shaped_model_through_the_driver(T, J):
+    """A GPT-2-shaped decoder (random init N(0, 0.02), uniform random tokens) through
+    ``quantize`` and back through ``use_quantized``: every Linear weight and the tied
+    embedding / output matrix are packed, nothing else is touched, and the packed model
+    reproduces the dense one."""
+    d, n_layer, vocab, n_ctx, n_head = 128, 2, 512, 64, 4
+    params = _gpt2_params(T, d, n_layer, vocab, n_ctx)
+    import copy
+    dense = copy.deepcopy(params)
+    g = T.Generator(device="cuda")
+    g.manual_seed(5)
+    batches = [T.randint(0, vocab, (4, n_ctx), generator=g, device="cuda") for _ in range(8)]
+    f = _gpt2(n_head)
+    ref = f(dense, batches[0])
+    q = J.quantize(f, params, batches, block_size=64)
+    for blk in q["h"]:
+        for name, sub in (("attn", "c_attn"), ("attn", "c_proj"), ("mlp", "c_fc"), ("mlp", "c_proj")):
+            assert isinstance(blk[name][sub]["w"], J.QuantizedMatrix)
+            assert isinstance(blk[name][sub]["b"], T.Tensor)
+        assert isinstance(blk["ln_1"]["g"], T.Tensor)
+    assert isinstance(q["wte"], J.QuantizedMatrix)
+    assert tuple(q["wte"].shape) == (vocab, d) and q["wte"].contraction_axis == 1   # used as wte.T
+    assert isinstance(q["wpe"], T.Tensor)
+    out = J.use_quantized(f)(q, batches[0])
+    out_k = J.use_quantized(f, use_kernel=True)(q, batches[0])
+    rel = float((out - ref).norm() / ref.norm())
+    assert rel < 0.25, rel
+    assert float((out_k - out).norm() / out.norm()) < 2e-2
