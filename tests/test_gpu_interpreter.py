@@ -295,3 +295,32 @@ def test_gpt2_shaped_model_through_the_driver(T, J):
     rel = float((out - ref).norm() / ref.norm())
     assert rel < 0.25, rel
     assert float((out_k - out).norm() / out.norm()) < 2e-2
+
+
+def test_gpt2_small_full_shape(T, J):
+    """GPT-2-small-shaped model at full size (12 layers, d = 768, 12 heads, MLP 3072, vocab
+    50257), 128 sequences x 512 uniform random tokens in 16 batches: all 48 Linear weights and
+    the tied embedding matrix are packed; the packed model tracks the dense one and the kernel
+    path tracks the unpack path."""
+    import copy
+    d, n_layer, vocab, n_ctx, n_head = 768, 12, 50257, 512, 12
+    params = _gpt2_params(T, d, n_layer, vocab, n_ctx)
+    dense = copy.deepcopy(params)
+    g = T.Generator(device="cuda")
+    g.manual_seed(5)
+    batches = [T.randint(0, vocab, (8, n_ctx), generator=g, device="cuda") for _ in range(16)]
+    f = _gpt2(n_head)
+    with T.no_grad():
+        ref = f(dense, batches[0])
+        q = J.quantize(f, params, batches)
+        packed = [blk[m][s]["w"] for blk in q["h"] for m, s in
+                  (("attn", "c_attn"), ("attn", "c_proj"), ("mlp", "c_fc"), ("mlp", "c_proj"))]
+        assert len(packed) == 48 and all(isinstance(w, J.QuantizedMatrix) for w in packed)
+        assert isinstance(q["wte"], J.QuantizedMatrix) and tuple(q["wte"].int_weight.shape) == (vocab, d // 2)
+        out = J.use_quantized(f)(q, batches[0])
+        assert float((out - ref).norm() / ref.norm()) < 0.3
+        import warnings
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")      # the embedding lookup is not a product: it unpacks
+            out_k = J.use_quantized(f, use_kernel=True)(q, batches[0])
+        assert float((out_k - out).norm() / out.norm()) < 5e-3
