@@ -14,6 +14,7 @@ Prints ONE JSON line.  Besides the contract keys it carries
   roofline       the dominant kernel (X^T X, fp32 MFMA) against the fp32 matrix peak,
   cpu_baseline   the NumPy/SciPy oracle timed on this host on a bounded sample,
   phases_ms      per-phase GPU time of one step,
+  fp16_calibration  the same layer with the calibration rows stored in fp16,
   qmatmul        packed-int4 matmul at M = 1, 16, 128 against the HBM roofline
                  (weights rotated over > 512 MB of copies so that they come from HBM).
 """
@@ -31,6 +32,7 @@ for _p in (ROOT, os.path.join(ROOT, "jax-gptq_amd")):
 K_IN, N_OUT = 4096, 11008
 N_BATCH, ROWS = 128, 2048
 FP32_MFMA_PEAK_TFLOPS = 157.3
+MFMA16_PEAK_TFLOPS = 2500.0
 HBM_PEAK_GBS = 8000.0
 
 
@@ -233,16 +235,20 @@ def main():
     executed_flop = flop_per_launch * (tiles + 1) / (2 * tiles)   # upper 128x128 tiles only
     achieved = flop_per_launch / (hess_ms * 1e-3) * 1e-12
     executed = executed_flop / (hess_ms * 1e-3) * 1e-12
-    roofline = {"kernel": "syrk_kernel<float> (X^T X, fp32 MFMA, upper tiles)", "bound": "mfma",
-                "achieved": round(achieved, 2), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
+    wide = args.x_dtype == "float32"
+    peak = FP32_MFMA_PEAK_TFLOPS if wide else MFMA16_PEAK_TFLOPS
+    roofline = {"kernel": "syrk_kernel<float> (X^T X, fp32 MFMA, upper tiles)" if wide else
+                          f"syrk16_kernel ({args.x_dtype} X^T X, 16-bit MFMA with fp32 accumulation, upper tiles)",
+                "bound": "mfma",
+                "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+                "frac": round(achieved / peak, 4),
                 # bytes per launch beyond L2 from rocprofv3 FETCH_SIZE + WRITE_SIZE (scaled by what the
                 # counters read for a 1 GiB copy: x2.000 / x1.000), summary kept under profiles/
-                "traffic": 6.48e10,
+                "traffic": 6.48e10 if wide else None,
                 "flop_per_launch": flop_per_launch, "avg_launch_ms": round(hess_ms, 4),
                 "launches_per_step": 1,
                 "executed_tflops": round(executed, 2),
-                "executed_frac": round(executed / FP32_MFMA_PEAK_TFLOPS, 4),
+                "executed_frac": round(executed / peak, 4),
                 "note": "achieved counts the algorithmic 2*n*K^2 flop; the kernel computes only the "
                         "upper tiles of the symmetric result (executed_*), which is what MFMA "
                         "utilisation counters see"}
@@ -251,13 +257,25 @@ def main():
         "metric": "GPTQ s/layer @4096x11008", "value": round(sec_per_step, 5), "unit": "s/layer",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(sec_per_step * 1e3, 3), "higher_is_better": False, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "vs_baseline": None, "dtype": "f32" if wide else "f16/bf16 products, f32 sums", "data": "synthetic",
         "config": {"workload": "llama7b_up_proj W[4096,11008] fp16, 128x[2048,4096] "
                                f"{args.x_dtype} calibration (262144 tokens), 4-bit, damp 0.01, block 128"},
         "roofline": roofline,
         "xtx_tflops": round(achieved, 2),
         "phases_ms": phases,
     }
+    if wide and args.section == "all":
+        # the same layer with the calibration rows stored in fp16 (as the activations of an fp16
+        # model are): products of fp16 numbers are exact in fp32, the Hessian runs on 16-bit MFMA
+        xs16 = [x.to(torch.float16) for x in xs]
+        one_layer(G, W, xs16)
+        t16 = {}
+        for _ in range(max(1, args.steps)):
+            one_layer(G, W, xs16, t16)
+        ph16 = {k: round(sum(v) / len(v), 3) for k, v in t16.items()}
+        result["fp16_calibration"] = {"ms_per_layer": round(sum(ph16.values()), 3), "phases_ms": ph16,
+                                      "xtx_tflops": round(flop_per_launch / (ph16["hessian"] * 1e-3) * 1e-12, 2)}
+        del xs16
     if not args.no_qmatmul:
         qm = bench_qmatmul()
         result["qmatmul"] = qm
