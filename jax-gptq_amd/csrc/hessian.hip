@@ -272,7 +272,19 @@ __global__ __launch_bounds__(256) void syrk16_kernel(SyrkArgs p) {
   // Slices are taken out of the concatenation of all batches and handed out slice-major: the
   // workgroups in flight then work on one or two slices (134 MB each for K = 4096 and 16384
   // rows), which the 256 MB Infinity Cache keeps while the tiles re-read them.
-  const int rs = blockIdx.x / ntiles, t = blockIdx.x - rs * ntiles;
+  // Workgroup ids are dealt round-robin to the 8 XCDs, each with an L2 of its own, and ~64
+  // workgroups run on an XCD at a time.  Renumber so that those 64 are consecutive work items
+  // (one 8 x 8 block of tiles of one slice, 16 feature panels between them) instead of every
+  // eighth one: item = ((q / 64) * 8 + xcd) * 64 + q % 64 for id = 8 q + xcd.
+  unsigned item = blockIdx.x;
+  {
+    const unsigned full = gridDim.x & ~511u;
+    if (item < full) {
+      const unsigned xcd = item & 7u, q = item >> 3;
+      item = ((q >> 6) * 8u + xcd) * 64u + (q & 63u);
+    }
+  }
+  const int rs = (int)item / ntiles, t = (int)item - rs * ntiles;
   int ti, tj;
   tile_decode(t, p.T, ti, tj);
   const int m0 = ti * HB, n0 = tj * HB, K = p.K;
@@ -280,10 +292,17 @@ __global__ __launch_bounds__(256) void syrk16_kernel(SyrkArgs p) {
   const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
 
   // staging role: wavefronts 0-1 bring in the ti panel (operand A), 2-3 the tj panel (B).
-  // Block assignment: 16 neighbouring lanes hold 8 row blocks x 2 feature groups.  Their
-  // transposed 16-byte stores then land 4 words apart (row blocks) and 32 banks apart (feature
-  // groups, 8 x 36 words), i.e. on 64 distinct banks; their loads form 128-byte row segments.
-  const int op = tid >> 7, t7 = tid & 127, kb = t7 & 7, fg = t7 >> 3;
+  // Block assignment: 16 neighbouring lanes hold the 16 feature groups of one row block, so a
+  // load instruction reads four 256-byte row segments (the vector memory pipe was measured to
+  // cost about as much per contiguous segment as per instruction: eight 128-byte segments took
+  // 8.3 ms for the loads alone, four 256-byte ones 5.6 ms).  The transposed 16-byte stores of
+  // those 16 lanes would all fall on two groups of four banks (feature groups are 8 x 36 words
+  // = 32 banks apart), so the 8-row blocks of a feature row are stored in a swizzled order:
+  // block kb of feature group fg goes to position kb ^ (fg >> 1).  Bank = 32 (fg & 1) +
+  // 4 (kb ^ (fg >> 1)) + const: 16 distinct groups of four banks.  A reader's 16 neighbouring
+  // lanes (16 consecutive features, i.e. two feature groups 2h, 2h + 1) share the swizzle h.
+  const int op = tid >> 7, t7 = tid & 127, fg = t7 & 15, kb = t7 >> 4;
+  const int kb_sw = kb ^ (fg >> 1);
   const int f0 = (op ? n0 : m0) + fg * 8;
   const bool f_ok = f0 + 8 <= K;
   const int f0c = f_ok ? f0 : 0;
@@ -350,7 +369,7 @@ __global__ __launch_bounds__(256) void syrk16_kernel(SyrkArgs p) {
 #pragma unroll
       for (int r = 0; r < 8; ++r) sl.r[r] = (r < sl.nvalid) ? sl.r[r] : zero4;
     }
-    uint16_t *dst = lds16 + (buf * 2 + op) * S16_OP + (fg * 8) * S16_PITCH + kb * 8;
+    uint16_t *dst = lds16 + (buf * 2 + op) * S16_OP + (fg * 8) * S16_PITCH + kb_sw * 8;
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
       const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;   // high / low halves of two words
@@ -379,21 +398,29 @@ __global__ __launch_bounds__(256) void syrk16_kernel(SyrkArgs p) {
   int buf = 0;
   if (nslabs > 0) store_slab(s0, 0);
   __syncthreads();
+  int sw_a[2], sw_b[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    sw_a[q] = ((wm * 64 + q * 32 + l32) >> 4) & 7;
+    sw_b[q] = ((wn * 64 + q * 32 + l32) >> 4) & 7;
+  }
   // one step: refill the ring slot whose slab is already in LDS, multiply the slab in LDS,
   // stage the next one.  The main loop runs whole triples with no conditions inside (every
   // early exit would be another path into the loop head on which the compiler has to assume
   // the worst about loads still in flight); the last one to three slabs follow it.
   auto step = [&](Slab &refill, Slab &next, bool do_load, bool has_next) __attribute__((always_inline)) {
     if (do_load) load_next(refill);
-    const uint16_t *as = lds16 + (buf * 2) * S16_OP + (wm * 64 + l32) * S16_PITCH + lhi * 8;
-    const uint16_t *bs = lds16 + (buf * 2 + 1) * S16_OP + (wn * 64 + l32) * S16_PITCH + lhi * 8;
+    const uint16_t *as = lds16 + (buf * 2) * S16_OP + (wm * 64 + l32) * S16_PITCH;
+    const uint16_t *bs = lds16 + (buf * 2 + 1) * S16_OP + (wn * 64 + l32) * S16_PITCH;
 #pragma unroll
     for (int ks = 0; ks < S16_BK; ks += 16) {
       v8 a[2], bq[2];
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
-        a[q] = *reinterpret_cast<const v8 *>(as + q * 32 * S16_PITCH + ks);
-        bq[q] = *reinterpret_cast<const v8 *>(bs + q * 32 * S16_PITCH + ks);
+        // 8-row block (ks / 8 + lhi) of feature 32 q + l32 (+ 64 wm / wn): swizzle (feature >> 4) & 7
+        const int blk = ks / 8 + lhi;
+        a[q] = *reinterpret_cast<const v8 *>(as + q * 32 * S16_PITCH + ((blk ^ sw_a[q]) * 8));
+        bq[q] = *reinterpret_cast<const v8 *>(bs + q * 32 * S16_PITCH + ((blk ^ sw_b[q]) * 8));
       }
 #pragma unroll
       for (int ii = 0; ii < 2; ++ii)
