@@ -1,5 +1,6 @@
 // Blocked GPTQ column loop: quantise block_size rows with error feedback, then push the
-// accumulated error into all remaining rows with one fp32 MFMA GEMM per block.
+// accumulated error into the remaining rows with fp32 MFMA GEMMs: after every block into the
+// rest of its 512-row group, after every group into everything below it.
 //
 // In-block kernel: the N output channels are independent, so one lane owns one channel and a
 // workgroup of four wavefronts owns 64 channels.  The workgroup first copies its channels of
@@ -156,6 +157,32 @@ int launch_block(hipStream_t st, const float *W, int64_t N, const float *L, int6
 
 bool block_size_ok(int bs) { return bs >= 1 && bs <= 128; }
 
+// Rows whose error rows are kept together for one trailing update (a whole number of blocks).
+// The rows below a group receive the updates of all its blocks in one product with k up to
+// 512 instead of one product per block: every product reads and writes the rows it updates,
+// so this cuts the traffic over the trailing part of W by the number of blocks in a group.
+constexpr int GROUP_ROWS = 512;
+int group_rows(int bs) { return (GROUP_ROWS / bs > 0 ? GROUP_ROWS / bs : 1) * bs; }
+
+// C[m, n] -= A[m, k] @ B[k, n]
+int trailing_update(hipStream_t st, const float *A, int64_t lda, const float *B, float *C,
+                    int64_t N, int64_t m, int64_t k) {
+  GemmArgs g;
+  g.A = A;
+  g.B = B;
+  g.C = C;
+  g.lda = lda;
+  g.ldb = N;
+  g.ldc = N;
+  g.m = (int)m;
+  g.n = (int)N;
+  g.k = (int)k;
+  g.alpha = -1.f;
+  g.beta = 1.f;
+  g.a_kmajor = 0;
+  return gptq_gemm_f32(st, g);
+}
+
 int process_block(hipStream_t st, const float *Wb, int64_t N, const float *Lb, int64_t ldl, int bs,
                   const float *scale, const float *zero, int maxq, void *Qb, int q_dtype,
                   uint8_t *cb, float *Err) {
@@ -175,7 +202,7 @@ extern "C" {
 
 size_t gptq_hip_solve_workspace_bytes(int64_t K, int64_t N, int block_size) {
   if (K <= 0 || N <= 0 || !block_size_ok(block_size)) return 0;
-  return (size_t)block_size * (size_t)N * sizeof(float);
+  return (size_t)group_rows(block_size) * (size_t)N * sizeof(float);
 }
 
 int gptq_hip_process_block(void *stream, const float *Wblock, int64_t N, const float *Lblock,
@@ -202,30 +229,29 @@ int gptq_hip_solve(void *stream, float *W, int64_t K, int64_t N, const float *L,
   hipStream_t st = as_stream(stream);
   float *Err = reinterpret_cast<float *>(ws);
   const size_t qsz = dtype_size(q_dtype);
-  for (int64_t start = 0; start < K; start += block_size) {
-    void *Qb = Q ? (void *)((char *)Q + (size_t)start * N * qsz) : nullptr;
-    uint8_t *cb = codes ? codes + start * N : nullptr;
-    int rc = process_block(st, W + start * N, N, L + start * K + start, K, block_size, scale, zero,
-                           maxq, Qb, q_dtype, cb, Err);
-    if (rc) return rc;
-    const int64_t end = start + block_size;
-    if (end >= K) break;
-    // W[end:, :] -= L[end:, start:end] @ Err
-    GemmArgs g;
-    g.A = L + end * K + start;
-    g.B = Err;
-    g.C = W + end * N;
-    g.lda = K;
-    g.ldb = N;
-    g.ldc = N;
-    g.m = (int)(K - end);
-    g.n = (int)N;
-    g.k = block_size;
-    g.alpha = -1.f;
-    g.beta = 1.f;
-    g.a_kmajor = 0;
-    rc = gptq_gemm_f32(st, g);
-    if (rc) return rc;
+  const int64_t grp = group_rows(block_size);
+  for (int64_t gs = 0; gs < K; gs += grp) {
+    const int64_t ge = gs + grp < K ? gs + grp : K;
+    for (int64_t start = gs; start < ge; start += block_size) {
+      void *Qb = Q ? (void *)((char *)Q + (size_t)start * N * qsz) : nullptr;
+      uint8_t *cb = codes ? codes + start * N : nullptr;
+      float *Eb = Err + (start - gs) * N;
+      int rc = process_block(st, W + start * N, N, L + start * K + start, K, block_size, scale, zero,
+                             maxq, Qb, q_dtype, cb, Eb);
+      if (rc) return rc;
+      const int64_t end = start + block_size;
+      if (end < ge) {
+        // rows of this group below the block: W[end:ge] -= L[end:ge, start:end] @ Err_block
+        rc = trailing_update(st, L + end * K + start, K, Eb, W + end * N, N, ge - end, block_size);
+        if (rc) return rc;
+      }
+    }
+    if (ge < K) {
+      // everything below the group: W[ge:] -= L[ge:, gs:ge] @ Err_group  (gptq.py:204-205, summed
+      // over the blocks of the group)
+      const int rc = trailing_update(st, L + ge * K + gs, K, Err, W + ge * N, N, K - ge, ge - gs);
+      if (rc) return rc;
+    }
   }
   return GPTQ_HIP_OK;
 }
