@@ -21,7 +21,10 @@ constexpr int LDT = 160;   // k-major LDS row stride (floats)
 constexpr int LDI = 17;    // idx-major LDS row stride (floats)
 constexpr int TILE_FLOATS = BK * LDT;  // 2560 >= BM * LDI (2176)
 
-template <typename T, bool AK>
+// FAST: every tile is full and every 4-element group aligned (checked on the host), so the
+// loads carry no guards: a load inside a branch makes the compiler wait for it at the join,
+// in front of the MFMAs it is meant to overlap with.
+template <typename T, bool AK, bool FAST>
 __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(GemmArgs p) {
   __shared__ __attribute__((aligned(16))) float As[2][TILE_FLOATS];
   __shared__ __attribute__((aligned(16))) float Bs[2][TILE_FLOATS];
@@ -70,7 +73,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(GemmArgs p) {
     const bool k_full = (kt + BK <= ke);
     if (AK) {
       const int r = tid >> 5, c4 = (tid & 31) * 4;
-      const bool fast = a_al && m_full && k_full;
+      const bool fast = FAST || (a_al && m_full && k_full);
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const int kk = kt + r + 8 * i;
@@ -80,7 +83,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(GemmArgs p) {
       }
     } else {
       const int row = tid >> 2, k4 = (tid & 3) * 4;
-      const bool fast = a_al && m_full && k_full;
+      const bool fast = FAST || (a_al && m_full && k_full);
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const int mm = m0 + row + 64 * i;
@@ -91,7 +94,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(GemmArgs p) {
     }
     {
       const int r = tid >> 5, c4 = (tid & 31) * 4;
-      const bool fast = b_al && n_full && k_full;
+      const bool fast = FAST || (b_al && n_full && k_full);
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const int kk = kt + r + 8 * i;
@@ -199,18 +202,28 @@ int gptq_gemm_f32(hipStream_t stream, const GemmArgs &a) {
   }
   if (grid.y > 65535u || grid.z > 65535u) return GPTQ_HIP_EINVAL;
   const dim3 block(NTHREADS);
+  const size_t es = a.in_dtype == GPTQ_HIP_F32 ? 4 : 2;
+  const bool fast = a.m % BM == 0 && a.n % BN == 0 && a.k % BK == 0 && a.m_step == 0 &&
+                    a.k_step == 0 && a.lda % 4 == 0 && a.ldb % 4 == 0 &&
+                    reinterpret_cast<uintptr_t>(a.A) % (4 * es) == 0 &&
+                    reinterpret_cast<uintptr_t>(a.B) % (4 * es) == 0 &&
+                    (a.batch == 1 || (a.strideA % 4 == 0 && a.strideB % 4 == 0));
+#define GPTQ_GEMM_LAUNCH(T, AK)                                                              \
+  do {                                                                                      \
+    if (fast) hipLaunchKernelGGL((gemm_f32_kernel<T, AK, true>), grid, block, 0, stream, a); \
+    else hipLaunchKernelGGL((gemm_f32_kernel<T, AK, false>), grid, block, 0, stream, a);     \
+  } while (0)
   if (a.in_dtype == GPTQ_HIP_F32) {
-    if (a.a_kmajor)
-      hipLaunchKernelGGL((gemm_f32_kernel<float, true>), grid, block, 0, stream, a);
-    else
-      hipLaunchKernelGGL((gemm_f32_kernel<float, false>), grid, block, 0, stream, a);
+    if (a.a_kmajor) GPTQ_GEMM_LAUNCH(float, true);
+    else GPTQ_GEMM_LAUNCH(float, false);
   } else if (a.in_dtype == GPTQ_HIP_F16 && a.a_kmajor) {
-    hipLaunchKernelGGL((gemm_f32_kernel<__half, true>), grid, block, 0, stream, a);
+    GPTQ_GEMM_LAUNCH(__half, true);
   } else if (a.in_dtype == GPTQ_HIP_BF16 && a.a_kmajor) {
-    hipLaunchKernelGGL((gemm_f32_kernel<__hip_bfloat16, true>), grid, block, 0, stream, a);
+    GPTQ_GEMM_LAUNCH(__hip_bfloat16, true);
   } else {
     return GPTQ_HIP_EDTYPE;
   }
+#undef GPTQ_GEMM_LAUNCH
   GPTQ_CHECK_LAUNCH();
   return GPTQ_HIP_OK;
 }
