@@ -102,14 +102,20 @@ def bench_qmatmul(reps=240):
         scale = (0.001 + 0.009 * torch.rand(N, generator=g, device="cuda")).to(torch.float16)
         zero = torch.randint(0, 16, (N,), generator=g, device="cuda").to(torch.float16)
         # forward at the decode / small-batch sizes, and the transposed (VJP) product at 2048 rows
-        for (M, tr) in ((1, 0), (16, 0), (128, 0), (2048, 0), (2048, 1)):
-            x = torch.randn((M, N if tr else K), generator=g, device="cuda").to(torch.float16)
-            y = torch.empty((M, K if tr else N), dtype=torch.float16, device="cuda")
+        cases = [(1, 0, "float16"), (16, 0, "float16"), (128, 0, "float16"), (2048, 0, "float16"),
+                 (2048, 1, "float16")]
+        if K == K_IN:
+            cases += [(1, 0, "bfloat16"), (16, 0, "bfloat16")]
+        for (M, tr, xdt) in cases:
+            tdt = getattr(torch, xdt)
+            xcode = _native.F16 if xdt == "float16" else _native.BF16
+            x = torch.randn((M, N if tr else K), generator=g, device="cuda").to(tdt)
+            y = torch.empty((M, K if tr else N), dtype=tdt, device="cuda")
             ws = torch.zeros(max(lib.gptq_hip_qmatmul_workspace_bytes(M, K // 2, N, tr), 256),
                              dtype=torch.uint8, device="cuda")
 
             def call(i):
-                rc = lib.gptq_hip_qmatmul(st, x.data_ptr(), _native.F16, M, iws[i % copies].data_ptr(),
+                rc = lib.gptq_hip_qmatmul(st, x.data_ptr(), xcode, M, iws[i % copies].data_ptr(),
                                           K // 2, N, zero.data_ptr(), scale.data_ptr(), _native.F16, tr,
                                           y.data_ptr(), ws.data_ptr(), ws.numel())
                 assert rc == 0, rc
@@ -125,7 +131,7 @@ def bench_qmatmul(reps=240):
             torch.cuda.synchronize()
             us = e0.elapsed_time(e1) * 1e3 / reps
             nbytes = K * N // 2 + 2 * N * 2 + M * K * 2 + M * N * 2
-            out.append({"M": M, "K": K, "N": N, "transpose_b": tr, "us": round(us, 2),
+            out.append({"M": M, "K": K, "N": N, "transpose_b": tr, "x_dtype": xdt, "us": round(us, 2),
                         "algorithmic_bytes": nbytes,
                         "GBps": round(nbytes / us * 1e-3, 1),
                         "hbm_frac": round(nbytes / us * 1e-3 / HBM_PEAK_GBS, 4),
@@ -279,7 +285,7 @@ def main():
     if not args.no_qmatmul:
         qm = bench_qmatmul()
         result["qmatmul"] = qm
-        m1 = [r for r in qm if r["M"] == 1 and r["K"] == 4096][0]
+        m1 = [r for r in qm if r["M"] == 1 and r["K"] == 4096 and r["x_dtype"] == "float16"][0]
         result["int4_matmul_hbm_gbps"] = m1["GBps"]
         result["roofline_qmatmul"] = {"kernel": "qmatmul M=1 4096x11008", "bound": "hbm",
                                       "achieved": m1["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",

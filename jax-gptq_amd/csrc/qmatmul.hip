@@ -57,7 +57,8 @@ __global__ __launch_bounds__(TPB) void qmm_bwd_simple(const TX *x, int64_t M, co
 }
 
 // ---------------------------------------------------------------------------- MFMA path
-// Forward, fp16 activations, C % 16 == 0.  One workgroup owns a strip of 256 output
+// Forward, fp16 or bf16 activations, C % 16 == 0 (described for fp16; bf16 differs only in the
+// dequantisation constants, see dequant_pair and the epilogue).  One workgroup owns a strip of 256 output
 // channels and a slice of NW * SPW * 16 packed rows (NW wavefronts, SPW MFMA k-steps of 16
 // packed rows each).  A wavefront first issues its (small, L2-resident) activation loads,
 // then ALL its weight loads in one burst (SPW * 4 loads of 16 B per lane), so that the
@@ -84,14 +85,46 @@ __device__ __forceinline__ uint32_t u4_comp(const uint4 &v, int w) {
   return w == 0 ? v.x : (w == 1 ? v.y : (w == 2 ? v.z : v.w));
 }
 
+template <bool BF>
 __device__ __forceinline__ void dequant_pair(uint32_t da, uint32_t db, uint32_t sel,
                                              uint32_t &lo, uint32_t &hi) {
-  // bytes of p: [7:0] = row a, [23:16] = row b.  lo = 1024 + code (even k), hi = 1024 + 16*code
-  // (odd k) as fp16 pairs; the offsets and the factor 16 are undone outside the MFMA.
+  // bytes of p: [7:0] = row a, [23:16] = row b.
   const uint32_t p = __builtin_amdgcn_perm(db, da, sel);
-  lo = (p & 0x000F000Fu) | 0x64006400u;
-  hi = (p & 0x00F000F0u) | 0x64006400u;
+  if (BF) {
+    // bf16 pairs 128 + code for both nibbles (0x4300 = 128.0; its 7 mantissa bits hold the code)
+    lo = (p & 0x000F000Fu) | 0x43004300u;
+    hi = ((p >> 4) & 0x000F000Fu) | 0x43004300u;
+  } else {
+    // fp16 pairs: lo = 1024 + code (even k), hi = 1024 + 16*code (odd k); the offsets and the
+    // factor 16 are undone outside the MFMA.
+    lo = (p & 0x000F000Fu) | 0x64006400u;
+    hi = (p & 0x00F000F0u) | 0x64006400u;
+  }
 }
+
+// 16-bit activation types of the MFMA kernels
+template <typename TX> struct Act;
+template <> struct Act<__half> {
+  static constexpr bool BF = false;
+  static __device__ __forceinline__ float lo(uint32_t w) { return (float)__builtin_bit_cast(half2_t, w)[0]; }
+  static __device__ __forceinline__ float hi(uint32_t w) { return (float)__builtin_bit_cast(half2_t, w)[1]; }
+  static __device__ __forceinline__ floatx4 mma(const uint4 &a, const uint4 &b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
+                                                  __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ __half out(float v) { return __float2half_rn(v); }
+};
+template <> struct Act<__hip_bfloat16> {
+  static constexpr bool BF = true;
+  typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
+  static __device__ __forceinline__ float lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+  static __device__ __forceinline__ float hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xFFFF0000u); }
+  static __device__ __forceinline__ floatx4 mma(const uint4 &a, const uint4 &b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, a),
+                                                   __builtin_bit_cast(bf8_t, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ __hip_bfloat16 out(float v) { return __float2bfloat16(v); }
+};
 
 // Workspace layout (only touched when the K range is split over S > 1 workgroups):
 //   [counters: QMM_COUNTER_BYTES, one int32 per (m-chunk, strip), zero between calls; the
@@ -108,10 +141,11 @@ struct QmmWs {
   float *part;
 };
 
-template <int SPW, typename TZ>
+template <int SPW, typename TZ, typename TX>
 __global__ __launch_bounds__(SPW == 2 ? 1024 : 512) void qmm_fwd_mfma_kernel(
-    const __half *x, int M, int K, const uint8_t *pk, int R, int C, const TZ *zero,
-    const TZ *scale, __half *out, QmmWs ws, int S) {
+    const TX *x, int M, int K, const uint8_t *pk, int R, int C, const TZ *zero,
+    const TZ *scale, TX *out, QmmWs ws, int S) {
+  constexpr bool BF = Act<TX>::BF;
   extern __shared__ float red[];   // [wave][mrows][256] partial tiles, then [wave][2][16] x sums
   __shared__ int s_last;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -125,7 +159,7 @@ __global__ __launch_bounds__(SPW == 2 ? 1024 : 512) void qmm_fwd_mfma_kernel(
   // ---- activation loads (k pairs 2r, 2r+1 of this lane's rows): small, L2 resident
   uint32_t pr[SPW][4];
   {
-    const __half *xr = x + (int64_t)(m0 + l16) * K;
+    const TX *xr = x + (int64_t)(m0 + l16) * K;
 #pragma unroll
     for (int s = 0; s < SPW; ++s)
 #pragma unroll
@@ -156,15 +190,16 @@ __global__ __launch_bounds__(SPW == 2 ? 1024 : 512) void qmm_fwd_mfma_kernel(
   for (int s = 0; s < SPW; ++s) {
     av[s].x = __builtin_amdgcn_perm(pr[s][1], pr[s][0], 0x05040100u);  // {x[2r0],   x[2r1]}
     av[s].z = __builtin_amdgcn_perm(pr[s][3], pr[s][2], 0x05040100u);
-    const half2_t o0 =
-        __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(pr[s][1], pr[s][0], 0x07060302u)) * sixteenth;
-    const half2_t o1 =
-        __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(pr[s][3], pr[s][2], 0x07060302u)) * sixteenth;
-    av[s].y = __builtin_bit_cast(uint32_t, o0);   // {x[2r0+1], x[2r1+1]} / 16
-    av[s].w = __builtin_bit_cast(uint32_t, o1);
-    const half2_t e0 = __builtin_bit_cast(half2_t, av[s].x), e1 = __builtin_bit_cast(half2_t, av[s].z);
-    se += ((float)e0[0] + (float)e0[1]) + ((float)e1[0] + (float)e1[1]);
-    so += ((float)o0[0] + (float)o0[1]) + ((float)o1[0] + (float)o1[1]);
+    uint32_t o0 = __builtin_amdgcn_perm(pr[s][1], pr[s][0], 0x07060302u);   // {x[2r0+1], x[2r1+1]}
+    uint32_t o1 = __builtin_amdgcn_perm(pr[s][3], pr[s][2], 0x07060302u);
+    if (!BF) {      // fp16: odd-k activations enter divided by 16 (bf16: both nibbles are 128 + code)
+      o0 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, o0) * sixteenth);
+      o1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, o1) * sixteenth);
+    }
+    av[s].y = o0;
+    av[s].w = o1;
+    se += (Act<TX>::lo(av[s].x) + Act<TX>::hi(av[s].x)) + (Act<TX>::lo(av[s].z) + Act<TX>::hi(av[s].z));
+    so += (Act<TX>::lo(o0) + Act<TX>::hi(o0)) + (Act<TX>::lo(o1) + Act<TX>::hi(o1));
   }
   se += __shfl_xor(se, 16);
   se += __shfl_xor(se, 32);
@@ -179,17 +214,15 @@ __global__ __launch_bounds__(SPW == 2 ? 1024 : 512) void qmm_fwd_mfma_kernel(
     for (int t = 0; t < 8; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < SPW; ++s) {
-      const half8_t a = __builtin_bit_cast(half8_t, av[s]);
 #pragma unroll
       for (int tt = 0; tt < 8; ++tt) {
         const int t = half * 8 + tt;
         const int w = t >> 2, tb = t & 3;
         const uint32_t sel = 0x0c000c00u | ((uint32_t)(4 + tb) << 16) | (uint32_t)tb;
         uint4 bv;
-        dequant_pair(u4_comp(d[s][0], w), u4_comp(d[s][1], w), sel, bv.x, bv.y);
-        dequant_pair(u4_comp(d[s][2], w), u4_comp(d[s][3], w), sel, bv.z, bv.w);
-        const half8_t b = __builtin_bit_cast(half8_t, bv);
-        acc[tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[tt], 0, 0, 0);
+        dequant_pair<BF>(u4_comp(d[s][0], w), u4_comp(d[s][1], w), sel, bv.x, bv.y);
+        dequant_pair<BF>(u4_comp(d[s][2], w), u4_comp(d[s][3], w), sel, bv.z, bv.w);
+        acc[tt] = Act<TX>::mma(av[s], bv, acc[tt]);
       }
     }
     // acc[tt][r] = tile[m = 4g + r][channel 16*l16 + half*8 + tt]
@@ -208,9 +241,12 @@ __global__ __launch_bounds__(SPW == 2 ? 1024 : 512) void qmm_fwd_mfma_kernel(
   __syncthreads();
 
   // epilogue value of one output from the accumulated tile sum v and the activation sums
-  auto finish = [&](float v, float e, float o, int n) -> __half {
+  // (bf16: both nibbles carry 128 + code and o is the plain odd-k sum)
+  auto finish = [&](float v, float e, float o, int n) -> TX {
     const float z = to_f32(zero[n]);
-    return __float2half_rn(to_f32(scale[n]) * ((v - 1024.f * (e + o)) - z * (e + 16.f * o)));
+    const float r = BF ? (v - 128.f * (e + o)) - z * (e + o)
+                       : (v - 1024.f * (e + o)) - z * (e + 16.f * o);
+    return Act<TX>::out(to_f32(scale[n]) * r);
   };
   const int n_items = mvalid * QSTRIP;
   // x sums of this workgroup: [split][2][16] per (m-chunk, strip)
@@ -327,7 +363,7 @@ FwdPlan fwd_plan(int64_t M, int64_t R, int64_t C) {
   return p;
 }
 
-template <int SPW, typename TZ>
+template <int SPW, typename TZ, typename TX>
 int launch_fwd_mfma(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, const uint8_t *pk,
                     int64_t R, int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
   QmmWs ws;
@@ -335,7 +371,7 @@ int launch_fwd_mfma(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, 
   ws.counters = reinterpret_cast<int32_t *>(base);
   ws.x1part = reinterpret_cast<float *>(base + p.counter_bytes);
   ws.part = reinterpret_cast<float *>(base + p.counter_bytes + p.x1_bytes);
-  auto kern = qmm_fwd_mfma_kernel<SPW, TZ>;
+  auto kern = qmm_fwd_mfma_kernel<SPW, TZ, TX>;
   if (p.lds_bytes > 48 * 1024 &&
       hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)p.lds_bytes) != hipSuccess)
@@ -351,20 +387,29 @@ int launch_fwd_mfma(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, 
     // the kernel sees the sub-problem rows [row0, row0 + rows); launches are stream ordered,
     // so they can share the workspace
     hipLaunchKernelGGL(kern, grid, dim3(p.nw * 64), p.lds_bytes, st,
-                       (const __half *)x + row0 * 2 * R, (int)rows, (int)(2 * R), pk, (int)R,
-                       (int)C, (const TZ *)zero, (const TZ *)scale, (__half *)out + row0 * C, ws,
+                       (const TX *)x + row0 * 2 * R, (int)rows, (int)(2 * R), pk, (int)R,
+                       (int)C, (const TZ *)zero, (const TZ *)scale, (TX *)out + row0 * C, ws,
                        p.S);
     GPTQ_CHECK_LAUNCH();
   }
   return GPTQ_HIP_OK;
 }
 
+template <typename TZ, typename TX>
+int launch_fwd_mfma_zx(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, const uint8_t *pk,
+                       int64_t R, int64_t C, const void *zero, const void *scale, void *out,
+                       void *wsp) {
+  if (p.spw == 2) return launch_fwd_mfma<2, TZ, TX>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
+  return launch_fwd_mfma<4, TZ, TX>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
+}
+
 template <typename TZ>
-int launch_fwd_mfma_z(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, const uint8_t *pk,
-                      int64_t R, int64_t C, const void *zero, const void *scale, void *out,
-                      void *wsp) {
-  if (p.spw == 2) return launch_fwd_mfma<2, TZ>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
-  return launch_fwd_mfma<4, TZ>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
+int launch_fwd_mfma_z(hipStream_t st, const FwdPlan &p, const void *x, int x_dtype, int64_t M,
+                      const uint8_t *pk, int64_t R, int64_t C, const void *zero, const void *scale,
+                      void *out, void *wsp) {
+  if (x_dtype == GPTQ_HIP_BF16)
+    return launch_fwd_mfma_zx<TZ, __hip_bfloat16>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
+  return launch_fwd_mfma_zx<TZ, __half>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
 }
 
 // ---------------------------------------------------------------------------- large M
@@ -748,7 +793,7 @@ bool bwd_fast_ok(int x_dtype, int64_t M, int64_t R, int64_t C, const void *x, co
 }
 
 bool fwd_fast_ok(int x_dtype, int64_t M, int64_t R, int64_t C, const void *x, const uint8_t *pk) {
-  return x_dtype == GPTQ_HIP_F16 && C % 16 == 0 && M >= 1 && M <= 65535 * 16LL &&
+  return (x_dtype == GPTQ_HIP_F16 || x_dtype == GPTQ_HIP_BF16) && C % 16 == 0 && M >= 1 && M <= 65535 * 16LL &&
          (reinterpret_cast<uintptr_t>(pk) & 15) == 0 && (reinterpret_cast<uintptr_t>(x) & 3) == 0 &&
          R < (1LL << 30) && C < (1LL << 30);
 }
@@ -803,7 +848,7 @@ int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const 
   hipStream_t st = as_stream(stream);
   // The tiled kernel has no split-K: it needs enough 64 x 128 output tiles to occupy the
   // chip; otherwise 16-row chunks through the split-K kernel (weights re-read from cache) win.
-  if (!transpose_b && fwd_fast_ok(x_dtype, M, R, C, x, packed) && M > 32 &&
+  if (!transpose_b && x_dtype == GPTQ_HIP_F16 && fwd_fast_ok(x_dtype, M, R, C, x, packed) && M > 32 &&
       ceil_div64(C, 128) * ceil_div64(M, GBM) >= 160 &&
       (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (2 * R) % 8 == 0) {
     switch (zs_dtype) {
@@ -828,11 +873,11 @@ int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const 
     if (p.total_bytes && (!ws || ws_bytes < p.total_bytes)) return GPTQ_HIP_EWORKSPACE;
     switch (zs_dtype) {
       case GPTQ_HIP_F32:
-        return launch_fwd_mfma_z<float>(st, p, x, M, packed, R, C, zero, scale, out, ws);
+        return launch_fwd_mfma_z<float>(st, p, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
       case GPTQ_HIP_F16:
-        return launch_fwd_mfma_z<__half>(st, p, x, M, packed, R, C, zero, scale, out, ws);
+        return launch_fwd_mfma_z<__half>(st, p, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
       case GPTQ_HIP_BF16:
-        return launch_fwd_mfma_z<__hip_bfloat16>(st, p, x, M, packed, R, C, zero, scale, out, ws);
+        return launch_fwd_mfma_z<__hip_bfloat16>(st, p, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
       default:
         return GPTQ_HIP_EDTYPE;
     }

@@ -100,6 +100,29 @@ def test_qmatmul_bf16_x(OP):
     assert np.allclose(to_np(got), ref, atol=3e-2, rtol=1e-2)    # bf16 result: 2^-8 relative
 
 
+@pytest.mark.parametrize("zs", ["float32", "bfloat16"])
+@pytest.mark.parametrize("M,N,K", [(1, 11008, 4096), (3, 4096, 11008), (16, 4096, 11008), (128, 4096, 1024),
+                                   (70, 2304, 768), (5, 48, 96)])
+def test_qmatmul_bf16_x_mfma_path(OP, M, N, K, zs):
+    """bf16 activations on the 16-bit MFMA kernel (both nibbles dequantise to 128 + code, which
+    bf16 holds exactly); the result is rounded once, to bf16 (2^-9 relative)."""
+    import torch
+    import jax_gptq_amd.gptq as G
+    rng = np.random.default_rng(M + N + K)
+    codes = rng.integers(0, 16, (K, N)).astype(np.uint8)
+    tdt = getattr(torch, zs)
+    scale = torch.from_numpy(rng.uniform(0.001, 0.01, N).astype(np.float32)).to(tdt)
+    zero = torch.from_numpy(rng.uniform(0.0, 15.0, N).astype(np.float32)).to(tdt)      # fractional, too
+    qm = G.QuantizedMatrix(torch.from_numpy(O.pack_colwise(codes)).cuda(), zero.cuda(), scale.cuda())
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16)
+    got = OP.quantized_matmul(x, qm)
+    assert got.dtype == torch.bfloat16 and tuple(got.shape) == (M, N)
+    dense = (codes.astype(np.float64) - zero.double().numpy()[None]) * scale.double().numpy()[None]
+    ref = x.double().numpy() @ dense
+    err = np.abs(to_np(got).astype(np.float64) - ref)
+    assert np.all(err <= 1e-2 + 2.0 ** -8 * np.abs(ref)), err.max()
+
+
 def test_qmatmul_leading_dims_and_errors(OP):
     qm = _matrix(8, 256, 192)
     rng = np.random.default_rng(7)
