@@ -433,11 +433,14 @@ __device__ __forceinline__ int g_off(int row, int k) {   // LDS offset (halves) 
   return (row >> 4) * GGROUP + (row & 15) * GPITCH + k;
 }
 
-template <int BN, typename TZ>
-__global__ __launch_bounds__(256) void qmm_fwd_gemm_kernel(const __half *x, int M, int K,
+// bf16 activations: the weights enter as 128 + code (bit operations only, exact in bf16) and
+// the whole 128 + zero is removed in the epilogue through the same row sums.
+template <int BN, typename TZ, typename TX>
+__global__ __launch_bounds__(256) void qmm_fwd_gemm_kernel(const TX *x, int M, int K,
                                                            const uint8_t *pk, int R, int C,
                                                            const TZ *zero, const TZ *scale,
-                                                           __half *out) {
+                                                           TX *out) {
+  constexpr bool BF = Act<TX>::BF;
   constexpr int A_HALVES = (GBM / 16) * GGROUP;
   constexpr int B_HALVES = (BN / 16) * GGROUP;
   constexpr int TN = BN / 32;                   // 16-wide MFMA tiles per wavefront along N
@@ -451,7 +454,7 @@ __global__ __launch_bounds__(256) void qmm_fwd_gemm_kernel(const __half *x, int 
   // A staging: thread -> row tid/4, 16 halves at k = (tid%4)*16
   const int a_row = tid >> 2, a_k = (tid & 3) * 16;
   const bool a_ok = (m0 + a_row) < M;
-  const __half *a_src = x + (int64_t)(m0 + a_row) * K + a_k;
+  const TX *a_src = x + (int64_t)(m0 + a_row) * K + a_k;
   // B staging: thread -> packed row tid / (BN/16), 16 channels at (tid % (BN/16)) * 16
   const int b_row = tid / (BN / 16), b_c = (tid % (BN / 16)) * 16;
   const bool b_thread = tid < B_THREADS;
@@ -463,7 +466,7 @@ __global__ __launch_bounds__(256) void qmm_fwd_gemm_kernel(const __half *x, int 
   uint32_t zc[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
-    const float z = b_ok ? rintf(to_f32(zero[n0 + b_c + i])) : 0.f;
+    const float z = (b_ok && !BF) ? rintf(to_f32(zero[n0 + b_c + i])) : 0.f;
     const _Float16 h = (_Float16)(-(1024.f + z));
     zc[i] = __builtin_bit_cast(uint32_t, half2_t{h, h});
   }
@@ -494,8 +497,12 @@ __global__ __launch_bounds__(256) void qmm_fwd_gemm_kernel(const __half *x, int 
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const uint32_t w0 = va0[i], w1 = va1[i];
-        xsum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, w0), ones, xsum, false);
-        xsum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, w1), ones, xsum, false);
+        if (BF) {
+          xsum += (Act<TX>::lo(w0) + Act<TX>::hi(w0)) + (Act<TX>::lo(w1) + Act<TX>::hi(w1));
+        } else {
+          xsum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, w0), ones, xsum, false);
+          xsum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, w1), ones, xsum, false);
+        }
       }
     }
     if (b_thread) {
@@ -505,10 +512,15 @@ __global__ __launch_bounds__(256) void qmm_fwd_gemm_kernel(const __half *x, int 
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const uint32_t b = (w[i >> 2] >> (8 * (i & 3))) & 0xFFu;
-        const uint32_t v = ((b | (b << 12)) & 0x000F000Fu) | 0x64006400u;   // {1024+lo, 1024+hi}
-        const half2_t d = __builtin_bit_cast(half2_t, v) + __builtin_bit_cast(half2_t, zc[i]);
-        *reinterpret_cast<uint32_t *>(&Bs[buf][g_off(b_c + i, 2 * b_row)]) =
-            __builtin_bit_cast(uint32_t, d);
+        uint32_t v;
+        if (BF) {
+          v = ((b | (b << 12)) & 0x000F000Fu) | 0x43004300u;                   // bf16 {128+lo, 128+hi}
+        } else {
+          v = ((b | (b << 12)) & 0x000F000Fu) | 0x64006400u;                   // fp16 {1024+lo, 1024+hi}
+          const half2_t d = __builtin_bit_cast(half2_t, v) + __builtin_bit_cast(half2_t, zc[i]);
+          v = __builtin_bit_cast(uint32_t, d);
+        }
+        *reinterpret_cast<uint32_t *>(&Bs[buf][g_off(b_c + i, 2 * b_row)]) = v;
       }
     }
   };
@@ -534,19 +546,18 @@ __global__ __launch_bounds__(256) void qmm_fwd_gemm_kernel(const __half *x, int 
     load_stage(k0 + 4 * GBK, refill);
 #pragma unroll
     for (int ks = 0; ks < GBK; ks += 32) {
-      half8_t a[2], b[TN];
+      uint4 a[2], b[TN];
 #pragma unroll
       for (int i = 0; i < 2; ++i)
-        a[i] = *reinterpret_cast<const half8_t *>(&As[buf][g_off(wm * 32 + i * 16 + l16, ks + 8 * g)]);
+        a[i] = *reinterpret_cast<const uint4 *>(&As[buf][g_off(wm * 32 + i * 16 + l16, ks + 8 * g)]);
 #pragma unroll
       for (int j = 0; j < TN; ++j)
-        b[j] = *reinterpret_cast<const half8_t *>(
+        b[j] = *reinterpret_cast<const uint4 *>(
             &Bs[buf][g_off(wn * (BN / 2) + j * 16 + l16, ks + 8 * g)]);
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < TN; ++j) acc[i][j] = Act<TX>::mma(a[i], b[j], acc[i][j]);
     }
     if (k0 + GBK < K) store_stage(buf ^ 1, k0 + GBK, next);
     __syncthreads();
@@ -571,26 +582,32 @@ __global__ __launch_bounds__(256) void qmm_fwd_gemm_kernel(const __half *x, int 
     if (n >= C) continue;
     const float sc = to_f32(scale[n]);
     const float z = to_f32(zero[n]);
-    const float zf = z - rintf(z);
+    const float zf = BF ? 128.f + z : z - rintf(z);
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int ml = wm * 32 + i * 16 + 4 * g + r;
         if (m0 + ml < M)
-          out[(int64_t)(m0 + ml) * C + n] = __float2half_rn(sc * (acc[i][j][r] - zf * rowsum[ml]));
+          out[(int64_t)(m0 + ml) * C + n] = Act<TX>::out(sc * (acc[i][j][r] - zf * rowsum[ml]));
       }
   }
 }
 
 template <typename TZ>
-int launch_fwd_gemm(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
-                    const void *zero, const void *scale, void *out) {
+int launch_fwd_gemm(hipStream_t st, const void *x, int x_dtype, int64_t M, const uint8_t *pk, int64_t R,
+                    int64_t C, const void *zero, const void *scale, void *out) {
   const int64_t mt = ceil_div64(M, GBM);
   if (mt > 65535) return GPTQ_HIP_EINVAL;
-  hipLaunchKernelGGL((qmm_fwd_gemm_kernel<128, TZ>), dim3((unsigned)ceil_div64(C, 128), (unsigned)mt),
-                     dim3(256), 0, st, (const __half *)x, (int)M, (int)(2 * R), pk, (int)R, (int)C,
-                     (const TZ *)zero, (const TZ *)scale, (__half *)out);
+  const dim3 grid((unsigned)ceil_div64(C, 128), (unsigned)mt);
+  if (x_dtype == GPTQ_HIP_BF16)
+    hipLaunchKernelGGL((qmm_fwd_gemm_kernel<128, TZ, __hip_bfloat16>), grid, dim3(256), 0, st,
+                       (const __hip_bfloat16 *)x, (int)M, (int)(2 * R), pk, (int)R, (int)C,
+                       (const TZ *)zero, (const TZ *)scale, (__hip_bfloat16 *)out);
+  else
+    hipLaunchKernelGGL((qmm_fwd_gemm_kernel<128, TZ, __half>), grid, dim3(256), 0, st,
+                       (const __half *)x, (int)M, (int)(2 * R), pk, (int)R, (int)C,
+                       (const TZ *)zero, (const TZ *)scale, (__half *)out);
   GPTQ_CHECK_LAUNCH();
   return GPTQ_HIP_OK;
 }
@@ -848,14 +865,14 @@ int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const 
   hipStream_t st = as_stream(stream);
   // The tiled kernel has no split-K: it needs enough 64 x 128 output tiles to occupy the
   // chip; otherwise 16-row chunks through the split-K kernel (weights re-read from cache) win.
-  if (!transpose_b && x_dtype == GPTQ_HIP_F16 && fwd_fast_ok(x_dtype, M, R, C, x, packed) && M > 32 &&
+  if (!transpose_b && fwd_fast_ok(x_dtype, M, R, C, x, packed) && M > 32 &&
       ceil_div64(C, 128) * ceil_div64(M, GBM) >= 160 &&
       (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (2 * R) % 8 == 0) {
     switch (zs_dtype) {
-      case GPTQ_HIP_F32: return launch_fwd_gemm<float>(st, x, M, packed, R, C, zero, scale, out);
-      case GPTQ_HIP_F16: return launch_fwd_gemm<__half>(st, x, M, packed, R, C, zero, scale, out);
+      case GPTQ_HIP_F32: return launch_fwd_gemm<float>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
+      case GPTQ_HIP_F16: return launch_fwd_gemm<__half>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
       case GPTQ_HIP_BF16:
-        return launch_fwd_gemm<__hip_bfloat16>(st, x, M, packed, R, C, zero, scale, out);
+        return launch_fwd_gemm<__hip_bfloat16>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
       default: return GPTQ_HIP_EDTYPE;
     }
   }

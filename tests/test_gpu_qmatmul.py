@@ -102,7 +102,7 @@ def test_qmatmul_bf16_x(OP):
 
 @pytest.mark.parametrize("zs", ["float32", "bfloat16"])
 @pytest.mark.parametrize("M,N,K", [(1, 11008, 4096), (3, 4096, 11008), (16, 4096, 11008), (128, 4096, 1024),
-                                   (70, 2304, 768), (5, 48, 96)])
+                                   (70, 2304, 768), (5, 48, 96), (200, 5120, 256), (300, 11008, 512)])
 def test_qmatmul_bf16_x_mfma_path(OP, M, N, K, zs):
     """bf16 activations on the 16-bit MFMA kernel (both nibbles dequantise to 128 + code, which
     bf16 holds exactly); the result is rounded once, to bf16 (2^-9 relative)."""
