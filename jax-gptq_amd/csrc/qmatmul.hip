@@ -414,7 +414,7 @@ int launch_fwd_mfma_z(hipStream_t st, const FwdPlan &p, const void *x, int x_dty
 
 // ---------------------------------------------------------------------------- large M
 // Forward, fp16 activations, M > 32: a tiled GEMM that dequantises on the way into LDS.
-// Workgroup tile 64 (M) x BN (N) x 64 (k) per stage, 4 wavefronts as 2 x 2, accumulators of
+// Workgroup tile BM = 64 or 128 (M) x BN (N) x 64 (k) per stage, 4 wavefronts as 2 x 2, accumulators of
 // v_mfma_f32_16x16x32_f16 in registers for the whole K loop (no split-K, no partials).
 //   A = activations: staged in their natural [m][k] layout (k contiguous = the operand order)
 //   B = weights: every thread loads 16 packed bytes (16 channels of one packed row), turns
@@ -435,24 +435,34 @@ __device__ __forceinline__ int g_off(int row, int k) {   // LDS offset (halves) 
 
 // bf16 activations: the weights enter as 128 + code (bit operations only, exact in bf16) and
 // the whole 128 + zero is removed in the epilogue through the same row sums.
-template <int BN, typename TZ, typename TX>
+template <int BM, int BN, typename TZ, typename TX, bool SPLIT>
 __global__ __launch_bounds__(256) void qmm_fwd_gemm_kernel(const TX *x, int M, int K,
                                                            const uint8_t *pk, int R, int C,
                                                            const TZ *zero, const TZ *scale,
-                                                           TX *out) {
+                                                           TX *out, QmmWs ws, int S) {
   constexpr bool BF = Act<TX>::BF;
-  constexpr int A_HALVES = (GBM / 16) * GGROUP;
+  __shared__ int s_last;
+  constexpr int A_HALVES = (BM / 16) * GGROUP;
   constexpr int B_HALVES = (BN / 16) * GGROUP;
-  constexpr int TN = BN / 32;                   // 16-wide MFMA tiles per wavefront along N
+  constexpr int TM = BM / 32;                   // 16-wide MFMA tiles per wavefront along M
+  constexpr int TN = BN / 32;                   // ... and along N
   constexpr int B_THREADS = 2 * BN;             // threads that stage weights: 32 rows x BN/16 segments
-  __shared__ __attribute__((aligned(16))) _Float16 As[2][A_HALVES];
-  __shared__ __attribute__((aligned(16))) _Float16 Bs[2][B_HALVES];
+  constexpr int TPR = 256 / BM;                 // threads that stage one activation row
+  constexpr int AL = 64 / TPR / 8;              // 16-byte loads per thread and stage
+  extern __shared__ __attribute__((aligned(16))) _Float16 qgemm_lds[];
+  _Float16 (*As)[A_HALVES] = reinterpret_cast<_Float16 (*)[A_HALVES]>(qgemm_lds);
+  _Float16 (*Bs)[B_HALVES] = reinterpret_cast<_Float16 (*)[B_HALVES]>(qgemm_lds + 2 * A_HALVES);
+  float *rowsum = reinterpret_cast<float *>(qgemm_lds + 2 * A_HALVES + 2 * B_HALVES);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1, g = lane >> 4, l16 = lane & 15;
-  const int n0 = blockIdx.x * BN, m0 = blockIdx.y * GBM;
+  const int n0 = blockIdx.x * BN, m0 = blockIdx.y * BM;
+  // split-K: this workgroup multiplies the stages [kbeg, kend) of the contraction axis
+  const int split = SPLIT ? blockIdx.z : 0;
+  const int sps = ((K + GBK - 1) / GBK + S - 1) / S;
+  const int kbeg = SPLIT ? split * sps * GBK : 0, kend = SPLIT ? min(K, kbeg + sps * GBK) : K;
 
-  // A staging: thread -> row tid/4, 16 halves at k = (tid%4)*16
-  const int a_row = tid >> 2, a_k = (tid & 3) * 16;
+  // A staging: TPR threads per row, 8 * AL consecutive halves each
+  const int a_row = tid / TPR, a_k = (tid % TPR) * (8 * AL);
   const bool a_ok = (m0 + a_row) < M;
   const TX *a_src = x + (int64_t)(m0 + a_row) * K + a_k;
   // B staging: thread -> packed row tid / (BN/16), 16 channels at (tid % (BN/16)) * 16
@@ -460,7 +470,6 @@ __global__ __launch_bounds__(256) void qmm_fwd_gemm_kernel(const TX *x, int M, i
   const bool b_thread = tid < B_THREADS;
   const bool b_ok = b_thread && (n0 + b_c) < C;
   const uint8_t *b_src = pk + (int64_t)b_row * C + n0 + b_c;
-  __shared__ float rowsum[GBM];
   float xsum = 0.f;     // sum over k of this thread's share of activation row a_row
   // -(1024 + rint(zero)) per staged channel, as fp16 pairs
   uint32_t zc[16];
@@ -475,38 +484,36 @@ __global__ __launch_bounds__(256) void qmm_fwd_gemm_kernel(const TX *x, int M, i
   // the loads of stage s + 4 are issued while stage s is being multiplied, so about four
   // stage times hide the memory latency even with one workgroup per CU.
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-  struct Stage { u32x4 a0, a1, b; };
+  struct Stage { u32x4 a[AL]; u32x4 b; };
   // Loads are unconditional (out-of-range lanes read a clamped, valid address and are zeroed
   // when the stage is written to LDS): a load inside a branch would make the compiler wait
   // for it at the join and defeat the prefetch.  K % 8 == 0 is guaranteed by the dispatcher.
   auto load_stage = [&](int k0, Stage &st) __attribute__((always_inline)) {
-    const bool ok0 = a_ok && (k0 + a_k + 8 <= K), ok1 = a_ok && (k0 + a_k + 16 <= K);
-    st.a0 = *reinterpret_cast<const u32x4 *>(ok0 ? a_src + k0 : x);
-    st.a1 = *reinterpret_cast<const u32x4 *>(ok1 ? a_src + k0 + 8 : x);
-    const bool okb = b_ok && ((k0 >> 1) + b_row < R);
+#pragma unroll
+    for (int l = 0; l < AL; ++l) {
+      const bool ok = a_ok && (k0 + a_k + 8 * (l + 1) <= kend);
+      st.a[l] = *reinterpret_cast<const u32x4 *>(ok ? a_src + k0 + 8 * l : x);
+    }
+    const bool okb = b_ok && ((k0 >> 1) + b_row < R) && (!SPLIT || k0 + 2 * b_row < kend);
     st.b = *reinterpret_cast<const u32x4 *>(okb ? b_src + (int64_t)(k0 >> 1) * C : pk);
   };
   auto store_stage = [&](int buf, int k0, const Stage &st) __attribute__((always_inline)) {
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
-    const bool ok0 = a_ok && (k0 + a_k + 8 <= K), ok1 = a_ok && (k0 + a_k + 16 <= K);
-    const u32x4 va0 = ok0 ? st.a0 : zero4, va1 = ok1 ? st.a1 : zero4;
-    *reinterpret_cast<u32x4 *>(&As[buf][g_off(a_row, a_k)]) = va0;
-    *reinterpret_cast<u32x4 *>(&As[buf][g_off(a_row, a_k + 8)]) = va1;
-    {
-      const half2_t ones = half2_t{(_Float16)1.f, (_Float16)1.f};
+    const half2_t ones = half2_t{(_Float16)1.f, (_Float16)1.f};
+#pragma unroll
+    for (int l = 0; l < AL; ++l) {
+      const bool ok = a_ok && (k0 + a_k + 8 * (l + 1) <= kend);
+      const u32x4 va = ok ? st.a[l] : zero4;
+      *reinterpret_cast<u32x4 *>(&As[buf][g_off(a_row, a_k + 8 * l)]) = va;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const uint32_t w0 = va0[i], w1 = va1[i];
-        if (BF) {
-          xsum += (Act<TX>::lo(w0) + Act<TX>::hi(w0)) + (Act<TX>::lo(w1) + Act<TX>::hi(w1));
-        } else {
-          xsum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, w0), ones, xsum, false);
-          xsum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, w1), ones, xsum, false);
-        }
+        const uint32_t w0 = va[i];
+        if (BF) xsum += Act<TX>::lo(w0) + Act<TX>::hi(w0);
+        else xsum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, w0), ones, xsum, false);
       }
     }
     if (b_thread) {
-      const bool okb = b_ok && ((k0 >> 1) + b_row < R);
+      const bool okb = b_ok && ((k0 >> 1) + b_row < R) && (!SPLIT || k0 + 2 * b_row < kend);
       const u32x4 pbm = okb ? st.b : zero4;
       const uint32_t w[4] = {pbm[0], pbm[1], pbm[2], pbm[3]};
 #pragma unroll
@@ -525,56 +532,117 @@ __global__ __launch_bounds__(256) void qmm_fwd_gemm_kernel(const TX *x, int M, i
     }
   };
 
-  floatx4 acc[2][TN];
+  floatx4 acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   Stage s0, s1, s2, s3;
-  load_stage(0, s0);
-  load_stage(GBK, s1);
-  load_stage(2 * GBK, s2);
-  load_stage(3 * GBK, s3);
+  load_stage(kbeg, s0);
+  load_stage(kbeg + GBK, s1);
+  load_stage(kbeg + 2 * GBK, s2);
+  load_stage(kbeg + 3 * GBK, s3);
   int buf = 0;
-  store_stage(0, 0, s0);
+  store_stage(0, kbeg, s0);
   __syncthreads();
   // one stage: refill the ring slot that was just consumed, multiply the stage in LDS, write
   // the next stage to the other LDS buffer
   auto step = [&](int k0, Stage &refill, const Stage &next) __attribute__((always_inline)) {
-    if (k0 >= K) return;
+    if (k0 >= kend) return;
     load_stage(k0 + 4 * GBK, refill);
 #pragma unroll
     for (int ks = 0; ks < GBK; ks += 32) {
-      uint4 a[2], b[TN];
+      uint4 a[TM], b[TN];
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
-        a[i] = *reinterpret_cast<const uint4 *>(&As[buf][g_off(wm * 32 + i * 16 + l16, ks + 8 * g)]);
+      for (int i = 0; i < TM; ++i)
+        a[i] = *reinterpret_cast<const uint4 *>(&As[buf][g_off(wm * (BM / 2) + i * 16 + l16, ks + 8 * g)]);
 #pragma unroll
       for (int j = 0; j < TN; ++j)
         b[j] = *reinterpret_cast<const uint4 *>(
             &Bs[buf][g_off(wn * (BN / 2) + j * 16 + l16, ks + 8 * g)]);
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = Act<TX>::mma(a[i], b[j], acc[i][j]);
     }
-    if (k0 + GBK < K) store_stage(buf ^ 1, k0 + GBK, next);
+    if (k0 + GBK < kend) store_stage(buf ^ 1, k0 + GBK, next);
     __syncthreads();
     buf ^= 1;
   };
-  for (int kb = 0; kb < K; kb += 4 * GBK) {
+  for (int kb = kbeg; kb < kend; kb += 4 * GBK) {
     step(kb, s0, s1);
     step(kb + GBK, s1, s2);
     step(kb + 2 * GBK, s2, s3);
     step(kb + 3 * GBK, s3, s0);
   }
 
-  // the four staging threads of a row are neighbouring lanes
+  // the staging threads of a row are neighbouring lanes
   xsum += __shfl_xor(xsum, 1);
-  xsum += __shfl_xor(xsum, 2);
-  if ((tid & 3) == 0) rowsum[a_row] = xsum;
+  if (TPR == 4) xsum += __shfl_xor(xsum, 2);
+  if ((tid % TPR) == 0) rowsum[a_row] = xsum;
   __syncthreads();
+  if (SPLIT) {
+    // Partial tile and partial row sums to the workspace (agent-scope write-through stores), an
+    // arrival ticket per output tile; the last workgroup of a tile adds the S partials in split
+    // order, so the result does not depend on the arrival order, and leaves the counter at zero.
+    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + wn * (BN / 2) + j * 16 + l16;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int m = m0 + wm * (BM / 2) + i * 16 + 4 * g + r;
+          if (n < C && m < M)
+            __hip_atomic_store(&ws.part[((int64_t)split * M + m) * C + n], acc[i][j][r],
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    float *xp = ws.x1part + ((int64_t)tile * S) * BM;
+    if (tid < BM)
+      __hip_atomic_store(&xp[split * BM + tid], rowsum[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (tid == 0) {
+      int32_t *ctr = ws.counters + tile;
+      const int ticket = atomicAdd(ctr, 1);
+      s_last = (ticket == S - 1);
+      if (ticket == S - 1) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    if (tid < BM) {
+      float a = 0.f;
+      for (int sp = 0; sp < S; ++sp)
+        a += __hip_atomic_load(&xp[sp * BM + tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      rowsum[tid] = a;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int sp = 0; sp < S; ++sp) {
+      floatx4 pv[TM][TN];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int n = min(n0 + wn * (BN / 2) + j * 16 + l16, C - 1);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int m = min(m0 + wm * (BM / 2) + i * 16 + 4 * g + r, M - 1);
+            pv[i][j][r] = __hip_atomic_load(&ws.part[((int64_t)sp * M + m) * C + n], __ATOMIC_RELAXED,
+                                            __HIP_MEMORY_SCOPE_AGENT);
+          }
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] += pv[i][j];
+    }
+    __syncthreads();
+  }
   // acc[i][j][r] = out[m0 + wm*32 + i*16 + 4g + r][n0 + wn*BN/2 + j*16 + l16]
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
@@ -584,32 +652,93 @@ __global__ __launch_bounds__(256) void qmm_fwd_gemm_kernel(const TX *x, int M, i
     const float z = to_f32(zero[n]);
     const float zf = BF ? 128.f + z : z - rintf(z);
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int ml = wm * 32 + i * 16 + 4 * g + r;
+        const int ml = wm * (BM / 2) + i * 16 + 4 * g + r;
         if (m0 + ml < M)
           out[(int64_t)(m0 + ml) * C + n] = Act<TX>::out(sc * (acc[i][j][r] - zf * rowsum[ml]));
       }
   }
 }
 
-template <typename TZ>
-int launch_fwd_gemm(hipStream_t st, const void *x, int x_dtype, int64_t M, const uint8_t *pk, int64_t R,
-                    int64_t C, const void *zero, const void *scale, void *out) {
-  const int64_t mt = ceil_div64(M, GBM);
-  if (mt > 65535) return GPTQ_HIP_EINVAL;
-  const dim3 grid((unsigned)ceil_div64(C, 128), (unsigned)mt);
-  if (x_dtype == GPTQ_HIP_BF16)
-    hipLaunchKernelGGL((qmm_fwd_gemm_kernel<128, TZ, __hip_bfloat16>), grid, dim3(256), 0, st,
-                       (const __hip_bfloat16 *)x, (int)M, (int)(2 * R), pk, (int)R, (int)C,
-                       (const TZ *)zero, (const TZ *)scale, (__hip_bfloat16 *)out);
-  else
-    hipLaunchKernelGGL((qmm_fwd_gemm_kernel<128, TZ, __half>), grid, dim3(256), 0, st,
-                       (const __half *)x, (int)M, (int)(2 * R), pk, (int)R, (int)C,
-                       (const TZ *)zero, (const TZ *)scale, (__half *)out);
+// Tiled kernel plan: S = 1 when the 64 x 128 output tiles alone fill the chip, else split-K
+// over S workgroups per tile (partials and arrival counters in the workspace, as above).
+struct GemmPlan {
+  bool use;
+  int bm;            // rows per output tile: 128 from M = 256 on (the dequantisation of a weight stage
+                     // is shared by twice as many rows; measured slower than 64 at M = 128), else 64
+  int S;
+  int64_t tiles;
+  size_t x1_bytes, part_bytes, total_bytes;
+};
+
+GemmPlan gemm_plan(int64_t M, int64_t R, int64_t C) {
+  GemmPlan p;
+  p.bm = M >= 256 ? 128 : 64;
+  p.tiles = ceil_div64(C, 128) * ceil_div64(M, p.bm);
+  const int64_t stages = ceil_div64(2 * R, GBK);
+  int64_t S = 1;
+  if (p.tiles < 384) {
+    // about two (64-row tiles) or one (128-row tiles) workgroups per CU; every further split adds
+    // an M x C fp32 partial that is written and read once more
+    S = ((p.bm == 64 ? 512 : 256) + p.tiles - 1) / p.tiles;
+    if (S > 8) S = 8;
+    while (S > 1 && stages / S < 8) --S;          // at least 8 stages per workgroup
+    // every split must own at least one stage
+    while (S > 1 && (S - 1) * ceil_div64(stages, S) >= stages) --S;
+  }
+  p.S = (int)S;
+  p.use = M > 32 && (2 * R) % 8 == 0 && p.tiles * S >= 160 && p.tiles <= QMM_MAX_COUNTERS &&
+          ceil_div64(M, p.bm) <= 65535;
+  p.x1_bytes = S > 1 ? (size_t)round_up64(p.tiles * S * p.bm * (int64_t)sizeof(float), 256) : 0;
+  p.part_bytes = S > 1 ? (size_t)S * M * C * sizeof(float) : 0;
+  p.total_bytes = S > 1 ? QMM_COUNTER_BYTES + p.x1_bytes + p.part_bytes : 0;
+  return p;
+}
+
+template <int BM, typename TZ, typename TX, bool SPLIT>
+int launch_fwd_gemm_inst(hipStream_t st, const GemmPlan &p, const void *x, int64_t M, const uint8_t *pk,
+                         int64_t R, int64_t C, const void *zero, const void *scale, void *out,
+                         const QmmWs &ws) {
+  constexpr size_t lds = (size_t)(2 * (BM / 16) * GGROUP + 2 * (128 / 16) * GGROUP) * sizeof(_Float16) +
+                         BM * sizeof(float);
+  auto kern = qmm_fwd_gemm_kernel<BM, 128, TZ, TX, SPLIT>;
+  if (lds > 64 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return GPTQ_HIP_ELAUNCH;
+  const dim3 grid((unsigned)ceil_div64(C, 128), (unsigned)ceil_div64(M, BM), (unsigned)p.S);
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (const TX *)x, (int)M, (int)(2 * R), pk, (int)R,
+                     (int)C, (const TZ *)zero, (const TZ *)scale, (TX *)out, ws, p.S);
   GPTQ_CHECK_LAUNCH();
   return GPTQ_HIP_OK;
+}
+
+template <typename TZ, typename TX>
+int launch_fwd_gemm_x(hipStream_t st, const GemmPlan &p, const void *x, int64_t M, const uint8_t *pk,
+                      int64_t R, int64_t C, const void *zero, const void *scale, void *out,
+                      const QmmWs &ws) {
+  if (p.bm == 128) {
+    if (p.S > 1) return launch_fwd_gemm_inst<128, TZ, TX, true>(st, p, x, M, pk, R, C, zero, scale, out, ws);
+    return launch_fwd_gemm_inst<128, TZ, TX, false>(st, p, x, M, pk, R, C, zero, scale, out, ws);
+  }
+  if (p.S > 1) return launch_fwd_gemm_inst<64, TZ, TX, true>(st, p, x, M, pk, R, C, zero, scale, out, ws);
+  return launch_fwd_gemm_inst<64, TZ, TX, false>(st, p, x, M, pk, R, C, zero, scale, out, ws);
+}
+
+template <typename TZ>
+int launch_fwd_gemm(hipStream_t st, const GemmPlan &p, const void *x, int x_dtype, int64_t M,
+                    const uint8_t *pk, int64_t R, int64_t C, const void *zero, const void *scale,
+                    void *out, void *wsp) {
+  QmmWs ws;
+  char *base = reinterpret_cast<char *>(wsp);
+  ws.counters = reinterpret_cast<int32_t *>(base);
+  ws.x1part = reinterpret_cast<float *>(base + QMM_COUNTER_BYTES);
+  ws.part = reinterpret_cast<float *>(base + QMM_COUNTER_BYTES + p.x1_bytes);
+  if (x_dtype == GPTQ_HIP_BF16)
+    return launch_fwd_gemm_x<TZ, __hip_bfloat16>(st, p, x, M, pk, R, C, zero, scale, out, ws);
+  return launch_fwd_gemm_x<TZ, __half>(st, p, x, M, pk, R, C, zero, scale, out, ws);
 }
 
 // ---------------------------------------------------------------------------- transposed
@@ -853,7 +982,9 @@ extern "C" {
 
 size_t gptq_hip_qmatmul_workspace_bytes(int64_t M, int64_t R, int64_t C, int transpose_b) {
   if (transpose_b || M <= 0 || R <= 0 || C <= 0) return 0;
-  return fwd_plan(M, R, C).total_bytes;
+  // which kernel runs also depends on pointer alignment: enough for either
+  const size_t a = fwd_plan(M, R, C).total_bytes, b = gemm_plan(M, R, C).total_bytes;
+  return a > b ? a : b;
 }
 
 int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
@@ -863,16 +994,19 @@ int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const 
   if (M == 0) return GPTQ_HIP_OK;
   if (!x || !packed || !zero || !scale || !out) return GPTQ_HIP_EINVAL;
   hipStream_t st = as_stream(stream);
-  // The tiled kernel has no split-K: it needs enough 64 x 128 output tiles to occupy the
-  // chip; otherwise 16-row chunks through the split-K kernel (weights re-read from cache) win.
-  if (!transpose_b && fwd_fast_ok(x_dtype, M, R, C, x, packed) && M > 32 &&
-      ceil_div64(C, 128) * ceil_div64(M, GBM) >= 160 &&
-      (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (2 * R) % 8 == 0) {
+  // GEMM-shaped work goes to the tiled kernel (split-K when the output tiles alone do not fill
+  // the chip); small M goes through the 16-row chunked kernel.
+  const GemmPlan gp = gemm_plan(M, R, C);
+  if (!transpose_b && fwd_fast_ok(x_dtype, M, R, C, x, packed) && gp.use &&
+      (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    if (gp.total_bytes && (!ws || ws_bytes < gp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
     switch (zs_dtype) {
-      case GPTQ_HIP_F32: return launch_fwd_gemm<float>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
-      case GPTQ_HIP_F16: return launch_fwd_gemm<__half>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
+      case GPTQ_HIP_F32:
+        return launch_fwd_gemm<float>(st, gp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
+      case GPTQ_HIP_F16:
+        return launch_fwd_gemm<__half>(st, gp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
       case GPTQ_HIP_BF16:
-        return launch_fwd_gemm<__hip_bfloat16>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
+        return launch_fwd_gemm<__hip_bfloat16>(st, gp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
       default: return GPTQ_HIP_EDTYPE;
     }
   }
