@@ -469,20 +469,227 @@ __global__ __launch_bounds__(256) void syrk16_kernel(SyrkArgs p) {
   }
 }
 
+// ---------------------------------------------------------------------------- 16-bit inputs, wide tiles
+// Same product as syrk16_kernel with a 256 x 256 tile per workgroup (128 x 128 per wavefront:
+// 4 x 4 MFMA tiles, 256 accumulator registers).  Two things bound the 128 x 128 version and both
+// scale with the tile edge: the vector-memory pipe costs about as much per contiguous row segment
+// as per instruction (here a load instruction covers two 512-byte segments instead of four
+// 256-byte ones, and feeds four times the MFMA work), and every 16-byte operand fetch from LDS
+// now feeds four 32-cycle MFMAs instead of two.  Slabs are 32 rows (80 KiB of LDS double
+// buffered, one workgroup per CU, one wavefront per SIMD), pitch 40 halves.
+constexpr int W16_TB = 256;
+constexpr int W16_BK = 32;
+constexpr int W16_PITCH = W16_BK + 8;
+constexpr int W16_OP = W16_TB * W16_PITCH;          // halves per operand buffer
+constexpr int W16_LDS_BYTES = 2 * 2 * W16_OP * 2;
+
+template <typename T>
+__global__ __launch_bounds__(256) void syrk16w_kernel(SyrkArgs p) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds16w[];   // [buffer][A, B][feature][k]
+  typedef typename Mfma16<T>::v8 v8;
+  const int ntiles = p.T * (p.T + 1) / 2;
+  // 32 workgroups (one per CU) run on an XCD at a time: make them consecutive work items
+  unsigned item = blockIdx.x;
+  {
+    const unsigned full = gridDim.x & ~255u;
+    if (item < full) {
+      const unsigned xcd = item & 7u, q = item >> 3;
+      item = ((q >> 5) * 8u + xcd) * 32u + (q & 31u);
+    }
+  }
+  const int rs = (int)item / ntiles, t = (int)item - rs * ntiles;
+  int ti, tj;
+  tile_decode(t, p.T, ti, tj);
+  const int m0 = ti * W16_TB, n0 = tj * W16_TB, K = p.K;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
+
+  // staging: wavefronts 0-1 bring in the ti panel (operand A), 2-3 the tj panel (B); 32
+  // neighbouring lanes hold the 32 feature groups of one 8-row block (512 contiguous bytes)
+  const int op = tid >> 7, t7 = tid & 127, fg = t7 & 31, kb = t7 >> 5;
+  const int kb_sw = kb ^ ((fg >> 1) & 3);
+  const int f0 = (op ? n0 : m0) + fg * 8;
+  const bool f_ok = f0 + 8 <= K;
+  const int f0c = f_ok ? f0 : 0;
+  const bool edge_tile = (n0 + W16_TB > K);
+
+  int b = 0, kt = 0, left = 0, nslabs = 0;
+  {
+    const int64_t g0 = (int64_t)rs * p.chunk;
+    int64_t base = 0;
+    bool started = false;
+    int rem = 0;
+    for (int bb = 0; bb < p.nb; ++bb) {
+      const int rows = p.rows[bb];
+      if (!started && g0 < base + rows) {
+        started = true;
+        b = bb;
+        kt = (int)(g0 - base);
+        rem = p.chunk;
+      }
+      if (started && rem > 0) {
+        const int from = (bb == b) ? kt : 0;
+        const int take = min(rows - from, rem);
+        nslabs += (take + W16_BK - 1) / W16_BK;
+        left += take;
+        rem -= take;
+      }
+      base += rows;
+    }
+  }
+
+  struct Slab { hu32x4 r[8]; int nvalid; bool full; };
+  auto load_next = [&](Slab &sl) __attribute__((always_inline)) {
+    const bool live = left > 0;
+    const int bb = live ? b : 0;
+    const int rows = p.rows[bb];
+    const uint16_t *X = reinterpret_cast<const uint16_t *>(p.ptr[bb]);
+    const int k0 = live ? kt : 0;
+    const int avail = live ? min(min(W16_BK, rows - k0), left) : 1;
+    const int row0 = k0 + kb * 8, kend = k0 + avail;
+    sl.nvalid = (live && f_ok) ? kend - row0 : 0;
+    sl.full = live && avail == W16_BK && !edge_tile;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int row = min(row0 + r, kend - 1);
+      sl.r[r] = *reinterpret_cast<const hu32x4 *>(X + (int64_t)row * K + f0c);
+    }
+    const int nkt = k0 + avail;
+    const bool wrap = nkt >= rows;
+    left = live ? left - avail : 0;
+    kt = live ? (wrap ? 0 : nkt) : kt;
+    b = (live && wrap) ? b + 1 : b;
+  };
+  auto store_slab = [&](Slab &sl, int buf) __attribute__((always_inline)) {
+    if (!sl.full) {
+      const hu32x4 zero4 = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int r = 0; r < 8; ++r) sl.r[r] = (r < sl.nvalid) ? sl.r[r] : zero4;
+    }
+    uint16_t *dst = lds16w + (buf * 2 + op) * W16_OP + (fg * 8) * W16_PITCH + kb_sw * 8;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+      hu32x4 o;
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const uint32_t w0 = sl.r[2 * m][c >> 1], w1 = sl.r[2 * m + 1][c >> 1];
+        o[m] = __builtin_amdgcn_perm(w1, w0, sel);
+      }
+      *reinterpret_cast<hu32x4 *>(dst + c * W16_PITCH) = o;
+    }
+  };
+
+  floatx16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  Slab s0, s1, s2;
+  load_next(s0);
+  load_next(s1);
+  load_next(s2);
+  int buf = 0;
+  if (nslabs > 0) store_slab(s0, 0);
+  __syncthreads();
+  int sw_a[4], sw_b[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    sw_a[q] = ((wm * 128 + q * 32 + l32) >> 4) & 3;
+    sw_b[q] = ((wn * 128 + q * 32 + l32) >> 4) & 3;
+  }
+  // operands of one 16-row half of a slab: a[q] / b[q] = rows 32 q + l32 of this wavefront's
+  // 128 features, eight consecutive k of block 2 * half + lhi
+  struct Ops { v8 a[4], b[4]; };
+  auto read_ops = [&](Ops &o, int bufi, int half) __attribute__((always_inline)) {
+    const uint16_t *as = lds16w + (bufi * 2) * W16_OP + (wm * 128 + l32) * W16_PITCH;
+    const uint16_t *bs = lds16w + (bufi * 2 + 1) * W16_OP + (wn * 128 + l32) * W16_PITCH;
+    const int blk = 2 * half + lhi;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      o.a[q] = *reinterpret_cast<const v8 *>(as + q * 32 * W16_PITCH + ((blk ^ sw_a[q]) * 8));
+      o.b[q] = *reinterpret_cast<const v8 *>(bs + q * 32 * W16_PITCH + ((blk ^ sw_b[q]) * 8));
+    }
+  };
+  auto mfma_all = [&](const Ops &o) __attribute__((always_inline)) {
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[ii][j] = Mfma16<T>::mma(o.a[ii], o.b[j], acc[ii][j]);
+  };
+  // One barrier per slab, and no LDS latency in front of the matrix pipe: the operands of the
+  // first half of slab s+1 are fetched (after the barrier that publishes slab s+1) while the
+  // MFMAs of the second half of slab s run, those of the second half while the first half runs.
+  // Slab s+2 goes into the buffer of slab s during step s+1, i.e. after the barrier of step s,
+  // which every wavefront reaches with its reads of slab s complete.
+  Ops o0, o1;
+  if (nslabs > 0) read_ops(o0, 0, 0);
+  auto step = [&](Slab &refill, Slab &next, bool do_load, bool has_next) __attribute__((always_inline)) {
+    if (do_load) load_next(refill);
+    read_ops(o1, buf, 1);
+    mfma_all(o0);
+    if (has_next) store_slab(next, buf ^ 1);
+    __syncthreads();
+    if (has_next) read_ops(o0, buf ^ 1, 0);
+    mfma_all(o1);
+    buf ^= 1;
+  };
+  int i = 0;
+  for (; i + 3 < nslabs; i += 3) {
+    step(s0, s1, true, true);
+    step(s1, s2, true, true);
+    step(s2, s0, true, true);
+  }
+  if (i < nslabs) step(s0, s1, false, i + 1 < nslabs);
+  if (i + 1 < nslabs) step(s1, s2, false, i + 2 < nslabs);
+  if (i + 2 < nslabs) step(s2, s0, false, false);
+
+  if (p.RS == 1) {
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int col = n0 + wn * 128 + j * 32 + l32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = m0 + wm * 128 + ii * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+          if (row < K && col < K) p.H[(int64_t)row * K + col] += acc[ii][j][r];
+        }
+      }
+  } else {
+    float *dst = p.ws + ((int64_t)rs * ntiles + t) * (W16_TB * W16_TB);
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int col = wn * 128 + j * 32 + l32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = wm * 128 + ii * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+          dst[row * W16_TB + col] = acc[ii][j][r];
+        }
+      }
+  }
+}
+
 // H tile += sum over the row slices, in slice order
+template <int TB>
 __global__ __launch_bounds__(256) void syrk_reduce_kernel(float *H, const float *ws, int K, int T,
                                                           int RS) {
   const int ntiles = T * (T + 1) / 2;
   const int t = blockIdx.x;
   int ti, tj;
   tile_decode(t, T, ti, tj);
-  const int m0 = ti * HB, n0 = tj * HB;
-  for (int e = threadIdx.x; e < HB * HB / 4; e += 256) {
-    const int row = e >> 5, c4 = (e & 31) * 4;
+  const int m0 = ti * TB, n0 = tj * TB;
+  for (int e = threadIdx.x; e < TB * TB / 4; e += 256) {
+    const int row = e / (TB / 4), c4 = (e % (TB / 4)) * 4;
     float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int rs = 0; rs < RS; ++rs) {
       const float4 v = *reinterpret_cast<const float4 *>(
-          ws + ((int64_t)rs * ntiles + t) * (HB * HB) + row * HB + c4);
+          ws + ((int64_t)rs * ntiles + t) * (TB * TB) + row * TB + c4);
       s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
     }
     const int gr = m0 + row, gc = n0 + c4;
@@ -502,6 +709,23 @@ int pick_rs(int64_t K) {
   if (rs > 4) rs = (rs <= 8) ? 8 : H_RSMAX;   // multiples of 8 get the per-XCD slice mapping
   return (int)rs;
 }
+
+// Row slices of the wide 16-bit kernel: one workgroup per CU, so the number of work items should
+// be close below a multiple of 256, with at least six rounds.
+int pick_rs_wide(int64_t K) {
+  const int64_t T = ceil_div64(K, W16_TB), ntiles = T * (T + 1) / 2;
+  int best = 1;
+  double best_eff = 0.0;
+  for (int rs = 1; rs <= 32; ++rs) {
+    const double rounds = (double)(ntiles * rs) / 256.0;
+    if (rounds < 6.0 && rs < 32) continue;
+    const double eff = rounds / (double)ceil_div64(ntiles * rs, 256);
+    if (eff > best_eff + 1e-9) { best_eff = eff; best = rs; }
+    if (eff >= 0.97) break;
+  }
+  return best;
+}
+bool use_wide16(int64_t K) { return K >= 1024; }
 
 constexpr int TS = 32;
 
@@ -541,10 +765,17 @@ extern "C" {
 
 size_t gptq_hip_hessian_accumulate_workspace_bytes(int64_t K, int h_dtype) {
   if (K <= 0 || h_dtype != GPTQ_HIP_F32) return 0;
+  // enough for either kernel (which one runs depends on the element type of the batches)
   const int rs = pick_rs(K);
-  if (rs == 1) return 0;
   const int64_t T = ceil_div64(K, HB), ntiles = T * (T + 1) / 2;
-  return (size_t)rs * ntiles * HB * HB * sizeof(float);
+  size_t need = rs == 1 ? 0 : (size_t)rs * ntiles * HB * HB * sizeof(float);
+  if (use_wide16(K)) {
+    const int rw = pick_rs_wide(K);
+    const int64_t Tw = ceil_div64(K, W16_TB), nw = Tw * (Tw + 1) / 2;
+    const size_t wide = rw == 1 ? 0 : (size_t)rw * nw * W16_TB * W16_TB * sizeof(float);
+    if (wide > need) need = wide;
+  }
+  return need;
 }
 
 int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const int64_t *x_rows,
@@ -617,6 +848,37 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
     bool mfma16 = (x_dtype == GPTQ_HIP_F16 || x_dtype == GPTQ_HIP_BF16) && K % 8 == 0;
     for (int i = 0; i < a.nb && mfma16; ++i)
       mfma16 = (reinterpret_cast<uintptr_t>(a.ptr[i]) & 15) == 0;
+    if (mfma16 && use_wide16(K)) {
+      int64_t total_rows = 0;
+      for (int i = 0; i < a.nb; ++i) total_rows += a.rows[i];
+      SyrkArgs w = a;
+      w.T = (int)ceil_div64(K, W16_TB);
+      const int64_t nt = (int64_t)w.T * (w.T + 1) / 2;
+      w.RS = pick_rs_wide(K);
+      const int64_t slabs = ceil_div64(total_rows, W16_BK);
+      if (w.RS > slabs) w.RS = (int)(slabs > 0 ? slabs : 1);
+      const int64_t chunk = round_up64(ceil_div64(total_rows, w.RS), W16_BK);
+      if (chunk > 2147483647LL) return GPTQ_HIP_EINVAL;
+      w.chunk = (int)chunk;
+      const void *fn = x_dtype == GPTQ_HIP_F16
+                           ? reinterpret_cast<const void *>(syrk16w_kernel<__half>)
+                           : reinterpret_cast<const void *>(syrk16w_kernel<__hip_bfloat16>);
+      if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, W16_LDS_BYTES) !=
+          hipSuccess)
+        return GPTQ_HIP_ELAUNCH;
+      const dim3 wgrid((unsigned)(nt * w.RS));
+      if (x_dtype == GPTQ_HIP_F16)
+        hipLaunchKernelGGL(syrk16w_kernel<__half>, wgrid, block, W16_LDS_BYTES, st, w);
+      else
+        hipLaunchKernelGGL(syrk16w_kernel<__hip_bfloat16>, wgrid, block, W16_LDS_BYTES, st, w);
+      GPTQ_CHECK_LAUNCH();
+      if (w.RS > 1) {
+        hipLaunchKernelGGL(syrk_reduce_kernel<W16_TB>, dim3((unsigned)nt), dim3(256), 0, st, H, w.ws,
+                           (int)K, w.T, w.RS);
+        GPTQ_CHECK_LAUNCH();
+      }
+      continue;
+    }
     if (mfma16) {
       int64_t total_rows = 0;
       for (int i = 0; i < a.nb; ++i) total_rows += a.rows[i];
@@ -635,7 +897,7 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
         hipLaunchKernelGGL(syrk16_kernel<__hip_bfloat16>, grid, block, S16_LDS_BYTES, st, a);
       GPTQ_CHECK_LAUNCH();
       if (a.RS > 1) {
-        hipLaunchKernelGGL(syrk_reduce_kernel, dim3((unsigned)ntiles), dim3(256), 0, st, H, a.ws,
+        hipLaunchKernelGGL(syrk_reduce_kernel<HB>, dim3((unsigned)ntiles), dim3(256), 0, st, H, a.ws,
                            (int)K, T, a.RS);
         GPTQ_CHECK_LAUNCH();
       }
@@ -657,7 +919,7 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
 #undef GPTQ_SYRK_LAUNCH
     GPTQ_CHECK_LAUNCH();
     if (a.RS > 1) {
-      hipLaunchKernelGGL(syrk_reduce_kernel, dim3((unsigned)ntiles), dim3(256), 0, st, H, a.ws,
+      hipLaunchKernelGGL(syrk_reduce_kernel<HB>, dim3((unsigned)ntiles), dim3(256), 0, st, H, a.ws,
                          (int)K, T, a.RS);
       GPTQ_CHECK_LAUNCH();
     }

@@ -61,7 +61,11 @@ def test_accumulate_H_half_inputs(G, dt):
 
 @pytest.mark.parametrize("dt", ["float16", "bfloat16"])
 @pytest.mark.parametrize("rows,K,nb", [(37, 256, 20), (2048, 768, 2), (33, 104, 4), (5, 136, 2),
-                                       (1, 384, 1), (130, 4096, 3), (64, 128, 1), (700, 520, 5)])
+                                       (1, 384, 1), (130, 4096, 3), (64, 128, 1), (700, 520, 5),
+                                       # K >= 1024: the 256 x 256-tile kernel (ragged slabs, features
+                                       # past K in the last tile, more row slices than slabs)
+                                       (37, 1032, 7), (1, 1024, 1), (2049, 1288, 2), (95, 2056, 40),
+                                       (3, 1024, 70), (4096, 1024, 4)])
 def test_accumulate_H_16bit_mfma_path(G, rows, K, nb, dt):
     """fp16 / bf16 batches with K % 8 == 0 run on the 16-bit matrix instructions: products of
     two such numbers are exact in fp32, so the result must agree with the closed form of the
