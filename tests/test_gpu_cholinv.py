@@ -39,6 +39,25 @@ def test_cholesky_inv_matches_lapack(G, K):
     assert np.abs(L - ref).max() <= 4 * np.abs(orc - ref).max() + 1e-6
 
 
+def test_cholesky_inv_two_level_blocking(G):
+    """K >= 6144 factorises with a second blocking level (512-row outer blocks; K = 6200 pads to
+    97 diagonal blocks, so the first outer block handled is a partial one).  Reference: LAPACK
+    in fp64 on the host."""
+    import torch
+    K = 6200
+    g = torch.Generator(device="cuda").manual_seed(11)
+    x = torch.randn((K + 300, K), generator=g, device="cuda", dtype=torch.float64)
+    x *= torch.linspace(0.3, 3.0, K, device="cuda", dtype=torch.float64)[None, :]
+    H64 = x.T @ x / x.shape[0]
+    H64 += 0.01 * H64.diagonal().mean() * torch.eye(K, device="cuda", dtype=torch.float64)
+    H = H64.float()
+    L = G._cholesky_inv(H).double()
+    assert bool((torch.triu(L, 1) == 0).all()) and bool((L.diagonal() > 0).all())
+    assert float((L @ L.T @ H.double() - torch.eye(K, device="cuda", dtype=torch.float64)).abs().max()) < 5e-3
+    ref = scipy.linalg.cholesky(np.linalg.inv(H.double().cpu().numpy()), lower=True)
+    assert np.abs(L.cpu().numpy() - ref).max() < 1e-3 * np.abs(ref).max()
+
+
 def test_damp_and_invert_dead_feature_and_damping(G):
     import torch
     rng = np.random.default_rng(4)
