@@ -95,8 +95,10 @@ def bench_qmatmul(reps=240):
     g = torch.Generator(device="cuda")
     g.manual_seed(1)
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    for (K, N) in ((4096, 11008), (11008, 4096)):
-        copies = 24
+    # the two Llama-7B MLP shapes of the benchmark layer, then the OPT-30B fc1 shape (103 MB packed:
+    # decode matmuls of that size run the streaming kernel)
+    for (K, N) in ((4096, 11008), (11008, 4096), (7168, 28672)):
+        copies = 24 if K * N < (1 << 27) else 6
         iws = [torch.randint(0, 256, (K // 2, N), generator=g, device="cuda", dtype=torch.uint8)
                for _ in range(copies)]
         scale = (0.001 + 0.009 * torch.rand(N, generator=g, device="cuda")).to(torch.float16)
@@ -106,6 +108,8 @@ def bench_qmatmul(reps=240):
                  (2048, 1, "float16")]
         if K == K_IN:
             cases += [(1, 0, "bfloat16"), (16, 0, "bfloat16")]
+        if K * N >= (1 << 27):
+            cases = [(1, 0, "float16"), (16, 0, "float16")]
         for (M, tr, xdt) in cases:
             tdt = getattr(torch, xdt)
             xcode = _native.F16 if xdt == "float16" else _native.BF16

@@ -66,7 +66,8 @@ __global__ __launch_bounds__(TPB) void qmm_bwd_simple(const TX *x, int64_t M, co
 // feeds v_mfma_f32_16x16x32_f16:
 //   A = activations  (lane: row m = l % 16, eight k slots of lane group g = l / 16)
 //   B = weights      (lane: channel 16*(l % 16) + t for t = 0..15, same eight k slots)
-// Lane group g owns the packed rows 16*s + 4*i + g (i = 0..3) of k-step s, i.e. the k slots
+// Lane group g owns the packed rows 16*s + 4*g + i (i = 0..3) of k-step s (eight consecutive k,
+// so its activations are 16 contiguous bytes), as the k slots
 // [2r0, 2r1, 2r0+1, 2r1+1, 2r2, 2r3, 2r2+1, 2r3+1]; both operands are built in that order.
 // Nibbles become fp16 with three VALU operations per four codes: one byte permute and two
 // and-or with 0x6400 (fp16 1024), giving 1024 + code for even k and 1024 + 16*code for odd
@@ -141,6 +142,128 @@ struct QmmWs {
   float *part;
 };
 
+// Cross-wavefront reduction and output of one (m-chunk, strip, split) workgroup.  On entry every
+// wavefront has written its partial tile to red[wave][mrows][QSTRIP]; se / so are this lane's
+// activation sums (already reduced over the four lane groups).  IT * blockDim.x >= 16 * QSTRIP.
+template <int IT, typename TZ, typename TX>
+__device__ __forceinline__ void qmm_reduce_and_store(float *red, int *s_last_p, int nw, int mrows,
+                                                     int mvalid, int strip, int split, int m0, int M,
+                                                     int C, int S, const TZ *zero, const TZ *scale,
+                                                     TX *out, const QmmWs &ws, float se, float so) {
+  constexpr bool BF = Act<TX>::BF;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 4, l16 = lane & 15;
+  float *xs = red + (size_t)nw * mrows * QSTRIP;   // [wave][2][16]
+  if (g == 0) { xs[wave * 32 + l16] = se; xs[wave * 32 + 16 + l16] = so; }
+  __syncthreads();
+
+  // epilogue value of one output from the accumulated tile sum v and the activation sums
+  // (bf16: both nibbles carry 128 + code and o is the plain odd-k sum)
+  auto finish = [&](float v, float e, float o, float z, float sc) -> TX {
+    const float r = BF ? (v - 128.f * (e + o)) - z * (e + o)
+                       : (v - 1024.f * (e + o)) - z * (e + 16.f * o);
+    return Act<TX>::out(sc * r);
+  };
+  const int n_items = mvalid * QSTRIP;
+  // x sums of this workgroup: [split][2][16] per (m-chunk, strip)
+  const int64_t x1base = (((int64_t)blockIdx.z * gridDim.x + strip) * S) * 32;
+  if (S == 1) {
+    for (int idx = tid; idx < n_items; idx += blockDim.x) {
+      const int m = idx >> 8, c = idx & 255, n = strip * QSTRIP + c;
+      if (n >= C) continue;
+      const float z = to_f32(zero[n]), sc = to_f32(scale[n]);
+      float v = 0.f, e = 0.f, o = 0.f;
+      for (int w = 0; w < nw; ++w) {
+        v += red[(w * mrows + m) * QSTRIP + c];
+        e += xs[w * 32 + m];
+        o += xs[w * 32 + 16 + m];
+      }
+      out[(int64_t)(m0 + m) * C + n] = finish(v, e, o, z, sc);
+    }
+    return;
+  }
+  for (int idx = tid; idx < n_items; idx += blockDim.x) {
+    const int m = idx >> 8, c = idx & 255, n = strip * QSTRIP + c;
+    if (n >= C) continue;
+    float v = 0.f;
+    for (int w = 0; w < nw; ++w) v += red[(w * mrows + m) * QSTRIP + c];
+    // agent-scope write-through store: visible to every XCD once it has completed
+    __hip_atomic_store(&ws.part[((int64_t)split * M + m0 + m) * C + n], v, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (tid < 32 && (tid & 15) < mvalid) {
+    float x1 = 0.f;
+    for (int w = 0; w < nw; ++w) x1 += xs[w * 32 + tid];
+    __hip_atomic_store(&ws.x1part[x1base + (int64_t)split * 32 + tid], x1, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+  }
+  // Each thread waits for its own write-through stores, then the barrier orders all of them
+  // before the ticket.  (A device-wide fence here would write back / invalidate the whole
+  // L2 of the XCD, which costs tens of microseconds.)
+  __syncthreads();
+  if (tid == 0) {
+    int32_t *ctr = ws.counters + blockIdx.z * gridDim.x + strip;
+    const int ticket = atomicAdd(ctr, 1);
+    *s_last_p = (ticket == S - 1);
+    if (ticket == S - 1)               // every other workgroup of this strip has arrived
+      __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (!*s_last_p) return;
+  // Last workgroup of the strip: sum the S partials in split order.  Loads are agent-scope
+  // (never served from a stale line of this XCD's L2).  Every thread keeps all its outputs
+  // in registers and walks the splits in order, so that the loads of one split (and, through
+  // unrolling, of the next) are in flight together instead of one latency per output.
+  if (tid < 32) {
+    float a = 0.f;
+    for (int sp0 = 0; sp0 < S; sp0 += 8) {
+      float px[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        px[u] = __hip_atomic_load(&ws.x1part[x1base + (int64_t)min(sp0 + u, S - 1) * 32 + tid],
+                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (sp0 + u < S) a += px[u];
+    }
+    xs[tid] = a;     // [0..15] even-k sums, [16..31] odd-k sums, per row m
+  }
+  // n_items <= 4096 = IT * blockDim.x.  The column parameters are fetched together with the
+  // partials (one memory latency less at the end of the chain).
+  float v[IT], zc[IT], scl[IT];
+#pragma unroll
+  for (int it = 0; it < IT; ++it) {
+    const int idx = tid + it * blockDim.x;
+    const int n = min(strip * QSTRIP + (idx & 255), C - 1);
+    v[it] = 0.f;
+    zc[it] = to_f32(zero[n]);
+    scl[it] = to_f32(scale[n]);
+  }
+#pragma unroll 2
+  for (int sp = 0; sp < S; ++sp) {
+    float pv[IT];
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+      const int idx = tid + it * blockDim.x;
+      const int m = idx >> 8, n = strip * QSTRIP + (idx & 255);
+      pv[it] = (idx < n_items && n < C)
+                   ? __hip_atomic_load(&ws.part[((int64_t)sp * M + m0 + m) * C + n],
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                   : 0.f;
+    }
+#pragma unroll
+    for (int it = 0; it < IT; ++it) v[it] += pv[it];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int it = 0; it < IT; ++it) {
+    const int idx = tid + it * blockDim.x;
+    const int m = idx >> 8, n = strip * QSTRIP + (idx & 255);
+    if (idx < n_items && n < C)
+      out[(int64_t)(m0 + m) * C + n] = finish(v[it], xs[m], xs[16 + m], zc[it], scl[it]);
+  }
+}
+
 template <int SPW, typename TZ, typename TX>
 __global__ __launch_bounds__(SPW == 2 ? 1024 : 512) void qmm_fwd_mfma_kernel(
     const TX *x, int M, int K, const uint8_t *pk, int R, int C, const TZ *zero,
@@ -164,7 +287,7 @@ __global__ __launch_bounds__(SPW == 2 ? 1024 : 512) void qmm_fwd_mfma_kernel(
     for (int s = 0; s < SPW; ++s)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int row = r_wave + s * 16 + 4 * i + g;
+        const int row = r_wave + s * 16 + 4 * g + i;
         pr[s][i] = (l16 < mvalid && row < R) ? *reinterpret_cast<const uint32_t *>(xr + 2 * row) : 0u;
       }
   }
@@ -175,7 +298,7 @@ __global__ __launch_bounds__(SPW == 2 ? 1024 : 512) void qmm_fwd_mfma_kernel(
   for (int s = 0; s < SPW; ++s)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int row = r_wave + s * 16 + 4 * i + g;
+      const int row = r_wave + s * 16 + 4 * g + i;
       d[s][i] = (row < R && col0 < C)
                     ? *reinterpret_cast<const uint4 *>(pk + (int64_t)row * C + col0)
                     : make_uint4(0, 0, 0, 0);
@@ -236,116 +359,142 @@ __global__ __launch_bounds__(SPW == 2 ? 1024 : 512) void qmm_fwd_mfma_kernel(
       }
     }
   }
-  float *xs = red + (size_t)nw * mrows * QSTRIP;   // [wave][2][16]
-  if (g == 0) { xs[wave * 32 + l16] = se; xs[wave * 32 + 16 + l16] = so; }
-  __syncthreads();
+  qmm_reduce_and_store<(SPW == 2) ? 4 : 8>(red, &s_last, nw, mrows, mvalid, strip, split, m0, M, C, S,
+                                           zero, scale, out, ws, se, so);
+}
 
-  // epilogue value of one output from the accumulated tile sum v and the activation sums
-  // (bf16: both nibbles carry 128 + code and o is the plain odd-k sum)
-  auto finish = [&](float v, float e, float o, int n) -> TX {
-    const float z = to_f32(zero[n]);
-    const float r = BF ? (v - 128.f * (e + o)) - z * (e + o)
-                       : (v - 1024.f * (e + o)) - z * (e + 16.f * o);
-    return Act<TX>::out(to_f32(scale[n]) * r);
+// ---------------------------------------------------------------------------- MFMA path, streaming
+// The same arithmetic for matrices that are several times larger than what the chip holds in
+// flight.  Above, a workgroup issues all its loads, waits, computes and reduces; its lifetime is
+// a chain of latencies, and with more workgroups than slots the chip runs them in rounds of
+// that lifetime (2.7 TB/s on a 103 MB matrix).  Here a workgroup (4 wavefronts) owns a strip and
+// a long row range and walks it in k-steps of 16 packed rows per wavefront, QS_RING k-steps of
+// loads in flight per wavefront in a register ring: a finished k-step is refilled at once with
+// the loads of k-step t + QS_RING.  The accumulators of all 16 tiles stay in registers, the
+// reduction across wavefronts and splits runs once at the end.  Steps past the end of the
+// range load clamped (valid) addresses and enter with zero activations.
+constexpr int QS_RING = 4;
+constexpr int QS_NW = 4;
+
+template <typename TZ, typename TX>
+__global__ __launch_bounds__(256, 2) void qmm_fwd_stream_kernel(
+    const TX *x, int M, int K, const uint8_t *pk, int R, int C, const TZ *zero,
+    const TZ *scale, TX *out, QmmWs ws, int S, int rows_per_split) {
+  constexpr bool BF = Act<TX>::BF;
+  extern __shared__ float red[];
+  __shared__ int s_last;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int strip = blockIdx.x, split = blockIdx.y, m0 = blockIdx.z * 16;
+  const int mvalid = min(16, M - m0);
+  const int mrows = mvalid <= 4 ? 4 : 16;
+  const int g = lane >> 4, l16 = lane & 15;
+  const int r_begin = split * rows_per_split, r_end = min(R, r_begin + rows_per_split);
+  // k-step t of this wavefront: packed rows r_begin + (t * QS_NW + wave) * 16 + [0, 16)
+  const int groups = (r_end - r_begin + 15) >> 4;                       // 16-row groups of the range
+  const int nsteps = groups > wave ? (groups - wave + QS_NW - 1) / QS_NW : 0;
+
+  const bool m_ok = l16 < mvalid;
+  const TX *xr = x + (int64_t)(m0 + (m_ok ? l16 : 0)) * K;
+  const int col0 = min(strip * QSTRIP + 16 * l16, C - 16);             // C % 16 == 0, C >= 16
+  const uint8_t *wp = pk + col0;
+
+  // Lane group g owns the packed rows 4g .. 4g+3 of a k-step, i.e. 8 consecutive k: its
+  // activations are one 16-byte load (R % 4 == 0 and x 16-byte aligned are preconditions; range
+  // boundaries are multiples of 4 rows, so a group of 4 rows is inside the range or outside).
+  struct Step { uint4 d[4]; uint4 pr; };
+  auto issue = [&](Step &st, int t) __attribute__((always_inline)) {
+    const int rbase = r_begin + (t * QS_NW + wave) * 16 + 4 * g;
+    st.pr = *reinterpret_cast<const uint4 *>(xr + 2 * min(rbase, R - 4));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = min(rbase + i, R - 1);
+      st.d[i] = *reinterpret_cast<const uint4 *>(wp + (int64_t)row * C);
+    }
   };
-  const int n_items = mvalid * QSTRIP;
-  // x sums of this workgroup: [split][2][16] per (m-chunk, strip)
-  const int64_t x1base = (((int64_t)blockIdx.z * gridDim.x + strip) * S) * 32;
-  if (S == 1) {
-    for (int idx = tid; idx < n_items; idx += blockDim.x) {
-      const int m = idx >> 8, c = idx & 255, n = strip * QSTRIP + c;
-      if (n >= C) continue;
-      float v = 0.f, e = 0.f, o = 0.f;
-      for (int w = 0; w < nw; ++w) {
-        v += red[(w * mrows + m) * QSTRIP + c];
-        e += xs[w * 32 + m];
-        o += xs[w * 32 + 16 + m];
-      }
-      out[(int64_t)(m0 + m) * C + n] = finish(v, e, o, n);
+
+  floatx4 acc[16];
+#pragma unroll
+  for (int t = 0; t < 16; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float se = 0.f, so = 0.f;
+  const half2_t sixteenth = half2_t{(_Float16)0.0625f, (_Float16)0.0625f};
+
+  auto consume = [&](Step &st, int t) __attribute__((always_inline)) {
+    const int rbase = r_begin + (t * QS_NW + wave) * 16 + 4 * g;
+    const bool ok = m_ok && t < nsteps && rbase < r_end;
+    uint32_t pr[4];
+    pr[0] = ok ? st.pr.x : 0u;
+    pr[1] = ok ? st.pr.y : 0u;
+    pr[2] = ok ? st.pr.z : 0u;
+    pr[3] = ok ? st.pr.w : 0u;
+    uint4 av;
+    av.x = __builtin_amdgcn_perm(pr[1], pr[0], 0x05040100u);
+    av.z = __builtin_amdgcn_perm(pr[3], pr[2], 0x05040100u);
+    uint32_t o0 = __builtin_amdgcn_perm(pr[1], pr[0], 0x07060302u);
+    uint32_t o1 = __builtin_amdgcn_perm(pr[3], pr[2], 0x07060302u);
+    if (!BF) {
+      o0 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, o0) * sixteenth);
+      o1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, o1) * sixteenth);
     }
-    return;
-  }
-  for (int idx = tid; idx < n_items; idx += blockDim.x) {
-    const int m = idx >> 8, c = idx & 255, n = strip * QSTRIP + c;
-    if (n >= C) continue;
-    float v = 0.f;
-    for (int w = 0; w < nw; ++w) v += red[(w * mrows + m) * QSTRIP + c];
-    // agent-scope write-through store: visible to every XCD once it has completed
-    __hip_atomic_store(&ws.part[((int64_t)split * M + m0 + m) * C + n], v, __ATOMIC_RELAXED,
-                       __HIP_MEMORY_SCOPE_AGENT);
-  }
-  if (tid < 32 && (tid & 15) < mvalid) {
-    float x1 = 0.f;
-    for (int w = 0; w < nw; ++w) x1 += xs[w * 32 + tid];
-    __hip_atomic_store(&ws.x1part[x1base + (int64_t)split * 32 + tid], x1, __ATOMIC_RELAXED,
-                       __HIP_MEMORY_SCOPE_AGENT);
-  }
-  // Each thread waits for its own write-through stores, then the barrier orders all of them
-  // before the ticket.  (A device-wide fence here would write back / invalidate the whole
-  // L2 of the XCD, which costs tens of microseconds.)
-  __syncthreads();
-  if (tid == 0) {
-    int32_t *ctr = ws.counters + blockIdx.z * gridDim.x + strip;
-    const int ticket = atomicAdd(ctr, 1);
-    s_last = (ticket == S - 1);
-    if (ticket == S - 1)               // every other workgroup of this strip has arrived
-      __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  __syncthreads();
-  if (!s_last) return;
-  // Last workgroup of the strip: sum the S partials in split order.  Loads are agent-scope
-  // (never served from a stale line of this XCD's L2).  Every thread keeps all its outputs
-  // in registers and walks the splits in order, so that the loads of one split (and, through
-  // unrolling, of the next) are in flight together instead of one latency per output.
-  if (tid < 32) {
-    float a = 0.f;
-    for (int sp0 = 0; sp0 < S; sp0 += 8) {
-      float px[8];
+    av.y = o0;
+    av.w = o1;
+    se += (Act<TX>::lo(av.x) + Act<TX>::hi(av.x)) + (Act<TX>::lo(av.z) + Act<TX>::hi(av.z));
+    so += (Act<TX>::lo(o0) + Act<TX>::hi(o0)) + (Act<TX>::lo(o1) + Act<TX>::hi(o1));
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
-        px[u] = __hip_atomic_load(&ws.x1part[x1base + (int64_t)min(sp0 + u, S - 1) * 32 + tid],
-                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-      for (int u = 0; u < 8; ++u)
-        if (sp0 + u < S) a += px[u];
+    for (int tl = 0; tl < 16; ++tl) {
+      const int w = tl >> 2, tb = tl & 3;
+      const uint32_t sel = 0x0c000c00u | ((uint32_t)(4 + tb) << 16) | (uint32_t)tb;
+      uint4 bv;
+      dequant_pair<BF>(u4_comp(st.d[0], w), u4_comp(st.d[1], w), sel, bv.x, bv.y);
+      dequant_pair<BF>(u4_comp(st.d[2], w), u4_comp(st.d[3], w), sel, bv.z, bv.w);
+      acc[tl] = Act<TX>::mma(av, bv, acc[tl]);
     }
-    xs[tid] = a;     // [0..15] even-k sums, [16..31] odd-k sums, per row m
-  }
-  // n_items <= 4096; the workgroup size is fixed per instantiation (1024 or 512 threads)
-  constexpr int IT = (SPW == 2) ? 4 : 8;
-  float v[IT];
+  };
+
+  Step ring[QS_RING];
 #pragma unroll
-  for (int it = 0; it < IT; ++it) v[it] = 0.f;
-#pragma unroll 2
-  for (int sp = 0; sp < S; ++sp) {
-    float pv[IT];
+  for (int u = 0; u < QS_RING; ++u) issue(ring[u], u);
+  int t0 = 0;
+  for (; t0 + QS_RING <= nsteps; t0 += QS_RING) {
 #pragma unroll
-    for (int it = 0; it < IT; ++it) {
-      const int idx = tid + it * blockDim.x;
-      const int m = idx >> 8, n = strip * QSTRIP + (idx & 255);
-      pv[it] = (idx < n_items && n < C)
-                   ? __hip_atomic_load(&ws.part[((int64_t)sp * M + m0 + m) * C + n],
-                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                   : 0.f;
+    for (int u = 0; u < QS_RING; ++u) {
+      consume(ring[u], t0 + u);
+      issue(ring[u], t0 + u + QS_RING);
     }
-#pragma unroll
-    for (int it = 0; it < IT; ++it) v[it] += pv[it];
   }
-  __syncthreads();
+  // at most QS_RING - 1 k-steps left, all of them loaded
 #pragma unroll
-  for (int it = 0; it < IT; ++it) {
-    const int idx = tid + it * blockDim.x;
-    const int m = idx >> 8, n = strip * QSTRIP + (idx & 255);
-    if (idx < n_items && n < C) out[(int64_t)(m0 + m) * C + n] = finish(v[it], xs[m], xs[16 + m], n);
+  for (int u = 0; u < QS_RING - 1; ++u)
+    if (t0 + u < nsteps) consume(ring[u], t0 + u);
+
+  se += __shfl_xor(se, 16);
+  se += __shfl_xor(se, 32);
+  so += __shfl_xor(so, 16);
+  so += __shfl_xor(so, 32);
+  // acc[tl][r] = tile[m = 4g + r][channel 16 * l16 + tl]
+  float *slot = red + (size_t)wave * mrows * QSTRIP;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int m = 4 * g + r;
+    if (m < mrows) {
+      float *dst = slot + m * QSTRIP + 16 * l16;
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<float4 *>(dst + 4 * q) =
+            make_float4(acc[4 * q][r], acc[4 * q + 1][r], acc[4 * q + 2][r], acc[4 * q + 3][r]);
+    }
   }
+  qmm_reduce_and_store<16>(red, &s_last, QS_NW, mrows, mvalid, strip, split, m0, M, C, S, zero, scale,
+                           out, ws, se, so);
 }
 
 struct FwdPlan {
   int nw, spw, S, strips, mch;
+  bool stream;             // qmm_fwd_stream_kernel: rows_per_split packed rows per workgroup
+  int rows_per_split;
   size_t lds_bytes, counter_bytes, x1_bytes, part_bytes, total_bytes;
 };
 
-FwdPlan fwd_plan(int64_t M, int64_t R, int64_t C) {
+FwdPlan fwd_plan(int64_t M, int64_t R, int64_t C, bool allow_stream) {
   FwdPlan p;
   p.strips = (int)ceil_div64(C, QSTRIP);
   p.mch = (int)ceil_div64(M, 16);
@@ -354,6 +503,22 @@ FwdPlan fwd_plan(int64_t M, int64_t R, int64_t C) {
   if (M <= 4) { p.nw = 16; p.spw = 2; }
   else { p.nw = 8; p.spw = 4; }
   p.S = (int)ceil_div64(R, (int64_t)p.nw * p.spw * 16);
+  p.stream = false;
+  p.rows_per_split = 0;
+  if (M <= 16 && allow_stream && R % 4 == 0 && C >= 16) {
+    // two 4-wavefront workgroups per CU; streaming pays once a wavefront has >= 8 k-steps
+    // (measured: even at 65 MB of packed weights, 20 - 35 % faster from 80 MB on)
+    int64_t S = 512 / p.strips;
+    if (S < 1) S = 1;
+    const int64_t rows = round_up64(ceil_div64(R, S), QS_NW * 16);
+    if (rows >= 8 * QS_NW * 16) {
+      p.stream = true;
+      p.rows_per_split = (int)rows;
+      p.S = (int)ceil_div64(R, rows);
+      p.nw = QS_NW;
+      p.spw = 1;
+    }
+  }
   const int mrows = (M <= 4) ? 4 : 16;
   p.lds_bytes = ((size_t)p.nw * mrows * QSTRIP + (size_t)p.nw * 32) * sizeof(float);
   p.counter_bytes = QMM_COUNTER_BYTES;
@@ -396,9 +561,32 @@ int launch_fwd_mfma(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, 
 }
 
 template <typename TZ, typename TX>
+int launch_fwd_stream(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, const uint8_t *pk,
+                      int64_t R, int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
+  QmmWs ws;
+  char *base = reinterpret_cast<char *>(wsp);
+  ws.counters = reinterpret_cast<int32_t *>(base);
+  ws.x1part = reinterpret_cast<float *>(base + p.counter_bytes);
+  ws.part = reinterpret_cast<float *>(base + p.counter_bytes + p.x1_bytes);
+  auto kern = qmm_fwd_stream_kernel<TZ, TX>;
+  if (p.strips > QMM_MAX_COUNTERS || p.mch != 1 || C < 16) return GPTQ_HIP_EINVAL;
+  if (p.lds_bytes > 48 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)p.lds_bytes) != hipSuccess)
+    return GPTQ_HIP_ELAUNCH;
+  const dim3 grid((unsigned)p.strips, (unsigned)p.S, 1);
+  hipLaunchKernelGGL(kern, grid, dim3(QS_NW * 64), p.lds_bytes, st, (const TX *)x, (int)M,
+                     (int)(2 * R), pk, (int)R, (int)C, (const TZ *)zero, (const TZ *)scale, (TX *)out,
+                     ws, p.S, p.rows_per_split);
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
+template <typename TZ, typename TX>
 int launch_fwd_mfma_zx(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, const uint8_t *pk,
                        int64_t R, int64_t C, const void *zero, const void *scale, void *out,
                        void *wsp) {
+  if (p.stream) return launch_fwd_stream<TZ, TX>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
   if (p.spw == 2) return launch_fwd_mfma<2, TZ, TX>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
   return launch_fwd_mfma<4, TZ, TX>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
 }
@@ -983,8 +1171,9 @@ extern "C" {
 size_t gptq_hip_qmatmul_workspace_bytes(int64_t M, int64_t R, int64_t C, int transpose_b) {
   if (transpose_b || M <= 0 || R <= 0 || C <= 0) return 0;
   // which kernel runs also depends on pointer alignment: enough for either
-  const size_t a = fwd_plan(M, R, C).total_bytes, b = gemm_plan(M, R, C).total_bytes;
-  return a > b ? a : b;
+  const size_t a = fwd_plan(M, R, C, false).total_bytes, b = gemm_plan(M, R, C).total_bytes;
+  const size_t c = fwd_plan(M, R, C, true).total_bytes;
+  return a > b ? (a > c ? a : c) : (b > c ? b : c);
 }
 
 int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
@@ -1020,7 +1209,7 @@ int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const 
     }
   }
   if (!transpose_b && fwd_fast_ok(x_dtype, M, R, C, x, packed)) {
-    const FwdPlan p = fwd_plan(M, R, C);
+    const FwdPlan p = fwd_plan(M, R, C, (reinterpret_cast<uintptr_t>(x) & 15) == 0);
     if (p.total_bytes && (!ws || ws_bytes < p.total_bytes)) return GPTQ_HIP_EWORKSPACE;
     switch (zs_dtype) {
       case GPTQ_HIP_F32:

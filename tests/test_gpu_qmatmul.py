@@ -123,6 +123,41 @@ def test_qmatmul_bf16_x_mfma_path(OP, M, N, K, zs):
     assert np.all(err <= 1e-2 + 2.0 ** -8 * np.abs(ref)), err.max()
 
 
+@pytest.mark.parametrize("M,N,K,xdt,zs", [(1, 28672, 7168, "float16", "float16"),
+                                            (16, 7168, 28672, "float16", "float32"),
+                                            (3, 29936, 9000, "float16", "float32"),
+                                            (5, 28672, 7168, "bfloat16", "bfloat16"),
+                                            (2, 32000, 5120, "float16", "float16")])
+def test_qmatmul_streaming_kernel_large_matrices(OP, M, N, K, xdt, zs):
+    """M <= 16 on matrices of 80 MB and more runs the streaming kernel (long row range per
+    workgroup, register ring of loads); (3, 29936, 9000) has a ragged last k-step, a partial
+    last strip and fractional zero points.  Reference: fp32 dense product by torch on the
+    device (the host evaluation of these sizes takes minutes)."""
+    import torch
+    import jax_gptq_amd.gptq as G
+    g = torch.Generator(device="cuda").manual_seed(M + N + K)
+    pk = torch.randint(0, 256, (K // 2, N), dtype=torch.uint8, device="cuda", generator=g)
+    tz = getattr(torch, zs)
+    zero = (15.0 * torch.rand((N,), device="cuda", generator=g)).to(tz)
+    scale = (0.001 + 0.009 * torch.rand((N,), device="cuda", generator=g)).to(tz)
+    x = torch.randn((M, K), device="cuda", generator=g).to(getattr(torch, xdt))
+    got = OP.quantized_matmul(x, G.QuantizedMatrix(pk, zero, scale))
+    assert got.dtype == x.dtype and tuple(got.shape) == (M, N)
+    codes = torch.stack([pk & 15, pk >> 4], dim=1).reshape(K, N).float()
+    dense = (codes - zero.float()[None]) * scale.float()[None]
+    del codes
+    ref = x.double() @ dense.double() if M <= 4 else (x.float() @ dense).double()
+    err = (got.double() - ref).abs()
+    rtol = 2.0 ** -8 if xdt == "bfloat16" else 2 * RTOL       # rounding of the result itself
+    assert bool((err <= ATOL + rtol * ref.abs()).all()), float(err.max())
+    # not 16-byte aligned activations take the chunked kernel: same values up to summation order
+    xu = torch.empty((M * K + 2,), device="cuda", dtype=x.dtype)[2:].view(M, K)
+    xu.copy_(x)
+    assert xu.data_ptr() % 16 != 0
+    got_u = OP.quantized_matmul(xu, G.QuantizedMatrix(pk, zero, scale))
+    assert bool(((got_u.double() - ref).abs() <= ATOL + rtol * ref.abs()).all())
+
+
 def test_qmatmul_leading_dims_and_errors(OP):
     qm = _matrix(8, 256, 192)
     rng = np.random.default_rng(7)
