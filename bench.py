@@ -249,20 +249,22 @@ def main():
     # reduction, the zero fill of H and the finalisation, which makes the figure conservative.
     n_tokens = N_BATCH * ROWS
     flop_per_launch = 2.0 * n_tokens * K_IN * K_IN          # the full GEMM the reference executes
-    tiles = (K_IN + 127) // 128
-    executed_flop = flop_per_launch * (tiles + 1) / (2 * tiles)   # upper 128x128 tiles only
+    wide = args.x_dtype == "float32"
+    # the kernels compute the upper tiles only: 128 x 128 (fp32 rows), 256 x 256 (16-bit rows, K >= 1024)
+    tile_edge = 128 if (wide or K_IN < 1024) else 256
+    tiles = (K_IN + tile_edge - 1) // tile_edge
+    executed_flop = flop_per_launch * (tiles + 1) / (2 * tiles)
     achieved = flop_per_launch / (hess_ms * 1e-3) * 1e-12
     executed = executed_flop / (hess_ms * 1e-3) * 1e-12
-    wide = args.x_dtype == "float32"
     peak = FP32_MFMA_PEAK_TFLOPS if wide else MFMA16_PEAK_TFLOPS
     roofline = {"kernel": "syrk_kernel<float> (X^T X, fp32 MFMA, upper tiles)" if wide else
-                          f"syrk16_kernel ({args.x_dtype} X^T X, 16-bit MFMA with fp32 accumulation, upper tiles)",
+                          f"syrk16w_kernel ({args.x_dtype} X^T X, 16-bit MFMA with fp32 accumulation, upper tiles)",
                 "bound": "mfma",
                 "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
                 "frac": round(achieved / peak, 4),
                 # bytes per launch beyond L2 from rocprofv3 FETCH_SIZE + WRITE_SIZE (scaled by what the
                 # counters read for a 1 GiB copy: x2.000 / x1.000), summary kept under profiles/
-                "traffic": 6.48e10 if wide else None,
+                "traffic": 5.79e10 if wide else 8.6e9,
                 "flop_per_launch": flop_per_launch, "avg_launch_ms": round(hess_ms, 4),
                 "launches_per_step": 1,
                 "executed_tflops": round(executed, 2),
