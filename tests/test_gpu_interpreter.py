@@ -324,3 +324,62 @@ def test_gpt2_small_full_shape(T, J):
             warnings.simplefilter("ignore")      # the embedding lookup is not a product: it unpacks
             out_k = J.use_quantized(f, use_kernel=True)(q, batches[0])
         assert float((out_k - out).norm() / out.norm()) < 5e-3
+
+
+def _llama_block_params(T, d, d_ff, seed=0, dtype=None):
+    g = T.Generator(device="cuda")
+    g.manual_seed(seed)
+    dtype = dtype or T.float16
+    n = lambda *s: (0.02 * T.randn(s, generator=g, device="cuda")).to(dtype)
+    return {"ln_1": T.ones(d, device="cuda", dtype=dtype), "ln_2": T.ones(d, device="cuda", dtype=dtype),
+            "q": n(d, d), "k": n(d, d), "v": n(d, d), "o": n(d, d),
+            "gate": n(d, d_ff), "up": n(d, d_ff), "down": n(d_ff, d)}
+
+
+def _llama_block(n_head):
+    import torch
+    import torch.nn.functional as F
+
+    def rms(x, w):
+        xf = x.float()
+        return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-6)).to(x.dtype) * w
+
+    def forward(p, x):                       # x: [B, S, d] hidden states
+        B, S, d = x.shape
+        h = rms(x, p["ln_1"])
+        q, k, v = ((h @ p[n]).reshape(B, S, n_head, d // n_head).transpose(1, 2) for n in ("q", "k", "v"))
+        a = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(B, S, d)
+        x = x + a @ p["o"]
+        h = rms(x, p["ln_2"])
+        return x + (F.silu(h @ p["gate"]) * (h @ p["up"])) @ p["down"]
+    return forward
+
+
+def test_llama7b_shaped_decoder_block(T, J):
+    """One Llama-7B-shaped decoder block (q/k/v/o 4096 x 4096, gate/up 4096 x 11008, down
+    11008 x 4096, fp16 weights N(0, 0.02)) on fp16 hidden states N(0, 1), 16 sequences of 2048
+    tokens: all seven matrices are solved in calling order on the activations of the already
+    quantised part, packed, and the packed block tracks the dense one."""
+    import copy
+    d, d_ff, n_head, S = 4096, 11008, 32, 2048
+    params = _llama_block_params(T, d, d_ff)
+    dense = copy.deepcopy(params)
+    g = T.Generator(device="cuda")
+    g.manual_seed(9)
+    batches = [T.randn((2, S, d), generator=g, device="cuda").half() for _ in range(8)]
+    f = _llama_block(n_head)
+    with T.no_grad():
+        ref = f(dense, batches[0])
+        q = J.quantize(f, params, batches)
+        for name, shape in (("q", (d, d)), ("k", (d, d)), ("v", (d, d)), ("o", (d, d)),
+                            ("gate", (d, d_ff)), ("up", (d, d_ff)), ("down", (d_ff, d))):
+            assert isinstance(q[name], J.QuantizedMatrix), name
+            assert tuple(q[name].shape) == shape and tuple(q[name].int_weight.shape) == (shape[0] // 2, shape[1])
+        assert isinstance(q["ln_1"], T.Tensor)
+        out = J.use_quantized(f)(q, batches[0])
+        out_k = J.use_quantized(f, use_kernel=True)(q, batches[0])
+    # the block's own contribution (output minus the residual input) is what quantisation perturbs
+    dref = (ref - batches[0]).float()
+    # (4-bit codes of Gaussian weights: ~0.28 relative, measured; round-to-nearest gives the same order)
+    assert float(((out - batches[0]).float() - dref).norm() / dref.norm()) < 0.35
+    assert float((out_k.float() - out.float()).norm() / out.float().norm()) < 5e-3
