@@ -359,12 +359,16 @@ def _solve(W, L, params, block_size, out_dtype, want_codes=False):
     return Q, codes
 
 
-def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False):
+def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=None):
     """The per-layer GPTQ solve (reference ``gptq.py:182-212``).
 
     ``W`` is ``[K, N]`` (input features x output channels), ``xs`` a list of calibration
     batches ``[..., K]``.  Returns ``(Q, params)``: ``Q`` the dequantised matrix in ``W``'s
     dtype, ``params`` with ``scale`` / ``zero`` (fp32, one per column) and ``maxq``.
+
+    ``H`` (not in the reference): the result of ``accumulate_H(xs, use_fp64)`` when the caller
+    already has it, e.g. for several matrices that are applied to the same activations; it is
+    left untouched.
     """
     Wt = _float_dev(W)
     if Wt.dim() != 2:
@@ -377,7 +381,9 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False):
     if W32.data_ptr() == Wt.data_ptr():
         W32 = W32.clone()              # the loop consumes its working copy
     quantize_params = get_col_quantize_params(W32)
-    H = accumulate_H(xs, use_fp64=use_fp64)
+    H = accumulate_H(xs, use_fp64=use_fp64) if H is None else H.clone()   # consumed below
+    if H.dim() != 2 or H.shape[0] != H.shape[1] or H.dtype != (torch.float64 if use_fp64 else torch.float32):
+        raise ValueError("H must be the square matrix accumulate_H(xs, use_fp64) returns")
     if H.shape[0] != K:
         raise ValueError(f"calibration feature dim {H.shape[0]} != K={K}")
 

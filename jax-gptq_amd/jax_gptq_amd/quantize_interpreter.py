@@ -26,7 +26,7 @@ import numpy as np
 import torch
 
 from . import _dots
-from .gptq import QuantizedMatrix, _device, gptq, pack_matrix
+from .gptq import QuantizedMatrix, _device, accumulate_H, gptq, pack_matrix
 from .transform import permute_quantized
 
 _tls = threading.local()
@@ -178,6 +178,7 @@ class _Session:
     def __init__(self, leaves, options):
         self.leaves = leaves              # device tensors, original layout, updated in place
         self.results = {}                 # leaf -> QuantizedMatrix in the leaf's layout
+        self._h_cache = None              # (signature, activations, H) of the last product
         self.options = options
         self.aborted = False
 
@@ -213,6 +214,18 @@ class _Session:
                                      "w_contract": dot.w_contract, "x_contract": dot.x_contract})
         return dot.evaluate(reply.to(w_plain.dtype), x)
 
+    def _hessian(self, xs):
+        """``accumulate_H(xs)``, reused when the previous product was applied to the very same
+        activations (q / k / v, gate / up): same memory, layout and version counter, with the
+        previous tensors kept alive so that the memory cannot have been handed out again."""
+        sig = [(x.data_ptr(), tuple(x.shape), tuple(x.stride()), x.dtype, x._version) for x in xs]
+        if self._h_cache is not None and self._h_cache[0] == sig:
+            return self._h_cache[2]
+        self._h_cache = None                      # release the previous activations first
+        H = accumulate_H(xs, use_fp64=self.options["use_fp64"])
+        self._h_cache = (sig, list(xs), H)
+        return H
+
     # -------- one quantisation step (runs on the coordinator)
     def solve(self, requests):
         first = requests[0]
@@ -230,7 +243,7 @@ class _Session:
             raise ValueError(f"block_size={o['block_size']} must divide the contraction size "
                              f"{W2.shape[0]} of parameter {leaf}")
         Q2, qp = gptq(W=W2, xs=xs, block_size=o["block_size"], actorder=o["actorder"],
-                      damping=o["damping"], use_fp64=o["use_fp64"])
+                      damping=o["damping"], use_fp64=o["use_fp64"], H=self._hessian(xs))
         Qt = _dots.from_matrix(Q2, tuple(w.shape), wc)                       # layout fn sees
         scale_shape = tuple(d for i, d in enumerate(w.shape) if i != wc)
         packed = pack_matrix(Qt.contiguous(),

@@ -84,6 +84,41 @@ def test_three_linear_layers_are_solved_sequentially(T, J, use_quantized_activat
     assert T.allclose(manual_result.float(), kernel_output.float(), atol=3e-2, rtol=1e-2)
 
 
+def test_products_on_the_same_activations_share_one_hessian(T, J, monkeypatch):
+    """q / k / v style: three matrices applied to the same activations are solved with one
+    Hessian accumulation; a product on other activations of the same shape gets its own.  The
+    results are those of independent ``gptq`` calls."""
+    G = J.gptq
+    import jax_gptq_amd.quantize_interpreter as QI
+    calls = []
+    real = QI.accumulate_H
+    monkeypatch.setattr(QI, "accumulate_H", lambda xs, use_fp64=False: (calls.append(len(xs)), real(xs, use_fp64))[1])
+    params = {n: _randn(T, 20 + i, 256, 384) / 16 for i, n in enumerate(("q", "k", "v", "o"))}
+    originals = {k: v.clone() for k, v in params.items()}
+    xs = [_randn(T, 200 + i, 48, 256) for i in range(6)]
+
+    def f(p, x):
+        h = x * 1.5
+        a = (h @ p["q"]) + (h @ p["k"]) + (h @ p["v"])
+        h2 = x * 0.5 + 1.0                      # same shape, other values
+        return a + h2 @ p["o"]
+
+    out = J.quantize(f, params, xs, block_size=64)
+    assert calls == [6, 6]                       # one for q/k/v, one for o
+    for n in ("q", "k", "v", "o"):
+        acts = [x * 1.5 for x in xs] if n != "o" else [x * 0.5 + 1.0 for x in xs]
+        Q, p = G.gptq(originals[n].clone(), acts, block_size=64)
+        assert T.equal(out[n].int_weight, G.pack_matrix(Q, p).int_weight), n
+    # gptq leaves a Hessian that it is given untouched
+    H = G.accumulate_H(xs)
+    H0 = H.clone()
+    Q1, _ = G.gptq(originals["q"].clone(), xs, block_size=64, H=H)
+    Q2, _ = G.gptq(originals["q"].clone(), xs, block_size=64)
+    assert T.equal(H, H0) and T.equal(Q1, Q2)
+    with pytest.raises(ValueError):
+        G.gptq(originals["q"].clone(), xs, block_size=64, H=H[:, :-1])
+
+
 def test_transform(T, J):
     """reference test_transform (tests.py:118-138), 1024 x 1024."""
     G = J.gptq
