@@ -561,7 +561,10 @@ __global__ __launch_bounds__(256) void syrk16w_kernel(SyrkArgs p) {
     b = (live && wrap) ? b + 1 : b;
   };
   auto store_slab = [&](Slab &sl, int buf) __attribute__((always_inline)) {
-    if (!sl.full) {
+    // rows past the end of a batch / slice and features past K become zeros; done with selects
+    // for every slab (full ones have nvalid >= 8): a branch here would cut the step into short
+    // scheduling regions and keep this work from being interleaved with the MFMAs
+    {
       const hu32x4 zero4 = {0u, 0u, 0u, 0u};
 #pragma unroll
       for (int r = 0; r < 8; ++r) sl.r[r] = (r < sl.nvalid) ? sl.r[r] : zero4;
@@ -627,14 +630,33 @@ __global__ __launch_bounds__(256) void syrk16w_kernel(SyrkArgs p) {
   // which every wavefront reaches with its reads of slab s complete.
   Ops o0, o1;
   if (nslabs > 0) read_ops(o0, 0, 0);
+  // A wavefront issues in order and is alone on its SIMD, so whatever is not placed between two
+  // MFMAs in program order runs while the matrix pipe idles.  Each half of a step is one
+  // scheduling region (no branches) with 16 MFMAs of 32 cycles; the group barriers spread the
+  // other work of the half over the gaps: operand reads, transposing permutes and LDS writes
+  // in the first half, address arithmetic, global loads and operand reads in the second.
   auto step = [&](Slab &refill, Slab &next, bool do_load, bool has_next) __attribute__((always_inline)) {
-    if (do_load) load_next(refill);
     read_ops(o1, buf, 1);
     mfma_all(o0);
     if (has_next) store_slab(next, buf ^ 1);
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
+      __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);   // VALU
+      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // LDS write
+    }
     __syncthreads();
+    if (do_load) load_next(refill);
     if (has_next) read_ops(o0, buf ^ 1, 0);
     mfma_all(o1);
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);   // VALU
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // global load
+    }
     buf ^= 1;
   };
   int i = 0;
