@@ -239,7 +239,8 @@ __device__ __forceinline__ void qmm_reduce_and_store(float *red, int *s_last_p, 
     zc[it] = to_f32(zero[n]);
     scl[it] = to_f32(scale[n]);
   }
-#pragma unroll 2
+  constexpr int SPLITS_IN_FLIGHT = IT <= 8 ? 4 : 2;     // IT * this many loads per thread at a time
+#pragma unroll SPLITS_IN_FLIGHT
   for (int sp = 0; sp < S; ++sp) {
     float pv[IT];
 #pragma unroll
@@ -264,7 +265,9 @@ __device__ __forceinline__ void qmm_reduce_and_store(float *red, int *s_last_p, 
   }
 }
 
-template <int SPW, typename TZ, typename TX>
+// X16: the activations are 16-byte aligned and R % 4 == 0, so the four (k, k+1) pairs of a lane group
+// (packed rows 4g .. 4g+3) are one 16-byte load instead of four 4-byte ones.
+template <int SPW, typename TZ, typename TX, bool X16>
 __global__ __launch_bounds__(SPW == 2 ? 1024 : 512) void qmm_fwd_mfma_kernel(
     const TX *x, int M, int K, const uint8_t *pk, int R, int C, const TZ *zero,
     const TZ *scale, TX *out, QmmWs ws, int S) {
@@ -284,12 +287,23 @@ __global__ __launch_bounds__(SPW == 2 ? 1024 : 512) void qmm_fwd_mfma_kernel(
   {
     const TX *xr = x + (int64_t)(m0 + l16) * K;
 #pragma unroll
-    for (int s = 0; s < SPW; ++s)
+    for (int s = 0; s < SPW; ++s) {
+      if (X16) {
+        const int row = r_wave + s * 16 + 4 * g;          // R % 4 == 0: the four rows are in or out together
+        const uint4 v = (l16 < mvalid && row < R) ? *reinterpret_cast<const uint4 *>(xr + 2 * row)
+                                                  : make_uint4(0u, 0u, 0u, 0u);
+        pr[s][0] = v.x;
+        pr[s][1] = v.y;
+        pr[s][2] = v.z;
+        pr[s][3] = v.w;
+      } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int row = r_wave + s * 16 + 4 * g + i;
-        pr[s][i] = (l16 < mvalid && row < R) ? *reinterpret_cast<const uint32_t *>(xr + 2 * row) : 0u;
+        for (int i = 0; i < 4; ++i) {
+          const int row = r_wave + s * 16 + 4 * g + i;
+          pr[s][i] = (l16 < mvalid && row < R) ? *reinterpret_cast<const uint32_t *>(xr + 2 * row) : 0u;
+        }
       }
+    }
   }
   // ---- weight loads of this wavefront, all in flight
   uint4 d[SPW][4];
@@ -528,7 +542,7 @@ FwdPlan fwd_plan(int64_t M, int64_t R, int64_t C, bool allow_stream) {
   return p;
 }
 
-template <int SPW, typename TZ, typename TX>
+template <int SPW, typename TZ, typename TX, bool X16>
 int launch_fwd_mfma(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, const uint8_t *pk,
                     int64_t R, int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
   QmmWs ws;
@@ -536,7 +550,7 @@ int launch_fwd_mfma(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, 
   ws.counters = reinterpret_cast<int32_t *>(base);
   ws.x1part = reinterpret_cast<float *>(base + p.counter_bytes);
   ws.part = reinterpret_cast<float *>(base + p.counter_bytes + p.x1_bytes);
-  auto kern = qmm_fwd_mfma_kernel<SPW, TZ, TX>;
+  auto kern = qmm_fwd_mfma_kernel<SPW, TZ, TX, X16>;
   if (p.lds_bytes > 48 * 1024 &&
       hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)p.lds_bytes) != hipSuccess)
@@ -587,8 +601,11 @@ int launch_fwd_mfma_zx(hipStream_t st, const FwdPlan &p, const void *x, int64_t 
                        int64_t R, int64_t C, const void *zero, const void *scale, void *out,
                        void *wsp) {
   if (p.stream) return launch_fwd_stream<TZ, TX>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
-  if (p.spw == 2) return launch_fwd_mfma<2, TZ, TX>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
-  return launch_fwd_mfma<4, TZ, TX>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
+  if (p.spw == 2) return launch_fwd_mfma<2, TZ, TX, false>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
+  // the m-chunks of one call start 16 rows (32 R bytes) apart: aligned together with x when R % 4 == 0
+  if ((reinterpret_cast<uintptr_t>(x) & 15) == 0 && R % 4 == 0)
+    return launch_fwd_mfma<4, TZ, TX, true>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
+  return launch_fwd_mfma<4, TZ, TX, false>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
 }
 
 template <typename TZ>
