@@ -90,6 +90,13 @@ int gptq_hip_damp_invert(void *stream, void *H, int h_dtype, float *W, int64_t K
                          int64_t ldw, double damping, int fix_dead, void *L, float *L32,
                          int32_t *status, void *ws, size_t ws_bytes);
 
+/* Only the dead-feature part of _damp_and_invert (gptq.py:157-159) for a caller that solves
+ * several matrices against one Hessian and keeps the factor L of the first call: rows i of
+ * W [K, N] (fp32, row pitch ldw) with H_ii == 0 are zeroed; H [K, K] (h_dtype F32 or F64) is
+ * the Hessian as accumulated (before damp_invert rewrote its diagonal) and is only read. */
+int gptq_hip_zero_dead_rows(void *stream, const void *H, int h_dtype, int64_t K, float *W, int64_t N,
+                            int64_t ldw);
+
 /* ---- blocked column loop ------------------------------------------------------------
  * Replaces the loop of gptq() with _process_block and the lazy update
  * (gptq.py:199-208, 130-153).  W [K, N] fp32 is consumed (overwritten).  L [K, K]

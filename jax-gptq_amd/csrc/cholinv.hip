@@ -64,6 +64,16 @@ __global__ __launch_bounds__(256) void zero_dead_rows_kernel(float *W, int64_t N
     W[row * ldw + c] = 0.f;
 }
 
+// The same, with the flags taken from the diagonal of an untouched H (H_ii == 0)
+template <typename R>
+__global__ __launch_bounds__(256) void zero_rows_of_dead_features_kernel(const R *H, int64_t K, float *W,
+                                                                         int64_t N, int64_t ldw) {
+  const int64_t row = blockIdx.y;
+  if (H[row * (K + 1)] != R(0)) return;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < N; c += (int64_t)gridDim.x * 256)
+    W[row * ldw + c] = 0.f;
+}
+
 // A (Kp x Kp, padded with the identity) <- H ; Minv <- 0
 template <typename R>
 __global__ __launch_bounds__(256) void pad_copy_kernel(const R *H, int64_t K, R *A, R *Minv,
@@ -376,6 +386,27 @@ int damp_invert(hipStream_t st, R *H, float *W, int64_t K, int64_t N, int64_t ld
 }  // namespace
 
 extern "C" {
+
+int gptq_hip_zero_dead_rows(void *stream, const void *H, int h_dtype, int64_t K, float *W, int64_t N,
+                            int64_t ldw) {
+  if (K < 0 || N < 0 || ldw < N) return GPTQ_HIP_EINVAL;
+  if (K == 0 || N == 0) return GPTQ_HIP_OK;
+  if (!H || !W) return GPTQ_HIP_EINVAL;
+  if (h_dtype != GPTQ_HIP_F32 && h_dtype != GPTQ_HIP_F64) return GPTQ_HIP_EDTYPE;
+  if (K > 65535) return GPTQ_HIP_EINVAL;          // one grid row per feature, as in damp_invert
+  hipStream_t st = as_stream(stream);
+  unsigned gx = (unsigned)ceil_div64(N, 256);
+  if (gx > 32) gx = 32;
+  const dim3 grid(gx, (unsigned)K);
+  if (h_dtype == GPTQ_HIP_F64)
+    hipLaunchKernelGGL(zero_rows_of_dead_features_kernel<double>, grid, dim3(256), 0, st,
+                       reinterpret_cast<const double *>(H), K, W, N, ldw);
+  else
+    hipLaunchKernelGGL(zero_rows_of_dead_features_kernel<float>, grid, dim3(256), 0, st,
+                       reinterpret_cast<const float *>(H), K, W, N, ldw);
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
 
 size_t gptq_hip_damp_invert_workspace_bytes(int64_t K, int h_dtype) {
   if (K <= 0) return 0;

@@ -28,6 +28,7 @@ SIGNATURES = {
     "gptq_hip_damp_invert_workspace_bytes": (_sz, [_i64, _i32]),
     "gptq_hip_damp_invert": (_i32, [_vp, _vp, _i32, _vp, _i64, _i64, _i64, _f64, _i32, _vp, _vp, _vp,
                                     _vp, _sz]),
+    "gptq_hip_zero_dead_rows": (_i32, [_vp, _vp, _i32, _i64, _vp, _i64, _i64]),
     "gptq_hip_solve_workspace_bytes": (_sz, [_i64, _i64, _i32]),
     "gptq_hip_solve": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _i32, _i32, _vp, _i32, _vp, _vp, _sz]),
     "gptq_hip_process_block": (_i32, [_vp, _vp, _i64, _vp, _i64, _i32, _vp, _vp, _i32, _vp, _i32, _vp, _vp]),

@@ -359,16 +359,19 @@ def _solve(W, L, params, block_size, out_dtype, want_codes=False):
     return Q, codes
 
 
-def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=None):
+def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=None, shared=None):
     """The per-layer GPTQ solve (reference ``gptq.py:182-212``).
 
     ``W`` is ``[K, N]`` (input features x output channels), ``xs`` a list of calibration
     batches ``[..., K]``.  Returns ``(Q, params)``: ``Q`` the dequantised matrix in ``W``'s
     dtype, ``params`` with ``scale`` / ``zero`` (fp32, one per column) and ``maxq``.
 
-    ``H`` (not in the reference): the result of ``accumulate_H(xs, use_fp64)`` when the caller
-    already has it, e.g. for several matrices that are applied to the same activations; it is
-    left untouched.
+    Not in the reference, for callers that solve several matrices against the same activations
+    (q / k / v of an attention block): ``H`` is the result of ``accumulate_H(xs, use_fp64)`` when
+    the caller already has it (left untouched); ``shared`` is a dict that this function fills and
+    reads across such calls: the Hessian, and, without ``actorder``, the factor of its damped
+    inverse, which depends on ``xs`` and ``damping`` only.  The results are those of independent
+    calls.
     """
     Wt = _float_dev(W)
     if Wt.dim() != 2:
@@ -381,22 +384,39 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=
     if W32.data_ptr() == Wt.data_ptr():
         W32 = W32.clone()              # the loop consumes its working copy
     quantize_params = get_col_quantize_params(W32)
-    H = accumulate_H(xs, use_fp64=use_fp64) if H is None else H.clone()   # consumed below
+    if H is None and shared is not None:
+        H = shared.get("H")
+    keep = H is not None or shared is not None      # somebody else still needs H as accumulated
+    if H is None:
+        H = accumulate_H(xs, use_fp64=use_fp64)
     if H.dim() != 2 or H.shape[0] != H.shape[1] or H.dtype != (torch.float64 if use_fp64 else torch.float32):
         raise ValueError("H must be the square matrix accumulate_H(xs, use_fp64) returns")
     if H.shape[0] != K:
         raise ValueError(f"calibration feature dim {H.shape[0]} != K={K}")
+    if shared is not None:
+        shared["H"] = H
 
     perm = None
-    if actorder:
-        W32, H, perm = _permute(W32, H)
-
-    # _damp_and_invert (gptq.py:193) and the fp32 cast of the factor (gptq.py:197) in one call
-    _, Hinv, status = _damp_invert(W32, H, damping, fix_dead=True, want_f32=True)
-    any_nan = bool(status[0].item() != 0)
-    if any_nan:
-        xs_nan = any(bool(torch.isnan(_float_dev(x)).any()) for x in xs)
-        raise ValueError(f"NaN when computing Hinv. Features NaN?: {xs_nan}")
+    factor_key = ("factor", float(damping))
+    Hinv = shared.get(factor_key) if (shared is not None and not actorder) else None
+    if Hinv is not None:
+        # same H, same damping: same factor; what is left of _damp_and_invert is the zeroing of
+        # the rows of dead features (gptq.py:157-159)
+        lib = N.load()
+        N.check(lib.gptq_hip_zero_dead_rows(_stream(), _ptr(H), _DT_H[H.dtype], K, _ptr(W32), Nc, Nc),
+                "zero_dead_rows")
+    else:
+        Hw = H.clone() if keep else H           # the factorisation rewrites the diagonal
+        if actorder:
+            W32, Hw, perm = _permute(W32, Hw)
+        # _damp_and_invert (gptq.py:193) and the fp32 cast of the factor (gptq.py:197) in one call
+        _, Hinv, status = _damp_invert(W32, Hw, damping, fix_dead=True, want_f32=True)
+        any_nan = bool(status[0].item() != 0)
+        if any_nan:
+            xs_nan = any(bool(torch.isnan(_float_dev(x)).any()) for x in xs)
+            raise ValueError(f"NaN when computing Hinv. Features NaN?: {xs_nan}")
+        if shared is not None and not actorder:
+            shared[factor_key] = Hinv
 
     Q, _ = _solve(W32, Hinv, quantize_params, block_size, orig_type)
     if perm is not None:

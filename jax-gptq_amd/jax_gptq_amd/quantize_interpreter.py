@@ -214,17 +214,18 @@ class _Session:
                                      "w_contract": dot.w_contract, "x_contract": dot.x_contract})
         return dot.evaluate(reply.to(w_plain.dtype), x)
 
-    def _hessian(self, xs):
-        """``accumulate_H(xs)``, reused when the previous product was applied to the very same
-        activations (q / k / v, gate / up): same memory, layout and version counter, with the
-        previous tensors kept alive so that the memory cannot have been handed out again."""
+    def _shared(self, xs):
+        """What ``gptq`` may reuse from the previous product (the Hessian and the factor of its
+        damped inverse) when that product was applied to the very same activations (q / k / v,
+        gate / up): same memory, layout and version counter, with the previous tensors kept
+        alive so that the memory cannot have been handed out again."""
         sig = [(x.data_ptr(), tuple(x.shape), tuple(x.stride()), x.dtype, x._version) for x in xs]
         if self._h_cache is not None and self._h_cache[0] == sig:
             return self._h_cache[2]
         self._h_cache = None                      # release the previous activations first
-        H = accumulate_H(xs, use_fp64=self.options["use_fp64"])
-        self._h_cache = (sig, list(xs), H)
-        return H
+        shared = {"H": accumulate_H(xs, use_fp64=self.options["use_fp64"])}
+        self._h_cache = (sig, list(xs), shared)
+        return shared
 
     # -------- one quantisation step (runs on the coordinator)
     def solve(self, requests):
@@ -243,7 +244,7 @@ class _Session:
             raise ValueError(f"block_size={o['block_size']} must divide the contraction size "
                              f"{W2.shape[0]} of parameter {leaf}")
         Q2, qp = gptq(W=W2, xs=xs, block_size=o["block_size"], actorder=o["actorder"],
-                      damping=o["damping"], use_fp64=o["use_fp64"], H=self._hessian(xs))
+                      damping=o["damping"], use_fp64=o["use_fp64"], shared=self._shared(xs))
         Qt = _dots.from_matrix(Q2, tuple(w.shape), wc)                       # layout fn sees
         scale_shape = tuple(d for i, d in enumerate(w.shape) if i != wc)
         packed = pack_matrix(Qt.contiguous(),

@@ -97,3 +97,29 @@ def test_gptq_fp64_matches_oracle(G, K, N, n, actorder):
     assert frac <= 1e-3 and mx <= 1, (frac, mx)
     e, er = recon_error(W, Q, X), recon_error(W, Qr, X)
     assert abs(e - er) <= 0.01 * er
+
+
+@pytest.mark.parametrize("use_fp64", [False, True])
+def test_gptq_shared_hessian_and_factor(G, use_fp64):
+    """Several matrices solved against the same activations through ``shared``: one Hessian,
+    one factorisation, results bit-identical to independent calls (a dead feature included)."""
+    import torch
+    rng = np.random.default_rng(17)
+    xs = [rng.standard_normal((96, 192)).astype(np.float32) for _ in range(4)]
+    for x in xs:
+        x[:, 5] = 0
+    Ws = [rng.standard_normal((192, 80 + 16 * i)).astype(np.float32) for i in range(3)]
+    shared = {}
+    got = [G.gptq(W.copy(), xs, block_size=64, use_fp64=use_fp64, shared=shared) for W in Ws]
+    assert set(shared) == {"H", ("factor", 0.01)}
+    assert shared["H"].dtype == (torch.float64 if use_fp64 else torch.float32)
+    for W, (Q, p) in zip(Ws, got):
+        Qi, pi = G.gptq(W.copy(), xs, block_size=64, use_fp64=use_fp64)
+        assert torch.equal(Q, Qi) and torch.equal(p["scale"], pi["scale"]) and torch.equal(p["zero"], pi["zero"])
+        assert bool((Q[5] == 0).all())
+    # another damping value gets a factor of its own; act-order never shares the factor
+    G.gptq(Ws[0].copy(), xs, block_size=64, use_fp64=use_fp64, damping=0.05, shared=shared)
+    assert ("factor", 0.05) in shared
+    Qa, _ = G.gptq(Ws[0].copy(), xs, block_size=64, use_fp64=use_fp64, actorder=True, shared=shared)
+    Qb, _ = G.gptq(Ws[0].copy(), xs, block_size=64, use_fp64=use_fp64, actorder=True)
+    assert torch.equal(Qa, Qb)

@@ -86,16 +86,22 @@ def test_three_linear_layers_are_solved_sequentially(T, J, use_quantized_activat
 
 def test_products_on_the_same_activations_share_one_hessian(T, J, monkeypatch):
     """q / k / v style: three matrices applied to the same activations are solved with one
-    Hessian accumulation; a product on other activations of the same shape gets its own.  The
-    results are those of independent ``gptq`` calls."""
+    Hessian accumulation and one factorisation; a product on other activations of the same shape
+    gets its own.  The results are those of independent ``gptq`` calls, including the zeroed
+    rows of a feature that is dead in the first set of activations only."""
     G = J.gptq
     import jax_gptq_amd.quantize_interpreter as QI
     calls = []
     real = QI.accumulate_H
     monkeypatch.setattr(QI, "accumulate_H", lambda xs, use_fp64=False: (calls.append(len(xs)), real(xs, use_fp64))[1])
+    factorisations = []
+    real_di = G._damp_invert
+    monkeypatch.setattr(G, "_damp_invert", lambda *a, **k: (factorisations.append(1), real_di(*a, **k))[1])
     params = {n: _randn(T, 20 + i, 256, 384) / 16 for i, n in enumerate(("q", "k", "v", "o"))}
     originals = {k: v.clone() for k, v in params.items()}
     xs = [_randn(T, 200 + i, 48, 256) for i in range(6)]
+    for x in xs:
+        x[:, 7] = 0                              # dead for q / k / v; 1.0 in the activations of o
 
     def f(p, x):
         h = x * 1.5
@@ -104,11 +110,14 @@ def test_products_on_the_same_activations_share_one_hessian(T, J, monkeypatch):
         return a + h2 @ p["o"]
 
     out = J.quantize(f, params, xs, block_size=64)
-    assert calls == [6, 6]                       # one for q/k/v, one for o
+    assert calls == [6, 6] and len(factorisations) == 2          # one each for q/k/v, one for o
+    factorisations.clear()
     for n in ("q", "k", "v", "o"):
         acts = [x * 1.5 for x in xs] if n != "o" else [x * 0.5 + 1.0 for x in xs]
         Q, p = G.gptq(originals[n].clone(), acts, block_size=64)
         assert T.equal(out[n].int_weight, G.pack_matrix(Q, p).int_weight), n
+        assert bool((Q[7] == 0).all()) == (n != "o")
+    assert len(factorisations) == 4
     # gptq leaves a Hessian that it is given untouched
     H = G.accumulate_H(xs)
     H0 = H.clone()
