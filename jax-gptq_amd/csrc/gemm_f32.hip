@@ -25,7 +25,7 @@ constexpr int TILE_FLOATS = BK * LDT;  // 2560 >= BM * LDI (2176)
 // loads carry no guards: a load inside a branch makes the compiler wait for it at the join,
 // in front of the MFMAs it is meant to overlap with.
 template <typename T, bool AK, bool FAST>
-__global__ __launch_bounds__(NTHREADS) void gemm_f32_kernel(GemmArgs p) {
+__global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void gemm_f32_kernel(GemmArgs p) {
   __shared__ __attribute__((aligned(16))) float As[2][TILE_FLOATS];
   __shared__ __attribute__((aligned(16))) float Bs[2][TILE_FLOATS];
 
