@@ -359,7 +359,8 @@ def _solve(W, L, params, block_size, out_dtype, want_codes=False):
     return Q, codes
 
 
-def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=None, shared=None):
+def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=None, shared=None,
+         bits=4):
     """The per-layer GPTQ solve (reference ``gptq.py:182-212``).
 
     ``W`` is ``[K, N]`` (input features x output channels), ``xs`` a list of calibration
@@ -371,7 +372,9 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=
     the caller already has it (left untouched); ``shared`` is a dict that this function fills and
     reads across such calls: the Hessian, and, without ``actorder``, the factor of its damped
     inverse, which depends on ``xs`` and ``damping`` only.  The results are those of independent
-    calls.
+    calls.  ``bits`` (1 to 8; the reference's ``gptq`` is fixed at the default of its
+    ``get_quantize_params``, 4): the code width, ``maxq = 2**bits - 1``; only 4-bit results can
+    be packed.
     """
     Wt = _float_dev(W)
     if Wt.dim() != 2:
@@ -383,7 +386,9 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=
     W32 = Wt.to(torch.float32)
     if W32.data_ptr() == Wt.data_ptr():
         W32 = W32.clone()              # the loop consumes its working copy
-    quantize_params = get_col_quantize_params(W32)
+    if not 1 <= int(bits) <= 8:
+        raise ValueError("bits must be between 1 and 8")
+    quantize_params = get_col_quantize_params(W32, bits=int(bits))
     if H is None and shared is not None:
         H = shared.get("H")
     keep = H is not None or shared is not None      # somebody else still needs H as accumulated
@@ -492,6 +497,8 @@ def unpack_colwise(w):
 def pack_matrix(Q, params, contraction_axis=0):
     """Dequantised floats -> integer codes -> packed container (reference ``gptq.py:214-228``)."""
     lib = N.load()
+    if int(params.get("maxq", 15)) != 15:
+        raise NotImplementedError("only 4-bit codes are packed (two per byte, gptq.py:241)")
     Qt = _float_dev(Q)
     scale = _dev(params["scale"])
     zero = _dev(params["zero"])

@@ -217,20 +217,21 @@ def unpermute(Q, perm):
 
 
 def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False,
-         _loop_dtype=np.float32, _H=None):
+         _loop_dtype=np.float32, _H=None, _bits=4):
     """The per-layer solve (reference ``gptq.py:182-212``).
 
     Returns ``(Q, params)``: ``Q`` is the DEQUANTISED matrix in ``W``'s dtype and
     ``params`` holds ``scale``, ``zero`` (fp32, one per column) and ``maxq``.
 
-    ``_loop_dtype`` and ``_H`` are test hooks only: the reference always runs the
-    column loop in fp32 (``gptq.py:184,197``) and always builds ``H`` from ``xs``.
+    ``_loop_dtype``, ``_H`` and ``_bits`` are test hooks only: the reference always runs the
+    column loop in fp32 (``gptq.py:184,197``), always builds ``H`` from ``xs`` and always takes
+    the default width of ``get_quantize_params`` (4 bits, ``gptq.py:105,185``).
     """
     W = np.asarray(W)
     orig_type = W.dtype
     loop_dtype = np.dtype(_loop_dtype)
     W = W.astype(loop_dtype)
-    quantize_params = get_col_quantize_params(W)
+    quantize_params = get_col_quantize_params(W, bits=_bits)
     H = accumulate_H(xs, use_fp64=use_fp64) if _H is None else np.asarray(_H)
 
     perm = None

@@ -140,3 +140,30 @@ def test_gptq_argument_errors(G):
         G.gptq(W, [X], block_size=48)          # does not divide K
     with pytest.raises(ValueError):
         G.gptq(W, [X[:, :32]], block_size=64)  # feature dimension mismatch
+
+
+@pytest.mark.parametrize("bits", [8, 3, 2])
+def test_gptq_other_code_widths(G, bits):
+    """``bits`` other than 4 (not in the reference's ``gptq``, whose parameters come from
+    ``get_quantize_params(w, bits=4)``): same bars against the oracle run at that width, and the
+    error falls with the width."""
+    W, X = _problem(70 + bits, 256, 160, 1500, correlated=True)
+    Q, p = G.gptq(W, [X], bits=bits)
+    Qr, pr = O.gptq(W, [X], _bits=bits)
+    assert p["maxq"] == 2 ** bits - 1 == pr["maxq"]
+    assert np.allclose(to_np(p["scale"]), pr["scale"], rtol=1e-5, atol=0)
+    assert np.allclose(to_np(p["zero"]), pr["zero"], rtol=1e-5, atol=0)
+    codes = lambda q: np.rint(q.astype(np.float32) / pr["scale"][None] + pr["zero"][None]).astype(np.int32)
+    c, cr = codes(to_np(Q)), codes(Qr)
+    assert c.min() >= 0 and c.max() <= 2 ** bits - 1
+    frac, mx = code_stats(c, cr)
+    # 8-bit steps are 1/17 of the 4-bit ones: summation-order differences flip more codes
+    assert frac <= (1e-3 if bits <= 4 else 2e-2) and mx <= 1, (frac, mx)
+    e, er = recon_error(W, to_np(Q), X), recon_error(W, Qr, X)
+    assert abs(e - er) <= 0.01 * er
+    e4 = recon_error(W, to_np(G.gptq(W, [X])[0]), X)
+    assert (e < e4 / 8) if bits == 8 else (e > e4)
+    with pytest.raises(NotImplementedError):
+        G.pack_matrix(Q, p)
+    with pytest.raises(ValueError):
+        G.gptq(W, [X], bits=9)
