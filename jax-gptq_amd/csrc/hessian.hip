@@ -697,6 +697,253 @@ __global__ __launch_bounds__(256) void syrk16w_kernel(SyrkArgs p) {
   }
 }
 
+// ---------------------------------------------------------------------------- 16-bit inputs, loads straight into LDS
+// Same tiles, slices and accumulators as syrk16w_kernel, for the regular case: K a multiple of
+// 256 and every batch a multiple of 32 rows (all slabs full, no feature past K).  There the rows
+// travel from global memory to LDS without touching a register (global_load_lds_dwordx4: a
+// wavefront instruction moves 64 x 16 bytes to 1 KB of consecutive LDS, i.e. two rows of a
+// 256-feature panel), LDS keeps them as they are in memory, [k][feature], and the MFMA operands
+// (eight k of one feature per lane) come from the transposing read ds_read_b64_tr_b16: within
+// 16 lanes, lanes 4r .. 4r+3 address four features each of row r, and lane i receives feature i
+// of the four rows.  Against the register-staged kernel this takes the 96 ring VGPRs, the byte
+// permutes, the LDS writes and the trip of every row through the vector-memory return path out
+// of the loop.
+//
+// LDS: 4 slab buffers of 32 rows; a slab holds, per operand, 16 row pairs of 1024 + 64 bytes.
+// The padding puts the four rows that a 16-lane group reads (the even or the odd rows of four
+// pairs) and the two feature halves of a 32-lane group on eight different 32-byte bank ranges.
+// The k slots of a lane are the even rows of its four pairs, then the odd rows; both operands
+// use the same assignment, so the products pair up.
+//
+// The loads are issued through inline assembly: the compiler then does not know that they
+// write LDS and inserts no waits of its own between them and the LDS reads (with the builtin it
+// waits for every outstanding load before any read, which serialises the pipeline).  The waits
+// that are needed are explicit: before the barrier of step s a wavefront waits for its own
+// loads of slab s (vmcnt leaves the two later slabs in flight) and for its LDS reads of slab
+// s-1, whose buffer is the target of the loads issued right after the barrier.
+constexpr int D16_BK = 32;
+constexpr int D16_NBUF = 4;
+constexpr int D16_PAIR = 1024 + 64;
+constexpr int D16_OP = (D16_BK / 2) * D16_PAIR;
+constexpr int D16_SLAB = 2 * D16_OP;
+constexpr int D16_LDS_BYTES = D16_NBUF * D16_SLAB;
+
+// 16 bytes per lane from global memory to LDS byte address dst (wave-uniform) + 16 * lane
+__device__ __forceinline__ void load_to_lds_16(const void *src, uint32_t dst) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(dst), "v"(src)
+               : "memory", "m0");
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void syrk16d_kernel(SyrkArgs p) {
+  extern __shared__ __attribute__((aligned(16))) char lds16d[];
+  typedef typename Mfma16<T>::v8 v8;
+  typedef short s4 __attribute__((ext_vector_type(4)));
+  typedef short s8 __attribute__((ext_vector_type(8)));
+  typedef __attribute__((address_space(3))) char lds_char;
+  const int ntiles = p.T * (p.T + 1) / 2;
+  unsigned item = blockIdx.x;
+  {
+    const unsigned full = gridDim.x & ~255u;
+    if (item < full) {
+      const unsigned xcd = item & 7u, q = item >> 3;
+      item = ((q >> 5) * 8u + xcd) * 32u + (q & 31u);
+    }
+  }
+  const int rs = (int)item / ntiles, t = (int)item - rs * ntiles;
+  int ti, tj;
+  tile_decode(t, p.T, ti, tj);
+  const int m0 = ti * W16_TB, n0 = tj * W16_TB, K = p.K;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
+
+  // slice [g0, g0 + chunk) of the concatenated batches: first slab (b, kt), number of slabs
+  int b = 0, kt = 0, nslabs = 0;
+  {
+    const int64_t g0 = (int64_t)rs * p.chunk;
+    int64_t base = 0;
+    bool started = false;
+    int rem = 0;
+    for (int bb = 0; bb < p.nb; ++bb) {
+      const int rows = p.rows[bb];
+      if (!started && g0 < base + rows) {
+        started = true;
+        b = bb;
+        kt = (int)(g0 - base);
+        rem = p.chunk;
+      }
+      if (started && rem > 0) {
+        const int from = (bb == b) ? kt : 0;
+        const int take = min(rows - from, rem);
+        nslabs += take / D16_BK;          // rows, chunk and kt are multiples of D16_BK here
+        rem -= take;
+      }
+      base += rows;
+    }
+  }
+
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_char *)lds16d;
+  // loads: wavefronts 0-1 bring in the ti panel (operand A), 2-3 the tj panel (B); a wavefront
+  // owns 8 row pairs of its operand; lanes 0-31 the even row of a pair, 32-63 the odd one
+  const int ld_op = wave >> 1, ld_pair0 = (wave & 1) * 8;
+  const int ld_feat = (ld_op ? n0 : m0) + l32 * 8;
+  const uint32_t ld_dst0 = lds0 + ld_op * D16_OP + ld_pair0 * D16_PAIR;
+  // position of the next slab to load: batch b (base pointer Xb, rows_b rows), row kt
+  const uint16_t *Xb = reinterpret_cast<const uint16_t *>(p.ptr[b]);
+  int rows_b = p.rows[b];
+  int issued = 0;
+  // source of this lane for the 8 loads of the next slab, LDS target of the first of them; then advance
+  auto next_slab = [&](const uint16_t *&src, uint32_t &dst) __attribute__((always_inline)) {
+    src = Xb + (int64_t)(kt + 2 * ld_pair0 + lhi) * K + ld_feat;
+    dst = __builtin_amdgcn_readfirstlane(ld_dst0 + (uint32_t)(issued & (D16_NBUF - 1)) * D16_SLAB);
+    ++issued;
+    kt += D16_BK;
+    if (kt >= rows_b && issued < nslabs) {      // rare: next batch
+      ++b;
+      kt = 0;
+      Xb = reinterpret_cast<const uint16_t *>(p.ptr[b]);
+      rows_b = p.rows[b];
+    }
+  };
+  auto load_pair = [&](const uint16_t *src, uint32_t dst, int j) __attribute__((always_inline)) {
+    load_to_lds_16(src + (int64_t)(2 * j) * K, dst + j * D16_PAIR);
+  };
+
+  // operand reads: 16-lane group g16 = lane / 16 covers features (g16 & 1) * 16 .. + 15 of a
+  // 32-feature MFMA row block and the k half lhi = g16 / 2; within it lane i addresses row pair
+  // 4 * lhi + i / 4 (+ 8 for the second 16 rows of the slab) at features 4 * (i % 4) .. + 3
+  const int rd_i = lane & 15;
+  const uint32_t rd_lane = (uint32_t)((4 * lhi + (rd_i >> 2)) * D16_PAIR + ((((lane >> 4) & 1) * 16 + (rd_i & 3) * 4) * 2));
+  const uint32_t rd_a = rd_lane + (uint32_t)(wm * 128 * 2);
+  const uint32_t rd_b = rd_lane + (uint32_t)(D16_OP + wn * 128 * 2);
+  auto tr8 = [&](uint32_t addr) __attribute__((always_inline)) -> v8 {
+    lds_char *q = (lds_char *)lds16d + addr;
+    const s4 even = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s4 __attribute__((address_space(3))) *)q);
+    const s4 odd = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s4 __attribute__((address_space(3))) *)(q + 512));
+    const s8 w = __builtin_shufflevector(even, odd, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(v8, w);
+  };
+
+  floatx16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // One slab: 8 groups of 4 MFMAs (one row block of A against the four of B).  A wavefront
+  // issues in order and is alone on its SIMD, and the four wavefronts leave the barrier
+  // together: eight loads each, issued at once, queue up in the vector-memory unit and stall the
+  // MFMA issue behind them (measured: a third of the kernel).  So the order is fixed by hand:
+  // one load and the operand reads of the next group between two groups of MFMAs.
+  auto slab_step = [&](int buf, bool dma, const uint16_t *src, uint32_t dst) __attribute__((always_inline)) {
+    const uint32_t h0 = (uint32_t)(buf * D16_SLAB), h1 = h0 + 8 * D16_PAIR;
+    v8 a0[4], b0[4], a1[4], b1[4];
+    auto group = [&](const v8 &a, const v8 (&bq)[4], int ii) __attribute__((always_inline)) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[ii][j] = Mfma16<T>::mma(a, bq[j], acc[ii][j]);
+    };
+    a0[0] = tr8(rd_a + h0);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) b0[q] = tr8(rd_b + h0 + q * 64);
+    if (dma) load_pair(src, dst, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    group(a0[0], b0, 0);
+    a0[1] = tr8(rd_a + h0 + 64);
+    if (dma) load_pair(src, dst, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    group(a0[1], b0, 1);
+    a0[2] = tr8(rd_a + h0 + 128);
+    if (dma) load_pair(src, dst, 2);
+    __builtin_amdgcn_sched_barrier(0);
+    group(a0[2], b0, 2);
+    a0[3] = tr8(rd_a + h0 + 192);
+    b1[0] = tr8(rd_b + h1);
+    b1[1] = tr8(rd_b + h1 + 64);
+    if (dma) load_pair(src, dst, 3);
+    __builtin_amdgcn_sched_barrier(0);
+    group(a0[3], b0, 3);
+    b1[2] = tr8(rd_b + h1 + 128);
+    b1[3] = tr8(rd_b + h1 + 192);
+    a1[0] = tr8(rd_a + h1);
+    if (dma) load_pair(src, dst, 4);
+    __builtin_amdgcn_sched_barrier(0);
+    group(a1[0], b1, 0);
+    a1[1] = tr8(rd_a + h1 + 64);
+    if (dma) load_pair(src, dst, 5);
+    __builtin_amdgcn_sched_barrier(0);
+    group(a1[1], b1, 1);
+    a1[2] = tr8(rd_a + h1 + 128);
+    if (dma) load_pair(src, dst, 6);
+    __builtin_amdgcn_sched_barrier(0);
+    group(a1[2], b1, 2);
+    a1[3] = tr8(rd_a + h1 + 192);
+    if (dma) load_pair(src, dst, 7);
+    __builtin_amdgcn_sched_barrier(0);
+    group(a1[3], b1, 3);
+  };
+
+  for (int s = 0; s < D16_NBUF - 1 && s < nslabs; ++s) {
+    const uint16_t *src;
+    uint32_t dst;
+    next_slab(src, dst);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) load_pair(src, dst, j);
+  }
+  int s = 0;
+  // steady state: slab s + 3 is loaded during step s, two later slabs (16 loads) stay in flight
+  for (; s + D16_NBUF - 1 < nslabs; ++s) {
+    const uint16_t *src;
+    uint32_t dst;
+    next_slab(src, dst);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x4070);        // vmcnt(16) lgkmcnt(0): own loads of slab s, own LDS reads
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    slab_step(s & (D16_NBUF - 1), true, src, dst);
+  }
+  for (; s < nslabs; ++s) {
+    const int later = min(2, nslabs - 1 - s);
+    asm volatile("" ::: "memory");
+    if (later == 2) __builtin_amdgcn_s_waitcnt(0x4070);        // vmcnt(16) lgkmcnt(0)
+    else if (later == 1) __builtin_amdgcn_s_waitcnt(0x0078);   // vmcnt(8) lgkmcnt(0)
+    else __builtin_amdgcn_s_waitcnt(0x0070);                   // vmcnt(0) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    slab_step(s & (D16_NBUF - 1), false, nullptr, 0u);
+  }
+
+  if (p.RS == 1) {
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int col = n0 + wn * 128 + j * 32 + l32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = m0 + wm * 128 + ii * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+          p.H[(int64_t)row * K + col] += acc[ii][j][r];
+        }
+      }
+  } else {
+    float *dst = p.ws + ((int64_t)rs * ntiles + t) * (W16_TB * W16_TB);
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int col = wn * 128 + j * 32 + l32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = wm * 128 + ii * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+          dst[row * W16_TB + col] = acc[ii][j][r];
+        }
+      }
+  }
+}
+
 // H tile += sum over the row slices, in slice order
 template <int TB>
 __global__ __launch_bounds__(256) void syrk_reduce_kernel(float *H, const float *ws, int K, int T,
@@ -882,17 +1129,26 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
       const int64_t chunk = round_up64(ceil_div64(total_rows, w.RS), W16_BK);
       if (chunk > 2147483647LL) return GPTQ_HIP_EINVAL;
       w.chunk = (int)chunk;
-      const void *fn = x_dtype == GPTQ_HIP_F16
-                           ? reinterpret_cast<const void *>(syrk16w_kernel<__half>)
-                           : reinterpret_cast<const void *>(syrk16w_kernel<__hip_bfloat16>);
-      if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, W16_LDS_BYTES) !=
-          hipSuccess)
+      // all slabs full and no feature past K: loads go straight into LDS
+      bool regular = (K % W16_TB == 0);
+      for (int i = 0; i < w.nb; ++i) regular = regular && (w.rows[i] % D16_BK == 0);
+      const bool f16 = x_dtype == GPTQ_HIP_F16;
+      const void *fn = regular ? (f16 ? reinterpret_cast<const void *>(syrk16d_kernel<__half>)
+                                      : reinterpret_cast<const void *>(syrk16d_kernel<__hip_bfloat16>))
+                               : (f16 ? reinterpret_cast<const void *>(syrk16w_kernel<__half>)
+                                      : reinterpret_cast<const void *>(syrk16w_kernel<__hip_bfloat16>));
+      const int lds_bytes = regular ? D16_LDS_BYTES : W16_LDS_BYTES;
+      if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
         return GPTQ_HIP_ELAUNCH;
       const dim3 wgrid((unsigned)(nt * w.RS));
-      if (x_dtype == GPTQ_HIP_F16)
-        hipLaunchKernelGGL(syrk16w_kernel<__half>, wgrid, block, W16_LDS_BYTES, st, w);
+      if (regular && f16)
+        hipLaunchKernelGGL(syrk16d_kernel<__half>, wgrid, block, lds_bytes, st, w);
+      else if (regular)
+        hipLaunchKernelGGL(syrk16d_kernel<__hip_bfloat16>, wgrid, block, lds_bytes, st, w);
+      else if (f16)
+        hipLaunchKernelGGL(syrk16w_kernel<__half>, wgrid, block, lds_bytes, st, w);
       else
-        hipLaunchKernelGGL(syrk16w_kernel<__hip_bfloat16>, wgrid, block, W16_LDS_BYTES, st, w);
+        hipLaunchKernelGGL(syrk16w_kernel<__hip_bfloat16>, wgrid, block, lds_bytes, st, w);
       GPTQ_CHECK_LAUNCH();
       if (w.RS > 1) {
         hipLaunchKernelGGL(syrk_reduce_kernel<W16_TB>, dim3((unsigned)nt), dim3(256), 0, st, H, w.ws,

@@ -65,7 +65,11 @@ def test_accumulate_H_half_inputs(G, dt):
                                        # K >= 1024: the 256 x 256-tile kernel (ragged slabs, features
                                        # past K in the last tile, more row slices than slabs)
                                        (37, 1032, 7), (1, 1024, 1), (2049, 1288, 2), (95, 2056, 40),
-                                       (3, 1024, 70), (4096, 1024, 4)])
+                                       (3, 1024, 70), (4096, 1024, 4),
+                                       # K % 256 == 0 and rows % 32 == 0: loads straight into LDS
+                                       # (one, two, three slabs in all; many short batches; long slices)
+                                       (32, 1024, 1), (64, 1024, 1), (96, 1024, 1), (32, 1280, 37),
+                                       (512, 2304, 9), (2048, 4096, 6)])
 def test_accumulate_H_16bit_mfma_path(G, rows, K, nb, dt):
     """fp16 / bf16 batches with K % 8 == 0 run on the 16-bit matrix instructions: products of
     two such numbers are exact in fp32, so the result must agree with the closed form of the
