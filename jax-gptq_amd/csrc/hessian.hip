@@ -834,86 +834,103 @@ __global__ __launch_bounds__(256) void syrk16d_kernel(SyrkArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // One slab: 8 groups of 4 MFMAs (one row block of A against the four of B).  A wavefront
-  // issues in order and is alone on its SIMD, and the four wavefronts leave the barrier
-  // together: eight loads each, issued at once, queue up in the vector-memory unit and stall the
-  // MFMA issue behind them (measured: a third of the kernel).  So the order is fixed by hand:
-  // one load and the operand reads of the next group between two groups of MFMAs.
-  auto slab_step = [&](int buf, bool dma, const uint16_t *src, uint32_t dst) __attribute__((always_inline)) {
+  // One slab: 8 groups of 4 MFMAs (one row block of A against the four of B), in two halves
+  // of 16 rows.  A wavefront issues in order and is alone on its SIMD, and the four wavefronts
+  // leave the barrier together: eight loads each, issued at once, queue up in the vector-memory
+  // unit and stall the MFMA issue behind them (measured: a third of the kernel).  So the order
+  // is fixed by hand: one load and the operand reads of a later group between two groups of
+  // MFMAs.  The loop is skewed by half a slab: a step runs the second half of slab s-1 from
+  // registers, then the first half of slab s, so that the first reads after a barrier have
+  // four groups of MFMAs in front of their first use.
+  struct Half { v8 a[4], b[4]; };
+  auto group = [&](const v8 &a, const v8 (&bq)[4], int ii) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[ii][j] = Mfma16<T>::mma(a, bq[j], acc[ii][j]);
+  };
+  // second half of the previous slab (operands in `prev`), then the first half of the slab in
+  // `buf`; leaves the operands of its second half in `prev`
+  auto step = [&](Half &prev, int buf, bool dma, const uint16_t *src, uint32_t dst) __attribute__((always_inline)) {
     const uint32_t h0 = (uint32_t)(buf * D16_SLAB), h1 = h0 + 8 * D16_PAIR;
-    v8 a0[4], b0[4], a1[4], b1[4];
-    auto group = [&](const v8 &a, const v8 (&bq)[4], int ii) __attribute__((always_inline)) {
+    Half cur, nxt;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[ii][j] = Mfma16<T>::mma(a, bq[j], acc[ii][j]);
-    };
-    a0[0] = tr8(rd_a + h0);
-#pragma unroll
-    for (int q = 0; q < 4; ++q) b0[q] = tr8(rd_b + h0 + q * 64);
+    for (int q = 0; q < 4; ++q) cur.b[q] = tr8(rd_b + h0 + q * 64);
+    cur.a[0] = tr8(rd_a + h0);
     if (dma) load_pair(src, dst, 0);
     __builtin_amdgcn_sched_barrier(0);
-    group(a0[0], b0, 0);
-    a0[1] = tr8(rd_a + h0 + 64);
+    group(prev.a[0], prev.b, 0);
+    cur.a[1] = tr8(rd_a + h0 + 64);
     if (dma) load_pair(src, dst, 1);
     __builtin_amdgcn_sched_barrier(0);
-    group(a0[1], b0, 1);
-    a0[2] = tr8(rd_a + h0 + 128);
+    group(prev.a[1], prev.b, 1);
+    cur.a[2] = tr8(rd_a + h0 + 128);
     if (dma) load_pair(src, dst, 2);
     __builtin_amdgcn_sched_barrier(0);
-    group(a0[2], b0, 2);
-    a0[3] = tr8(rd_a + h0 + 192);
-    b1[0] = tr8(rd_b + h1);
-    b1[1] = tr8(rd_b + h1 + 64);
+    group(prev.a[2], prev.b, 2);
+    cur.a[3] = tr8(rd_a + h0 + 192);
     if (dma) load_pair(src, dst, 3);
     __builtin_amdgcn_sched_barrier(0);
-    group(a0[3], b0, 3);
-    b1[2] = tr8(rd_b + h1 + 128);
-    b1[3] = tr8(rd_b + h1 + 192);
-    a1[0] = tr8(rd_a + h1);
+    group(prev.a[3], prev.b, 3);
+    nxt.b[0] = tr8(rd_b + h1);
+    nxt.b[1] = tr8(rd_b + h1 + 64);
     if (dma) load_pair(src, dst, 4);
     __builtin_amdgcn_sched_barrier(0);
-    group(a1[0], b1, 0);
-    a1[1] = tr8(rd_a + h1 + 64);
+    group(cur.a[0], cur.b, 0);
+    nxt.b[2] = tr8(rd_b + h1 + 128);
+    nxt.b[3] = tr8(rd_b + h1 + 192);
+    nxt.a[0] = tr8(rd_a + h1);
     if (dma) load_pair(src, dst, 5);
     __builtin_amdgcn_sched_barrier(0);
-    group(a1[1], b1, 1);
-    a1[2] = tr8(rd_a + h1 + 128);
+    group(cur.a[1], cur.b, 1);
+    nxt.a[1] = tr8(rd_a + h1 + 64);
     if (dma) load_pair(src, dst, 6);
     __builtin_amdgcn_sched_barrier(0);
-    group(a1[2], b1, 2);
-    a1[3] = tr8(rd_a + h1 + 192);
+    group(cur.a[2], cur.b, 2);
+    nxt.a[2] = tr8(rd_a + h1 + 128);
     if (dma) load_pair(src, dst, 7);
     __builtin_amdgcn_sched_barrier(0);
-    group(a1[3], b1, 3);
+    group(cur.a[3], cur.b, 3);
+    nxt.a[3] = tr8(rd_a + h1 + 192);
+    __builtin_amdgcn_sched_barrier(0);
+    prev = nxt;
   };
-
-  for (int s = 0; s < D16_NBUF - 1 && s < nslabs; ++s) {
-    const uint16_t *src;
-    uint32_t dst;
-    next_slab(src, dst);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) load_pair(src, dst, j);
-  }
-  int s = 0;
-  // steady state: slab s + 3 is loaded during step s, two later slabs (16 loads) stay in flight
-  for (; s + D16_NBUF - 1 < nslabs; ++s) {
-    const uint16_t *src;
-    uint32_t dst;
-    next_slab(src, dst);
+  // own loads of slab s done (`later` slabs of 8 loads each may stay in flight), own LDS reads
+  // done, then the workgroup barrier: slab s is visible, nobody reads the buffer of slab s-1 any more
+  auto publish = [&](int later) __attribute__((always_inline)) {
     asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_waitcnt(0x4070);        // vmcnt(16) lgkmcnt(0): own loads of slab s, own LDS reads
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    slab_step(s & (D16_NBUF - 1), true, src, dst);
-  }
-  for (; s < nslabs; ++s) {
-    const int later = min(2, nslabs - 1 - s);
-    asm volatile("" ::: "memory");
-    if (later == 2) __builtin_amdgcn_s_waitcnt(0x4070);        // vmcnt(16) lgkmcnt(0)
+    if (later >= 2) __builtin_amdgcn_s_waitcnt(0x4070);        // vmcnt(16) lgkmcnt(0)
     else if (later == 1) __builtin_amdgcn_s_waitcnt(0x0078);   // vmcnt(8) lgkmcnt(0)
     else __builtin_amdgcn_s_waitcnt(0x0070);                   // vmcnt(0) lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    slab_step(s & (D16_NBUF - 1), false, nullptr, 0u);
+  };
+
+  if (nslabs > 0) {
+    for (int s = 0; s < D16_NBUF - 1 && s < nslabs; ++s) {
+      const uint16_t *src;
+      uint32_t dst;
+      next_slab(src, dst);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) load_pair(src, dst, j);
+    }
+    Half prev;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) prev.a[q] = prev.b[q] = v8{0, 0, 0, 0, 0, 0, 0, 0};   // "slab -1": adds zeros
+    int s = 0;
+    // steady state: slab s + 3 is loaded during step s, two later slabs (16 loads) stay in flight
+    for (; s + D16_NBUF - 1 < nslabs; ++s) {
+      const uint16_t *src;
+      uint32_t dst;
+      next_slab(src, dst);
+      publish(2);
+      step(prev, s & (D16_NBUF - 1), true, src, dst);
+    }
+    for (; s < nslabs; ++s) {
+      publish(nslabs - 1 - s);
+      step(prev, s & (D16_NBUF - 1), false, nullptr, 0u);
+    }
+    // second half of the last slab
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii) group(prev.a[ii], prev.b, ii);
   }
 
   if (p.RS == 1) {
