@@ -258,7 +258,7 @@ def main():
     executed = executed_flop / (hess_ms * 1e-3) * 1e-12
     peak = FP32_MFMA_PEAK_TFLOPS if wide else MFMA16_PEAK_TFLOPS
     roofline = {"kernel": "syrk_kernel<float> (X^T X, fp32 MFMA, upper tiles)" if wide else
-                          f"syrk16w_kernel ({args.x_dtype} X^T X, 16-bit MFMA with fp32 accumulation, upper tiles)",
+                          f"syrk16d_kernel ({args.x_dtype} X^T X, 16-bit MFMA with fp32 accumulation, upper tiles)",
                 "bound": "mfma",
                 "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
                 "frac": round(achieved / peak, 4),
