@@ -187,6 +187,100 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(4, 4))
     }
 }
 
+// ---------------------------------------------------------------------------- k = 64, A stored [k][m]
+// The panel products and trailing updates of the blocked factorisation have k = 64: with the
+// pipeline above (16 rows per stage, one stage ahead) such a launch is four exposed memory
+// latencies long, whatever its size.  Here a workgroup issues all the loads of its two
+// 64 x 128 operand tiles at once (16 loads of 16 bytes per thread), stores them to LDS, and
+// multiplies: one latency, one barrier.  fp32 operands, rows 16-byte aligned, m and n
+// multiples of 4; tiles at the edge load clamped (valid) columns and do not store them.
+// In-place use (C == B with m <= 128, or C == A / B tiles that only this workgroup reads) is
+// safe because every load of a tile completes before its first store.
+constexpr int K64 = 64;
+constexpr int K64_LD = BM + 4;                  // LDS row stride (floats): rows stay 16-byte aligned
+constexpr int K64_LDS_BYTES = 2 * K64 * K64_LD * 4;
+
+__global__ __launch_bounds__(NTHREADS) void gemm_f32_tn_k64_kernel(GemmArgs p) {
+  extern __shared__ __attribute__((aligned(16))) float k64_lds[];
+  float *As = k64_lds, *Bs = k64_lds + K64 * K64_LD;
+  int tm, tn;
+  if (p.tri) {
+    const int t = blockIdx.x;
+    int i = (int)((sqrtf(8.f * (float)t + 1.f) - 1.f) * 0.5f);
+    while ((i + 1) * (i + 2) / 2 <= t) ++i;
+    while (i * (i + 1) / 2 > t) --i;
+    const int j = t - i * (i + 1) / 2;  // j <= i
+    if (p.tri == 2) { tm = i; tn = j; } else { tm = j; tn = i; }
+  } else {
+    tn = blockIdx.x;
+    tm = blockIdx.y;
+  }
+  const int m0 = tm * BM, n0 = tn * BN;
+  if (m0 >= p.m || n0 >= p.n) return;
+  const float *A = reinterpret_cast<const float *>(p.A);
+  const float *B = reinterpret_cast<const float *>(p.B);
+  float *C = reinterpret_cast<float *>(p.C);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
+
+  // thread -> rows r, r + 8, ..., r + 56 of both operands, columns c4 .. c4 + 3 of the tile
+  const int r = tid >> 5, c4 = (tid & 31) * 4;
+  const int ca = min(m0 + c4, p.m - 4), cb = min(n0 + c4, p.n - 4);
+  float4 ra[8], rb[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    ra[i] = *reinterpret_cast<const float4 *>(A + (int64_t)(r + 8 * i) * p.lda + ca);
+    rb[i] = *reinterpret_cast<const float4 *>(B + (int64_t)(r + 8 * i) * p.ldb + cb);
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    *reinterpret_cast<float4 *>(&As[(r + 8 * i) * K64_LD + c4]) = ra[i];
+    *reinterpret_cast<float4 *>(&Bs[(r + 8 * i) * K64_LD + c4]) = rb[i];
+  }
+  __syncthreads();
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+#pragma unroll 8
+  for (int kk = 0; kk < K64; kk += 2) {
+    const int krow = kk + lhi;
+    float a[2], b[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      a[t] = As[krow * K64_LD + wm * 64 + t * 32 + l32];
+      b[t] = Bs[krow * K64_LD + wn * 64 + t * 32 + l32];
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+  }
+
+  const float alpha = p.alpha, beta = p.beta;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = n0 + wn * 64 + j * 32 + l32;
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const int row = m0 + wm * 64 + i * 32 + 8 * (q >> 2) + 4 * lhi + (q & 3);
+        if (row < p.m && col < p.n) {
+          float *dst = C + (int64_t)row * p.ldc + col;
+          float v = alpha * acc[i][j][q];
+          if (beta != 0.f) v += beta * (*dst);
+          *dst = v;
+        }
+      }
+    }
+}
+
 }  // namespace
 
 int gptq_gemm_f32(hipStream_t stream, const GemmArgs &a) {
@@ -202,6 +296,17 @@ int gptq_gemm_f32(hipStream_t stream, const GemmArgs &a) {
   }
   if (grid.y > 65535u || grid.z > 65535u) return GPTQ_HIP_EINVAL;
   const dim3 block(NTHREADS);
+  if (a.k == K64 && a.a_kmajor && a.in_dtype == GPTQ_HIP_F32 && a.kskip == 0 && a.batch == 1 &&
+      a.m_step == 0 && a.k_step == 0 && a.m >= 4 && a.n >= 4 && a.m % 4 == 0 && a.n % 4 == 0 &&
+      a.lda % 4 == 0 && a.ldb % 4 == 0 && reinterpret_cast<uintptr_t>(a.A) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(a.B) % 16 == 0) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f32_tn_k64_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, K64_LDS_BYTES) != hipSuccess)
+      return GPTQ_HIP_ELAUNCH;
+    hipLaunchKernelGGL(gemm_f32_tn_k64_kernel, grid, block, K64_LDS_BYTES, stream, a);
+    GPTQ_CHECK_LAUNCH();
+    return GPTQ_HIP_OK;
+  }
   const size_t es = a.in_dtype == GPTQ_HIP_F32 ? 4 : 2;
   const bool fast = a.m % BM == 0 && a.n % BN == 0 && a.k % BK == 0 && a.m_step == 0 &&
                     a.k_step == 0 && a.lda % 4 == 0 && a.ldb % 4 == 0 &&
