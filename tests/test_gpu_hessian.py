@@ -106,3 +106,26 @@ def test_accumulate_H_zero_feature_is_exact_zero(G):
     x[:, 5] = 0
     H = to_np(G.accumulate_H([x]))
     assert np.all(H[5] == 0) and np.all(H[:, 5] == 0)
+
+
+@pytest.mark.parametrize("dt", ["float16", "bfloat16"])
+def test_accumulate_H_16bit_mixed_batch_sizes(G, dt):
+    """Batches of different lengths, all multiples of 32 rows (the loads-straight-into-LDS
+    kernel: row slices then start and end inside batches and cross several of them), and the
+    same data with one batch shortened by a row (the register-staged kernel): both against the
+    closed form."""
+    import torch
+    rng = np.random.default_rng(99)
+    tdt = getattr(torch, dt)
+    K = 1536
+    sizes = [64, 96, 32, 2048, 160, 32, 32, 1024, 448, 32]
+    xs_t = [torch.from_numpy(rng.standard_normal((n, K)).astype(np.float32)).to(tdt).cuda() for n in sizes]
+    ref = _closed_form([x.float().cpu().numpy() for x in xs_t])
+    H = to_np(G.accumulate_H(xs_t))
+    assert np.array_equal(H, H.T)
+    assert np.abs(H - ref).max() < TOL * max(1.0, np.abs(ref).max())
+    ragged = list(xs_t)
+    ragged[3] = xs_t[3][:-1]
+    ref2 = _closed_form([x.float().cpu().numpy() for x in ragged])
+    H2 = to_np(G.accumulate_H(ragged))
+    assert np.abs(H2 - ref2).max() < TOL * max(1.0, np.abs(ref2).max())
