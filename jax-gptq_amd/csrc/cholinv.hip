@@ -105,8 +105,8 @@ __global__ __launch_bounds__(256) void copy_out_kernel(const R *Minv, int64_t Kp
 // standard Cholesky of the index-reversed block: G G^T = J D J, M_bb = J G^T J.  Writes
 // M_bb over A[b,b] (upper part zeroed) and M_bb^-1 = J G^-T J into Minv[b,b].
 //
-// One wavefront and no barrier inside the factorisation: lane r keeps row r of G (64
-// VGPRs) and later column r of G^-1; the loops are fully unrolled.  During the factorisation
+// Lane r of the factorising wavefront keeps row r of G (64 VGPRs), lane j of the inverting
+// wavefront column j of G^-1; the loops are fully unrolled.  During the factorisation
 // the scaled pivot column is handed to the other lanes with v_readlane (lane c's entry
 // becomes a scalar operand of the update of column c), so a step is two instructions per
 // remaining column and touches no memory; during the inversion a row of G is read from LDS
@@ -142,69 +142,79 @@ __device__ __forceinline__ void root_and_inverse(double piv, double &root, doubl
 }
 
 template <typename R>
-__global__ __launch_bounds__(64) void chol_diag_kernel(R *A, R *Minv, int64_t ld, int b,
-                                                       int32_t *status) {
-  __shared__ __attribute__((aligned(16))) R dinv[NB];   // 1 / G[k][k]
-  __shared__ __attribute__((aligned(16))) R Gs[NB * GSTR];   // G, later reused for X = G^-1
-  const int r = threadIdx.x;
+__global__ __launch_bounds__(128) void chol_diag_kernel(R *A, R *Minv, int64_t ld, int b,
+                                                        int32_t *status) {
+  __shared__ __attribute__((aligned(16))) R dinv[NB];        // 1 / G[k][k]
+  __shared__ __attribute__((aligned(16))) R Gs[NB * GSTR];   // G, row major
+  __shared__ __attribute__((aligned(16))) R Xs[NB * (NB + 1)];   // X = G^-1, row major
+  constexpr int XSTR = NB + 1;
+  const int r = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
   R *D = A + (int64_t)b * NB * ld + (int64_t)b * NB;
   R *Dinv = Minv + (int64_t)b * NB * ld + (int64_t)b * NB;
-
-  // G[r][c] (c <= r) = D[63-c][63-r]: for fixed c the lanes read one row of D (coalesced)
   typedef R rowvec __attribute__((ext_vector_type(NB)));   // a vector value, never an alloca
-  rowvec g;
-#pragma unroll
-  for (int c = 0; c < NB; ++c) {
-    g[c] = D[(int64_t)(NB - 1 - c) * ld + (NB - 1 - r)];   // c > r: finite garbage, never used
-  }
 
-  // ---- Cholesky, right-looking: after step k, g[k] of lane r >= k holds G[r][k]
-  bool bad = false;
+  // Two wavefronts, one behind the other: wavefront 0 factorises (lane r keeps row r of G),
+  // publishes column k of G in LDS as soon as it is final and goes on with the trailing update
+  // of step k; wavefront 1 meanwhile computes row k of X = G^-1 (lane j keeps column j of X),
+  // which needs exactly the columns 0..k of row k of G.  One workgroup barrier per step on
+  // both sides (64 each, no other barrier inside the loops).
+  if (wave == 0) {
+    // G[r][c] (c <= r) = D[63-c][63-r]: for fixed c the lanes read one row of D (coalesced)
+    rowvec g;
 #pragma unroll
-  for (int k = 0; k < NB; ++k) {
-    const R piv = lane_bcast(g[k], k);
-    bad = bad || !(piv > R(0));
-    R root, rinv;
-    root_and_inverse(piv, root, rinv);
-    const R l = (r == k) ? root : g[k] * rinv;
-    g[k] = l;
-    if (r == k) dinv[k] = rinv;
-#pragma unroll
-    for (int c = k + 1; c < NB; ++c) {
-      R t = g[c] - l * lane_bcast(l, c);   // G[r][c] -= G[r][k] G[c][k]
-      // Pin the update to this step: left free, the compiler may defer every update until the
-      // element is needed and keep the operands of all steps alive.
-      asm volatile("" : "+v"(t));
-      g[c] = t;
+    for (int c = 0; c < NB; ++c) {
+      g[c] = D[(int64_t)(NB - 1 - c) * ld + (NB - 1 - r)];   // c > r: finite garbage, never used
     }
+    // ---- Cholesky, right-looking: after step k, g[k] of lane r >= k holds G[r][k]
+    bool bad = false;
+#pragma unroll
+    for (int k = 0; k < NB; ++k) {
+      const R piv = lane_bcast(g[k], k);
+      bad = bad || !(piv > R(0));
+      R root, rinv;
+      root_and_inverse(piv, root, rinv);
+      const R l = (r == k) ? root : g[k] * rinv;
+      g[k] = l;
+      Gs[r * GSTR + k] = (k <= r) ? l : R(0);
+      if (r == k) dinv[k] = rinv;
+      __syncthreads();                       // column k is in LDS
+#pragma unroll
+      for (int c = k + 1; c < NB; ++c) {
+        R t = g[c] - l * lane_bcast(l, c);   // G[r][c] -= G[r][k] G[c][k]
+        // Pin the update to this step: left free, the compiler may defer every update until the
+        // element is needed and keep the operands of all steps alive.
+        asm volatile("" : "+v"(t));
+        g[c] = t;
+      }
+    }
+    if (__any(bad) && r == 0) atomicMax(status, b + 1);
+  } else {
+    // ---- X = G^-1, lane j computes column j: x[i] = (delta_ij - sum_{k<i} G[i][k] x[k]) / G[i][i]
+    rowvec x;
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      __syncthreads();                       // row i of G (columns 0..i) is complete
+      R acc = (i == r) ? 1 : 0;
+#pragma unroll
+      for (int k = 0; k < i; ++k) acc -= Gs[i * GSTR + k] * x[k];
+      R xi = acc * dinv[i];   // stays 0 for i < j since every term is 0
+      asm volatile("" : "+v"(xi));         // keeps the row reads of later steps from being hoisted
+      x[i] = xi;
+    }
+#pragma unroll
+    for (int i = 0; i < NB; ++i) Xs[i * XSTR + r] = x[i];
   }
-#pragma unroll
-  for (int c = 0; c < NB; ++c) Gs[r * GSTR + c] = (c <= r) ? g[c] : R(0);
   __syncthreads();
-
-  // ---- X = G^-1, lane j computes column j: x[i] = (delta_ij - sum_{k<i} G[i][k] x[k]) / G[i][i]
-  rowvec x;
-#pragma unroll
-  for (int i = 0; i < NB; ++i) {
-    R acc = (i == r) ? 1 : 0;
-#pragma unroll
-    for (int k = 0; k < i; ++k) acc -= Gs[i * GSTR + k] * x[k];
-    R xi = acc * dinv[i];   // stays 0 for i < j since every term is 0
-    asm volatile("" : "+v"(xi));         // keeps the row reads of later steps from being hoisted
-    x[i] = xi;
+  // M_bb[i][j] = G[63-j][63-i], Minv_bb[i][j] = X[63-j][63-i]  (i >= j), zero above; wavefront 0
+  // writes M_bb, wavefront 1 the inverse
+  if (wave == 0) {
+    for (int i = 0; i < NB; ++i)
+      D[(int64_t)i * ld + r] = (i >= r) ? Gs[(NB - 1 - r) * GSTR + (NB - 1 - i)] : R(0);
+  } else {
+    for (int i = 0; i < NB; ++i)
+      Dinv[(int64_t)i * ld + r] = (i >= r) ? Xs[(NB - 1 - r) * XSTR + (NB - 1 - i)] : R(0);
   }
-  // M_bb[i][j] = G[63-j][63-i]  (i >= j), zero above
-  for (int i = 0; i < NB; ++i)
-    D[(int64_t)i * ld + r] = (i >= r) ? Gs[(NB - 1 - r) * GSTR + (NB - 1 - i)] : R(0);
-  __syncthreads();   // G is not needed any more: its LDS holds X from here on
-  constexpr int XSTR = NB + 1;
-#pragma unroll
-  for (int i = 0; i < NB; ++i) Gs[i * XSTR + r] = x[i];
-  __syncthreads();
-  // Minv_bb[i][j] = X[63-j][63-i]  (i >= j), zero above
-  for (int i = 0; i < NB; ++i)
-    Dinv[(int64_t)i * ld + r] = (i >= r) ? Gs[(NB - 1 - r) * XSTR + (NB - 1 - i)] : R(0);
-  if (__any(bad) && r == 0) atomicMax(status, b + 1);
 }
 
 template <typename R>
@@ -267,7 +277,7 @@ int damp_invert(hipStream_t st, R *H, float *W, int64_t K, int64_t N, int64_t ld
   for (int b1 = nblk; b1 > 0;) {
     const int b0 = ((b1 - 1) / OUTER) * OUTER;      // outer block = diagonal blocks [b0, b1)
     for (int b = b1 - 1; b >= b0; --b) {
-      hipLaunchKernelGGL(chol_diag_kernel<R>, dim3(1), dim3(64), 0, st, p.A, p.Minv, Kp, b, status);
+      hipLaunchKernelGGL(chol_diag_kernel<R>, dim3(1), dim3(128), 0, st, p.A, p.Minv, Kp, b, status);
       GPTQ_CHECK_LAUNCH();
       if (b == 0) break;
       R *panel = p.A + (int64_t)b * NB * Kp;  // rows of block b, columns 0 .. b*NB
