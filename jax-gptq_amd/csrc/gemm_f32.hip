@@ -197,12 +197,20 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(4, 4))
 // In-place use (C == B with m <= 128, or C == A / B tiles that only this workgroup reads) is
 // safe because every load of a tile completes before its first store.
 constexpr int K64 = 64;
-constexpr int K64_LD = BM + 4;                  // LDS row stride (floats): rows stay 16-byte aligned
-constexpr int K64_LDS_BYTES = 2 * K64 * K64_LD * 4;
+constexpr int k64_lds_bytes(int tb) { return 2 * K64 * (tb + 4) * 4; }
 
+// TB = 128: the tile of the kernel above; TB = 64 (32 x 32 per wavefront, a quarter of the MFMA
+// chain) for launches with few tiles, where the length of one workgroup is what counts.
+template <int TB>
 __global__ __launch_bounds__(NTHREADS) void gemm_f32_tn_k64_kernel(GemmArgs p) {
+  constexpr int LD = TB + 4;                    // LDS row stride (floats): rows stay 16-byte aligned
+  constexpr int TPR = TB / 4;                   // threads per operand row
+  constexpr int RPP = NTHREADS / TPR;           // rows per pass
+  constexpr int NP = K64 / RPP;                 // passes (float4 loads per thread and operand)
+  constexpr int WT = TB / 2;                    // wavefront tile edge
+  constexpr int NT = WT / 32;                   // 32 x 32 MFMA tiles per wavefront and dimension
   extern __shared__ __attribute__((aligned(16))) float k64_lds[];
-  float *As = k64_lds, *Bs = k64_lds + K64 * K64_LD;
+  float *As = k64_lds, *Bs = k64_lds + K64 * LD;
   int tm, tn;
   if (p.tri) {
     const int t = blockIdx.x;
@@ -215,7 +223,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_tn_k64_kernel(GemmArgs p) {
     tn = blockIdx.x;
     tm = blockIdx.y;
   }
-  const int m0 = tm * BM, n0 = tn * BN;
+  const int m0 = tm * TB, n0 = tn * TB;
   if (m0 >= p.m || n0 >= p.n) return;
   const float *A = reinterpret_cast<const float *>(p.A);
   const float *B = reinterpret_cast<const float *>(p.B);
@@ -223,54 +231,54 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_tn_k64_kernel(GemmArgs p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
 
-  // thread -> rows r, r + 8, ..., r + 56 of both operands, columns c4 .. c4 + 3 of the tile
-  const int r = tid >> 5, c4 = (tid & 31) * 4;
+  // thread -> rows r, r + RPP, ... of both operands, columns c4 .. c4 + 3 of the tile
+  const int r = tid / TPR, c4 = (tid % TPR) * 4;
   const int ca = min(m0 + c4, p.m - 4), cb = min(n0 + c4, p.n - 4);
-  float4 ra[8], rb[8];
+  float4 ra[NP], rb[NP];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    ra[i] = *reinterpret_cast<const float4 *>(A + (int64_t)(r + 8 * i) * p.lda + ca);
-    rb[i] = *reinterpret_cast<const float4 *>(B + (int64_t)(r + 8 * i) * p.ldb + cb);
+  for (int i = 0; i < NP; ++i) {
+    ra[i] = *reinterpret_cast<const float4 *>(A + (int64_t)(r + RPP * i) * p.lda + ca);
+    rb[i] = *reinterpret_cast<const float4 *>(B + (int64_t)(r + RPP * i) * p.ldb + cb);
   }
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    *reinterpret_cast<float4 *>(&As[(r + 8 * i) * K64_LD + c4]) = ra[i];
-    *reinterpret_cast<float4 *>(&Bs[(r + 8 * i) * K64_LD + c4]) = rb[i];
+  for (int i = 0; i < NP; ++i) {
+    *reinterpret_cast<float4 *>(&As[(r + RPP * i) * LD + c4]) = ra[i];
+    *reinterpret_cast<float4 *>(&Bs[(r + RPP * i) * LD + c4]) = rb[i];
   }
   __syncthreads();
 
-  floatx16 acc[2][2];
+  floatx16 acc[NT][NT];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < NT; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NT; ++j)
 #pragma unroll
       for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
 #pragma unroll 8
   for (int kk = 0; kk < K64; kk += 2) {
     const int krow = kk + lhi;
-    float a[2], b[2];
+    float a[NT], b[NT];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      a[t] = As[krow * K64_LD + wm * 64 + t * 32 + l32];
-      b[t] = Bs[krow * K64_LD + wn * 64 + t * 32 + l32];
+    for (int t = 0; t < NT; ++t) {
+      a[t] = As[krow * LD + wm * WT + t * 32 + l32];
+      b[t] = Bs[krow * LD + wn * WT + t * 32 + l32];
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < NT; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < NT; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
   }
 
   const float alpha = p.alpha, beta = p.beta;
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < NT; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int col = n0 + wn * 64 + j * 32 + l32;
+    for (int j = 0; j < NT; ++j) {
+      const int col = n0 + wn * WT + j * 32 + l32;
 #pragma unroll
       for (int q = 0; q < 16; ++q) {
-        const int row = m0 + wm * 64 + i * 32 + 8 * (q >> 2) + 4 * lhi + (q & 3);
+        const int row = m0 + wm * WT + i * 32 + 8 * (q >> 2) + 4 * lhi + (q & 3);
         if (row < p.m && col < p.n) {
           float *dst = C + (int64_t)row * p.ldc + col;
           float v = alpha * acc[i][j][q];
@@ -300,10 +308,27 @@ int gptq_gemm_f32(hipStream_t stream, const GemmArgs &a) {
       a.m_step == 0 && a.k_step == 0 && a.m >= 4 && a.n >= 4 && a.m % 4 == 0 && a.n % 4 == 0 &&
       a.lda % 4 == 0 && a.ldb % 4 == 0 && reinterpret_cast<uintptr_t>(a.A) % 16 == 0 &&
       reinterpret_cast<uintptr_t>(a.B) % 16 == 0) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f32_tn_k64_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, K64_LDS_BYTES) != hipSuccess)
-      return GPTQ_HIP_ELAUNCH;
-    hipLaunchKernelGGL(gemm_f32_tn_k64_kernel, grid, block, K64_LDS_BYTES, stream, a);
+    // 64 x 64 tiles up to 512 tiles of 128 x 128 (measured: faster up to there, equal beyond), and
+    // when m is a single 64-row block
+    const int64_t t128 = a.tri ? (int64_t)(tm > tn ? tm : tn) * ((tm > tn ? tm : tn) + 1) / 2 : (int64_t)tm * tn;
+    const bool small = a.m <= 64 || t128 < 512;
+    if (small) {
+      const int sm = (a.m + 63) / 64, sn = (a.n + 63) / 64;
+      dim3 g64;
+      if (a.tri) {
+        const int t = sm > sn ? sm : sn;
+        g64 = dim3((unsigned)((int64_t)t * (t + 1) / 2), 1, 1);
+      } else {
+        g64 = dim3((unsigned)sn, (unsigned)sm, 1);
+      }
+      if (g64.y > 65535u) return GPTQ_HIP_EINVAL;
+      hipLaunchKernelGGL(gemm_f32_tn_k64_kernel<64>, g64, block, k64_lds_bytes(64), stream, a);
+    } else {
+      if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f32_tn_k64_kernel<128>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, k64_lds_bytes(128)) != hipSuccess)
+        return GPTQ_HIP_ELAUNCH;
+      hipLaunchKernelGGL(gemm_f32_tn_k64_kernel<128>, grid, block, k64_lds_bytes(128), stream, a);
+    }
     GPTQ_CHECK_LAUNCH();
     return GPTQ_HIP_OK;
   }
