@@ -289,6 +289,86 @@ __global__ __launch_bounds__(NTHREADS) void gemm_f32_tn_k64_kernel(GemmArgs p) {
     }
 }
 
+// ---------------------------------------------------------------------------- k <= 128, A stored [m][k]
+// The same idea for the products of the column loop inside a 512-row group,
+// W[end:ge] -= L[end:ge, start:end] @ Err with k = block size <= 128: 64 x 64 tiles, all loads of
+// both operand tiles in flight at once.  A is kept [row][k] in LDS with an odd stride (129), which
+// makes the MFMA operand reads (32 consecutive rows at one k) conflict free.  fp32, k = 128, 64 or
+// 32, n a multiple of 4, rows 16-byte aligned.
+constexpr int WK_LDB = 64 + 4;
+constexpr int wk_lds_bytes(int k) { return (64 * (k + 1) + k * WK_LDB) * 4; }
+
+template <int KK>   // k, a power of two from 32 to 128: every count below is a compile-time constant
+__global__ __launch_bounds__(NTHREADS) void gemm_f32_nn_wk_kernel(GemmArgs p) {
+  constexpr int LDA = KK + 1;
+  constexpr int KQ = KK / 4;                   // float4 per row of A
+  constexpr int NP = 64 * KQ / NTHREADS;       // float4 per thread and operand (A: 64 x KK, B: KK x 64)
+  extern __shared__ __attribute__((aligned(16))) float wk_lds[];
+  float *As = wk_lds, *Bs = wk_lds + 64 * LDA;
+  const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  const float *A = reinterpret_cast<const float *>(p.A);
+  const float *B = reinterpret_cast<const float *>(p.B);
+  float *C = reinterpret_cast<float *>(p.C);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
+
+  float4 ra[NP], rb[NP];
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const int ia = tid + NTHREADS * i;
+    const int row = min(m0 + ia / KQ, p.m - 1);
+    ra[i] = *reinterpret_cast<const float4 *>(A + (int64_t)row * p.lda + (ia % KQ) * 4);
+    const int col = min(n0 + (ia & 15) * 4, p.n - 4);
+    rb[i] = *reinterpret_cast<const float4 *>(B + (int64_t)(ia >> 4) * p.ldb + col);
+  }
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const int ia = tid + NTHREADS * i;
+    float *dst = &As[(ia / KQ) * LDA + (ia % KQ) * 4];
+    dst[0] = ra[i].x;
+    dst[1] = ra[i].y;
+    dst[2] = ra[i].z;
+    dst[3] = ra[i].w;
+    *reinterpret_cast<float4 *>(&Bs[(ia >> 4) * WK_LDB + (ia & 15) * 4]) = rb[i];
+  }
+  __syncthreads();
+
+  floatx16 acc;
+#pragma unroll
+  for (int q = 0; q < 16; ++q) acc[q] = 0.f;
+  const float *as = As + (wm * 32 + l32) * LDA + lhi;
+  const float *bs = Bs + lhi * WK_LDB + wn * 32 + l32;
+#pragma unroll 16
+  for (int kk = 0; kk < KK; kk += 2)
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(as[kk], bs[kk * WK_LDB], acc, 0, 0, 0);
+
+  const float alpha = p.alpha, beta = p.beta;
+  const int col = n0 + wn * 32 + l32;
+#pragma unroll
+  for (int q = 0; q < 16; ++q) {
+    const int row = m0 + wm * 32 + 8 * (q >> 2) + 4 * lhi + (q & 3);
+    if (row < p.m && col < p.n) {
+      float *dst = C + (int64_t)row * p.ldc + col;
+      float v = alpha * acc[q];
+      if (beta != 0.f) v += beta * (*dst);
+      *dst = v;
+    }
+  }
+}
+
+template <int KK>
+int launch_nn_wk(hipStream_t stream, const GemmArgs &a) {
+  const dim3 g64((unsigned)((a.n + 63) / 64), (unsigned)((a.m + 63) / 64), 1);
+  if (g64.y > 65535u) return GPTQ_HIP_EINVAL;
+  if (wk_lds_bytes(KK) > 48 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f32_nn_wk_kernel<KK>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, wk_lds_bytes(KK)) != hipSuccess)
+    return GPTQ_HIP_ELAUNCH;
+  hipLaunchKernelGGL(gemm_f32_nn_wk_kernel<KK>, g64, dim3(NTHREADS), wk_lds_bytes(KK), stream, a);
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
 }  // namespace
 
 int gptq_gemm_f32(hipStream_t stream, const GemmArgs &a) {
@@ -331,6 +411,14 @@ int gptq_gemm_f32(hipStream_t stream, const GemmArgs &a) {
     }
     GPTQ_CHECK_LAUNCH();
     return GPTQ_HIP_OK;
+  }
+  if (!a.a_kmajor && a.in_dtype == GPTQ_HIP_F32 && (a.k == 128 || a.k == 64 || a.k == 32) &&
+      a.kskip == 0 && a.tri == 0 && a.batch == 1 && a.m_step == 0 && a.k_step == 0 && a.n >= 4 &&
+      a.n % 4 == 0 && a.lda % 4 == 0 && a.ldb % 4 == 0 && reinterpret_cast<uintptr_t>(a.A) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(a.B) % 16 == 0) {
+    if (a.k == 128) return launch_nn_wk<128>(stream, a);
+    if (a.k == 64) return launch_nn_wk<64>(stream, a);
+    return launch_nn_wk<32>(stream, a);
   }
   const size_t es = a.in_dtype == GPTQ_HIP_F32 ? 4 : 2;
   const bool fast = a.m % BM == 0 && a.n % BN == 0 && a.k % BK == 0 && a.m_step == 0 &&
