@@ -339,6 +339,29 @@ int damp_invert(hipStream_t st, R *H, float *W, int64_t K, int64_t N, int64_t ld
   for (int64_t s = NB; s < Kp; s *= 2) {
     const int npairs = (int)ceil_div64(Kp, 2 * s);
     const int64_t pair_stride = 2 * s * (Kp + 1);
+    // The complete pairs go in one batched launch without the ragged-size logic (which would
+    // keep every tile on the guarded load path), the incomplete last pair, if any, in its own.
+    const int nfull = (int)(Kp / (2 * s));
+    auto merge_gemm = [&](const GemmArgs &a) -> int {
+      if (nfull > 0) {
+        GemmArgs f = a;
+        f.batch = nfull;
+        f.m_total = f.m_step = f.k_total = f.k_step = 0;
+        const int rc = gptq_gemm(st, f, (R *)nullptr);
+        if (rc) return rc;
+      }
+      if (nfull < npairs && Kp - s - (int64_t)nfull * 2 * s > 0) {
+        GemmArgs r = a;
+        r.batch = 1;
+        r.A = reinterpret_cast<const R *>(a.A) + (int64_t)nfull * pair_stride;
+        r.B = reinterpret_cast<const R *>(a.B) + (int64_t)nfull * pair_stride;
+        r.C = reinterpret_cast<R *>(a.C) + (int64_t)nfull * pair_stride;
+        r.m_total = a.m_total - nfull * a.m_step;
+        if (a.k_step) r.k_total = a.k_total - nfull * a.k_step;
+        return gptq_gemm(st, r, (R *)nullptr);
+      }
+      return GPTQ_HIP_OK;
+    };
     // T = C * Ainv
     GemmArgs g;
     g.A = p.A + s * Kp;             // C of pair 0: rows [s, 2s), cols [0, s)
@@ -357,7 +380,7 @@ int damp_invert(hipStream_t st, R *H, float *W, int64_t K, int64_t N, int64_t ld
     g.strideA = g.strideB = g.strideC = pair_stride;
     g.m_total = (int)(Kp - s);
     g.m_step = (int)(2 * s);
-    int rc = gptq_gemm(st, g, (R *)nullptr);
+    int rc = merge_gemm(g);
     if (rc) return rc;
     // Minv[B rows, A cols] = -Binv * T
     GemmArgs h;
@@ -379,7 +402,7 @@ int damp_invert(hipStream_t st, R *H, float *W, int64_t K, int64_t N, int64_t ld
     h.m_step = (int)(2 * s);
     h.k_total = (int)(Kp - s);
     h.k_step = (int)(2 * s);
-    rc = gptq_gemm(st, h, (R *)nullptr);
+    rc = merge_gemm(h);
     if (rc) return rc;
   }
 
