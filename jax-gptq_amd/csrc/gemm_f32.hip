@@ -369,6 +369,103 @@ int launch_nn_wk(hipStream_t stream, const GemmArgs &a) {
   return GPTQ_HIP_OK;
 }
 
+// ---------------------------------------------------------------------------- long k, few tiles, A stored [m][k]
+// The triangular-inverse merges are products with k up to K/2 on a handful of tiles (K = 4096:
+// 256 tiles of 128 x 128 at every level): one workgroup per CU walks a long k loop, and with a
+// single slab of prefetch every slab pays most of a memory latency (50 TFLOP/s at best).  This
+// kernel trades operand reuse for parallelism and depth: 64 x 64 tiles (four times the
+// workgroups), and a register ring that keeps three slabs of 16 in flight per thread (one
+// 16-byte load per operand and slab).  Guard-free: m, n multiples of 64, k of 16, rows 16-byte
+// aligned; structural zeros (kskip) and batching as in the general kernel.
+constexpr int N64_LDA = 17;
+constexpr int N64_LDB = 64 + 4;
+
+__global__ __launch_bounds__(NTHREADS) void gemm_f32_nn64_kernel(GemmArgs p) {
+  __shared__ __attribute__((aligned(16))) float As[2][64 * N64_LDA];
+  __shared__ __attribute__((aligned(16))) float Bs[2][BK * N64_LDB];
+  const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64, z = blockIdx.z;
+  int kb = 0, ke = p.k;
+  if (p.kskip & 1) kb = min(n0, ke) & ~(BK - 1);
+  if (p.kskip & 2) ke = min(ke, m0 + 64);
+  const float *A = reinterpret_cast<const float *>(p.A) + (int64_t)z * p.strideA;
+  const float *B = reinterpret_cast<const float *>(p.B) + (int64_t)z * p.strideB;
+  float *C = reinterpret_cast<float *>(p.C) + (int64_t)z * p.strideC;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
+  const int a_row = tid >> 2, a_k = (tid & 3) * 4;       // A: 64 rows x 16 k per slab
+  const int b_row = tid >> 4, b_c = (tid & 15) * 4;      // B: 16 k x 64 columns per slab
+  const float *a_src = A + (int64_t)(m0 + a_row) * p.lda + a_k;
+  const float *b_src = B + (int64_t)b_row * p.ldb + n0 + b_c;
+  const int k_last = max(ke - BK, 0);                    // clamp for the loads past the end (never used)
+
+  struct Slab { float4 a, b; };
+  auto load_slab = [&](int kt, Slab &sl) __attribute__((always_inline)) {
+    const int kc = min(kt, k_last);
+    sl.a = *reinterpret_cast<const float4 *>(a_src + kc);
+    sl.b = *reinterpret_cast<const float4 *>(b_src + (int64_t)kc * p.ldb);
+  };
+  auto store_slab = [&](int buf, const Slab &sl) __attribute__((always_inline)) {
+    float *da = &As[buf][a_row * N64_LDA + a_k];
+    da[0] = sl.a.x;
+    da[1] = sl.a.y;
+    da[2] = sl.a.z;
+    da[3] = sl.a.w;
+    *reinterpret_cast<float4 *>(&Bs[buf][b_row * N64_LDB + b_c]) = sl.b;
+  };
+  floatx16 acc;
+#pragma unroll
+  for (int q = 0; q < 16; ++q) acc[q] = 0.f;
+
+  const int nst = (ke - kb + BK - 1) / BK;
+  if (nst > 0) {
+    Slab s0, s1, s2, s3;
+    load_slab(kb, s0);
+    load_slab(kb + BK, s1);
+    load_slab(kb + 2 * BK, s2);
+    load_slab(kb + 3 * BK, s3);
+    int buf = 0;
+    store_slab(0, s0);
+    __syncthreads();
+    auto step = [&](int kt, Slab &refill, const Slab &next, bool do_load, bool has_next)
+                    __attribute__((always_inline)) {
+      if (do_load) load_slab(kt + 4 * BK, refill);
+      const float *as = &As[buf][(wm * 32 + l32) * N64_LDA + lhi];
+      const float *bs = &Bs[buf][lhi * N64_LDB + wn * 32 + l32];
+#pragma unroll
+      for (int kk = 0; kk < BK; kk += 2)
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(as[kk], bs[kk * N64_LDB], acc, 0, 0, 0);
+      if (has_next) store_slab(buf ^ 1, next);
+      __syncthreads();
+      buf ^= 1;
+    };
+    // full groups of four without exits (the ring stays in flight across the loop head), then a
+    // tail that issues no loads
+    int si = 0, kt = kb;
+    for (; si + 4 < nst; si += 4, kt += 4 * BK) {
+      step(kt, s0, s1, true, true);
+      step(kt + BK, s1, s2, true, true);
+      step(kt + 2 * BK, s2, s3, true, true);
+      step(kt + 3 * BK, s3, s0, true, true);
+    }
+    for (; si < nst; ++si, kt += BK) {      // at most four slabs, all of them loaded
+      step(kt, s0, s1, false, si + 1 < nst);
+      s1 = s2;
+      s2 = s3;
+    }
+  }
+
+  const float alpha = p.alpha, beta = p.beta;
+  const int col = n0 + wn * 32 + l32;
+#pragma unroll
+  for (int q = 0; q < 16; ++q) {
+    const int row = m0 + wm * 32 + 8 * (q >> 2) + 4 * lhi + (q & 3);
+    float *dst = C + (int64_t)row * p.ldc + col;
+    float v = alpha * acc[q];
+    if (beta != 0.f) v += beta * (*dst);
+    *dst = v;
+  }
+}
+
 }  // namespace
 
 int gptq_gemm_f32(hipStream_t stream, const GemmArgs &a) {
@@ -419,6 +516,18 @@ int gptq_gemm_f32(hipStream_t stream, const GemmArgs &a) {
     if (a.k == 128) return launch_nn_wk<128>(stream, a);
     if (a.k == 64) return launch_nn_wk<64>(stream, a);
     return launch_nn_wk<32>(stream, a);
+  }
+  // few tiles and a long k loop: 64 x 64 tiles with a deep register ring
+  if (!a.a_kmajor && a.in_dtype == GPTQ_HIP_F32 && a.tri == 0 && a.m_step == 0 && a.k_step == 0 &&
+      a.m % 64 == 0 && a.n % 64 == 0 && a.k % BK == 0 && a.k >= 4 * BK &&
+      (int64_t)tm * tn * a.batch <= 512 && a.lda % 4 == 0 && a.ldb % 4 == 0 &&
+      reinterpret_cast<uintptr_t>(a.A) % 16 == 0 && reinterpret_cast<uintptr_t>(a.B) % 16 == 0 &&
+      (a.batch == 1 || (a.strideA % 4 == 0 && a.strideB % 4 == 0))) {
+    const dim3 g64((unsigned)(a.n / 64), (unsigned)(a.m / 64), (unsigned)a.batch);
+    if (g64.y > 65535u || g64.z > 65535u) return GPTQ_HIP_EINVAL;
+    hipLaunchKernelGGL(gemm_f32_nn64_kernel, g64, block, 0, stream, a);
+    GPTQ_CHECK_LAUNCH();
+    return GPTQ_HIP_OK;
   }
   const size_t es = a.in_dtype == GPTQ_HIP_F32 ? 4 : 2;
   const bool fast = a.m % BM == 0 && a.n % BN == 0 && a.k % BK == 0 && a.m_step == 0 &&
