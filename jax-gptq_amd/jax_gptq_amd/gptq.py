@@ -410,22 +410,28 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=
         lib = N.load()
         N.check(lib.gptq_hip_zero_dead_rows(_stream(), _ptr(H), _DT_H[H.dtype], K, _ptr(W32), Nc, Nc),
                 "zero_dead_rows")
-    else:
+    if Hinv is None:
         Hw = H.clone() if keep else H           # the factorisation rewrites the diagonal
         if actorder:
             W32, Hw, perm = _permute(W32, Hw)
         # _damp_and_invert (gptq.py:193) and the fp32 cast of the factor (gptq.py:197) in one call
         _, Hinv, status = _damp_invert(W32, Hw, damping, fix_dead=True, want_f32=True)
+    else:
+        status = None
+
+    # The column loop is enqueued before the host reads the status word back, so that the GPU
+    # does not sit idle while the host waits and then launches; with a NaN factor the loop
+    # computes garbage that is thrown away by the exception below (gptq.py:194-196).
+    Q, _ = _solve(W32, Hinv, quantize_params, block_size, orig_type)
+    if perm is not None:
+        Q = _unpermute(Q, perm)
+    if status is not None:
         any_nan = bool(status[0].item() != 0)
         if any_nan:
             xs_nan = any(bool(torch.isnan(_float_dev(x)).any()) for x in xs)
             raise ValueError(f"NaN when computing Hinv. Features NaN?: {xs_nan}")
         if shared is not None and not actorder:
             shared[factor_key] = Hinv
-
-    Q, _ = _solve(W32, Hinv, quantize_params, block_size, orig_type)
-    if perm is not None:
-        Q = _unpermute(Q, perm)
     return Q, quantize_params
 
 
