@@ -993,6 +993,12 @@ int launch_fwd_gemm(hipStream_t st, const GemmPlan &p, const void *x, int x_dtyp
 // packed fma applies zero and scale) and stores them k-contiguous, which is the operand
 // order.  Same 64 x 128 x 64 tiles, LDS layout, register ring and MFMA loop as the forward
 // kernel; zero and scale of a stage's 64 channels travel in the ring with the weights.
+//
+// bf16 activations: (code - zero) * scale rounded to bf16 would lose five of fp16's mantissa bits,
+// so the scale goes to the other operand.  A = bf16(x[m, n] * scale[n]) (rounded once, on the
+// way into LDS), B = 128 + code (one byte permute against 0x43, exact), and
+//   out[m, 2j + h] = sum_n A[m, n] * (128 + code) - t[m],  t[m] = sum_n A[m, n] * (128 + zero[n]),
+// with t[m] summed in fp32 by the staging threads from the rounded values the MFMA sees.
 template <typename TZ> struct ZsRaw;          // 16 consecutive zero / scale values as loaded
 template <> struct ZsRaw<__half> { static constexpr int NV = 2; };
 template <> struct ZsRaw<__hip_bfloat16> { static constexpr int NV = 2; };
@@ -1029,76 +1035,165 @@ __device__ __forceinline__ void zs_to_half2(const qu32x4 *v, half2_t out[8]) {
   }
 }
 
+// PV consecutive zero / scale values, loaded as PW words, as fp32
+template <typename TZ> struct ParamQuad { static constexpr int PW = sizeof(TZ) == 4 ? 4 : 2; };
 template <typename TZ>
-__global__ __launch_bounds__(256) void qmm_bwd_gemm_kernel(const __half *x, int M, const uint8_t *pk,
+__device__ __forceinline__ void quad_to_f32(const uint32_t *w, float out[4]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if constexpr (sizeof(TZ) == 4) out[i] = __builtin_bit_cast(float, w[i]);
+    else if constexpr (std::is_same<TZ, __half>::value) out[i] = (float)__builtin_bit_cast(half2_t, w[i >> 1])[i & 1];
+    else out[i] = (i & 1) ? __builtin_bit_cast(float, w[i >> 1] & 0xFFFF0000u) : __builtin_bit_cast(float, w[i >> 1] << 16);
+  }
+}
+
+template <typename TZ, typename TX>
+__global__ __launch_bounds__(256, 2) void qmm_bwd_gemm_kernel(const TX *x, int M, const uint8_t *pk,
                                                            int R, int C, const TZ *zero,
-                                                           const TZ *scale, __half *out) {
+                                                           const TZ *scale, TX *out) {
+  constexpr bool BF = Act<TX>::BF;
   constexpr int BN = 128;                       // output columns per tile = 64 packed rows
   constexpr int A_HALVES = (GBM / 16) * GGROUP;
   constexpr int B_HALVES = (BN / 16) * GGROUP;
   constexpr int TN = BN / 32;
   constexpr int NV = ZsRaw<TZ>::NV;
+  constexpr int PW = ParamQuad<TZ>::PW;
   __shared__ __attribute__((aligned(16))) _Float16 As[2][A_HALVES];
   __shared__ __attribute__((aligned(16))) _Float16 Bs[2][B_HALVES];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1, g = lane >> 4, l16 = lane & 15;
   const int j0 = blockIdx.x * (BN / 2), m0 = blockIdx.y * GBM;
 
-  // A staging: thread -> row tid/4, 16 halves at n = (tid%4)*16 of the stage
-  // B staging: thread -> packed row j0 + tid/4, the same 16 channels
+  // B staging: thread -> packed row j0 + tid/4, 16 channels at (tid%4)*16 of the stage
+  // A staging, fp16: thread -> row tid/4, the same 16 channels (whose zero and scale the thread
+  //   needs for the weights anyway)
+  // A staging, bf16: thread -> rows 4*(tid/16) .. +3, 4 channels at (tid%16)*4: the scale and the
+  //   zero point go with the activations here, and this way a thread needs 4 + 4 of them per
+  //   stage instead of 16 + 16 (fp32 parameters: 8 registers per ring slot instead of 32)
   const int s_row = tid >> 2, s_k = (tid & 3) * 16;
+  const int q_row = (tid >> 4) * 4, q_k = (tid & 15) * 4;
   const bool a_ok = (m0 + s_row) < M;
   const bool b_ok = (j0 + s_row) < R;
-  const __half *a_src = x + (int64_t)(m0 + s_row) * C + s_k;
+  const TX *a_src = x + (int64_t)(m0 + (BF ? q_row : s_row)) * C + (BF ? q_k : s_k);
   const uint8_t *b_src = pk + (int64_t)(j0 + s_row) * C + s_k;
+  float tsum[4] = {0.f, 0.f, 0.f, 0.f};     // bf16: this thread's share of t[m0 + q_row + i]
 
-  struct Stage { qu32x4 a0, a1, b; qu32x4 z[NV], s[NV]; };
+  // Activations and weights come from HBM and travel in a ring of four stages; zero and scale
+  // of a stage's channels are cache hits (a few tens of KB, read by every workgroup) and need
+  // only two stages of lead, which keeps fp32 parameters affordable.
+  struct Stage { qu32x4 a0, a1, b; };          // bf16: a0 = rows 0, 1 (2 words each), a1 = rows 2, 3
+  struct Params16 { qu32x4 z[NV], s[NV]; };
+  struct Params4 { uint32_t z[PW], s[PW]; };
+  typedef typename std::conditional<BF, Params4, Params16>::type Params;
+  typedef uint32_t qu32x2 __attribute__((ext_vector_type(2)));
   // unconditional, clamped loads (see the forward kernel); C % 16 == 0 is guaranteed
   auto load_stage = [&](int k0, Stage &st) __attribute__((always_inline)) {
     const bool in = (k0 + s_k + 16 <= C);
-    const int n = in ? k0 + s_k : 0;
-    st.a0 = *reinterpret_cast<const qu32x4 *>(a_ok && in ? a_src + k0 : x);
-    st.a1 = *reinterpret_cast<const qu32x4 *>(a_ok && in ? a_src + k0 + 8 : x);
-    st.b = *reinterpret_cast<const qu32x4 *>(b_ok && in ? b_src + k0 : pk);
+    if constexpr (BF) {
+      const bool ina = (k0 + q_k + 4 <= C);
+      qu32x2 r[4];
 #pragma unroll
-    for (int v = 0; v < NV; ++v) {
-      st.z[v] = reinterpret_cast<const qu32x4 *>(zero + n)[v];
-      st.s[v] = reinterpret_cast<const qu32x4 *>(scale + n)[v];
+      for (int i = 0; i < 4; ++i)
+        r[i] = *reinterpret_cast<const qu32x2 *>((m0 + q_row + i < M) && ina ? a_src + (int64_t)i * C + k0 : x);
+      st.a0 = qu32x4{r[0][0], r[0][1], r[1][0], r[1][1]};
+      st.a1 = qu32x4{r[2][0], r[2][1], r[3][0], r[3][1]};
+    } else {
+      st.a0 = *reinterpret_cast<const qu32x4 *>(a_ok && in ? a_src + k0 : x);
+      st.a1 = *reinterpret_cast<const qu32x4 *>(a_ok && in ? a_src + k0 + 8 : x);
     }
+    st.b = *reinterpret_cast<const qu32x4 *>(b_ok && in ? b_src + k0 : pk);
   };
-  auto store_stage = [&](int buf, int k0, const Stage &st) __attribute__((always_inline)) {
-    const qu32x4 zero4 = {0u, 0u, 0u, 0u};
-    const bool in = (k0 + s_k + 16 <= C);
-    *reinterpret_cast<qu32x4 *>(&As[buf][g_off(s_row, s_k)]) = (a_ok && in) ? st.a0 : zero4;
-    *reinterpret_cast<qu32x4 *>(&As[buf][g_off(s_row, s_k + 8)]) = (a_ok && in) ? st.a1 : zero4;
-    half2_t sc[8], nzs[8];
-    zs_to_half2<TZ, false>(st.s, sc);
-    zs_to_half2<TZ, true>(st.z, nzs);
+  auto load_params = [&](int k0, Params &zs) __attribute__((always_inline)) {
+    if constexpr (BF) {
+      const int n = (k0 + q_k + 4 <= C) ? k0 + q_k : 0;
+      typedef uint32_t vec __attribute__((ext_vector_type(PW)));
+      const vec vz = *reinterpret_cast<const vec *>(zero + n), vs = *reinterpret_cast<const vec *>(scale + n);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) nzs[i] = nzs[i] * sc[i];        // -zero * scale
-    const bool okb = b_ok && in;
-    const half2_t k1024 = half2_t{(_Float16)1024.f, (_Float16)1024.f};
-    qu32x4 lo[2], hi[2];
+      for (int v = 0; v < PW; ++v) {
+        zs.z[v] = vz[v];
+        zs.s[v] = vs[v];
+      }
+    } else {
+      const int n = (k0 + s_k + 16 <= C) ? k0 + s_k : 0;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const uint32_t w = okb ? st.b[q] : 0u;
-      const uint32_t l = w & 0x0F0F0F0Fu, h = (w >> 4) & 0x0F0F0F0Fu;
-#pragma unroll
-      for (int e = 0; e < 2; ++e) {
-        const uint32_t sel = e ? 0x04030402u : 0x04010400u;      // bytes (2e, 2e+1) -> 0x64xx pairs
-        const half2_t cl = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, l, sel)) - k1024;
-        const half2_t ch = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, h, sel)) - k1024;
-        const int i = 2 * q + e;                                   // pair index: n = s_k + 2i, 2i+1
-        const half2_t dl = okb ? cl * sc[i] + nzs[i] : half2_t{(_Float16)0.f, (_Float16)0.f};
-        const half2_t dh = okb ? ch * sc[i] + nzs[i] : half2_t{(_Float16)0.f, (_Float16)0.f};
-        lo[i >> 2][i & 3] = __builtin_bit_cast(uint32_t, dl);
-        hi[i >> 2][i & 3] = __builtin_bit_cast(uint32_t, dh);
+      for (int v = 0; v < NV; ++v) {
+        zs.z[v] = reinterpret_cast<const qu32x4 *>(zero + n)[v];
+        zs.s[v] = reinterpret_cast<const qu32x4 *>(scale + n)[v];
       }
     }
-    *reinterpret_cast<qu32x4 *>(&Bs[buf][g_off(2 * s_row, s_k)]) = lo[0];
-    *reinterpret_cast<qu32x4 *>(&Bs[buf][g_off(2 * s_row, s_k + 8)]) = lo[1];
-    *reinterpret_cast<qu32x4 *>(&Bs[buf][g_off(2 * s_row + 1, s_k)]) = hi[0];
-    *reinterpret_cast<qu32x4 *>(&Bs[buf][g_off(2 * s_row + 1, s_k + 8)]) = hi[1];
+  };
+  auto store_stage = [&](int buf, int k0, const Stage &st, const Params &zs) __attribute__((always_inline)) {
+    const qu32x4 zero4 = {0u, 0u, 0u, 0u};
+    const bool in = (k0 + s_k + 16 <= C);
+    if constexpr (BF) {
+      typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
+      float sc[4], zz[4];
+      quad_to_f32<TZ>(zs.s, sc);
+      quad_to_f32<TZ>(zs.z, zz);
+      const bool ina = (k0 + q_k + 4 <= C);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const bool ok = (m0 + q_row + i < M) && ina;
+        const qu32x4 src = i < 2 ? st.a0 : st.a1;
+        const uint32_t w0 = ok ? src[2 * (i & 1)] : 0u, w1 = ok ? src[2 * (i & 1) + 1] : 0u;
+        const bf2_t p0 = bf2_t{(__bf16)(Act<TX>::lo(w0) * sc[0]), (__bf16)(Act<TX>::hi(w0) * sc[1])};
+        const bf2_t p1 = bf2_t{(__bf16)(Act<TX>::lo(w1) * sc[2]), (__bf16)(Act<TX>::hi(w1) * sc[3])};
+        const uint32_t u0 = __builtin_bit_cast(uint32_t, p0), u1 = __builtin_bit_cast(uint32_t, p1);
+        tsum[i] += (Act<TX>::lo(u0) * (128.f + zz[0]) + Act<TX>::hi(u0) * (128.f + zz[1])) +
+                   (Act<TX>::lo(u1) * (128.f + zz[2]) + Act<TX>::hi(u1) * (128.f + zz[3]));
+        *reinterpret_cast<qu32x2 *>(&As[buf][g_off(q_row + i, q_k)]) = qu32x2{u0, u1};
+      }
+      // rows past R produce columns that are never stored, channels past C meet A = 0: any
+      // finite weight value will do there
+      qu32x4 lo[2], hi[2];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint32_t w = st.b[q];
+        const uint32_t l = w & 0x0F0F0F0Fu, h = (w >> 4) & 0x0F0F0F0Fu;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const uint32_t sel = e ? 0x04030402u : 0x04010400u;      // bytes (2e, 2e+1) -> 0x43xx pairs
+          const int i = 2 * q + e;
+          lo[i >> 2][i & 3] = __builtin_amdgcn_perm(0x43434343u, l, sel);
+          hi[i >> 2][i & 3] = __builtin_amdgcn_perm(0x43434343u, h, sel);
+        }
+      }
+      *reinterpret_cast<qu32x4 *>(&Bs[buf][g_off(2 * s_row, s_k)]) = lo[0];
+      *reinterpret_cast<qu32x4 *>(&Bs[buf][g_off(2 * s_row, s_k + 8)]) = lo[1];
+      *reinterpret_cast<qu32x4 *>(&Bs[buf][g_off(2 * s_row + 1, s_k)]) = hi[0];
+      *reinterpret_cast<qu32x4 *>(&Bs[buf][g_off(2 * s_row + 1, s_k + 8)]) = hi[1];
+    } else {
+      *reinterpret_cast<qu32x4 *>(&As[buf][g_off(s_row, s_k)]) = (a_ok && in) ? st.a0 : zero4;
+      *reinterpret_cast<qu32x4 *>(&As[buf][g_off(s_row, s_k + 8)]) = (a_ok && in) ? st.a1 : zero4;
+      half2_t sc[8], nzs[8];
+      zs_to_half2<TZ, false>(zs.s, sc);
+      zs_to_half2<TZ, true>(zs.z, nzs);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) nzs[i] = nzs[i] * sc[i];        // -zero * scale
+      const bool okb = b_ok && in;
+      const half2_t k1024 = half2_t{(_Float16)1024.f, (_Float16)1024.f};
+      qu32x4 lo[2], hi[2];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint32_t w = okb ? st.b[q] : 0u;
+        const uint32_t l = w & 0x0F0F0F0Fu, h = (w >> 4) & 0x0F0F0F0Fu;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const uint32_t sel = e ? 0x04030402u : 0x04010400u;      // bytes (2e, 2e+1) -> 0x64xx pairs
+          const half2_t cl = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, l, sel)) - k1024;
+          const half2_t ch = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, h, sel)) - k1024;
+          const int i = 2 * q + e;                                   // pair index: n = s_k + 2i, 2i+1
+          const half2_t dl = okb ? cl * sc[i] + nzs[i] : half2_t{(_Float16)0.f, (_Float16)0.f};
+          const half2_t dh = okb ? ch * sc[i] + nzs[i] : half2_t{(_Float16)0.f, (_Float16)0.f};
+          lo[i >> 2][i & 3] = __builtin_bit_cast(uint32_t, dl);
+          hi[i >> 2][i & 3] = __builtin_bit_cast(uint32_t, dh);
+        }
+      }
+      *reinterpret_cast<qu32x4 *>(&Bs[buf][g_off(2 * s_row, s_k)]) = lo[0];
+      *reinterpret_cast<qu32x4 *>(&Bs[buf][g_off(2 * s_row, s_k + 8)]) = lo[1];
+      *reinterpret_cast<qu32x4 *>(&Bs[buf][g_off(2 * s_row + 1, s_k)]) = hi[0];
+      *reinterpret_cast<qu32x4 *>(&Bs[buf][g_off(2 * s_row + 1, s_k + 8)]) = hi[1];
+    }
   };
 
   floatx4 acc[2][TN];
@@ -1108,48 +1203,65 @@ __global__ __launch_bounds__(256) void qmm_bwd_gemm_kernel(const __half *x, int 
     for (int j = 0; j < TN; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   Stage s0, s1, s2, s3;
+  Params q0, q1;
+  load_params(0, q0);
+  load_params(GBK, q1);
   load_stage(0, s0);
   load_stage(GBK, s1);
   load_stage(2 * GBK, s2);
   load_stage(3 * GBK, s3);
   int buf = 0;
-  store_stage(0, 0, s0);
+  store_stage(0, 0, s0, q0);
+  load_params(2 * GBK, q0);
   __syncthreads();
-  auto step = [&](int k0, Stage &refill, const Stage &next, bool do_load, bool has_next)
+  // multiplies the stage at k0 out of LDS, writes the next one (whose parameters are in zs) and
+  // reloads zs for the stage that is written two steps from now
+  auto step = [&](int k0, Stage &refill, const Stage &next, Params &zs, bool do_load, bool has_next)
                   __attribute__((always_inline)) {
     if (do_load) load_stage(k0 + 4 * GBK, refill);
 #pragma unroll
     for (int ks = 0; ks < GBK; ks += 32) {
-      half8_t a[2], b[TN];
+      uint4 a[2], b[TN];
 #pragma unroll
       for (int i = 0; i < 2; ++i)
-        a[i] = *reinterpret_cast<const half8_t *>(&As[buf][g_off(wm * 32 + i * 16 + l16, ks + 8 * g)]);
+        a[i] = *reinterpret_cast<const uint4 *>(&As[buf][g_off(wm * 32 + i * 16 + l16, ks + 8 * g)]);
 #pragma unroll
       for (int j = 0; j < TN; ++j)
-        b[j] = *reinterpret_cast<const half8_t *>(
+        b[j] = *reinterpret_cast<const uint4 *>(
             &Bs[buf][g_off(wn * (BN / 2) + j * 16 + l16, ks + 8 * g)]);
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < TN; ++j) acc[i][j] = Act<TX>::mma(a[i], b[j], acc[i][j]);
     }
-    if (has_next) store_stage(buf ^ 1, k0 + GBK, next);
+    if (has_next) store_stage(buf ^ 1, k0 + GBK, next, zs);
+    if (do_load) load_params(k0 + 3 * GBK, zs);
     __syncthreads();
     buf ^= 1;
   };
   // (the exit-free form of the forward kernel was measured 4 % slower here)
-  auto stepx = [&](int k0, Stage &refill, const Stage &next) __attribute__((always_inline)) {
+  auto stepx = [&](int k0, Stage &refill, const Stage &next, Params &zs) __attribute__((always_inline)) {
     if (k0 >= C) return;
-    step(k0, refill, next, true, k0 + GBK < C);
+    step(k0, refill, next, zs, true, k0 + GBK < C);
   };
   for (int kb = 0; kb < C; kb += 4 * GBK) {
-    stepx(kb, s0, s1);
-    stepx(kb + GBK, s1, s2);
-    stepx(kb + 2 * GBK, s2, s3);
-    stepx(kb + 3 * GBK, s3, s0);
+    stepx(kb, s0, s1, q1);
+    stepx(kb + GBK, s1, s2, q0);
+    stepx(kb + 2 * GBK, s2, s3, q1);
+    stepx(kb + 3 * GBK, s3, s0, q0);
   }
 
+  __shared__ float trow[GBM];
+  if constexpr (BF) {     // t[m]: the sixteen staging threads of a row are neighbouring lanes
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float v = tsum[i];
+#pragma unroll
+      for (int off = 1; off < 16; off <<= 1) v += __shfl_xor(v, off);
+      if ((tid & 15) == 0) trow[q_row + i] = v;
+    }
+    __syncthreads();
+  }
   // acc[i][j][r] = out[m0 + wm*32 + i*16 + 4g + r][2*j0 + wn*64 + j*16 + l16]
   const int KO = 2 * R;
 #pragma unroll
@@ -1160,27 +1272,34 @@ __global__ __launch_bounds__(256) void qmm_bwd_gemm_kernel(const __half *x, int 
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int m = m0 + wm * 32 + i * 16 + 4 * g + r;
-        if (m < M) out[(int64_t)m * KO + c] = __float2half_rn(acc[i][j][r]);
+        const int ml = wm * 32 + i * 16 + 4 * g + r;
+        const float v = BF ? acc[i][j][r] - trow[ml] : acc[i][j][r];
+        if (m0 + ml < M) out[(int64_t)(m0 + ml) * KO + c] = Act<TX>::out(v);
       }
   }
 }
 
 template <typename TZ>
-int launch_bwd_gemm(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
-                    const void *zero, const void *scale, void *out) {
+int launch_bwd_gemm(hipStream_t st, const void *x, int x_dtype, int64_t M, const uint8_t *pk, int64_t R,
+                    int64_t C, const void *zero, const void *scale, void *out) {
   const int64_t mt = ceil_div64(M, GBM);
   if (mt > 65535) return GPTQ_HIP_EINVAL;
-  hipLaunchKernelGGL((qmm_bwd_gemm_kernel<TZ>), dim3((unsigned)ceil_div64(R, 64), (unsigned)mt),
-                     dim3(256), 0, st, (const __half *)x, (int)M, pk, (int)R, (int)C,
-                     (const TZ *)zero, (const TZ *)scale, (__half *)out);
+  const dim3 grid((unsigned)ceil_div64(R, 64), (unsigned)mt);
+  if (x_dtype == GPTQ_HIP_BF16)
+    hipLaunchKernelGGL((qmm_bwd_gemm_kernel<TZ, __hip_bfloat16>), grid, dim3(256), 0, st,
+                       (const __hip_bfloat16 *)x, (int)M, pk, (int)R, (int)C, (const TZ *)zero,
+                       (const TZ *)scale, (__hip_bfloat16 *)out);
+  else
+    hipLaunchKernelGGL((qmm_bwd_gemm_kernel<TZ, __half>), grid, dim3(256), 0, st, (const __half *)x,
+                       (int)M, pk, (int)R, (int)C, (const TZ *)zero, (const TZ *)scale, (__half *)out);
   GPTQ_CHECK_LAUNCH();
   return GPTQ_HIP_OK;
 }
 
 bool bwd_fast_ok(int x_dtype, int64_t M, int64_t R, int64_t C, const void *x, const uint8_t *pk,
                  const void *zero, const void *scale) {
-  return x_dtype == GPTQ_HIP_F16 && C % 16 == 0 && M >= 1 && R < (1LL << 30) && C < (1LL << 30) &&
+  return (x_dtype == GPTQ_HIP_F16 || x_dtype == GPTQ_HIP_BF16) && C % 16 == 0 && M >= 1 &&
+         R < (1LL << 30) && C < (1LL << 30) &&
          ((reinterpret_cast<uintptr_t>(pk) | reinterpret_cast<uintptr_t>(x) |
            reinterpret_cast<uintptr_t>(zero) | reinterpret_cast<uintptr_t>(scale)) & 15) == 0;
 }
@@ -1260,10 +1379,10 @@ int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const 
   }
   if (transpose_b && bwd_fast_ok(x_dtype, M, R, C, x, packed, zero, scale)) {
     switch (zs_dtype) {
-      case GPTQ_HIP_F32: return launch_bwd_gemm<float>(st, x, M, packed, R, C, zero, scale, out);
-      case GPTQ_HIP_F16: return launch_bwd_gemm<__half>(st, x, M, packed, R, C, zero, scale, out);
+      case GPTQ_HIP_F32: return launch_bwd_gemm<float>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
+      case GPTQ_HIP_F16: return launch_bwd_gemm<__half>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
       case GPTQ_HIP_BF16:
-        return launch_bwd_gemm<__hip_bfloat16>(st, x, M, packed, R, C, zero, scale, out);
+        return launch_bwd_gemm<__hip_bfloat16>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
       default: return GPTQ_HIP_EDTYPE;
     }
   }

@@ -123,6 +123,36 @@ def test_qmatmul_bf16_x_mfma_path(OP, M, N, K, zs):
     assert np.all(err <= 1e-2 + 2.0 ** -8 * np.abs(ref)), err.max()
 
 
+@pytest.mark.parametrize("zs", ["float32", "float16", "bfloat16"])
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 11008), (16, 11008, 4096), (128, 4096, 1024), (70, 2304, 768),
+                                   (5, 48, 96), (200, 5120, 256), (300, 1008, 514), (2048, 4096, 512)])
+def test_qmatmul_bf16_x_transposed_mfma_path(OP, M, N, K, zs):
+    """Transposed product with bf16 activations: the scale multiplies the activations (rounded
+    once to bf16, which is their own precision), the weights enter as 128 + code, and the term in
+    128 + zero leaves through fp32 row sums; the result is rounded once, to bf16."""
+    import torch
+    import jax_gptq_amd.gptq as G
+    rng = np.random.default_rng(M + N + K)
+    codes = rng.integers(0, 16, (K, N)).astype(np.uint8)
+    tdt = getattr(torch, zs)
+    scale = torch.from_numpy(rng.uniform(0.001, 0.01, N).astype(np.float32)).to(tdt)
+    zero = torch.from_numpy(rng.uniform(0.0, 15.0, N).astype(np.float32)).to(tdt)      # fractional, too
+    qm = G.QuantizedMatrix(torch.from_numpy(O.pack_colwise(codes)).cuda(), zero.cuda(), scale.cuda())
+    x = torch.from_numpy((0.05 * rng.standard_normal((M, N))).astype(np.float32)).to(torch.bfloat16)
+    got = OP.quantized_matmul(x, qm, transpose_b=True)
+    assert got.dtype == torch.bfloat16 and tuple(got.shape) == (M, K)
+    dense = (codes.astype(np.float64) - zero.double().numpy()[None]) * scale.double().numpy()[None]
+    ref = x.double().numpy() @ dense.T
+    err = np.abs(to_np(got).astype(np.float64) - ref)
+    # rounding of x * scale to bf16 (2^-9 per term, random signs) and of the result (2^-9)
+    assert np.all(err <= 1e-2 + 2.0 ** -8 * np.abs(ref)), err.max()
+    # the fp16 kernel on the same values (exactly representable: bf16 -> fp16 of |x| < 1 loses nothing
+    # above 2^-14) agrees to the bf16 rounding of the result
+    got16 = OP.quantized_matmul(x.to(torch.float16), qm, transpose_b=True)
+    d = np.abs(to_np(got).astype(np.float64) - to_np(got16).astype(np.float64))
+    assert np.all(d <= 1e-2 + 2.0 ** -7 * np.abs(ref)), d.max()
+
+
 @pytest.mark.parametrize("M,N,K,xdt,zs", [(1, 28672, 7168, "float16", "float16"),
                                             (16, 7168, 28672, "float16", "float32"),
                                             (3, 29936, 9000, "float16", "float32"),
