@@ -161,10 +161,16 @@ int gptq_hip_dequant(void *stream, const uint8_t *packed, int64_t outer,
  *   transpose_b = 1: Kx = C,  out [M, 2R] = x @ ((code - zero) * scale)^T
  * fp32 accumulation; the result is rounded to fp16 and then converted to x_dtype, as
  * op.py:43,66-68 does.  ws: gptq_hip_qmatmul_workspace_bytes(M, R, C, transpose_b) bytes.
+ * fp32 activations (the reference's dot rounds them to TF32, kernel.py:106): with a workspace of
+ * gptq_hip_qmatmul_workspace_bytes_x(..., GPTQ_HIP_F32) bytes and C % 16 == 0 they are rounded
+ * to fp16 precision (after a per-row power-of-two scaling that keeps any fp32 magnitude in
+ * range; the result is scaled back after its rounding to fp16) and run on the same matrix-core kernels as fp16 ones; with the smaller workspace, or
+ * other shapes, they run unrounded on plain kernels that are an order of magnitude slower.
  * The workspace begins with arrival counters of the split-K reduction: it must be
  * ZERO-FILLED before its first use; every call leaves the counters zero again, so one
  * buffer can serve any sequence of calls that do not overlap in time. */
 size_t gptq_hip_qmatmul_workspace_bytes(int64_t M, int64_t R, int64_t C, int transpose_b);
+size_t gptq_hip_qmatmul_workspace_bytes_x(int64_t M, int64_t R, int64_t C, int transpose_b, int x_dtype);
 int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
                      int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype,
                      int transpose_b, void *out, void *ws, size_t ws_bytes);

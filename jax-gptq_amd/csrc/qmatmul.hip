@@ -1342,6 +1342,83 @@ int dispatch_z(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int6
   }
 }
 
+// ---------------------------------------------------------------------------- fp32 activations
+// The 16-bit MFMA kernels serve fp32 activations through two small passes around them: every row
+// of x is scaled by the power of two that brings its largest finite magnitude into [2, 4) and
+// rounded to fp16, the product runs on the fp16 kernels, and the fp16 result is widened and scaled
+// back (powers of two: exact), so rows of any fp32 magnitude keep fp16's relative precision in
+// operand and result.  The reference's dot rounds fp32 operands to TF32 (tl.dot at kernel.py:106
+// with Triton's default), which has fp16's mantissa width, and its result is rounded to fp16 as
+// well (op.py:43).  Rows are processed in chunks so that the staging buffers stay bounded for any M.
+constexpr int64_t F32_CHUNK_ROWS = 8192;
+
+__global__ __launch_bounds__(256) void x32_to_f16_rows_kernel(const float *x, int64_t kin, __half *x16,
+                                                              int32_t *rowexp) {
+  const int64_t m = blockIdx.x;
+  const float *xr = x + m * kin;
+  __half *dst = x16 + m * kin;
+  __shared__ float smax[4];
+  float amax = 0.f;
+  for (int64_t k = threadIdx.x; k < kin; k += 256) {
+    const float a = fabsf(xr[k]);
+    amax = (a <= 3.4028235e38f && a > amax) ? a : amax;   // NaN and infinity do not set the scale
+  }
+  for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+  if ((threadIdx.x & 63) == 0) smax[threadIdx.x >> 6] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3]));
+  int ex = 0;
+  (void)frexpf(amax, &ex);                    // 2^(ex-1) <= amax < 2^ex
+  const int e = amax > 0.f ? ex - 2 : 0;      // largest magnitude of the scaled row in [2, 4)
+  for (int64_t k = threadIdx.x; k < kin; k += 256) dst[k] = __float2half_rn(ldexpf(xr[k], -e));
+  if (threadIdx.x == 0) rowexp[m] = e;
+}
+
+__global__ __launch_bounds__(256) void f16_rows_to_f32_kernel(const __half *o16, int64_t nout,
+                                                              const int32_t *rowexp, float *out) {
+  const int64_t m = blockIdx.y;
+  const int e = rowexp[m];
+  for (int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x; n < nout; n += (int64_t)gridDim.x * 256)
+    out[m * nout + n] = ldexpf(__half2float(o16[m * nout + n]), e);
+}
+
+struct F32Plan {
+  bool use;
+  int64_t mc;                 // rows per chunk
+  size_t inner;               // workspace of the fp16 product of one chunk (at offset 0: its counters)
+  size_t x16_off, o16_off, exp_off, total_bytes;
+};
+
+size_t round_up_256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+}  // namespace
+
+extern "C" size_t gptq_hip_qmatmul_workspace_bytes(int64_t M, int64_t R, int64_t C, int transpose_b);
+
+namespace {
+
+F32Plan f32_plan(int64_t M, int64_t R, int64_t C, int transpose_b) {
+  F32Plan p{};
+  p.use = M >= 1 && C % 16 == 0 && R < (1LL << 30) && C < (1LL << 30);
+  if (!p.use) return p;
+  p.mc = M < F32_CHUNK_ROWS ? M : F32_CHUNK_ROWS;
+  const int64_t tail = M % p.mc;
+  size_t inner = gptq_hip_qmatmul_workspace_bytes(p.mc, R, C, transpose_b);
+  if (tail) {
+    const size_t t = gptq_hip_qmatmul_workspace_bytes(tail, R, C, transpose_b);
+    inner = t > inner ? t : inner;
+  }
+  const int64_t kin = transpose_b ? C : 2 * R, nout = transpose_b ? 2 * R : C;
+  p.inner = inner;
+  // the counter region stays out of reach of the staging buffers whatever this call's own product
+  // needs: a later call on the same workspace expects its counters to be zero
+  p.x16_off = round_up_256(inner > (size_t)QMM_COUNTER_BYTES ? inner : (size_t)QMM_COUNTER_BYTES);
+  p.o16_off = p.x16_off + round_up_256((size_t)p.mc * kin * sizeof(__half));
+  p.exp_off = p.o16_off + round_up_256((size_t)p.mc * nout * sizeof(__half));
+  p.total_bytes = p.exp_off + round_up_256((size_t)p.mc * sizeof(int32_t));
+  return p;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1354,6 +1431,15 @@ size_t gptq_hip_qmatmul_workspace_bytes(int64_t M, int64_t R, int64_t C, int tra
   return a > b ? (a > c ? a : c) : (b > c ? b : c);
 }
 
+size_t gptq_hip_qmatmul_workspace_bytes_x(int64_t M, int64_t R, int64_t C, int transpose_b, int x_dtype) {
+  if (M <= 0 || R <= 0 || C <= 0) return 0;
+  if (x_dtype == GPTQ_HIP_F32) {
+    const F32Plan fp = f32_plan(M, R, C, transpose_b);
+    if (fp.use) return fp.total_bytes;
+  }
+  return gptq_hip_qmatmul_workspace_bytes(M, R, C, transpose_b);
+}
+
 int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
                      int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype,
                      int transpose_b, void *out, void *ws, size_t ws_bytes) {
@@ -1361,6 +1447,35 @@ int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const 
   if (M == 0) return GPTQ_HIP_OK;
   if (!x || !packed || !zero || !scale || !out) return GPTQ_HIP_EINVAL;
   hipStream_t st = as_stream(stream);
+  if (x_dtype == GPTQ_HIP_F32) {
+    // through the fp16 kernels, if the shape suits them and the caller sized the workspace for
+    // it (gptq_hip_qmatmul_workspace_bytes_x); else the plain fp32 kernels below
+    const F32Plan fp = f32_plan(M, R, C, transpose_b);
+    const uintptr_t align = reinterpret_cast<uintptr_t>(packed) | reinterpret_cast<uintptr_t>(zero) |
+                            reinterpret_cast<uintptr_t>(scale) | reinterpret_cast<uintptr_t>(ws);
+    if (fp.use && ws && ws_bytes >= fp.total_bytes && (align & 15) == 0) {
+      char *base = reinterpret_cast<char *>(ws);
+      __half *x16 = reinterpret_cast<__half *>(base + fp.x16_off);
+      __half *o16 = reinterpret_cast<__half *>(base + fp.o16_off);
+      int32_t *rowexp = reinterpret_cast<int32_t *>(base + fp.exp_off);
+      const int64_t kin = transpose_b ? C : 2 * R, nout = transpose_b ? 2 * R : C;
+      for (int64_t r0 = 0; r0 < M; r0 += fp.mc) {
+        const int64_t mm = M - r0 < fp.mc ? M - r0 : fp.mc;
+        hipLaunchKernelGGL(x32_to_f16_rows_kernel, dim3((unsigned)mm), dim3(256), 0, st,
+                           reinterpret_cast<const float *>(x) + r0 * kin, kin, x16, rowexp);
+        GPTQ_CHECK_LAUNCH();
+        const int rc = gptq_hip_qmatmul(stream, x16, GPTQ_HIP_F16, mm, packed, R, C, zero, scale, zs_dtype,
+                                        transpose_b, o16, ws, fp.inner);
+        if (rc) return rc;
+        unsigned gx = (unsigned)ceil_div64(nout, 1024);
+        if (gx > 64) gx = 64;
+        hipLaunchKernelGGL(f16_rows_to_f32_kernel, dim3(gx, (unsigned)mm), dim3(256), 0, st, o16, nout,
+                           rowexp, reinterpret_cast<float *>(out) + r0 * nout);
+        GPTQ_CHECK_LAUNCH();
+      }
+      return GPTQ_HIP_OK;
+    }
+  }
   // GEMM-shaped work goes to the tiled kernel (split-K when the output tiles alone do not fill
   // the chip); small M goes through the 16-row chunked kernel.
   const GemmPlan gp = gemm_plan(M, R, C);

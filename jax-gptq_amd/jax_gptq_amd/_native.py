@@ -39,6 +39,7 @@ SIGNATURES = {
     "gptq_hip_quantize_pack": (_i32, [_vp, _vp, _i32, _i64, _i64, _i64, _vp, _vp, _vp]),
     "gptq_hip_dequant": (_i32, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i32, _vp]),
     "gptq_hip_qmatmul_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
+    "gptq_hip_qmatmul_workspace_bytes_x": (_sz, [_i64, _i64, _i64, _i32, _i32]),
     "gptq_hip_qmatmul": (_i32, [_vp, _vp, _i32, _i64, _vp, _i64, _i64, _vp, _vp, _i32, _i32, _vp, _vp, _sz]),
 }
 

@@ -50,7 +50,7 @@ def _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b):
     if zero.dtype != scale.dtype:
         scale = scale.to(zero.dtype)
     out = torch.empty((M, out_n), dtype=x.dtype, device=x.device)
-    ws = _qmm_workspace(lib.gptq_hip_qmatmul_workspace_bytes(M, R, C, int(transpose_b)), x.device)
+    ws = _qmm_workspace(lib.gptq_hip_qmatmul_workspace_bytes_x(M, R, C, int(transpose_b), _DT[x.dtype]), x.device)
     N.check(lib.gptq_hip_qmatmul(_stream(), _ptr(x), _DT[x.dtype], M, _ptr(int_weight), R, C,
                                  _ptr(zero), _ptr(scale), _DT[zero.dtype], int(transpose_b),
                                  _ptr(out), _ptr(ws), ws.numel()), "qmatmul")

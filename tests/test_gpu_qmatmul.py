@@ -69,6 +69,51 @@ def test_qmatmul_fp32_x_and_params(OP, M, N, K, transpose):
 
 
 @pytest.mark.parametrize("transpose", [False, True])
+@pytest.mark.parametrize("M,N,K", [(1, 11008, 4096), (16, 4096, 11008), (200, 5120, 256), (2048, 4096, 1024),
+                                   (9000, 256, 128)])
+def test_qmatmul_fp32_x_on_the_matrix_core_kernels(OP, M, N, K, transpose):
+    """fp32 activations with C % 16 == 0 are rounded to fp16 precision (the reference's dot rounds
+    them to TF32: same mantissa width) after a per-row power-of-two scaling and run on the fp16
+    kernels.  Rows of very different magnitude (1e-20 to 1e20, far outside fp16) check the scaling;
+    M = 9000 spans two row chunks.  With the workspace of the 16-bit query the same call stays on the
+    unrounded kernels."""
+    import torch
+    import jax_gptq_amd._native as NV
+    qm = _matrix(M + N + K, K, N, np.float32)
+    rng = np.random.default_rng(11)
+    rowscale = np.array([1.0, 1e-3, 3e4, 1e20, 1e-20])[np.arange(M) % 5][:, None]
+    x = (rng.standard_normal((M, N if transpose else K)) * (0.05 if transpose else 1.0) * rowscale).astype(np.float32)
+    got = to_np(OP.quantized_matmul(x, qm, transpose_b=transpose)).astype(np.float64)
+    assert got.dtype == np.float64 and to_np(OP.quantized_matmul(x, qm, transpose_b=transpose)).dtype == np.float32
+    dense = ((O.unpack_colwise(qm.int_weight).astype(np.float64) - qm.zero.astype(np.float64)[None])
+             * qm.scale.astype(np.float64)[None])
+    ref = x.astype(np.float64) @ (dense.T if transpose else dense)
+    tol = (ATOL + RTOL * np.abs(ref / rowscale)) * rowscale       # relative to the row's magnitude
+    err = np.abs(got - ref)
+    assert np.all(err <= tol), float((err / tol).max())
+    if M > 200:
+        return
+    # the same call with the smaller workspace: plain kernels, fp32 activations unrounded
+    lib = NV.load()
+    xt = torch.from_numpy(x).cuda()
+    pk = torch.from_numpy(np.ascontiguousarray(qm.int_weight)).cuda()
+    zero, scale = torch.from_numpy(qm.zero).cuda(), torch.from_numpy(qm.scale).cuda()
+    R, C = pk.shape
+    out = torch.empty((M, 2 * R if transpose else C), dtype=torch.float32, device="cuda")
+    nb = lib.gptq_hip_qmatmul_workspace_bytes(M, R, C, int(transpose))
+    assert nb < lib.gptq_hip_qmatmul_workspace_bytes_x(M, R, C, int(transpose), 0)
+    ws = torch.zeros(max(nb, 256), dtype=torch.uint8, device="cuda")
+    rc = lib.gptq_hip_qmatmul(OP._stream(), xt.data_ptr(), 0, M, pk.data_ptr(), R, C, zero.data_ptr(), scale.data_ptr(),
+                              0, int(transpose), out.data_ptr(), ws.data_ptr(), nb)
+    assert rc == 0
+    torch.cuda.synchronize()
+    # (rows whose results leave the fp16 range become infinite there, as in the reference: op.py:43)
+    small = (rowscale <= 1.0)[:, 0]
+    err = np.abs(out.cpu().numpy().astype(np.float64) - ref)[small]
+    assert np.all(err <= 1e-4 + 2.0 ** -10 * np.abs(ref[small]))
+
+
+@pytest.mark.parametrize("transpose", [False, True])
 @pytest.mark.parametrize("zs", ["float32", "float16", "bfloat16"])
 @pytest.mark.parametrize("M", [1, 16, 200])
 def test_qmatmul_fractional_zero_points_and_param_dtypes(OP, M, zs, transpose):
