@@ -15,6 +15,7 @@ Prints ONE JSON line.  Besides the contract keys it carries
   cpu_baseline   the NumPy/SciPy oracle timed on this host on a bounded sample,
   phases_ms      per-phase GPU time of one step,
   fp16_calibration  the same layer with the calibration rows stored in fp16,
+  fp32_rows_split_fp16  the fp32 rows multiplied as pairs of fp16 numbers (opt-in path),
   qmatmul        packed-int4 matmul at M = 1, 16, 128 against the HBM roofline
                  (weights rotated over > 512 MB of copies so that they come from HBM).
 """
@@ -51,7 +52,7 @@ def make_inputs(k_in, n_out, n_batch, rows, x_dtype):
     return W, xs
 
 
-def one_layer(G, W, xs, timers=None):
+def one_layer(G, W, xs, timers=None, split_fp16=False):
     """The hot path, phase by phase (same calls as jax_gptq_amd.gptq.gptq + pack_matrix)."""
     import torch
     ev = _events(6) if timers is not None else None
@@ -64,7 +65,7 @@ def one_layer(G, W, xs, timers=None):
     W32 = W.to(torch.float32)
     params = G.get_col_quantize_params(W32)
     mark(1)
-    H = G.accumulate_H(xs)
+    H = G.accumulate_H(xs, split_fp16=split_fp16)
     mark(2)
     W32, L, any_nan = G._damp_and_invert(W32, H, 0.01)     # reads one status word (host sync)
     mark(3)
@@ -186,6 +187,8 @@ def main():
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--x-dtype", default="float32", choices=["float32", "float16", "bfloat16"])
+    ap.add_argument("--split-fp16", action="store_true",
+                    help="--section hessian only: fp32 rows as pairs of fp16 numbers (accumulate_H(split_fp16=True))")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-qmatmul", action="store_true", help="skip the int4 matmul section")
     ap.add_argument("--section", default="all", choices=["all", "hessian", "qmatmul", "copy"],
@@ -217,11 +220,11 @@ def main():
     W, xs = make_inputs(K_IN, N_OUT, N_BATCH, ROWS, getattr(torch, args.x_dtype))
     torch.cuda.synchronize()
     if args.section == "hessian":
-        G.accumulate_H(xs)
+        G.accumulate_H(xs, split_fp16=args.split_fp16)
         e0, e1 = _events(2)
         e0.record()
         for _ in range(max(1, args.steps)):
-            G.accumulate_H(xs)
+            G.accumulate_H(xs, split_fp16=args.split_fp16)
         e1.record()
         torch.cuda.synchronize()
         ms = e0.elapsed_time(e1) / max(1, args.steps)
@@ -296,6 +299,19 @@ def main():
         result["fp16_calibration"] = {"ms_per_layer": round(sum(ph16.values()), 3), "phases_ms": ph16,
                                       "xtx_tflops": round(flop_per_launch / (ph16["hessian"] * 1e-3) * 1e-12, 2)}
         del xs16
+        # the fp32 rows again, multiplied as pairs of fp16 numbers on the 16-bit matrix cores (opt-in:
+        # accumulate_H(..., split_fp16=True)); codes_equal compares the packed result with the one above
+        ref_packed = one_layer(G, W, xs)
+        got_packed = one_layer(G, W, xs, split_fp16=True)
+        ts = {}
+        for _ in range(max(1, args.steps)):
+            one_layer(G, W, xs, ts, split_fp16=True)
+        phs = {k: round(sum(v) / len(v), 3) for k, v in ts.items()}
+        rb, gb = ref_packed.int_weight, got_packed.int_weight
+        same = ((rb & 15) == (gb & 15)).sum() + ((rb >> 4) == (gb >> 4)).sum()
+        result["fp32_rows_split_fp16"] = {"ms_per_layer": round(sum(phs.values()), 3), "phases_ms": phs,
+                                          "xtx_tflops": round(flop_per_launch / (phs["hessian"] * 1e-3) * 1e-12, 2),
+                                          "codes_equal": round(float(same) / (2 * rb.numel()), 6)}
     if not args.no_qmatmul:
         qm = bench_qmatmul()
         result["qmatmul"] = qm

@@ -26,6 +26,7 @@ constexpr int H_NBMAX = 128;   // batches per launch (pointer table lives in the
 constexpr int H_RSMAX = 16;
 
 struct SyrkArgs {
+  static constexpr bool DUAL = false;
   const void *ptr[H_NBMAX];
   int rows[H_NBMAX];
   int nb;
@@ -35,6 +36,15 @@ struct SyrkArgs {
   int chunk;   // 16-bit kernel: rows of the concatenated batches per slice (multiple of 64)
   float *H;
   float *ws;   // [RS][tiles][128][128] when RS > 1
+};
+
+// Two-matrix form of the 16-bit kernel: sum_b A_b^T B_b for batch pairs whose sum is symmetric
+// (operand A of a tile comes from ptr[b], operand B from ptrB[b]).
+struct SyrkArgsDual : SyrkArgs {
+  static constexpr bool DUAL = true;
+  const void *ptrB[H_NBMAX];
+  const float *factor;   // device scalar: the sums are in units of 1 / factor
+  int accum;             // partial tiles: add to what the workspace holds instead of overwriting
 };
 
 // upper-triangular pair number t -> (i <= j), column by column
@@ -736,8 +746,8 @@ __device__ __forceinline__ void load_to_lds_16(const void *src, uint32_t dst) {
                : "memory", "m0");
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void syrk16d_kernel(SyrkArgs p) {
+template <typename T, typename ARGS>
+__global__ __launch_bounds__(256) void syrk16d_kernel(ARGS p) {
   extern __shared__ __attribute__((aligned(16))) char lds16d[];
   typedef typename Mfma16<T>::v8 v8;
   typedef short s4 __attribute__((ext_vector_type(4)));
@@ -791,7 +801,11 @@ __global__ __launch_bounds__(256) void syrk16d_kernel(SyrkArgs p) {
   const int ld_feat = (ld_op ? n0 : m0) + l32 * 8;
   const uint32_t ld_dst0 = lds0 + ld_op * D16_OP + ld_pair0 * D16_PAIR;
   // position of the next slab to load: batch b (base pointer Xb, rows_b rows), row kt
-  const uint16_t *Xb = reinterpret_cast<const uint16_t *>(p.ptr[b]);
+  auto batch_ptr = [&](int bb) __attribute__((always_inline)) -> const uint16_t * {
+    if constexpr (ARGS::DUAL) return reinterpret_cast<const uint16_t *>(ld_op ? p.ptrB[bb] : p.ptr[bb]);
+    else return reinterpret_cast<const uint16_t *>(p.ptr[bb]);
+  };
+  const uint16_t *Xb = batch_ptr(b);
   int rows_b = p.rows[b];
   int issued = 0;
   // source of this lane for the 8 loads of the next slab, LDS target of the first of them; then advance
@@ -803,7 +817,7 @@ __global__ __launch_bounds__(256) void syrk16d_kernel(SyrkArgs p) {
     if (kt >= rows_b && issued < nslabs) {      // rare: next batch
       ++b;
       kt = 0;
-      Xb = reinterpret_cast<const uint16_t *>(p.ptr[b]);
+      Xb = batch_ptr(b);
       rows_b = p.rows[b];
     }
   };
@@ -933,6 +947,12 @@ __global__ __launch_bounds__(256) void syrk16d_kernel(SyrkArgs p) {
     for (int ii = 0; ii < 4; ++ii) group(prev.a[ii], prev.b, ii);
   }
 
+  float unit = 1.f;
+  bool accum = false;
+  if constexpr (ARGS::DUAL) {
+    unit = *p.factor;
+    accum = p.accum != 0;
+  }
   if (p.RS == 1) {
 #pragma unroll
     for (int ii = 0; ii < 4; ++ii)
@@ -942,7 +962,7 @@ __global__ __launch_bounds__(256) void syrk16d_kernel(SyrkArgs p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int row = m0 + wm * 128 + ii * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-          p.H[(int64_t)row * K + col] += acc[ii][j][r];
+          p.H[(int64_t)row * K + col] += ARGS::DUAL ? acc[ii][j][r] * unit : acc[ii][j][r];
         }
       }
   } else {
@@ -955,16 +975,18 @@ __global__ __launch_bounds__(256) void syrk16d_kernel(SyrkArgs p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int row = wm * 128 + ii * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-          dst[row * W16_TB + col] = acc[ii][j][r];
+          if (ARGS::DUAL && accum) dst[row * W16_TB + col] += acc[ii][j][r];
+          else dst[row * W16_TB + col] = acc[ii][j][r];
         }
       }
   }
 }
 
-// H tile += sum over the row slices, in slice order
+// H tile += unit * sum over the row slices, in slice order (unit: device scalar, 1 if null)
 template <int TB>
 __global__ __launch_bounds__(256) void syrk_reduce_kernel(float *H, const float *ws, int K, int T,
-                                                          int RS) {
+                                                          int RS, const float *unit_ptr) {
+  const float unit = unit_ptr ? *unit_ptr : 1.f;
   const int ntiles = T * (T + 1) / 2;
   const int t = blockIdx.x;
   int ti, tj;
@@ -981,10 +1003,10 @@ __global__ __launch_bounds__(256) void syrk_reduce_kernel(float *H, const float 
     const int gr = m0 + row, gc = n0 + c4;
     if (gr >= K) continue;
     float *dst = H + (int64_t)gr * K + gc;
-    if (gc + 0 < K) dst[0] += s.x;
-    if (gc + 1 < K) dst[1] += s.y;
-    if (gc + 2 < K) dst[2] += s.z;
-    if (gc + 3 < K) dst[3] += s.w;
+    if (gc + 0 < K) dst[0] += s.x * unit;
+    if (gc + 1 < K) dst[1] += s.y * unit;
+    if (gc + 2 < K) dst[2] += s.z * unit;
+    if (gc + 3 < K) dst[3] += s.w * unit;
   }
 }
 
@@ -1012,6 +1034,101 @@ int pick_rs_wide(int64_t K) {
   return best;
 }
 bool use_wide16(int64_t K) { return K >= 1024; }
+
+// ---------------------------------------------------------------------------- fp32 rows on the 16-bit matrix cores
+// Opt-in path for fp32 calibration rows: x = (hi + lo) * 2^e with hi = fp16(x 2^-e), lo =
+// fp16(x 2^-e - hi), e chosen so that the largest magnitude of the call lands in [2^14, 2^15).
+// hi + lo carries 22 mantissa bits of x (fewer only for entries more than 2^18 below the largest),
+// all products of two fp16 numbers are exact in the fp32 accumulators, and
+//   X^T X = 4^e (hi^T hi + hi^T lo + lo^T hi)  up to lo^T lo (relative 2^-22 per product).
+// The three products are one launch of the two-matrix 16-bit kernel over the batch pairs
+// (hi, hi), (hi, lo), (lo, hi): three times the 16-bit work instead of fp32 MFMAs at a
+// sixteenth of the rate.  Steps: largest magnitude of all batches (one read of X), then per
+// group of batches split into two fp16 planes (workspace), multiply, and at the end one reduction
+// that applies 4^e.  No host synchronisation: e lives in device memory.
+struct SplitScalars { uint32_t amax_bits; float down, unit; };
+
+__global__ void split_reset_kernel(SplitScalars *sc) {
+  sc->amax_bits = 0u;
+  sc->down = 1.f;
+  sc->unit = 1.f;
+}
+
+// largest finite |x| over the batches of the table (grid: blocks x batches)
+__global__ __launch_bounds__(256) void split_absmax_kernel(SyrkArgs p, SplitScalars *sc) {
+  const int b = blockIdx.y;
+  const float4 *x = reinterpret_cast<const float4 *>(p.ptr[b]);
+  const int64_t n4 = (int64_t)p.rows[b] * p.K / 4;
+  float m = 0.f;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
+    const float4 v = x[i];
+    const float a = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    // fmaxf drops NaN operands; infinities are left out, too (they reach H through the planes)
+    m = (a <= 3.4028235e38f) ? fmaxf(m, a) : m;
+  }
+  for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+  if ((threadIdx.x & 63) == 0 && m > 0.f) atomicMax(&sc->amax_bits, __float_as_uint(m));
+}
+
+__global__ void split_scale_kernel(SplitScalars *sc) {
+  const float amax = __uint_as_float(sc->amax_bits);
+  int ex = 0;
+  (void)frexpf(amax, &ex);                       // 2^(ex-1) <= amax < 2^ex
+  int e = amax > 0.f ? ex - 15 : 0;
+  e = e < -60 ? -60 : (e > 60 ? 60 : e);         // 2^-e and 4^e stay normal fp32 numbers
+  sc->down = ldexpf(1.f, -e);
+  sc->unit = ldexpf(1.f, 2 * e);
+}
+
+// planes: rows of the table's batches one after the other, [row][K] fp16 each
+__global__ __launch_bounds__(256) void split_planes_kernel(SyrkArgs p, const SplitScalars *sc, __half *hi,
+                                                           __half *lo) {
+  const int b = blockIdx.y;
+  int64_t row0 = 0;
+  for (int i = 0; i < b; ++i) row0 += p.rows[i];
+  const float down = sc->down;
+  const float4 *x = reinterpret_cast<const float4 *>(p.ptr[b]);
+  const int64_t n4 = (int64_t)p.rows[b] * p.K / 4, o4 = row0 * p.K / 4;
+  typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+  h4 *dh = reinterpret_cast<h4 *>(hi) + o4, *dl = reinterpret_cast<h4 *>(lo) + o4;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
+    const float4 v = x[i];
+    const float s[4] = {v.x * down, v.y * down, v.z * down, v.w * down};
+    h4 h, l;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      h[c] = (_Float16)s[c];
+      l[c] = (_Float16)(s[c] - (float)h[c]);     // the difference is exact in fp32
+    }
+    dh[i] = h;
+    dl[i] = l;
+  }
+}
+
+constexpr int SPLIT_BATCHES = H_NBMAX / 3;        // real batches per launch (three table entries each)
+
+struct SplitPlan {
+  int64_t cap_rows;            // rows of a batch group (one launch)
+  int rs, T;
+  size_t part_bytes, sc_off, hi_off, lo_off, total_bytes;
+};
+
+SplitPlan split_plan(int64_t K, int64_t max_batch_rows) {
+  SplitPlan p{};
+  p.T = (int)ceil_div64(K, W16_TB);
+  const int64_t nt = (int64_t)p.T * (p.T + 1) / 2;
+  p.rs = pick_rs_wide(K);
+  p.part_bytes = p.rs == 1 ? 0 : (size_t)p.rs * nt * W16_TB * W16_TB * sizeof(float);
+  int64_t cap = ((int64_t)1 << 29) / K / D16_BK * D16_BK;     // planes of about 1 GB each
+  if (cap < max_batch_rows) cap = max_batch_rows;
+  p.cap_rows = cap;
+  p.sc_off = (p.part_bytes + 255) & ~(size_t)255;
+  p.hi_off = p.sc_off + 256;
+  const size_t plane = (((size_t)cap * K * sizeof(__half)) + 255) & ~(size_t)255;
+  p.lo_off = p.hi_off + plane;
+  p.total_bytes = p.lo_off + plane;
+  return p;
+}
 
 constexpr int TS = 32;
 
@@ -1150,8 +1267,8 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
       bool regular = (K % W16_TB == 0);
       for (int i = 0; i < w.nb; ++i) regular = regular && (w.rows[i] % D16_BK == 0);
       const bool f16 = x_dtype == GPTQ_HIP_F16;
-      const void *fn = regular ? (f16 ? reinterpret_cast<const void *>(syrk16d_kernel<__half>)
-                                      : reinterpret_cast<const void *>(syrk16d_kernel<__hip_bfloat16>))
+      const void *fn = regular ? (f16 ? reinterpret_cast<const void *>(syrk16d_kernel<__half, SyrkArgs>)
+                                      : reinterpret_cast<const void *>(syrk16d_kernel<__hip_bfloat16, SyrkArgs>))
                                : (f16 ? reinterpret_cast<const void *>(syrk16w_kernel<__half>)
                                       : reinterpret_cast<const void *>(syrk16w_kernel<__hip_bfloat16>));
       const int lds_bytes = regular ? D16_LDS_BYTES : W16_LDS_BYTES;
@@ -1159,9 +1276,9 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
         return GPTQ_HIP_ELAUNCH;
       const dim3 wgrid((unsigned)(nt * w.RS));
       if (regular && f16)
-        hipLaunchKernelGGL(syrk16d_kernel<__half>, wgrid, block, lds_bytes, st, w);
+        hipLaunchKernelGGL((syrk16d_kernel<__half, SyrkArgs>), wgrid, block, lds_bytes, st, w);
       else if (regular)
-        hipLaunchKernelGGL(syrk16d_kernel<__hip_bfloat16>, wgrid, block, lds_bytes, st, w);
+        hipLaunchKernelGGL((syrk16d_kernel<__hip_bfloat16, SyrkArgs>), wgrid, block, lds_bytes, st, w);
       else if (f16)
         hipLaunchKernelGGL(syrk16w_kernel<__half>, wgrid, block, lds_bytes, st, w);
       else
@@ -1169,7 +1286,7 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
       GPTQ_CHECK_LAUNCH();
       if (w.RS > 1) {
         hipLaunchKernelGGL(syrk_reduce_kernel<W16_TB>, dim3((unsigned)nt), dim3(256), 0, st, H, w.ws,
-                           (int)K, w.T, w.RS);
+                           (int)K, w.T, w.RS, (const float *)nullptr);
         GPTQ_CHECK_LAUNCH();
       }
       continue;
@@ -1193,7 +1310,7 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
       GPTQ_CHECK_LAUNCH();
       if (a.RS > 1) {
         hipLaunchKernelGGL(syrk_reduce_kernel<HB>, dim3((unsigned)ntiles), dim3(256), 0, st, H, a.ws,
-                           (int)K, T, a.RS);
+                           (int)K, T, a.RS, (const float *)nullptr);
         GPTQ_CHECK_LAUNCH();
       }
       continue;
@@ -1215,9 +1332,117 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
     GPTQ_CHECK_LAUNCH();
     if (a.RS > 1) {
       hipLaunchKernelGGL(syrk_reduce_kernel<HB>, dim3((unsigned)ntiles), dim3(256), 0, st, H, a.ws,
-                         (int)K, T, a.RS);
+                         (int)K, T, a.RS, (const float *)nullptr);
       GPTQ_CHECK_LAUNCH();
     }
+  }
+  return GPTQ_HIP_OK;
+}
+
+size_t gptq_hip_hessian_accumulate_split16_workspace_bytes(int64_t K, int64_t max_batch_rows) {
+  if (K <= 0 || K % W16_TB != 0 || max_batch_rows <= 0 || max_batch_rows % D16_BK != 0) return 0;
+  return split_plan(K, max_batch_rows).total_bytes;
+}
+
+int gptq_hip_hessian_accumulate_split16(void *stream, const void *const *x_ptrs, const int64_t *x_rows,
+                                        int n_batches, int64_t K, float *H, void *ws, size_t ws_bytes) {
+  if (n_batches < 0 || K <= 0 || K > 46000 || !H) return GPTQ_HIP_EINVAL;
+  if (n_batches > 0 && (!x_ptrs || !x_rows)) return GPTQ_HIP_EINVAL;
+  if (K % W16_TB != 0) return GPTQ_HIP_EINVAL;
+  int64_t max_rows = 0;
+  for (int b = 0; b < n_batches; ++b) {
+    const int64_t rows = x_rows[b];
+    if (rows < 0 || rows > 2147483647LL || rows % D16_BK != 0) return GPTQ_HIP_EINVAL;
+    if (rows > 0 && (!x_ptrs[b] || (reinterpret_cast<uintptr_t>(x_ptrs[b]) & 15))) return GPTQ_HIP_EINVAL;
+    if (rows > max_rows) max_rows = rows;
+  }
+  if (max_rows == 0) return GPTQ_HIP_OK;
+  const SplitPlan sp = split_plan(K, max_rows);
+  if (!ws || ws_bytes < sp.total_bytes || (reinterpret_cast<uintptr_t>(ws) & 15)) return GPTQ_HIP_EWORKSPACE;
+  hipStream_t st = as_stream(stream);
+  char *base = reinterpret_cast<char *>(ws);
+  SplitScalars *sc = reinterpret_cast<SplitScalars *>(base + sp.sc_off);
+  __half *hi = reinterpret_cast<__half *>(base + sp.hi_off), *lo = reinterpret_cast<__half *>(base + sp.lo_off);
+
+  // ---- largest magnitude over all batches -> e
+  hipLaunchKernelGGL(split_reset_kernel, dim3(1), dim3(1), 0, st, sc);
+  GPTQ_CHECK_LAUNCH();
+  for (int b0 = 0; b0 < n_batches;) {
+    SyrkArgs a;
+    a.nb = 0;
+    a.K = (int)K;
+    while (b0 < n_batches && a.nb < H_NBMAX) {
+      if (x_rows[b0] > 0) {
+        a.ptr[a.nb] = x_ptrs[b0];
+        a.rows[a.nb] = (int)x_rows[b0];
+        ++a.nb;
+      }
+      ++b0;
+    }
+    if (a.nb == 0) continue;
+    hipLaunchKernelGGL(split_absmax_kernel, dim3(64, (unsigned)a.nb), dim3(256), 0, st, a, sc);
+    GPTQ_CHECK_LAUNCH();
+  }
+  hipLaunchKernelGGL(split_scale_kernel, dim3(1), dim3(1), 0, st, sc);
+  GPTQ_CHECK_LAUNCH();
+
+  // ---- groups of batches: split, multiply into the partial tiles (or into H when there is one slice)
+  const void *fn = reinterpret_cast<const void *>(syrk16d_kernel<__half, SyrkArgsDual>);
+  if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, D16_LDS_BYTES) != hipSuccess)
+    return GPTQ_HIP_ELAUNCH;
+  const int64_t nt = (int64_t)sp.T * (sp.T + 1) / 2;
+  bool first = true;
+  for (int b0 = 0; b0 < n_batches;) {
+    SyrkArgs src;
+    src.nb = 0;
+    src.K = (int)K;
+    int64_t rows_total = 0;
+    while (b0 < n_batches && src.nb < SPLIT_BATCHES) {
+      const int64_t rows = x_rows[b0];
+      if (rows > 0) {
+        if (rows_total + rows > sp.cap_rows) break;      // (a single batch always fits)
+        src.ptr[src.nb] = x_ptrs[b0];
+        src.rows[src.nb] = (int)rows;
+        ++src.nb;
+        rows_total += rows;
+      }
+      ++b0;
+    }
+    if (src.nb == 0) continue;
+    hipLaunchKernelGGL(split_planes_kernel, dim3(256, (unsigned)src.nb), dim3(256), 0, st, src, sc, hi, lo);
+    GPTQ_CHECK_LAUNCH();
+    SyrkArgsDual w;
+    w.nb = 3 * src.nb;
+    w.K = (int)K;
+    w.T = sp.T;
+    w.RS = sp.rs;
+    w.H = H;
+    w.ws = reinterpret_cast<float *>(base);
+    w.factor = &sc->unit;
+    w.accum = first ? 0 : 1;
+    int64_t row0 = 0;
+    for (int i = 0; i < src.nb; ++i) {
+      const __half *h = hi + row0 * K, *l = lo + row0 * K;
+      w.ptr[3 * i] = h;      w.ptrB[3 * i] = h;
+      w.ptr[3 * i + 1] = h;  w.ptrB[3 * i + 1] = l;
+      w.ptr[3 * i + 2] = l;  w.ptrB[3 * i + 2] = h;
+      w.rows[3 * i] = w.rows[3 * i + 1] = w.rows[3 * i + 2] = src.rows[i];
+      row0 += src.rows[i];
+    }
+    const int64_t total_rows = 3 * rows_total;
+    // (slices past the end of a short group get no slab and contribute zeros)
+    const int64_t chunk = round_up64(ceil_div64(total_rows, w.RS), W16_BK);
+    if (chunk > 2147483647LL) return GPTQ_HIP_EINVAL;
+    w.chunk = (int)chunk;
+    hipLaunchKernelGGL((syrk16d_kernel<__half, SyrkArgsDual>), dim3((unsigned)(nt * w.RS)), dim3(256),
+                       D16_LDS_BYTES, st, w);
+    GPTQ_CHECK_LAUNCH();
+    first = false;
+  }
+  if (!first && sp.rs > 1) {
+    hipLaunchKernelGGL(syrk_reduce_kernel<W16_TB>, dim3((unsigned)nt), dim3(256), 0, st, H,
+                       reinterpret_cast<const float *>(base), (int)K, sp.T, sp.rs, &sc->unit);
+    GPTQ_CHECK_LAUNCH();
   }
   return GPTQ_HIP_OK;
 }

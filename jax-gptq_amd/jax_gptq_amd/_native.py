@@ -24,6 +24,8 @@ SIGNATURES = {
     "gptq_hip_col_params": (_i32, [_vp, _vp, _i32, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _sz]),
     "gptq_hip_hessian_accumulate_workspace_bytes": (_sz, [_i64, _i32]),
     "gptq_hip_hessian_accumulate": (_i32, [_vp, _vp, _vp, _i32, _i32, _i64, _vp, _i32, _vp, _sz]),
+    "gptq_hip_hessian_accumulate_split16_workspace_bytes": (_sz, [_i64, _i64]),
+    "gptq_hip_hessian_accumulate_split16": (_i32, [_vp, _vp, _vp, _i32, _i64, _vp, _vp, _sz]),
     "gptq_hip_hessian_finalize": (_i32, [_vp, _vp, _i32, _i64, _f64]),
     "gptq_hip_damp_invert_workspace_bytes": (_sz, [_i64, _i32]),
     "gptq_hip_damp_invert": (_i32, [_vp, _vp, _i32, _vp, _i64, _i64, _i64, _f64, _i32, _vp, _vp, _vp,

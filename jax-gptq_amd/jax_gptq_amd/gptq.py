@@ -186,6 +186,27 @@ def _accumulate_H_step(H, running_mean, n_samples, batch):
     return H, running_mean, n_samples + batch.shape[0]
 
 
+def _split16_ok(H, batches):
+    """Shapes that gptq_hip_hessian_accumulate_split16 takes: fp32 rows and sums, K a multiple of
+    256, every batch a multiple of 32 rows and 16-byte aligned."""
+    K = H.shape[0]
+    return (H.dtype == torch.float32 and K % 256 == 0 and len(batches) > 0
+            and all(b.dtype == torch.float32 and b.shape[0] % 32 == 0 and b.data_ptr() % 16 == 0 for b in batches)
+            and sum(b.shape[0] for b in batches) >= 32)
+
+
+def _hessian_accumulate_split16(H, batches):
+    lib = N.load()
+    K = H.shape[0]
+    batches = [b for b in batches if b.shape[0] > 0]
+    ws = _ws(lib.gptq_hip_hessian_accumulate_split16_workspace_bytes(K, max(b.shape[0] for b in batches)))
+    nb = len(batches)
+    ptrs = (ctypes.c_void_p * nb)(*[b.data_ptr() for b in batches])
+    rows = (ctypes.c_int64 * nb)(*[b.shape[0] for b in batches])
+    N.check(lib.gptq_hip_hessian_accumulate_split16(_stream(), ptrs, rows, nb, K, _ptr(H), _ptr(ws), ws.numel()),
+            "hessian_accumulate_split16")
+
+
 def _hessian_accumulate(H, batches):
     lib = N.load()
     K = H.shape[0]
@@ -206,9 +227,11 @@ def _hessian_accumulate(H, batches):
                 "hessian_accumulate")
 
 
-def accumulate_H(xs, use_fp64=False):
+def accumulate_H(xs, use_fp64=False, split_fp16=False):
     """``H = sum_b X_b^T X_b / n`` over a list of calibration batches (``gptq.py:76-103``);
-    fp32, or fp64 products and sums with ``use_fp64`` (``gptq.py:88``)."""
+    fp32, or fp64 products and sums with ``use_fp64`` (``gptq.py:88``).  ``split_fp16`` (not in
+    the reference) multiplies fp32 rows as pairs of fp16 numbers on the 16-bit matrix cores where
+    the shapes allow it: about three times faster, products exact to 2^-22."""
     lib = N.load()
     hdt = torch.float64 if use_fp64 else torch.float32
     batches = []
@@ -224,7 +247,10 @@ def accumulate_H(xs, use_fp64=False):
         if b.shape[-1] != K:
             raise ValueError("all calibration batches must share the feature dimension")
     H = torch.zeros((K, K), dtype=hdt, device=_device())
-    _hessian_accumulate(H, batches)
+    if split_fp16 and _split16_ok(H, batches):
+        _hessian_accumulate_split16(H, batches)
+    else:
+        _hessian_accumulate(H, batches)
     n = sum(b.shape[0] for b in batches)
     N.check(lib.gptq_hip_hessian_finalize(_stream(), _ptr(H), _DT_H[hdt], K, float(n)),
             "hessian_finalize")
@@ -360,7 +386,7 @@ def _solve(W, L, params, block_size, out_dtype, want_codes=False):
 
 
 def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=None, shared=None,
-         bits=4):
+         bits=4, split_fp16=False):
     """The per-layer GPTQ solve (reference ``gptq.py:182-212``).
 
     ``W`` is ``[K, N]`` (input features x output channels), ``xs`` a list of calibration
@@ -374,7 +400,8 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=
     inverse, which depends on ``xs`` and ``damping`` only.  The results are those of independent
     calls.  ``bits`` (1 to 8; the reference's ``gptq`` is fixed at the default of its
     ``get_quantize_params``, 4): the code width, ``maxq = 2**bits - 1``; only 4-bit results can
-    be packed.
+    be packed.  ``split_fp16``: see
+    ``accumulate_H``.
     """
     Wt = _float_dev(W)
     if Wt.dim() != 2:
@@ -393,7 +420,7 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=
         H = shared.get("H")
     keep = H is not None or shared is not None      # somebody else still needs H as accumulated
     if H is None:
-        H = accumulate_H(xs, use_fp64=use_fp64)
+        H = accumulate_H(xs, use_fp64=use_fp64, split_fp16=split_fp16 and not use_fp64)
     if H.dim() != 2 or H.shape[0] != H.shape[1] or H.dtype != (torch.float64 if use_fp64 else torch.float32):
         raise ValueError("H must be the square matrix accumulate_H(xs, use_fp64) returns")
     if H.shape[0] != K:

@@ -129,3 +129,49 @@ def test_accumulate_H_16bit_mixed_batch_sizes(G, dt):
     ref2 = _closed_form([x.float().cpu().numpy() for x in ragged])
     H2 = to_np(G.accumulate_H(ragged))
     assert np.abs(H2 - ref2).max() < TOL * max(1.0, np.abs(ref2).max())
+
+
+@pytest.mark.parametrize("rows,K,nb,scale", [(2048, 256, 2, 1.0), (512, 768, 9, 1e-4), (96, 1024, 50, 3e5),
+                                             (4096, 512, 3, 1.0), (32, 256, 1, 1.0)])
+def test_accumulate_H_fp32_rows_as_fp16_pairs(G, rows, K, nb, scale):
+    """split_fp16: x = (hi + lo) 2^e with fp16 hi and lo, X^T X from hi^T hi + hi^T lo + lo^T hi on
+    the 16-bit matrix cores.  Same tolerance against the closed form as the fp32 kernel (the
+    dropped lo^T lo term is 2^-22 of a product); the exponent is chosen from the data, so the
+    scale of the rows (1e-4 .. 3e5 here: products far outside fp16) does not matter.  50 batches
+    span two launches, whose partial tiles accumulate before the one reduction."""
+    import torch
+    rng = np.random.default_rng(rows + K + nb)
+    xs = [(rng.standard_normal((rows, K)) * scale).astype(np.float32) for _ in range(nb)]
+    # a feature 1e6 times smaller than the rest and one that is exactly zero
+    for x in xs:
+        x[:, 3] *= 1e-6
+        x[:, 5] = 0.0
+    ref = _closed_form(xs)
+    Hs = to_np(G.accumulate_H(xs, split_fp16=True))
+    H32 = to_np(G.accumulate_H(xs))
+    assert Hs.shape == (K, K) and Hs.dtype == np.float32 and np.array_equal(Hs, Hs.T)
+    top = np.abs(ref).max()
+    assert np.abs(Hs - ref).max() < TOL * top
+    assert np.abs(Hs - H32).max() < 2 * TOL * top
+    assert np.all(Hs[5] == 0) and np.all(Hs[:, 5] == 0)
+    # the small feature keeps its relative accuracy on the diagonal
+    assert abs(Hs[3, 3] - ref[3, 3]) < 1e-4 * ref[3, 3]
+    # through gptq(): same codes as with the fp32 Hessian up to the usual handful of ties
+    if K == 768:
+        W = (0.02 * rng.standard_normal((K, 256))).astype(np.float32)
+        q1, p1 = G.gptq(W, xs)
+        q2, p2 = G.gptq(W, xs, split_fp16=True)
+        c1 = np.rint(to_np(q1) / to_np(p1["scale"]) + to_np(p1["zero"]))
+        c2 = np.rint(to_np(q2) / to_np(p2["scale"]) + to_np(p2["zero"]))
+        assert np.mean(c1 == c2) >= 0.999 and np.abs(c1 - c2).max() <= 1
+
+
+def test_accumulate_H_split_fp16_falls_back_on_other_shapes(G):
+    """Shapes outside the split path's requirements (K % 256, rows % 32, 16-bit rows) run on the
+    ordinary kernels and give the ordinary result."""
+    rng = np.random.default_rng(3)
+    for rows, K in [(40, 256), (64, 200)]:
+        xs = [rng.standard_normal((rows, K)).astype(np.float32) for _ in range(3)]
+        assert np.array_equal(to_np(G.accumulate_H(xs, split_fp16=True)), to_np(G.accumulate_H(xs)))
+    xs = [rng.standard_normal((64, 256)).astype(np.float16) for _ in range(3)]
+    assert np.array_equal(to_np(G.accumulate_H(xs, split_fp16=True)), to_np(G.accumulate_H(xs)))
