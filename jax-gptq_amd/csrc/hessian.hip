@@ -1391,13 +1391,19 @@ int gptq_hip_hessian_accumulate_split16(void *stream, const void *const *x_ptrs,
   if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, D16_LDS_BYTES) != hipSuccess)
     return GPTQ_HIP_ELAUNCH;
   const int64_t nt = (int64_t)sp.T * (sp.T + 1) / 2;
+  // batches per launch: as even as the table allows (a short last launch costs as much per
+  // workgroup as a long one)
+  int n_real = 0;
+  for (int b = 0; b < n_batches; ++b) n_real += x_rows[b] > 0 ? 1 : 0;
+  const int n_groups = (n_real + SPLIT_BATCHES - 1) / SPLIT_BATCHES;
+  const int per_group = (n_real + n_groups - 1) / n_groups;
   bool first = true;
   for (int b0 = 0; b0 < n_batches;) {
     SyrkArgs src;
     src.nb = 0;
     src.K = (int)K;
     int64_t rows_total = 0;
-    while (b0 < n_batches && src.nb < SPLIT_BATCHES) {
+    while (b0 < n_batches && src.nb < per_group) {
       const int64_t rows = x_rows[b0];
       if (rows > 0) {
         if (rows_total + rows > sp.cap_rows) break;      // (a single batch always fits)
