@@ -223,7 +223,8 @@ class _Session:
         if self._h_cache is not None and self._h_cache[0] == sig:
             return self._h_cache[2]
         self._h_cache = None                      # release the previous activations first
-        shared = {"H": accumulate_H(xs, use_fp64=self.options["use_fp64"])}
+        shared = {"H": accumulate_H(xs, use_fp64=self.options["use_fp64"],
+                                    split_fp16=self.options["split_fp16"] and not self.options["use_fp64"])}
         self._h_cache = (sig, list(xs), shared)
         return shared
 
@@ -265,7 +266,7 @@ class _Session:
 
 
 def quantize(fn, params, inputs, block_size=128, actorder=False, damping=0.01,
-             use_quantized_activations=True, use_fp64=False, use_params_fp32=False):
+             use_quantized_activations=True, use_fp64=False, use_params_fp32=False, split_fp16=False):
     """Run GPTQ over the parameters of ``fn`` (reference ``quantize_interpreter.py:25-80``).
 
     ``fn(params, batch)``: the model; ``params``: a nested dict / list / tuple of arrays;
@@ -274,7 +275,7 @@ def quantize(fn, params, inputs, block_size=128, actorder=False, damping=0.01,
     :class:`QuantizedMatrix` (packed along its contraction axis, in its original layout);
     everything else is returned as it came.  Buffers of ``params`` that already live on the
     GPU are overwritten with the quantised values, so do not reuse them (the reference frees
-    them, ``:42``).
+    them, ``:42``).  ``split_fp16`` (not in the reference): see ``accumulate_H``.
     """
     if not inputs:
         raise ValueError("quantize needs at least one calibration batch")
@@ -290,7 +291,7 @@ def quantize(fn, params, inputs, block_size=128, actorder=False, damping=0.01,
         flat.append(t)
     session = _Session(flat, dict(block_size=block_size, actorder=actorder, damping=damping,
                                   use_quantized_activations=use_quantized_activations,
-                                  use_fp64=use_fp64))
+                                  use_fp64=use_fp64, split_fp16=split_fp16))
     wrapped = [(_Target(t, i, range(t.dim())) if isinstance(t, torch.Tensor) and t.is_floating_point()
                 and t.dim() > 1 else t) for i, t in enumerate(flat)]
     fn_params = _unflatten(struct, wrapped)

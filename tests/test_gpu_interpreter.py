@@ -93,7 +93,7 @@ def test_products_on_the_same_activations_share_one_hessian(T, J, monkeypatch):
     import jax_gptq_amd.quantize_interpreter as QI
     calls = []
     real = QI.accumulate_H
-    monkeypatch.setattr(QI, "accumulate_H", lambda xs, use_fp64=False: (calls.append(len(xs)), real(xs, use_fp64))[1])
+    monkeypatch.setattr(QI, "accumulate_H", lambda xs, **kw: (calls.append(len(xs)), real(xs, **kw))[1])
     factorisations = []
     real_di = G._damp_invert
     monkeypatch.setattr(G, "_damp_invert", lambda *a, **k: (factorisations.append(1), real_di(*a, **k))[1])
@@ -339,6 +339,33 @@ def test_gpt2_shaped_model_through_the_driver(T, J):
     rel = float((out - ref).norm() / ref.norm())
     assert rel < 0.25, rel
     assert float((out_k - out).norm() / out.norm()) < 2e-2
+
+
+def test_quantize_with_split_fp16_hessians(T, J):
+    """``quantize(..., split_fp16=True)``: fp32 activations of a GPT-2-shaped model (d = 256, so
+    every Linear input has a multiple of 256 features) go through the fp16-pair Hessian.  The
+    first product sees identical inputs: its codes agree up to a handful of ties.  Every flipped
+    tie changes the activations that later products are calibrated on, and the error feedback of
+    the column loop turns such a change into many different (equally good) codes, so for the
+    model as a whole the check is the distance to the dense model."""
+    import copy
+    d, n_layer, vocab, n_ctx, n_head = 256, 1, 512, 64, 4
+    params = _gpt2_params(T, d, n_layer, vocab, n_ctx)
+    dense = copy.deepcopy(params)
+    params2 = copy.deepcopy(params)
+    g = T.Generator(device="cuda")
+    g.manual_seed(6)
+    batches = [T.randint(0, vocab, (4, n_ctx), generator=g, device="cuda") for _ in range(8)]
+    f = _gpt2(n_head)
+    ref = f(dense, batches[0])
+    q1 = J.quantize(f, params, batches, block_size=64)
+    q2 = J.quantize(f, params2, batches, block_size=64, split_fp16=True)
+    a, b = q1["h"][0]["attn"]["c_attn"]["w"].int_weight, q2["h"][0]["attn"]["c_attn"]["w"].int_weight
+    same = ((a & 15) == (b & 15)).float().mean() + ((a >> 4) == (b >> 4)).float().mean()
+    assert float(same) / 2 >= 0.999, float(same) / 2
+    e1 = float((J.use_quantized(f)(q1, batches[0]) - ref).norm() / ref.norm())
+    e2 = float((J.use_quantized(f)(q2, batches[0]) - ref).norm() / ref.norm())
+    assert e2 < 1.1 * e1 + 1e-3, (e1, e2)
 
 
 def test_gpt2_small_full_shape(T, J):
