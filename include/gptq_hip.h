@@ -57,7 +57,7 @@ int gptq_hip_col_params(void *stream, const void *W, int w_dtype, int64_t K, int
  * gptq.py:65-72 multiplies in fp32).  Every element is split as x = (hi + lo) 2^e, hi and lo
  * fp16, e one exponent for the whole call, and X^T X = 4^e (hi^T hi + hi^T lo + lo^T hi) is
  * accumulated in fp32 from exact fp16 products; the dropped lo^T lo term is below 2^-22 of each
- * product.  1.8 times faster than gptq_hip_hessian_accumulate on fp32 rows (K = 4096).  Requires
+ * product.  2.2 times faster than gptq_hip_hessian_accumulate on fp32 rows (K = 4096).  Requires
  * K % 256 == 0 and every batch a multiple of 32 rows and 16-byte aligned; returns
  * GPTQ_HIP_EINVAL otherwise (use gptq_hip_hessian_accumulate then).
  * H += sum_b X_b^T X_b (upper tiles), fp32; ws: ..._split16_workspace_bytes(K, largest batch). */

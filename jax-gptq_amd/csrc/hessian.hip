@@ -801,9 +801,16 @@ __global__ __launch_bounds__(256) void syrk16d_kernel(ARGS p) {
   const int ld_feat = (ld_op ? n0 : m0) + l32 * 8;
   const uint32_t ld_dst0 = lds0 + ld_op * D16_OP + ld_pair0 * D16_PAIR;
   // position of the next slab to load: batch b (base pointer Xb, rows_b rows), row kt
+  // (the choice of the table is made on a scalar: left to a per-lane select, the batch pointer
+  //  would live in vector registers, of which this kernel has none to spare)
+  const bool from_b = ARGS::DUAL && __builtin_amdgcn_readfirstlane(ld_op) != 0;
   auto batch_ptr = [&](int bb) __attribute__((always_inline)) -> const uint16_t * {
-    if constexpr (ARGS::DUAL) return reinterpret_cast<const uint16_t *>(ld_op ? p.ptrB[bb] : p.ptr[bb]);
-    else return reinterpret_cast<const uint16_t *>(p.ptr[bb]);
+    if constexpr (ARGS::DUAL) {
+      const void *const *tab = from_b ? p.ptrB : p.ptr;
+      return reinterpret_cast<const uint16_t *>(tab[bb]);
+    } else {
+      return reinterpret_cast<const uint16_t *>(p.ptr[bb]);
+    }
   };
   const uint16_t *Xb = batch_ptr(b);
   int rows_b = p.rows[b];
@@ -972,11 +979,17 @@ __global__ __launch_bounds__(256) void syrk16d_kernel(ARGS p) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int col = wn * 128 + j * 32 + l32;
+        // (accumulating: the sixteen loads of a block first, so that they are in flight together)
+        float old[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int row = wm * 128 + ii * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-          if (ARGS::DUAL && accum) dst[row * W16_TB + col] += acc[ii][j][r];
-          else dst[row * W16_TB + col] = acc[ii][j][r];
+          old[r] = (ARGS::DUAL && accum) ? dst[row * W16_TB + col] : 0.f;
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = wm * 128 + ii * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+          dst[row * W16_TB + col] = ARGS::DUAL ? acc[ii][j][r] + old[r] : acc[ii][j][r];
         }
       }
   }
@@ -1043,7 +1056,7 @@ bool use_wide16(int64_t K) { return K >= 1024; }
 //   X^T X = 4^e (hi^T hi + hi^T lo + lo^T hi)  up to lo^T lo (relative 2^-22 per product).
 // The three products are one launch of the two-matrix 16-bit kernel over the batch pairs
 // (hi, hi), (hi, lo), (lo, hi): three times the 16-bit work instead of fp32 MFMAs at a
-// sixteenth of the rate (K = 4096, 262144 rows: 19.7 ms against 35.4 ms).  Steps: largest magnitude of all batches (one read of X), then per
+// sixteenth of the rate (K = 4096, 262144 rows: 15.7 ms against 35.4 ms).  Steps: largest magnitude of all batches (one read of X), then per
 // group of batches split into two fp16 planes (workspace), multiply, and at the end one reduction
 // that applies 4^e.  No host synchronisation: e lives in device memory.
 struct SplitScalars { uint32_t amax_bits; float down, unit; };
