@@ -187,10 +187,11 @@ def _accumulate_H_step(H, running_mean, n_samples, batch):
 
 
 def _split16_ok(H, batches):
-    """Shapes that gptq_hip_hessian_accumulate_split16 takes: fp32 rows and sums, K a multiple of
-    256, every batch a multiple of 32 rows and 16-byte aligned."""
+    """Shapes that gptq_hip_hessian_accumulate_split16 takes (fp32 rows and sums, K a multiple of
+    256, every batch a multiple of 32 rows and 16-byte aligned) and on which it is the faster one
+    (K >= 1024: at K = 768 the fp32 kernel needs 0.8 ms for 65536 rows, the split path 1.0 ms)."""
     K = H.shape[0]
-    return (H.dtype == torch.float32 and K % 256 == 0 and len(batches) > 0
+    return (H.dtype == torch.float32 and K % 256 == 0 and K >= 1024 and len(batches) > 0
             and all(b.dtype == torch.float32 and b.shape[0] % 32 == 0 and b.data_ptr() % 16 == 0 for b in batches)
             and sum(b.shape[0] for b in batches) >= 32)
 

@@ -131,8 +131,23 @@ def test_accumulate_H_16bit_mixed_batch_sizes(G, dt):
     assert np.abs(H2 - ref2).max() < TOL * max(1.0, np.abs(ref2).max())
 
 
+def _split_H(G, xs):
+    """accumulate_H(xs, split_fp16=True) without the wrapper's K >= 1024 rule (below that the fp32
+    kernel is the faster one and the wrapper keeps it): the split entry point on any K % 256 == 0."""
+    import torch
+    import jax_gptq_amd._native as NV
+    batches = [torch.from_numpy(x).cuda() for x in xs]
+    K = batches[0].shape[1]
+    H = torch.zeros((K, K), dtype=torch.float32, device="cuda")
+    assert G._split16_ok(H, batches) or K < 1024
+    G._hessian_accumulate_split16(H, batches)
+    NV.check(NV.load().gptq_hip_hessian_finalize(G._stream(), H.data_ptr(), 0, K, float(sum(b.shape[0] for b in batches))),
+             "hessian_finalize")
+    return H
+
+
 @pytest.mark.parametrize("rows,K,nb,scale", [(2048, 256, 2, 1.0), (512, 768, 9, 1e-4), (96, 1024, 50, 3e5),
-                                             (4096, 512, 3, 1.0), (32, 256, 1, 1.0)])
+                                             (4096, 512, 3, 1.0), (32, 256, 1, 1.0), (512, 1280, 5, 1.0)])
 def test_accumulate_H_fp32_rows_as_fp16_pairs(G, rows, K, nb, scale):
     """split_fp16: x = (hi + lo) 2^e with fp16 hi and lo, X^T X from hi^T hi + hi^T lo + lo^T hi on
     the 16-bit matrix cores.  Same tolerance against the closed form as the fp32 kernel (the
@@ -147,7 +162,9 @@ def test_accumulate_H_fp32_rows_as_fp16_pairs(G, rows, K, nb, scale):
         x[:, 3] *= 1e-6
         x[:, 5] = 0.0
     ref = _closed_form(xs)
-    Hs = to_np(G.accumulate_H(xs, split_fp16=True))
+    Hs = to_np(_split_H(G, xs))
+    if K >= 1024:
+        assert np.array_equal(Hs, to_np(G.accumulate_H(xs, split_fp16=True)))
     H32 = to_np(G.accumulate_H(xs))
     assert Hs.shape == (K, K) and Hs.dtype == np.float32 and np.array_equal(Hs, Hs.T)
     top = np.abs(ref).max()
@@ -157,7 +174,7 @@ def test_accumulate_H_fp32_rows_as_fp16_pairs(G, rows, K, nb, scale):
     # the small feature keeps its relative accuracy on the diagonal
     assert abs(Hs[3, 3] - ref[3, 3]) < 1e-4 * ref[3, 3]
     # through gptq(): same codes as with the fp32 Hessian up to the usual handful of ties
-    if K == 768:
+    if K == 1280:
         W = (0.02 * rng.standard_normal((K, 256))).astype(np.float32)
         q1, p1 = G.gptq(W, xs)
         q2, p2 = G.gptq(W, xs, split_fp16=True)
@@ -167,11 +184,11 @@ def test_accumulate_H_fp32_rows_as_fp16_pairs(G, rows, K, nb, scale):
 
 
 def test_accumulate_H_split_fp16_falls_back_on_other_shapes(G):
-    """Shapes outside the split path's requirements (K % 256, rows % 32, 16-bit rows) run on the
-    ordinary kernels and give the ordinary result."""
+    """Shapes outside the split path's requirements (K % 256, rows % 32, K >= 1024, fp32 rows) run on
+    the ordinary kernels and give the ordinary result."""
     rng = np.random.default_rng(3)
-    for rows, K in [(40, 256), (64, 200)]:
+    for rows, K in [(40, 1024), (64, 1000), (64, 768)]:
         xs = [rng.standard_normal((rows, K)).astype(np.float32) for _ in range(3)]
         assert np.array_equal(to_np(G.accumulate_H(xs, split_fp16=True)), to_np(G.accumulate_H(xs)))
-    xs = [rng.standard_normal((64, 256)).astype(np.float16) for _ in range(3)]
+    xs = [rng.standard_normal((64, 1024)).astype(np.float16) for _ in range(3)]
     assert np.array_equal(to_np(G.accumulate_H(xs, split_fp16=True)), to_np(G.accumulate_H(xs)))
