@@ -108,7 +108,7 @@ def bench_qmatmul(reps=240):
         cases = [(1, 0, "float16"), (16, 0, "float16"), (128, 0, "float16"), (2048, 0, "float16"),
                  (2048, 1, "float16")]
         if K == K_IN:
-            cases += [(1, 0, "bfloat16"), (16, 0, "bfloat16")]
+            cases += [(1, 0, "bfloat16"), (16, 0, "bfloat16"), (2048, 1, "bfloat16")]
         if K * N >= (1 << 27):
             cases = [(1, 0, "float16"), (16, 0, "float16")]
         for (M, tr, xdt) in cases:
