@@ -192,3 +192,18 @@ def test_accumulate_H_split_fp16_falls_back_on_other_shapes(G):
         assert np.array_equal(to_np(G.accumulate_H(xs, split_fp16=True)), to_np(G.accumulate_H(xs)))
     xs = [rng.standard_normal((64, 1024)).astype(np.float16) for _ in range(3)]
     assert np.array_equal(to_np(G.accumulate_H(xs, split_fp16=True)), to_np(G.accumulate_H(xs)))
+
+
+def test_accumulate_H_split_fp16_empty_and_3d_batches(G):
+    """An empty batch and a [4, 64, K] batch in the list: the empty one is skipped, the 3-D one is
+    256 rows; rows that are all NaN-free but contain an infinity make H non-finite, as on the fp32 path."""
+    rng = np.random.default_rng(21)
+    K = 1024
+    xs = [rng.standard_normal((64, K)).astype(np.float32), np.zeros((0, K), np.float32),
+          rng.standard_normal((4, 64, K)).astype(np.float32)]
+    ref = _closed_form([xs[0], xs[2]])
+    Hs = to_np(G.accumulate_H(xs, split_fp16=True))
+    assert np.abs(Hs - ref).max() < TOL * np.abs(ref).max()
+    assert np.abs(Hs - to_np(G.accumulate_H(xs))).max() < 2 * TOL * np.abs(ref).max()
+    xs[0][3, 7] = np.inf
+    assert not np.isfinite(to_np(G.accumulate_H(xs, split_fp16=True))).all()
