@@ -105,16 +105,19 @@ __global__ __launch_bounds__(256) void copy_out_kernel(const R *Minv, int64_t Kp
 // standard Cholesky of the index-reversed block: G G^T = J D J, M_bb = J G^T J.  Writes
 // M_bb over A[b,b] (upper part zeroed) and M_bb^-1 = J G^-T J into Minv[b,b].
 //
-// Lane r of the factorising wavefront keeps row r of G (64 VGPRs), lane j of the inverting
-// wavefront column j of G^-1; the loops are fully unrolled.  During the factorisation
-// the scaled pivot column is handed to the other lanes with v_readlane (lane c's entry
-// becomes a scalar operand of the update of column c), so a step is two instructions per
-// remaining column and touches no memory; during the inversion a row of G is read from LDS
-// with broadcast reads (every lane the same address, four values per read).  The block is
-// on the critical path of the blocked factorisation (nothing else can run while it does),
-// so latency is what counts here.  Entries above the diagonal of G hold garbage while the
-// factorisation runs (masking them would cost a third instruction per element) and are
-// replaced by zeros when G is written out.
+// Five wavefronts.  Four factorise: lane r of each keeps row r of G for the 16 columns c = 4 j + w
+// of wavefront w (fully unrolled loops).  The wavefront that owns column k scales it (pivot by
+// v_readlane, reciprocal square root) and publishes it through LDS; after the barrier every
+// factorising wavefront holds the column in one VGPR, from which lane c's entry becomes a scalar
+// operand (v_readlane) of the update of its column c: two instructions per remaining column, at
+// most 16 columns per wavefront and step.  The owner of column k + 1 updates that column first
+// and scales and publishes it before it turns to its other columns, so the chain from one pivot
+// to the next is one LDS round trip, one update and the scaling.  The fifth wavefront follows
+// one step behind and computes row k of X = G^-1 (lane j keeps column j of X) from row k of G,
+// which it reads from LDS with broadcast reads.  One workgroup barrier per step.  The block is on
+// the critical path of the blocked factorisation (nothing else can run while it does), so latency
+// is what counts here.  Entries above the diagonal of G hold garbage while the factorisation
+// runs (masking them would cost a third instruction per element) and are written out as zeros.
 static_assert(NB == 64, "the diagonal kernel maps one matrix row to one lane of a wavefront");
 constexpr int GSTR = NB + 4;   // LDS row stride of G: rows stay 16-byte aligned
 
@@ -141,51 +144,79 @@ __device__ __forceinline__ void root_and_inverse(double piv, double &root, doubl
   rinv = 1.0 / root;
 }
 
+constexpr int DIAG_FW = 4;                       // factorising wavefronts
+constexpr int DIAG_THREADS = (DIAG_FW + 1) * 64;
+
 template <typename R>
-__global__ __launch_bounds__(128) void chol_diag_kernel(R *A, R *Minv, int64_t ld, int b,
-                                                        int32_t *status) {
+__global__ __launch_bounds__(DIAG_THREADS) void chol_diag_kernel(R *A, R *Minv, int64_t ld, int b,
+                                                                 int32_t *status) {
   __shared__ __attribute__((aligned(16))) R dinv[NB];        // 1 / G[k][k]
   __shared__ __attribute__((aligned(16))) R Gs[NB * GSTR];   // G, row major
   __shared__ __attribute__((aligned(16))) R Xs[NB * (NB + 1)];   // X = G^-1, row major
+  __shared__ __attribute__((aligned(16))) R Lcol[2][NB];     // column k of G, by step parity
   constexpr int XSTR = NB + 1;
+  constexpr int CW = NB / DIAG_FW;                           // columns per factorising wavefront
   const int r = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   R *D = A + (int64_t)b * NB * ld + (int64_t)b * NB;
   R *Dinv = Minv + (int64_t)b * NB * ld + (int64_t)b * NB;
-  typedef R rowvec __attribute__((ext_vector_type(NB)));   // a vector value, never an alloca
+  typedef R colvec __attribute__((ext_vector_type(CW)));    // vector values, never an alloca
+  typedef R rowvec __attribute__((ext_vector_type(NB)));
 
-  // Two wavefronts, one behind the other: wavefront 0 factorises (lane r keeps row r of G),
-  // publishes column k of G in LDS as soon as it is final and goes on with the trailing update
-  // of step k; wavefront 1 meanwhile computes row k of X = G^-1 (lane j keeps column j of X),
-  // which needs exactly the columns 0..k of row k of G.  One workgroup barrier per step on
-  // both sides (64 each, no other barrier inside the loops).
-  if (wave == 0) {
+  if (wave < DIAG_FW) {
     // G[r][c] (c <= r) = D[63-c][63-r]: for fixed c the lanes read one row of D (coalesced)
-    rowvec g;
+    colvec g;
 #pragma unroll
-    for (int c = 0; c < NB; ++c) {
-      g[c] = D[(int64_t)(NB - 1 - c) * ld + (NB - 1 - r)];   // c > r: finite garbage, never used
+    for (int j = 0; j < CW; ++j) {
+      const int c = DIAG_FW * j + wave;
+      g[j] = D[(int64_t)(NB - 1 - c) * ld + (NB - 1 - r)];   // c > r: finite garbage, never used
     }
-    // ---- Cholesky, right-looking: after step k, g[k] of lane r >= k holds G[r][k]
     bool bad = false;
-#pragma unroll
-    for (int k = 0; k < NB; ++k) {
-      const R piv = lane_bcast(g[k], k);
+    // scales column k (held by this wavefront as g[k / 4]) and publishes it
+    auto scale_and_publish = [&](int k) __attribute__((always_inline)) {
+      const int jk = k / DIAG_FW;
+      const R piv = lane_bcast(g[jk], k);
       bad = bad || !(piv > R(0));
       R root, rinv;
       root_and_inverse(piv, root, rinv);
-      const R l = (r == k) ? root : g[k] * rinv;
-      g[k] = l;
+      const R l = (r == k) ? root : g[jk] * rinv;
+      g[jk] = l;
+      Lcol[k & 1][r] = l;
       Gs[r * GSTR + k] = (k <= r) ? l : R(0);
       if (r == k) dinv[k] = rinv;
-      __syncthreads();                       // column k is in LDS
+    };
+    if (wave == 0) scale_and_publish(0);
 #pragma unroll
-      for (int c = k + 1; c < NB; ++c) {
-        R t = g[c] - l * lane_bcast(l, c);   // G[r][c] -= G[r][k] G[c][k]
+    for (int k = 0; k < NB; ++k) {
+      __syncthreads();                        // column k is in LDS
+      const R l = Lcol[k & 1][r];
+      const int owner = k % DIAG_FW, jk = k / DIAG_FW;
+      // G[r][c] -= G[r][k] G[c][k] for this wavefront's column c = 4 j + wave
+      auto update = [&](int j) __attribute__((always_inline)) {
+        R t = g[j] - l * lane_bcast(l, DIAG_FW * j + wave);
         // Pin the update to this step: left free, the compiler may defer every update until the
         // element is needed and keep the operands of all steps alive.
         asm volatile("" : "+v"(t));
-        g[c] = t;
+        g[j] = t;
+      };
+      if (k + 1 < NB) {
+        // column k + 1 first, by its owner, which then scales and publishes it
+        const int nown = (k + 1) % DIAG_FW, jn = (k + 1) / DIAG_FW;
+        if (wave == nown) {
+          update(jn);
+          scale_and_publish(k + 1);
+        }
+#pragma unroll
+        for (int j = jk; j < CW; ++j) {
+          // columns c > k of this wavefront, except k + 1 (done above by its owner)
+          if (j == jk) {
+            if (wave > owner && !(wave == nown && j == jn)) update(j);
+          } else if (j == jn) {
+            if (wave != nown) update(j);
+          } else {
+            update(j);
+          }
+        }
       }
     }
     if (__any(bad) && r == 0) atomicMax(status, b + 1);
@@ -206,14 +237,17 @@ __global__ __launch_bounds__(128) void chol_diag_kernel(R *A, R *Minv, int64_t l
     for (int i = 0; i < NB; ++i) Xs[i * XSTR + r] = x[i];
   }
   __syncthreads();
-  // M_bb[i][j] = G[63-j][63-i], Minv_bb[i][j] = X[63-j][63-i]  (i >= j), zero above; wavefront 0
-  // writes M_bb, wavefront 1 the inverse
-  if (wave == 0) {
-    for (int i = 0; i < NB; ++i)
-      D[(int64_t)i * ld + r] = (i >= r) ? Gs[(NB - 1 - r) * GSTR + (NB - 1 - i)] : R(0);
-  } else {
-    for (int i = 0; i < NB; ++i)
-      Dinv[(int64_t)i * ld + r] = (i >= r) ? Xs[(NB - 1 - r) * XSTR + (NB - 1 - i)] : R(0);
+  // M_bb[i][j] = G[63-j][63-i], Minv_bb[i][j] = X[63-j][63-i]  (i >= j), zero above; wavefronts 0-1
+  // write M_bb (half of the rows each), 2-3 the inverse
+  if (wave < 4) {
+    const int half = wave & 1;
+    if (wave < 2) {
+      for (int i = half * (NB / 2); i < (half + 1) * (NB / 2); ++i)
+        D[(int64_t)i * ld + r] = (i >= r) ? Gs[(NB - 1 - r) * GSTR + (NB - 1 - i)] : R(0);
+    } else {
+      for (int i = half * (NB / 2); i < (half + 1) * (NB / 2); ++i)
+        Dinv[(int64_t)i * ld + r] = (i >= r) ? Xs[(NB - 1 - r) * XSTR + (NB - 1 - i)] : R(0);
+    }
   }
 }
 
@@ -277,7 +311,7 @@ int damp_invert(hipStream_t st, R *H, float *W, int64_t K, int64_t N, int64_t ld
   for (int b1 = nblk; b1 > 0;) {
     const int b0 = ((b1 - 1) / OUTER) * OUTER;      // outer block = diagonal blocks [b0, b1)
     for (int b = b1 - 1; b >= b0; --b) {
-      hipLaunchKernelGGL(chol_diag_kernel<R>, dim3(1), dim3(128), 0, st, p.A, p.Minv, Kp, b, status);
+      hipLaunchKernelGGL(chol_diag_kernel<R>, dim3(1), dim3(DIAG_THREADS), 0, st, p.A, p.Minv, Kp, b, status);
       GPTQ_CHECK_LAUNCH();
       if (b == 0) break;
       R *panel = p.A + (int64_t)b * NB * Kp;  // rows of block b, columns 0 .. b*NB
