@@ -345,6 +345,7 @@ int damp_invert(hipStream_t st, R *H, float *W, int64_t K, int64_t N, int64_t ld
       s.beta = 1.f;
       s.a_kmajor = 1;
       s.in_dtype = DT;
+      if (s.m == s.n) s.tri = 2;         // single level: a square, of which only the lower tiles are read
       rc = gptq_gemm(st, s, (R *)nullptr);
       if (rc) return rc;
     }
