@@ -267,7 +267,7 @@ def main():
                 "frac": round(achieved / peak, 4),
                 # bytes per launch beyond L2 from rocprofv3 FETCH_SIZE + WRITE_SIZE (scaled by what the
                 # counters read for a 1 GiB copy: x2.000 / x1.000), summary kept under profiles/
-                "traffic": 5.79e10 if wide else 8.6e9,
+                "traffic": 5.71e10 if wide else 1.06e10,
                 "flop_per_launch": flop_per_launch, "avg_launch_ms": round(hess_ms, 4),
                 "launches_per_step": 1,
                 "executed_tflops": round(executed, 2),
