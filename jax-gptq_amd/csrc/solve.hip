@@ -3,15 +3,15 @@
 // rest of its 512-row group, after every group into everything below it.
 //
 // In-block kernel: the N output channels are independent, so one lane owns one channel and a
-// workgroup of four wavefronts owns 64 channels.  The workgroup first copies its channels of
+// workgroup of eight wavefronts owns 64 channels.  The workgroup first copies its channels of
 // the block's rows and the block's corner of L into LDS (all loads of a wavefront in flight
 // at once), then works out of LDS only.  The block is walked in sub-blocks of SB rows:
 //   * the SB rows of a sub-block and their SB errors live in VGPRs (statically indexed,
-//     fully unrolled triangle).  This part is a sequential chain per channel; all four
+//     fully unrolled triangle).  This part is a sequential chain per channel; all
 //     wavefronts evaluate it redundantly (same instructions, same values), which saves a
-//     broadcast of the errors and costs nothing, since they sit on different SIMDs;
+//     broadcast of the errors and costs nothing: the chain is bound by latency, not by issue;
 //   * the rows of the block below the sub-block are then updated in the LDS tile, the rows
-//     dealt round-robin to the four wavefronts; one barrier per sub-block.
+//     dealt round-robin to the wavefronts; one barrier per sub-block.
 // Each lane touches only its own column of the tile (no bank conflicts); L is read with
 // broadcast reads (every lane the same address), the SB factors of one row are consecutive.
 // W itself is not written.
@@ -26,7 +26,7 @@
 namespace {
 
 constexpr int SOLVE_CH = 64;               // channels per workgroup (one per lane)
-constexpr int SOLVE_NW = 4;                // wavefronts per workgroup
+constexpr int SOLVE_NW = 8;                // wavefronts per workgroup (4: 45 us per block, 8: 40, 16: 52)
 constexpr int SOLVE_TPB = SOLVE_CH * SOLVE_NW;
 
 template <int SB, typename TQ>
