@@ -87,7 +87,13 @@ def _quantized_matmul(x, quantized_matrix, transpose_b):
 
 
 def quantized_matmul(x, quantized_matrix, transpose_b=False):
-    """``x @ dequant(W)`` (``transpose_b``: ``x @ dequant(W).T``), reference ``op.py:11-14``."""
+    """``x @ dequant(W)`` (``transpose_b``: ``x @ dequant(W).T``), reference ``op.py:11-14``.
+
+    fp32 accumulation; the result is rounded to fp16 and returned in ``x``'s dtype (``op.py:43,66-68``).
+    fp16 and bf16 activations enter the matrix cores as they are; fp32 activations are rounded to
+    fp16 precision after a per-row power-of-two scaling (the reference's Triton dot rounds them to
+    TF32, which has the same mantissa width) when the matrix has a multiple of 16 columns, and run
+    unrounded on plain kernels otherwise."""
     return _quantized_matmul(x, quantized_matrix, transpose_b)
 
 
