@@ -275,3 +275,37 @@ def test_qmatmul_after_gptq_matches_dense(OP):
         qw = to_np(quant_w)
         expected = inp @ (qw.T if transpose else qw)
         assert np.mean(np.abs(ret - expected)) < 3e-2        # reference test_kernel.py:41
+
+
+@pytest.mark.parametrize("M,xdt", [(1, "float16"), (16, "bfloat16"), (200, "float16"), (3, "float32")])
+def test_qmatmul_in_a_captured_graph(OP, M, xdt):
+    """A decode loop would capture the matmul in a HIP graph: the call only enqueues kernels (no
+    memset, no allocation of its own, split-K counters left at zero by every launch), so a graph
+    that holds it can be replayed; every replay, with eager calls in between, must give the eager
+    result for the input contents of that moment."""
+    import torch
+    import jax_gptq_amd.gptq as G
+    K, N = 4096, 11008
+    g = torch.Generator(device="cuda").manual_seed(M)
+    pk = torch.randint(0, 256, (K // 2, N), dtype=torch.uint8, device="cuda", generator=g)
+    zero = torch.randint(0, 16, (N,), device="cuda", generator=g).float()
+    scale = 0.001 + 0.009 * torch.rand((N,), device="cuda", generator=g)
+    qm = G.QuantizedMatrix(pk, zero, scale)
+    x = torch.randn((M, K), device="cuda", generator=g).to(getattr(torch, xdt))
+    eager = OP.quantized_matmul(x, qm).clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        OP.quantized_matmul(x, qm)                       # warm-up on the capture stream (workspace)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        y = OP.quantized_matmul(x, qm)
+    for rep in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager), rep
+        # eager work and new input contents between the replays
+        x.copy_(torch.randn((M, K), device="cuda", generator=g).to(x.dtype))
+        eager = OP.quantized_matmul(x, qm).clone()
+        torch.cuda.synchronize()
