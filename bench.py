@@ -253,21 +253,21 @@ def main():
     n_tokens = N_BATCH * ROWS
     flop_per_launch = 2.0 * n_tokens * K_IN * K_IN          # the full GEMM the reference executes
     wide = args.x_dtype == "float32"
-    # the kernels compute the upper tiles only: 128 x 128 (fp32 rows), 256 x 256 (16-bit rows, K >= 1024)
-    tile_edge = 128 if (wide or K_IN < 1024) else 256
+    # the kernels compute the upper tiles only: 256 x 256 from K = 1024 on, 128 x 128 below
+    tile_edge = 128 if K_IN < 1024 else 256
     tiles = (K_IN + tile_edge - 1) // tile_edge
     executed_flop = flop_per_launch * (tiles + 1) / (2 * tiles)
     achieved = flop_per_launch / (hess_ms * 1e-3) * 1e-12
     executed = executed_flop / (hess_ms * 1e-3) * 1e-12
     peak = FP32_MFMA_PEAK_TFLOPS if wide else MFMA16_PEAK_TFLOPS
-    roofline = {"kernel": "syrk_kernel<float> (X^T X, fp32 MFMA, upper tiles)" if wide else
+    roofline = {"kernel": "syrk32d_kernel (fp32 X^T X, fp32 MFMA, upper 256 x 256 tiles)" if wide else
                           f"syrk16d_kernel ({args.x_dtype} X^T X, 16-bit MFMA with fp32 accumulation, upper tiles)",
                 "bound": "mfma",
                 "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
                 "frac": round(achieved / peak, 4),
                 # bytes per launch beyond L2 from rocprofv3 FETCH_SIZE + WRITE_SIZE (scaled by what the
                 # counters read for a 1 GiB copy: x2.000 / x1.000), summary kept under profiles/
-                "traffic": 5.71e10 if wide else 1.06e10,
+                "traffic": 1.74e10 if wide else 1.06e10,
                 "flop_per_launch": flop_per_launch, "avg_launch_ms": round(hess_ms, 4),
                 "launches_per_step": 1,
                 "executed_tflops": round(executed, 2),

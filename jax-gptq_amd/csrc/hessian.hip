@@ -995,6 +995,211 @@ __global__ __launch_bounds__(256) void syrk16d_kernel(ARGS p) {
   }
 }
 
+// ---------------------------------------------------------------------------- fp32 inputs, loads straight into LDS
+// The fp32 counterpart of syrk16d_kernel for the regular case (K a multiple of 256, every batch a
+// multiple of 16 rows, 16-byte aligned): 256 x 256 tiles, four wavefronts with 128 x 128 each (16
+// accumulator tiles of v_mfma_f32_32x32x2_f32 = 256 registers), slabs of 16 rows, four slab
+// buffers.  A row of a 256-feature panel is 1 KB, i.e. exactly one global_load_lds_dwordx4 of a
+// wavefront; LDS keeps the rows as they are in memory ([k][feature], 1 KB + 128 B apart so that
+// the two rows of an MFMA's k pair fall on different banks), which is the operand order of this
+// MFMA: lane l reads feature l % 32 of row 2 kp + l / 32 with one ds_read_b32.  Against the
+// 128 x 128-tile kernel at the top of this file: a quarter of the barriers and half of the LDS
+// operand reads per MFMA, no staging registers, no LDS writes.
+//
+// Per slab and wavefront: 8 k pairs x 16 MFMAs (64 cycles each), 8 loads, 64 operand reads; the
+// order is fixed by hand as in syrk16d_kernel: before the MFMAs of k pair kp one load of a later
+// slab and the operand reads of k pair kp + 1 are issued.  The loop is skewed by one k pair: a
+// step starts with the last k pair of the previous slab out of registers, so that the first
+// reads after a barrier have 16 MFMAs in front of their first use.
+constexpr int D32_BK = 16;
+constexpr int D32_NBUF = 4;
+constexpr int D32_ROW = 1024 + 128;
+constexpr int D32_OP = D32_BK * D32_ROW;
+constexpr int D32_SLAB = 2 * D32_OP;
+constexpr int D32_LDS_BYTES = D32_NBUF * D32_SLAB;
+
+__global__ __launch_bounds__(256) void syrk32d_kernel(SyrkArgs p) {
+  extern __shared__ __attribute__((aligned(16))) char lds32d[];
+  typedef __attribute__((address_space(3))) char lds_char;
+  const int ntiles = p.T * (p.T + 1) / 2;
+  unsigned item = blockIdx.x;
+  {
+    const unsigned full = gridDim.x & ~255u;
+    if (item < full) {
+      const unsigned xcd = item & 7u, q = item >> 3;
+      item = ((q >> 5) * 8u + xcd) * 32u + (q & 31u);
+    }
+  }
+  const int rs = (int)item / ntiles, t = (int)item - rs * ntiles;
+  int ti, tj;
+  tile_decode(t, p.T, ti, tj);
+  const int m0 = ti * W16_TB, n0 = tj * W16_TB, K = p.K;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
+
+  // slice [g0, g0 + chunk) of the concatenated batches: first slab (b, kt), number of slabs
+  int b = 0, kt = 0, nslabs = 0;
+  {
+    const int64_t g0 = (int64_t)rs * p.chunk;
+    int64_t base = 0;
+    bool started = false;
+    int rem = 0;
+    for (int bb = 0; bb < p.nb; ++bb) {
+      const int rows = p.rows[bb];
+      if (!started && g0 < base + rows) {
+        started = true;
+        b = bb;
+        kt = (int)(g0 - base);
+        rem = p.chunk;
+      }
+      if (started && rem > 0) {
+        const int from = (bb == b) ? kt : 0;
+        const int take = min(rows - from, rem);
+        nslabs += take / D32_BK;          // rows, chunk and kt are multiples of D32_BK here
+        rem -= take;
+      }
+      base += rows;
+    }
+  }
+
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_char *)lds32d;
+  // loads: wavefronts 0-1 bring in the ti panel (operand A), 2-3 the tj panel (B); a wavefront
+  // owns 8 rows of its operand, one load each (lane l: features 4 l .. 4 l + 3 of the panel)
+  const int ld_op = wave >> 1, ld_row0 = (wave & 1) * 8;
+  const int ld_feat = (ld_op ? n0 : m0) + lane * 4;
+  const uint32_t ld_dst0 = lds0 + ld_op * D32_OP + ld_row0 * D32_ROW;
+  const float *Xb = reinterpret_cast<const float *>(p.ptr[b]);
+  int rows_b = p.rows[b];
+  int issued = 0;
+  auto next_slab = [&](const float *&src, uint32_t &dst) __attribute__((always_inline)) {
+    src = Xb + (int64_t)(kt + ld_row0) * K + ld_feat;
+    dst = __builtin_amdgcn_readfirstlane(ld_dst0 + (uint32_t)(issued & (D32_NBUF - 1)) * D32_SLAB);
+    ++issued;
+    kt += D32_BK;
+    if (kt >= rows_b && issued < nslabs) {      // rare: next batch
+      ++b;
+      kt = 0;
+      Xb = reinterpret_cast<const float *>(p.ptr[b]);
+      rows_b = p.rows[b];
+    }
+  };
+  auto load_row = [&](const float *src, uint32_t dst, int j) __attribute__((always_inline)) {
+    load_to_lds_16(src + (int64_t)j * K, dst + j * D32_ROW);
+  };
+
+  // operand reads of k pair kp: row 2 kp + lhi, feature (32-feature block) + l32
+  const uint32_t rd_a = (uint32_t)(lhi * D32_ROW + (wm * 128 + l32) * 4);
+  const uint32_t rd_b = (uint32_t)(D32_OP + lhi * D32_ROW + (wn * 128 + l32) * 4);
+  struct Ops { float a[4], b[4]; };
+  auto read_ops = [&](int buf, int kp, Ops &o) __attribute__((always_inline)) {
+    const lds_char *base = (const lds_char *)lds32d + buf * D32_SLAB + kp * 2 * D32_ROW;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      o.a[q] = *reinterpret_cast<const __attribute__((address_space(3))) float *>(base + rd_a + q * 128);
+      o.b[q] = *reinterpret_cast<const __attribute__((address_space(3))) float *>(base + rd_b + q * 128);
+    }
+  };
+
+  floatx16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  auto mfma_all = [&](const Ops &o) __attribute__((always_inline)) {
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[ii][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(o.a[ii], o.b[j], acc[ii][j], 0, 0, 0);
+  };
+  // the last k pair of the previous slab (operands in `prev`), then k pairs 0 .. 6 of the slab in
+  // `buf`; leaves the operands of its k pair 7 in `prev`
+  auto step = [&](Ops &prev, int buf, bool dma, const float *src, uint32_t dst) __attribute__((always_inline)) {
+    Ops cur;
+    read_ops(buf, 0, cur);
+    if (dma) load_row(src, dst, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_all(prev);
+#pragma unroll
+    for (int kp = 0; kp < 7; ++kp) {
+      Ops nxt;
+      read_ops(buf, kp + 1, nxt);
+      if (dma) load_row(src, dst, kp + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_all(cur);
+      __builtin_amdgcn_sched_barrier(0);
+      cur = nxt;
+    }
+    prev = cur;
+  };
+  // own loads of slab s done (`later` slabs of 8 loads each may stay in flight), own LDS reads
+  // done, then the workgroup barrier: slab s is visible, nobody reads the buffer of slab s-1 any more
+  auto publish = [&](int later) __attribute__((always_inline)) {
+    asm volatile("" ::: "memory");
+    if (later >= 2) __builtin_amdgcn_s_waitcnt(0x4070);        // vmcnt(16) lgkmcnt(0)
+    else if (later == 1) __builtin_amdgcn_s_waitcnt(0x0078);   // vmcnt(8) lgkmcnt(0)
+    else __builtin_amdgcn_s_waitcnt(0x0070);                   // vmcnt(0) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+
+  if (nslabs > 0) {
+    for (int s = 0; s < D32_NBUF - 1 && s < nslabs; ++s) {
+      const float *src;
+      uint32_t dst;
+      next_slab(src, dst);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) load_row(src, dst, j);
+    }
+    Ops prev;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) prev.a[q] = prev.b[q] = 0.f;   // "slab -1": adds zeros
+    int s = 0;
+    // steady state: slab s + 3 is loaded during step s, two later slabs (16 loads) stay in flight
+    for (; s + D32_NBUF - 1 < nslabs; ++s) {
+      const float *src;
+      uint32_t dst;
+      next_slab(src, dst);
+      publish(2);
+      step(prev, s & (D32_NBUF - 1), true, src, dst);
+    }
+    for (; s < nslabs; ++s) {
+      publish(nslabs - 1 - s);
+      step(prev, s & (D32_NBUF - 1), false, nullptr, 0u);
+    }
+    mfma_all(prev);          // last k pair of the last slab
+  }
+
+  if (p.RS == 1) {
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int col = n0 + wn * 128 + j * 32 + l32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = m0 + wm * 128 + ii * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+          p.H[(int64_t)row * K + col] += acc[ii][j][r];
+        }
+      }
+  } else {
+    float *dst = p.ws + ((int64_t)rs * ntiles + t) * (W16_TB * W16_TB);
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int col = wn * 128 + j * 32 + l32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = wm * 128 + ii * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+          dst[row * W16_TB + col] = acc[ii][j][r];
+        }
+      }
+  }
+}
+
 // H tile += unit * sum over the row slices, in slice order (unit: device scalar, 1 if null)
 template <int TB>
 __global__ __launch_bounds__(256) void syrk_reduce_kernel(float *H, const float *ws, int K, int T,
@@ -1324,6 +1529,34 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
       if (a.RS > 1) {
         hipLaunchKernelGGL(syrk_reduce_kernel<HB>, dim3((unsigned)ntiles), dim3(256), 0, st, H, a.ws,
                            (int)K, T, a.RS, (const float *)nullptr);
+        GPTQ_CHECK_LAUNCH();
+      }
+      continue;
+    }
+    // fp32 batches, regular shapes from K = 1024 on: 256 x 256 tiles, loads straight into LDS
+    bool wide32 = x_dtype == GPTQ_HIP_F32 && use_wide16(K) && K % W16_TB == 0;
+    for (int i = 0; i < a.nb && wide32; ++i)
+      wide32 = (a.rows[i] % D32_BK == 0) && ((reinterpret_cast<uintptr_t>(a.ptr[i]) & 15) == 0);
+    if (wide32) {
+      int64_t total_rows = 0;
+      for (int i = 0; i < a.nb; ++i) total_rows += a.rows[i];
+      SyrkArgs w = a;
+      w.T = (int)(K / W16_TB);
+      const int64_t nt = (int64_t)w.T * (w.T + 1) / 2;
+      w.RS = pick_rs_wide(K);
+      const int64_t slabs = total_rows / D32_BK;
+      if (w.RS > slabs) w.RS = (int)(slabs > 0 ? slabs : 1);
+      const int64_t chunk = round_up64(ceil_div64(total_rows, w.RS), D32_BK);
+      if (chunk > 2147483647LL) return GPTQ_HIP_EINVAL;
+      w.chunk = (int)chunk;
+      if (hipFuncSetAttribute(reinterpret_cast<const void *>(syrk32d_kernel),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, D32_LDS_BYTES) != hipSuccess)
+        return GPTQ_HIP_ELAUNCH;
+      hipLaunchKernelGGL(syrk32d_kernel, dim3((unsigned)(nt * w.RS)), block, D32_LDS_BYTES, st, w);
+      GPTQ_CHECK_LAUNCH();
+      if (w.RS > 1) {
+        hipLaunchKernelGGL(syrk_reduce_kernel<W16_TB>, dim3((unsigned)nt), dim3(256), 0, st, H, w.ws,
+                           (int)K, w.T, w.RS, (const float *)nullptr);
         GPTQ_CHECK_LAUNCH();
       }
       continue;

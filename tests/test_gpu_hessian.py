@@ -207,3 +207,24 @@ def test_accumulate_H_split_fp16_empty_and_3d_batches(G):
     assert np.abs(Hs - to_np(G.accumulate_H(xs))).max() < 2 * TOL * np.abs(ref).max()
     xs[0][3, 7] = np.inf
     assert not np.isfinite(to_np(G.accumulate_H(xs, split_fp16=True))).all()
+
+
+@pytest.mark.parametrize("rows,K,nb", [(48, 1024, 5), (2048, 1280, 2), (16, 2048, 3), (4096, 1024, 1), (272, 1536, 7)])
+def test_accumulate_H_fp32_wide_tile_kernel(G, rows, K, nb):
+    """fp32 rows with K a multiple of 256 (from 1024 on) and batches of a multiple of 16 rows run the
+    256 x 256-tile kernel that loads straight into LDS; same bars as the 128 x 128-tile kernel, and
+    a batch list that breaks the row rule (one batch of 40 rows) takes that kernel and agrees."""
+    rng = np.random.default_rng(rows + K + nb)
+    xs = [rng.standard_normal((rows, K)).astype(np.float32) for _ in range(nb)]
+    for x in xs:
+        x[:, 7] = 0.0
+    H = to_np(G.accumulate_H(xs))
+    ref = _closed_form(xs)
+    assert H.shape == (K, K) and np.array_equal(H, H.T)
+    assert np.abs(H - ref).max() < TOL * max(1.0, np.abs(ref).max())
+    assert np.all(H[7] == 0) and np.all(H[:, 7] == 0)
+    ragged = xs + [rng.standard_normal((40, K)).astype(np.float32)]
+    ragged[-1][:, 7] = 0.0
+    H2 = to_np(G.accumulate_H(ragged))
+    ref2 = _closed_form(ragged)
+    assert np.abs(H2 - ref2).max() < TOL * max(1.0, np.abs(ref2).max())
