@@ -15,7 +15,8 @@
  *     allocation.  Scratch memory is passed in by the caller (`ws`, `ws_bytes`);
  *     the matching `*_workspace_bytes` query gives the required size;
  *   - return value 0 means success, otherwise a GPTQ_HIP_E* code; nothing throws.
- *   - thread-safe; no mutable global state.
+ *   - thread-safe; no mutable global state (gptq_hip_qmatmul_static, at the end of this
+ *     file, is the one exception: its calls share a fixed array per GPU).
  */
 #ifndef GPTQ_HIP_H_
 #define GPTQ_HIP_H_
@@ -38,7 +39,8 @@ enum {
   GPTQ_HIP_EINVAL = 1,      /* bad shape / null pointer / unsupported block size */
   GPTQ_HIP_EDTYPE = 2,      /* unsupported element type */
   GPTQ_HIP_EWORKSPACE = 3,  /* workspace too small */
-  GPTQ_HIP_ELAUNCH = 4      /* the HIP runtime refused a launch */
+  GPTQ_HIP_ELAUNCH = 4,     /* the HIP runtime refused a launch */
+  GPTQ_HIP_ETOOBIG = 5      /* the problem needs more than the fixed scratch of gptq_hip_qmatmul_static */
 };
 
 int gptq_hip_abi_version(void);
@@ -186,6 +188,23 @@ size_t gptq_hip_qmatmul_workspace_bytes_x(int64_t M, int64_t R, int64_t C, int t
 int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
                      int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype,
                      int transpose_b, void *out, void *ws, size_t ws_bytes);
+
+/* ---- packed-int4 matmul that allocates nothing and takes no workspace ----------------------
+ * No counterpart in the reference.  For callers that cannot allocate device memory: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same operation,
+ * arguments and results as gptq_hip_qmatmul; the workspace is a fixed array of
+ * GPTQ_HIP_QMATMUL_STATIC_BYTES bytes of device memory inside the library (one copy per GPU,
+ * held until the process ends), so the call makes no hipMalloc / hipFree and calls no allocating
+ * routine.  A problem whose gptq_hip_qmatmul_workspace_bytes_x(M, R, C, transpose_b, x_dtype)
+ * exceeds GPTQ_HIP_QMATMUL_STATIC_BYTES is refused with GPTQ_HIP_ETOOBIG and nothing is enqueued.
+ * All calls on one GPU share the one array: calls that may overlap in time on a GPU (different
+ * streams, different threads) race on it; serialise them or use gptq_hip_qmatmul with a workspace
+ * per stream.  The first call on a device looks up the array's address and clears its arrival
+ * counters with a small kernel on `stream`. */
+#define GPTQ_HIP_QMATMUL_STATIC_BYTES ((size_t)32 << 20)
+int gptq_hip_qmatmul_static(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
+                            int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype,
+                            int transpose_b, void *out);
 
 #ifdef __cplusplus
 }

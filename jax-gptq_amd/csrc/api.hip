@@ -12,6 +12,7 @@ const char *gptq_hip_error_string(int code) {
     case GPTQ_HIP_EDTYPE: return "unsupported element type";
     case GPTQ_HIP_EWORKSPACE: return "workspace missing or too small";
     case GPTQ_HIP_ELAUNCH: return "HIP launch failed";
+    case GPTQ_HIP_ETOOBIG: return "problem needs more scratch than the call that allocates nothing holds";
     default: return "unknown error";
   }
 }

@@ -1,5 +1,6 @@
 // Packed-int4 matmul: out = x @ dequant(Wpacked)  (and the transposed form).
 #include "common.h"
+#include <mutex>
 #include <type_traits>
 
 namespace {
@@ -1526,6 +1527,70 @@ int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const 
     default:
       return GPTQ_HIP_EDTYPE;
   }
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------- the call that allocates nothing
+// gptq_hip_qmatmul_static is gptq_hip_qmatmul with the workspace (arrival counters, split-K
+// partials, fp16 staging of fp32 activations) taken from a fixed array in device memory instead of
+// a caller's buffer, for callers that cannot allocate: code under graph capture, serving loops,
+// harnesses that forbid hipMalloc.  Every GPU the library runs on holds its own copy of the array
+// until the process ends.  In host code the array's name is only a stand-in: the address a kernel
+// may use is the one hipGetSymbolAddress returns with that device current, looked up once per
+// device below and used for everything the host does with the memory.
+constexpr size_t QMM_STATIC_BYTES = GPTQ_HIP_QMATMUL_STATIC_BYTES;
+static __device__ __align__(256) unsigned char scratch[QMM_STATIC_BYTES];
+
+namespace {
+
+constexpr int QMM_STATIC_MAX_DEVICES = 64;
+std::mutex g_static_mutex;
+void *g_static_ptr[QMM_STATIC_MAX_DEVICES] = {};
+
+__global__ __launch_bounds__(256) void qmm_static_clear_kernel(uint32_t *p, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
+// Address of the current device's copy of the array; on the first call on a device also clears the
+// arrival counters at its start (a fill kernel on the caller's stream, ahead of the product).
+int qmm_static_base(hipStream_t st, void **base) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= QMM_STATIC_MAX_DEVICES) return GPTQ_HIP_EINVAL;
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  if (!g_static_ptr[dev]) {
+    void *ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+      (void)hipGetLastError();
+      return GPTQ_HIP_ELAUNCH;
+    }
+    const int words = QMM_COUNTER_BYTES / 4;
+    hipLaunchKernelGGL(qmm_static_clear_kernel, dim3((words + 255) / 256), dim3(256), 0, st,
+                       reinterpret_cast<uint32_t *>(ptr), words);
+    GPTQ_CHECK_LAUNCH();
+    g_static_ptr[dev] = ptr;
+  }
+  *base = g_static_ptr[dev];
+  return GPTQ_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int gptq_hip_qmatmul_static(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
+                            int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype,
+                            int transpose_b, void *out) {
+  if (M < 0 || R <= 0 || C <= 0) return GPTQ_HIP_EINVAL;
+  if (M == 0) return GPTQ_HIP_OK;
+  if (gptq_hip_qmatmul_workspace_bytes_x(M, R, C, transpose_b, x_dtype) > QMM_STATIC_BYTES)
+    return GPTQ_HIP_ETOOBIG;
+  void *base = nullptr;
+  const int rc = qmm_static_base(as_stream(stream), &base);
+  if (rc) return rc;
+  return gptq_hip_qmatmul(stream, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out,
+                          base, QMM_STATIC_BYTES);
 }
 
 }  // extern "C"

@@ -11,7 +11,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("GPTQ_HIP_LIBRARY") or os.path.join(HERE, "libgptq_hip.so")
 
 F32, F16, BF16, F64 = 0, 1, 2, 3
-OK, EINVAL, EDTYPE, EWORKSPACE, ELAUNCH = 0, 1, 2, 3, 4
+OK, EINVAL, EDTYPE, EWORKSPACE, ELAUNCH, ETOOBIG = 0, 1, 2, 3, 4, 5
+QMATMUL_STATIC_BYTES = 32 << 20
 
 _vp, _i64, _i32, _f32, _f64, _sz = (ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float,
                                    ctypes.c_double, ctypes.c_size_t)
@@ -43,6 +44,7 @@ SIGNATURES = {
     "gptq_hip_qmatmul_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
     "gptq_hip_qmatmul_workspace_bytes_x": (_sz, [_i64, _i64, _i64, _i32, _i32]),
     "gptq_hip_qmatmul": (_i32, [_vp, _vp, _i32, _i64, _vp, _i64, _i64, _vp, _vp, _i32, _i32, _vp, _vp, _sz]),
+    "gptq_hip_qmatmul_static": (_i32, [_vp, _vp, _i32, _i64, _vp, _i64, _i64, _vp, _vp, _i32, _i32, _vp]),
 }
 
 _lib = None
