@@ -1228,6 +1228,9 @@ __global__ __launch_bounds__(256) void syrk_reduce_kernel(float *H, const float 
   }
 }
 
+// rows per row slice and launch (a multiple of 64, so that a cut batch keeps full slabs)
+constexpr int64_t H_CHAIN_ROWS = 32768;
+
 int pick_rs(int64_t K) {
   const int64_t T = ceil_div64(K, HB), ntiles = T * (T + 1) / 2;
   int64_t rs = ceil_div64(6144, ntiles);   // about eight waves of workgroups over 768 slots
@@ -1438,22 +1441,39 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
   if (need && (!ws || ws_bytes < need)) return GPTQ_HIP_EWORKSPACE;
   const int T = (int)ceil_div64(K, HB);
   const int ntiles = T * (T + 1) / 2;
+  // One launch sums its rows in registers, one chain of MFMA accumulations per row slice.  The
+  // matrix instructions align their addends to the running sum with a few guard bits and drop
+  // what falls below them, which biases a long sum of squares (the diagonal of H) low: measured
+  // 5.5e-5 relative after 262144 rows in one chain, 4e-6 after 20000.  So a launch gets at most
+  // H_CHAIN_ROWS rows per slice; longer calibration sets (and longer single batches) are cut
+  // into several launches that add into H, as the reference adds batch by batch (gptq.py:97-98).
+  const int rs_k = (use_wide16(K) && x_dtype != GPTQ_HIP_F64) ? pick_rs_wide(K) : pick_rs(K);
+  const int64_t launch_rows = (int64_t)H_CHAIN_ROWS * rs_k;
   int b0 = 0;
+  int64_t off = 0;                 // rows of batch b0 already handed to a launch
+  const size_t x_elem = dtype_size(x_dtype);
   while (b0 < n_batches) {
     SyrkArgs a;
     a.nb = 0;
-    int64_t max_rows = 0;
-    while (b0 < n_batches && a.nb < H_NBMAX) {
+    int64_t max_rows = 0, sum_rows = 0;
+    while (b0 < n_batches && a.nb < H_NBMAX && sum_rows < launch_rows) {
       const int64_t rows = x_rows[b0];
       if (rows < 0 || rows > 2147483647LL) return GPTQ_HIP_EINVAL;
-      if (rows > 0) {
+      if (rows - off > 0) {
         if (!x_ptrs[b0]) return GPTQ_HIP_EINVAL;
-        a.ptr[a.nb] = x_ptrs[b0];
-        a.rows[a.nb] = (int)rows;
+        int64_t take = rows - off;
+        if (take > launch_rows - sum_rows) take = launch_rows - sum_rows;     // a multiple of 64 rows
+        a.ptr[a.nb] = reinterpret_cast<const char *>(x_ptrs[b0]) + (size_t)off * (size_t)K * x_elem;
+        a.rows[a.nb] = (int)take;
         ++a.nb;
-        if (rows > max_rows) max_rows = rows;
+        sum_rows += take;
+        if (take > max_rows) max_rows = take;
+        off += take;
       }
-      ++b0;
+      if (off >= rows) {
+        ++b0;
+        off = 0;
+      }
     }
     if (a.nb == 0) continue;
     a.K = (int)K;

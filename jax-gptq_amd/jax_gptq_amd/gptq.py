@@ -174,15 +174,25 @@ _MAX_BATCHES_PER_CALL = 1024
 def _accumulate_H_step(H, running_mean, n_samples, batch):
     """One batch of the Hessian accumulation (reference ``gptq.py:57-74``).
 
-    The state differs from the reference's in representation, not in meaning: ``H``
-    carries the raw second-moment sum (upper 128x128 tiles) and ``running_mean`` stays
-    zero, so that the reference's closing formula ``H / n + outer(mean, mean)`` still
-    yields ``sum X^T X / n``.
+    The state differs from the reference's in representation, not in meaning: ``H`` carries the
+    raw second-moment sum ``sum_b X_b^T X_b`` as a full symmetric matrix and ``running_mean`` stays
+    zero, so that the reference's closing formula ``H / n + outer(mean, mean)`` (``gptq.py:100-101``)
+    yields ``sum X^T X / n``, the matrix ``accumulate_H`` returns.  The kernel adds to the upper
+    tiles; the mirror into the lower triangle is redone after every step, so ``H`` is a valid
+    state whenever the caller looks at it.
     """
+    lib = N.load()
     batch = _float_dev(batch, keep_fp64=(H.dtype == torch.float64))
     if batch.dim() > 2:
         batch = batch.reshape(-1, batch.shape[-1])
-    _hessian_accumulate(H, [batch.contiguous()])
+    elif batch.dim() == 1:
+        batch = batch.reshape(1, -1)
+    if batch.shape[-1] != H.shape[0]:
+        raise ValueError("the batch and H disagree on the feature dimension")
+    if batch.shape[0] > 0:
+        _hessian_accumulate(H, [batch.contiguous()])
+        N.check(lib.gptq_hip_hessian_finalize(_stream(), _ptr(H), _DT_H[H.dtype], H.shape[0], 1.0),
+                "hessian_finalize")
     return H, running_mean, n_samples + batch.shape[0]
 
 

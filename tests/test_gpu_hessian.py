@@ -228,3 +228,113 @@ def test_accumulate_H_fp32_wide_tile_kernel(G, rows, K, nb):
     H2 = to_np(G.accumulate_H(ragged))
     ref2 = _closed_form(ragged)
     assert np.abs(H2 - ref2).max() < TOL * max(1.0, np.abs(ref2).max())
+
+
+@pytest.mark.parametrize("rows,K,nb,dt", [(64, 384, 5, "float32"), (37, 200, 4, "float32"), (256, 1024, 6, "float32"),
+                                          (2048, 4096, 3, "float32"), (96, 1280, 4, "float16"),
+                                          (50, 520, 3, "bfloat16")])
+def test_accumulate_H_step_chain_equals_accumulate_H(G, rows, K, nb, dt):
+    """The reference's streaming use (gptq.py:97-101): one `_accumulate_H_step` per batch, then the
+    closing formula H / n + outer(mean, mean).  After every step the state must be a full symmetric
+    matrix (K > one tile: the kernels add to the upper tiles only), the closed state must equal
+    what `accumulate_H` returns for the list, and the factor computed from it the one-shot factor."""
+    import torch
+    rng = np.random.default_rng(rows + K + nb)
+    tdt = getattr(torch, dt)
+    xs = [torch.from_numpy(rng.standard_normal((rows, K)).astype(np.float32)).to(tdt).cuda() for _ in range(nb)]
+    H = torch.zeros((K, K), dtype=torch.float32, device="cuda")
+    mean = torch.zeros(K, dtype=torch.float32, device="cuda")
+    n = 0
+    seen = []
+    for x in xs:
+        H, mean, n = G._accumulate_H_step(H, mean, n, x)
+        seen.append(x.float().cpu().numpy())
+        part = np.concatenate(seen)
+        raw = part.astype(np.float64).T @ part.astype(np.float64)
+        Hn = to_np(H)
+        assert np.array_equal(Hn, Hn.T), "the state is not symmetric after a step"
+        assert np.abs(Hn - raw).max() < TOL * max(1.0, np.abs(raw).max())
+    assert n == rows * nb
+    closed = H / n + torch.outer(mean, mean)          # gptq.py:100-101
+    one_shot = G.accumulate_H(xs)
+    ref = _closed_form([x.float().cpu().numpy() for x in xs])
+    assert np.abs(to_np(closed) - ref).max() < TOL * max(1.0, np.abs(ref).max())
+    assert np.abs(to_np(closed) - to_np(one_shot)).max() < TOL * max(1.0, np.abs(ref).max())
+    if rows * nb >= K:
+        # the streamed matrix is as good an input to the factorisation as the one-shot matrix
+        _, L1, bad1 = G._damp_and_invert(torch.zeros((K, 8), device="cuda"), closed.clone(), 0.01)
+        _, L2, bad2 = G._damp_and_invert(torch.zeros((K, 8), device="cuda"), one_shot.clone(), 0.01)
+        assert not bad1 and not bad2
+        assert float((L1 - L2).abs().max()) < 1e-3 * float(L2.abs().max())
+
+
+def test_accumulate_H_step_takes_3d_and_empty_batches(G):
+    import torch
+    rng = np.random.default_rng(5)
+    K = 256
+    a = rng.standard_normal((3, 11, K)).astype(np.float32)
+    H = torch.zeros((K, K), dtype=torch.float32, device="cuda")
+    H, m, n = G._accumulate_H_step(H, torch.zeros(K, device="cuda"), 0, a)
+    H, m, n = G._accumulate_H_step(H, m, n, np.zeros((0, K), np.float32))
+    assert n == 33
+    flat = a.reshape(-1, K).astype(np.float64)
+    assert np.abs(to_np(H) - flat.T @ flat).max() < TOL * np.abs(flat.T @ flat).max()
+    with pytest.raises(ValueError):
+        G._accumulate_H_step(H, m, n, np.zeros((4, K + 1), np.float32))
+
+
+@pytest.mark.parametrize("nb,rows,K", [(300, 16, 256), (1100, 4, 136), (260, 32, 1024)])
+def test_accumulate_H_long_batch_lists(G, nb, rows, K):
+    """More batches than one launch table holds (128) and than one call of the binding passes
+    (1024): the list is cut into several launches that add into the same H."""
+    rng = np.random.default_rng(nb)
+    xs = [rng.standard_normal((rows, K)).astype(np.float32) for _ in range(nb)]
+    H = to_np(G.accumulate_H(xs))
+    ref = _closed_form(xs)
+    assert np.array_equal(H, H.T)
+    assert np.abs(H - ref).max() < TOL * max(1.0, np.abs(ref).max())
+
+
+def test_accumulate_H_mixed_dtype_batch_list(G):
+    """fp32, fp16 and bf16 batches in one list (one launch table holds one element type, so the
+    binding falls back to a launch per batch); the closed form is taken of the values as stored."""
+    import torch
+    rng = np.random.default_rng(31)
+    K = 1024
+    dts = [torch.float32, torch.float16, torch.float32, torch.bfloat16, torch.float16]
+    xs = [torch.from_numpy(rng.standard_normal((64 + 32 * i, K)).astype(np.float32)).to(dt).cuda()
+          for i, dt in enumerate(dts)]
+    H = to_np(G.accumulate_H(xs))
+    ref = _closed_form([x.float().cpu().numpy() for x in xs])
+    assert np.array_equal(H, H.T)
+    assert np.abs(H - ref).max() < TOL * max(1.0, np.abs(ref).max())
+
+
+def test_accumulate_H_full_calibration_set_of_the_benchmark_layer(G):
+    """The launch the benchmark times: 128 batches of [2048, 4096] fp32 rows (262144 tokens, the
+    full 128-entry pointer table, every row slice) against a double-precision product of the same
+    rows formed on the device batch by batch (test-only: torch's fp64 matmul)."""
+    import torch
+    g = torch.Generator(device="cuda")
+    g.manual_seed(4096)
+    K, nb, rows = 4096, 128, 2048
+    xs = [torch.randn((rows, K), generator=g, device="cuda") for _ in range(nb)]
+    H = G.accumulate_H(xs)
+    ref = torch.zeros((K, K), dtype=torch.float64, device="cuda")
+    for x in xs:
+        xd = x.double()
+        ref.addmm_(xd.T, xd)
+    ref /= nb * rows
+    assert bool((H == H.T).all())
+    top = float(ref.abs().max())
+    assert float((H.double() - ref).abs().max()) < TOL * max(1.0, top)
+    # fp16 copies of the same rows on the 16-bit kernel, against the product of the rounded rows
+    xs16 = [x.to(torch.float16) for x in xs]
+    del xs
+    H16 = G.accumulate_H(xs16)
+    ref.zero_()
+    for x in xs16:
+        xd = x.double()
+        ref.addmm_(xd.T, xd)
+    ref /= nb * rows
+    assert float((H16.double() - ref).abs().max()) < TOL * max(1.0, top)

@@ -454,3 +454,63 @@ def test_llama7b_shaped_decoder_block(T, J):
     # (4-bit codes of Gaussian weights: ~0.28 relative, measured; round-to-nearest gives the same order)
     assert float(((out - batches[0]).float() - dref).norm() / dref.norm()) < 0.35
     assert float((out_k.float() - out.float()).norm() / out.float().norm()) < 5e-3
+
+
+def test_three_layer_chain_against_the_oracle_chain(T, J):
+    """`quantize` over three fp32 linear layers against the same chain run by the CPU oracle:
+    layer 0 sees identical inputs on both sides, so its codes must match to the solve's bar
+    (>= 99.9 % equal, the rest off by one); later layers are calibrated on what the (nearly
+    identical) quantised layers before them produce, so they are compared through their layer
+    reconstruction error, within 1 % of the oracle's."""
+    from helpers import code_stats, recon_error
+    from oracle import gptq_oracle as O
+    G = J.gptq
+    dims = [256, 512, 384, 320]
+    rng = np.random.default_rng(42)
+    Ws = [(rng.standard_normal((dims[i], dims[i + 1])) / np.sqrt(dims[i])).astype(np.float32) for i in range(3)]
+    xs = [rng.standard_normal((64, 256)).astype(np.float32) for _ in range(16)]
+    params = {f"l{i}": T.from_numpy(Ws[i].copy()).cuda() for i in range(3)}
+
+    def f(p, x):
+        for i in range(3):
+            x = x @ p[f"l{i}"]
+        return x
+
+    qp = J.quantize(f, params, [T.from_numpy(x).cuda() for x in xs])
+    acts = list(xs)                      # the oracle's chain, fed by its own quantised layers
+    for i in range(3):
+        Qr, pr = O.gptq(Ws[i], acts)
+        got = qp[f"l{i}"]
+        Qg = to_np(G.unpack_matrix(got))
+        assert np.allclose(to_np(got.scale), pr["scale"], rtol=1e-5) and np.allclose(to_np(got.zero), pr["zero"], rtol=1e-5)
+        X = np.concatenate(acts)
+        e, er = recon_error(Ws[i], Qg, X), recon_error(Ws[i], Qr, X)
+        assert abs(e - er) <= 0.01 * er, (i, e, er)
+        if i == 0:
+            frac, mx = code_stats(to_np(G.unpack_colwise(got.int_weight)), O.codes_from_q(Qr, pr))
+            assert frac <= 1e-3 and mx <= 1, (frac, mx)
+        acts = [a @ Qr for a in acts]
+
+
+def test_shape_helpers_of_utils(T, J):
+    """reference utils.py:6-21: a QuantizedMatrix maps to an abstract array of its logical shape and
+    of zero's dtype, anything else maps to itself, containers keep their structure."""
+    from jax_gptq_amd import utils as U
+    G = J.gptq
+    qm = G.QuantizedMatrix(T.zeros((64, 48), dtype=T.uint8, device="cuda"), T.zeros(48, dtype=T.float16, device="cuda"),
+                           T.ones(48, dtype=T.float16, device="cuda"), contraction_axis=0)
+    a = U._shape_from_param(qm)
+    assert tuple(a.shape) == (128, 48) and a.dtype == T.float16 and a.device.type == "meta"
+    qm1 = G.QuantizedMatrix(T.zeros((5, 30, 7), dtype=T.uint8, device="cuda"), T.zeros((5, 7), device="cuda"),
+                            T.ones((5, 7), device="cuda"), contraction_axis=1)
+    assert tuple(U._shape_from_param(qm1).shape) == (5, 60, 7) and U._shape_from_param(qm1).dtype == T.float32
+    assert tuple(G.quant_matrix_shape(qm1)) == (5, 60, 7) and tuple(qm1.shape) == (5, 60, 7)
+    plain = T.ones(3, device="cuda")
+    assert U._shape_from_param(plain) is plain
+    tree = {"a": qm, "b": [plain, (qm1, 4)], "c": None}
+    out = U.quantized_params_to_shaped_arrays(tree)
+    assert set(out) == {"a", "b", "c"} and out["c"] is None
+    assert tuple(out["a"].shape) == (128, 48)
+    assert isinstance(out["b"], list) and out["b"][0] is plain
+    assert isinstance(out["b"][1], tuple) and tuple(out["b"][1][0].shape) == (5, 60, 7) and out["b"][1][1] == 4
+    assert tuple(U.quantized_params_to_shaped_arrays(qm).shape) == (128, 48)

@@ -16,6 +16,11 @@ SHAPES = [
     (11008, 4096, 4),    # LLaMA-7B down projection
     (7168, 28672, 2),    # OPT-30B fc1
     (28672, 7168, 16),   # OPT-30B fc2: H is 28672^2 fp32 (rows >= K keeps H well conditioned)
+    # the configurations' full calibration sets: 128 batches of 2048 rows (262144 tokens)
+    (4096, 11008, 128),
+    (11008, 4096, 128),
+    (7168, 28672, 128),
+    (28672, 7168, 128),  # 30 GB of calibration rows resident
 ]
 
 
@@ -34,6 +39,20 @@ def test_layer_properties(K, N, nb):
     params = G.get_col_quantize_params(W32)
     H = G.accumulate_H(xs)
     assert bool((H == H.T).all())
+    if nb > 16:
+        # a long calibration set: keep two batches for the checks below; the Hessian's diagonal and
+        # a band of its rows against double-precision sums over ALL rows
+        diag = torch.zeros(K, dtype=torch.float64, device="cuda")
+        band = torch.zeros((64, K), dtype=torch.float64, device="cuda")
+        for x in xs:
+            xd = x.double()
+            diag += (xd * xd).sum(0)
+            band.addmm_(xd[:, K - 64:].T, xd)
+        n = nb * 2048
+        assert float((H.diagonal().double() - diag / n).abs().max()) < 2e-5
+        assert float((H[K - 64:].double() - band / n).abs().max()) < 2e-5
+        del diag, band, xd
+        xs = xs[:2]
     Hd = H.clone()
     Hd.diagonal().add_(0.01 * float(H.diagonal().mean()))
     W32, L, bad = G._damp_and_invert(W32, H, 0.01)
@@ -62,9 +81,49 @@ def test_layer_properties(K, N, nb):
     ref = (X @ Wf).norm()
     e_gptq = float((X @ (Wf - Q.float())).norm() / ref)
     e_rtn = float((X @ (Wf - rtn)).norm() / ref)
-    assert e_gptq < 0.98 * e_rtn, (e_gptq, e_rtn)
+    # (262144 independent N(0, 1) rows make H nearly the identity, where GPTQ is round-to-nearest
+    # plus a small correction: the margin is for the short sets)
+    assert e_gptq < (0.98 if nb <= 16 else 1.0) * e_rtn, (e_gptq, e_rtn)
 
     x16 = X[:40].to(torch.float16)
     y = quantized_matmul(x16, packed).float()
     y_ref = x16.float() @ Q.float()
     assert torch.allclose(y, y_ref, atol=1e-2 * float(y_ref.abs().max()), rtol=1e-3)
+
+
+@pytest.mark.timeout(600)
+@pytest.mark.parametrize("K,N,nb", [(4096, 11008, 8), (11008, 4096, 8)])
+def test_gptq_against_the_oracle_at_the_llama7b_mlp_shapes(K, N, nb):
+    """gptq() against the CPU oracle on the same seeded inputs at the benchmark layer's shape and
+    at the down projection's: fp16 weights, nb batches of 2048 fp32 rows.  Bars as everywhere:
+    scale / zero within 1e-5 relative, at least 99.9 % of the codes equal and the rest off by one,
+    reconstruction error within 1 % of the oracle's, packing bit-exact."""
+    import numpy as np
+    import torch
+    import jax_gptq_amd.gptq as G
+    from helpers import code_stats, to_np
+    from oracle import gptq_oracle as O
+
+    rng = np.random.default_rng(K + N)
+    W = (0.02 * rng.standard_normal((K, N), dtype=np.float32)).astype(np.float16)
+    xs = [rng.standard_normal((2048, K), dtype=np.float32) for _ in range(nb)]
+
+    Q, p = G.gptq(W, xs)
+    packed = G.pack_matrix(Q, p)
+    Q = to_np(Q)
+    Qr, pr = O.gptq(W, xs)
+    assert Q.dtype == W.dtype and Q.shape == W.shape
+    assert np.allclose(to_np(p["scale"]), pr["scale"], rtol=1e-5, atol=0)
+    assert np.allclose(to_np(p["zero"]), pr["zero"], rtol=1e-5, atol=0)
+    c, cr = O.codes_from_q(Q, pr), O.codes_from_q(Qr, pr)
+    frac, mx = code_stats(c, cr)
+    assert frac <= 1e-3, f"{frac:.2e} of the codes differ"
+    assert mx <= 1
+    assert np.array_equal(to_np(packed.int_weight), O.pack_matrix(Q, pr).int_weight)
+    # reconstruction error over the first two batches, in double on the device (test-only)
+    X = torch.from_numpy(np.concatenate(xs[:2])).cuda().double()
+    Wd = torch.from_numpy(W).cuda().double()
+    ref = (X @ Wd).norm()
+    e = float((X @ (Wd - torch.from_numpy(Q).cuda().double())).norm() / ref)
+    er = float((X @ (Wd - torch.from_numpy(Qr).cuda().double())).norm() / ref)
+    assert abs(e - er) <= 0.01 * er, (e, er)

@@ -309,3 +309,21 @@ def test_qmatmul_in_a_captured_graph(OP, M, xdt):
         x.copy_(torch.randn((M, K), device="cuda", generator=g).to(x.dtype))
         eager = OP.quantized_matmul(x, qm).clone()
         torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("xdt", ["float16", "float32"])
+@pytest.mark.parametrize("kind", ["positive", "tiny"])
+@pytest.mark.parametrize("M,N,K", [(1, 11008, 4096), (16, 11008, 4096), (1, 4096, 11008), (16, 4096, 11008),
+                                   (16, 28672, 7168)])
+def test_qmatmul_decode_shapes_with_nonzero_mean_and_tiny_activations(OP, M, N, K, kind, xdt):
+    """Activations that are all positive (|N(0,1)| + 1, as after a GELU / SiLU: any constant the
+    kernel adds to the codes and removes afterwards is multiplied by a large sum of x) and
+    activations of magnitude 1e-3 (anything the kernel scales down inside fp16 would go
+    subnormal), at the decode shapes, against the fp64 dense product at the operator's bar."""
+    qm = _matrix(M + N + K, K, N, np.float16)
+    rng = np.random.default_rng(17)
+    x = rng.standard_normal((M, K))
+    x = (np.abs(x) + 1.0) if kind == "positive" else 1e-3 * x
+    x = x.astype(xdt)
+    got = OP.quantized_matmul(x, qm)
+    _check(got, x.astype(np.float32), qm, False)
