@@ -1200,31 +1200,60 @@ __global__ __launch_bounds__(256) void syrk32d_kernel(SyrkArgs p) {
   }
 }
 
-// H tile += unit * sum over the row slices, in slice order (unit: device scalar, 1 if null)
+// H tile += unit * sum over the row slices, in slice order (unit: device scalar, 1 if null).
+// A tile is cut into RED_PARTS pieces, one workgroup each, and a thread keeps the loads of all its
+// elements of four slices in flight: the reduction reads RS partial copies of the upper triangle,
+// which is HBM traffic worth the bandwidth (one workgroup per tile with one load in flight per
+// thread took 0.47 ms for 13 slices at K = 4096; the bytes need 0.1 ms).
 template <int TB>
 __global__ __launch_bounds__(256) void syrk_reduce_kernel(float *H, const float *ws, int K, int T,
                                                           int RS, const float *unit_ptr) {
+  constexpr int RED_PARTS = TB * TB / 4096;          // 4096 elements = 4 float4 per thread
   const float unit = unit_ptr ? *unit_ptr : 1.f;
   const int ntiles = T * (T + 1) / 2;
-  const int t = blockIdx.x;
+  const int t = blockIdx.x / RED_PARTS, part = blockIdx.x % RED_PARTS;
   int ti, tj;
   tile_decode(t, T, ti, tj);
   const int m0 = ti * TB, n0 = tj * TB;
-  for (int e = threadIdx.x; e < TB * TB / 4; e += 256) {
-    const int row = e / (TB / 4), c4 = (e % (TB / 4)) * 4;
-    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int rs = 0; rs < RS; ++rs) {
-      const float4 v = *reinterpret_cast<const float4 *>(
-          ws + ((int64_t)rs * ntiles + t) * (TB * TB) + row * TB + c4);
-      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
-    }
+  float4 s[4];
+  int e[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    e[u] = part * 1024 + u * 256 + threadIdx.x;      // float4 index inside the tile
+    s[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  const float4 *base = reinterpret_cast<const float4 *>(ws) + (int64_t)t * (TB * TB / 4);
+  const int64_t slice_stride = (int64_t)ntiles * (TB * TB / 4);
+  for (int rs0 = 0; rs0 < RS; rs0 += 4) {
+    float4 v[4][4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        v[q][u] = (rs0 + q < RS) ? base[(int64_t)(rs0 + q) * slice_stride + e[u]] : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        s[u].x += v[q][u].x; s[u].y += v[q][u].y; s[u].z += v[q][u].z; s[u].w += v[q][u].w;
+      }
+  }
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int row = e[u] / (TB / 4), c4 = (e[u] % (TB / 4)) * 4;
     const int gr = m0 + row, gc = n0 + c4;
     if (gr >= K) continue;
     float *dst = H + (int64_t)gr * K + gc;
-    if (gc + 0 < K) dst[0] += s.x * unit;
-    if (gc + 1 < K) dst[1] += s.y * unit;
-    if (gc + 2 < K) dst[2] += s.z * unit;
-    if (gc + 3 < K) dst[3] += s.w * unit;
+    if (gc + 3 < K && (K & 3) == 0) {
+      float4 h = *reinterpret_cast<float4 *>(dst);
+      h.x += s[u].x * unit; h.y += s[u].y * unit; h.z += s[u].z * unit; h.w += s[u].w * unit;
+      *reinterpret_cast<float4 *>(dst) = h;
+    } else {
+      if (gc + 0 < K) dst[0] += s[u].x * unit;
+      if (gc + 1 < K) dst[1] += s[u].y * unit;
+      if (gc + 2 < K) dst[2] += s[u].z * unit;
+      if (gc + 3 < K) dst[3] += s[u].w * unit;
+    }
   }
 }
 
@@ -1255,6 +1284,29 @@ int pick_rs_wide(int64_t K) {
   return best;
 }
 bool use_wide16(int64_t K) { return K >= 1024; }
+
+// Row slices of one launch of a 256 x 256-tile kernel over `total_rows` rows.  pick_rs_wide(K) suits a
+// long calibration set and sizes the workspace; a short call (one batch per call, the reference's
+// streaming use, gptq.py:97-98) pays a fixed cost per round of workgroups (pipeline fill, 64 MB of
+// partial tiles written and read again), so fewer, longer slices win there.  Model fitted to
+// measurements at K = 4096 (2048 rows per call, 1 .. 13 slices, within 5 %):
+//   time = rounds * (us_per_row * rows_per_slice + 30 us),  rounds = ceil(tiles * slices / 256 CUs).
+int pick_rs_call(int64_t K, int64_t total_rows, int slab_rows, double us_per_row) {
+  const int rs_max = pick_rs_wide(K);
+  const int64_t T = ceil_div64(K, W16_TB), ntiles = T * (T + 1) / 2;
+  int best = rs_max;
+  double best_cost = 0.0;
+  for (int rs = rs_max; rs >= 1; --rs) {
+    // fewer workgroups than CUs: each is bound by the latency of its own loads (measured slower
+    // than the model at one slice of 136 tiles)
+    if (ntiles * rs < 256 && rs < rs_max) break;
+    const int64_t rows = round_up64(ceil_div64(total_rows, rs), slab_rows);
+    const double cost = (double)ceil_div64(ntiles * rs, 256) * (us_per_row * (double)rows + 30.0);
+    if (rs == rs_max || cost < 0.97 * best_cost) { best = rs; best_cost = cost; }
+  }
+  return best;
+}
+constexpr double H_US_PER_ROW_F32 = 0.228, H_US_PER_ROW_16 = 0.0305;
 
 // ---------------------------------------------------------------------------- fp32 rows on the 16-bit matrix cores
 // Opt-in path for fp32 calibration rows: x = (hi + lo) * 2^e with hi = fp16(x 2^-e), lo =
@@ -1495,7 +1547,7 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
       SyrkArgs w = a;
       w.T = (int)ceil_div64(K, W16_TB);
       const int64_t nt = (int64_t)w.T * (w.T + 1) / 2;
-      w.RS = pick_rs_wide(K);
+      w.RS = pick_rs_call(K, total_rows, W16_BK, H_US_PER_ROW_16);
       const int64_t slabs = ceil_div64(total_rows, W16_BK);
       if (w.RS > slabs) w.RS = (int)(slabs > 0 ? slabs : 1);
       const int64_t chunk = round_up64(ceil_div64(total_rows, w.RS), W16_BK);
@@ -1523,7 +1575,7 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
         hipLaunchKernelGGL(syrk16w_kernel<__hip_bfloat16>, wgrid, block, lds_bytes, st, w);
       GPTQ_CHECK_LAUNCH();
       if (w.RS > 1) {
-        hipLaunchKernelGGL(syrk_reduce_kernel<W16_TB>, dim3((unsigned)nt), dim3(256), 0, st, H, w.ws,
+        hipLaunchKernelGGL(syrk_reduce_kernel<W16_TB>, dim3((unsigned)(nt * (W16_TB * W16_TB / 4096))), dim3(256), 0, st, H, w.ws,
                            (int)K, w.T, w.RS, (const float *)nullptr);
         GPTQ_CHECK_LAUNCH();
       }
@@ -1547,7 +1599,7 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
         hipLaunchKernelGGL(syrk16_kernel<__hip_bfloat16>, grid, block, S16_LDS_BYTES, st, a);
       GPTQ_CHECK_LAUNCH();
       if (a.RS > 1) {
-        hipLaunchKernelGGL(syrk_reduce_kernel<HB>, dim3((unsigned)ntiles), dim3(256), 0, st, H, a.ws,
+        hipLaunchKernelGGL(syrk_reduce_kernel<HB>, dim3((unsigned)(ntiles * (HB * HB / 4096))), dim3(256), 0, st, H, a.ws,
                            (int)K, T, a.RS, (const float *)nullptr);
         GPTQ_CHECK_LAUNCH();
       }
@@ -1563,7 +1615,7 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
       SyrkArgs w = a;
       w.T = (int)(K / W16_TB);
       const int64_t nt = (int64_t)w.T * (w.T + 1) / 2;
-      w.RS = pick_rs_wide(K);
+      w.RS = pick_rs_call(K, total_rows, D32_BK, H_US_PER_ROW_F32);
       const int64_t slabs = total_rows / D32_BK;
       if (w.RS > slabs) w.RS = (int)(slabs > 0 ? slabs : 1);
       const int64_t chunk = round_up64(ceil_div64(total_rows, w.RS), D32_BK);
@@ -1575,7 +1627,7 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
       hipLaunchKernelGGL(syrk32d_kernel, dim3((unsigned)(nt * w.RS)), block, D32_LDS_BYTES, st, w);
       GPTQ_CHECK_LAUNCH();
       if (w.RS > 1) {
-        hipLaunchKernelGGL(syrk_reduce_kernel<W16_TB>, dim3((unsigned)nt), dim3(256), 0, st, H, w.ws,
+        hipLaunchKernelGGL(syrk_reduce_kernel<W16_TB>, dim3((unsigned)(nt * (W16_TB * W16_TB / 4096))), dim3(256), 0, st, H, w.ws,
                            (int)K, w.T, w.RS, (const float *)nullptr);
         GPTQ_CHECK_LAUNCH();
       }
@@ -1597,7 +1649,7 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
 #undef GPTQ_SYRK_LAUNCH
     GPTQ_CHECK_LAUNCH();
     if (a.RS > 1) {
-      hipLaunchKernelGGL(syrk_reduce_kernel<HB>, dim3((unsigned)ntiles), dim3(256), 0, st, H, a.ws,
+      hipLaunchKernelGGL(syrk_reduce_kernel<HB>, dim3((unsigned)(ntiles * (HB * HB / 4096))), dim3(256), 0, st, H, a.ws,
                          (int)K, T, a.RS, (const float *)nullptr);
       GPTQ_CHECK_LAUNCH();
     }
@@ -1712,7 +1764,7 @@ int gptq_hip_hessian_accumulate_split16(void *stream, const void *const *x_ptrs,
     first = false;
   }
   if (!first && sp.rs > 1) {
-    hipLaunchKernelGGL(syrk_reduce_kernel<W16_TB>, dim3((unsigned)nt), dim3(256), 0, st, H,
+    hipLaunchKernelGGL(syrk_reduce_kernel<W16_TB>, dim3((unsigned)(nt * (W16_TB * W16_TB / 4096))), dim3(256), 0, st, H,
                        reinterpret_cast<const float *>(base), (int)K, sp.T, sp.rs, &sc->unit);
     GPTQ_CHECK_LAUNCH();
   }
