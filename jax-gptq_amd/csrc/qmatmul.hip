@@ -83,24 +83,48 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int QSTRIP = 256;    // channels per workgroup
 
+// LDS layout of one row of a wavefront's partial tile (256 floats): a lane holds the 16 channels
+// 16 l16 + 4 q + j (q, j = 0..3) and stores them as four 16-byte chunks.  Chunk q of lane l16 sits at
+// float offset 64 q + ((4 l16) ^ (16 q)): the sixteen lanes of a lane group then write 256
+// consecutive bytes per chunk (in channel order they would be 64 bytes apart: 4 of 16 banks), and the
+// XOR keeps the reading side, where consecutive threads take consecutive channels, on distinct banks.
+__device__ __forceinline__ int qtile_chunk(int l16, int q) { return 64 * q + ((4 * l16) ^ (16 * q)); }
+__device__ __forceinline__ int qtile_pos(int c) {      // c = channel within the strip
+  const int q = (c >> 2) & 3;
+  return 64 * q + ((((c >> 4) << 2) | (c & 3)) ^ (16 * q));
+}
+
 __device__ __forceinline__ uint32_t u4_comp(const uint4 &v, int w) {
   return w == 0 ? v.x : (w == 1 ? v.y : (w == 2 ? v.z : v.w));
 }
 
+// The masks live in scalar registers and the 16-bit constant in a vector register, all three opaque
+// to the compiler: (p & mask) | c is then one v_and_or_b32 (a VOP3 instruction takes no literal
+// and one scalar operand; from literals the compiler forms v_and_b32 + v_or_b32, ten instead of
+// six vector instructions per MFMA, and the dequantisation is what bounds these kernels' tail).
+struct DqConst { uint32_t mlo, mhi, c; };
 template <bool BF>
-__device__ __forceinline__ void dequant_pair(uint32_t da, uint32_t db, uint32_t sel,
+__device__ __forceinline__ DqConst dq_const() {
+  DqConst k{0x000F000Fu, BF ? 0x000F000Fu : 0x00F000F0u, BF ? 0x43004300u : 0x64006400u};
+  asm volatile("" : "+s"(k.mlo), "+s"(k.mhi));
+  asm volatile("" : "+v"(k.c));
+  return k;
+}
+
+template <bool BF>
+__device__ __forceinline__ void dequant_pair(const DqConst &k, uint32_t da, uint32_t db, uint32_t sel,
                                              uint32_t &lo, uint32_t &hi) {
   // bytes of p: [7:0] = row a, [23:16] = row b.
   const uint32_t p = __builtin_amdgcn_perm(db, da, sel);
   if (BF) {
     // bf16 pairs 128 + code for both nibbles (0x4300 = 128.0; its 7 mantissa bits hold the code)
-    lo = (p & 0x000F000Fu) | 0x43004300u;
-    hi = ((p >> 4) & 0x000F000Fu) | 0x43004300u;
+    lo = (p & k.mlo) | k.c;
+    hi = ((p >> 4) & k.mhi) | k.c;
   } else {
     // fp16 pairs: lo = 1024 + code (even k), hi = 1024 + 16*code (odd k); the offsets and the
     // factor 16 are undone outside the MFMA.
-    lo = (p & 0x000F000Fu) | 0x64006400u;
-    hi = (p & 0x00F000F0u) | 0x64006400u;
+    lo = (p & k.mlo) | k.c;
+    hi = (p & k.mhi) | k.c;
   }
 }
 
@@ -131,17 +155,34 @@ template <> struct Act<__hip_bfloat16> {
 // Workspace layout (only touched when the K range is split over S > 1 workgroups):
 //   [counters: QMM_COUNTER_BYTES, one int32 per (m-chunk, strip), zero between calls; the
 //    size is fixed so that no other region of an earlier call can alias a counter]
+//   [acc64: QMM_ACC_BYTES, see below]
 //   [x1part:  (m-chunk, strip, split, 2, 16) fp32]   [part: (split, M, C) fp32]
 // The last workgroup to finish a strip (atomic ticket) sums the S partials in split order,
 // so the result does not depend on the arrival order, and resets the counter.
 constexpr int QMM_COUNTER_BYTES = 65536;
 constexpr int QMM_MAX_COUNTERS = QMM_COUNTER_BYTES / 4;
+// After the counters: 64-bit accumulators of the decode kernel's split-K sum (M <= 4), one per output,
+// zero between calls like the counters.  Counters and accumulators form the head of every workspace
+// at fixed offsets, whatever the shape, so that calls of different shapes can share one buffer.
+constexpr int QMM_ACC_BYTES = 4 << 20;
+constexpr int QMM_HEAD_BYTES = QMM_COUNTER_BYTES + QMM_ACC_BYTES;
 
 struct QmmWs {
   int32_t *counters;
+  unsigned long long *acc64;
   float *x1part;
   float *part;
 };
+
+__host__ __device__ inline QmmWs qmm_ws(void *base_v, size_t x1_bytes) {
+  char *base = reinterpret_cast<char *>(base_v);
+  QmmWs ws;
+  ws.counters = reinterpret_cast<int32_t *>(base);
+  ws.acc64 = reinterpret_cast<unsigned long long *>(base + QMM_COUNTER_BYTES);
+  ws.x1part = reinterpret_cast<float *>(base + QMM_HEAD_BYTES);
+  ws.part = reinterpret_cast<float *>(base + QMM_HEAD_BYTES + x1_bytes);
+  return ws;
+}
 
 // Cross-wavefront reduction and output of one (m-chunk, strip, split) workgroup.  On entry every
 // wavefront has written its partial tile to red[wave][mrows][QSTRIP]; se / so are this lane's
@@ -175,7 +216,7 @@ __device__ __forceinline__ void qmm_reduce_and_store(float *red, int *s_last_p, 
       const float z = to_f32(zero[n]), sc = to_f32(scale[n]);
       float v = 0.f, e = 0.f, o = 0.f;
       for (int w = 0; w < nw; ++w) {
-        v += red[(w * mrows + m) * QSTRIP + c];
+        v += red[(w * mrows + m) * QSTRIP + qtile_pos(c)];
         e += xs[w * 32 + m];
         o += xs[w * 32 + 16 + m];
       }
@@ -187,7 +228,7 @@ __device__ __forceinline__ void qmm_reduce_and_store(float *red, int *s_last_p, 
     const int m = idx >> 8, c = idx & 255, n = strip * QSTRIP + c;
     if (n >= C) continue;
     float v = 0.f;
-    for (int w = 0; w < nw; ++w) v += red[(w * mrows + m) * QSTRIP + c];
+    for (int w = 0; w < nw; ++w) v += red[(w * mrows + m) * QSTRIP + qtile_pos(c)];
     // agent-scope write-through store: visible to every XCD once it has completed
     __hip_atomic_store(&ws.part[((int64_t)split * M + m0 + m) * C + n], v, __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);
@@ -345,6 +386,7 @@ __global__ __launch_bounds__(SPW == 2 ? 1024 : 512) void qmm_fwd_mfma_kernel(
   so += __shfl_xor(so, 32);
 
   float *slot = red + (size_t)wave * mrows * QSTRIP;
+  const DqConst dqk = dq_const<BF>();
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
     floatx4 acc[8];
@@ -358,8 +400,8 @@ __global__ __launch_bounds__(SPW == 2 ? 1024 : 512) void qmm_fwd_mfma_kernel(
         const int w = t >> 2, tb = t & 3;
         const uint32_t sel = 0x0c000c00u | ((uint32_t)(4 + tb) << 16) | (uint32_t)tb;
         uint4 bv;
-        dequant_pair<BF>(u4_comp(d[s][0], w), u4_comp(d[s][1], w), sel, bv.x, bv.y);
-        dequant_pair<BF>(u4_comp(d[s][2], w), u4_comp(d[s][3], w), sel, bv.z, bv.w);
+        dequant_pair<BF>(dqk, u4_comp(d[s][0], w), u4_comp(d[s][1], w), sel, bv.x, bv.y);
+        dequant_pair<BF>(dqk, u4_comp(d[s][2], w), u4_comp(d[s][3], w), sel, bv.z, bv.w);
         acc[tt] = Act<TX>::mma(av[s], bv, acc[tt]);
       }
     }
@@ -368,9 +410,11 @@ __global__ __launch_bounds__(SPW == 2 ? 1024 : 512) void qmm_fwd_mfma_kernel(
     for (int r = 0; r < 4; ++r) {
       const int m = 4 * g + r;
       if (m < mrows) {
-        float *dst = slot + m * QSTRIP + 16 * l16 + half * 8;
-        *reinterpret_cast<float4 *>(dst) = make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]);
-        *reinterpret_cast<float4 *>(dst + 4) = make_float4(acc[4][r], acc[5][r], acc[6][r], acc[7][r]);
+        float *dst = slot + m * QSTRIP;
+        *reinterpret_cast<float4 *>(dst + qtile_chunk(l16, 2 * half)) =
+            make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]);
+        *reinterpret_cast<float4 *>(dst + qtile_chunk(l16, 2 * half + 1)) =
+            make_float4(acc[4][r], acc[5][r], acc[6][r], acc[7][r]);
       }
     }
   }
@@ -432,6 +476,7 @@ __global__ __launch_bounds__(256, 2) void qmm_fwd_stream_kernel(
   for (int t = 0; t < 16; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
   float se = 0.f, so = 0.f;
   const half2_t sixteenth = half2_t{(_Float16)0.0625f, (_Float16)0.0625f};
+  const DqConst dqk = dq_const<BF>();
 
   auto consume = [&](Step &st, int t) __attribute__((always_inline)) {
     const int rbase = r_begin + (t * QS_NW + wave) * 16 + 4 * g;
@@ -459,8 +504,8 @@ __global__ __launch_bounds__(256, 2) void qmm_fwd_stream_kernel(
       const int w = tl >> 2, tb = tl & 3;
       const uint32_t sel = 0x0c000c00u | ((uint32_t)(4 + tb) << 16) | (uint32_t)tb;
       uint4 bv;
-      dequant_pair<BF>(u4_comp(st.d[0], w), u4_comp(st.d[1], w), sel, bv.x, bv.y);
-      dequant_pair<BF>(u4_comp(st.d[2], w), u4_comp(st.d[3], w), sel, bv.z, bv.w);
+      dequant_pair<BF>(dqk, u4_comp(st.d[0], w), u4_comp(st.d[1], w), sel, bv.x, bv.y);
+      dequant_pair<BF>(dqk, u4_comp(st.d[2], w), u4_comp(st.d[3], w), sel, bv.z, bv.w);
       acc[tl] = Act<TX>::mma(av, bv, acc[tl]);
     }
   };
@@ -491,15 +536,180 @@ __global__ __launch_bounds__(256, 2) void qmm_fwd_stream_kernel(
   for (int r = 0; r < 4; ++r) {
     const int m = 4 * g + r;
     if (m < mrows) {
-      float *dst = slot + m * QSTRIP + 16 * l16;
+      float *dst = slot + m * QSTRIP;
 #pragma unroll
       for (int q = 0; q < 4; ++q)
-        *reinterpret_cast<float4 *>(dst + 4 * q) =
+        *reinterpret_cast<float4 *>(dst + qtile_chunk(l16, q)) =
             make_float4(acc[4 * q][r], acc[4 * q + 1][r], acc[4 * q + 2][r], acc[4 * q + 3][r]);
     }
   }
   qmm_reduce_and_store<16>(red, &s_last, QS_NW, mrows, mvalid, strip, split, m0, M, C, S, zero, scale,
                            out, ws, se, so);
+}
+
+// ---------------------------------------------------------------------------- MFMA path, decode
+// M <= 16 on matrices that the chip holds in flight (up to ~50 MB packed).  Same operands and
+// arithmetic as qmm_fwd_mfma_kernel; what differs is everything around the MFMAs, which is where
+// the time of a 22 MB product goes once the loads run at the memory's pace:
+//  * a workgroup of NW wavefronts owns a strip and `rows_per_split` packed rows; k-step t of
+//    wavefront w is the 16 rows (t NW + w) 16 .. + 15 of that range, KS k-steps per wavefront, all
+//    loads issued before anything else; k-steps past the range are skipped (wave-uniform branch);
+//  * the column parameters of the outputs a thread will finish are fetched under the weight loads;
+//  * M <= 8 (ATOM; MR = 1, 4 or 16 rows of the tile kept): the workgroups of a strip add their partial results to 64-bit
+//    accumulators with ONE returning atomic per output: the word is value * 2^28 (fixed point,
+//    a partial beyond +-65536 or not finite adds the poison 3 * 2^49 instead) << 8 | 1, so the
+//    returned old word tells the caller whether it was the last of the S contributions, and the
+//    last one has the complete sum in hand: it rounds, stores the output and zeroes the word.
+//    Integer addition is exact and commutative: the result does not depend on the arrival order.
+//    One round trip to the memory side instead of three (partial stores -> ticket -> partial
+//    loads).  A poisoned sum yields NaN.  S <= 32.
+//  * M > 8: the atomics of that many rows take longer than the ticket scheme (the memory side
+//    retires them at a limited rate: 350000 of them add 2 us, 700000 add 4), so those keep
+//    qmm_reduce_and_store (ATOM = false).
+constexpr int QD_FRAC = 28;
+constexpr long long QD_POISON = 3LL << 49;
+constexpr int QD_MAX_SPLITS = 32;
+
+template <int NW, int KS, int MR, bool ATOM, typename TZ, typename TX>
+__global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
+    const TX *x, int M, int K, const uint8_t *pk, int R, int C, const TZ *zero, const TZ *scale,
+    TX *out, QmmWs ws, int S, int rows_per_split) {
+  constexpr bool BF = Act<TX>::BF;
+  extern __shared__ float red[];   // [NW][MR][256] partial tiles, then [NW][2][16] x sums
+  __shared__ int s_last;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int strip = blockIdx.x, split = blockIdx.y, m0 = blockIdx.z * 16;
+  const int mvalid = min(16, M - m0);
+  const int g = lane >> 4, l16 = lane & 15;
+  const int r_begin = split * rows_per_split, r_end = min(R, r_begin + rows_per_split);
+
+  // ---- activations (16 bytes = the 8 k of this lane group's four packed rows), then all weight loads
+  uint4 pr[KS];
+  {
+    const TX *xr = x + (int64_t)(m0 + (l16 < mvalid ? l16 : 0)) * K;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int row = r_begin + (s * NW + wave) * 16 + 4 * g;      // range boundaries are multiples of 4 rows
+      pr[s] = (l16 < mvalid && row < r_end) ? *reinterpret_cast<const uint4 *>(xr + 2 * row)
+                                            : make_uint4(0u, 0u, 0u, 0u);
+    }
+  }
+  uint4 d[KS][4];
+  const int col0 = strip * QSTRIP + 16 * l16;
+#pragma unroll
+  for (int s = 0; s < KS; ++s)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = r_begin + (s * NW + wave) * 16 + 4 * g + i;
+      d[s][i] = (row < r_end && col0 < C)
+                    ? *reinterpret_cast<const uint4 *>(pk + (int64_t)row * C + col0)
+                    : make_uint4(0, 0, 0, 0);
+    }
+  // ---- column parameters of the outputs this thread finishes
+  constexpr int NT = NW * 64;
+  constexpr int ITEMS = MR * QSTRIP;
+  constexpr int IT = (ITEMS + NT - 1) / NT;
+  float pz[ATOM ? IT : 1], psc[ATOM ? IT : 1];
+  if (ATOM) {
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+      const int n = min(strip * QSTRIP + ((tid + it * NT) & 255), C - 1);
+      pz[it] = to_f32(zero[n]);
+      psc[it] = to_f32(scale[n]);
+    }
+  }
+
+  const DqConst dqk = dq_const<BF>();
+  const half2_t sixteenth = half2_t{(_Float16)0.0625f, (_Float16)0.0625f};
+  floatx4 acc[16];
+#pragma unroll
+  for (int t = 0; t < 16; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float se = 0.f, so = 0.f;
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    if (s > 0 && r_begin + (s * NW + wave) * 16 >= r_end) break;       // nothing was loaded for this k-step
+    uint4 av;
+    av.x = __builtin_amdgcn_perm(pr[s].y, pr[s].x, 0x05040100u);  // {x[2r0],   x[2r1]}
+    av.z = __builtin_amdgcn_perm(pr[s].w, pr[s].z, 0x05040100u);
+    uint32_t o0 = __builtin_amdgcn_perm(pr[s].y, pr[s].x, 0x07060302u);   // {x[2r0+1], x[2r1+1]}
+    uint32_t o1 = __builtin_amdgcn_perm(pr[s].w, pr[s].z, 0x07060302u);
+    if (!BF) {      // fp16: odd-k activations enter divided by 16 (bf16: both nibbles are 128 + code)
+      o0 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, o0) * sixteenth);
+      o1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, o1) * sixteenth);
+    }
+    av.y = o0;
+    av.w = o1;
+    se += (Act<TX>::lo(av.x) + Act<TX>::hi(av.x)) + (Act<TX>::lo(av.z) + Act<TX>::hi(av.z));
+    so += (Act<TX>::lo(o0) + Act<TX>::hi(o0)) + (Act<TX>::lo(o1) + Act<TX>::hi(o1));
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      const int w = t >> 2, tb = t & 3;
+      const uint32_t sel = 0x0c000c00u | ((uint32_t)(4 + tb) << 16) | (uint32_t)tb;
+      uint4 bv;
+      dequant_pair<BF>(dqk, u4_comp(d[s][0], w), u4_comp(d[s][1], w), sel, bv.x, bv.y);
+      dequant_pair<BF>(dqk, u4_comp(d[s][2], w), u4_comp(d[s][3], w), sel, bv.z, bv.w);
+      acc[t] = Act<TX>::mma(av, bv, acc[t]);
+    }
+  }
+  se += __shfl_xor(se, 16);
+  se += __shfl_xor(se, 32);
+  so += __shfl_xor(so, 16);
+  so += __shfl_xor(so, 32);
+
+  // acc[t][r] = tile[m = 4g + r][channel 16 * l16 + t]
+  float *slot = red + (size_t)wave * MR * QSTRIP;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int m = 4 * g + r;
+    if (m < MR) {
+      float *dst = slot + m * QSTRIP;
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<float4 *>(dst + qtile_chunk(l16, q)) =
+            make_float4(acc[4 * q][r], acc[4 * q + 1][r], acc[4 * q + 2][r], acc[4 * q + 3][r]);
+    }
+  }
+  if (!ATOM) {
+    qmm_reduce_and_store<IT>(red, &s_last, NW, MR, mvalid, strip, split, m0, M, C, S, zero, scale, out, ws,
+                             se, so);
+    return;
+  }
+  float *xs = red + (size_t)NW * MR * QSTRIP;   // [wave][2][16]
+  if (g == 0) { xs[wave * 32 + l16] = se; xs[wave * 32 + 16 + l16] = so; }
+  __syncthreads();
+#pragma unroll
+  for (int it = 0; it < IT; ++it) {
+    const int idx = tid + it * NT;
+    const int m = idx >> 8, c = idx & 255, n = strip * QSTRIP + c;
+    if (idx >= ITEMS || m >= mvalid || n >= C) continue;
+    float v = 0.f, e = 0.f, o = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      v += red[(w * MR + m) * QSTRIP + qtile_pos(c)];
+      e += xs[w * 32 + m];
+      o += xs[w * 32 + 16 + m];
+    }
+    const float r = BF ? (v - 128.f * (e + o)) - pz[it] * (e + o)
+                       : (v - 1024.f * (e + o)) - pz[it] * (e + 16.f * o);
+    const float pv = psc[it] * r;
+    TX *dst = out + (int64_t)(m0 + m) * C + n;
+    if (S == 1) {
+      *dst = Act<TX>::out(pv);
+      continue;
+    }
+    const bool ok = fabsf(pv) <= 65536.f;                       // false for NaN, too
+    const long long fx = ok ? __float2ll_rn(pv * (float)(1 << QD_FRAC)) : QD_POISON;
+    const unsigned long long word = ((unsigned long long)fx << 8) + 1ull;
+    unsigned long long *cell = ws.acc64 + (int64_t)(m0 + m) * C + n;
+    const unsigned long long total = atomicAdd(cell, word) + word;
+    if ((int)(total & 255ull) == S) {                           // every contribution is in
+      const long long sum = (long long)total >> 8;
+      const bool fine = sum <= (1LL << 49) && sum >= -(1LL << 49);
+      const float res = fine ? (float)sum * (1.f / (float)(1 << QD_FRAC)) : __builtin_nanf("");
+      *dst = Act<TX>::out(res);
+      __hip_atomic_store(cell, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
 }
 
 struct FwdPlan {
@@ -536,7 +746,7 @@ FwdPlan fwd_plan(int64_t M, int64_t R, int64_t C, bool allow_stream) {
   }
   const int mrows = (M <= 4) ? 4 : 16;
   p.lds_bytes = ((size_t)p.nw * mrows * QSTRIP + (size_t)p.nw * 32) * sizeof(float);
-  p.counter_bytes = QMM_COUNTER_BYTES;
+  p.counter_bytes = QMM_HEAD_BYTES;
   p.x1_bytes = (size_t)round_up64((int64_t)p.strips * p.mch * p.S * 32 * sizeof(float), 256);
   p.part_bytes = (size_t)p.S * M * C * sizeof(float);
   p.total_bytes = p.S > 1 ? p.counter_bytes + p.x1_bytes + p.part_bytes : 0;
@@ -546,11 +756,7 @@ FwdPlan fwd_plan(int64_t M, int64_t R, int64_t C, bool allow_stream) {
 template <int SPW, typename TZ, typename TX, bool X16>
 int launch_fwd_mfma(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, const uint8_t *pk,
                     int64_t R, int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
-  QmmWs ws;
-  char *base = reinterpret_cast<char *>(wsp);
-  ws.counters = reinterpret_cast<int32_t *>(base);
-  ws.x1part = reinterpret_cast<float *>(base + p.counter_bytes);
-  ws.part = reinterpret_cast<float *>(base + p.counter_bytes + p.x1_bytes);
+  const QmmWs ws = qmm_ws(wsp, p.x1_bytes);
   auto kern = qmm_fwd_mfma_kernel<SPW, TZ, TX, X16>;
   if (p.lds_bytes > 48 * 1024 &&
       hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -578,11 +784,7 @@ int launch_fwd_mfma(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, 
 template <typename TZ, typename TX>
 int launch_fwd_stream(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, const uint8_t *pk,
                       int64_t R, int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
-  QmmWs ws;
-  char *base = reinterpret_cast<char *>(wsp);
-  ws.counters = reinterpret_cast<int32_t *>(base);
-  ws.x1part = reinterpret_cast<float *>(base + p.counter_bytes);
-  ws.part = reinterpret_cast<float *>(base + p.counter_bytes + p.x1_bytes);
+  const QmmWs ws = qmm_ws(wsp, p.x1_bytes);
   auto kern = qmm_fwd_stream_kernel<TZ, TX>;
   if (p.strips > QMM_MAX_COUNTERS || p.mch != 1 || C < 16) return GPTQ_HIP_EINVAL;
   if (p.lds_bytes > 48 * 1024 &&
@@ -595,6 +797,117 @@ int launch_fwd_stream(hipStream_t st, const FwdPlan &p, const void *x, int64_t M
                      ws, p.S, p.rows_per_split);
   GPTQ_CHECK_LAUNCH();
   return GPTQ_HIP_OK;
+}
+
+// Which instantiation of qmm_fwd_dec_kernel serves M rows of a [2R, C] matrix, if any.
+struct DecPlan {
+  bool use, atom;
+  int nw, ks, mr, S, rows, strips;
+  size_t lds_bytes, x1_bytes, part_bytes, total_bytes;
+};
+
+DecPlan dec_plan(int64_t M, int64_t R, int64_t C) {
+  DecPlan p{};
+  if (M < 1 || M > 16 || R % 4 != 0 || C % 16 != 0 || C < 16 || R >= (1LL << 30) || C >= (1LL << 30)) return p;
+  p.strips = (int)ceil_div64(C, QSTRIP);
+  if (p.strips > QMM_MAX_COUNTERS) return p;
+  p.mr = M == 1 ? 1 : (M <= 4 ? 4 : 16);
+  p.atom = M <= 8 && M * C * 8 <= QMM_ACC_BYTES;
+  if (p.mr <= 4) {
+    if (!p.atom) return p;
+    // eight wavefronts, two workgroups per CU: as many splits as 512 slots allow, at least 128 rows each
+    int64_t S = 512 / p.strips;
+    if (S > QD_MAX_SPLITS) S = QD_MAX_SPLITS;
+    if (S > R / 128) S = R / 128;
+    if (S < 1) S = 1;
+    int64_t rows = round_up64(ceil_div64(R, S), 4);
+    if (rows <= 256) {
+      p.nw = 8;
+      p.ks = rows <= 128 ? 1 : 2;
+    } else {
+      // sixteen wavefronts, one workgroup per CU
+      S = 256 / p.strips;
+      if (S > QD_MAX_SPLITS) S = QD_MAX_SPLITS;
+      if (S < 1) S = 1;
+      rows = round_up64(ceil_div64(R, S), 4);
+      if (rows > 512) return p;                 // larger matrices stream (qmm_fwd_stream_kernel)
+      p.nw = 16;
+      p.ks = 2;
+    }
+    p.S = (int)ceil_div64(R, rows);
+    p.rows = (int)rows;
+    p.x1_bytes = p.part_bytes = 0;
+    p.total_bytes = p.S > 1 ? QMM_HEAD_BYTES : 0;
+  } else {
+    // 16 rows kept: eight wavefronts of four k-steps, one workgroup per CU (132 KB of LDS)
+    p.nw = 8;
+    p.ks = 4;
+    p.rows = 512;
+    p.S = (int)ceil_div64(R, 512);
+    if ((int64_t)p.strips * p.S > 256) return p;                     // larger matrices stream
+    if (p.S > QD_MAX_SPLITS) p.atom = false;
+    if (p.atom) {
+      p.x1_bytes = p.part_bytes = 0;
+      p.total_bytes = p.S > 1 ? QMM_HEAD_BYTES : 0;
+    } else {
+      p.x1_bytes = (size_t)round_up64((int64_t)p.strips * p.S * 32 * sizeof(float), 256);
+      p.part_bytes = (size_t)p.S * M * C * sizeof(float);
+      p.total_bytes = p.S > 1 ? QMM_HEAD_BYTES + p.x1_bytes + p.part_bytes : 0;
+    }
+  }
+  p.lds_bytes = ((size_t)p.nw * p.mr * QSTRIP + (size_t)p.nw * 32) * sizeof(float);
+  p.use = true;
+  return p;
+}
+
+template <int NW, int KS, int MR, bool ATOM, typename TZ, typename TX>
+int launch_dec_inst(hipStream_t st, const DecPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
+                    int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
+  auto kern = qmm_fwd_dec_kernel<NW, KS, MR, ATOM, TZ, TX>;
+  // the LDS limit of a kernel is raised once per device and instantiation (a repeated or concurrent
+  // call sets the same value again, which is harmless)
+  static bool attr_set[64] = {};
+  int dev = 0;
+  if (p.lds_bytes > 48 * 1024 && (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64 || !attr_set[dev])) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)p.lds_bytes) != hipSuccess)
+      return GPTQ_HIP_ELAUNCH;
+    if (dev >= 0 && dev < 64) attr_set[dev] = true;
+  }
+  const QmmWs ws = qmm_ws(wsp, p.x1_bytes);
+  hipLaunchKernelGGL(kern, dim3((unsigned)p.strips, (unsigned)p.S, 1), dim3(NW * 64), p.lds_bytes, st,
+                     (const TX *)x, (int)M, (int)(2 * R), pk, (int)R, (int)C, (const TZ *)zero,
+                     (const TZ *)scale, (TX *)out, ws, p.S, p.rows);
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
+template <typename TZ, typename TX>
+int launch_dec_zx(hipStream_t st, const DecPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
+                  int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
+#define GPTQ_DEC(NW, KS, MR, ATOM) \
+  return launch_dec_inst<NW, KS, MR, ATOM, TZ, TX>(st, p, x, M, pk, R, C, zero, scale, out, wsp)
+  if (p.mr == 16) {
+    if (p.atom) GPTQ_DEC(8, 4, 16, true);
+    GPTQ_DEC(8, 4, 16, false);
+  }
+  if (p.mr == 1) {
+    if (p.nw == 16) GPTQ_DEC(16, 2, 1, true);
+    if (p.ks == 1) GPTQ_DEC(8, 1, 1, true);
+    GPTQ_DEC(8, 2, 1, true);
+  }
+  if (p.nw == 16) GPTQ_DEC(16, 2, 4, true);
+  if (p.ks == 1) GPTQ_DEC(8, 1, 4, true);
+  GPTQ_DEC(8, 2, 4, true);
+#undef GPTQ_DEC
+}
+
+template <typename TZ>
+int launch_dec_z(hipStream_t st, const DecPlan &p, const void *x, int x_dtype, int64_t M, const uint8_t *pk,
+                 int64_t R, int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
+  if (x_dtype == GPTQ_HIP_BF16)
+    return launch_dec_zx<TZ, __hip_bfloat16>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
+  return launch_dec_zx<TZ, __half>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
 }
 
 template <typename TZ, typename TX>
@@ -936,7 +1249,7 @@ GemmPlan gemm_plan(int64_t M, int64_t R, int64_t C) {
           ceil_div64(M, p.bm) <= 65535;
   p.x1_bytes = S > 1 ? (size_t)round_up64(p.tiles * S * p.bm * (int64_t)sizeof(float), 256) : 0;
   p.part_bytes = S > 1 ? (size_t)S * M * C * sizeof(float) : 0;
-  p.total_bytes = S > 1 ? QMM_COUNTER_BYTES + p.x1_bytes + p.part_bytes : 0;
+  p.total_bytes = S > 1 ? QMM_HEAD_BYTES + p.x1_bytes + p.part_bytes : 0;
   return p;
 }
 
@@ -974,11 +1287,7 @@ template <typename TZ>
 int launch_fwd_gemm(hipStream_t st, const GemmPlan &p, const void *x, int x_dtype, int64_t M,
                     const uint8_t *pk, int64_t R, int64_t C, const void *zero, const void *scale,
                     void *out, void *wsp) {
-  QmmWs ws;
-  char *base = reinterpret_cast<char *>(wsp);
-  ws.counters = reinterpret_cast<int32_t *>(base);
-  ws.x1part = reinterpret_cast<float *>(base + QMM_COUNTER_BYTES);
-  ws.part = reinterpret_cast<float *>(base + QMM_COUNTER_BYTES + p.x1_bytes);
+  const QmmWs ws = qmm_ws(wsp, p.x1_bytes);
   if (x_dtype == GPTQ_HIP_BF16)
     return launch_fwd_gemm_x<TZ, __hip_bfloat16>(st, p, x, M, pk, R, C, zero, scale, out, ws);
   return launch_fwd_gemm_x<TZ, __half>(st, p, x, M, pk, R, C, zero, scale, out, ws);
@@ -1413,7 +1722,7 @@ F32Plan f32_plan(int64_t M, int64_t R, int64_t C, int transpose_b) {
   p.inner = inner;
   // the counter region stays out of reach of the staging buffers whatever this call's own product
   // needs: a later call on the same workspace expects its counters to be zero
-  p.x16_off = round_up_256(inner > (size_t)QMM_COUNTER_BYTES ? inner : (size_t)QMM_COUNTER_BYTES);
+  p.x16_off = round_up_256(inner > (size_t)QMM_HEAD_BYTES ? inner : (size_t)QMM_HEAD_BYTES);
   p.o16_off = p.x16_off + round_up_256((size_t)p.mc * kin * sizeof(__half));
   p.exp_off = p.o16_off + round_up_256((size_t)p.mc * nout * sizeof(__half));
   p.total_bytes = p.exp_off + round_up_256((size_t)p.mc * sizeof(int32_t));
@@ -1429,7 +1738,10 @@ size_t gptq_hip_qmatmul_workspace_bytes(int64_t M, int64_t R, int64_t C, int tra
   // which kernel runs also depends on pointer alignment: enough for either
   const size_t a = fwd_plan(M, R, C, false).total_bytes, b = gemm_plan(M, R, C).total_bytes;
   const size_t c = fwd_plan(M, R, C, true).total_bytes;
-  return a > b ? (a > c ? a : c) : (b > c ? b : c);
+  const DecPlan dp = dec_plan(M, R, C);
+  const size_t d = dp.use ? dp.total_bytes : 0;
+  const size_t abc = a > b ? (a > c ? a : c) : (b > c ? b : c);
+  return abc > d ? abc : d;
 }
 
 size_t gptq_hip_qmatmul_workspace_bytes_x(int64_t M, int64_t R, int64_t C, int transpose_b, int x_dtype) {
@@ -1502,6 +1814,19 @@ int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const 
       default: return GPTQ_HIP_EDTYPE;
     }
   }
+  if (!transpose_b && fwd_fast_ok(x_dtype, M, R, C, x, packed) && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    const DecPlan dp = dec_plan(M, R, C);
+    if (dp.use) {
+      if (dp.total_bytes && (!ws || ws_bytes < dp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+      switch (zs_dtype) {
+        case GPTQ_HIP_F32: return launch_dec_z<float>(st, dp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
+        case GPTQ_HIP_F16: return launch_dec_z<__half>(st, dp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
+        case GPTQ_HIP_BF16:
+          return launch_dec_z<__hip_bfloat16>(st, dp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
+        default: return GPTQ_HIP_EDTYPE;
+      }
+    }
+  }
   if (!transpose_b && fwd_fast_ok(x_dtype, M, R, C, x, packed)) {
     const FwdPlan p = fwd_plan(M, R, C, (reinterpret_cast<uintptr_t>(x) & 15) == 0);
     if (p.total_bytes && (!ws || ws_bytes < p.total_bytes)) return GPTQ_HIP_EWORKSPACE;
@@ -1565,7 +1890,7 @@ int qmm_static_base(hipStream_t st, void **base) {
       (void)hipGetLastError();
       return GPTQ_HIP_ELAUNCH;
     }
-    const int words = QMM_COUNTER_BYTES / 4;
+    const int words = QMM_HEAD_BYTES / 4;
     hipLaunchKernelGGL(qmm_static_clear_kernel, dim3((words + 255) / 256), dim3(256), 0, st,
                        reinterpret_cast<uint32_t *>(ptr), words);
     GPTQ_CHECK_LAUNCH();
