@@ -570,7 +570,7 @@ constexpr int QD_FRAC = 28;
 constexpr long long QD_POISON = 3LL << 49;
 constexpr int QD_MAX_SPLITS = 32;
 
-template <int NW, int KS, int MR, bool ATOM, typename TZ, typename TX>
+template <int NW, int KS, int MR, bool ATOM, bool LOOP, typename TZ, typename TX>
 __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
     const TX *x, int M, int K, const uint8_t *pk, int R, int C, const TZ *zero, const TZ *scale,
     TX *out, QmmWs ws, int S, int rows_per_split) {
@@ -582,30 +582,81 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
   const int mvalid = min(16, M - m0);
   const int g = lane >> 4, l16 = lane & 15;
   const int r_begin = split * rows_per_split, r_end = min(R, r_begin + rows_per_split);
+  // k-step t of this wavefront: packed rows r_begin + (t NW + wave) 16 + [0, 16)
+  const int groups = (r_end - r_begin + 15) >> 4;
+  const int nsteps = groups > wave ? (groups - wave + NW - 1) / NW : 0;
 
-  // ---- activations (16 bytes = the 8 k of this lane group's four packed rows), then all weight loads
-  uint4 pr[KS];
-  {
-    const TX *xr = x + (int64_t)(m0 + (l16 < mvalid ? l16 : 0)) * K;
+  // One k-step of loads: the activations of the lane group's four packed rows (16 bytes = 8 k; range
+  // boundaries are multiples of 4 rows, so the four rows are inside the range or outside together)
+  // and the four weight rows.  LOOP (a ring of KS k-steps that is refilled as it is consumed, for
+  // matrices beyond what the chip holds in flight): loads past the range read clamped, valid
+  // addresses and their k-step enters with zero activations.  Otherwise (all KS k-steps of the
+  // range issued at once) they are predicated off.
+  struct Step { uint4 d[4]; uint4 pr; };
+  const bool m_ok = l16 < mvalid;
+  const TX *xr = x + (int64_t)(m0 + (m_ok ? l16 : 0)) * K;
+  const int col0 = LOOP ? min(strip * QSTRIP + 16 * l16, C - 16) : strip * QSTRIP + 16 * l16;
+  const uint8_t *wp = pk + col0;
+  auto issue = [&](Step &st, int t) __attribute__((always_inline)) {
+    const int rbase = r_begin + (t * NW + wave) * 16 + 4 * g;
+    if (LOOP) {
+      st.pr = *reinterpret_cast<const uint4 *>(xr + 2 * min(rbase, R - 4));
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const int row = r_begin + (s * NW + wave) * 16 + 4 * g;      // range boundaries are multiples of 4 rows
-      pr[s] = (l16 < mvalid && row < r_end) ? *reinterpret_cast<const uint4 *>(xr + 2 * row)
-                                            : make_uint4(0u, 0u, 0u, 0u);
+      for (int i = 0; i < 4; ++i)
+        st.d[i] = *reinterpret_cast<const uint4 *>(wp + (int64_t)min(rbase + i, R - 1) * C);
+    } else {
+      const bool in = rbase < r_end;
+      st.pr = (m_ok && in) ? *reinterpret_cast<const uint4 *>(xr + 2 * rbase) : make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        st.d[i] = (in && col0 < C) ? *reinterpret_cast<const uint4 *>(wp + (int64_t)(rbase + i) * C)
+                                   : make_uint4(0u, 0u, 0u, 0u);
     }
-  }
-  uint4 d[KS][4];
-  const int col0 = strip * QSTRIP + 16 * l16;
+  };
+
+  const DqConst dqk = dq_const<BF>();
+  const half2_t sixteenth = half2_t{(_Float16)0.0625f, (_Float16)0.0625f};
+  floatx4 acc[16];
 #pragma unroll
-  for (int s = 0; s < KS; ++s)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int row = r_begin + (s * NW + wave) * 16 + 4 * g + i;
-      d[s][i] = (row < r_end && col0 < C)
-                    ? *reinterpret_cast<const uint4 *>(pk + (int64_t)row * C + col0)
-                    : make_uint4(0, 0, 0, 0);
+  for (int t = 0; t < 16; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float se = 0.f, so = 0.f;
+  auto consume = [&](Step &st, int t) __attribute__((always_inline)) {
+    uint4 pr = st.pr;
+    if (LOOP) {
+      const bool ok = m_ok && t < nsteps && r_begin + (t * NW + wave) * 16 + 4 * g < r_end;
+      pr.x = ok ? pr.x : 0u;
+      pr.y = ok ? pr.y : 0u;
+      pr.z = ok ? pr.z : 0u;
+      pr.w = ok ? pr.w : 0u;
     }
-  // ---- column parameters of the outputs this thread finishes
+    uint4 av;
+    av.x = __builtin_amdgcn_perm(pr.y, pr.x, 0x05040100u);  // {x[2r0],   x[2r1]}
+    av.z = __builtin_amdgcn_perm(pr.w, pr.z, 0x05040100u);
+    uint32_t o0 = __builtin_amdgcn_perm(pr.y, pr.x, 0x07060302u);   // {x[2r0+1], x[2r1+1]}
+    uint32_t o1 = __builtin_amdgcn_perm(pr.w, pr.z, 0x07060302u);
+    if (!BF) {      // fp16: odd-k activations enter divided by 16 (bf16: both nibbles are 128 + code)
+      o0 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, o0) * sixteenth);
+      o1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, o1) * sixteenth);
+    }
+    av.y = o0;
+    av.w = o1;
+    se += (Act<TX>::lo(av.x) + Act<TX>::hi(av.x)) + (Act<TX>::lo(av.z) + Act<TX>::hi(av.z));
+    so += (Act<TX>::lo(o0) + Act<TX>::hi(o0)) + (Act<TX>::lo(o1) + Act<TX>::hi(o1));
+#pragma unroll
+    for (int tl = 0; tl < 16; ++tl) {
+      const int w = tl >> 2, tb = tl & 3;
+      const uint32_t sel = 0x0c000c00u | ((uint32_t)(4 + tb) << 16) | (uint32_t)tb;
+      uint4 bv;
+      dequant_pair<BF>(dqk, u4_comp(st.d[0], w), u4_comp(st.d[1], w), sel, bv.x, bv.y);
+      dequant_pair<BF>(dqk, u4_comp(st.d[2], w), u4_comp(st.d[3], w), sel, bv.z, bv.w);
+      acc[tl] = Act<TX>::mma(av, bv, acc[tl]);
+    }
+  };
+
+  Step ring[KS];
+#pragma unroll
+  for (int u = 0; u < KS; ++u) issue(ring[u], u);
+  // ---- column parameters of the outputs this thread finishes, fetched under the weight loads
   constexpr int NT = NW * 64;
   constexpr int ITEMS = MR * QSTRIP;
   constexpr int IT = (ITEMS + NT - 1) / NT;
@@ -618,37 +669,24 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
       psc[it] = to_f32(scale[n]);
     }
   }
-
-  const DqConst dqk = dq_const<BF>();
-  const half2_t sixteenth = half2_t{(_Float16)0.0625f, (_Float16)0.0625f};
-  floatx4 acc[16];
+  if (LOOP) {
+    int t0 = 0;
+    for (; t0 + KS <= nsteps; t0 += KS) {
 #pragma unroll
-  for (int t = 0; t < 16; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-  float se = 0.f, so = 0.f;
-#pragma unroll
-  for (int s = 0; s < KS; ++s) {
-    if (s > 0 && r_begin + (s * NW + wave) * 16 >= r_end) break;       // nothing was loaded for this k-step
-    uint4 av;
-    av.x = __builtin_amdgcn_perm(pr[s].y, pr[s].x, 0x05040100u);  // {x[2r0],   x[2r1]}
-    av.z = __builtin_amdgcn_perm(pr[s].w, pr[s].z, 0x05040100u);
-    uint32_t o0 = __builtin_amdgcn_perm(pr[s].y, pr[s].x, 0x07060302u);   // {x[2r0+1], x[2r1+1]}
-    uint32_t o1 = __builtin_amdgcn_perm(pr[s].w, pr[s].z, 0x07060302u);
-    if (!BF) {      // fp16: odd-k activations enter divided by 16 (bf16: both nibbles are 128 + code)
-      o0 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, o0) * sixteenth);
-      o1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, o1) * sixteenth);
+      for (int u = 0; u < KS; ++u) {
+        consume(ring[u], t0 + u);
+        issue(ring[u], t0 + u + KS);
+      }
     }
-    av.y = o0;
-    av.w = o1;
-    se += (Act<TX>::lo(av.x) + Act<TX>::hi(av.x)) + (Act<TX>::lo(av.z) + Act<TX>::hi(av.z));
-    so += (Act<TX>::lo(o0) + Act<TX>::hi(o0)) + (Act<TX>::lo(o1) + Act<TX>::hi(o1));
+    // at most KS - 1 k-steps left, all of them loaded
 #pragma unroll
-    for (int t = 0; t < 16; ++t) {
-      const int w = t >> 2, tb = t & 3;
-      const uint32_t sel = 0x0c000c00u | ((uint32_t)(4 + tb) << 16) | (uint32_t)tb;
-      uint4 bv;
-      dequant_pair<BF>(dqk, u4_comp(d[s][0], w), u4_comp(d[s][1], w), sel, bv.x, bv.y);
-      dequant_pair<BF>(dqk, u4_comp(d[s][2], w), u4_comp(d[s][3], w), sel, bv.z, bv.w);
-      acc[t] = Act<TX>::mma(av, bv, acc[t]);
+    for (int u = 0; u < KS - 1; ++u)
+      if (t0 + u < nsteps) consume(ring[u], t0 + u);
+  } else {
+#pragma unroll
+    for (int u = 0; u < KS; ++u) {
+      if (u > 0 && u >= nsteps) break;        // wave-uniform: nothing was loaded for this k-step
+      consume(ring[u], u);
     }
   }
   se += __shfl_xor(se, 16);
@@ -801,7 +839,7 @@ int launch_fwd_stream(hipStream_t st, const FwdPlan &p, const void *x, int64_t M
 
 // Which instantiation of qmm_fwd_dec_kernel serves M rows of a [2R, C] matrix, if any.
 struct DecPlan {
-  bool use, atom;
+  bool use, atom, loop;
   int nw, ks, mr, S, rows, strips;
   size_t lds_bytes, x1_bytes, part_bytes, total_bytes;
 };
@@ -830,9 +868,9 @@ DecPlan dec_plan(int64_t M, int64_t R, int64_t C) {
       if (S > QD_MAX_SPLITS) S = QD_MAX_SPLITS;
       if (S < 1) S = 1;
       rows = round_up64(ceil_div64(R, S), 4);
-      if (rows > 512) return p;                 // larger matrices stream (qmm_fwd_stream_kernel)
       p.nw = 16;
       p.ks = 2;
+      p.loop = rows > 512;                      // beyond two k-steps per wavefront: a ring of two
     }
     p.S = (int)ceil_div64(R, rows);
     p.rows = (int)rows;
@@ -844,7 +882,16 @@ DecPlan dec_plan(int64_t M, int64_t R, int64_t C) {
     p.ks = 4;
     p.rows = 512;
     p.S = (int)ceil_div64(R, 512);
-    if ((int64_t)p.strips * p.S > 256) return p;                     // larger matrices stream
+    if ((int64_t)p.strips * p.S > 256) {
+      // more than one workgroup per CU that way: as many splits as 256 slots allow, a ring of four k-steps
+      int64_t S = 256 / p.strips;
+      if (S > QD_MAX_SPLITS) S = QD_MAX_SPLITS;
+      if (S < 1) S = 1;
+      const int64_t rows = round_up64(ceil_div64(R, S), 4);
+      p.S = (int)ceil_div64(R, rows);
+      p.rows = (int)rows;
+      p.loop = true;
+    }
     if (p.S > QD_MAX_SPLITS) p.atom = false;
     if (p.atom) {
       p.x1_bytes = p.part_bytes = 0;
@@ -860,10 +907,10 @@ DecPlan dec_plan(int64_t M, int64_t R, int64_t C) {
   return p;
 }
 
-template <int NW, int KS, int MR, bool ATOM, typename TZ, typename TX>
+template <int NW, int KS, int MR, bool ATOM, bool LOOP, typename TZ, typename TX>
 int launch_dec_inst(hipStream_t st, const DecPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
                     int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
-  auto kern = qmm_fwd_dec_kernel<NW, KS, MR, ATOM, TZ, TX>;
+  auto kern = qmm_fwd_dec_kernel<NW, KS, MR, ATOM, LOOP, TZ, TX>;
   // the LDS limit of a kernel is raised once per device and instantiation (a repeated or concurrent
   // call sets the same value again, which is harmless)
   static bool attr_set[64] = {};
@@ -885,20 +932,24 @@ int launch_dec_inst(hipStream_t st, const DecPlan &p, const void *x, int64_t M, 
 template <typename TZ, typename TX>
 int launch_dec_zx(hipStream_t st, const DecPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
                   int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
-#define GPTQ_DEC(NW, KS, MR, ATOM) \
-  return launch_dec_inst<NW, KS, MR, ATOM, TZ, TX>(st, p, x, M, pk, R, C, zero, scale, out, wsp)
+#define GPTQ_DEC(NW, KS, MR, ATOM, LOOP) \
+  return launch_dec_inst<NW, KS, MR, ATOM, LOOP, TZ, TX>(st, p, x, M, pk, R, C, zero, scale, out, wsp)
   if (p.mr == 16) {
-    if (p.atom) GPTQ_DEC(8, 4, 16, true);
-    GPTQ_DEC(8, 4, 16, false);
+    if (p.loop && p.atom) GPTQ_DEC(8, 4, 16, true, true);
+    if (p.loop) GPTQ_DEC(8, 4, 16, false, true);
+    if (p.atom) GPTQ_DEC(8, 4, 16, true, false);
+    GPTQ_DEC(8, 4, 16, false, false);
   }
   if (p.mr == 1) {
-    if (p.nw == 16) GPTQ_DEC(16, 2, 1, true);
-    if (p.ks == 1) GPTQ_DEC(8, 1, 1, true);
-    GPTQ_DEC(8, 2, 1, true);
+    if (p.loop) GPTQ_DEC(16, 2, 1, true, true);
+    if (p.nw == 16) GPTQ_DEC(16, 2, 1, true, false);
+    if (p.ks == 1) GPTQ_DEC(8, 1, 1, true, false);
+    GPTQ_DEC(8, 2, 1, true, false);
   }
-  if (p.nw == 16) GPTQ_DEC(16, 2, 4, true);
-  if (p.ks == 1) GPTQ_DEC(8, 1, 4, true);
-  GPTQ_DEC(8, 2, 4, true);
+  if (p.loop) GPTQ_DEC(16, 2, 4, true, true);
+  if (p.nw == 16) GPTQ_DEC(16, 2, 4, true, false);
+  if (p.ks == 1) GPTQ_DEC(8, 1, 4, true, false);
+  GPTQ_DEC(8, 2, 4, true, false);
 #undef GPTQ_DEC
 }
 
