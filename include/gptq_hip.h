@@ -166,6 +166,16 @@ int gptq_hip_dequant(void *stream, const uint8_t *packed, int64_t outer,
                      int64_t packed_axis_len, int64_t inner, const void *zero,
                      const void *scale, int zs_dtype, void *out);
 
+/* The same two for 8-bit codes (no counterpart in the reference, which packs 4-bit codes only,
+ * gptq.py:241,253): bits = 4 is exactly the call above; bits = 8 stores / reads one code per byte,
+ * c = uint8(rint(Q/scale + zero)) clipped to [0, 255], so `packed` has axis_len (quantize) resp.
+ * packed_axis_len (dequant) bytes along the middle axis and the dense tensor has as many elements. */
+int gptq_hip_quantize_pack_bits(void *stream, const void *Q, int q_dtype, int64_t outer, int64_t axis_len,
+                                int64_t inner, const float *scale, const float *zero, int bits,
+                                uint8_t *packed);
+int gptq_hip_dequant_bits(void *stream, const uint8_t *packed, int64_t outer, int64_t packed_axis_len,
+                          int64_t inner, const void *zero, const void *scale, int zs_dtype, int bits, void *out);
+
 /* ---- packed-int4 matmul ------------------------------------------------------------------
  * Replaces the jt.triton_call custom call of _quantized_matmul (op.py:19-69) and the two
  * Triton kernels behind it (kernel.py:17-127, 141-253).
@@ -188,6 +198,19 @@ size_t gptq_hip_qmatmul_workspace_bytes_x(int64_t M, int64_t R, int64_t C, int t
 int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
                      int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype,
                      int transpose_b, void *out, void *ws, size_t ws_bytes);
+
+/* ---- the same product for 8-bit codes -----------------------------------------------------------
+ * No counterpart in the reference, whose packing and kernels are fixed at 4 bits (gptq.py:241,253,
+ * kernel.py:92-104); for the 8-bit codes gptq() can produce here (bits = 8).  bits = 4: exactly
+ * gptq_hip_qmatmul.  bits = 8: packed [R, C] uint8 holds one code per byte, W is [R, C] (Kx = R for
+ * transpose_b = 0, out [M, R] for transpose_b = 1); everything else as above.
+ * ws: gptq_hip_qmatmul_bits_workspace_bytes(M, R, C, transpose_b, x_dtype, bits) bytes, zero-filled before
+ * its first use like the workspace of gptq_hip_qmatmul (one buffer can serve both). */
+size_t gptq_hip_qmatmul_bits_workspace_bytes(int64_t M, int64_t R, int64_t C, int transpose_b, int x_dtype,
+                                             int bits);
+int gptq_hip_qmatmul_bits(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
+                          int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, int bits,
+                          int transpose_b, void *out, void *ws, size_t ws_bytes);
 
 /* ---- packed-int4 matmul that allocates nothing and takes no workspace ----------------------
  * No counterpart in the reference.  For callers that cannot allocate device memory: code under

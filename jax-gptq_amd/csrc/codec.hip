@@ -118,6 +118,33 @@ __global__ __launch_bounds__(TPB) void dequant_kernel(const uint8_t *packed, int
   }
 }
 
+// 8-bit codes: one byte per element, same [outer, axis, inner] view and parameter indexing
+template <typename TQ>
+__global__ __launch_bounds__(TPB) void quantize_codes8_kernel(const TQ *Q, int64_t outer, int64_t alen,
+                                                              int64_t inner, const float *scale,
+                                                              const float *zero, uint8_t *codes) {
+  const int64_t total = outer * alen * inner;
+  for (int64_t idx = (int64_t)blockIdx.x * TPB + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * TPB) {
+    const int64_t i = idx % inner, o = idx / (inner * alen);
+    codes[idx] = code_of(to_f32(Q[idx]), scale[o * inner + i], zero[o * inner + i]);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(TPB) void dequant8_kernel(const uint8_t *codes, int64_t outer, int64_t alen,
+                                                       int64_t inner, const T *zero, const T *scale, T *out) {
+#pragma clang fp contract(off)
+  const int64_t total = outer * alen * inner;
+  for (int64_t idx = (int64_t)blockIdx.x * TPB + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * TPB) {
+    const int64_t i = idx % inner, o = idx / (inner * alen);
+    const float z = to_f32(zero[o * inner + i]), sc = to_f32(scale[o * inner + i]);
+    const float d = to_f32(from_f32<T>((float)codes[idx] - z));
+    out[idx] = from_f32<T>(d * sc);
+  }
+}
+
 // ------------------------------------------------------------------ gathers
 template <typename T>
 __global__ __launch_bounds__(TPB) void gather_rows_kernel(const T *in, T *out, int64_t N,
@@ -281,6 +308,66 @@ int gptq_hip_dequant(void *stream, const uint8_t *packed, int64_t outer,
       hipLaunchKernelGGL(dequant_kernel<__hip_bfloat16>, grid, block, 0, st, packed, outer,
                          packed_axis_len, inner, (const __hip_bfloat16 *)zero,
                          (const __hip_bfloat16 *)scale, (__hip_bfloat16 *)out);
+      break;
+    default:
+      return GPTQ_HIP_EDTYPE;
+  }
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
+int gptq_hip_quantize_pack_bits(void *stream, const void *Q, int q_dtype, int64_t outer, int64_t axis_len,
+                                int64_t inner, const float *scale, const float *zero, int bits,
+                                uint8_t *packed) {
+  if (bits == 4) return gptq_hip_quantize_pack(stream, Q, q_dtype, outer, axis_len, inner, scale, zero, packed);
+  if (bits != 8 || outer < 0 || axis_len < 0 || inner < 0) return GPTQ_HIP_EINVAL;
+  const int64_t total = outer * axis_len * inner;
+  if (total == 0) return GPTQ_HIP_OK;
+  if (!Q || !scale || !zero || !packed) return GPTQ_HIP_EINVAL;
+  hipStream_t st = as_stream(stream);
+  const dim3 grid(grid_for(total)), block(TPB);
+  switch (q_dtype) {
+    case GPTQ_HIP_F32:
+      hipLaunchKernelGGL(quantize_codes8_kernel<float>, grid, block, 0, st, (const float *)Q, outer, axis_len,
+                         inner, scale, zero, packed);
+      break;
+    case GPTQ_HIP_F16:
+      hipLaunchKernelGGL(quantize_codes8_kernel<__half>, grid, block, 0, st, (const __half *)Q, outer, axis_len,
+                         inner, scale, zero, packed);
+      break;
+    case GPTQ_HIP_BF16:
+      hipLaunchKernelGGL(quantize_codes8_kernel<__hip_bfloat16>, grid, block, 0, st, (const __hip_bfloat16 *)Q,
+                         outer, axis_len, inner, scale, zero, packed);
+      break;
+    default:
+      return GPTQ_HIP_EDTYPE;
+  }
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
+int gptq_hip_dequant_bits(void *stream, const uint8_t *packed, int64_t outer, int64_t packed_axis_len,
+                          int64_t inner, const void *zero, const void *scale, int zs_dtype, int bits, void *out) {
+  if (bits == 4) return gptq_hip_dequant(stream, packed, outer, packed_axis_len, inner, zero, scale, zs_dtype, out);
+  if (bits != 8 || outer < 0 || packed_axis_len < 0 || inner < 0) return GPTQ_HIP_EINVAL;
+  const int64_t total = outer * packed_axis_len * inner;
+  if (total == 0) return GPTQ_HIP_OK;
+  if (!packed || !zero || !scale || !out) return GPTQ_HIP_EINVAL;
+  hipStream_t st = as_stream(stream);
+  const dim3 grid(grid_for(total)), block(TPB);
+  switch (zs_dtype) {
+    case GPTQ_HIP_F32:
+      hipLaunchKernelGGL(dequant8_kernel<float>, grid, block, 0, st, packed, outer, packed_axis_len, inner,
+                         (const float *)zero, (const float *)scale, (float *)out);
+      break;
+    case GPTQ_HIP_F16:
+      hipLaunchKernelGGL(dequant8_kernel<__half>, grid, block, 0, st, packed, outer, packed_axis_len, inner,
+                         (const __half *)zero, (const __half *)scale, (__half *)out);
+      break;
+    case GPTQ_HIP_BF16:
+      hipLaunchKernelGGL(dequant8_kernel<__hip_bfloat16>, grid, block, 0, st, packed, outer, packed_axis_len,
+                         inner, (const __hip_bfloat16 *)zero, (const __hip_bfloat16 *)scale,
+                         (__hip_bfloat16 *)out);
       break;
     default:
       return GPTQ_HIP_EDTYPE;

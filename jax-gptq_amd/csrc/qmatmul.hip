@@ -1,35 +1,45 @@
 // Packed-int4 matmul: out = x @ dequant(Wpacked)  (and the transposed form).
 #include "common.h"
+#include "qmm_common.h"
+#include "qmatmul_reg.h"
 #include <mutex>
 #include <type_traits>
 
 namespace {
 
+using namespace qmm;
+
 constexpr int TPB = 256;
 
 // ---------------------------------------------------------------------------- baseline
 // One thread per output element; used for shapes the tuned kernels do not cover.
-template <typename TX, typename TZ>
+template <typename TX, typename TZ, int BITS>
 __global__ __launch_bounds__(TPB) void qmm_fwd_simple(const TX *x, int64_t M, const uint8_t *pk,
                                                       int64_t R, int64_t C, const TZ *zero,
                                                       const TZ *scale, TX *out) {
   const int64_t n = (int64_t)blockIdx.x * TPB + threadIdx.x;
   const int64_t m = blockIdx.y;
   if (n >= C) return;
-  const TX *xr = x + m * (2 * R);
+  const TX *xr = x + m * (BITS == 4 ? 2 * R : R);
   float acc = 0.f, xs = 0.f;
   for (int64_t j = 0; j < R; ++j) {
     const uint8_t b = pk[j * C + n];
-    const float x0 = to_f32(xr[2 * j]), x1 = to_f32(xr[2 * j + 1]);
-    acc += x0 * (float)(b & 0xF) + x1 * (float)(b >> 4);
-    xs += x0 + x1;
+    if (BITS == 4) {
+      const float x0 = to_f32(xr[2 * j]), x1 = to_f32(xr[2 * j + 1]);
+      acc += x0 * (float)(b & 0xF) + x1 * (float)(b >> 4);
+      xs += x0 + x1;
+    } else {
+      const float x0 = to_f32(xr[j]);
+      acc += x0 * (float)b;
+      xs += x0;
+    }
   }
   const float v = to_f32(scale[n]) * (acc - to_f32(zero[n]) * xs);
   out[m * C + n] = from_f32<TX>(__half2float(__float2half_rn(v)));
 }
 
 // transposed: out[m, 2r+p] = sum_c x[m,c] * (nibble_p(pk[r,c]) - zero[c]) * scale[c]
-template <typename TX, typename TZ>
+template <typename TX, typename TZ, int BITS>
 __global__ __launch_bounds__(TPB) void qmm_bwd_simple(const TX *x, int64_t M, const uint8_t *pk,
                                                       int64_t R, int64_t C, const TZ *zero,
                                                       const TZ *scale, TX *out) {
@@ -44,7 +54,7 @@ __global__ __launch_bounds__(TPB) void qmm_bwd_simple(const TX *x, int64_t M, co
     const uint8_t b = pk[r * C + c];
     const float xv = to_f32(xr[c]) * to_f32(scale[c]);
     const float z = to_f32(zero[c]);
-    a0 += xv * ((float)(b & 0xF) - z);
+    a0 += xv * ((float)(BITS == 4 ? (b & 0xF) : b) - z);
     a1 += xv * ((float)(b >> 4) - z);
   }
   for (int off = 32; off > 0; off >>= 1) {
@@ -52,8 +62,12 @@ __global__ __launch_bounds__(TPB) void qmm_bwd_simple(const TX *x, int64_t M, co
     a1 += __shfl_xor(a1, off);
   }
   if (lane == 0) {
-    out[m * (2 * R) + 2 * r] = from_f32<TX>(__half2float(__float2half_rn(a0)));
-    out[m * (2 * R) + 2 * r + 1] = from_f32<TX>(__half2float(__float2half_rn(a1)));
+    if (BITS == 4) {
+      out[m * (2 * R) + 2 * r] = from_f32<TX>(__half2float(__float2half_rn(a0)));
+      out[m * (2 * R) + 2 * r + 1] = from_f32<TX>(__half2float(__float2half_rn(a1)));
+    } else {
+      out[m * R + r] = from_f32<TX>(__half2float(__float2half_rn(a0)));
+    }
   }
 }
 
@@ -77,10 +91,6 @@ __global__ __launch_bounds__(TPB) void qmm_bwd_simple(const TX *x, int64_t M, co
 // and with the two activation sums (kept per lane in fp32) the epilogue computes
 //   out = scale * (acc - 1024*(se + so) - zero * (se + 16*so)),  se = sum_even x, so = sum_odd x/16.
 // No LDS or barrier is used before the final cross-wavefront reduction.
-typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-
 constexpr int QSTRIP = 256;    // channels per workgroup
 
 // LDS layout of one row of a wavefront's partial tile (256 floats): a lane holds the 16 channels
@@ -126,62 +136,6 @@ __device__ __forceinline__ void dequant_pair(const DqConst &k, uint32_t da, uint
     lo = (p & k.mlo) | k.c;
     hi = (p & k.mhi) | k.c;
   }
-}
-
-// 16-bit activation types of the MFMA kernels
-template <typename TX> struct Act;
-template <> struct Act<__half> {
-  static constexpr bool BF = false;
-  static __device__ __forceinline__ float lo(uint32_t w) { return (float)__builtin_bit_cast(half2_t, w)[0]; }
-  static __device__ __forceinline__ float hi(uint32_t w) { return (float)__builtin_bit_cast(half2_t, w)[1]; }
-  static __device__ __forceinline__ floatx4 mma(const uint4 &a, const uint4 &b, floatx4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
-                                                  __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ __half out(float v) { return __float2half_rn(v); }
-};
-template <> struct Act<__hip_bfloat16> {
-  static constexpr bool BF = true;
-  typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
-  static __device__ __forceinline__ float lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
-  static __device__ __forceinline__ float hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xFFFF0000u); }
-  static __device__ __forceinline__ floatx4 mma(const uint4 &a, const uint4 &b, floatx4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, a),
-                                                   __builtin_bit_cast(bf8_t, b), c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ __hip_bfloat16 out(float v) { return __float2bfloat16(v); }
-};
-
-// Workspace layout (only touched when the K range is split over S > 1 workgroups):
-//   [counters: QMM_COUNTER_BYTES, one int32 per (m-chunk, strip), zero between calls; the
-//    size is fixed so that no other region of an earlier call can alias a counter]
-//   [acc64: QMM_ACC_BYTES, see below]
-//   [x1part:  (m-chunk, strip, split, 2, 16) fp32]   [part: (split, M, C) fp32]
-// The last workgroup to finish a strip (atomic ticket) sums the S partials in split order,
-// so the result does not depend on the arrival order, and resets the counter.
-constexpr int QMM_COUNTER_BYTES = 65536;
-constexpr int QMM_MAX_COUNTERS = QMM_COUNTER_BYTES / 4;
-// After the counters: 64-bit accumulators of the decode kernel's split-K sum (M <= 4), one per output,
-// zero between calls like the counters.  Counters and accumulators form the head of every workspace
-// at fixed offsets, whatever the shape, so that calls of different shapes can share one buffer.
-constexpr int QMM_ACC_BYTES = 4 << 20;
-constexpr int QMM_HEAD_BYTES = QMM_COUNTER_BYTES + QMM_ACC_BYTES;
-
-struct QmmWs {
-  int32_t *counters;
-  unsigned long long *acc64;
-  float *x1part;
-  float *part;
-};
-
-__host__ __device__ inline QmmWs qmm_ws(void *base_v, size_t x1_bytes) {
-  char *base = reinterpret_cast<char *>(base_v);
-  QmmWs ws;
-  ws.counters = reinterpret_cast<int32_t *>(base);
-  ws.acc64 = reinterpret_cast<unsigned long long *>(base + QMM_COUNTER_BYTES);
-  ws.x1part = reinterpret_cast<float *>(base + QMM_HEAD_BYTES);
-  ws.part = reinterpret_cast<float *>(base + QMM_HEAD_BYTES + x1_bytes);
-  return ws;
 }
 
 // Cross-wavefront reduction and output of one (m-chunk, strip, split) workgroup.  On entry every
@@ -1269,300 +1223,6 @@ __global__ __launch_bounds__(256, 2) void qmm_fwd_gemm_kernel(const TX *x, int M
   }
 }
 
-// ---------------------------------------------------------------------------- 16 < M <= 256
-// Few rows against a whole matrix: the work is the weights' (every packed byte is dequantised once
-// per 64-row tile) and there are not many output tiles, so a workgroup owns a 64 x 128 output tile
-// over ALL of K and its four wavefronts split K among them (k-step t of 32 k = 16 packed rows goes
-// to wavefront t % 4): no partial results leave the workgroup, the only traffic beyond the inputs
-// is the output.  Both MFMA operands come straight from registers, nothing is staged and the k loop
-// has no barrier:
-//   B: lane (l16, g) loads 8 bytes = 8 channels of the packed rows 4g .. 4g+3 of the k-step; tile t8
-//      is byte t8, the k slots 2i, 2i+1 of the lane are the two nibbles of row 4g + i in natural
-//      order.  Per byte: one byte permute, one and-or under the exponent of 1024, one packed fma
-//      that rescales the high nibble and subtracts 1024 + rint(zero): exact small integers in fp16.
-//      (bf16: 128 + code by shifts and masks, the offset 128 + zero leaves in the epilogue.)
-//   A: lane (l16, g) loads the 16 bytes x[m][32 t + 8 g ..+7] of row m = 16 rb + l16, which is the
-//      operand as it stands.
-// A ring of three k-steps keeps 3 x (4 + 4) loads per lane in flight.  At the end the four partial
-// tiles are summed through LDS (wavefront j writes, wavefront 0 adds), the row sums of x that the
-// fractional part of a zero point (fp16) or the whole offset (bf16) needs are summed the same way.
-constexpr int RK_BMB = 4;                       // 16-row blocks per tile
-constexpr int RK_BM = 16 * RK_BMB;
-constexpr int RK_BN = 128;
-constexpr int RK_RING = 3;
-
-template <typename TZ, typename TX>
-__global__ __launch_bounds__(256) void qmm_fwd_rk_kernel(const TX *x, int M, int K, const uint8_t *pk, int R,
-                                                         int C, const TZ *zero, const TZ *scale, TX *out,
-                                                         QmmWs ws, int S, int steps_per_split) {
-  constexpr bool BF = Act<TX>::BF;
-  extern __shared__ __attribute__((aligned(16))) float rk_lds[];     // [RK_BMB * 8 tiles][64 lanes][4] + row sums
-  const int tid = threadIdx.x, lane = tid & 63, wk = tid >> 6;
-  const int g = lane >> 4, l16 = lane & 15;
-  const int m0 = blockIdx.y * RK_BM, nbase = blockIdx.x * RK_BN, split = blockIdx.z;
-  const int T = (R + 15) >> 4;
-  // this workgroup's k-steps [t_begin, t_end); wavefront wk takes t_begin + wk, + 4, ...
-  const int t_begin = split * steps_per_split, t_end = min(T, t_begin + steps_per_split);
-  const int range = max(0, t_end - t_begin);
-  const int iters = range > wk ? (range - wk + 3) >> 2 : 0;
-
-  const int col = min(nbase + 8 * l16, C - 8);                       // C % 8 == 0
-  const bool col_ok = nbase + 8 * l16 < C;
-  const uint8_t *wp = pk + col;
-  int xrow[RK_BMB];
-#pragma unroll
-  for (int rb = 0; rb < RK_BMB; ++rb) xrow[rb] = min(m0 + 16 * rb + l16, M - 1) * K + 8 * g;   // M K < 2^31
-  uint2 wr[RK_RING][4];
-  uint4 aq[RK_RING][RK_BMB];
-  auto load_step = [&](int slot, int s) __attribute__((always_inline)) {
-    const int t = min(t_begin + 4 * s + wk, T - 1);
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      wr[slot][i] = *reinterpret_cast<const uint2 *>(wp + (int64_t)min(16 * t + 4 * g + i, R - 1) * C);
-    const int koff = min(32 * t, K - 8 - 8 * g);                     // K % 8 == 0: a valid 16-byte chunk
-#pragma unroll
-    for (int rb = 0; rb < RK_BMB; ++rb) aq[slot][rb] = *reinterpret_cast<const uint4 *>(x + xrow[rb] + koff);
-  };
-
-  // -(1024 + rint(zero)), -(64 + rint(zero)) of this lane's 8 channels (fp16 only)
-  uint32_t zc[8];
-#pragma unroll
-  for (int t8 = 0; t8 < 8; ++t8) {
-    const float z = (col_ok && !BF) ? rintf(to_f32(zero[col + t8])) : 0.f;
-    zc[t8] = __builtin_bit_cast(uint32_t, half2_t{(_Float16)(-(1024.f + z)), (_Float16)(-(64.f + z))});
-  }
-  uint32_t mask = BF ? 0x000F000Fu : 0x00F0000Fu, cexp = BF ? 0x43004300u : 0x64006400u;
-  asm volatile("" : "+s"(mask));
-  asm volatile("" : "+v"(cexp));
-  const half2_t unscale = half2_t{(_Float16)1.f, (_Float16)0.0625f};
-
-  floatx4 acc[RK_BMB][8];
-#pragma unroll
-  for (int i = 0; i < RK_BMB; ++i)
-#pragma unroll
-    for (int j = 0; j < 8; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
-  float xsum[RK_BMB];
-#pragma unroll
-  for (int rb = 0; rb < RK_BMB; ++rb) xsum[rb] = 0.f;
-
-#pragma unroll
-  for (int u = 0; u < RK_RING; ++u) load_step(u, u);
-
-  auto compute = [&](int slot, int s) __attribute__((always_inline)) {
-    const bool k_ok = 32 * (t_begin + 4 * s + wk) + 8 * g < K;   // the last k-step may be ragged (K % 32 != 0)
-    uint4 b[8];
-#pragma unroll
-    for (int t8 = 0; t8 < 8; ++t8) {
-      // fp16: the byte in both halves; bf16: in the low half only
-      const uint32_t sel = BF ? (0x0c0c0c00u | (uint32_t)(t8 & 3))
-                              : (0x0c000c00u | (uint32_t)(t8 & 3) | ((uint32_t)(t8 & 3) << 16));
-      uint32_t r4[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const uint32_t w = (t8 < 4) ? wr[slot][i].x : wr[slot][i].y;
-        const uint32_t pb = __builtin_amdgcn_perm(0u, w, sel);
-        if (BF) {
-          r4[i] = (((pb << 12) | pb) & mask) | cexp;                   // {128 + lo, 128 + hi}
-        } else {
-          const uint32_t v = (pb & mask) | cexp;                       // {1024 + lo, 1024 + 16 hi}
-          const half2_t d = __builtin_bit_cast(half2_t, v) * unscale + __builtin_bit_cast(half2_t, zc[t8]);
-          r4[i] = __builtin_bit_cast(uint32_t, d);
-        }
-      }
-      b[t8] = make_uint4(r4[0], r4[1], r4[2], r4[3]);
-    }
-#pragma unroll
-    for (int rb = 0; rb < RK_BMB; ++rb) {
-      uint4 a = aq[slot][rb];
-      a.x = k_ok ? a.x : 0u;
-      a.y = k_ok ? a.y : 0u;
-      a.z = k_ok ? a.z : 0u;
-      a.w = k_ok ? a.w : 0u;
-      xsum[rb] += (Act<TX>::lo(a.x) + Act<TX>::hi(a.x)) + (Act<TX>::lo(a.y) + Act<TX>::hi(a.y)) +
-                  (Act<TX>::lo(a.z) + Act<TX>::hi(a.z)) + (Act<TX>::lo(a.w) + Act<TX>::hi(a.w));
-#pragma unroll
-      for (int t8 = 0; t8 < 8; ++t8) acc[rb][t8] = Act<TX>::mma(a, b[t8], acc[rb][t8]);
-    }
-  };
-  int s0 = 0;
-  for (; s0 + RK_RING <= iters; s0 += RK_RING) {
-#pragma unroll
-    for (int u = 0; u < RK_RING; ++u) {
-      compute(u, s0 + u);
-      load_step(u, s0 + u + RK_RING);
-    }
-  }
-#pragma unroll
-  for (int u = 0; u < RK_RING - 1; ++u)
-    if (s0 + u < iters) compute(u, s0 + u);
-
-  // ---- the four wavefronts' tiles and row sums through LDS
-#pragma unroll
-  for (int rb = 0; rb < RK_BMB; ++rb) {
-    xsum[rb] += __shfl_xor(xsum[rb], 16);
-    xsum[rb] += __shfl_xor(xsum[rb], 32);
-  }
-  float *rowsum = rk_lds + RK_BMB * 8 * 256;       // [4 wavefronts][RK_BM]
-  if (g == 0) {
-#pragma unroll
-    for (int rb = 0; rb < RK_BMB; ++rb) rowsum[wk * RK_BM + 16 * rb + l16] = xsum[rb];
-  }
-  for (int j = 1; j < 4; ++j) {
-    if (wk == j) {
-#pragma unroll
-      for (int rb = 0; rb < RK_BMB; ++rb)
-#pragma unroll
-        for (int t8 = 0; t8 < 8; ++t8)
-          *reinterpret_cast<floatx4 *>(rk_lds + ((rb * 8 + t8) * 64 + lane) * 4) = acc[rb][t8];
-    }
-    __syncthreads();
-    if (wk == 0) {
-#pragma unroll
-      for (int rb = 0; rb < RK_BMB; ++rb)
-#pragma unroll
-        for (int t8 = 0; t8 < 8; ++t8)
-          acc[rb][t8] += *reinterpret_cast<const floatx4 *>(rk_lds + ((rb * 8 + t8) * 64 + lane) * 4);
-    }
-    __syncthreads();
-  }
-  if (wk != 0) return;
-  float rs_lane = (rowsum[lane] + rowsum[RK_BM + lane]) + (rowsum[2 * RK_BM + lane] + rowsum[3 * RK_BM + lane]);
-  if (S > 1) {
-    // Split over K across workgroups: wavefront 0 writes the workgroup's partial tile in register
-    // layout ([rb][t8][r][lane]: 256 bytes contiguous per wavefront store) and the 64 row sums with
-    // agent-scope write-through stores, waits for them, takes an arrival ticket; the last workgroup
-    // of the tile adds the S partials in split order (agent-scope loads), so the sum does not depend
-    // on the arrival order, and leaves the counter at zero.
-    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
-    float *part = ws.part + ((int64_t)tile * S) * (RK_BMB * 8 * 256);
-    float *rsp = ws.x1part + ((int64_t)tile * S) * RK_BM;
-    {
-      float *dst = part + (int64_t)split * (RK_BMB * 8 * 256) + lane;
-#pragma unroll
-      for (int rb = 0; rb < RK_BMB; ++rb)
-#pragma unroll
-        for (int t8 = 0; t8 < 8; ++t8)
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            __hip_atomic_store(dst + ((rb * 8 + t8) * 4 + r) * 64, acc[rb][t8][r], __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(rsp + split * RK_BM + lane, rs_lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // this wavefront's write-through stores have completed
-    int last = 0;
-    if (lane == 0) {
-      int32_t *ctr = ws.counters + tile;
-      const int ticket = atomicAdd(ctr, 1);
-      last = (ticket == S - 1);
-      if (last) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    last = __builtin_amdgcn_readfirstlane(last);
-    if (!last) return;
-    rs_lane = 0.f;
-#pragma unroll
-    for (int rb = 0; rb < RK_BMB; ++rb)
-#pragma unroll
-      for (int t8 = 0; t8 < 8; ++t8) acc[rb][t8] = floatx4{0.f, 0.f, 0.f, 0.f};
-    for (int sp = 0; sp < S; ++sp) {
-      const float *src = part + (int64_t)sp * (RK_BMB * 8 * 256) + lane;
-      rs_lane += __hip_atomic_load(rsp + sp * RK_BM + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-      for (int rb = 0; rb < RK_BMB; ++rb)
-#pragma unroll
-        for (int t8 = 0; t8 < 8; ++t8)
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            acc[rb][t8][r] += __hip_atomic_load(src + ((rb * 8 + t8) * 4 + r) * 64, __ATOMIC_RELAXED,
-                                                __HIP_MEMORY_SCOPE_AGENT);
-    }
-  }
-  // the row sums to where the epilogue's lanes find them (wavefront 0 alone is left: no barrier needed
-  // beyond the LDS counter wait the compiler places)
-  rowsum[lane] = rs_lane;
-  if (!col_ok) return;
-  // acc[rb][t8][r] = sum_k x[m0 + 16 rb + 4 g + r][k] (code - rint(zero))[k][col + t8]
-  float sc[8], zf[8];
-#pragma unroll
-  for (int t8 = 0; t8 < 8; ++t8) {
-    sc[t8] = to_f32(scale[col + t8]);
-    const float z = to_f32(zero[col + t8]);
-    zf[t8] = BF ? 128.f + z : z - rintf(z);
-  }
-#pragma unroll
-  for (int rb = 0; rb < RK_BMB; ++rb)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int ml = 16 * rb + 4 * g + r, m = m0 + ml;
-      if (m >= M) continue;
-      const float rs = rowsum[ml];
-      TX o[8];
-#pragma unroll
-      for (int t8 = 0; t8 < 8; ++t8) o[t8] = Act<TX>::out(sc[t8] * (acc[rb][t8][r] - zf[t8] * rs));
-      *reinterpret_cast<uint4 *>(out + (int64_t)m * C + col) = *reinterpret_cast<const uint4 *>(o);
-    }
-}
-
-// Shapes the register-operand kernel takes: operands aligned for its 8- and 16-byte loads, 32-bit
-// element offsets into x, and enough work per workgroup.  With fewer than ~200 output tiles K is split
-// over S workgroups per tile (at least four k-steps per wavefront).
-struct RkPlan {
-  bool use;
-  int S, steps;
-  int64_t tiles;
-  size_t x1_bytes, part_bytes, total_bytes;
-};
-
-RkPlan rk_plan(int64_t M, int64_t R, int64_t C) {
-  RkPlan p{};
-  if (M <= 16 || M > 256 || C % 8 != 0 || C < 8 || (2 * R) % 8 != 0 || M * 2 * R >= (1LL << 31) ||
-      R >= (1LL << 27))
-    return p;
-  p.tiles = ceil_div64(C, RK_BN) * ceil_div64(M, RK_BM);
-  if (p.tiles > QMM_MAX_COUNTERS) return p;
-  const int64_t T = ceil_div64(R, 16);
-  int64_t S = 1;
-  if (p.tiles < 200) {
-    S = 256 / p.tiles;
-    if (S > 16) S = 16;
-    while (S > 1 && T / S < 16) --S;
-    if (S < 1) S = 1;
-  }
-  if (p.tiles * S < 64) return p;                 // too little to fill the chip: the tiled kernels split finer
-  p.steps = (int)ceil_div64(T, S);
-  p.S = (int)ceil_div64(T, p.steps);
-  p.x1_bytes = p.S > 1 ? (size_t)round_up64(p.tiles * p.S * RK_BM * (int64_t)sizeof(float), 256) : 0;
-  p.part_bytes = p.S > 1 ? (size_t)p.tiles * p.S * RK_BMB * 8 * 64 * 16 : 0;
-  p.total_bytes = p.S > 1 ? QMM_HEAD_BYTES + p.x1_bytes + p.part_bytes : 0;
-  p.use = true;
-  return p;
-}
-
-bool rk_ptrs_ok(int x_dtype, const void *x, const uint8_t *pk, const void *out) {
-  return (x_dtype == GPTQ_HIP_F16 || x_dtype == GPTQ_HIP_BF16) &&
-         ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) & 15) == 0 &&
-         (reinterpret_cast<uintptr_t>(pk) & 7) == 0;
-}
-
-template <typename TZ, typename TX>
-int launch_rk_zx(hipStream_t st, const RkPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
-                 int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
-  constexpr size_t lds = (size_t)(RK_BMB * 8 * 256 + 4 * RK_BM) * sizeof(float);
-  const QmmWs ws = qmm_ws(wsp, p.x1_bytes);
-  const dim3 grid((unsigned)ceil_div64(C, RK_BN), (unsigned)ceil_div64(M, RK_BM), (unsigned)p.S);
-  hipLaunchKernelGGL((qmm_fwd_rk_kernel<TZ, TX>), grid, dim3(256), lds, st, (const TX *)x, (int)M, (int)(2 * R),
-                     pk, (int)R, (int)C, (const TZ *)zero, (const TZ *)scale, (TX *)out, ws, p.S, p.steps);
-  GPTQ_CHECK_LAUNCH();
-  return GPTQ_HIP_OK;
-}
-
-template <typename TZ>
-int launch_rk(hipStream_t st, const RkPlan &p, const void *x, int x_dtype, int64_t M, const uint8_t *pk,
-              int64_t R, int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
-  if (x_dtype == GPTQ_HIP_BF16)
-    return launch_rk_zx<TZ, __hip_bfloat16>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
-  return launch_rk_zx<TZ, __half>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
-}
-
 // Tiled kernel plan: S = 1 when the 64 x 128 output tiles alone fill the chip, else split-K
 // over S workgroups per tile (partials and arrival counters in the workspace, as above).
 struct GemmPlan {
@@ -1965,35 +1625,52 @@ bool fwd_fast_ok(int x_dtype, int64_t M, int64_t R, int64_t C, const void *x, co
          R < (1LL << 30) && C < (1LL << 30);
 }
 
-template <typename TX, typename TZ>
+template <typename TX, typename TZ, int BITS>
 int launch_simple(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
                   const void *zero, const void *scale, int transpose_b, void *out) {
-  if (M > 65535) return GPTQ_HIP_EINVAL;
-  if (!transpose_b) {
-    hipLaunchKernelGGL((qmm_fwd_simple<TX, TZ>), dim3((unsigned)ceil_div64(C, TPB), (unsigned)M),
-                       dim3(TPB), 0, st, (const TX *)x, M, pk, R, C, (const TZ *)zero,
-                       (const TZ *)scale, (TX *)out);
-  } else {
-    hipLaunchKernelGGL((qmm_bwd_simple<TX, TZ>),
-                       dim3((unsigned)ceil_div64(R, TPB / 64), (unsigned)M), dim3(TPB), 0, st,
-                       (const TX *)x, M, pk, R, C, (const TZ *)zero, (const TZ *)scale, (TX *)out);
+  const int64_t kin = transpose_b ? C : (BITS == 4 ? 2 * R : R), nout = transpose_b ? (BITS == 4 ? 2 * R : R) : C;
+  // the rows are the grid's y dimension: 65535 of them per launch
+  for (int64_t r0 = 0; r0 < M; r0 += 65535) {
+    const int64_t rows = M - r0 < 65535 ? M - r0 : 65535;
+    const TX *xs = (const TX *)x + r0 * kin;
+    TX *os = (TX *)out + r0 * nout;
+    if (!transpose_b) {
+      hipLaunchKernelGGL((qmm_fwd_simple<TX, TZ, BITS>), dim3((unsigned)ceil_div64(C, TPB), (unsigned)rows),
+                         dim3(TPB), 0, st, xs, rows, pk, R, C, (const TZ *)zero, (const TZ *)scale, os);
+    } else {
+      hipLaunchKernelGGL((qmm_bwd_simple<TX, TZ, BITS>),
+                         dim3((unsigned)ceil_div64(R, TPB / 64), (unsigned)rows), dim3(TPB), 0, st, xs, rows, pk,
+                         R, C, (const TZ *)zero, (const TZ *)scale, os);
+    }
+    GPTQ_CHECK_LAUNCH();
   }
-  GPTQ_CHECK_LAUNCH();
   return GPTQ_HIP_OK;
 }
 
-template <typename TX>
+template <typename TX, int BITS>
 int dispatch_z(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
                const void *zero, const void *scale, int zs_dtype, int transpose_b, void *out) {
   switch (zs_dtype) {
     case GPTQ_HIP_F32:
-      return launch_simple<TX, float>(st, x, M, pk, R, C, zero, scale, transpose_b, out);
+      return launch_simple<TX, float, BITS>(st, x, M, pk, R, C, zero, scale, transpose_b, out);
     case GPTQ_HIP_F16:
-      return launch_simple<TX, __half>(st, x, M, pk, R, C, zero, scale, transpose_b, out);
+      return launch_simple<TX, __half, BITS>(st, x, M, pk, R, C, zero, scale, transpose_b, out);
     case GPTQ_HIP_BF16:
-      return launch_simple<TX, __hip_bfloat16>(st, x, M, pk, R, C, zero, scale, transpose_b, out);
+      return launch_simple<TX, __hip_bfloat16, BITS>(st, x, M, pk, R, C, zero, scale, transpose_b, out);
     default:
       return GPTQ_HIP_EDTYPE;
+  }
+}
+
+template <int BITS>
+int dispatch_simple(hipStream_t st, const void *x, int x_dtype, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
+                    const void *zero, const void *scale, int zs_dtype, int transpose_b, void *out) {
+  switch (x_dtype) {
+    case GPTQ_HIP_F32: return dispatch_z<float, BITS>(st, x, M, pk, R, C, zero, scale, zs_dtype, transpose_b, out);
+    case GPTQ_HIP_F16: return dispatch_z<__half, BITS>(st, x, M, pk, R, C, zero, scale, zs_dtype, transpose_b, out);
+    case GPTQ_HIP_BF16:
+      return dispatch_z<__hip_bfloat16, BITS>(st, x, M, pk, R, C, zero, scale, zs_dtype, transpose_b, out);
+    default: return GPTQ_HIP_EDTYPE;
   }
 }
 
@@ -2048,22 +1725,47 @@ size_t round_up_256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 }  // namespace
 
-extern "C" size_t gptq_hip_qmatmul_workspace_bytes(int64_t M, int64_t R, int64_t C, int transpose_b);
-
 namespace {
 
-F32Plan f32_plan(int64_t M, int64_t R, int64_t C, int transpose_b) {
+// workspace of a product whose activations are fp16 or bf16
+size_t ws16_bytes(int64_t M, int64_t R, int64_t C, int transpose_b, int bits) {
+  if (M <= 0 || R <= 0 || C <= 0) return 0;
+  if (transpose_b) {
+    const RegBwdPlan bp = reg_bwd_plan(M, R, C, bits, true);
+    return bp.use ? bp.total_bytes : 0;
+  }
+  const RegPlan rp = reg_fwd_plan(M, R, C, bits, true);
+  size_t need = rp.use ? rp.total_bytes : 0;
+  if (bits != 4) return need;
+  // which kernel runs also depends on pointer alignment: enough for any of them
+  const size_t cand[4] = {fwd_plan(M, R, C, false).total_bytes, gemm_plan(M, R, C).total_bytes,
+                          fwd_plan(M, R, C, true).total_bytes, 0};
+  for (size_t c : cand) need = c > need ? c : need;
+  const DecPlan dp = dec_plan(M, R, C);
+  if (dp.use && dp.total_bytes > need) need = dp.total_bytes;
+  return need;
+}
+
+// whether a matrix-core kernel serves this shape for 16-bit activations
+bool has_fast16(int64_t M, int64_t R, int64_t C, int transpose_b, int bits) {
+  if (M < 1 || R >= (1LL << 30) || C >= (1LL << 30)) return false;
+  if (bits == 4 && C % 16 == 0) return true;
+  return transpose_b ? reg_bwd_plan(M, R, C, bits, true).use : reg_fwd_plan(M, R, C, bits, true).use;
+}
+
+F32Plan f32_plan(int64_t M, int64_t R, int64_t C, int transpose_b, int bits) {
   F32Plan p{};
-  p.use = M >= 1 && C % 16 == 0 && R < (1LL << 30) && C < (1LL << 30);
+  p.use = has_fast16(M, R, C, transpose_b, bits);
   if (!p.use) return p;
   p.mc = M < F32_CHUNK_ROWS ? M : F32_CHUNK_ROWS;
   const int64_t tail = M % p.mc;
-  size_t inner = gptq_hip_qmatmul_workspace_bytes(p.mc, R, C, transpose_b);
+  size_t inner = ws16_bytes(p.mc, R, C, transpose_b, bits);
   if (tail) {
-    const size_t t = gptq_hip_qmatmul_workspace_bytes(tail, R, C, transpose_b);
+    const size_t t = ws16_bytes(tail, R, C, transpose_b, bits);
     inner = t > inner ? t : inner;
   }
-  const int64_t kin = transpose_b ? C : 2 * R, nout = transpose_b ? 2 * R : C;
+  const int64_t Kl = bits == 4 ? 2 * R : R;
+  const int64_t kin = transpose_b ? C : Kl, nout = transpose_b ? Kl : C;
   p.inner = inner;
   // the counter region stays out of reach of the staging buffers whatever this call's own product
   // needs: a later call on the same workspace expects its counters to be zero
@@ -2074,59 +1776,35 @@ F32Plan f32_plan(int64_t M, int64_t R, int64_t C, int transpose_b) {
   return p;
 }
 
-}  // namespace
-
-extern "C" {
-
-size_t gptq_hip_qmatmul_workspace_bytes(int64_t M, int64_t R, int64_t C, int transpose_b) {
-  if (transpose_b || M <= 0 || R <= 0 || C <= 0) return 0;
-  // which kernel runs also depends on pointer alignment: enough for either
-  const size_t a = fwd_plan(M, R, C, false).total_bytes, b = gemm_plan(M, R, C).total_bytes;
-  const size_t c = fwd_plan(M, R, C, true).total_bytes;
-  const DecPlan dp = dec_plan(M, R, C);
-  const size_t d = dp.use ? dp.total_bytes : 0;
-  const RkPlan rp = rk_plan(M, R, C);
-  const size_t e = rp.use ? rp.total_bytes : 0;
-  size_t abc = a > b ? (a > c ? a : c) : (b > c ? b : c);
-  if (e > abc) abc = e;
-  return abc > d ? abc : d;
+bool aligned16(const void *a, const void *b) {
+  return ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) == 0;
 }
 
-size_t gptq_hip_qmatmul_workspace_bytes_x(int64_t M, int64_t R, int64_t C, int transpose_b, int x_dtype) {
-  if (M <= 0 || R <= 0 || C <= 0) return 0;
-  if (x_dtype == GPTQ_HIP_F32) {
-    const F32Plan fp = f32_plan(M, R, C, transpose_b);
-    if (fp.use) return fp.total_bytes;
-  }
-  return gptq_hip_qmatmul_workspace_bytes(M, R, C, transpose_b);
-}
-
-int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
-                     int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype,
-                     int transpose_b, void *out, void *ws, size_t ws_bytes) {
-  if (M < 0 || R <= 0 || C <= 0) return GPTQ_HIP_EINVAL;
+int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed, int64_t R, int64_t C,
+                 const void *zero, const void *scale, int zs_dtype, int bits, int transpose_b, void *out, void *ws,
+                 size_t ws_bytes) {
+  if (M < 0 || R <= 0 || C <= 0 || (bits != 4 && bits != 8)) return GPTQ_HIP_EINVAL;
   if (M == 0) return GPTQ_HIP_OK;
   if (!x || !packed || !zero || !scale || !out) return GPTQ_HIP_EINVAL;
   hipStream_t st = as_stream(stream);
   if (x_dtype == GPTQ_HIP_F32) {
-    // through the fp16 kernels, if the shape suits them and the caller sized the workspace for
+    // through the 16-bit kernels, if the shape suits them and the caller sized the workspace for
     // it (gptq_hip_qmatmul_workspace_bytes_x); else the plain fp32 kernels below
-    const F32Plan fp = f32_plan(M, R, C, transpose_b);
-    const uintptr_t align = reinterpret_cast<uintptr_t>(packed) | reinterpret_cast<uintptr_t>(zero) |
-                            reinterpret_cast<uintptr_t>(scale) | reinterpret_cast<uintptr_t>(ws);
-    if (fp.use && ws && ws_bytes >= fp.total_bytes && (align & 15) == 0) {
+    const F32Plan fp = f32_plan(M, R, C, transpose_b, bits);
+    if (fp.use && ws && ws_bytes >= fp.total_bytes && (reinterpret_cast<uintptr_t>(ws) & 15) == 0) {
       char *base = reinterpret_cast<char *>(ws);
       __half *x16 = reinterpret_cast<__half *>(base + fp.x16_off);
       __half *o16 = reinterpret_cast<__half *>(base + fp.o16_off);
       int32_t *rowexp = reinterpret_cast<int32_t *>(base + fp.exp_off);
-      const int64_t kin = transpose_b ? C : 2 * R, nout = transpose_b ? 2 * R : C;
+      const int64_t Kl = bits == 4 ? 2 * R : R;
+      const int64_t kin = transpose_b ? C : Kl, nout = transpose_b ? Kl : C;
       for (int64_t r0 = 0; r0 < M; r0 += fp.mc) {
         const int64_t mm = M - r0 < fp.mc ? M - r0 : fp.mc;
         hipLaunchKernelGGL(x32_to_f16_rows_kernel, dim3((unsigned)mm), dim3(256), 0, st,
                            reinterpret_cast<const float *>(x) + r0 * kin, kin, x16, rowexp);
         GPTQ_CHECK_LAUNCH();
-        const int rc = gptq_hip_qmatmul(stream, x16, GPTQ_HIP_F16, mm, packed, R, C, zero, scale, zs_dtype,
-                                        transpose_b, o16, ws, fp.inner);
+        const int rc = qmatmul_impl(stream, x16, GPTQ_HIP_F16, mm, packed, R, C, zero, scale, zs_dtype, bits,
+                                    transpose_b, o16, ws, fp.inner);
         if (rc) return rc;
         unsigned gx = (unsigned)ceil_div64(nout, 1024);
         if (gx > 64) gx = 64;
@@ -2136,81 +1814,114 @@ int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const 
       }
       return GPTQ_HIP_OK;
     }
+    return bits == 4 ? dispatch_simple<4>(st, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out)
+                     : dispatch_simple<8>(st, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out);
   }
-  // GEMM-shaped work goes to the tiled kernel (split-K when the output tiles alone do not fill
-  // the chip); small M goes through the 16-row chunked kernel.
-  const RkPlan rp = rk_plan(M, R, C);
-  if (!transpose_b && rp.use && rk_ptrs_ok(x_dtype, x, packed, out)) {
+  if (x_dtype != GPTQ_HIP_F16 && x_dtype != GPTQ_HIP_BF16) return GPTQ_HIP_EDTYPE;
+  if (zs_dtype != GPTQ_HIP_F32 && zs_dtype != GPTQ_HIP_F16 && zs_dtype != GPTQ_HIP_BF16) return GPTQ_HIP_EDTYPE;
+  const bool al = aligned16(x, out) && (reinterpret_cast<uintptr_t>(packed) & 7) == 0;
+  const RegPlan rp = transpose_b ? RegPlan{} : reg_fwd_plan(M, R, C, bits, al);
+  auto run_reg_fwd = [&]() -> int {
     if (rp.total_bytes && (!ws || ws_bytes < rp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
-    switch (zs_dtype) {
-      case GPTQ_HIP_F32: return launch_rk<float>(st, rp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
-      case GPTQ_HIP_F16: return launch_rk<__half>(st, rp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
-      case GPTQ_HIP_BF16:
-        return launch_rk<__hip_bfloat16>(st, rp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
-      default: return GPTQ_HIP_EDTYPE;
-    }
-  }
-  const GemmPlan gp = gemm_plan(M, R, C);
-  if (!transpose_b && fwd_fast_ok(x_dtype, M, R, C, x, packed) && gp.use &&
-      (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
-    if (gp.total_bytes && (!ws || ws_bytes < gp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
-    switch (zs_dtype) {
-      case GPTQ_HIP_F32:
-        return launch_fwd_gemm<float>(st, gp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
-      case GPTQ_HIP_F16:
-        return launch_fwd_gemm<__half>(st, gp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
-      case GPTQ_HIP_BF16:
-        return launch_fwd_gemm<__hip_bfloat16>(st, gp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
-      default: return GPTQ_HIP_EDTYPE;
-    }
-  }
-  if (transpose_b && bwd_fast_ok(x_dtype, M, R, C, x, packed, zero, scale)) {
-    switch (zs_dtype) {
-      case GPTQ_HIP_F32: return launch_bwd_gemm<float>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
-      case GPTQ_HIP_F16: return launch_bwd_gemm<__half>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
-      case GPTQ_HIP_BF16:
-        return launch_bwd_gemm<__hip_bfloat16>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
-      default: return GPTQ_HIP_EDTYPE;
-    }
-  }
-  if (!transpose_b && fwd_fast_ok(x_dtype, M, R, C, x, packed) && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
-    const DecPlan dp = dec_plan(M, R, C);
-    if (dp.use) {
-      if (dp.total_bytes && (!ws || ws_bytes < dp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+    return reg_fwd_launch(st, rp, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, out, ws);
+  };
+  if (bits == 4 && !transpose_b) {
+    // few rows against a whole matrix (16 < M <= 256): the register-operand kernel, unless its tiles are too
+    // few to fill the chip even when split (the tiled kernel below splits finer)
+    if (rp.use && !rp.ragged && M > 16 && M <= 256 && rp.tiles * rp.S >= 64) return run_reg_fwd();
+    // GEMM-shaped work goes to the tiled kernel (split-K when the output tiles alone do not fill
+    // the chip); small M goes through the decode kernel or the 16-row chunked kernels.
+    const GemmPlan gp = gemm_plan(M, R, C);
+    if (fwd_fast_ok(x_dtype, M, R, C, x, packed) && gp.use && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+      if (gp.total_bytes && (!ws || ws_bytes < gp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
       switch (zs_dtype) {
-        case GPTQ_HIP_F32: return launch_dec_z<float>(st, dp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
-        case GPTQ_HIP_F16: return launch_dec_z<__half>(st, dp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
-        case GPTQ_HIP_BF16:
-          return launch_dec_z<__hip_bfloat16>(st, dp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
-        default: return GPTQ_HIP_EDTYPE;
+        case GPTQ_HIP_F32:
+          return launch_fwd_gemm<float>(st, gp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
+        case GPTQ_HIP_F16:
+          return launch_fwd_gemm<__half>(st, gp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
+        default:
+          return launch_fwd_gemm<__hip_bfloat16>(st, gp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
+      }
+    }
+    if (fwd_fast_ok(x_dtype, M, R, C, x, packed) && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+      const DecPlan dp = dec_plan(M, R, C);
+      if (dp.use) {
+        if (dp.total_bytes && (!ws || ws_bytes < dp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+        switch (zs_dtype) {
+          case GPTQ_HIP_F32: return launch_dec_z<float>(st, dp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
+          case GPTQ_HIP_F16: return launch_dec_z<__half>(st, dp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
+          default:
+            return launch_dec_z<__hip_bfloat16>(st, dp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
+        }
+      }
+    }
+    if (fwd_fast_ok(x_dtype, M, R, C, x, packed)) {
+      const FwdPlan p = fwd_plan(M, R, C, (reinterpret_cast<uintptr_t>(x) & 15) == 0);
+      if (p.total_bytes && (!ws || ws_bytes < p.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+      switch (zs_dtype) {
+        case GPTQ_HIP_F32:
+          return launch_fwd_mfma_z<float>(st, p, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
+        case GPTQ_HIP_F16:
+          return launch_fwd_mfma_z<__half>(st, p, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
+        default:
+          return launch_fwd_mfma_z<__hip_bfloat16>(st, p, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
       }
     }
   }
-  if (!transpose_b && fwd_fast_ok(x_dtype, M, R, C, x, packed)) {
-    const FwdPlan p = fwd_plan(M, R, C, (reinterpret_cast<uintptr_t>(x) & 15) == 0);
-    if (p.total_bytes && (!ws || ws_bytes < p.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+  if (bits == 4 && transpose_b && bwd_fast_ok(x_dtype, M, R, C, x, packed, zero, scale)) {
     switch (zs_dtype) {
-      case GPTQ_HIP_F32:
-        return launch_fwd_mfma_z<float>(st, p, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
-      case GPTQ_HIP_F16:
-        return launch_fwd_mfma_z<__half>(st, p, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
-      case GPTQ_HIP_BF16:
-        return launch_fwd_mfma_z<__hip_bfloat16>(st, p, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
-      default:
-        return GPTQ_HIP_EDTYPE;
+      case GPTQ_HIP_F32: return launch_bwd_gemm<float>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
+      case GPTQ_HIP_F16: return launch_bwd_gemm<__half>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
+      default: return launch_bwd_gemm<__hip_bfloat16>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
     }
   }
-  switch (x_dtype) {
-    case GPTQ_HIP_F32:
-      return dispatch_z<float>(st, x, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out);
-    case GPTQ_HIP_F16:
-      return dispatch_z<__half>(st, x, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out);
-    case GPTQ_HIP_BF16:
-      return dispatch_z<__hip_bfloat16>(st, x, M, packed, R, C, zero, scale, zs_dtype, transpose_b,
-                                        out);
-    default:
-      return GPTQ_HIP_EDTYPE;
+  // 8-bit codes, and 4-bit shapes whose rows are not multiples of 16 channels or that are not aligned
+  if (!transpose_b && rp.use) return run_reg_fwd();
+  if (transpose_b) {
+    const RegBwdPlan bp = reg_bwd_plan(M, R, C, bits, al);
+    if (bp.use) {
+      if (bp.total_bytes && (!ws || ws_bytes < bp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+      return reg_bwd_launch(st, bp, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, out, ws);
+    }
   }
+  return bits == 4 ? dispatch_simple<4>(st, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out)
+                   : dispatch_simple<8>(st, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out);
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t gptq_hip_qmatmul_workspace_bytes(int64_t M, int64_t R, int64_t C, int transpose_b) {
+  return ws16_bytes(M, R, C, transpose_b, 4);
+}
+
+size_t gptq_hip_qmatmul_workspace_bytes_x(int64_t M, int64_t R, int64_t C, int transpose_b, int x_dtype) {
+  return gptq_hip_qmatmul_bits_workspace_bytes(M, R, C, transpose_b, x_dtype, 4);
+}
+
+size_t gptq_hip_qmatmul_bits_workspace_bytes(int64_t M, int64_t R, int64_t C, int transpose_b, int x_dtype,
+                                             int bits) {
+  if (M <= 0 || R <= 0 || C <= 0 || (bits != 4 && bits != 8)) return 0;
+  if (x_dtype == GPTQ_HIP_F32) {
+    const F32Plan fp = f32_plan(M, R, C, transpose_b, bits);
+    if (fp.use) return fp.total_bytes;
+  }
+  return ws16_bytes(M, R, C, transpose_b, bits);
+}
+
+int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
+                     int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype,
+                     int transpose_b, void *out, void *ws, size_t ws_bytes) {
+  return qmatmul_impl(stream, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, 4, transpose_b, out, ws,
+                      ws_bytes);
+}
+
+int gptq_hip_qmatmul_bits(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
+                          int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, int bits,
+                          int transpose_b, void *out, void *ws, size_t ws_bytes) {
+  return qmatmul_impl(stream, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, bits, transpose_b, out, ws,
+                      ws_bytes);
 }
 
 }  // extern "C"

@@ -1,0 +1,36 @@
+// Register-operand packed-weight matmul kernels (qmatmul_reg.hip), as the dispatcher in qmatmul.hip sees them.
+#pragma once
+#include "common.h"
+
+namespace qmm {
+
+// Plan of one forward product out[M, C] = x[M, K] @ dequant(packed[R, C]); bits = 4 (K = 2 R, two codes
+// per byte along the rows) or 8 (K = R, one code per byte).
+struct RegPlan {
+  bool use;
+  int bits, rb;            // rb: 16-row blocks per output tile (1 for M <= 16, else 4)
+  bool ragged;             // C % 8 != 0, K % 8 != 0 or operands not 16-byte aligned: unaligned loads, element stores
+  int S, steps;            // split of the contraction over S workgroups per tile, k-steps (32 k) per split
+  int64_t tiles;           // output tiles of one launch
+  size_t part_bytes, total_bytes;
+};
+
+RegPlan reg_fwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned);
+// x / out element type x_dtype (F16 or BF16), zero / scale element type zs_dtype (F32, F16, BF16)
+int reg_fwd_launch(hipStream_t st, const RegPlan &p, const void *x, int x_dtype, int64_t M, const uint8_t *pk,
+                   int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws);
+
+// Transposed product out[M, K] = x[M, C] @ dequant(packed[R, C])^T.
+struct RegBwdPlan {
+  bool use;
+  int bits;
+  bool ragged;
+  int S, steps;
+  int64_t tiles;
+  size_t part_bytes, total_bytes;
+};
+RegBwdPlan reg_bwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned);
+int reg_bwd_launch(hipStream_t st, const RegBwdPlan &p, const void *x, int x_dtype, int64_t M, const uint8_t *pk,
+                   int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws);
+
+}  // namespace qmm

@@ -1,0 +1,310 @@
+// Packed-weight matmul, forward, with both MFMA operands built in registers:
+//   out[M, C] = x[M, K] @ ((code - zero) * scale),  codes packed as 4-bit pairs (K = 2 R) or bytes (K = R).
+// Serves what the tuned 4-bit kernels of qmatmul.hip do not: 8-bit codes (any M), shapes whose rows are
+// not 8- or 16-byte multiples (C % 8 != 0, e.g. a vocabulary-sized C; K % 8 != 0; unaligned operands), and
+// for 4-bit codes the range 16 < M <= 256, where the work is the weights' and the output tiles are few.
+//
+// A workgroup owns a (16 RB) x 128 output tile over a range of k-steps (all of K unless the contraction is
+// split over S workgroups) and its four wavefronts split those k-steps among them (k-step t of 32 k goes to
+// wavefront t % 4): nothing is staged in LDS and the k loop has no barrier.
+//   B: lane (l16, g) loads 8 bytes = 8 channels of each packed row that holds its 8 k of the k-step
+//      (4-bit: rows 4g .. 4g+3, 8-bit: rows 8g .. 8g+7); the MFMA tile t8 takes byte t8 of every row.
+//      4-bit, fp16: byte permute, and-or under the exponent of 1024, one packed fma that rescales the high
+//      nibble and subtracts 1024 + rint(zero): exact small integers.  4-bit, bf16: 128 + code by shifts and
+//      masks, the offset 128 + zero leaves in the epilogue.  8-bit, fp16: byte permute of two rows, or with
+//      the exponent of 1024, one packed add of -(1024 + rint(zero)).  8-bit, bf16: byte -> fp32, minus
+//      rint(zero), rounded to bf16 (exact: magnitude <= 255).
+//   A: lane (l16, g) loads the 16 bytes x[m][32 t + 8 g ..+7] of row m = 16 rb + l16: the operand as it stands.
+// A ninth tile per row block multiplies the activations with ones: the row sums of x that the epilogue
+// needs for the part of the zero point not folded into B (its fraction; for 4-bit bf16 all of 128 + zero).
+// Out-of-range rows, channels and k are handled by clamped addresses: loads never leave the operands.
+#include "qmatmul_reg.h"
+#include "qmm_reg_common.h"
+#include <type_traits>
+
+namespace {
+
+using namespace qmm;
+
+constexpr int RG_BN = 128;                       // channels per output tile
+
+template <int BITS, int RB, int RING, bool RAGGED, typename TX>
+__global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, int K, const uint8_t *pk, int R,
+                                                          int C, const void *zero, const void *scale,
+                                                          int zs_dtype, TX *out, float *part, int32_t *counters,
+                                                          int S, int steps_per_split) {
+  constexpr bool BF = Act<TX>::BF;
+  constexpr int NL = BITS == 4 ? 4 : 8;          // packed rows per lane and k-step
+  constexpr int PR = 4 * NL;                     // packed rows per k-step
+  extern __shared__ __attribute__((aligned(16))) float rg_lds[];   // [4 wavefronts][RB][RG_NT][64 lanes][4]
+  __shared__ int s_flag;
+  const int tid = threadIdx.x, lane = tid & 63, wk = tid >> 6;
+  const int g = lane >> 4, l16 = lane & 15;
+  const int m0 = blockIdx.y * (16 * RB), nbase = blockIdx.x * RG_BN, split = blockIdx.z;
+  const int T = (K + 31) >> 5;
+  // this workgroup's k-steps [t_begin, t_end); wavefront wk takes t_begin + wk, + 4, ...
+  const int t_begin = split * steps_per_split, t_end = min(T, t_begin + steps_per_split);
+  const int range = max(0, t_end - t_begin);
+  const int iters = range > wk ? (range - wk + 3) >> 2 : 0;
+  // a ragged last k-step (K % 32 != 0) is multiplied after the loop, with masked activations
+  const bool has_tail = (K & 31) != 0 && iters > 0 && (t_begin + 4 * (iters - 1) + wk == T - 1);
+  const int iters_full = iters - (has_tail ? 1 : 0);
+
+  const int col = nbase + 8 * l16;
+  const bool col_ok = col < C;
+  const int colc = min(col, C - 8);                                   // C >= 8
+  const int wshift = (RAGGED && col_ok) ? col - colc : 0;             // bytes to drop from a load at colc
+  const uint8_t *wp = pk + colc;
+  int xrow[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) xrow[rb] = min(m0 + 16 * rb + l16, M - 1) * K;      // M K < 2^31
+
+  uint2 wr[RING][NL];
+  uint4 aq[RING][RB];
+  auto load_step = [&](int slot, int s) __attribute__((always_inline)) {
+    const int t = min(t_begin + 4 * s + wk, T - 1);
+#pragma unroll
+    for (int i = 0; i < NL; ++i)
+      wr[slot][i] = rg_load8<RAGGED>(wp + (int64_t)min(PR * t + NL * g + i, R - 1) * C);
+    const int koff = min(32 * t + 8 * g, K - 8);                      // K >= 8: a chunk inside the row
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) aq[slot][rb] = rg_load16<RAGGED>(x + xrow[rb] + koff);
+  };
+
+  // ---- per-channel constants of the dequantisation (the integer part of the zero point)
+  uint32_t zc[8];
+  float zi8[(BF && BITS == 8) ? 8 : 1];
+#pragma unroll
+  for (int t8 = 0; t8 < 8; ++t8) {
+    const float z = rg_param(zero, zs_dtype, min(col + t8, C - 1));
+    const float zi = fminf(fmaxf(rintf(z), -512.f), 512.f);
+    if constexpr (BF) {
+      zc[t8] = 0u;
+      if constexpr (BITS == 8) zi8[t8] = zi;
+    } else if constexpr (BITS == 4) {
+      zc[t8] = __builtin_bit_cast(uint32_t, half2_t{(_Float16)(-(1024.f + zi)), (_Float16)(-(64.f + zi))});
+    } else {
+      zc[t8] = __builtin_bit_cast(uint32_t, half2_t{(_Float16)(-(1024.f + zi)), (_Float16)(-(1024.f + zi))});
+    }
+  }
+  uint32_t mask = BF ? 0x000F000Fu : 0x00F0000Fu, cexp = BF ? 0x43004300u : 0x64006400u;
+  asm volatile("" : "+s"(mask));
+  asm volatile("" : "+v"(cexp));
+  const half2_t unscale = half2_t{(_Float16)1.f, (_Float16)0.0625f};
+  const uint32_t one2 = BF ? 0x3F803F80u : 0x3C003C00u;
+  const uint4 ones = make_uint4(one2, one2, one2, one2);
+
+  floatx4 acc[RB][RG_NT];
+#pragma unroll
+  for (int i = 0; i < RB; ++i)
+#pragma unroll
+    for (int j = 0; j < RG_NT; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+  for (int u = 0; u < RING; ++u) load_step(u, u);
+
+  auto compute = [&](int slot, auto masked) __attribute__((always_inline)) {
+    uint4 a[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      a[rb] = aq[slot][rb];
+      if (decltype(masked)::value) {
+        const int k0 = 32 * (T - 1) + 8 * g;
+        a[rb] = rg_mask_tail(a[rb], k0, min(k0, K - 8), K);
+      }
+    }
+    uint2 w[NL];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) w[i] = RAGGED ? rg_shr_bytes(wr[slot][i], wshift) : wr[slot][i];
+#pragma unroll
+    for (int t8 = 0; t8 < 8; ++t8) {
+      const uint32_t tb = (uint32_t)(t8 & 3);
+      uint32_t r4[4];
+      if constexpr (BITS == 4) {
+        // fp16: the byte in both halves; bf16: in the low half only
+        const uint32_t sel = BF ? (0x0c0c0c00u | tb) : (0x0c000c00u | tb | (tb << 16));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t pb = __builtin_amdgcn_perm(0u, t8 < 4 ? w[i].x : w[i].y, sel);
+          if (BF) {
+            r4[i] = (((pb << 12) | pb) & mask) | cexp;                   // {128 + lo, 128 + hi}
+          } else {
+            const uint32_t v = (pb & mask) | cexp;                       // {1024 + lo, 1024 + 16 hi}
+            const half2_t d = __builtin_bit_cast(half2_t, v) * unscale + __builtin_bit_cast(half2_t, zc[t8]);
+            r4[i] = __builtin_bit_cast(uint32_t, d);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t wa = t8 < 4 ? w[2 * i].x : w[2 * i].y, wb = t8 < 4 ? w[2 * i + 1].x : w[2 * i + 1].y;
+          if constexpr (BF) {
+            typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
+            typedef float f2_t __attribute__((ext_vector_type(2)));
+            const float fa = (float)((wa >> (8 * tb)) & 0xFFu) - zi8[t8];
+            const float fb = (float)((wb >> (8 * tb)) & 0xFFu) - zi8[t8];
+            r4[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f2_t{fa, fb}, bf2_t));
+          } else {
+            const uint32_t pb = __builtin_amdgcn_perm(wb, wa, 0x0c000c00u | ((4u + tb) << 16) | tb);
+            const half2_t d = __builtin_bit_cast(half2_t, pb | cexp) + __builtin_bit_cast(half2_t, zc[t8]);
+            r4[i] = __builtin_bit_cast(uint32_t, d);
+          }
+        }
+      }
+      const uint4 b = make_uint4(r4[0], r4[1], r4[2], r4[3]);
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) acc[rb][t8] = Act<TX>::mma(a[rb], b, acc[rb][t8]);
+    }
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) acc[rb][8] = Act<TX>::mma(a[rb], ones, acc[rb][8]);
+  };
+  const std::integral_constant<bool, false> plain{};
+  const std::integral_constant<bool, true> tail{};
+  int s0 = 0;
+  for (; s0 + RING <= iters_full; s0 += RING) {
+#pragma unroll
+    for (int u = 0; u < RING; ++u) {
+      compute(u, plain);
+      load_step(u, s0 + u + RING);
+    }
+  }
+  // at most RING - 1 full k-steps left, all of them loaded; then the ragged one
+#pragma unroll
+  for (int u = 0; u < RING - 1; ++u)
+    if (s0 + u < iters_full) compute(u, plain);
+  if (has_tail) {
+    const int slot = iters_full - s0;            // 0 .. RING - 1
+#pragma unroll
+    for (int u = 0; u < RING; ++u)
+      if (u == slot) compute(u, tail);
+  }
+
+  floatx4 sum[RG_NT];
+  const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+  if (!rg_reduce<RB>(acc, sum, rg_lds, &s_flag, part, counters, tile, split, S)) return;
+  // sum[t8][r] = sum_k x[m][k] (code - zi)[k][col + t8] (bf16, 4-bit: code + 128), sum[8][r] = sum_k x[m][k],
+  // m = m0 + 16 rb + 4 g + r
+  if (!col_ok) return;
+  const int rb = RB == 4 ? wk : 0;
+  float sc[8], zf[8];
+#pragma unroll
+  for (int t8 = 0; t8 < 8; ++t8) {
+    const int n = min(col + t8, C - 1);
+    sc[t8] = rg_param(scale, zs_dtype, n);
+    const float z = rg_param(zero, zs_dtype, n);
+    zf[t8] = (BF && BITS == 4) ? 128.f + z : z - fminf(fmaxf(rintf(z), -512.f), 512.f);
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int m = m0 + 16 * rb + 4 * g + r;
+    if (m >= M) continue;
+    const float rs = sum[8][r];
+    TX o[8];
+#pragma unroll
+    for (int t8 = 0; t8 < 8; ++t8) o[t8] = Act<TX>::out(sc[t8] * (sum[t8][r] - zf[t8] * rs));
+    TX *dst = out + (int64_t)m * C + col;
+    if (RAGGED) {
+#pragma unroll
+      for (int t8 = 0; t8 < 8; ++t8)
+        if (col + t8 < C) dst[t8] = o[t8];
+    } else {
+      *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(o);
+    }
+  }
+}
+
+template <int BITS, int RB, int RING, bool RAGGED, typename TX>
+int launch_inst(hipStream_t st, const RegPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
+                int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *wsp) {
+  constexpr size_t lds = (size_t)4 * RB * RG_NT * RG_TILE_FLOATS * sizeof(float);
+  auto kern = qmm_fwd_reg_kernel<BITS, RB, RING, RAGGED, TX>;
+  // the LDS limit of a kernel is raised once per device and instantiation (a repeated or concurrent call
+  // sets the same value again, which is harmless)
+  static bool attr_set[64] = {};
+  int dev = 0;
+  if (lds > 64 * 1024 && (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64 || !attr_set[dev])) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess)
+      return GPTQ_HIP_ELAUNCH;
+    if (dev >= 0 && dev < 64) attr_set[dev] = true;
+  }
+  const int64_t K = BITS == 4 ? 2 * R : R;
+  int32_t *counters = reinterpret_cast<int32_t *>(wsp);
+  float *part = reinterpret_cast<float *>(reinterpret_cast<char *>(wsp) + QMM_HEAD_BYTES);
+  const int64_t tiles_x = ceil_div64(C, RG_BN);
+  // rows per launch: 32-bit element offsets into x, grid.y, one arrival counter per tile, the partial region
+  int64_t rows_max = ((1LL << 31) - 1) / K;
+  if (rows_max > 65535LL * 16 * RB) rows_max = 65535LL * 16 * RB;
+  const int64_t tiles_y_max = p.tiles / tiles_x;                       // what the plan sized the workspace for
+  if (rows_max > tiles_y_max * 16 * RB) rows_max = tiles_y_max * 16 * RB;
+  rows_max -= rows_max % (16 * RB);
+  if (rows_max < 16 * RB) return GPTQ_HIP_EINVAL;
+  for (int64_t r0 = 0; r0 < M; r0 += rows_max) {
+    const int64_t rows = M - r0 < rows_max ? M - r0 : rows_max;
+    const dim3 grid((unsigned)tiles_x, (unsigned)ceil_div64(rows, 16 * RB), (unsigned)p.S);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (const TX *)x + r0 * K, (int)rows, (int)K, pk, (int)R,
+                       (int)C, zero, scale, zs_dtype, (TX *)out + r0 * C, part, counters, p.S, p.steps);
+    GPTQ_CHECK_LAUNCH();
+  }
+  return GPTQ_HIP_OK;
+}
+
+template <int BITS, typename TX>
+int launch_bx(hipStream_t st, const RegPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
+              const void *zero, const void *scale, int zs_dtype, void *out, void *ws) {
+  // a ring of three k-steps for 64-row tiles (registers), of six for the 16-row tiles of the decode case
+  if (p.rb == 4) {
+    if (p.ragged) return launch_inst<BITS, 4, 3, true, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+    return launch_inst<BITS, 4, 3, false, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+  }
+  if (p.ragged) return launch_inst<BITS, 1, 6, true, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+  return launch_inst<BITS, 1, 6, false, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+}
+
+}  // namespace
+
+namespace qmm {
+
+RegPlan reg_fwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned) {
+  RegPlan p{};
+  const int64_t K = bits == 4 ? 2 * R : R;
+  if ((bits != 4 && bits != 8) || M < 1 || C < 8 || K < 8 || R >= (1LL << 30) || C >= (1LL << 30)) return p;
+  p.bits = bits;
+  p.rb = M <= 16 ? 1 : 4;
+  p.ragged = !aligned || C % 8 != 0 || K % 8 != 0;
+  const int64_t tiles_x = ceil_div64(C, RG_BN);
+  if (tiles_x > QMM_MAX_COUNTERS) return p;
+  int64_t tiles_y = ceil_div64(M, 16 * p.rb);
+  if (tiles_y > QMM_MAX_COUNTERS / tiles_x) tiles_y = QMM_MAX_COUNTERS / tiles_x;    // further rows: further launches
+  p.tiles = tiles_x * tiles_y;
+  const int64_t T = ceil_div64(K, 32);
+  // workgroups wanted: one per CU for 64-row tiles (their registers allow no more), two for 16-row tiles;
+  // every wavefront of a split keeps at least four k-steps
+  const int64_t want = p.rb == 4 ? 256 : 512;
+  int64_t S = 1;
+  if (p.tiles < want) {
+    S = want / p.tiles;
+    if (S > 32) S = 32;
+    while (S > 1 && T / S < 16) --S;
+  }
+  p.steps = (int)ceil_div64(T, S);
+  p.S = (int)ceil_div64(T, p.steps);
+  p.part_bytes = p.S > 1 ? (size_t)p.tiles * p.S * p.rb * RG_NT * RG_TILE_FLOATS * sizeof(float) : 0;
+  p.total_bytes = p.S > 1 ? QMM_HEAD_BYTES + p.part_bytes : 0;
+  p.use = true;
+  return p;
+}
+
+int reg_fwd_launch(hipStream_t st, const RegPlan &p, const void *x, int x_dtype, int64_t M, const uint8_t *pk,
+                   int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws) {
+  if (zs_dtype != GPTQ_HIP_F32 && zs_dtype != GPTQ_HIP_F16 && zs_dtype != GPTQ_HIP_BF16) return GPTQ_HIP_EDTYPE;
+  if (x_dtype == GPTQ_HIP_BF16) {
+    if (p.bits == 4) return launch_bx<4, __hip_bfloat16>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+    return launch_bx<8, __hip_bfloat16>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+  }
+  if (x_dtype != GPTQ_HIP_F16) return GPTQ_HIP_EDTYPE;
+  if (p.bits == 4) return launch_bx<4, __half>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+  return launch_bx<8, __half>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+}
+
+}  // namespace qmm

@@ -1,0 +1,67 @@
+// Types, activation traits and the workspace layout shared by the packed-weight matmul kernels.
+#pragma once
+#include "common.h"
+
+namespace qmm {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// 16-bit activation types of the MFMA kernels
+template <typename TX> struct Act;
+template <> struct Act<__half> {
+  static constexpr bool BF = false;
+  static __device__ __forceinline__ float lo(uint32_t w) { return (float)__builtin_bit_cast(half2_t, w)[0]; }
+  static __device__ __forceinline__ float hi(uint32_t w) { return (float)__builtin_bit_cast(half2_t, w)[1]; }
+  static __device__ __forceinline__ floatx4 mma(const uint4 &a, const uint4 &b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
+                                                  __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ __half out(float v) { return __float2half_rn(v); }
+};
+template <> struct Act<__hip_bfloat16> {
+  static constexpr bool BF = true;
+  typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
+  static __device__ __forceinline__ float lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+  static __device__ __forceinline__ float hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xFFFF0000u); }
+  static __device__ __forceinline__ floatx4 mma(const uint4 &a, const uint4 &b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, a),
+                                                   __builtin_bit_cast(bf8_t, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ __hip_bfloat16 out(float v) { return __float2bfloat16(v); }
+};
+
+// Workspace layout (only touched when the K range is split over S > 1 workgroups):
+//   [counters: QMM_COUNTER_BYTES, one int32 per (m-chunk, strip), zero between calls; the
+//    size is fixed so that no other region of an earlier call can alias a counter]
+//   [acc64: QMM_ACC_BYTES, see below]
+//   [x1part:  (m-chunk, strip, split, 2, 16) fp32]   [part: (split, M, C) fp32]
+// The last workgroup to finish a strip (atomic ticket) sums the S partials in split order,
+// so the result does not depend on the arrival order, and resets the counter.
+constexpr int QMM_COUNTER_BYTES = 65536;
+constexpr int QMM_MAX_COUNTERS = QMM_COUNTER_BYTES / 4;
+// After the counters: 64-bit accumulators of the decode kernel's split-K sum (M <= 4), one per output,
+// zero between calls like the counters.  Counters and accumulators form the head of every workspace
+// at fixed offsets, whatever the shape, so that calls of different shapes can share one buffer.
+constexpr int QMM_ACC_BYTES = 4 << 20;
+constexpr int QMM_HEAD_BYTES = QMM_COUNTER_BYTES + QMM_ACC_BYTES;
+
+struct QmmWs {
+  int32_t *counters;
+  unsigned long long *acc64;
+  float *x1part;
+  float *part;
+};
+
+__host__ __device__ inline QmmWs qmm_ws(void *base_v, size_t x1_bytes) {
+  char *base = reinterpret_cast<char *>(base_v);
+  QmmWs ws;
+  ws.counters = reinterpret_cast<int32_t *>(base);
+  ws.acc64 = reinterpret_cast<unsigned long long *>(base + QMM_COUNTER_BYTES);
+  ws.x1part = reinterpret_cast<float *>(base + QMM_HEAD_BYTES);
+  ws.part = reinterpret_cast<float *>(base + QMM_HEAD_BYTES + x1_bytes);
+  return ws;
+}
+
+}  // namespace qmm

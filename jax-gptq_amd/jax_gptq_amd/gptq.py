@@ -64,13 +64,17 @@ def _ws(nbytes):
 
 class QuantizedMatrix:
     """Packed matrix container (reference ``gptq.py:8-22``): ``int_weight`` uint8 with two
-    4-bit codes per byte along ``contraction_axis``, per-channel ``zero`` and ``scale``."""
+    4-bit codes per byte along ``contraction_axis``, per-channel ``zero`` and ``scale``.
+    ``bits`` (not in the reference, which is fixed at 4): 8 means one code per byte."""
 
-    def __init__(self, int_weight, zero, scale, contraction_axis=0):
+    def __init__(self, int_weight, zero, scale, contraction_axis=0, bits=4):
+        if bits not in (4, 8):
+            raise ValueError("bits must be 4 or 8")
         self.int_weight = int_weight
         self.zero = zero
         self.scale = scale
         self.contraction_axis = contraction_axis
+        self.bits = bits
 
     @property
     def shape(self):
@@ -82,11 +86,13 @@ class QuantizedMatrix:
 
     # pytree-style helpers (the reference registers the class as a pytree, gptq.py:24-32)
     def tree_flatten(self):
-        return (self.int_weight, self.zero, self.scale), self.contraction_axis
+        aux = self.contraction_axis if self.bits == 4 else (self.contraction_axis, self.bits)
+        return (self.int_weight, self.zero, self.scale), aux
 
     @classmethod
-    def tree_unflatten(cls, contraction_axis, children):
-        return cls(*children, contraction_axis=contraction_axis)
+    def tree_unflatten(cls, aux, children):
+        axis, bits = aux if isinstance(aux, tuple) else (aux, 4)
+        return cls(*children, contraction_axis=axis, bits=bits)
 
     def to(self, *args, **kwargs):
         """Move to a device.  Element-type requests are ignored: a cast of a packed parameter
@@ -98,7 +104,7 @@ class QuantizedMatrix:
         if device is None:
             return self
         return QuantizedMatrix(self.int_weight.to(device), self.zero.to(device),
-                               self.scale.to(device), self.contraction_axis)
+                               self.scale.to(device), self.contraction_axis, self.bits)
 
     # ---- array-like behaviour inside model functions.  A model written for dense weights
     # (x @ w, F.linear(x, w), w.T @ x, torch.tensordot(w, x, ...)) runs unchanged on packed ones:
@@ -153,13 +159,16 @@ class QuantizedMatrix:
     def __getattr__(self, name):
         # any other tensor method (w.sum(), w.abs(), ...): unpack, then do as written
         # (reference transform.py:74-79)
-        if name.startswith("_") or name in ("int_weight", "zero", "scale", "contraction_axis"):
+        if name.startswith("_") or name in ("int_weight", "zero", "scale", "contraction_axis", "bits"):
             raise AttributeError(name)
         return getattr(unpack_matrix(self), name)
 
 
-def quant_matrix_shape(quantized_matrix, bits=4):
-    """Logical shape of a packed matrix (reference ``gptq.py:34-42``)."""
+def quant_matrix_shape(quantized_matrix, bits=None):
+    """Logical shape of a packed matrix (reference ``gptq.py:34-42``); ``bits`` defaults to the
+    container's code width (the reference's 4 where it has none)."""
+    if bits is None:
+        bits = getattr(quantized_matrix, "bits", 4)
     mat = quantized_matrix.int_weight
     ele_width = mat.element_size() * 8 if isinstance(mat, torch.Tensor) else mat.dtype.itemsize * 8
     shape = list(mat.shape)
@@ -410,8 +419,8 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=
     reads across such calls: the Hessian, and, without ``actorder``, the factor of its damped
     inverse, which depends on ``xs`` and ``damping`` only.  The results are those of independent
     calls.  ``bits`` (1 to 8; the reference's ``gptq`` is fixed at the default of its
-    ``get_quantize_params``, 4): the code width, ``maxq = 2**bits - 1``; only 4-bit results can
-    be packed.  ``split_fp16``: see
+    ``get_quantize_params``, 4): the code width, ``maxq = 2**bits - 1``; ``pack_matrix`` stores
+    4-bit results two per byte and 8-bit results one per byte.  ``split_fp16``: see
     ``accumulate_H``.
     """
     Wt = _float_dev(W)
@@ -541,26 +550,29 @@ def unpack_colwise(w):
 def pack_matrix(Q, params, contraction_axis=0):
     """Dequantised floats -> integer codes -> packed container (reference ``gptq.py:214-228``)."""
     lib = N.load()
-    if int(params.get("maxq", 15)) != 15:
-        raise NotImplementedError("only 4-bit codes are packed (two per byte, gptq.py:241)")
+    maxq = int(params.get("maxq", 15))
+    if maxq not in (15, 255):
+        raise NotImplementedError("4-bit codes are packed two per byte (gptq.py:241), 8-bit codes are stored "
+                                  "one per byte; other widths have no packed form")
+    bits = 4 if maxq == 15 else 8
     Qt = _float_dev(Q)
     scale = _dev(params["scale"])
     zero = _dev(params["zero"])
     outer, alen, inner = _view3(Qt.shape, contraction_axis)
-    if alen % 2:
+    if bits == 4 and alen % 2:
         raise ValueError("the contraction axis must have even length")
     if scale.numel() != outer * inner or zero.numel() != outer * inner:
         raise ValueError("scale/zero must have the shape of Q without the contraction axis")
     shape = list(Qt.shape)
-    shape[contraction_axis] = alen // 2
+    shape[contraction_axis] = alen // 2 if bits == 4 else alen
     packed = torch.empty(shape, dtype=torch.uint8, device=Qt.device)
     scale32 = scale.to(torch.float32).contiguous()     # kept alive across the launch
     zero32 = zero.to(torch.float32).contiguous()
-    N.check(lib.gptq_hip_quantize_pack(
-        _stream(), _ptr(Qt), _DT[Qt.dtype], outer, alen, inner, _ptr(scale32), _ptr(zero32),
+    N.check(lib.gptq_hip_quantize_pack_bits(
+        _stream(), _ptr(Qt), _DT[Qt.dtype], outer, alen, inner, _ptr(scale32), _ptr(zero32), bits,
         _ptr(packed)), "quantize_pack")
     return QuantizedMatrix(int_weight=packed, zero=zero, scale=scale,
-                           contraction_axis=contraction_axis)
+                           contraction_axis=contraction_axis, bits=bits)
 
 
 def unpack_matrix(weight):
@@ -572,9 +584,10 @@ def unpack_matrix(weight):
     outer, plen, inner = _view3(iw.shape, weight.contraction_axis)
     if zero.numel() != outer * inner or scale.numel() != outer * inner:
         raise ValueError("scale/zero must have the shape of the matrix without the contraction axis")
+    bits = int(getattr(weight, "bits", 4))
     shape = list(iw.shape)
-    shape[weight.contraction_axis] = plen * 2
+    shape[weight.contraction_axis] = plen * (8 // bits)
     out = torch.empty(shape, dtype=zero.dtype, device=iw.device)
-    N.check(lib.gptq_hip_dequant(_stream(), _ptr(iw), outer, plen, inner, _ptr(zero), _ptr(scale),
-                                 _DT[zero.dtype], _ptr(out)), "dequant")
+    N.check(lib.gptq_hip_dequant_bits(_stream(), _ptr(iw), outer, plen, inner, _ptr(zero), _ptr(scale),
+                                      _DT[zero.dtype], bits, _ptr(out)), "dequant")
     return out

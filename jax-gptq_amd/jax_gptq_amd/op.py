@@ -29,7 +29,7 @@ def _qmm_workspace(nbytes, device):
     return ws
 
 
-def _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b):
+def _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b, bits=4):
     lib = N.load()
     leading_dims = None
     if x.dim() > 2:
@@ -42,18 +42,20 @@ def _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b):
     if int_weight.dim() != 2:
         raise ValueError("quantized_matmul needs a 2-D packed matrix (contraction axis 0)")
     R, C = int_weight.shape
+    Kw = R * (8 // bits)                 # logical rows of the packed matrix
     if transpose_b:
-        K2, out_n = C, 2 * R
+        K2, out_n = C, Kw
     else:
-        K2, out_n = 2 * R, C
+        K2, out_n = Kw, C
     assert K == K2, f"Inner dim mismatch: {K} != {K2}"
     if zero.dtype != scale.dtype:
         scale = scale.to(zero.dtype)
     out = torch.empty((M, out_n), dtype=x.dtype, device=x.device)
-    ws = _qmm_workspace(lib.gptq_hip_qmatmul_workspace_bytes_x(M, R, C, int(transpose_b), _DT[x.dtype]), x.device)
-    N.check(lib.gptq_hip_qmatmul(_stream(), _ptr(x), _DT[x.dtype], M, _ptr(int_weight), R, C,
-                                 _ptr(zero), _ptr(scale), _DT[zero.dtype], int(transpose_b),
-                                 _ptr(out), _ptr(ws), ws.numel()), "qmatmul")
+    ws = _qmm_workspace(lib.gptq_hip_qmatmul_bits_workspace_bytes(M, R, C, int(transpose_b), _DT[x.dtype], bits),
+                        x.device)
+    N.check(lib.gptq_hip_qmatmul_bits(_stream(), _ptr(x), _DT[x.dtype], M, _ptr(int_weight), R, C,
+                                      _ptr(zero), _ptr(scale), _DT[zero.dtype], bits, int(transpose_b),
+                                      _ptr(out), _ptr(ws), ws.numel()), "qmatmul")
     if leading_dims is not None:
         out = out.reshape(tuple(leading_dims) + (out_n,))
     return out
@@ -61,17 +63,18 @@ def _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b):
 
 class _QuantizedMatmulFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, int_weight, zero, scale, transpose_b):
+    def forward(ctx, x, int_weight, zero, scale, transpose_b, bits):
         ctx.save_for_backward(int_weight, zero, scale)
         ctx.transpose_b = transpose_b
-        return _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b)
+        ctx.bits = bits
+        return _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b, bits)
 
     @staticmethod
     def backward(ctx, y_bar):
         int_weight, zero, scale = ctx.saved_tensors
         x_bar = _quantized_matmul_raw(y_bar.contiguous(), int_weight, zero, scale,
-                                      not ctx.transpose_b)
-        return x_bar, None, None, None, None
+                                      not ctx.transpose_b, ctx.bits)
+        return x_bar, None, None, None, None, None
 
 
 def _quantized_matmul(x, quantized_matrix, transpose_b):
@@ -81,9 +84,12 @@ def _quantized_matmul(x, quantized_matrix, transpose_b):
     iw = _dev(quantized_matrix.int_weight, torch.uint8)
     zero = _float_dev(quantized_matrix.zero)
     scale = _float_dev(quantized_matrix.scale)
+    bits = int(getattr(quantized_matrix, "bits", 4))
+    if bits not in (4, 8):
+        raise ValueError("quantized_matmul takes 4-bit or 8-bit codes")
     if x.requires_grad:
-        return _QuantizedMatmulFn.apply(x, iw, zero, scale, bool(transpose_b))
-    return _quantized_matmul_raw(x, iw, zero, scale, bool(transpose_b))
+        return _QuantizedMatmulFn.apply(x, iw, zero, scale, bool(transpose_b), bits)
+    return _quantized_matmul_raw(x, iw, zero, scale, bool(transpose_b), bits)
 
 
 def quantized_matmul(x, quantized_matrix, transpose_b=False):
@@ -92,8 +98,8 @@ def quantized_matmul(x, quantized_matrix, transpose_b=False):
     fp32 accumulation; the result is rounded to fp16 and returned in ``x``'s dtype (``op.py:43,66-68``).
     fp16 and bf16 activations enter the matrix cores as they are; fp32 activations are rounded to
     fp16 precision after a per-row power-of-two scaling (the reference's Triton dot rounds them to
-    TF32, which has the same mantissa width) when the matrix has a multiple of 16 columns, and run
-    unrounded on plain kernels otherwise."""
+    TF32, which has the same mantissa width).  ``quantized_matrix.bits`` (4, the reference's width,
+    unless ``pack_matrix`` was given 8-bit parameters) selects the code width."""
     return _quantized_matmul(x, quantized_matrix, transpose_b)
 
 

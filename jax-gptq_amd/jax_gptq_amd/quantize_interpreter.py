@@ -245,7 +245,7 @@ class _Session:
             raise ValueError(f"block_size={o['block_size']} must divide the contraction size "
                              f"{W2.shape[0]} of parameter {leaf}")
         Q2, qp = gptq(W=W2, xs=xs, block_size=o["block_size"], actorder=o["actorder"],
-                      damping=o["damping"], use_fp64=o["use_fp64"], shared=self._shared(xs))
+                      damping=o["damping"], use_fp64=o["use_fp64"], shared=self._shared(xs), bits=o["bits"])
         Qt = _dots.from_matrix(Q2, tuple(w.shape), wc)                       # layout fn sees
         scale_shape = tuple(d for i, d in enumerate(w.shape) if i != wc)
         packed = pack_matrix(Qt.contiguous(),
@@ -256,7 +256,7 @@ class _Session:
         if inverse != tuple(range(len(perm))):
             packed = permute_quantized(packed, inverse)
             packed = QuantizedMatrix(packed.int_weight.contiguous(), packed.zero.contiguous(),
-                                     packed.scale.contiguous(), packed.contraction_axis)
+                                     packed.scale.contiguous(), packed.contraction_axis, packed.bits)
         self.results[leaf] = packed
         # the product is evaluated with the quantised or the original weight; every later use
         # of the parameter sees the quantised one (quantize_interpreter.py:241-243, 289-291)
@@ -266,7 +266,8 @@ class _Session:
 
 
 def quantize(fn, params, inputs, block_size=128, actorder=False, damping=0.01,
-             use_quantized_activations=True, use_fp64=False, use_params_fp32=False, split_fp16=False):
+             use_quantized_activations=True, use_fp64=False, use_params_fp32=False, split_fp16=False,
+             bits=4):
     """Run GPTQ over the parameters of ``fn`` (reference ``quantize_interpreter.py:25-80``).
 
     ``fn(params, batch)``: the model; ``params``: a nested dict / list / tuple of arrays;
@@ -275,8 +276,11 @@ def quantize(fn, params, inputs, block_size=128, actorder=False, damping=0.01,
     :class:`QuantizedMatrix` (packed along its contraction axis, in its original layout);
     everything else is returned as it came.  Buffers of ``params`` that already live on the
     GPU are overwritten with the quantised values, so do not reuse them (the reference frees
-    them, ``:42``).  ``split_fp16`` (not in the reference): see ``accumulate_H``.
+    them, ``:42``).  ``split_fp16`` (not in the reference): see ``accumulate_H``.  ``bits`` (not in
+    the reference, whose code width is fixed at 4): 4 or 8.
     """
+    if int(bits) not in (4, 8):
+        raise ValueError("quantize packs 4-bit or 8-bit codes")
     if not inputs:
         raise ValueError("quantize needs at least one calibration batch")
     device = _device()
@@ -291,7 +295,7 @@ def quantize(fn, params, inputs, block_size=128, actorder=False, damping=0.01,
         flat.append(t)
     session = _Session(flat, dict(block_size=block_size, actorder=actorder, damping=damping,
                                   use_quantized_activations=use_quantized_activations,
-                                  use_fp64=use_fp64, split_fp16=split_fp16))
+                                  use_fp64=use_fp64, split_fp16=split_fp16, bits=int(bits)))
     wrapped = [(_Target(t, i, range(t.dim())) if isinstance(t, torch.Tensor) and t.is_floating_point()
                 and t.dim() > 1 else t) for i, t in enumerate(flat)]
     fn_params = _unflatten(struct, wrapped)

@@ -128,4 +128,4 @@ def permute_quantized(qm, perm):
     def move(v):
         return v.permute(scale_perm) if isinstance(v, torch.Tensor) and v.dim() > 1 else v
     return QuantizedMatrix(int_weight=qm.int_weight.permute(perm), zero=move(qm.zero),
-                           scale=move(qm.scale), contraction_axis=new_ca)
+                           scale=move(qm.scale), contraction_axis=new_ca, bits=getattr(qm, "bits", 4))

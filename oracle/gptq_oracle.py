@@ -54,11 +54,12 @@ __all__ = [
 class QuantizedMatrix:
     """Container of a packed matrix (reference ``gptq.py:8-22``)."""
 
-    def __init__(self, int_weight, zero, scale, contraction_axis=0):
+    def __init__(self, int_weight, zero, scale, contraction_axis=0, bits=4):
         self.int_weight = int_weight
         self.zero = zero
         self.scale = scale
         self.contraction_axis = contraction_axis
+        self.bits = bits        # 8 (an extension; the reference packs 4-bit codes only): one code per byte
 
     @property
     def shape(self):
@@ -69,8 +70,10 @@ class QuantizedMatrix:
         return self.zero.dtype
 
 
-def quant_matrix_shape(quantized_matrix, bits=4):
+def quant_matrix_shape(quantized_matrix, bits=None):
     """Logical shape of a packed matrix (reference ``gptq.py:34-42``)."""
+    if bits is None:
+        bits = getattr(quantized_matrix, "bits", 4)
     mat = quantized_matrix.int_weight
     ele_width = mat.dtype.itemsize * 8
     shape = list(mat.shape)
@@ -269,16 +272,19 @@ def codes_from_q(Q, params, contraction_axis=0):
 def pack_matrix(Q, params, contraction_axis=0):
     """Floats -> codes -> nibble-packed container (reference ``gptq.py:214-228``)."""
     int_matrix = codes_from_q(Q, params, contraction_axis)
-    packed = pack_along_axis(contraction_axis, int_matrix)
+    bits = 8 if int(params.get("maxq", 15)) == 255 else 4
+    # 8-bit codes (not in the reference) are the uint8 matrix itself
+    packed = pack_along_axis(contraction_axis, int_matrix) if bits == 4 else int_matrix
     return QuantizedMatrix(int_weight=packed, zero=np.asarray(params["zero"]),
-                           scale=np.asarray(params["scale"]), contraction_axis=contraction_axis)
+                           scale=np.asarray(params["scale"]), contraction_axis=contraction_axis, bits=bits)
 
 
 def unpack_matrix(weight):
     """Dense ``(code - zero) * scale`` (reference ``gptq.py:230-235``)."""
     zero = np.expand_dims(weight.zero, axis=weight.contraction_axis)
     scale = np.expand_dims(weight.scale, axis=weight.contraction_axis)
-    unpacked = unpack_along_axis(weight.contraction_axis, weight.int_weight)
+    unpacked = (unpack_along_axis(weight.contraction_axis, weight.int_weight)
+                if getattr(weight, "bits", 4) == 4 else np.asarray(weight.int_weight))
     return (unpacked.astype(zero.dtype) - zero) * scale
 
 
@@ -341,7 +347,8 @@ def quantized_matmul(x, quantized_matrix, transpose_b=False):
         lead = x.shape[:-1]
         x = x.reshape(-1, x.shape[-1])
     w = quantized_matrix.int_weight
-    codes = unpack_along_axis(0, w).astype(np.float32)
+    bits = getattr(quantized_matrix, "bits", 4)
+    codes = (unpack_along_axis(0, w) if bits == 4 else np.asarray(w)).astype(np.float32)
     dense = (codes - quantized_matrix.zero.astype(np.float32)[None, :]) * \
         quantized_matrix.scale.astype(np.float32)[None, :]
     K = x.shape[1]
@@ -349,7 +356,7 @@ def quantized_matmul(x, quantized_matrix, transpose_b=False):
         assert K == w.shape[1], f"Inner dim mismatch: {K} != {w.shape[1]}"
         out = x.astype(np.float32) @ dense.T
     else:
-        assert K == 2 * w.shape[0], f"Inner dim mismatch: {K} != {2 * w.shape[0]}"
+        assert K == codes.shape[0], f"Inner dim mismatch: {K} != {codes.shape[0]}"
         out = x.astype(np.float32) @ dense
     out = out.astype(np.float16)
     if lead is not None:
