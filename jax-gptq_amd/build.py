@@ -66,5 +66,40 @@ def build(force=False, verbose=True):
     return LIB
 
 
+JAX_SHIM = os.path.join(OUT_DIR, "libgptq_hip_jax.so")
+
+
+def jax_ffi_include_dir():
+    """Directory of the XLA FFI headers (xla/ffi/api/ffi.h) that ships inside jaxlib, or None where JAX
+    or its FFI module is absent."""
+    try:
+        import jax.ffi
+        inc = jax.ffi.include_dir()
+    except Exception:
+        return None
+    return inc if os.path.exists(os.path.join(inc, "xla", "ffi", "api", "ffi.h")) else None
+
+
+def build_jax_ffi(verbose=True):
+    """Compile csrc/jax_ffi.cc (XLA FFI handlers over the C ABI) into libgptq_hip_jax.so, linked against
+    libgptq_hip.so.  Returns the path, or None where the XLA FFI headers are not installed: the shim is
+    optional, the ctypes binding is the one that is always built."""
+    inc = jax_ffi_include_dir()
+    if inc is None:
+        if verbose:
+            print("[build] jax.ffi.include_dir() does not resolve: the XLA FFI shim is not built")
+        return None
+    build()
+    cmd = [_hipcc(), "-O2", "-fPIC", "-std=c++17", "-shared", "-x", "hip", "--offload-arch=gfx950",
+           "-I", inc, os.path.join(CSRC, "jax_ffi.cc"), "-o", JAX_SHIM,
+           "-L", OUT_DIR, "-l:libgptq_hip.so", "-Wl,-rpath,$ORIGIN"]
+    subprocess.check_call(cmd)
+    if verbose:
+        print(f"[build] wrote {JAX_SHIM}")
+    return JAX_SHIM
+
+
 if __name__ == "__main__":
     build(force="--force" in sys.argv)
+    if "--jax" in sys.argv:
+        build_jax_ffi()

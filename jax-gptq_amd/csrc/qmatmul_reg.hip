@@ -34,6 +34,7 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
                                                           int zs_dtype, TX *out, float *part, int32_t *counters,
                                                           int S, int steps_per_split) {
   constexpr bool BF = Act<TX>::BF;
+  constexpr int SCHED = RB == 4 ? 4 : 0;         // vector instructions between two MFMAs of the main loop (0: compiler's order)
   constexpr int NL = BITS == 4 ? 4 : 8;          // packed rows per lane and k-step
   constexpr int PR = 4 * NL;                     // packed rows per k-step
   extern __shared__ __attribute__((aligned(16))) float rg_lds[];   // [4 wavefronts][RB][RG_NT][64 lanes][4]
@@ -166,6 +167,18 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
     for (int u = 0; u < RING; ++u) {
       compute(u, plain);
       load_step(u, s0 + u + RING);
+      // One wavefront per SIMD issues in order: an MFMA occupies the matrix pipe for four passes, during
+      // which the wavefront can issue only what stands behind it in program order and does not depend on it.
+      // So the dequantisation of the next tile goes between the MFMAs of this one: one MFMA, then a few
+      // vector instructions, and the k-step's loads spread over its first groups.
+      if (SCHED) {
+#pragma unroll
+        for (int i = 0; i < RB * RG_NT; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (i < NL + RB) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, SCHED, 0);
+        }
+      }
     }
   }
   // at most RING - 1 full k-steps left, all of them loaded; then the ragged one
@@ -185,7 +198,7 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
   // sum[t8][r] = sum_k x[m][k] (code - zi)[k][col + t8] (bf16, 4-bit: code + 128), sum[8][r] = sum_k x[m][k],
   // m = m0 + 16 rb + 4 g + r
   if (!col_ok) return;
-  const int rb = RB == 4 ? wk : 0;
+  const int rb = wk;                             // rg_reduce returned true: wk < RB
   float sc[8], zf[8];
 #pragma unroll
   for (int t8 = 0; t8 < 8; ++t8) {

@@ -84,8 +84,7 @@ __device__ __forceinline__ floatx4 rg_load_part_issue(const float *p) {
 
 // Sum of the four wavefronts' accumulators and, when the contraction is split over S workgroups per output
 // tile, of the S workgroups' partial tiles.  A workgroup is four wavefronts that each hold RB x RG_NT tiles
-// over a quarter of the workgroup's k-steps.  Row block rb is finished by wavefront rb (RB == 4) or by
-// wavefront 0 (RB == 1); on return `sum` holds that row block's complete tiles and the return value says
+// over a quarter of the workgroup's k-steps.  Row block rb is finished by wavefront rb (RB <= 4); on return `sum` holds that row block's complete tiles and the return value says
 // whether this wavefront is to write them out (false for the wavefronts that own nothing and for all
 // workgroups but the last arrival of a split tile).
 //   S > 1: the owner wavefronts write their sums to part[tile][split][rb] with agent-scope write-through
@@ -104,8 +103,8 @@ __device__ __forceinline__ bool rg_reduce(floatx4 (&acc)[RB][RG_NT], floatx4 (&s
     for (int t = 0; t < RG_NT; ++t)
       *reinterpret_cast<floatx4 *>(lds + (((wk * RB + rb) * RG_NT + t) * 64 + lane) * 4) = acc[rb][t];
   __syncthreads();
-  const bool owner = RB == 4 ? true : wk == 0;
-  const int rb_own = RB == 4 ? wk : 0;
+  const bool owner = wk < RB;
+  const int rb_own = owner ? wk : 0;
 #pragma unroll
   for (int t = 0; t < RG_NT; ++t) {
     floatx4 v = floatx4{0.f, 0.f, 0.f, 0.f};
