@@ -46,6 +46,16 @@ enum {
 int gptq_hip_abi_version(void);
 const char *gptq_hip_error_string(int code);
 
+/* ---- buffer helpers of the solve's driver --------------------------------------------------------
+ * What the reference gets from XLA around its kernels: the zero-filled H and mean (gptq.py:90-95),
+ * the fp32 working copy of W (gptq.py:184) and the copy of a matrix that a later step still needs.
+ * fill_zero / copy: device pointers, 16-byte aligned, any byte count.  to_f32: n elements of type
+ * in_dtype (F32, F16, BF16) widened to fp32.  Fill kernels rather than memsets, so that the calls can
+ * be recorded into a captured graph. */
+int gptq_hip_fill_zero(void *stream, void *ptr, size_t bytes);
+int gptq_hip_copy(void *stream, void *dst, const void *src, size_t bytes);
+int gptq_hip_to_f32(void *stream, const void *in, int in_dtype, int64_t n, float *out);
+
 /* ---- per-column quantisation parameters -------------------------------------
  * Replaces get_quantize_params / get_col_quantize_params (gptq.py:105-118).
  * W [K, N] (element type w_dtype, row stride ldw) -> scale[N], zero[N] (fp32).

@@ -1,6 +1,26 @@
 // ABI version and error strings.
 #include "common.h"
 
+#include <map>
+#include <mutex>
+#include <utility>
+
+bool gptq_raise_lds_limit(const void *kernel, int bytes) {
+  static std::mutex mu;
+  static std::map<std::pair<int, const void *>, int> raised;      // (device, kernel) -> limit set
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = raised.find({dev, kernel});
+  if (it != raised.end() && it->second >= bytes) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  raised[{dev, kernel}] = bytes;
+  return true;
+}
+
 extern "C" {
 
 int gptq_hip_abi_version(void) { return GPTQ_HIP_ABI_VERSION; }

@@ -164,6 +164,25 @@ __global__ __launch_bounds__(TPB) void gather_sym_kernel(const T *in, T *out, in
     out[row * K + c] = in[src * K + perm[c]];
 }
 
+// ------------------------------------------------------------------ fills, copies, widening
+// 16 bytes per thread and step; n16 = number of 16-byte units, the tail bytes are handled by thread 0
+__global__ __launch_bounds__(TPB) void fill_zero_kernel(uint4 *p, int64_t n16, uint8_t *tail, int ntail) {
+  for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < n16; i += (int64_t)gridDim.x * TPB)
+    p[i] = make_uint4(0u, 0u, 0u, 0u);
+  if (blockIdx.x == 0 && threadIdx.x < ntail) tail[threadIdx.x] = 0;
+}
+
+__global__ __launch_bounds__(TPB) void copy_kernel(uint4 *dst, const uint4 *src, int64_t n16, uint8_t *dtail,
+                                                   const uint8_t *stail, int ntail) {
+  for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < n16; i += (int64_t)gridDim.x * TPB) dst[i] = src[i];
+  if (blockIdx.x == 0 && threadIdx.x < ntail) dtail[threadIdx.x] = stail[threadIdx.x];
+}
+
+template <typename T>
+__global__ __launch_bounds__(TPB) void to_f32_kernel(const T *in, int64_t n, float *out) {
+  for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < n; i += (int64_t)gridDim.x * TPB) out[i] = to_f32(in[i]);
+}
+
 inline unsigned grid_for(int64_t total) {
   int64_t g = ceil_div64(total, TPB);
   if (g > 1 << 20) g = 1 << 20;
@@ -421,6 +440,59 @@ int gptq_hip_gather_sym(void *stream, const void *in, void *out, int elem_bytes,
                        (const uint64_t *)in, (uint64_t *)out, K, perm);
   else
     return GPTQ_HIP_EDTYPE;
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
+
+int gptq_hip_fill_zero(void *stream, void *ptr, size_t bytes) {
+  if (bytes == 0) return GPTQ_HIP_OK;
+  if (!ptr || (reinterpret_cast<uintptr_t>(ptr) & 15)) return GPTQ_HIP_EINVAL;
+  const int64_t n16 = (int64_t)(bytes / 16);
+  int64_t g = ceil_div64(n16, (int64_t)TPB * 4);
+  if (g > 4096) g = 4096;
+  if (g < 1) g = 1;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)g), dim3(TPB), 0, as_stream(stream),
+                     reinterpret_cast<uint4 *>(ptr), n16, reinterpret_cast<uint8_t *>(ptr) + n16 * 16,
+                     (int)(bytes % 16));
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
+int gptq_hip_copy(void *stream, void *dst, const void *src, size_t bytes) {
+  if (bytes == 0) return GPTQ_HIP_OK;
+  if (!dst || !src || ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15))
+    return GPTQ_HIP_EINVAL;
+  const int64_t n16 = (int64_t)(bytes / 16);
+  int64_t g = ceil_div64(n16, (int64_t)TPB * 4);
+  if (g > 4096) g = 4096;
+  if (g < 1) g = 1;
+  hipLaunchKernelGGL(copy_kernel, dim3((unsigned)g), dim3(TPB), 0, as_stream(stream), reinterpret_cast<uint4 *>(dst),
+                     reinterpret_cast<const uint4 *>(src), n16, reinterpret_cast<uint8_t *>(dst) + n16 * 16,
+                     reinterpret_cast<const uint8_t *>(src) + n16 * 16, (int)(bytes % 16));
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
+int gptq_hip_to_f32(void *stream, const void *in, int in_dtype, int64_t n, float *out) {
+  if (n < 0) return GPTQ_HIP_EINVAL;
+  if (n == 0) return GPTQ_HIP_OK;
+  if (!in || !out) return GPTQ_HIP_EINVAL;
+  hipStream_t st = as_stream(stream);
+  const dim3 grid(grid_for(ceil_div64(n, 4))), block(TPB);
+  switch (in_dtype) {
+    case GPTQ_HIP_F32:
+      hipLaunchKernelGGL(to_f32_kernel<float>, grid, block, 0, st, (const float *)in, n, out);
+      break;
+    case GPTQ_HIP_F16:
+      hipLaunchKernelGGL(to_f32_kernel<__half>, grid, block, 0, st, (const __half *)in, n, out);
+      break;
+    case GPTQ_HIP_BF16:
+      hipLaunchKernelGGL(to_f32_kernel<__hip_bfloat16>, grid, block, 0, st, (const __hip_bfloat16 *)in, n, out);
+      break;
+    default:
+      return GPTQ_HIP_EDTYPE;
+  }
   GPTQ_CHECK_LAUNCH();
   return GPTQ_HIP_OK;
 }

@@ -13,6 +13,11 @@
     if (hipGetLastError() != hipSuccess) return GPTQ_HIP_ELAUNCH; \
   } while (0)
 
+// Raises the dynamic-LDS limit of a kernel (hipFuncAttributeMaxDynamicSharedMemorySize) the first time
+// the kernel is used on a device with that size and remembers it: later calls are a table lookup and
+// make no HIP call.  Returns false if the runtime refuses.  (api.hip)
+bool gptq_raise_lds_limit(const void *kernel, int bytes);
+
 static inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 
 static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }

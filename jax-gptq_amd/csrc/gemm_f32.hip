@@ -361,8 +361,7 @@ int launch_nn_wk(hipStream_t stream, const GemmArgs &a) {
   const dim3 g64((unsigned)((a.n + 63) / 64), (unsigned)((a.m + 63) / 64), 1);
   if (g64.y > 65535u) return GPTQ_HIP_EINVAL;
   if (wk_lds_bytes(KK) > 48 * 1024 &&
-      hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f32_nn_wk_kernel<KK>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, wk_lds_bytes(KK)) != hipSuccess)
+      !gptq_raise_lds_limit(reinterpret_cast<const void *>(gemm_f32_nn_wk_kernel<KK>), wk_lds_bytes(KK)))
     return GPTQ_HIP_ELAUNCH;
   hipLaunchKernelGGL(gemm_f32_nn_wk_kernel<KK>, g64, dim3(NTHREADS), wk_lds_bytes(KK), stream, a);
   GPTQ_CHECK_LAUNCH();
@@ -501,8 +500,7 @@ int gptq_gemm_f32(hipStream_t stream, const GemmArgs &a) {
       if (g64.y > 65535u) return GPTQ_HIP_EINVAL;
       hipLaunchKernelGGL(gemm_f32_tn_k64_kernel<64>, g64, block, k64_lds_bytes(64), stream, a);
     } else {
-      if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f32_tn_k64_kernel<128>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, k64_lds_bytes(128)) != hipSuccess)
+      if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(gemm_f32_tn_k64_kernel<128>), k64_lds_bytes(128)))
         return GPTQ_HIP_ELAUNCH;
       hipLaunchKernelGGL(gemm_f32_tn_k64_kernel<128>, grid, block, k64_lds_bytes(128), stream, a);
     }

@@ -1562,8 +1562,7 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
                                : (f16 ? reinterpret_cast<const void *>(syrk16w_kernel<__half>)
                                       : reinterpret_cast<const void *>(syrk16w_kernel<__hip_bfloat16>));
       const int lds_bytes = regular ? D16_LDS_BYTES : W16_LDS_BYTES;
-      if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
-        return GPTQ_HIP_ELAUNCH;
+      if (!gptq_raise_lds_limit(fn, lds_bytes)) return GPTQ_HIP_ELAUNCH;
       const dim3 wgrid((unsigned)(nt * w.RS));
       if (regular && f16)
         hipLaunchKernelGGL((syrk16d_kernel<__half, SyrkArgs>), wgrid, block, lds_bytes, st, w);
@@ -1590,9 +1589,7 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
       const void *fn = x_dtype == GPTQ_HIP_F16
                            ? reinterpret_cast<const void *>(syrk16_kernel<__half>)
                            : reinterpret_cast<const void *>(syrk16_kernel<__hip_bfloat16>);
-      if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, S16_LDS_BYTES) !=
-          hipSuccess)
-        return GPTQ_HIP_ELAUNCH;
+      if (!gptq_raise_lds_limit(fn, S16_LDS_BYTES)) return GPTQ_HIP_ELAUNCH;
       if (x_dtype == GPTQ_HIP_F16)
         hipLaunchKernelGGL(syrk16_kernel<__half>, grid, block, S16_LDS_BYTES, st, a);
       else
@@ -1621,8 +1618,7 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
       const int64_t chunk = round_up64(ceil_div64(total_rows, w.RS), D32_BK);
       if (chunk > 2147483647LL) return GPTQ_HIP_EINVAL;
       w.chunk = (int)chunk;
-      if (hipFuncSetAttribute(reinterpret_cast<const void *>(syrk32d_kernel),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, D32_LDS_BYTES) != hipSuccess)
+      if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(syrk32d_kernel), D32_LDS_BYTES))
         return GPTQ_HIP_ELAUNCH;
       hipLaunchKernelGGL(syrk32d_kernel, dim3((unsigned)(nt * w.RS)), block, D32_LDS_BYTES, st, w);
       GPTQ_CHECK_LAUNCH();
@@ -1706,8 +1702,7 @@ int gptq_hip_hessian_accumulate_split16(void *stream, const void *const *x_ptrs,
 
   // ---- groups of batches: split, multiply into the partial tiles (or into H when there is one slice)
   const void *fn = reinterpret_cast<const void *>(syrk16d_kernel<__half, SyrkArgsDual>);
-  if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, D16_LDS_BYTES) != hipSuccess)
-    return GPTQ_HIP_ELAUNCH;
+  if (!gptq_raise_lds_limit(fn, D16_LDS_BYTES)) return GPTQ_HIP_ELAUNCH;
   const int64_t nt = (int64_t)sp.T * (sp.T + 1) / 2;
   // batches per launch: as even as the table allows (a short last launch costs as much per
   // workgroup as a long one)

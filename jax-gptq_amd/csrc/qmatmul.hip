@@ -750,9 +750,7 @@ int launch_fwd_mfma(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, 
                     int64_t R, int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
   const QmmWs ws = qmm_ws(wsp, p.x1_bytes);
   auto kern = qmm_fwd_mfma_kernel<SPW, TZ, TX, X16>;
-  if (p.lds_bytes > 48 * 1024 &&
-      hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)p.lds_bytes) != hipSuccess)
+  if (p.lds_bytes > 48 * 1024 && !gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), (int)p.lds_bytes))
     return GPTQ_HIP_ELAUNCH;
   // at most QMM_MAX_COUNTERS (m-chunk, strip) pairs per launch
   const int mch_per = QMM_MAX_COUNTERS / p.strips;
@@ -779,9 +777,7 @@ int launch_fwd_stream(hipStream_t st, const FwdPlan &p, const void *x, int64_t M
   const QmmWs ws = qmm_ws(wsp, p.x1_bytes);
   auto kern = qmm_fwd_stream_kernel<TZ, TX>;
   if (p.strips > QMM_MAX_COUNTERS || p.mch != 1 || C < 16) return GPTQ_HIP_EINVAL;
-  if (p.lds_bytes > 48 * 1024 &&
-      hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)p.lds_bytes) != hipSuccess)
+  if (p.lds_bytes > 48 * 1024 && !gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), (int)p.lds_bytes))
     return GPTQ_HIP_ELAUNCH;
   const dim3 grid((unsigned)p.strips, (unsigned)p.S, 1);
   hipLaunchKernelGGL(kern, grid, dim3(QS_NW * 64), p.lds_bytes, st, (const TX *)x, (int)M,
@@ -865,16 +861,8 @@ template <int NW, int KS, int MR, bool ATOM, bool LOOP, typename TZ, typename TX
 int launch_dec_inst(hipStream_t st, const DecPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
                     int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
   auto kern = qmm_fwd_dec_kernel<NW, KS, MR, ATOM, LOOP, TZ, TX>;
-  // the LDS limit of a kernel is raised once per device and instantiation (a repeated or concurrent
-  // call sets the same value again, which is harmless)
-  static bool attr_set[64] = {};
-  int dev = 0;
-  if (p.lds_bytes > 48 * 1024 && (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64 || !attr_set[dev])) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)p.lds_bytes) != hipSuccess)
-      return GPTQ_HIP_ELAUNCH;
-    if (dev >= 0 && dev < 64) attr_set[dev] = true;
-  }
+  if (p.lds_bytes > 48 * 1024 && !gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), (int)p.lds_bytes))
+    return GPTQ_HIP_ELAUNCH;
   const QmmWs ws = qmm_ws(wsp, p.x1_bytes);
   hipLaunchKernelGGL(kern, dim3((unsigned)p.strips, (unsigned)p.S, 1), dim3(NW * 64), p.lds_bytes, st,
                      (const TX *)x, (int)M, (int)(2 * R), pk, (int)R, (int)C, (const TZ *)zero,
@@ -1265,10 +1253,7 @@ int launch_fwd_gemm_inst(hipStream_t st, const GemmPlan &p, const void *x, int64
   constexpr size_t lds = (size_t)(2 * (BM / 16) * GGROUP + 2 * (128 / 16) * GGROUP) * sizeof(_Float16) +
                          BM * sizeof(float);
   auto kern = qmm_fwd_gemm_kernel<BM, 128, TZ, TX, SPLIT>;
-  if (lds > 64 * 1024 &&
-      hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-    return GPTQ_HIP_ELAUNCH;
+  if (lds > 64 * 1024 && !gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), (int)lds)) return GPTQ_HIP_ELAUNCH;
   const dim3 grid((unsigned)ceil_div64(C, 128), (unsigned)ceil_div64(M, BM), (unsigned)p.S);
   hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (const TX *)x, (int)M, (int)(2 * R), pk, (int)R,
                      (int)C, (const TZ *)zero, (const TZ *)scale, (TX *)out, ws, p.S);

@@ -231,16 +231,7 @@ int launch_inst(hipStream_t st, const RegPlan &p, const void *x, int64_t M, cons
                 int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *wsp) {
   constexpr size_t lds = (size_t)4 * RB * RG_NT * RG_TILE_FLOATS * sizeof(float);
   auto kern = qmm_fwd_reg_kernel<BITS, RB, RING, RAGGED, TX>;
-  // the LDS limit of a kernel is raised once per device and instantiation (a repeated or concurrent call
-  // sets the same value again, which is harmless)
-  static bool attr_set[64] = {};
-  int dev = 0;
-  if (lds > 64 * 1024 && (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64 || !attr_set[dev])) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds) != hipSuccess)
-      return GPTQ_HIP_ELAUNCH;
-    if (dev >= 0 && dev < 64) attr_set[dev] = true;
-  }
+  if (lds > 64 * 1024 && !gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), (int)lds)) return GPTQ_HIP_ELAUNCH;
   const int64_t K = BITS == 4 ? 2 * R : R;
   int32_t *counters = reinterpret_cast<int32_t *>(wsp);
   float *part = reinterpret_cast<float *>(reinterpret_cast<char *>(wsp) + QMM_HEAD_BYTES);

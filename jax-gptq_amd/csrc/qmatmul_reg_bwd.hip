@@ -275,14 +275,7 @@ int launch_inst(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, c
                 int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *wsp) {
   constexpr int NJ = BITS == 4 ? 64 : 128;
   auto kern = qmm_bwd_reg_kernel<BITS, RAGGED, TX>;
-  static bool attr_set[64] = {};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64 || !attr_set[dev]) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            RGB_LDS_BYTES) != hipSuccess)
-      return GPTQ_HIP_ELAUNCH;
-    if (dev >= 0 && dev < 64) attr_set[dev] = true;
-  }
+  if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), RGB_LDS_BYTES)) return GPTQ_HIP_ELAUNCH;
   const int64_t KO = BITS == 4 ? 2 * R : R;
   int32_t *counters = reinterpret_cast<int32_t *>(wsp);
   float *part = reinterpret_cast<float *>(reinterpret_cast<char *>(wsp) + QMM_HEAD_BYTES);

@@ -132,8 +132,7 @@ int launch_block(hipStream_t st, const float *W, int64_t N, const float *L, int6
                          : (q_dtype == GPTQ_HIP_F16
                                 ? reinterpret_cast<const void *>(block_quant_kernel<SB, __half>)
                                 : reinterpret_cast<const void *>(block_quant_kernel<SB, __hip_bfloat16>));
-    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return GPTQ_HIP_ELAUNCH;
+    if (!gptq_raise_lds_limit(fn, (int)lds)) return GPTQ_HIP_ELAUNCH;
   }
   switch (q_dtype) {
     case GPTQ_HIP_F32:

@@ -21,6 +21,9 @@ _vp, _i64, _i32, _f32, _f64, _sz = (ctypes.c_void_p, ctypes.c_int64, ctypes.c_in
 SIGNATURES = {
     "gptq_hip_abi_version": (_i32, []),
     "gptq_hip_error_string": (ctypes.c_char_p, [_i32]),
+    "gptq_hip_fill_zero": (_i32, [_vp, _vp, _sz]),
+    "gptq_hip_copy": (_i32, [_vp, _vp, _vp, _sz]),
+    "gptq_hip_to_f32": (_i32, [_vp, _vp, _i32, _i64, _vp]),
     "gptq_hip_col_params_workspace_bytes": (_sz, [_i64, _i64]),
     "gptq_hip_col_params": (_i32, [_vp, _vp, _i32, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _sz]),
     "gptq_hip_hessian_accumulate_workspace_bytes": (_sz, [_i64, _i32]),

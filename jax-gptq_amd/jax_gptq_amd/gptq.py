@@ -62,6 +62,26 @@ def _ws(nbytes):
     return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=_device())
 
 
+def _zeros(shape, dtype):
+    """Zero-filled device tensor: torch allocates, the library's fill kernel writes."""
+    t = torch.empty(shape, dtype=dtype, device=_device())
+    N.check(N.load().gptq_hip_fill_zero(_stream(), _ptr(t), t.numel() * t.element_size()), "fill_zero")
+    return t
+
+
+def _clone(t):
+    out = torch.empty_like(t)
+    N.check(N.load().gptq_hip_copy(_stream(), _ptr(out), _ptr(t), t.numel() * t.element_size()), "copy")
+    return out
+
+
+def _to_f32_copy(t):
+    """fp32 working copy of a float tensor (always a new buffer: the column loop consumes it)."""
+    out = torch.empty(t.shape, dtype=torch.float32, device=t.device)
+    N.check(N.load().gptq_hip_to_f32(_stream(), _ptr(t), _DT[t.dtype], t.numel(), _ptr(out)), "to_f32")
+    return out
+
+
 class QuantizedMatrix:
     """Packed matrix container (reference ``gptq.py:8-22``): ``int_weight`` uint8 with two
     4-bit codes per byte along ``contraction_axis``, per-channel ``zero`` and ``scale``.
@@ -266,7 +286,7 @@ def accumulate_H(xs, use_fp64=False, split_fp16=False):
     for b in batches:
         if b.shape[-1] != K:
             raise ValueError("all calibration batches must share the feature dimension")
-    H = torch.zeros((K, K), dtype=hdt, device=_device())
+    H = _zeros((K, K), hdt)
     if split_fp16 and _split16_ok(H, batches):
         _hessian_accumulate_split16(H, batches)
     else:
@@ -312,7 +332,7 @@ def _damp_invert(W, H, damping, fix_dead=True, want_f32=False):
     if want_f32:
         L32 = L if H.dtype == torch.float32 else torch.empty((K, K), dtype=torch.float32,
                                                              device=H.device)
-    status = torch.zeros(2, dtype=torch.int32, device=H.device)
+    status = _zeros((2,), torch.int32)
     hdt = _DT_H[H.dtype]
     ws = _ws(lib.gptq_hip_damp_invert_workspace_bytes(K, hdt))
     N.check(lib.gptq_hip_damp_invert(_stream(), _ptr(H), hdt, _ptr(W), K, Nc, Nc, float(damping),
@@ -430,9 +450,7 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=
     K, Nc = Wt.shape
     if block_size < 1 or block_size > 128 or K % block_size != 0:
         raise ValueError(f"block_size={block_size} must divide K={K} and be at most 128")
-    W32 = Wt.to(torch.float32)
-    if W32.data_ptr() == Wt.data_ptr():
-        W32 = W32.clone()              # the loop consumes its working copy
+    W32 = _to_f32_copy(Wt)            # the loop consumes its working copy
     if not 1 <= int(bits) <= 8:
         raise ValueError("bits must be between 1 and 8")
     quantize_params = get_col_quantize_params(W32, bits=int(bits))
@@ -458,7 +476,7 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=
         N.check(lib.gptq_hip_zero_dead_rows(_stream(), _ptr(H), _DT_H[H.dtype], K, _ptr(W32), Nc, Nc),
                 "zero_dead_rows")
     if Hinv is None:
-        Hw = H.clone() if keep else H           # the factorisation rewrites the diagonal
+        Hw = _clone(H) if keep else H           # the factorisation rewrites the diagonal
         if actorder:
             W32, Hw, perm = _permute(W32, Hw)
         # _damp_and_invert (gptq.py:193) and the fp32 cast of the factor (gptq.py:197) in one call

@@ -163,7 +163,13 @@ def test_gptq_other_code_widths(G, bits):
     assert abs(e - er) <= 0.01 * er
     e4 = recon_error(W, to_np(G.gptq(W, [X])[0]), X)
     assert (e < e4 / 8) if bits == 8 else (e > e4)
-    with pytest.raises(NotImplementedError):
-        G.pack_matrix(Q, p)
+    if bits == 8:
+        # one code per byte, equal to the codes of the dequantised result
+        packed = G.pack_matrix(Q, p)
+        assert packed.bits == 8 and packed.shape == W.shape
+        assert np.array_equal(to_np(packed.int_weight).astype(np.int32), c)
+    else:
+        with pytest.raises(NotImplementedError):
+            G.pack_matrix(Q, p)
     with pytest.raises(ValueError):
         G.gptq(W, [X], bits=9)
