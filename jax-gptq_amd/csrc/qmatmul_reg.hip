@@ -72,13 +72,19 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
     for (int rb = 0; rb < RB; ++rb) aq[slot][rb] = rg_load16<RAGGED>(x + xrow[rb] + koff);
   };
 
+  // the first k-steps' loads go out before anything that has to wait for memory
+#pragma unroll
+  for (int u = 0; u < RING; ++u) load_step(u, u);
+
   // ---- per-channel constants of the dequantisation (the integer part of the zero point)
   uint32_t zc[8];
   float zi8[(BF && BITS == 8) ? 8 : 1];
+  {
+    float z8[8];
+    rg_params8(zero, zs_dtype, col, C, z8);
 #pragma unroll
-  for (int t8 = 0; t8 < 8; ++t8) {
-    const float z = rg_param(zero, zs_dtype, min(col + t8, C - 1));
-    const float zi = fminf(fmaxf(rintf(z), -512.f), 512.f);
+    for (int t8 = 0; t8 < 8; ++t8) {
+    const float zi = fminf(fmaxf(rintf(z8[t8]), -512.f), 512.f);
     if constexpr (BF) {
       zc[t8] = 0u;
       if constexpr (BITS == 8) zi8[t8] = zi;
@@ -86,6 +92,7 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
       zc[t8] = __builtin_bit_cast(uint32_t, half2_t{(_Float16)(-(1024.f + zi)), (_Float16)(-(64.f + zi))});
     } else {
       zc[t8] = __builtin_bit_cast(uint32_t, half2_t{(_Float16)(-(1024.f + zi)), (_Float16)(-(1024.f + zi))});
+    }
     }
   }
   uint32_t mask = BF ? 0x000F000Fu : 0x00F0000Fu, cexp = BF ? 0x43004300u : 0x64006400u;
@@ -100,9 +107,6 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
   for (int i = 0; i < RB; ++i)
 #pragma unroll
     for (int j = 0; j < RG_NT; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-#pragma unroll
-  for (int u = 0; u < RING; ++u) load_step(u, u);
 
   auto compute = [&](int slot, auto masked) __attribute__((always_inline)) {
     uint4 a[RB];
@@ -192,6 +196,10 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
       if (u == slot) compute(u, tail);
   }
 
+  // scale and zero point of this lane's channels, in flight while the tiles are summed
+  float sc[8], zf[8];
+  rg_params8(scale, zs_dtype, col, C, sc);
+  rg_params8(zero, zs_dtype, col, C, zf);
   floatx4 sum[RG_NT];
   const int tile = blockIdx.y * gridDim.x + blockIdx.x;
   if (!rg_reduce<RB>(acc, sum, rg_lds, &s_flag, part, counters, tile, split, S)) return;
@@ -199,14 +207,9 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
   // m = m0 + 16 rb + 4 g + r
   if (!col_ok) return;
   const int rb = wk;                             // rg_reduce returned true: wk < RB
-  float sc[8], zf[8];
 #pragma unroll
-  for (int t8 = 0; t8 < 8; ++t8) {
-    const int n = min(col + t8, C - 1);
-    sc[t8] = rg_param(scale, zs_dtype, n);
-    const float z = rg_param(zero, zs_dtype, n);
-    zf[t8] = (BF && BITS == 4) ? 128.f + z : z - fminf(fmaxf(rintf(z), -512.f), 512.f);
-  }
+  for (int t8 = 0; t8 < 8; ++t8)
+    zf[t8] = (BF && BITS == 4) ? 128.f + zf[t8] : zf[t8] - fminf(fmaxf(rintf(zf[t8]), -512.f), 512.f);
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int m = m0 + 16 * rb + 4 * g + r;

@@ -58,26 +58,40 @@ __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, co
   _Float16 *tab_nz = tab_s + nch;
   float *tab_sf = rg_lds;
   uint32_t *tab_zt = reinterpret_cast<uint32_t *>(rg_lds + nch);
-  for (int i = tid; i < nch; i += 256) {
+  auto put = [&](int i, float s, float z) __attribute__((always_inline)) {
     const int c = c_begin + i;
-    float s = 0.f, z = 0.f;
-    if (c < C) {
-      s = rg_param(scale, zs_dtype, c);
-      z = rg_param(zero, zs_dtype, c);
-    }
     if (BF) {
       typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
       typedef float f2_t __attribute__((ext_vector_type(2)));
       // off + zi must be an integer bf16 holds exactly (magnitude <= 256)
       const float lim = BITS == 4 ? 128.f : 256.f, off = BITS == 4 ? 128.f : 0.f;
       const float zi = fminf(fmaxf(rintf(z), -lim), lim);
-      tab_sf[i] = s;
+      tab_sf[i] = c < C ? s : 0.f;
       tab_zt[i] = c < C ? __builtin_bit_cast(uint32_t, __builtin_convertvector(f2_t{off + zi, z - zi}, bf2_t)) : 0u;
     } else {
-      tab_s[i] = (_Float16)s;
-      tab_nz[i] = (_Float16)(-z * s);
+      tab_s[i] = (_Float16)(c < C ? s : 0.f);
+      tab_nz[i] = (_Float16)(c < C ? -z * s : 0.f);
     }
-  }
+  };
+  // the element type is switched on outside the loops, and a thread's loads of a round are independent:
+  // four channels' zero and scale in flight per thread instead of one load at a time
+  auto fill = [&](auto *zp, auto *sp) __attribute__((always_inline)) {
+    for (int i0 = tid; i0 < nch; i0 += 4 * 256) {
+      float zv[4], sv[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int c = min(c_begin + i0 + u * 256, C - 1);
+        zv[u] = to_f32(zp[c]);
+        sv[u] = to_f32(sp[c]);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (i0 + u * 256 < nch) put(i0 + u * 256, sv[u], zv[u]);
+    }
+  };
+  if (zs_dtype == GPTQ_HIP_F32) fill(reinterpret_cast<const float *>(zero), reinterpret_cast<const float *>(scale));
+  else if (zs_dtype == GPTQ_HIP_F16) fill(reinterpret_cast<const __half *>(zero), reinterpret_cast<const __half *>(scale));
+  else fill(reinterpret_cast<const __hip_bfloat16 *>(zero), reinterpret_cast<const __hip_bfloat16 *>(scale));
 
   const uint8_t *wpj[NG];
 #pragma unroll

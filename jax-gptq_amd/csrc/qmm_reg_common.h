@@ -38,6 +38,34 @@ __device__ __forceinline__ float rg_param(const void *p, int dtype, int i) {
   return __bfloat162float(reinterpret_cast<const __hip_bfloat16 *>(p)[i]);
 }
 
+// Elements first .. first + 7 (indices clamped to n - 1) of a zero / scale vector as fp32.  The element
+// type is switched on once, around eight independent loads: a switch per element would put every load
+// behind a branch and make the wavefront wait for each in turn.
+__device__ __forceinline__ void rg_params8(const void *p, int dtype, int first, int n, float (&out)[8]) {
+  int idx[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) idx[i] = min(first + i, n - 1);
+  if (dtype == GPTQ_HIP_F32) {
+    const float *q = reinterpret_cast<const float *>(p);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = q[idx[i]];
+  } else if (dtype == GPTQ_HIP_F16) {
+    const __half *q = reinterpret_cast<const __half *>(p);
+    __half h[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) h[i] = q[idx[i]];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = __half2float(h[i]);
+  } else {
+    const __hip_bfloat16 *q = reinterpret_cast<const __hip_bfloat16 *>(p);
+    __hip_bfloat16 h[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) h[i] = q[idx[i]];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = __bfloat162float(h[i]);
+  }
+}
+
 // Activations of a ragged last k-step: the lane wants the 8 elements [k0, k0 + 8) of its row, of which
 // only those below K exist; `a` was loaded from [kl, kl + 8) with kl = min(k0, K - 8) <= k0.  Returns the
 // wanted elements with zeros past K (element = 16 bits).
@@ -125,7 +153,11 @@ __device__ __forceinline__ bool rg_reduce(floatx4 (&acc)[RB][RG_NT], floatx4 (&s
   __syncthreads();
   if (tid == 0) {
     int32_t *ctr = counters + tile;
+#ifdef GPTQ_TICKET_RELACQ
+    const int ticket = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+#else
     const int ticket = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#endif
     const int last = ticket == S - 1;
     if (last) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     *s_flag = last;
@@ -135,29 +167,32 @@ __device__ __forceinline__ bool rg_reduce(floatx4 (&acc)[RB][RG_NT], floatx4 (&s
 #pragma unroll
   for (int t = 0; t < RG_NT; ++t) sum[t] = floatx4{0.f, 0.f, 0.f, 0.f};
   const float *src = part + (((int64_t)tile * S) * RB + rb_own) * (RG_NT * RG_TILE_FLOATS) + lane * 4;
-  // two splits' partials in flight at a time
-  for (int sp = 0; sp < S; sp += 2) {
-    const int sq = min(sp + 1, S - 1);
-    floatx4 pv[RG_NT], pw[RG_NT];
+  // NF splits' partials in flight at a time (a 16-row workgroup has the registers for four)
+  constexpr int NF = RB == 1 ? 4 : 2;
+  for (int sp = 0; sp < S; sp += NF) {
+    floatx4 pv[NF][RG_NT];
 #pragma unroll
-    for (int t = 0; t < RG_NT; ++t)
-      pv[t] = rg_load_part_issue(src + (int64_t)sp * RB * (RG_NT * RG_TILE_FLOATS) + t * RG_TILE_FLOATS);
+    for (int f = 0; f < NF; ++f) {
+      const int sq = min(sp + f, S - 1);
 #pragma unroll
-    for (int t = 0; t < RG_NT; ++t)
-      pw[t] = rg_load_part_issue(src + (int64_t)sq * RB * (RG_NT * RG_TILE_FLOATS) + t * RG_TILE_FLOATS);
+      for (int t = 0; t < RG_NT; ++t)
+        pv[f][t] = rg_load_part_issue(src + (int64_t)sq * RB * (RG_NT * RG_TILE_FLOATS) + t * RG_TILE_FLOATS);
+    }
     // the loads above are invisible to the compiler's wait counting: wait here, and make every use of
     // the values depend on this statement
-    asm volatile("s_waitcnt vmcnt(0)"
-                 : "+v"(pv[0]), "+v"(pv[1]), "+v"(pv[2]), "+v"(pv[3]), "+v"(pv[4]), "+v"(pv[5]), "+v"(pv[6]),
-                   "+v"(pv[7]), "+v"(pv[8]), "+v"(pw[0]), "+v"(pw[1]), "+v"(pw[2]), "+v"(pw[3]), "+v"(pw[4]),
-                   "+v"(pw[5]), "+v"(pw[6]), "+v"(pw[7]), "+v"(pw[8])
-                 :
-                 : "memory");
 #pragma unroll
-    for (int t = 0; t < RG_NT; ++t) sum[t] += pv[t];
-    if (sp + 1 < S) {
+    for (int f = 0; f < NF; ++f)
+      asm volatile("s_waitcnt vmcnt(0)"
+                   : "+v"(pv[f][0]), "+v"(pv[f][1]), "+v"(pv[f][2]), "+v"(pv[f][3]), "+v"(pv[f][4]), "+v"(pv[f][5]),
+                     "+v"(pv[f][6]), "+v"(pv[f][7]), "+v"(pv[f][8])
+                   :
+                   : "memory");
 #pragma unroll
-      for (int t = 0; t < RG_NT; ++t) sum[t] += pw[t];
+    for (int f = 0; f < NF; ++f) {
+      if (sp + f < S) {
+#pragma unroll
+        for (int t = 0; t < RG_NT; ++t) sum[t] += pv[f][t];
+      }
     }
   }
   return true;

@@ -194,3 +194,36 @@ def test_qmatmul_8bit_gradient_wrt_x(OP):
     ref = w.double().cpu().numpy() @ _dense(qm).T
     err = np.abs(x.grad.double().cpu().numpy() - ref)
     assert np.all(err <= ATOL + RTOL * np.abs(ref))
+
+
+@pytest.mark.parametrize("xdt", ["float16", "bfloat16"])
+@pytest.mark.parametrize("M,N,K", [(17, 1024, 4096), (64, 11008, 512), (100, 2048, 1000), (200, 4096, 1064),
+                                   (256, 1152, 2048), (33, 8192, 8192)])
+def test_qmatmul_4bit_few_rows_against_a_whole_matrix(OP, M, N, K, xdt):
+    """16 < M <= 256 on aligned shapes: the register-operand kernel with and without a split of the
+    contraction, full and ragged last k-steps (K % 32 != 0), fractional zero points."""
+    import torch
+    import jax_gptq_amd.gptq as G
+    rng = np.random.default_rng(M + N + K)
+    codes = rng.integers(0, 16, (K, N)).astype(np.uint8)
+    scale = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    zero = rng.uniform(0.0, 15.0, N).astype(np.float32)
+    qm_ref = O.QuantizedMatrix(O.pack_colwise(codes), zero, scale)
+    qm = G.QuantizedMatrix(torch.from_numpy(qm_ref.int_weight).cuda(), torch.from_numpy(zero).cuda(),
+                           torch.from_numpy(scale).cuda())
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(getattr(torch, xdt))
+    for rep in range(2):                       # the second call finds the arrival counters as the first left them
+        got = OP.quantized_matmul(x, qm)
+        _check(got, x.double().numpy(), qm_ref, False, rtol=RTOL if xdt == "float16" else 2.0 ** -8)
+
+
+def test_qmatmul_more_rows_than_a_grid_dimension_on_the_plain_kernels(OP):
+    """Shapes no matrix-core kernel takes (fewer than 8 channels) with M > 65535: several launches."""
+    import torch
+    qm = _matrix4(5, 16, 4, np.float32)
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((70000, 16)).astype(np.float16)
+    got = OP.quantized_matmul(x, qm)
+    _check(got, x.astype(np.float64), qm, False)
+    y = (0.05 * rng.standard_normal((70000, 4))).astype(np.float16)
+    _check(OP.quantized_matmul(y, qm, transpose_b=True), y.astype(np.float64), qm, True)

@@ -22,10 +22,12 @@ SHAPES = [
     (7168, 28672, 128),
     (28672, 7168, 128),  # 30 GB of calibration rows resident
 ]
+# the large-layer configuration also names 8-bit codes (one per byte; not in the reference)
+SHAPES = [s + (4,) for s in SHAPES] + [(7168, 28672, 128, 8), (28672, 7168, 16, 8)]
 
 
-@pytest.mark.parametrize("K,N,nb", SHAPES)
-def test_layer_properties(K, N, nb):
+@pytest.mark.parametrize("K,N,nb,bits", SHAPES)
+def test_layer_properties(K, N, nb, bits):
     import torch
     import jax_gptq_amd.gptq as G
     from jax_gptq_amd.op import quantized_matmul
@@ -36,7 +38,9 @@ def test_layer_properties(K, N, nb):
     xs = [torch.randn((2048, K), generator=g, device="cuda") for _ in range(nb)]
 
     W32 = W.float()
-    params = G.get_col_quantize_params(W32)
+    params = G.get_col_quantize_params(W32, bits=bits)
+    maxq = 2 ** bits - 1
+    assert params["maxq"] == maxq
     H = G.accumulate_H(xs)
     assert bool((H == H.T).all())
     if nb > 16:
@@ -68,16 +72,18 @@ def test_layer_properties(K, N, nb):
     del L
     sc, z = params["scale"], params["zero"]
     codes = Q.float() / sc + z
-    assert float((codes - codes.round()).abs().max()) < 2e-2   # fp16 rounding of scale*(c-z)
-    assert float(codes.round().min()) >= 0 and float(codes.round().max()) <= 15
+    # fp16 rounding of scale*(c-z): 2^-11 of a magnitude of up to maxq code steps
+    assert float((codes - codes.round()).abs().max()) < (2e-2 if bits == 4 else 0.2)
+    assert float(codes.round().min()) >= 0 and float(codes.round().max()) <= maxq
 
     packed = G.pack_matrix(Q, params)
-    assert packed.int_weight.shape == (K // 2, N) and packed.int_weight.dtype == torch.uint8
+    assert packed.bits == bits and packed.shape == (K, N)
+    assert packed.int_weight.shape == (K // 2 if bits == 4 else K, N) and packed.int_weight.dtype == torch.uint8
     assert bool((G.unpack_matrix(packed).to(torch.float16) == Q).all())
 
     X = xs[0]
     Wf = W.float()
-    rtn = sc * (torch.clamp(torch.round(Wf / sc) + z, 0, 15) - z)
+    rtn = sc * (torch.clamp(torch.round(Wf / sc) + z, 0, maxq) - z)
     ref = (X @ Wf).norm()
     e_gptq = float((X @ (Wf - Q.float())).norm() / ref)
     e_rtn = float((X @ (Wf - rtn)).norm() / ref)
