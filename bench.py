@@ -18,8 +18,10 @@ Prints ONE JSON line.  Besides the contract keys it carries
   phases_ms      per-phase GPU time of one step,
   fp16_calibration  the same layer with the calibration rows stored in fp16,
   fp32_rows_split_fp16  the fp32 rows multiplied as pairs of fp16 numbers (opt-in path),
-  qmatmul        packed-int4 matmul at M = 1, 16, 128 against the HBM roofline
-                 (weights rotated over > 512 MB of copies so that they come from HBM).
+  qmatmul        packed-int4 matmul at M = 1, 16, 128, 2048 against the HBM and 16-bit MFMA rooflines
+                 (weights rotated over > 512 MB of copies so that they come from HBM), 8-bit codes and
+                 a vocabulary-sized N included,
+  hbm_read_ceiling  a kernel that only reads, at the packed sizes of the matmul cases.
 """
 import argparse
 import json
@@ -64,7 +66,7 @@ def one_layer(G, W, xs, timers=None, split_fp16=False):
             ev[i].record()
 
     mark(0)
-    W32 = W.to(torch.float32)
+    W32 = G._to_f32_copy(W)
     params = G.get_col_quantize_params(W32)
     mark(1)
     H = G.accumulate_H(xs, split_fp16=split_fp16)
@@ -129,15 +131,15 @@ def bench_hessian_streamed(G, xs, reps=2):
     n = sum(x.shape[0] for x in xs)
 
     def streamed():
-        H = torch.zeros((K, K), dtype=torch.float32, device="cuda")
+        H = G._zeros((K, K), torch.float32)
         for x in xs:
             G._hessian_accumulate(H, [x])
         _native.check(lib.gptq_hip_hessian_finalize(G._stream(), G._ptr(H), _native.F32, K, float(n)), "finalize")
         return H
 
     def stepped():
-        H = torch.zeros((K, K), dtype=torch.float32, device="cuda")
-        m = torch.zeros(K, dtype=torch.float32, device="cuda")
+        H = G._zeros((K, K), torch.float32)
+        m = G._zeros((K,), torch.float32)
         cnt = 0
         for x in xs:
             H, m, cnt = G._accumulate_H_step(H, m, cnt, x)
@@ -179,31 +181,36 @@ def bench_qmatmul(reps=240):
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     # the two Llama-7B MLP shapes of the benchmark layer, then the OPT-30B fc1 shape (103 MB packed:
     # decode matmuls of that size run the streaming kernel)
-    for (K, N) in ((4096, 11008), (11008, 4096), (7168, 28672)):
-        copies = 24 if K * N < (1 << 27) else 6
-        iws = [torch.randint(0, 256, (K // 2, N), generator=g, device="cuda", dtype=torch.uint8)
+    # (K, N, bits): the last two are what the register-operand kernels serve: 8-bit codes (one per byte)
+    # and a vocabulary-sized N that is not a multiple of 16 channels
+    for (K, N, bits) in ((4096, 11008, 4), (11008, 4096, 4), (7168, 28672, 4), (4096, 11008, 8), (768, 50257, 4)):
+        R = K // 2 if bits == 4 else K
+        copies = max(6, min(24, (560 << 20) // (R * N)))
+        iws = [torch.randint(0, 256, (R, N), generator=g, device="cuda", dtype=torch.uint8)
                for _ in range(copies)]
         scale = (0.001 + 0.009 * torch.rand(N, generator=g, device="cuda")).to(torch.float16)
         zero = torch.randint(0, 16, (N,), generator=g, device="cuda").to(torch.float16)
         # forward at the decode / small-batch sizes, and the transposed (VJP) product at 2048 rows
         cases = [(1, 0, "float16"), (16, 0, "float16"), (128, 0, "float16"), (2048, 0, "float16"),
                  (2048, 1, "float16")]
-        if K == K_IN:
+        if K == K_IN and bits == 4:
             cases += [(1, 0, "bfloat16"), (16, 0, "bfloat16"), (2048, 1, "bfloat16")]
         if K * N >= (1 << 27):
             cases = [(1, 0, "float16"), (16, 0, "float16")]
+        if N % 16:
+            cases = [(1, 0, "float16"), (16, 0, "float16"), (512, 0, "float16"), (512, 1, "float16")]
         for (M, tr, xdt) in cases:
             tdt = getattr(torch, xdt)
             xcode = _native.F16 if xdt == "float16" else _native.BF16
             x = torch.randn((M, N if tr else K), generator=g, device="cuda").to(tdt)
             y = torch.empty((M, K if tr else N), dtype=tdt, device="cuda")
-            ws = torch.zeros(max(lib.gptq_hip_qmatmul_workspace_bytes(M, K // 2, N, tr), 256),
+            ws = torch.zeros(max(lib.gptq_hip_qmatmul_bits_workspace_bytes(M, R, N, tr, xcode, bits), 256),
                              dtype=torch.uint8, device="cuda")
 
             def call(i):
-                rc = lib.gptq_hip_qmatmul(st, x.data_ptr(), xcode, M, iws[i % copies].data_ptr(),
-                                          K // 2, N, zero.data_ptr(), scale.data_ptr(), _native.F16, tr,
-                                          y.data_ptr(), ws.data_ptr(), ws.numel())
+                rc = lib.gptq_hip_qmatmul_bits(st, x.data_ptr(), xcode, M, iws[i % copies].data_ptr(),
+                                               R, N, zero.data_ptr(), scale.data_ptr(), _native.F16, bits, tr,
+                                               y.data_ptr(), ws.data_ptr(), ws.numel())
                 assert rc == 0, rc
 
             for i in range(copies):
@@ -223,13 +230,49 @@ def bench_qmatmul(reps=240):
             e1.record()
             torch.cuda.synchronize()
             us_cached = e0.elapsed_time(e1) * 1e3 / reps
-            nbytes = K * N // 2 + 2 * N * 2 + M * K * 2 + M * N * 2
-            out.append({"M": M, "K": K, "N": N, "transpose_b": tr, "x_dtype": xdt, "us": round(us, 2),
+            nbytes = R * N + 2 * N * 2 + M * K * 2 + M * N * 2
+            out.append({"M": M, "K": K, "N": N, "bits": bits, "transpose_b": tr, "x_dtype": xdt, "us": round(us, 2),
                         "us_cache_resident": round(us_cached, 2),
                         "algorithmic_bytes": nbytes,
                         "GBps": round(nbytes / us * 1e-3, 1),
                         "hbm_frac": round(nbytes / us * 1e-3 / HBM_PEAK_GBS, 4),
-                        "TFLOPs": round(2.0 * M * K * N / us * 1e-6, 2)})
+                        "TFLOPs": round(2.0 * M * K * N / us * 1e-6, 2),
+                        "mfma16_frac": round(2.0 * M * K * N / us * 1e-6 / MFMA16_PEAK_TFLOPS, 4)})
+        del iws
+    return out
+
+
+def bench_read_ceiling(reps=100):
+    """What a kernel that only reads gets from the memory system at the packed sizes of the matmul cases
+    (gptq_hip_read_probe: linear 16-byte loads, eight in flight per thread; buffers rotated like the weights):
+    the practical ceiling of any HBM-bound kernel launched on its own at that size."""
+    import ctypes
+    import torch
+    from jax_gptq_amd import _native
+    lib = _native.load()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+    out = []
+    for nbytes in (4096 * 11008 // 2, 4096 * 11008, 7168 * 28672 // 2, 1 << 30):
+        copies = max(2, min(24, (1200 << 20) // nbytes))
+        bufs = [torch.full((nbytes,), i + 1, dtype=torch.uint8, device="cuda") for i in range(copies)]
+        best = None
+        for wgs in (256, 512, 2048):
+            for i in range(copies):
+                assert lib.gptq_hip_read_probe(st, bufs[i].data_ptr(), nbytes, wgs, sink.data_ptr()) == 0
+            torch.cuda.synchronize()
+            e0, e1 = _events(2)
+            e0.record()
+            for i in range(reps):
+                lib.gptq_hip_read_probe(st, bufs[i % copies].data_ptr(), nbytes, wgs, sink.data_ptr())
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / reps
+            if best is None or us < best[0]:
+                best = (us, wgs)
+        out.append({"bytes": nbytes, "us": round(best[0], 2), "workgroups": best[1],
+                    "GBps": round(nbytes / best[0] * 1e-3, 1), "hbm_frac": round(nbytes / best[0] * 1e-3 / HBM_PEAK_GBS, 4)})
+        del bufs
     return out
 
 
@@ -306,10 +349,11 @@ def main():
                     help="--section hessian only: fp32 rows as pairs of fp16 numbers (accumulate_H(split_fp16=True))")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-qmatmul", action="store_true", help="skip the int4 matmul section")
-    ap.add_argument("--section", default="all", choices=["all", "hessian", "qmatmul", "copy"],
-                    help="profiling aid: run only one part (hessian: X^T X over the 128 batches; "
-                         "qmatmul: the int4 matmul loop; copy: a plain 1 GiB device copy used to "
-                         "calibrate the FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--section", default="all", choices=["all", "hessian", "factor", "solve", "qmatmul", "copy"],
+                    help="profiling aid: run only one part (hessian: X^T X over the 128 batches; factor: damping + "
+                         "Cholesky factor of the inverse of a K = 4096 Hessian; solve: the blocked column loop of the "
+                         "4096 x 11008 layer; qmatmul: the packed matmul loop; copy: a plain 1 GiB device copy used "
+                         "to calibrate the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (use --gpus 1)")
@@ -329,7 +373,33 @@ def main():
                           "bytes_written": src.numel() * 4, "launches": max(1, args.steps)}))
         return
     if args.section == "qmatmul":
-        print(json.dumps({"section": "qmatmul", "qmatmul": bench_qmatmul()}))
+        print(json.dumps({"section": "qmatmul", "qmatmul": bench_qmatmul(), "hbm_read_ceiling": bench_read_ceiling()}))
+        return
+    if args.section in ("factor", "solve"):
+        # a well-conditioned Hessian from 8 batches is enough: the phases below do not depend on its content
+        W, xs = make_inputs(K_IN, N_OUT, 8, ROWS, torch.float16)
+        H0 = G.accumulate_H(xs)
+        params = G.get_col_quantize_params(G._to_f32_copy(W))
+        n = max(1, args.steps)
+        if args.section == "factor":
+            G._damp_invert(None, G._clone(H0), 0.01, fix_dead=False)
+            e0, e1 = _events(2)
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(n):
+                G._damp_invert(None, G._clone(H0), 0.01, fix_dead=False)
+            e1.record()
+        else:
+            L, _, _ = G._damp_invert(None, G._clone(H0), 0.01, fix_dead=False)
+            G._solve(G._to_f32_copy(W), L, params, 128, W.dtype)
+            e0, e1 = _events(2)
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(n):
+                G._solve(G._to_f32_copy(W), L, params, 128, W.dtype)
+            e1.record()
+        torch.cuda.synchronize()
+        print(json.dumps({"section": args.section, "ms": round(e0.elapsed_time(e1) / n, 3)}))
         return
 
     W, xs = make_inputs(K_IN, N_OUT, N_BATCH, ROWS, getattr(torch, args.x_dtype))
@@ -435,6 +505,8 @@ def main():
         result["roofline_qmatmul"] = {"kernel": "qmatmul M=1 4096x11008", "bound": "hbm",
                                       "achieved": m1["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                       "frac": m1["hbm_frac"], "traffic": qmatmul_traffic_bytes()}
+        # the practical ceiling: a kernel that only reads, at the same sizes
+        result["hbm_read_ceiling"] = bench_read_ceiling()
     if args.section == "all":
         result["hessian_streamed"] = bench_hessian_streamed(G, xs)
     if not args.no_cpu:

@@ -56,6 +56,12 @@ int gptq_hip_fill_zero(void *stream, void *ptr, size_t bytes);
 int gptq_hip_copy(void *stream, void *dst, const void *src, size_t bytes);
 int gptq_hip_to_f32(void *stream, const void *in, int in_dtype, int64_t n, float *out);
 
+/* Measurement aid, not part of the path: reads `bytes` bytes (16-byte aligned) linearly with `workgroups`
+ * workgroups of 256 threads, eight 16-byte loads in flight per thread, and does nothing else.  Its duration
+ * is what the memory system delivers to a pure read of that size on this device: the yardstick bench.py
+ * reports next to the HBM-bound matmul.  `sink` is a device word that is (practically) never written. */
+int gptq_hip_read_probe(void *stream, const void *ptr, size_t bytes, int workgroups, uint32_t *sink);
+
 /* ---- per-column quantisation parameters -------------------------------------
  * Replaces get_quantize_params / get_col_quantize_params (gptq.py:105-118).
  * W [K, N] (element type w_dtype, row stride ldw) -> scale[N], zero[N] (fp32).

@@ -509,7 +509,7 @@ __global__ __launch_bounds__(256, 2) void qmm_fwd_stream_kernel(
 //    wavefront w is the 16 rows (t NW + w) 16 .. + 15 of that range, KS k-steps per wavefront, all
 //    loads issued before anything else; k-steps past the range are skipped (wave-uniform branch);
 //  * the column parameters of the outputs a thread will finish are fetched under the weight loads;
-//  * M <= 8 (ATOM; MR = 1, 4 or 16 rows of the tile kept): the workgroups of a strip add their partial results to 64-bit
+//  * ATOM (M <= 8, and larger M while the atomics stay few; MR = 1, 4 or 16 rows of the tile kept): the workgroups of a strip add their partial results to 64-bit
 //    accumulators with ONE returning atomic per output: the word is value * 2^28 (fixed point,
 //    a partial beyond +-65536 or not finite adds the poison 3 * 2^49 instead) << 8 | 1, so the
 //    returned old word tells the caller whether it was the last of the S contributions, and the
@@ -517,9 +517,9 @@ __global__ __launch_bounds__(256, 2) void qmm_fwd_stream_kernel(
 //    Integer addition is exact and commutative: the result does not depend on the arrival order.
 //    One round trip to the memory side instead of three (partial stores -> ticket -> partial
 //    loads).  A poisoned sum yields NaN.  S <= 32.
-//  * M > 8: the atomics of that many rows take longer than the ticket scheme (the memory side
-//    retires them at a limited rate: 350000 of them add 2 us, 700000 add 4), so those keep
-//    qmm_reduce_and_store (ATOM = false).
+//  * M > 8: the memory side retires the atomics at a limited rate (350000 of them add 2 us, 700000
+//    add 4); where there would be more than ~760000, or the matrix runs in ring-loop mode, the
+//    workgroups keep qmm_reduce_and_store (ATOM = false).
 constexpr int QD_FRAC = 28;
 constexpr long long QD_POISON = 3LL << 49;
 constexpr int QD_MAX_SPLITS = 32;
@@ -800,7 +800,7 @@ DecPlan dec_plan(int64_t M, int64_t R, int64_t C) {
   p.strips = (int)ceil_div64(C, QSTRIP);
   if (p.strips > QMM_MAX_COUNTERS) return p;
   p.mr = M == 1 ? 1 : (M <= 4 ? 4 : 16);
-  p.atom = M <= 8 && M * C * 8 <= QMM_ACC_BYTES;
+  p.atom = M * C * 8 <= QMM_ACC_BYTES;
   if (p.mr <= 4) {
     if (!p.atom) return p;
     // eight wavefronts, two workgroups per CU: as many splits as 512 slots allow, at least 128 rows each
@@ -843,6 +843,10 @@ DecPlan dec_plan(int64_t M, int64_t R, int64_t C) {
       p.loop = true;
     }
     if (p.S > QD_MAX_SPLITS) p.atom = false;
+    // Beyond 8 rows the atomics pay only while there are few of them (the memory side retires them at a
+    // limited rate) and the matrix is one the chip holds in flight: 4096 x 11008 at M = 16 (700000 atomics)
+    // 15.4 -> 14.4 us, 11008 x 4096 18.2 -> 13.9 us, but 7168 x 28672 (ring-loop mode, 920000) 26.8 -> 29.0 us.
+    if (M > 8 && (p.loop || M * C * p.S > 760000)) p.atom = false;
     if (p.atom) {
       p.x1_bytes = p.part_bytes = 0;
       p.total_bytes = p.S > 1 ? QMM_HEAD_BYTES : 0;

@@ -24,6 +24,7 @@ SIGNATURES = {
     "gptq_hip_fill_zero": (_i32, [_vp, _vp, _sz]),
     "gptq_hip_copy": (_i32, [_vp, _vp, _vp, _sz]),
     "gptq_hip_to_f32": (_i32, [_vp, _vp, _i32, _i64, _vp]),
+    "gptq_hip_read_probe": (_i32, [_vp, _vp, _sz, _i32, _vp]),
     "gptq_hip_col_params_workspace_bytes": (_sz, [_i64, _i64]),
     "gptq_hip_col_params": (_i32, [_vp, _vp, _i32, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _sz]),
     "gptq_hip_hessian_accumulate_workspace_bytes": (_sz, [_i64, _i32]),
