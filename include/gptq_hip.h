@@ -96,7 +96,9 @@ int gptq_hip_hessian_accumulate_split16(void *stream, const void *const *x_ptrs,
  * algebraically (H = sum X^T X / n), so none is kept.
  * ws: gptq_hip_hessian_accumulate_workspace_bytes(K, h_dtype) bytes (0 for large K and for fp64).
  * gptq_hip_hessian_finalize multiplies by 1/n_samples and mirrors the upper
- * triangle into the lower one, giving the full symmetric H the reference returns. */
+ * triangle into the lower one, giving the full symmetric H the reference returns.
+ * Limits: K <= 46000 (one launch's table of tiles), a call's batches at most 2^31 rows in all;
+ * GPTQ_HIP_EINVAL beyond them. */
 size_t gptq_hip_hessian_accumulate_workspace_bytes(int64_t K, int h_dtype);
 int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const int64_t *x_rows,
                                 int n_batches, int x_dtype, int64_t K, void *H, int h_dtype,
@@ -114,7 +116,9 @@ int gptq_hip_hessian_finalize(void *stream, void *H, int h_dtype, int64_t K, dou
  * status (device int32[2]): status[0] = 0, or 1 + index of the first 64-block whose
  * pivot was not positive (L then holds NaN, as the reference's does, gptq.py:166);
  * status[1] = number of dead features.  fix_dead = 0 skips the dead-feature fix (with
- * damping = 0 the call is then exactly _cholesky_inv, gptq.py:44-48). */
+ * damping = 0 the call is then exactly _cholesky_inv, gptq.py:44-48).
+ * Limit: K <= 65535 (rows are a grid dimension), also for gptq_hip_zero_dead_rows and the
+ * gathers below; GPTQ_HIP_EINVAL beyond it. */
 size_t gptq_hip_damp_invert_workspace_bytes(int64_t K, int h_dtype);
 int gptq_hip_damp_invert(void *stream, void *H, int h_dtype, float *W, int64_t K, int64_t N,
                          int64_t ldw, double damping, int fix_dead, void *L, float *L32,
@@ -206,6 +210,10 @@ int gptq_hip_dequant_bits(void *stream, const uint8_t *packed, int64_t outer, in
  * to fp16 precision (after a per-row power-of-two scaling that keeps any fp32 magnitude in
  * range; the result is scaled back after its rounding to fp16) and run on the same matrix-core kernels as fp16 ones; with the smaller workspace, or
  * other shapes, they run unrounded on plain kernels that are an order of magnitude slower.
+ * Any M, R, C below 2^30: shapes with C % 16 == 0 and 16-byte aligned operands run on the tuned
+ * kernels, other shapes with C >= 8 and 2R >= 8 (rows that are not multiples of 16 channels, e.g. a
+ * vocabulary-sized C; unaligned views) on matrix-core kernels that take unaligned loads, the rest on
+ * plain kernels (several launches where M exceeds a grid dimension).
  * The workspace begins with arrival counters of the split-K reduction: it must be
  * ZERO-FILLED before its first use; every call leaves the counters zero again, so one
  * buffer can serve any sequence of calls that do not overlap in time. */

@@ -972,7 +972,9 @@ __global__ __launch_bounds__(256, 2) void qmm_fwd_gemm_kernel(const TX *x, int M
   float *rowsum = reinterpret_cast<float *>(qgemm_lds + 2 * A_HALVES + 2 * B_HALVES);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1, g = lane >> 4, l16 = lane & 15;
-  const int n0 = blockIdx.x * BN, m0 = blockIdx.y * BM;
+  int tx, ty;
+  qmm_tile_coords(tx, ty);
+  const int n0 = tx * BN, m0 = ty * BM;
   // split-K: this workgroup multiplies the stages [kbeg, kend) of the contraction axis
   const int split = SPLIT ? blockIdx.z : 0;
   const int sps = ((K + GBK - 1) / GBK + S - 1) / S;
@@ -1139,7 +1141,7 @@ __global__ __launch_bounds__(256, 2) void qmm_fwd_gemm_kernel(const TX *x, int M
     // Partial tile and partial row sums to the workspace (agent-scope write-through stores), an
     // arrival ticket per output tile; the last workgroup of a tile adds the S partials in split
     // order, so the result does not depend on the arrival order, and leaves the counter at zero.
-    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+    const int tile = ty * gridDim.x + tx;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int n = n0 + wn * (BN / 2) + j * 16 + l16;
@@ -1366,7 +1368,9 @@ __global__ __launch_bounds__(256, 2) void qmm_bwd_gemm_kernel(const TX *x, int M
   __shared__ __attribute__((aligned(16))) _Float16 Bs[2][B_HALVES];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1, g = lane >> 4, l16 = lane & 15;
-  const int j0 = blockIdx.x * (BN / 2), m0 = blockIdx.y * GBM;
+  int tx, ty;
+  qmm_tile_coords(tx, ty);
+  const int j0 = tx * (BN / 2), m0 = ty * GBM;
 
   // B staging: thread -> packed row j0 + tid/4, 16 channels at (tid%4)*16 of the stage
   // A staging, fp16: thread -> row tid/4, the same 16 channels (whose zero and scale the thread

@@ -41,7 +41,9 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
   __shared__ int s_flag;
   const int tid = threadIdx.x, lane = tid & 63, wk = tid >> 6;
   const int g = lane >> 4, l16 = lane & 15;
-  const int m0 = blockIdx.y * (16 * RB), nbase = blockIdx.x * RG_BN, split = blockIdx.z;
+  int tx, ty;
+  qmm_tile_coords(tx, ty);
+  const int m0 = ty * (16 * RB), nbase = tx * RG_BN, split = blockIdx.z;
   const int T = (K + 31) >> 5;
   // this workgroup's k-steps [t_begin, t_end); wavefront wk takes t_begin + wk, + 4, ...
   const int t_begin = split * steps_per_split, t_end = min(T, t_begin + steps_per_split);
@@ -63,7 +65,8 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
   uint2 wr[RING][NL];
   uint4 aq[RING][RB];
   auto load_step = [&](int slot, int s) __attribute__((always_inline)) {
-    const int t = min(t_begin + 4 * s + wk, T - 1);
+    // (steps past this workgroup's range re-read its own last k-step, a cache hit, not the next split's rows)
+    const int t = min(t_begin + 4 * s + wk, max(t_end - 1, 0));
 #pragma unroll
     for (int i = 0; i < NL; ++i)
       wr[slot][i] = rg_load8<RAGGED>(wp + (int64_t)min(PR * t + NL * g + i, R - 1) * C);
@@ -201,7 +204,7 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
   rg_params8(scale, zs_dtype, col, C, sc);
   rg_params8(zero, zs_dtype, col, C, zf);
   floatx4 sum[RG_NT];
-  const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+  const int tile = ty * gridDim.x + tx;
   if (!rg_reduce<RB>(acc, sum, rg_lds, &s_flag, part, counters, tile, split, S)) return;
   // sum[t8][r] = sum_k x[m][k] (code - zi)[k][col + t8] (bf16, 4-bit: code + 128), sum[8][r] = sum_k x[m][k],
   // m = m0 + 16 rb + 4 g + r

@@ -43,7 +43,9 @@ __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, co
   __shared__ int s_flag;
   const int tid = threadIdx.x, lane = tid & 63, wk = tid >> 6;
   const int g = lane >> 4, l16 = lane & 15;
-  const int j0 = blockIdx.x * NJ, m0 = blockIdx.y * (16 * RB), split = blockIdx.z;
+  int tx, ty;
+  qmm_tile_coords(tx, ty);
+  const int j0 = tx * NJ, m0 = ty * (16 * RB), split = blockIdx.z;
   const int T = (C + 31) >> 5;
   const int t_begin = split * steps_per_split, t_end = min(T, t_begin + steps_per_split);
   const int range = max(0, t_end - t_begin);
@@ -103,7 +105,8 @@ __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, co
   uint2 wr[RING][NG];
   uint4 aq[RING][RB];
   auto load_step = [&](int slot, int s) __attribute__((always_inline)) {
-    const int t = min(t_begin + 4 * s + wk, T - 1);
+    // (steps past this workgroup's range re-read its own last k-step, a cache hit, not the next split's rows)
+    const int t = min(t_begin + 4 * s + wk, max(t_end - 1, 0));
     const int c = min(32 * t + 8 * g, C - 8);                        // C >= 8
 #pragma unroll
     for (int jg = 0; jg < NG; ++jg) wr[slot][jg] = rg_load8<RAGGED>(wpj[jg] + c);
@@ -256,7 +259,7 @@ __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, co
 
   __syncthreads();                                                   // every wavefront is done with the tables
   floatx4 sum[RG_NT];
-  const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+  const int tile = ty * gridDim.x + tx;
   if (!rg_reduce<RB>(acc, sum, rg_lds, &s_flag, part, counters, tile, split, S)) return;
   const int rb = wk;
   const int64_t KO = BITS == 4 ? 2 * (int64_t)R : R;

@@ -64,4 +64,27 @@ __host__ __device__ inline QmmWs qmm_ws(void *base_v, size_t x1_bytes) {
   return ws;
 }
 
+// Output tile of this workgroup.  Workgroups are dealt to the 8 XCDs round-robin in dispatch order (x fastest),
+// and each XCD has its own L2.  Column tile tx belongs to XCD tx % 8, which walks its column tiles in blocks of
+// up to 8 row tiles: the workgroups running on an XCD at one time form a block of a few column tiles x a few row
+// tiles, so a weight tile is fetched once per block of row tiles (not once per row tile and XCD) and a row tile's
+// activations once per group of column tiles.  The last gx % 8 column tiles keep the plain order.
+__device__ __forceinline__ void qmm_tile_coords(int &tx, int &ty) {
+  const int gx = gridDim.x, gy = gridDim.y;
+  const int id = blockIdx.x + gx * blockIdx.y;
+  const int full = (gx >> 3) << 3;
+  if (id < full * gy) {
+    constexpr int BY = 8;
+    const int c = id & 7, sl = id >> 3, nq = full >> 3;
+    const int yb = min(sl / (BY * nq), (gy - 1) / BY);
+    const int r = sl - yb * BY * nq, by = min(BY, gy - yb * BY);
+    tx = (r / by) * 8 + c;
+    ty = yb * BY + r % by;
+  } else {
+    const int r = id - full * gy, rem = gx - full;
+    tx = full + r % rem;
+    ty = r / rem;
+  }
+}
+
 }  // namespace qmm
