@@ -236,6 +236,33 @@ int gptq_hip_qmatmul_bits(void *stream, const void *x, int x_dtype, int64_t M, c
                           int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, int bits,
                           int transpose_b, void *out, void *ws, size_t ws_bytes);
 
+/* ---- grouped parameters ------------------------------------------------------------------------
+ * No counterpart in the reference, which has one scale / zero per output channel (gptq.py:105-118):
+ * here every group of group_size consecutive input features (rows of W) has its own scale / zero per
+ * channel, tables [K / group_size, N] (fp32 from the solve).
+ * gptq_hip_solve_grouped is gptq_hip_solve with the parameters of rows [r0, r0 + group_size) taken, when
+ * the column loop reaches r0, from the column minima / maxima of those rows as they then stand (every
+ * correction of the rows above applied), by the rule of get_col_quantize_params (gptq.py:105-118) with
+ * maxq = 2^bits - 1, and written to row r0 / group_size of scale_g / zero_g.  group_size must be a multiple
+ * of block_size, divide K and divide the loop's update group (512 rows for block_size 128): 128, 256, 512.
+ * ws: gptq_hip_solve_grouped_workspace_bytes.
+ * quantize_pack_grouped / dequant_grouped: pack_matrix / unpack_matrix (gptq.py:214-235) for a 2-D W [K, N]
+ * packed along the rows with such tables (group_size even, dividing K; bits 4 or 8).
+ * gptq_hip_qmatmul_grouped: the product of gptq_hip_qmatmul_bits with zero / scale [K / group_size, C];
+ * matrix-core kernels for group_size % 32 == 0 (transpose_b = 1: % 128 == 0), plain kernels otherwise;
+ * ws as for gptq_hip_qmatmul_bits (gptq_hip_qmatmul_bits_workspace_bytes). */
+size_t gptq_hip_solve_grouped_workspace_bytes(int64_t K, int64_t N, int block_size, int group_size);
+int gptq_hip_solve_grouped(void *stream, float *W, int64_t K, int64_t N, const float *L, int group_size, int bits,
+                           int block_size, void *Q, int q_dtype, uint8_t *codes, float *scale_g, float *zero_g,
+                           void *ws, size_t ws_bytes);
+int gptq_hip_quantize_pack_grouped(void *stream, const void *Q, int q_dtype, int64_t K, int64_t N, const float *scale,
+                                   const float *zero, int64_t group_size, int bits, uint8_t *packed);
+int gptq_hip_dequant_grouped(void *stream, const uint8_t *packed, int64_t R, int64_t C, const void *zero,
+                             const void *scale, int zs_dtype, int64_t group_size, int bits, void *out);
+int gptq_hip_qmatmul_grouped(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
+                             int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype,
+                             int64_t group_size, int bits, int transpose_b, void *out, void *ws, size_t ws_bytes);
+
 /* ---- packed-int4 matmul that allocates nothing and takes no workspace ----------------------
  * No counterpart in the reference.  For callers that cannot allocate device memory: code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same operation,

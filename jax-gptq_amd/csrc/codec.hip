@@ -145,6 +145,52 @@ __global__ __launch_bounds__(TPB) void dequant8_kernel(const uint8_t *codes, int
   }
 }
 
+// Grouped parameters (an extension: the reference has one scale / zero per channel): W [K, N] with the
+// contraction along the rows, scale / zero [K / group, N]; row r uses row r / group of the tables.
+template <typename TQ, int BITS>
+__global__ __launch_bounds__(TPB) void quantize_pack_grouped_kernel(const TQ *Q, int64_t K, int64_t N,
+                                                                    const float *scale, const float *zero,
+                                                                    int64_t group, uint8_t *packed) {
+  const int64_t rows = BITS == 4 ? K / 2 : K, total = rows * N;
+  for (int64_t idx = (int64_t)blockIdx.x * TPB + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * TPB) {
+    const int64_t i = idx % N, j = idx / N;
+    if (BITS == 4) {
+      const int64_t gi = (2 * j) / group;                       // group is even: both rows in one group
+      const float sc = scale[gi * N + i], z = zero[gi * N + i];
+      const uint8_t lo = code_of(to_f32(Q[(2 * j) * N + i]), sc, z);
+      const uint8_t hi = code_of(to_f32(Q[(2 * j + 1) * N + i]), sc, z);
+      packed[idx] = (uint8_t)(lo | (uint8_t)(hi << 4));
+    } else {
+      const int64_t gi = j / group;
+      packed[idx] = code_of(to_f32(Q[idx]), scale[gi * N + i], zero[gi * N + i]);
+    }
+  }
+}
+
+template <typename T, int BITS>
+__global__ __launch_bounds__(TPB) void dequant_grouped_kernel(const uint8_t *packed, int64_t R, int64_t C,
+                                                              const T *zero, const T *scale, int64_t group,
+                                                              T *out) {
+#pragma clang fp contract(off)
+  const int64_t total = R * C;
+  for (int64_t idx = (int64_t)blockIdx.x * TPB + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * TPB) {
+    const int64_t i = idx % C, j = idx / C;
+    const uint8_t b = packed[idx];
+    if (BITS == 4) {
+      const int64_t gi = (2 * j) / group;
+      const float z = to_f32(zero[gi * C + i]), sc = to_f32(scale[gi * C + i]);
+      const float d0 = to_f32(from_f32<T>((float)(b & 0xF) - z));
+      const float d1 = to_f32(from_f32<T>((float)((b >> 4) & 0xF) - z));
+      out[(2 * j) * C + i] = from_f32<T>(d0 * sc);
+      out[(2 * j + 1) * C + i] = from_f32<T>(d1 * sc);
+    } else {
+      const int64_t gi = j / group;
+      const float z = to_f32(zero[gi * C + i]), sc = to_f32(scale[gi * C + i]);
+      out[idx] = from_f32<T>(to_f32(from_f32<T>((float)b - z)) * sc);
+    }
+  }
+}
+
 // ------------------------------------------------------------------ gathers
 template <typename T>
 __global__ __launch_bounds__(TPB) void gather_rows_kernel(const T *in, T *out, int64_t N,
@@ -464,6 +510,60 @@ int gptq_hip_gather_sym(void *stream, const void *in, void *out, int elem_bytes,
   return GPTQ_HIP_OK;
 }
 
+
+int gptq_hip_quantize_pack_grouped(void *stream, const void *Q, int q_dtype, int64_t K, int64_t N, const float *scale,
+                                   const float *zero, int64_t group_size, int bits, uint8_t *packed) {
+  if ((bits != 4 && bits != 8) || K < 0 || N < 0 || group_size <= 0 || group_size % 2 != 0 || K % group_size != 0)
+    return GPTQ_HIP_EINVAL;
+  const int64_t total = (bits == 4 ? K / 2 : K) * N;
+  if (total == 0) return GPTQ_HIP_OK;
+  if (!Q || !scale || !zero || !packed) return GPTQ_HIP_EINVAL;
+  hipStream_t st = as_stream(stream);
+  const dim3 grid(grid_for(total)), block(TPB);
+#define GPTQ_QPG(T)                                                                                                  \
+  if (bits == 4)                                                                                                     \
+    hipLaunchKernelGGL((quantize_pack_grouped_kernel<T, 4>), grid, block, 0, st, (const T *)Q, K, N, scale, zero,   \
+                       group_size, packed);                                                                          \
+  else                                                                                                               \
+    hipLaunchKernelGGL((quantize_pack_grouped_kernel<T, 8>), grid, block, 0, st, (const T *)Q, K, N, scale, zero,   \
+                       group_size, packed)
+  switch (q_dtype) {
+    case GPTQ_HIP_F32: GPTQ_QPG(float); break;
+    case GPTQ_HIP_F16: GPTQ_QPG(__half); break;
+    case GPTQ_HIP_BF16: GPTQ_QPG(__hip_bfloat16); break;
+    default: return GPTQ_HIP_EDTYPE;
+  }
+#undef GPTQ_QPG
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
+
+int gptq_hip_dequant_grouped(void *stream, const uint8_t *packed, int64_t R, int64_t C, const void *zero,
+                             const void *scale, int zs_dtype, int64_t group_size, int bits, void *out) {
+  const int64_t K = bits == 4 ? 2 * R : R;
+  if ((bits != 4 && bits != 8) || R < 0 || C < 0 || group_size <= 0 || group_size % 2 != 0 || K % group_size != 0)
+    return GPTQ_HIP_EINVAL;
+  if (R * C == 0) return GPTQ_HIP_OK;
+  if (!packed || !zero || !scale || !out) return GPTQ_HIP_EINVAL;
+  hipStream_t st = as_stream(stream);
+  const dim3 grid(grid_for(R * C)), block(TPB);
+#define GPTQ_DQG(T)                                                                                                \
+  if (bits == 4)                                                                                                   \
+    hipLaunchKernelGGL((dequant_grouped_kernel<T, 4>), grid, block, 0, st, packed, R, C, (const T *)zero,         \
+                       (const T *)scale, group_size, (T *)out);                                                    \
+  else                                                                                                             \
+    hipLaunchKernelGGL((dequant_grouped_kernel<T, 8>), grid, block, 0, st, packed, R, C, (const T *)zero,         \
+                       (const T *)scale, group_size, (T *)out)
+  switch (zs_dtype) {
+    case GPTQ_HIP_F32: GPTQ_DQG(float); break;
+    case GPTQ_HIP_F16: GPTQ_DQG(__half); break;
+    case GPTQ_HIP_BF16: GPTQ_DQG(__hip_bfloat16); break;
+    default: return GPTQ_HIP_EDTYPE;
+  }
+#undef GPTQ_DQG
+  GPTQ_CHECK_LAUNCH();
+  return GPTQ_HIP_OK;
+}
 
 int gptq_hip_fill_zero(void *stream, void *ptr, size_t bytes) {
   if (bytes == 0) return GPTQ_HIP_OK;

@@ -16,12 +16,26 @@ constexpr int TPB = 256;
 template <typename TX, typename TZ, int BITS>
 __global__ __launch_bounds__(TPB) void qmm_fwd_simple(const TX *x, int64_t M, const uint8_t *pk,
                                                       int64_t R, int64_t C, const TZ *zero,
-                                                      const TZ *scale, TX *out) {
+                                                      const TZ *scale, TX *out, int64_t group) {
   const int64_t n = (int64_t)blockIdx.x * TPB + threadIdx.x;
   const int64_t m = blockIdx.y;
   if (n >= C) return;
   const TX *xr = x + m * (BITS == 4 ? 2 * R : R);
   float acc = 0.f, xs = 0.f;
+  if (group > 0) {
+    // zero / scale [K / group, C]: applied term by term
+    for (int64_t j = 0; j < R; ++j) {
+      const uint8_t b = pk[j * C + n];
+      const int64_t gi = (BITS == 4 ? 2 * j : j) / group;
+      const float z = to_f32(zero[gi * C + n]), sc = to_f32(scale[gi * C + n]);
+      if (BITS == 4)
+        acc += to_f32(xr[2 * j]) * (((float)(b & 0xF) - z) * sc) + to_f32(xr[2 * j + 1]) * (((float)(b >> 4) - z) * sc);
+      else
+        acc += to_f32(xr[j]) * (((float)b - z) * sc);
+    }
+    out[m * C + n] = from_f32<TX>(__half2float(__float2half_rn(acc)));
+    return;
+  }
   for (int64_t j = 0; j < R; ++j) {
     const uint8_t b = pk[j * C + n];
     if (BITS == 4) {
@@ -41,14 +55,17 @@ __global__ __launch_bounds__(TPB) void qmm_fwd_simple(const TX *x, int64_t M, co
 // transposed: out[m, 2r+p] = sum_c x[m,c] * (nibble_p(pk[r,c]) - zero[c]) * scale[c]
 template <typename TX, typename TZ, int BITS>
 __global__ __launch_bounds__(TPB) void qmm_bwd_simple(const TX *x, int64_t M, const uint8_t *pk,
-                                                      int64_t R, int64_t C, const TZ *zero,
-                                                      const TZ *scale, TX *out) {
+                                                      int64_t R, int64_t C, const TZ *zero0,
+                                                      const TZ *scale0, TX *out, int64_t group) {
   // one wavefront per (m, r): lanes stride over c, then reduce
   const int lane = threadIdx.x & 63;
   const int64_t r = (int64_t)blockIdx.x * (TPB / 64) + (threadIdx.x >> 6);
   const int64_t m = blockIdx.y;
   if (r >= R) return;
   const TX *xr = x + m * C;
+  // grouped parameters: the row's group (both nibbles of a packed row lie in one group: group is even)
+  const int64_t prow = group > 0 ? ((BITS == 4 ? 2 * r : r) / group) * C : 0;
+  const TZ *zero = zero0 + prow, *scale = scale0 + prow;
   float a0 = 0.f, a1 = 0.f;
   for (int64_t c = lane; c < C; c += 64) {
     const uint8_t b = pk[r * C + c];
@@ -1620,7 +1637,7 @@ bool fwd_fast_ok(int x_dtype, int64_t M, int64_t R, int64_t C, const void *x, co
 
 template <typename TX, typename TZ, int BITS>
 int launch_simple(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
-                  const void *zero, const void *scale, int transpose_b, void *out) {
+                  const void *zero, const void *scale, int transpose_b, void *out, int64_t group) {
   const int64_t kin = transpose_b ? C : (BITS == 4 ? 2 * R : R), nout = transpose_b ? (BITS == 4 ? 2 * R : R) : C;
   // the rows are the grid's y dimension: 65535 of them per launch
   for (int64_t r0 = 0; r0 < M; r0 += 65535) {
@@ -1629,11 +1646,11 @@ int launch_simple(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, i
     TX *os = (TX *)out + r0 * nout;
     if (!transpose_b) {
       hipLaunchKernelGGL((qmm_fwd_simple<TX, TZ, BITS>), dim3((unsigned)ceil_div64(C, TPB), (unsigned)rows),
-                         dim3(TPB), 0, st, xs, rows, pk, R, C, (const TZ *)zero, (const TZ *)scale, os);
+                         dim3(TPB), 0, st, xs, rows, pk, R, C, (const TZ *)zero, (const TZ *)scale, os, group);
     } else {
       hipLaunchKernelGGL((qmm_bwd_simple<TX, TZ, BITS>),
                          dim3((unsigned)ceil_div64(R, TPB / 64), (unsigned)rows), dim3(TPB), 0, st, xs, rows, pk,
-                         R, C, (const TZ *)zero, (const TZ *)scale, os);
+                         R, C, (const TZ *)zero, (const TZ *)scale, os, group);
     }
     GPTQ_CHECK_LAUNCH();
   }
@@ -1642,14 +1659,14 @@ int launch_simple(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, i
 
 template <typename TX, int BITS>
 int dispatch_z(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
-               const void *zero, const void *scale, int zs_dtype, int transpose_b, void *out) {
+               const void *zero, const void *scale, int zs_dtype, int transpose_b, void *out, int64_t group) {
   switch (zs_dtype) {
     case GPTQ_HIP_F32:
-      return launch_simple<TX, float, BITS>(st, x, M, pk, R, C, zero, scale, transpose_b, out);
+      return launch_simple<TX, float, BITS>(st, x, M, pk, R, C, zero, scale, transpose_b, out, group);
     case GPTQ_HIP_F16:
-      return launch_simple<TX, __half, BITS>(st, x, M, pk, R, C, zero, scale, transpose_b, out);
+      return launch_simple<TX, __half, BITS>(st, x, M, pk, R, C, zero, scale, transpose_b, out, group);
     case GPTQ_HIP_BF16:
-      return launch_simple<TX, __hip_bfloat16, BITS>(st, x, M, pk, R, C, zero, scale, transpose_b, out);
+      return launch_simple<TX, __hip_bfloat16, BITS>(st, x, M, pk, R, C, zero, scale, transpose_b, out, group);
     default:
       return GPTQ_HIP_EDTYPE;
   }
@@ -1657,12 +1674,12 @@ int dispatch_z(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int6
 
 template <int BITS>
 int dispatch_simple(hipStream_t st, const void *x, int x_dtype, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
-                    const void *zero, const void *scale, int zs_dtype, int transpose_b, void *out) {
+                    const void *zero, const void *scale, int zs_dtype, int transpose_b, void *out, int64_t group) {
   switch (x_dtype) {
-    case GPTQ_HIP_F32: return dispatch_z<float, BITS>(st, x, M, pk, R, C, zero, scale, zs_dtype, transpose_b, out);
-    case GPTQ_HIP_F16: return dispatch_z<__half, BITS>(st, x, M, pk, R, C, zero, scale, zs_dtype, transpose_b, out);
+    case GPTQ_HIP_F32: return dispatch_z<float, BITS>(st, x, M, pk, R, C, zero, scale, zs_dtype, transpose_b, out, group);
+    case GPTQ_HIP_F16: return dispatch_z<__half, BITS>(st, x, M, pk, R, C, zero, scale, zs_dtype, transpose_b, out, group);
     case GPTQ_HIP_BF16:
-      return dispatch_z<__hip_bfloat16, BITS>(st, x, M, pk, R, C, zero, scale, zs_dtype, transpose_b, out);
+      return dispatch_z<__hip_bfloat16, BITS>(st, x, M, pk, R, C, zero, scale, zs_dtype, transpose_b, out, group);
     default: return GPTQ_HIP_EDTYPE;
   }
 }
@@ -1773,10 +1790,16 @@ bool aligned16(const void *a, const void *b) {
   return ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) == 0;
 }
 
+// group_size = 0: zero / scale [C]; group_size > 0: zero / scale [K / group_size, C] (register-operand kernels,
+// whose k-steps of 32 and tiles of 128 output columns must not straddle a group, or the plain kernels)
 int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed, int64_t R, int64_t C,
-                 const void *zero, const void *scale, int zs_dtype, int bits, int transpose_b, void *out, void *ws,
-                 size_t ws_bytes) {
+                 const void *zero, const void *scale, int zs_dtype, int bits, int64_t group_size, int transpose_b,
+                 void *out, void *ws, size_t ws_bytes) {
   if (M < 0 || R <= 0 || C <= 0 || (bits != 4 && bits != 8)) return GPTQ_HIP_EINVAL;
+  if (group_size < 0 || group_size % 2 != 0 || (group_size > 0 && (bits == 4 ? 2 * R : R) % group_size != 0) ||
+      group_size > (1LL << 30))
+    return GPTQ_HIP_EINVAL;
+  const bool reg_groups_ok = group_size == 0 || group_size % (transpose_b ? 128 : 32) == 0;
   if (M == 0) return GPTQ_HIP_OK;
   if (!x || !packed || !zero || !scale || !out) return GPTQ_HIP_EINVAL;
   hipStream_t st = as_stream(stream);
@@ -1784,7 +1807,7 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
     // through the 16-bit kernels, if the shape suits them and the caller sized the workspace for
     // it (gptq_hip_qmatmul_workspace_bytes_x); else the plain fp32 kernels below
     const F32Plan fp = f32_plan(M, R, C, transpose_b, bits);
-    if (fp.use && ws && ws_bytes >= fp.total_bytes && (reinterpret_cast<uintptr_t>(ws) & 15) == 0) {
+    if (fp.use && reg_groups_ok && ws && ws_bytes >= fp.total_bytes && (reinterpret_cast<uintptr_t>(ws) & 15) == 0) {
       char *base = reinterpret_cast<char *>(ws);
       __half *x16 = reinterpret_cast<__half *>(base + fp.x16_off);
       __half *o16 = reinterpret_cast<__half *>(base + fp.o16_off);
@@ -1797,7 +1820,7 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
                            reinterpret_cast<const float *>(x) + r0 * kin, kin, x16, rowexp);
         GPTQ_CHECK_LAUNCH();
         const int rc = qmatmul_impl(stream, x16, GPTQ_HIP_F16, mm, packed, R, C, zero, scale, zs_dtype, bits,
-                                    transpose_b, o16, ws, fp.inner);
+                                    group_size, transpose_b, o16, ws, fp.inner);
         if (rc) return rc;
         unsigned gx = (unsigned)ceil_div64(nout, 1024);
         if (gx > 64) gx = 64;
@@ -1807,18 +1830,19 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
       }
       return GPTQ_HIP_OK;
     }
-    return bits == 4 ? dispatch_simple<4>(st, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out)
-                     : dispatch_simple<8>(st, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out);
+    return bits == 4
+               ? dispatch_simple<4>(st, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out, group_size)
+               : dispatch_simple<8>(st, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out, group_size);
   }
   if (x_dtype != GPTQ_HIP_F16 && x_dtype != GPTQ_HIP_BF16) return GPTQ_HIP_EDTYPE;
   if (zs_dtype != GPTQ_HIP_F32 && zs_dtype != GPTQ_HIP_F16 && zs_dtype != GPTQ_HIP_BF16) return GPTQ_HIP_EDTYPE;
   const bool al = aligned16(x, out) && (reinterpret_cast<uintptr_t>(packed) & 7) == 0;
-  const RegPlan rp = transpose_b ? RegPlan{} : reg_fwd_plan(M, R, C, bits, al);
+  const RegPlan rp = (transpose_b || !reg_groups_ok) ? RegPlan{} : reg_fwd_plan(M, R, C, bits, al);
   auto run_reg_fwd = [&]() -> int {
     if (rp.total_bytes && (!ws || ws_bytes < rp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
-    return reg_fwd_launch(st, rp, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, out, ws);
+    return reg_fwd_launch(st, rp, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, out, ws, (int)group_size);
   };
-  if (bits == 4 && !transpose_b) {
+  if (bits == 4 && !transpose_b && group_size == 0) {
     // few rows against a whole matrix (16 < M <= 256): the register-operand kernel, unless its tiles are too
     // few to fill the chip even when split (the tiled kernel below splits finer)
     if (rp.use && !rp.ragged && M > 16 && M <= 256 && rp.tiles * rp.S >= 64) return run_reg_fwd();
@@ -1861,7 +1885,7 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
       }
     }
   }
-  if (bits == 4 && transpose_b && bwd_fast_ok(x_dtype, M, R, C, x, packed, zero, scale)) {
+  if (bits == 4 && transpose_b && group_size == 0 && bwd_fast_ok(x_dtype, M, R, C, x, packed, zero, scale)) {
     switch (zs_dtype) {
       case GPTQ_HIP_F32: return launch_bwd_gemm<float>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
       case GPTQ_HIP_F16: return launch_bwd_gemm<__half>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
@@ -1870,15 +1894,16 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
   }
   // 8-bit codes, and 4-bit shapes whose rows are not multiples of 16 channels or that are not aligned
   if (!transpose_b && rp.use) return run_reg_fwd();
-  if (transpose_b) {
+  if (transpose_b && reg_groups_ok) {
     const RegBwdPlan bp = reg_bwd_plan(M, R, C, bits, al);
     if (bp.use) {
       if (bp.total_bytes && (!ws || ws_bytes < bp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
-      return reg_bwd_launch(st, bp, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, out, ws);
+      return reg_bwd_launch(st, bp, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, out, ws, (int)group_size);
     }
   }
-  return bits == 4 ? dispatch_simple<4>(st, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out)
-                   : dispatch_simple<8>(st, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out);
+  return bits == 4
+             ? dispatch_simple<4>(st, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out, group_size)
+             : dispatch_simple<8>(st, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out, group_size);
 }
 
 }  // namespace
@@ -1906,15 +1931,23 @@ size_t gptq_hip_qmatmul_bits_workspace_bytes(int64_t M, int64_t R, int64_t C, in
 int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
                      int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype,
                      int transpose_b, void *out, void *ws, size_t ws_bytes) {
-  return qmatmul_impl(stream, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, 4, transpose_b, out, ws,
+  return qmatmul_impl(stream, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, 4, 0, transpose_b, out, ws,
                       ws_bytes);
 }
 
 int gptq_hip_qmatmul_bits(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
                           int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, int bits,
                           int transpose_b, void *out, void *ws, size_t ws_bytes) {
-  return qmatmul_impl(stream, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, bits, transpose_b, out, ws,
+  return qmatmul_impl(stream, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, bits, 0, transpose_b, out, ws,
                       ws_bytes);
+}
+
+int gptq_hip_qmatmul_grouped(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
+                             int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype,
+                             int64_t group_size, int bits, int transpose_b, void *out, void *ws, size_t ws_bytes) {
+  if (group_size <= 0) return GPTQ_HIP_EINVAL;
+  return qmatmul_impl(stream, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, bits, group_size, transpose_b, out,
+                      ws, ws_bytes);
 }
 
 }  // extern "C"

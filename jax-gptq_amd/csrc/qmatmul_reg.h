@@ -16,9 +16,11 @@ struct RegPlan {
 };
 
 RegPlan reg_fwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned);
-// x / out element type x_dtype (F16 or BF16), zero / scale element type zs_dtype (F32, F16, BF16)
+// x / out element type x_dtype (F16 or BF16), zero / scale element type zs_dtype (F32, F16, BF16).
+// group_size = 0: zero / scale [C]; group_size > 0 (a multiple of 32): zero / scale [K / group_size, C].
 int reg_fwd_launch(hipStream_t st, const RegPlan &p, const void *x, int x_dtype, int64_t M, const uint8_t *pk,
-                   int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws);
+                   int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws,
+                   int group_size);
 
 // Transposed product out[M, K] = x[M, C] @ dequant(packed[R, C])^T.
 struct RegBwdPlan {
@@ -30,7 +32,9 @@ struct RegBwdPlan {
   size_t part_bytes, total_bytes;
 };
 RegBwdPlan reg_bwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned);
+// group_size > 0: a multiple of 128 (the 128 output columns of a tile share one group)
 int reg_bwd_launch(hipStream_t st, const RegBwdPlan &p, const void *x, int x_dtype, int64_t M, const uint8_t *pk,
-                   int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws);
+                   int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws,
+                   int group_size);
 
 }  // namespace qmm

@@ -28,12 +28,15 @@ using namespace qmm;
 
 constexpr int RG_BN = 128;                       // channels per output tile
 
-template <int BITS, int RB, int RING, bool RAGGED, typename TX>
+// GROUPED (an extension: the reference has one scale / zero per channel): zero / scale are [K / group, C] tables;
+// the parameters of a k-step's group travel with its loads, and B = (code - zero) scale is formed in fp16
+// (converted for bf16 activations), so the accumulators need no offset or scale afterwards.
+template <int BITS, int RB, int RING, bool RAGGED, typename TX, bool GROUPED>
 __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, int K, const uint8_t *pk, int R,
                                                           int C, const void *zero, const void *scale,
                                                           int zs_dtype, TX *out, float *part, int32_t *counters,
-                                                          int S, int steps_per_split) {
-  constexpr bool BF = Act<TX>::BF;
+                                                          int S, int steps_per_split, int group_size) {
+  constexpr bool BF = Act<TX>::BF && !GROUPED;      // grouped: the fp16 form of the dequantisation for both types
   constexpr int SCHED = RB == 4 ? 4 : 0;         // vector instructions between two MFMAs of the main loop (0: compiler's order)
   constexpr int NL = BITS == 4 ? 4 : 8;          // packed rows per lane and k-step
   constexpr int PR = 4 * NL;                     // packed rows per k-step
@@ -64,6 +67,7 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
 
   uint2 wr[RING][NL];
   uint4 aq[RING][RB];
+  uint32_t zraw[GROUPED ? RING : 1][8], sraw[GROUPED ? RING : 1][8];
   auto load_step = [&](int slot, int s) __attribute__((always_inline)) {
     // (steps past this workgroup's range re-read its own last k-step, a cache hit, not the next split's rows)
     const int t = min(t_begin + 4 * s + wk, max(t_end - 1, 0));
@@ -73,6 +77,11 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
     const int koff = min(32 * t + 8 * g, K - 8);                      // K >= 8: a chunk inside the row
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) aq[slot][rb] = rg_load16<RAGGED>(x + xrow[rb] + koff);
+    if constexpr (GROUPED) {
+      const int64_t row_base = (int64_t)((32 * t) / group_size) * C;
+      rg_params8_raw(zero, zs_dtype, row_base, col, C, zraw[slot]);
+      rg_params8_raw(scale, zs_dtype, row_base, col, C, sraw[slot]);
+    }
   };
 
   // the first k-steps' loads go out before anything that has to wait for memory
@@ -82,7 +91,7 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
   // ---- per-channel constants of the dequantisation (the integer part of the zero point)
   uint32_t zc[8];
   float zi8[(BF && BITS == 8) ? 8 : 1];
-  {
+  if constexpr (!GROUPED) {
     float z8[8];
     rg_params8(zero, zs_dtype, col, C, z8);
 #pragma unroll
@@ -124,6 +133,34 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
     uint2 w[NL];
 #pragma unroll
     for (int i = 0; i < NL; ++i) w[i] = RAGGED ? rg_shr_bytes(wr[slot][i], wshift) : wr[slot][i];
+    uint32_t s2[GROUPED ? 8 : 1], nzf2[GROUPED ? 8 : 1];
+    if constexpr (GROUPED) {
+#pragma unroll
+      for (int t8 = 0; t8 < 8; ++t8) {
+        const float z = rg_raw_to_f32(zraw[slot][t8], zs_dtype), sc = rg_raw_to_f32(sraw[slot][t8], zs_dtype);
+        const float zi = fminf(fmaxf(rintf(z), -512.f), 512.f);
+        const _Float16 hs = (_Float16)sc, hz = (_Float16)(-(z - zi) * sc);
+        s2[t8] = __builtin_bit_cast(uint32_t, half2_t{hs, hs});
+        nzf2[t8] = __builtin_bit_cast(uint32_t, half2_t{hz, hz});
+        zc[t8] = BITS == 4
+                     ? __builtin_bit_cast(uint32_t, half2_t{(_Float16)(-(1024.f + zi)), (_Float16)(-(64.f + zi))})
+                     : __builtin_bit_cast(uint32_t, half2_t{(_Float16)(-(1024.f + zi)), (_Float16)(-(1024.f + zi))});
+      }
+    }
+    // grouped: (code - zi) * scale - (zero - zi) * scale in fp16, as bf16 for bf16 activations
+    auto finish_b = [&](half2_t d, int t8) __attribute__((always_inline)) -> uint32_t {
+      if constexpr (GROUPED) {
+        const half2_t e = d * __builtin_bit_cast(half2_t, s2[t8]) + __builtin_bit_cast(half2_t, nzf2[t8]);
+        if constexpr (Act<TX>::BF) {
+          typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
+          typedef float f2_t __attribute__((ext_vector_type(2)));
+          return __builtin_bit_cast(uint32_t, __builtin_convertvector(f2_t{(float)e[0], (float)e[1]}, bf2_t));
+        }
+        return __builtin_bit_cast(uint32_t, e);
+      } else {
+        return __builtin_bit_cast(uint32_t, d);
+      }
+    };
 #pragma unroll
     for (int t8 = 0; t8 < 8; ++t8) {
       const uint32_t tb = (uint32_t)(t8 & 3);
@@ -139,7 +176,7 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
           } else {
             const uint32_t v = (pb & mask) | cexp;                       // {1024 + lo, 1024 + 16 hi}
             const half2_t d = __builtin_bit_cast(half2_t, v) * unscale + __builtin_bit_cast(half2_t, zc[t8]);
-            r4[i] = __builtin_bit_cast(uint32_t, d);
+            r4[i] = finish_b(d, t8);
           }
         }
       } else {
@@ -155,7 +192,7 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
           } else {
             const uint32_t pb = __builtin_amdgcn_perm(wb, wa, 0x0c000c00u | ((4u + tb) << 16) | tb);
             const half2_t d = __builtin_bit_cast(half2_t, pb | cexp) + __builtin_bit_cast(half2_t, zc[t8]);
-            r4[i] = __builtin_bit_cast(uint32_t, d);
+            r4[i] = finish_b(d, t8);
           }
         }
       }
@@ -163,8 +200,10 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) acc[rb][t8] = Act<TX>::mma(a[rb], b, acc[rb][t8]);
     }
+    if constexpr (!GROUPED) {
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) acc[rb][8] = Act<TX>::mma(a[rb], ones, acc[rb][8]);
+      for (int rb = 0; rb < RB; ++rb) acc[rb][8] = Act<TX>::mma(a[rb], ones, acc[rb][8]);
+    }
   };
   const std::integral_constant<bool, false> plain{};
   const std::integral_constant<bool, true> tail{};
@@ -201,8 +240,10 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
 
   // scale and zero point of this lane's channels, in flight while the tiles are summed
   float sc[8], zf[8];
-  rg_params8(scale, zs_dtype, col, C, sc);
-  rg_params8(zero, zs_dtype, col, C, zf);
+  if constexpr (!GROUPED) {
+    rg_params8(scale, zs_dtype, col, C, sc);
+    rg_params8(zero, zs_dtype, col, C, zf);
+  }
   floatx4 sum[RG_NT];
   const int tile = ty * gridDim.x + tx;
   if (!rg_reduce<RB>(acc, sum, rg_lds, &s_flag, part, counters, tile, split, S)) return;
@@ -211,8 +252,14 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
   if (!col_ok) return;
   const int rb = wk;                             // rg_reduce returned true: wk < RB
 #pragma unroll
-  for (int t8 = 0; t8 < 8; ++t8)
-    zf[t8] = (BF && BITS == 4) ? 128.f + zf[t8] : zf[t8] - fminf(fmaxf(rintf(zf[t8]), -512.f), 512.f);
+  for (int t8 = 0; t8 < 8; ++t8) {
+    if (GROUPED) {
+      sc[t8] = 1.f;
+      zf[t8] = 0.f;
+    } else {
+      zf[t8] = (BF && BITS == 4) ? 128.f + zf[t8] : zf[t8] - fminf(fmaxf(rintf(zf[t8]), -512.f), 512.f);
+    }
+  }
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int m = m0 + 16 * rb + 4 * g + r;
@@ -232,11 +279,11 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
   }
 }
 
-template <int BITS, int RB, int RING, bool RAGGED, typename TX>
+template <int BITS, int RB, int RING, bool RAGGED, typename TX, bool GROUPED>
 int launch_inst(hipStream_t st, const RegPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
-                int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *wsp) {
+                int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *wsp, int group_size) {
   constexpr size_t lds = (size_t)4 * RB * RG_NT * RG_TILE_FLOATS * sizeof(float);
-  auto kern = qmm_fwd_reg_kernel<BITS, RB, RING, RAGGED, TX>;
+  auto kern = qmm_fwd_reg_kernel<BITS, RB, RING, RAGGED, TX, GROUPED>;
   if (lds > 64 * 1024 && !gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), (int)lds)) return GPTQ_HIP_ELAUNCH;
   const int64_t K = BITS == 4 ? 2 * R : R;
   int32_t *counters = reinterpret_cast<int32_t *>(wsp);
@@ -253,7 +300,7 @@ int launch_inst(hipStream_t st, const RegPlan &p, const void *x, int64_t M, cons
     const int64_t rows = M - r0 < rows_max ? M - r0 : rows_max;
     const dim3 grid((unsigned)tiles_x, (unsigned)ceil_div64(rows, 16 * RB), (unsigned)p.S);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (const TX *)x + r0 * K, (int)rows, (int)K, pk, (int)R,
-                       (int)C, zero, scale, zs_dtype, (TX *)out + r0 * C, part, counters, p.S, p.steps);
+                       (int)C, zero, scale, zs_dtype, (TX *)out + r0 * C, part, counters, p.S, p.steps, group_size);
     GPTQ_CHECK_LAUNCH();
   }
   return GPTQ_HIP_OK;
@@ -261,14 +308,26 @@ int launch_inst(hipStream_t st, const RegPlan &p, const void *x, int64_t M, cons
 
 template <int BITS, typename TX>
 int launch_bx(hipStream_t st, const RegPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
-              const void *zero, const void *scale, int zs_dtype, void *out, void *ws) {
+              const void *zero, const void *scale, int zs_dtype, void *out, void *ws, int group_size) {
+#define GPTQ_REG(RB, RING, RAGGED, GROUPED) \
+  return launch_inst<BITS, RB, RING, RAGGED, TX, GROUPED>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size)
+  if (group_size > 0) {
+    // the group's parameters ride in the ring: shorter rings
+    if (p.rb == 4) {
+      if (p.ragged) GPTQ_REG(4, 2, true, true);
+      GPTQ_REG(4, 2, false, true);
+    }
+    if (p.ragged) GPTQ_REG(1, 3, true, true);
+    GPTQ_REG(1, 3, false, true);
+  }
   // a ring of three k-steps for 64-row tiles (registers), of six for the 16-row tiles of the decode case
   if (p.rb == 4) {
-    if (p.ragged) return launch_inst<BITS, 4, 3, true, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
-    return launch_inst<BITS, 4, 3, false, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+    if (p.ragged) GPTQ_REG(4, 3, true, false);
+    GPTQ_REG(4, 3, false, false);
   }
-  if (p.ragged) return launch_inst<BITS, 1, 6, true, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
-  return launch_inst<BITS, 1, 6, false, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+  if (p.ragged) GPTQ_REG(1, 6, true, false);
+  GPTQ_REG(1, 6, false, false);
+#undef GPTQ_REG
 }
 
 }  // namespace
@@ -306,15 +365,17 @@ RegPlan reg_fwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned) {
 }
 
 int reg_fwd_launch(hipStream_t st, const RegPlan &p, const void *x, int x_dtype, int64_t M, const uint8_t *pk,
-                   int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws) {
+                   int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws,
+                   int group_size) {
+  if (group_size < 0 || group_size % 32 != 0) return GPTQ_HIP_EINVAL;
   if (zs_dtype != GPTQ_HIP_F32 && zs_dtype != GPTQ_HIP_F16 && zs_dtype != GPTQ_HIP_BF16) return GPTQ_HIP_EDTYPE;
   if (x_dtype == GPTQ_HIP_BF16) {
-    if (p.bits == 4) return launch_bx<4, __hip_bfloat16>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
-    return launch_bx<8, __hip_bfloat16>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+    if (p.bits == 4) return launch_bx<4, __hip_bfloat16>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
+    return launch_bx<8, __hip_bfloat16>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
   }
   if (x_dtype != GPTQ_HIP_F16) return GPTQ_HIP_EDTYPE;
-  if (p.bits == 4) return launch_bx<4, __half>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
-  return launch_bx<8, __half>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+  if (p.bits == 4) return launch_bx<4, __half>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
+  return launch_bx<8, __half>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
 }
 
 }  // namespace qmm

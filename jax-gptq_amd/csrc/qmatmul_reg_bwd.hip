@@ -34,7 +34,7 @@ template <int BITS, bool RAGGED, typename TX>
 __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, const uint8_t *pk, int R, int C,
                                                           const void *zero, const void *scale, int zs_dtype,
                                                           TX *out, float *part, int32_t *counters, int S,
-                                                          int steps_per_split) {
+                                                          int steps_per_split, int group_size) {
   constexpr bool BF = Act<TX>::BF;
   constexpr int RB = RGB_RB, RING = RGB_RING;
   constexpr int NG = BITS == 4 ? 4 : 8;          // groups of 16 packed rows: 8 MFMA tiles either way
@@ -77,7 +77,11 @@ __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, co
   };
   // the element type is switched on outside the loops, and a thread's loads of a round are independent:
   // four channels' zero and scale in flight per thread instead of one load at a time
-  auto fill = [&](auto *zp, auto *sp) __attribute__((always_inline)) {
+  // grouped parameters ([K / group, C] tables): the tile's 128 output columns lie in one group
+  const int64_t prow = group_size > 0 ? (int64_t)(((int64_t)j0 * (BITS == 4 ? 2 : 1)) / group_size) * C : 0;
+  auto fill = [&](auto *zp0, auto *sp0) __attribute__((always_inline)) {
+    auto *zp = zp0 + prow;
+    auto *sp = sp0 + prow;
     for (int i0 = tid; i0 < nch; i0 += 4 * 256) {
       float zv[4], sv[4];
 #pragma unroll
@@ -289,7 +293,7 @@ __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, co
 
 template <int BITS, bool RAGGED, typename TX>
 int launch_inst(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
-                int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *wsp) {
+                int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *wsp, int group_size) {
   constexpr int NJ = BITS == 4 ? 64 : 128;
   auto kern = qmm_bwd_reg_kernel<BITS, RAGGED, TX>;
   if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), RGB_LDS_BYTES)) return GPTQ_HIP_ELAUNCH;
@@ -307,7 +311,7 @@ int launch_inst(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, c
     const int64_t rows = M - r0 < rows_max ? M - r0 : rows_max;
     const dim3 grid((unsigned)tiles_x, (unsigned)ceil_div64(rows, 64), (unsigned)p.S);
     hipLaunchKernelGGL(kern, grid, dim3(256), RGB_LDS_BYTES, st, (const TX *)x + r0 * C, (int)rows, pk, (int)R,
-                       (int)C, zero, scale, zs_dtype, (TX *)out + r0 * KO, part, counters, p.S, p.steps);
+                       (int)C, zero, scale, zs_dtype, (TX *)out + r0 * KO, part, counters, p.S, p.steps, group_size);
     GPTQ_CHECK_LAUNCH();
   }
   return GPTQ_HIP_OK;
@@ -315,9 +319,9 @@ int launch_inst(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, c
 
 template <int BITS, typename TX>
 int launch_bx(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
-              int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws) {
-  if (p.ragged) return launch_inst<BITS, true, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
-  return launch_inst<BITS, false, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+              int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws, int group_size) {
+  if (p.ragged) return launch_inst<BITS, true, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
+  return launch_inst<BITS, false, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
 }
 
 }  // namespace
@@ -352,15 +356,17 @@ RegBwdPlan reg_bwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned)
 }
 
 int reg_bwd_launch(hipStream_t st, const RegBwdPlan &p, const void *x, int x_dtype, int64_t M, const uint8_t *pk,
-                   int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws) {
+                   int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws,
+                   int group_size) {
+  if (group_size < 0 || group_size % 128 != 0) return GPTQ_HIP_EINVAL;
   if (zs_dtype != GPTQ_HIP_F32 && zs_dtype != GPTQ_HIP_F16 && zs_dtype != GPTQ_HIP_BF16) return GPTQ_HIP_EDTYPE;
   if (x_dtype == GPTQ_HIP_BF16) {
-    if (p.bits == 4) return launch_bx<4, __hip_bfloat16>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
-    return launch_bx<8, __hip_bfloat16>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+    if (p.bits == 4) return launch_bx<4, __hip_bfloat16>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
+    return launch_bx<8, __hip_bfloat16>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
   }
   if (x_dtype != GPTQ_HIP_F16) return GPTQ_HIP_EDTYPE;
-  if (p.bits == 4) return launch_bx<4, __half>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
-  return launch_bx<8, __half>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+  if (p.bits == 4) return launch_bx<4, __half>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
+  return launch_bx<8, __half>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
 }
 
 }  // namespace qmm

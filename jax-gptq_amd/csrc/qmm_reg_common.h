@@ -66,6 +66,29 @@ __device__ __forceinline__ void rg_params8(const void *p, int dtype, int first, 
   }
 }
 
+// The same eight elements as raw bits (16-bit types zero-extended), for values that are fetched one k-step ahead
+// and converted when they are used: the conversion is what would make the wavefront wait for the loads.
+__device__ __forceinline__ void rg_params8_raw(const void *p, int dtype, int64_t row_base, int first, int n,
+                                               uint32_t (&out)[8]) {
+  int idx[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) idx[i] = min(first + i, n - 1);
+  if (dtype == GPTQ_HIP_F32) {
+    const uint32_t *q = reinterpret_cast<const uint32_t *>(p) + row_base;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = q[idx[i]];
+  } else {
+    const uint16_t *q = reinterpret_cast<const uint16_t *>(p) + row_base;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = q[idx[i]];
+  }
+}
+__device__ __forceinline__ float rg_raw_to_f32(uint32_t raw, int dtype) {
+  if (dtype == GPTQ_HIP_F32) return __builtin_bit_cast(float, raw);
+  if (dtype == GPTQ_HIP_F16) return (float)__builtin_bit_cast(half2_t, raw)[0];
+  return __builtin_bit_cast(float, raw << 16);
+}
+
 // Activations of a ragged last k-step: the lane wants the 8 elements [k0, k0 + 8) of its row, of which
 // only those below K exist; `a` was loaded from [kl, kl + 8) with kl = min(k0, K - 8) <= k0.  Returns the
 // wanted elements with zeros past K (element = 16 bits).

@@ -215,28 +215,39 @@ int gptq_hip_process_block(void *stream, const float *Wblock, int64_t N, const f
                        Qblock, q_dtype, codes_block, errors);
 }
 
-int gptq_hip_solve(void *stream, float *W, int64_t K, int64_t N, const float *L,
-                   const float *scale, const float *zero, int maxq, int block_size, void *Q,
-                   int q_dtype, uint8_t *codes, void *ws, size_t ws_bytes) {
-  if (!W || !L || !scale || !zero || K <= 0 || N <= 0 || K > 2147483647LL || N > 2147483647LL)
-    return GPTQ_HIP_EINVAL;
-  if (!block_size_ok(block_size) || K % block_size != 0 || maxq < 1 || maxq > 255)
-    return GPTQ_HIP_EINVAL;
-  if (q_dtype != GPTQ_HIP_F32 && q_dtype != GPTQ_HIP_F16 && q_dtype != GPTQ_HIP_BF16)
-    return GPTQ_HIP_EDTYPE;
-  if (!ws || ws_bytes < gptq_hip_solve_workspace_bytes(K, N, block_size)) return GPTQ_HIP_EWORKSPACE;
-  hipStream_t st = as_stream(stream);
-  float *Err = reinterpret_cast<float *>(ws);
+}  // extern "C"
+
+namespace {
+
+// The column loop.  group_size = 0: one scale / zero per channel for the whole column (the reference).
+// group_size > 0: the parameters of rows [r0, r0 + group_size) are taken, when the loop reaches r0, from the
+// column minima and maxima of those rows as they then stand (all corrections of the rows above applied), and
+// written to row r0 / group_size of scale_g / zero_g [K / group_size, N].
+int solve_impl(hipStream_t st, float *W, int64_t K, int64_t N, const float *L, const float *scale, const float *zero,
+               float *scale_g, float *zero_g, int group_size, int bits, int maxq, int block_size, void *Q,
+               int q_dtype, uint8_t *codes, float *Err, void *cp_ws, size_t cp_ws_bytes) {
   const size_t qsz = dtype_size(q_dtype);
   const int64_t grp = group_rows(block_size);
   for (int64_t gs = 0; gs < K; gs += grp) {
     const int64_t ge = gs + grp < K ? gs + grp : K;
     for (int64_t start = gs; start < ge; start += block_size) {
+      const float *sc = scale, *zr = zero;
+      if (group_size > 0) {
+        const int64_t gi = start / group_size;
+        if (start % group_size == 0) {
+          // the group's rows lie inside the current update group (group_size divides its height), so they are current
+          const int rc = gptq_hip_col_params(st, W + start * N, GPTQ_HIP_F32, group_size, N, N, bits,
+                                             scale_g + gi * N, zero_g + gi * N, cp_ws, cp_ws_bytes);
+          if (rc) return rc;
+        }
+        sc = scale_g + gi * N;
+        zr = zero_g + gi * N;
+      }
       void *Qb = Q ? (void *)((char *)Q + (size_t)start * N * qsz) : nullptr;
       uint8_t *cb = codes ? codes + start * N : nullptr;
       float *Eb = Err + (start - gs) * N;
-      int rc = process_block(st, W + start * N, N, L + start * K + start, K, block_size, scale, zero,
-                             maxq, Qb, q_dtype, cb, Eb);
+      int rc = process_block(st, W + start * N, N, L + start * K + start, K, block_size, sc, zr, maxq, Qb,
+                             q_dtype, cb, Eb);
       if (rc) return rc;
       const int64_t end = start + block_size;
       if (end < ge) {
@@ -253,6 +264,49 @@ int gptq_hip_solve(void *stream, float *W, int64_t K, int64_t N, const float *L,
     }
   }
   return GPTQ_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int gptq_hip_solve(void *stream, float *W, int64_t K, int64_t N, const float *L,
+                   const float *scale, const float *zero, int maxq, int block_size, void *Q,
+                   int q_dtype, uint8_t *codes, void *ws, size_t ws_bytes) {
+  if (!W || !L || !scale || !zero || K <= 0 || N <= 0 || K > 2147483647LL || N > 2147483647LL)
+    return GPTQ_HIP_EINVAL;
+  if (!block_size_ok(block_size) || K % block_size != 0 || maxq < 1 || maxq > 255)
+    return GPTQ_HIP_EINVAL;
+  if (q_dtype != GPTQ_HIP_F32 && q_dtype != GPTQ_HIP_F16 && q_dtype != GPTQ_HIP_BF16)
+    return GPTQ_HIP_EDTYPE;
+  if (!ws || ws_bytes < gptq_hip_solve_workspace_bytes(K, N, block_size)) return GPTQ_HIP_EWORKSPACE;
+  return solve_impl(as_stream(stream), W, K, N, L, scale, zero, nullptr, nullptr, 0, 0, maxq, block_size, Q, q_dtype,
+                    codes, reinterpret_cast<float *>(ws), nullptr, 0);
+}
+
+size_t gptq_hip_solve_grouped_workspace_bytes(int64_t K, int64_t N, int block_size, int group_size) {
+  if (K <= 0 || N <= 0 || !block_size_ok(block_size) || group_size <= 0) return 0;
+  const size_t a = (gptq_hip_solve_workspace_bytes(K, N, block_size) + 255) & ~(size_t)255;
+  return a + gptq_hip_col_params_workspace_bytes(group_size, N);
+}
+
+int gptq_hip_solve_grouped(void *stream, float *W, int64_t K, int64_t N, const float *L, int group_size, int bits,
+                           int block_size, void *Q, int q_dtype, uint8_t *codes, float *scale_g, float *zero_g,
+                           void *ws, size_t ws_bytes) {
+  if (!W || !L || !scale_g || !zero_g || K <= 0 || N <= 0 || K > 2147483647LL || N > 2147483647LL)
+    return GPTQ_HIP_EINVAL;
+  if (!block_size_ok(block_size) || K % block_size != 0 || bits < 1 || bits > 8) return GPTQ_HIP_EINVAL;
+  // a group is a whole number of blocks, lies inside one update group of the loop, and groups tile K
+  if (group_size <= 0 || group_size % block_size != 0 || group_rows(block_size) % group_size != 0 ||
+      K % group_size != 0)
+    return GPTQ_HIP_EINVAL;
+  if (q_dtype != GPTQ_HIP_F32 && q_dtype != GPTQ_HIP_F16 && q_dtype != GPTQ_HIP_BF16)
+    return GPTQ_HIP_EDTYPE;
+  if (!ws || ws_bytes < gptq_hip_solve_grouped_workspace_bytes(K, N, block_size, group_size)) return GPTQ_HIP_EWORKSPACE;
+  const size_t a = (gptq_hip_solve_workspace_bytes(K, N, block_size) + 255) & ~(size_t)255;
+  return solve_impl(as_stream(stream), W, K, N, L, nullptr, nullptr, scale_g, zero_g, group_size, bits, (1 << bits) - 1,
+                    block_size, Q, q_dtype, codes, reinterpret_cast<float *>(ws), reinterpret_cast<char *>(ws) + a,
+                    ws_bytes - a);
 }
 
 }  // extern "C"

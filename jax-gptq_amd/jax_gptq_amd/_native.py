@@ -53,6 +53,12 @@ SIGNATURES = {
     "gptq_hip_qmatmul_bits_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32, _i32, _i32]),
     "gptq_hip_qmatmul_bits": (_i32, [_vp, _vp, _i32, _i64, _vp, _i64, _i64, _vp, _vp, _i32, _i32, _i32, _vp, _vp,
                                      _sz]),
+    "gptq_hip_solve_grouped_workspace_bytes": (_sz, [_i64, _i64, _i32, _i32]),
+    "gptq_hip_solve_grouped": (_i32, [_vp, _vp, _i64, _i64, _vp, _i32, _i32, _i32, _vp, _i32, _vp, _vp, _vp, _vp, _sz]),
+    "gptq_hip_quantize_pack_grouped": (_i32, [_vp, _vp, _i32, _i64, _i64, _vp, _vp, _i64, _i32, _vp]),
+    "gptq_hip_dequant_grouped": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp, _i32, _i64, _i32, _vp]),
+    "gptq_hip_qmatmul_grouped": (_i32, [_vp, _vp, _i32, _i64, _vp, _i64, _i64, _vp, _vp, _i32, _i64, _i32, _i32, _vp,
+                                        _vp, _sz]),
     "gptq_hip_qmatmul_static": (_i32, [_vp, _vp, _i32, _i64, _vp, _i64, _i64, _vp, _vp, _i32, _i32, _vp]),
 }
 

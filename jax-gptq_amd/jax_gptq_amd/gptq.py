@@ -85,11 +85,16 @@ def _to_f32_copy(t):
 class QuantizedMatrix:
     """Packed matrix container (reference ``gptq.py:8-22``): ``int_weight`` uint8 with two
     4-bit codes per byte along ``contraction_axis``, per-channel ``zero`` and ``scale``.
-    ``bits`` (not in the reference, which is fixed at 4): 8 means one code per byte."""
+    ``bits`` (not in the reference, which is fixed at 4): 8 means one code per byte.  ``group_size`` (not in
+    the reference either): ``zero`` / ``scale`` are ``[K / group_size, N]`` tables of a 2-D matrix packed along
+    axis 0, one row per group of ``group_size`` consecutive input features; 0 means one value per channel."""
 
-    def __init__(self, int_weight, zero, scale, contraction_axis=0, bits=4):
+    def __init__(self, int_weight, zero, scale, contraction_axis=0, bits=4, group_size=0):
         if bits not in (4, 8):
             raise ValueError("bits must be 4 or 8")
+        if group_size and contraction_axis != 0:
+            raise ValueError("grouped parameters need contraction_axis == 0")
+        self.group_size = int(group_size)
         self.int_weight = int_weight
         self.zero = zero
         self.scale = scale
@@ -106,13 +111,14 @@ class QuantizedMatrix:
 
     # pytree-style helpers (the reference registers the class as a pytree, gptq.py:24-32)
     def tree_flatten(self):
-        aux = self.contraction_axis if self.bits == 4 else (self.contraction_axis, self.bits)
+        plain = self.bits == 4 and not self.group_size
+        aux = self.contraction_axis if plain else (self.contraction_axis, self.bits, self.group_size)
         return (self.int_weight, self.zero, self.scale), aux
 
     @classmethod
     def tree_unflatten(cls, aux, children):
-        axis, bits = aux if isinstance(aux, tuple) else (aux, 4)
-        return cls(*children, contraction_axis=axis, bits=bits)
+        axis, bits, group = aux if isinstance(aux, tuple) else (aux, 4, 0)
+        return cls(*children, contraction_axis=axis, bits=bits, group_size=group)
 
     def to(self, *args, **kwargs):
         """Move to a device.  Element-type requests are ignored: a cast of a packed parameter
@@ -124,7 +130,7 @@ class QuantizedMatrix:
         if device is None:
             return self
         return QuantizedMatrix(self.int_weight.to(device), self.zero.to(device),
-                               self.scale.to(device), self.contraction_axis, self.bits)
+                               self.scale.to(device), self.contraction_axis, self.bits, self.group_size)
 
     # ---- array-like behaviour inside model functions.  A model written for dense weights
     # (x @ w, F.linear(x, w), w.T @ x, torch.tensordot(w, x, ...)) runs unchanged on packed ones:
@@ -179,7 +185,7 @@ class QuantizedMatrix:
     def __getattr__(self, name):
         # any other tensor method (w.sum(), w.abs(), ...): unpack, then do as written
         # (reference transform.py:74-79)
-        if name.startswith("_") or name in ("int_weight", "zero", "scale", "contraction_axis", "bits"):
+        if name.startswith("_") or name in ("int_weight", "zero", "scale", "contraction_axis", "bits", "group_size"):
             raise AttributeError(name)
         return getattr(unpack_matrix(self), name)
 
@@ -425,8 +431,22 @@ def _solve(W, L, params, block_size, out_dtype, want_codes=False):
     return Q, codes
 
 
+def _solve_grouped(W, L, bits, group_size, block_size, out_dtype):
+    """The column loop with one scale / zero per channel and group of ``group_size`` input features."""
+    lib = N.load()
+    K, Nc = W.shape
+    Q = torch.empty((K, Nc), dtype=out_dtype, device=W.device)
+    scale = torch.empty((K // group_size, Nc), dtype=torch.float32, device=W.device)
+    zero = torch.empty((K // group_size, Nc), dtype=torch.float32, device=W.device)
+    ws = _ws(lib.gptq_hip_solve_grouped_workspace_bytes(K, Nc, block_size, group_size))
+    N.check(lib.gptq_hip_solve_grouped(_stream(), _ptr(W), K, Nc, _ptr(L), group_size, bits, block_size, _ptr(Q),
+                                       _DT[out_dtype], _ptr(None), _ptr(scale), _ptr(zero), _ptr(ws), ws.numel()),
+            "solve_grouped")
+    return Q, {"maxq": 2 ** bits - 1, "scale": scale, "zero": zero, "group_size": group_size}
+
+
 def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=None, shared=None,
-         bits=4, split_fp16=False):
+         bits=4, split_fp16=False, group_size=None):
     """The per-layer GPTQ solve (reference ``gptq.py:182-212``).
 
     ``W`` is ``[K, N]`` (input features x output channels), ``xs`` a list of calibration
@@ -441,8 +461,20 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=
     calls.  ``bits`` (1 to 8; the reference's ``gptq`` is fixed at the default of its
     ``get_quantize_params``, 4): the code width, ``maxq = 2**bits - 1``; ``pack_matrix`` stores
     4-bit results two per byte and 8-bit results one per byte.  ``split_fp16``: see
-    ``accumulate_H``.
+    ``accumulate_H``.  ``group_size`` (not in the reference): one scale / zero per output channel and group of
+    ``group_size`` consecutive input features instead of one per channel; a group's parameters are the min-max
+    parameters of its rows as they stand when the column loop reaches them.  ``params['scale']`` /
+    ``['zero']`` are then ``[K / group_size, N]`` and ``params['group_size']`` is set.  Must be a multiple of
+    ``block_size`` that divides ``K`` and 512; not combinable with ``actorder`` (the permutation would scatter a
+    group's rows).
     """
+    if group_size:
+        group_size = int(group_size)
+        if actorder:
+            raise ValueError("group_size and actorder cannot be combined")
+        if group_size % block_size or 512 % group_size or _float_dev(W).shape[0] % group_size:
+            raise ValueError(f"group_size={group_size} must be a multiple of block_size={block_size} "
+                             "that divides K and 512")
     Wt = _float_dev(W)
     if Wt.dim() != 2:
         raise ValueError("W must be a 2-D matrix [K, N]")
@@ -487,7 +519,10 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=
     # The column loop is enqueued before the host reads the status word back, so that the GPU
     # does not sit idle while the host waits and then launches; with a NaN factor the loop
     # computes garbage that is thrown away by the exception below (gptq.py:194-196).
-    Q, _ = _solve(W32, Hinv, quantize_params, block_size, orig_type)
+    if group_size:
+        Q, quantize_params = _solve_grouped(W32, Hinv, int(bits), group_size, block_size, orig_type)
+    else:
+        Q, _ = _solve(W32, Hinv, quantize_params, block_size, orig_type)
     if perm is not None:
         Q = _unpermute(Q, perm)
     if status is not None:
@@ -576,6 +611,20 @@ def pack_matrix(Q, params, contraction_axis=0):
     Qt = _float_dev(Q)
     scale = _dev(params["scale"])
     zero = _dev(params["zero"])
+    group = int(params.get("group_size", 0) or 0)
+    if group:
+        if Qt.dim() != 2 or contraction_axis != 0:
+            raise ValueError("grouped parameters need a 2-D matrix packed along axis 0")
+        K, Nc = Qt.shape
+        if K % group or group % 2 or tuple(scale.shape) != (K // group, Nc) or tuple(zero.shape) != (K // group, Nc):
+            raise ValueError("scale/zero must be [K / group_size, N]")
+        packed = torch.empty((K // 2 if bits == 4 else K, Nc), dtype=torch.uint8, device=Qt.device)
+        scale32 = scale.to(torch.float32).contiguous()
+        zero32 = zero.to(torch.float32).contiguous()
+        N.check(lib.gptq_hip_quantize_pack_grouped(_stream(), _ptr(Qt), _DT[Qt.dtype], K, Nc, _ptr(scale32),
+                                                   _ptr(zero32), group, bits, _ptr(packed)), "quantize_pack_grouped")
+        return QuantizedMatrix(int_weight=packed, zero=zero, scale=scale, contraction_axis=0, bits=bits,
+                               group_size=group)
     outer, alen, inner = _view3(Qt.shape, contraction_axis)
     if bits == 4 and alen % 2:
         raise ValueError("the contraction axis must have even length")
@@ -599,6 +648,14 @@ def unpack_matrix(weight):
     iw = _dev(weight.int_weight, torch.uint8)
     zero = _float_dev(weight.zero)
     scale = _float_dev(weight.scale).to(zero.dtype)
+    group = int(getattr(weight, "group_size", 0) or 0)
+    if group:
+        bits = int(getattr(weight, "bits", 4))
+        R, C = iw.shape
+        out = torch.empty((R * (8 // bits), C), dtype=zero.dtype, device=iw.device)
+        N.check(lib.gptq_hip_dequant_grouped(_stream(), _ptr(iw), R, C, _ptr(zero), _ptr(scale), _DT[zero.dtype],
+                                             group, bits, _ptr(out)), "dequant_grouped")
+        return out
     outer, plen, inner = _view3(iw.shape, weight.contraction_axis)
     if zero.numel() != outer * inner or scale.numel() != outer * inner:
         raise ValueError("scale/zero must have the shape of the matrix without the contraction axis")

@@ -29,7 +29,7 @@ def _qmm_workspace(nbytes, device):
     return ws
 
 
-def _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b, bits=4):
+def _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b, bits=4, group_size=0):
     lib = N.load()
     leading_dims = None
     if x.dim() > 2:
@@ -53,9 +53,17 @@ def _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b, bits=4):
     out = torch.empty((M, out_n), dtype=x.dtype, device=x.device)
     ws = _qmm_workspace(lib.gptq_hip_qmatmul_bits_workspace_bytes(M, R, C, int(transpose_b), _DT[x.dtype], bits),
                         x.device)
-    N.check(lib.gptq_hip_qmatmul_bits(_stream(), _ptr(x), _DT[x.dtype], M, _ptr(int_weight), R, C,
-                                      _ptr(zero), _ptr(scale), _DT[zero.dtype], bits, int(transpose_b),
-                                      _ptr(out), _ptr(ws), ws.numel()), "qmatmul")
+    if group_size:
+        zero, scale = zero.contiguous(), scale.contiguous()
+        if tuple(zero.shape) != (Kw // group_size, C) or tuple(scale.shape) != (Kw // group_size, C):
+            raise ValueError("grouped zero/scale must be [K / group_size, N]")
+        N.check(lib.gptq_hip_qmatmul_grouped(_stream(), _ptr(x), _DT[x.dtype], M, _ptr(int_weight), R, C,
+                                             _ptr(zero), _ptr(scale), _DT[zero.dtype], group_size, bits,
+                                             int(transpose_b), _ptr(out), _ptr(ws), ws.numel()), "qmatmul")
+    else:
+        N.check(lib.gptq_hip_qmatmul_bits(_stream(), _ptr(x), _DT[x.dtype], M, _ptr(int_weight), R, C,
+                                          _ptr(zero), _ptr(scale), _DT[zero.dtype], bits, int(transpose_b),
+                                          _ptr(out), _ptr(ws), ws.numel()), "qmatmul")
     if leading_dims is not None:
         out = out.reshape(tuple(leading_dims) + (out_n,))
     return out
@@ -63,18 +71,19 @@ def _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b, bits=4):
 
 class _QuantizedMatmulFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, int_weight, zero, scale, transpose_b, bits):
+    def forward(ctx, x, int_weight, zero, scale, transpose_b, bits, group_size):
         ctx.save_for_backward(int_weight, zero, scale)
         ctx.transpose_b = transpose_b
         ctx.bits = bits
-        return _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b, bits)
+        ctx.group_size = group_size
+        return _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b, bits, group_size)
 
     @staticmethod
     def backward(ctx, y_bar):
         int_weight, zero, scale = ctx.saved_tensors
         x_bar = _quantized_matmul_raw(y_bar.contiguous(), int_weight, zero, scale,
-                                      not ctx.transpose_b, ctx.bits)
-        return x_bar, None, None, None, None, None
+                                      not ctx.transpose_b, ctx.bits, ctx.group_size)
+        return x_bar, None, None, None, None, None, None
 
 
 def _quantized_matmul(x, quantized_matrix, transpose_b):
@@ -87,9 +96,10 @@ def _quantized_matmul(x, quantized_matrix, transpose_b):
     bits = int(getattr(quantized_matrix, "bits", 4))
     if bits not in (4, 8):
         raise ValueError("quantized_matmul takes 4-bit or 8-bit codes")
+    group = int(getattr(quantized_matrix, "group_size", 0) or 0)
     if x.requires_grad:
-        return _QuantizedMatmulFn.apply(x, iw, zero, scale, bool(transpose_b), bits)
-    return _quantized_matmul_raw(x, iw, zero, scale, bool(transpose_b), bits)
+        return _QuantizedMatmulFn.apply(x, iw, zero, scale, bool(transpose_b), bits, group)
+    return _quantized_matmul_raw(x, iw, zero, scale, bool(transpose_b), bits, group)
 
 
 def quantized_matmul(x, quantized_matrix, transpose_b=False):

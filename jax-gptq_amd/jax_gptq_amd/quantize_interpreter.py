@@ -245,18 +245,25 @@ class _Session:
             raise ValueError(f"block_size={o['block_size']} must divide the contraction size "
                              f"{W2.shape[0]} of parameter {leaf}")
         Q2, qp = gptq(W=W2, xs=xs, block_size=o["block_size"], actorder=o["actorder"],
-                      damping=o["damping"], use_fp64=o["use_fp64"], shared=self._shared(xs), bits=o["bits"])
+                      damping=o["damping"], use_fp64=o["use_fp64"], shared=self._shared(xs), bits=o["bits"],
+                      group_size=o["group_size"])
         Qt = _dots.from_matrix(Q2, tuple(w.shape), wc)                       # layout fn sees
-        scale_shape = tuple(d for i, d in enumerate(w.shape) if i != wc)
-        packed = pack_matrix(Qt.contiguous(),
-                             {"scale": qp["scale"].reshape(scale_shape),
-                              "zero": qp["zero"].reshape(scale_shape), "maxq": qp["maxq"]},
-                             contraction_axis=wc)
+        if o["group_size"]:
+            if w.dim() != 2 or wc != 0 or tuple(perm) != (0, 1):
+                raise NotImplementedError("grouped parameters need a 2-D weight that fn contracts along axis 0")
+            packed = pack_matrix(Qt.contiguous(), qp, contraction_axis=0)
+        else:
+            scale_shape = tuple(d for i, d in enumerate(w.shape) if i != wc)
+            packed = pack_matrix(Qt.contiguous(),
+                                 {"scale": qp["scale"].reshape(scale_shape),
+                                  "zero": qp["zero"].reshape(scale_shape), "maxq": qp["maxq"]},
+                                 contraction_axis=wc)
         inverse = tuple(int(i) for i in np.argsort(perm))
         if inverse != tuple(range(len(perm))):
             packed = permute_quantized(packed, inverse)
             packed = QuantizedMatrix(packed.int_weight.contiguous(), packed.zero.contiguous(),
-                                     packed.scale.contiguous(), packed.contraction_axis, packed.bits)
+                                     packed.scale.contiguous(), packed.contraction_axis, packed.bits,
+                                     packed.group_size)
         self.results[leaf] = packed
         # the product is evaluated with the quantised or the original weight; every later use
         # of the parameter sees the quantised one (quantize_interpreter.py:241-243, 289-291)
@@ -267,7 +274,7 @@ class _Session:
 
 def quantize(fn, params, inputs, block_size=128, actorder=False, damping=0.01,
              use_quantized_activations=True, use_fp64=False, use_params_fp32=False, split_fp16=False,
-             bits=4):
+             bits=4, group_size=None):
     """Run GPTQ over the parameters of ``fn`` (reference ``quantize_interpreter.py:25-80``).
 
     ``fn(params, batch)``: the model; ``params``: a nested dict / list / tuple of arrays;
@@ -277,7 +284,8 @@ def quantize(fn, params, inputs, block_size=128, actorder=False, damping=0.01,
     everything else is returned as it came.  Buffers of ``params`` that already live on the
     GPU are overwritten with the quantised values, so do not reuse them (the reference frees
     them, ``:42``).  ``split_fp16`` (not in the reference): see ``accumulate_H``.  ``bits`` (not in
-    the reference, whose code width is fixed at 4): 4 or 8.
+    the reference, whose code width is fixed at 4): 4 or 8.  ``group_size`` (not in the reference): see
+    ``gptq``; for 2-D weights that ``fn`` contracts along axis 0 (``x @ w``).
     """
     if int(bits) not in (4, 8):
         raise ValueError("quantize packs 4-bit or 8-bit codes")
@@ -295,7 +303,8 @@ def quantize(fn, params, inputs, block_size=128, actorder=False, damping=0.01,
         flat.append(t)
     session = _Session(flat, dict(block_size=block_size, actorder=actorder, damping=damping,
                                   use_quantized_activations=use_quantized_activations,
-                                  use_fp64=use_fp64, split_fp16=split_fp16, bits=int(bits)))
+                                  use_fp64=use_fp64, split_fp16=split_fp16, bits=int(bits),
+                                  group_size=int(group_size) if group_size else None))
     wrapped = [(_Target(t, i, range(t.dim())) if isinstance(t, torch.Tensor) and t.is_floating_point()
                 and t.dim() > 1 else t) for i, t in enumerate(flat)]
     fn_params = _unflatten(struct, wrapped)

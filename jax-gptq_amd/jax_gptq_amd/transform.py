@@ -121,6 +121,10 @@ def permute_quantized(qm, perm):
     """The packed matrix of ``dense.permute(perm)`` (reference ``inverse_transpose``,
     ``quantize_interpreter.py:533-554``)."""
     perm = tuple(int(p) % len(perm) for p in perm)
+    if getattr(qm, "group_size", 0):
+        if perm != tuple(range(len(perm))):
+            raise NotImplementedError("a matrix with grouped parameters cannot be transposed in packed form")
+        return qm
     ca = qm.contraction_axis
     new_ca = perm.index(ca)
     scale_perm = [p if p < ca else p - 1 for p in perm if p != ca]
@@ -128,4 +132,5 @@ def permute_quantized(qm, perm):
     def move(v):
         return v.permute(scale_perm) if isinstance(v, torch.Tensor) and v.dim() > 1 else v
     return QuantizedMatrix(int_weight=qm.int_weight.permute(perm), zero=move(qm.zero),
-                           scale=move(qm.scale), contraction_axis=new_ca, bits=getattr(qm, "bits", 4))
+                           scale=move(qm.scale), contraction_axis=new_ca, bits=getattr(qm, "bits", 4),
+                           group_size=getattr(qm, "group_size", 0))

@@ -54,7 +54,8 @@ __all__ = [
 class QuantizedMatrix:
     """Container of a packed matrix (reference ``gptq.py:8-22``)."""
 
-    def __init__(self, int_weight, zero, scale, contraction_axis=0, bits=4):
+    def __init__(self, int_weight, zero, scale, contraction_axis=0, bits=4, group_size=0):
+        self.group_size = group_size   # > 0 (an extension): zero / scale are [K / group_size, N] tables
         self.int_weight = int_weight
         self.zero = zero
         self.scale = scale
@@ -220,7 +221,7 @@ def unpermute(Q, perm):
 
 
 def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False,
-         _loop_dtype=np.float32, _H=None, _bits=4):
+         _loop_dtype=np.float32, _H=None, _bits=4, _group_size=0):
     """The per-layer solve (reference ``gptq.py:182-212``).
 
     Returns ``(Q, params)``: ``Q`` is the DEQUANTISED matrix in ``W``'s dtype and
@@ -229,6 +230,12 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False,
     ``_loop_dtype``, ``_H`` and ``_bits`` are test hooks only: the reference always runs the
     column loop in fp32 (``gptq.py:184,197``), always builds ``H`` from ``xs`` and always takes
     the default width of ``get_quantize_params`` (4 bits, ``gptq.py:105,185``).
+
+    ``_group_size`` (an extension with no counterpart in the reference, stated here as the specification
+    the HIP path is checked against): when the loop reaches a row ``r0`` that is a multiple of it, the
+    parameters of rows ``[r0, r0 + group)`` are ``get_col_quantize_params`` of those rows of the working
+    matrix as they then stand (every correction of the rows above applied); ``scale`` / ``zero`` come back
+    as ``[K / group, N]``.  Must be a multiple of ``block_size``.
     """
     W = np.asarray(W)
     orig_type = W.dtype
@@ -248,8 +255,13 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False,
 
     K = W.shape[0]
     blocks = []
+    group_scale, group_zero = [], []
     for start in range(0, K, block_size):
         end = start + block_size
+        if _group_size and start % _group_size == 0:
+            quantize_params = get_col_quantize_params(W[start:start + _group_size], bits=_bits)
+            group_scale.append(quantize_params["scale"])
+            group_zero.append(quantize_params["zero"])
         q_block, errors = process_block(W, Hinv, start, quantize_params, block_size)
         if end < K:
             update = (Hinv[end:, start:end] @ errors).astype(W.dtype)
@@ -259,13 +271,21 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False,
     Q = np.concatenate(blocks, axis=0).astype(orig_type)
     if perm is not None:
         Q = unpermute(Q, perm)
+    if _group_size:
+        quantize_params = {"maxq": quantize_params["maxq"], "scale": np.stack(group_scale),
+                           "zero": np.stack(group_zero), "group_size": _group_size}
     return Q, quantize_params
 
 
 def codes_from_q(Q, params, contraction_axis=0):
     """Integer codes of a dequantised matrix (first line of ``pack_matrix``, ``gptq.py:221``)."""
-    scale = np.expand_dims(np.asarray(params["scale"]), axis=contraction_axis)
-    zero = np.expand_dims(np.asarray(params["zero"]), axis=contraction_axis)
+    group = int(params.get("group_size", 0) or 0)
+    if group:      # [K / group, N] tables of a 2-D matrix: every row takes its group's row
+        scale = np.repeat(np.asarray(params["scale"]), group, axis=0)
+        zero = np.repeat(np.asarray(params["zero"]), group, axis=0)
+    else:
+        scale = np.expand_dims(np.asarray(params["scale"]), axis=contraction_axis)
+        zero = np.expand_dims(np.asarray(params["zero"]), axis=contraction_axis)
     return np.round(np.asarray(Q) / scale + zero).astype(np.uint8)
 
 
@@ -276,13 +296,18 @@ def pack_matrix(Q, params, contraction_axis=0):
     # 8-bit codes (not in the reference) are the uint8 matrix itself
     packed = pack_along_axis(contraction_axis, int_matrix) if bits == 4 else int_matrix
     return QuantizedMatrix(int_weight=packed, zero=np.asarray(params["zero"]),
-                           scale=np.asarray(params["scale"]), contraction_axis=contraction_axis, bits=bits)
+                           scale=np.asarray(params["scale"]), contraction_axis=contraction_axis, bits=bits,
+                           group_size=int(params.get("group_size", 0) or 0))
 
 
 def unpack_matrix(weight):
     """Dense ``(code - zero) * scale`` (reference ``gptq.py:230-235``)."""
-    zero = np.expand_dims(weight.zero, axis=weight.contraction_axis)
-    scale = np.expand_dims(weight.scale, axis=weight.contraction_axis)
+    group = getattr(weight, "group_size", 0)
+    if group:
+        zero, scale = np.repeat(weight.zero, group, axis=0), np.repeat(weight.scale, group, axis=0)
+    else:
+        zero = np.expand_dims(weight.zero, axis=weight.contraction_axis)
+        scale = np.expand_dims(weight.scale, axis=weight.contraction_axis)
     unpacked = (unpack_along_axis(weight.contraction_axis, weight.int_weight)
                 if getattr(weight, "bits", 4) == 4 else np.asarray(weight.int_weight))
     return (unpacked.astype(zero.dtype) - zero) * scale
@@ -349,8 +374,13 @@ def quantized_matmul(x, quantized_matrix, transpose_b=False):
     w = quantized_matrix.int_weight
     bits = getattr(quantized_matrix, "bits", 4)
     codes = (unpack_along_axis(0, w) if bits == 4 else np.asarray(w)).astype(np.float32)
-    dense = (codes - quantized_matrix.zero.astype(np.float32)[None, :]) * \
-        quantized_matrix.scale.astype(np.float32)[None, :]
+    group = getattr(quantized_matrix, "group_size", 0)
+    if group:
+        dense = (codes - np.repeat(quantized_matrix.zero.astype(np.float32), group, axis=0)) * \
+            np.repeat(quantized_matrix.scale.astype(np.float32), group, axis=0)
+    else:
+        dense = (codes - quantized_matrix.zero.astype(np.float32)[None, :]) * \
+            quantized_matrix.scale.astype(np.float32)[None, :]
     K = x.shape[1]
     if transpose_b:
         assert K == w.shape[1], f"Inner dim mismatch: {K} != {w.shape[1]}"

@@ -307,3 +307,38 @@ def test_quantized_matmul_equals_dense(transpose):
     assert np.allclose(out, ref, atol=1e-2, rtol=1e-3)
     with pytest.raises(AssertionError):
         O.quantized_matmul(x[..., :-2], qm, transpose_b=transpose)
+
+
+# ---------------------------------------------------------------------------- grouped parameters (extension)
+def test_grouped_parameters_reduce_to_the_per_channel_solve_and_to_rtn():
+    """The group_size extension has no counterpart in the reference; what pins its restatement:
+    (i) one group spanning all of K is the per-channel solve, bit for bit; (ii) with H = c I nothing is
+    corrected, so every group is plain round-to-nearest on the min-max grid of that group's rows of the
+    ORIGINAL matrix (brute force below); (iii) every output lies on its group's grid."""
+    rng = np.random.default_rng(5)
+    K, N, g = 256, 12, 128
+    W = (0.02 * rng.standard_normal((K, N))).astype(np.float32)
+    X = rng.standard_normal((700, K)).astype(np.float32)
+    Q0, p0 = O.gptq(W, [X])
+    Qk, pk = O.gptq(W, [X], _group_size=K)
+    assert np.array_equal(Q0, Qk) and np.array_equal(pk["scale"][0], p0["scale"]) and pk["group_size"] == K
+    # (ii) orthogonal calibration columns: H = c I exactly
+    Hc = 3.0 * np.eye(K, dtype=np.float32)
+    Qi, pi = O.gptq(W, None, _H=Hc, _group_size=g)
+    assert pi["scale"].shape == (K // g, N)
+    for gi in range(K // g):
+        rows = W[gi * g:(gi + 1) * g]
+        ref = O.get_col_quantize_params(rows)
+        assert np.array_equal(pi["scale"][gi], ref["scale"]) and np.array_equal(pi["zero"][gi], ref["zero"])
+        grid = ref["scale"][None, None, :] * (np.arange(16, dtype=np.float32)[None, :, None] - ref["zero"][None, None, :])
+        nearest = np.take_along_axis(grid, np.abs(rows[:, None, :] - grid).argmin(1)[:, None, :], 1)[:, 0, :]
+        got = Qi[gi * g:(gi + 1) * g]
+        # ties aside (none with random data), round-to-nearest-even on the grid is the nearest grid point
+        assert np.allclose(got, nearest, rtol=0, atol=1e-7)
+    # (iii) on the grid, and a different result from the per-channel one
+    Qg, pg = O.gptq(W, [X], _group_size=g)
+    codes = Qg / np.repeat(pg["scale"], g, 0) + np.repeat(pg["zero"], g, 0)
+    assert np.abs(codes - np.rint(codes)).max() < 1e-3 and codes.min() > -0.5 and codes.max() < 15.5
+    assert not np.array_equal(Qg, Q0)
+    packed = O.pack_matrix(Qg, pg)
+    assert packed.group_size == g and np.array_equal(O.unpack_matrix(packed), Qg.astype(np.float32))
