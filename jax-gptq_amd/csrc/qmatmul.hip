@@ -534,9 +534,11 @@ __global__ __launch_bounds__(256, 2) void qmm_fwd_stream_kernel(
 //    Integer addition is exact and commutative: the result does not depend on the arrival order.
 //    One round trip to the memory side instead of three (partial stores -> ticket -> partial
 //    loads).  A poisoned sum yields NaN.  S <= 32.
-//  * M > 8: the memory side retires the atomics at a limited rate (350000 of them add 2 us, 700000
-//    add 4); where there would be more than ~760000, or the matrix runs in ring-loop mode, the
-//    workgroups keep qmm_reduce_and_store (ATOM = false).
+//    A thread issues the atomics of all its outputs before it looks at any returned word: one round
+//    trip per thread, not per output (M = 16 on 4096 x 11008: 14.2 -> 12.8 us).
+//  * M > 8: the memory side retires the atomics at a limited rate (700000 of them add about 3 us);
+//    where there would be more than ~760000 in at most three splits, the workgroups keep
+//    qmm_reduce_and_store (ATOM = false).
 constexpr int QD_FRAC = 28;
 constexpr long long QD_POISON = 3LL << 49;
 constexpr int QD_MAX_SPLITS = 32;
@@ -686,11 +688,17 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
   float *xs = red + (size_t)NW * MR * QSTRIP;   // [wave][2][16]
   if (g == 0) { xs[wave * 32 + l16] = se; xs[wave * 32 + 16 + l16] = so; }
   __syncthreads();
+  // Two passes over this thread's outputs, so that its atomics are in flight together: a pass that used each
+  // returned word at once would pay one round trip to the memory side per output.
+  unsigned long long old[IT], word[IT];
+  bool live[IT];
 #pragma unroll
   for (int it = 0; it < IT; ++it) {
     const int idx = tid + it * NT;
     const int m = idx >> 8, c = idx & 255, n = strip * QSTRIP + c;
-    if (idx >= ITEMS || m >= mvalid || n >= C) continue;
+    live[it] = idx < ITEMS && m < mvalid && n < C;
+    old[it] = word[it] = 0ull;
+    if (!live[it]) continue;
     float v = 0.f, e = 0.f, o = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) {
@@ -701,23 +709,27 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
     const float r = BF ? (v - 128.f * (e + o)) - pz[it] * (e + o)
                        : (v - 1024.f * (e + o)) - pz[it] * (e + 16.f * o);
     const float pv = psc[it] * r;
-    TX *dst = out + (int64_t)(m0 + m) * C + n;
     if (S == 1) {
-      *dst = Act<TX>::out(pv);
+      out[(int64_t)(m0 + m) * C + n] = Act<TX>::out(pv);
+      live[it] = false;
       continue;
     }
     const bool ok = fabsf(pv) <= 65536.f;                       // false for NaN, too
     const long long fx = ok ? __float2ll_rn(pv * (float)(1 << QD_FRAC)) : QD_POISON;
-    const unsigned long long word = ((unsigned long long)fx << 8) + 1ull;
-    unsigned long long *cell = ws.acc64 + (int64_t)(m0 + m) * C + n;
-    const unsigned long long total = atomicAdd(cell, word) + word;
-    if ((int)(total & 255ull) == S) {                           // every contribution is in
-      const long long sum = (long long)total >> 8;
-      const bool fine = sum <= (1LL << 49) && sum >= -(1LL << 49);
-      const float res = fine ? (float)sum * (1.f / (float)(1 << QD_FRAC)) : __builtin_nanf("");
-      *dst = Act<TX>::out(res);
-      __hip_atomic_store(cell, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+    word[it] = ((unsigned long long)fx << 8) + 1ull;
+    old[it] = atomicAdd(ws.acc64 + (int64_t)(m0 + m) * C + n, word[it]);     // (used in the second pass only)
+  }
+#pragma unroll
+  for (int it = 0; it < IT; ++it) {
+    const unsigned long long total = old[it] + word[it];
+    if (!live[it] || (int)(total & 255ull) != S) continue;      // not the last of the S contributions
+    const int idx = tid + it * NT;
+    const int m = idx >> 8, n = strip * QSTRIP + (idx & 255);
+    const long long sum = (long long)total >> 8;
+    const bool fine = sum <= (1LL << 49) && sum >= -(1LL << 49);
+    const float res = fine ? (float)sum * (1.f / (float)(1 << QD_FRAC)) : __builtin_nanf("");
+    out[(int64_t)(m0 + m) * C + n] = Act<TX>::out(res);
+    __hip_atomic_store(ws.acc64 + (int64_t)(m0 + m) * C + n, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
@@ -860,10 +872,11 @@ DecPlan dec_plan(int64_t M, int64_t R, int64_t C) {
       p.loop = true;
     }
     if (p.S > QD_MAX_SPLITS) p.atom = false;
-    // Beyond 8 rows the atomics pay only while there are few of them (the memory side retires them at a
-    // limited rate) and the matrix is one the chip holds in flight: 4096 x 11008 at M = 16 (700000 atomics)
-    // 15.4 -> 14.4 us, 11008 x 4096 18.2 -> 13.9 us, but 7168 x 28672 (ring-loop mode, 920000) 26.8 -> 29.0 us.
-    if (M > 8 && (p.loop || M * C * p.S > 760000)) p.atom = false;
+    // Beyond 8 rows the memory side's rate of atomics shows (700000 of them add about 3 us), and so does what the
+    // other path costs, whose last workgroup reads S partial tiles: with many atomics and at most three splits
+    // the workgroups keep qmm_reduce_and_store (7168 x 28672 at M = 16, S = 2, 920000 atomics: 27.3 us against
+    // 28.1), otherwise the atomic sum wins (28672 x 7168, S = 9: 30.3 -> 28.9 us; 8192 x 8192, S = 8: 18.1 -> 16.6).
+    if (M > 8 && M * C * p.S > 760000 && p.S < 4) p.atom = false;
     if (p.atom) {
       p.x1_bytes = p.part_bytes = 0;
       p.total_bytes = p.S > 1 ? QMM_HEAD_BYTES : 0;
