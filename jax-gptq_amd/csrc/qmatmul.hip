@@ -550,6 +550,10 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
   constexpr bool BF = Act<TX>::BF;
   extern __shared__ float red[];   // [NW][MR][256] partial tiles, then [NW][2][16] x sums
   __shared__ int s_last;
+  // every kernel argument in registers before the first address is formed (left to itself the compiler
+  // fetches them one by one where they are first used, and waits for each)
+  asm volatile("" ::"s"(x), "s"(pk), "s"(zero), "s"(scale), "s"(out), "s"(ws.acc64), "s"(ws.counters), "s"(ws.part),
+               "s"(ws.x1part), "s"(M), "s"(K), "s"(R), "s"(C), "s"(S), "s"(rows_per_split));
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int strip = blockIdx.x, split = blockIdx.y, m0 = blockIdx.z * 16;
   const int mvalid = min(16, M - m0);
@@ -561,30 +565,23 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
 
   // One k-step of loads: the activations of the lane group's four packed rows (16 bytes = 8 k; range
   // boundaries are multiples of 4 rows, so the four rows are inside the range or outside together)
-  // and the four weight rows.  LOOP (a ring of KS k-steps that is refilled as it is consumed, for
-  // matrices beyond what the chip holds in flight): loads past the range read clamped, valid
-  // addresses and their k-step enters with zero activations.  Otherwise (all KS k-steps of the
-  // range issued at once) they are predicated off.
+  // and the four weight rows.  Nothing is predicated per lane (a predicated load is a branch, and its
+  // zero fill a register move per word: they delayed the last load of a workgroup by several hundred
+  // cycles): loads past the range or past the last column read clamped, valid addresses, and such a
+  // k-step enters with zero activations.  LOOP: a ring of KS k-steps that is refilled as it is consumed,
+  // for matrices beyond what the chip holds in flight; otherwise all KS k-steps of the range are issued
+  // at once, and a wavefront skips the k-steps that lie past its range altogether.
   struct Step { uint4 d[4]; uint4 pr; };
   const bool m_ok = l16 < mvalid;
   const TX *xr = x + (int64_t)(m0 + (m_ok ? l16 : 0)) * K;
-  const int col0 = LOOP ? min(strip * QSTRIP + 16 * l16, C - 16) : strip * QSTRIP + 16 * l16;
+  const int col0 = min(strip * QSTRIP + 16 * l16, C - 16);
   const uint8_t *wp = pk + col0;
   auto issue = [&](Step &st, int t) __attribute__((always_inline)) {
     const int rbase = r_begin + (t * NW + wave) * 16 + 4 * g;
-    if (LOOP) {
-      st.pr = *reinterpret_cast<const uint4 *>(xr + 2 * min(rbase, R - 4));
+    st.pr = *reinterpret_cast<const uint4 *>(xr + 2 * min(rbase, R - 4));
+    const uint8_t *row = wp + (int64_t)min(rbase, R - 4) * C;       // R % 4 == 0: four rows inside the matrix
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        st.d[i] = *reinterpret_cast<const uint4 *>(wp + (int64_t)min(rbase + i, R - 1) * C);
-    } else {
-      const bool in = rbase < r_end;
-      st.pr = (m_ok && in) ? *reinterpret_cast<const uint4 *>(xr + 2 * rbase) : make_uint4(0u, 0u, 0u, 0u);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        st.d[i] = (in && col0 < C) ? *reinterpret_cast<const uint4 *>(wp + (int64_t)(rbase + i) * C)
-                                   : make_uint4(0u, 0u, 0u, 0u);
-    }
+    for (int i = 0; i < 4; ++i) st.d[i] = *reinterpret_cast<const uint4 *>(row + (int64_t)i * C);
   };
 
   const DqConst dqk = dq_const<BF>();
@@ -595,7 +592,7 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
   float se = 0.f, so = 0.f;
   auto consume = [&](Step &st, int t) __attribute__((always_inline)) {
     uint4 pr = st.pr;
-    if (LOOP) {
+    {
       const bool ok = m_ok && t < nsteps && r_begin + (t * NW + wave) * 16 + 4 * g < r_end;
       pr.x = ok ? pr.x : 0u;
       pr.y = ok ? pr.y : 0u;
@@ -628,7 +625,8 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
 
   Step ring[KS];
 #pragma unroll
-  for (int u = 0; u < KS; ++u) issue(ring[u], u);
+  for (int u = 0; u < KS; ++u)
+    if (LOOP || u == 0 || u < nsteps) issue(ring[u], u);      // (wave-uniform)
   // ---- column parameters of the outputs this thread finishes, fetched under the weight loads
   constexpr int NT = NW * 64;
   constexpr int ITEMS = MR * QSTRIP;
@@ -642,6 +640,9 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
       psc[it] = to_f32(scale[n]);
     }
   }
+  // (without this the scheduler sinks the parameter loads below the wait for the weights, and their latency
+  // is paid after the last k-step instead of under it)
+  __builtin_amdgcn_sched_barrier(0);
   if (LOOP) {
     int t0 = 0;
     for (; t0 + KS <= nsteps; t0 += KS) {
