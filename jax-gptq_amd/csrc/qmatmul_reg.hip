@@ -42,6 +42,10 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
   constexpr int PR = 4 * NL;                     // packed rows per k-step
   extern __shared__ __attribute__((aligned(16))) float rg_lds[];   // [4 wavefronts][RB][RG_NT][64 lanes][4]
   __shared__ int s_flag;
+  // every kernel argument in registers before the first address is formed (left to itself the compiler
+  // fetches them in groups where they are first used, and waits for each group)
+  asm volatile("" ::"s"(x), "s"(pk), "s"(zero), "s"(scale), "s"(out), "s"(part), "s"(counters), "s"(M), "s"(K),
+               "s"(R), "s"(C), "s"(zs_dtype), "s"(S), "s"(steps_per_split), "s"(group_size));
   const int tid = threadIdx.x, lane = tid & 63, wk = tid >> 6;
   const int g = lane >> 4, l16 = lane & 15;
   int tx, ty;
@@ -84,19 +88,22 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
     }
   };
 
-  // the first k-steps' loads go out before anything that has to wait for memory
+  // Loads return in the order of their issue: the zero points, which the first k-step's dequantisation needs,
+  // go out first, then the first k-steps' loads, all before anything that has to wait for memory.
+  uint32_t zraw0[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+  if constexpr (!GROUPED) rg_params8_raw(zero, zs_dtype, 0, col, C, zraw0);
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int u = 0; u < RING; ++u) load_step(u, u);
+  __builtin_amdgcn_sched_barrier(0);
 
   // ---- per-channel constants of the dequantisation (the integer part of the zero point)
   uint32_t zc[8];
   float zi8[(BF && BITS == 8) ? 8 : 1];
   if constexpr (!GROUPED) {
-    float z8[8];
-    rg_params8(zero, zs_dtype, col, C, z8);
 #pragma unroll
     for (int t8 = 0; t8 < 8; ++t8) {
-    const float zi = fminf(fmaxf(rintf(z8[t8]), -512.f), 512.f);
+    const float zi = fminf(fmaxf(rintf(rg_raw_to_f32(zraw0[t8], zs_dtype)), -512.f), 512.f);
     if constexpr (BF) {
       zc[t8] = 0u;
       if constexpr (BITS == 8) zi8[t8] = zi;

@@ -71,6 +71,11 @@ __host__ __device__ inline QmmWs qmm_ws(void *base_v, size_t x1_bytes) {
 // activations once per group of column tiles.  The last gx % 8 column tiles keep the plain order.
 __device__ __forceinline__ void qmm_tile_coords(int &tx, int &ty) {
   const int gx = gridDim.x, gy = gridDim.y;
+  if (gy == 1) {                   // one row of tiles: the order below is the identity, without its divisions
+    tx = blockIdx.x;
+    ty = 0;
+    return;
+  }
   const int id = blockIdx.x + gx * blockIdx.y;
   const int full = (gx >> 3) << 3;
   if (id < full * gy) {
