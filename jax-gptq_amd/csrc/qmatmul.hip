@@ -539,8 +539,6 @@ __global__ __launch_bounds__(256, 2) void qmm_fwd_stream_kernel(
 //  * M > 8: the memory side retires the atomics at a limited rate (700000 of them add about 3 us);
 //    where there would be more than ~760000 in at most three splits, the workgroups keep
 //    qmm_reduce_and_store (ATOM = false).
-constexpr int QD_FRAC = 28;
-constexpr long long QD_POISON = 3LL << 49;
 constexpr int QD_MAX_SPLITS = 32;
 
 template <int NW, int KS, int MR, bool ATOM, bool LOOP, typename TZ, typename TX>

@@ -11,6 +11,8 @@ struct RegPlan {
   int bits, rb;            // rb: 16-row blocks per output tile (1 for M <= 16, else 4)
   bool ragged;             // C % 8 != 0, K % 8 != 0 or operands not 16-byte aligned: unaligned loads, element stores
   int S, steps;            // split of the contraction over S workgroups per tile, k-steps (32 k) per split
+  bool atom;               // 16-row tiles: the splits add their results to 64-bit fixed-point cells (one returning
+                           // atomic per output) instead of writing partial tiles and taking a ticket
   int64_t tiles;           // output tiles of one launch
   size_t part_bytes, total_bytes;
 };

@@ -32,10 +32,11 @@ constexpr int RG_BN = 128;                       // channels per output tile
 // the parameters of a k-step's group travel with its loads, and B = (code - zero) scale is formed in fp16
 // (converted for bf16 activations), so the accumulators need no offset or scale afterwards.
 template <int BITS, int RB, int RING, bool RAGGED, typename TX, bool GROUPED>
-__global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, int K, const uint8_t *pk, int R,
+__global__ __launch_bounds__(256, (RB == 1 ? 2 : 1)) void qmm_fwd_reg_kernel(const TX *x, int M, int K, const uint8_t *pk, int R,
                                                           int C, const void *zero, const void *scale,
                                                           int zs_dtype, TX *out, float *part, int32_t *counters,
-                                                          int S, int steps_per_split, int group_size) {
+                                                          int S, int steps_per_split, int group_size,
+                                                          unsigned long long *acc64) {
   constexpr bool BF = Act<TX>::BF && !GROUPED;      // grouped: the fp16 form of the dequantisation for both types
   constexpr int SCHED = RB == 4 ? 4 : 0;         // vector instructions between two MFMAs of the main loop (0: compiler's order)
   constexpr int NL = BITS == 4 ? 4 : 8;          // packed rows per lane and k-step
@@ -45,7 +46,7 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
   // every kernel argument in registers before the first address is formed (left to itself the compiler
   // fetches them in groups where they are first used, and waits for each group)
   asm volatile("" ::"s"(x), "s"(pk), "s"(zero), "s"(scale), "s"(out), "s"(part), "s"(counters), "s"(M), "s"(K),
-               "s"(R), "s"(C), "s"(zs_dtype), "s"(S), "s"(steps_per_split), "s"(group_size));
+               "s"(R), "s"(C), "s"(zs_dtype), "s"(S), "s"(steps_per_split), "s"(group_size), "s"(acc64));
   const int tid = threadIdx.x, lane = tid & 63, wk = tid >> 6;
   const int g = lane >> 4, l16 = lane & 15;
   int tx, ty;
@@ -219,7 +220,9 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
 #pragma unroll
     for (int u = 0; u < RING; ++u) {
       compute(u, plain);
-      load_step(u, s0 + u + RING);
+      // (16-row tiles: nothing is fetched for k-steps past this wavefront's last; wave-uniform.  64-row tiles keep
+      // one basic block per k-step for the instruction order below, and re-read their last k-step instead)
+      if (SCHED != 0 || s0 + u + RING < iters) load_step(u, s0 + u + RING);
       // One wavefront per SIMD issues in order: an MFMA occupies the matrix pipe for four passes, during
       // which the wavefront can issue only what stands behind it in program order and does not depend on it.
       // So the dequantisation of the next tile goes between the MFMAs of this one: one MFMA, then a few
@@ -253,10 +256,12 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
   }
   floatx4 sum[RG_NT];
   const int tile = ty * gridDim.x + tx;
-  if (!rg_reduce<RB>(acc, sum, rg_lds, &s_flag, part, counters, tile, split, S)) return;
+  // acc64 (16-row tiles only): every split finishes its own outputs and adds them to the cells
+  const bool atom = RB == 1 && acc64 != nullptr && S > 1;
+  if (!rg_reduce<RB>(acc, sum, rg_lds, &s_flag, part, counters, tile, split, atom ? 1 : S)) return;
   // sum[t8][r] = sum_k x[m][k] (code - zi)[k][col + t8] (bf16, 4-bit: code + 128), sum[8][r] = sum_k x[m][k],
   // m = m0 + 16 rb + 4 g + r
-  if (!col_ok) return;
+  if (!col_ok && !atom) return;
   const int rb = wk;                             // rg_reduce returned true: wk < RB
 #pragma unroll
   for (int t8 = 0; t8 < 8; ++t8) {
@@ -265,6 +270,57 @@ __global__ __launch_bounds__(256) void qmm_fwd_reg_kernel(const TX *x, int M, in
       zf[t8] = 0.f;
     } else {
       zf[t8] = (BF && BITS == 4) ? 128.f + zf[t8] : zf[t8] - fminf(fmaxf(rintf(zf[t8]), -512.f), 512.f);
+    }
+  }
+  if constexpr (RB == 1) {
+    if (atom) {
+      // This wavefront's finished values go through the LDS (the other wavefronts are done with it) so that
+      // consecutive lanes hold consecutive channels: the memory side takes an atomic per 64-byte segment,
+      // not per lane.  Then two passes per eight rows, so that a lane's atomics are in flight together.  The
+      // word that comes back tells the last of the S contributions that it is the last, and gives it the
+      // complete sum: it rounds, stores the output and zeroes the cell.  Integer addition is exact and
+      // commutative: the result does not depend on the order of arrival.
+      float *tr = rg_lds;                                  // [16 rows][128 channels]
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float rs = sum[8][r];
+        float pv[8];
+#pragma unroll
+        for (int t8 = 0; t8 < 8; ++t8) pv[t8] = sc[t8] * (sum[t8][r] - zf[t8] * rs);
+        float *dst = tr + (4 * g + r) * RG_BN + 8 * l16;
+        *reinterpret_cast<float4 *>(dst) = make_float4(pv[0], pv[1], pv[2], pv[3]);
+        *reinterpret_cast<float4 *>(dst + 4) = make_float4(pv[4], pv[5], pv[6], pv[7]);
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // one wavefront: its LDS accesses complete in order
+#pragma unroll
+      for (int mh = 0; mh < 2; ++mh) {
+        if (8 * mh >= M - m0) break;
+        unsigned long long old[16], word[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int mr = 8 * mh + (i >> 1), c = 64 * (i & 1) + lane;
+          old[i] = word[i] = 0ull;
+          if (m0 + mr >= M || nbase + c >= C) continue;
+          const float pv = tr[mr * RG_BN + c];
+          const bool ok = fabsf(pv) <= 65536.f;                       // false for NaN, too
+          const long long fx = ok ? __float2ll_rn(pv * (float)(1 << QD_FRAC)) : QD_POISON;
+          word[i] = ((unsigned long long)fx << 8) + 1ull;
+          old[i] = atomicAdd(acc64 + (int64_t)(m0 + mr) * C + nbase + c, word[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int mr = 8 * mh + (i >> 1), c = 64 * (i & 1) + lane;
+          const unsigned long long total = old[i] + word[i];
+          if ((int)(total & 255ull) != S) continue;                   // (also the lanes that added nothing: 0 != S)
+          const long long fsum = (long long)total >> 8;
+          const bool fine = fsum <= (1LL << 49) && fsum >= -(1LL << 49);
+          const float res = fine ? (float)fsum * (1.f / (float)(1 << QD_FRAC)) : __builtin_nanf("");
+          out[(int64_t)(m0 + mr) * C + nbase + c] = Act<TX>::out(res);
+          __hip_atomic_store(acc64 + (int64_t)(m0 + mr) * C + nbase + c, 0ull, __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+      return;
     }
   }
 #pragma unroll
@@ -295,6 +351,8 @@ int launch_inst(hipStream_t st, const RegPlan &p, const void *x, int64_t M, cons
   const int64_t K = BITS == 4 ? 2 * R : R;
   int32_t *counters = reinterpret_cast<int32_t *>(wsp);
   float *part = reinterpret_cast<float *>(reinterpret_cast<char *>(wsp) + QMM_HEAD_BYTES);
+  unsigned long long *acc64 =
+      p.atom ? reinterpret_cast<unsigned long long *>(reinterpret_cast<char *>(wsp) + QMM_COUNTER_BYTES) : nullptr;
   const int64_t tiles_x = ceil_div64(C, RG_BN);
   // rows per launch: 32-bit element offsets into x, grid.y, one arrival counter per tile, the partial region
   int64_t rows_max = ((1LL << 31) - 1) / K;
@@ -307,7 +365,7 @@ int launch_inst(hipStream_t st, const RegPlan &p, const void *x, int64_t M, cons
     const int64_t rows = M - r0 < rows_max ? M - r0 : rows_max;
     const dim3 grid((unsigned)tiles_x, (unsigned)ceil_div64(rows, 16 * RB), (unsigned)p.S);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (const TX *)x + r0 * K, (int)rows, (int)K, pk, (int)R,
-                       (int)C, zero, scale, zs_dtype, (TX *)out + r0 * C, part, counters, p.S, p.steps, group_size);
+                       (int)C, zero, scale, zs_dtype, (TX *)out + r0 * C, part, counters, p.S, p.steps, group_size, acc64);
     GPTQ_CHECK_LAUNCH();
   }
   return GPTQ_HIP_OK;
@@ -365,7 +423,11 @@ RegPlan reg_fwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned) {
   }
   p.steps = (int)ceil_div64(T, S);
   p.S = (int)ceil_div64(T, p.steps);
-  p.part_bytes = p.S > 1 ? (size_t)p.tiles * p.S * p.rb * RG_NT * RG_TILE_FLOATS * sizeof(float) : 0;
+  // 16-row tiles (one launch, M <= 16): the atomic sum where the cells hold the output and the atomics are few
+  // (the memory side retires them at a limited rate: 900000 of them cost what the ticket path costs on
+  // 4096 x 11008 and 4 us more on 7168 x 28672)
+  p.atom = p.rb == 1 && p.S > 1 && M * C * 8 <= QMM_ACC_BYTES && M * C * p.S <= 500000;
+  p.part_bytes = (p.S > 1 && !p.atom) ? (size_t)p.tiles * p.S * p.rb * RG_NT * RG_TILE_FLOATS * sizeof(float) : 0;
   p.total_bytes = p.S > 1 ? QMM_HEAD_BYTES + p.part_bytes : 0;
   p.use = true;
   return p;

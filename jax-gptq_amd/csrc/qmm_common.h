@@ -46,6 +46,10 @@ constexpr int QMM_MAX_COUNTERS = QMM_COUNTER_BYTES / 4;
 // at fixed offsets, whatever the shape, so that calls of different shapes can share one buffer.
 constexpr int QMM_ACC_BYTES = 4 << 20;
 constexpr int QMM_HEAD_BYTES = QMM_COUNTER_BYTES + QMM_ACC_BYTES;
+// Split-K sums through acc64: a contribution is value * 2^QD_FRAC in fixed point (a value beyond +-65536 or
+// not finite adds QD_POISON instead) << 8 | 1; the low byte of the word counts the contributions.
+constexpr int QD_FRAC = 28;
+constexpr long long QD_POISON = 3LL << 49;
 
 struct QmmWs {
   int32_t *counters;
