@@ -75,8 +75,12 @@ __host__ __device__ inline QmmWs qmm_ws(void *base_v, size_t x1_bytes) {
 // activations once per group of column tiles.  The last gx % 8 column tiles keep the plain order.
 __device__ __forceinline__ void qmm_tile_coords(int &tx, int &ty) {
   const int gx = gridDim.x, gy = gridDim.y;
-  if (gy == 1) {                   // one row of tiles: the order below is the identity, without its divisions
-    tx = blockIdx.x;
+  if (gy == 1) {
+    // One row of tiles: XCD j (workgroup ids j, j + 8, ...) takes a contiguous range of column tiles, so that a
+    // cache line that two neighbouring tiles share (rows that do not start on line boundaries) is fetched into
+    // one L2, not two.
+    const int j = blockIdx.x & 7, k = blockIdx.x >> 3, q = gx >> 3, rem = gx & 7;
+    tx = j * q + min(j, rem) + k;
     ty = 0;
     return;
   }
