@@ -38,7 +38,13 @@ __global__ __launch_bounds__(256, (RB == 1 ? 2 : 1)) void qmm_fwd_reg_kernel(con
                                                           int S, int steps_per_split, int group_size,
                                                           unsigned long long *acc64) {
   constexpr bool BF = Act<TX>::BF && !GROUPED;      // grouped: the fp16 form of the dequantisation for both types
-  constexpr int SCHED = RB == 4 ? 4 : 0;         // vector instructions between two MFMAs of the main loop (0: compiler's order)
+  // vector instructions between two MFMAs of the main loop (0: compiler's order)
+  constexpr int SCHED = RB == 4 ? 4 : 0;
+  // 128-row tiles: 256 accumulation registers hold the 8 x 8 product tiles, the row-sum tiles live in vector
+  // registers, and every MFMA accumulates in place (Act::mma_acc)
+  constexpr bool TIED = RB == 8;
+  constexpr int RBT = RB > 4 ? 4 : RB;           // row blocks per pass of the final reduction (LDS: 36 KB each)
+  constexpr int NH = RB / RBT;                   // passes
   constexpr int NL = BITS == 4 ? 4 : 8;          // packed rows per lane and k-step
   constexpr int PR = 4 * NL;                     // packed rows per k-step
   extern __shared__ __attribute__((aligned(16))) float rg_lds[];   // [4 wavefronts][RB][RG_NT][64 lanes][4]
@@ -206,23 +212,96 @@ __global__ __launch_bounds__(256, (RB == 1 ? 2 : 1)) void qmm_fwd_reg_kernel(con
       }
       const uint4 b = make_uint4(r4[0], r4[1], r4[2], r4[3]);
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) acc[rb][t8] = Act<TX>::mma(a[rb], b, acc[rb][t8]);
+      for (int rb = 0; rb < RB; ++rb) {
+        if constexpr (TIED) Act<TX>::mma_acc(acc[rb][t8], a[rb], b);
+        else acc[rb][t8] = Act<TX>::mma(a[rb], b, acc[rb][t8]);
+      }
     }
     if constexpr (!GROUPED) {
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) acc[rb][8] = Act<TX>::mma(a[rb], ones, acc[rb][8]);
+      for (int rb = 0; rb < RB; ++rb) {
+        if constexpr (TIED) Act<TX>::mma_accv(acc[rb][8], a[rb], ones);
+        else acc[rb][8] = Act<TX>::mma(a[rb], ones, acc[rb][8]);
+      }
+    }
+  };
+  // ---- 128-row tiles, per-channel parameters: the k-step in software-pipelined form.  The in-place MFMAs are
+  // inline asm, which the scheduler does not move; so the source order is the issue order: after every second
+  // MFMA of a tile the three vector instructions that build one operand register of the NEXT tile, and under the
+  // row-sum tile's MFMAs the first tile of the next k-step, whose weights are in the other ring slot.
+  auto dq_reg = [&](const uint2 (&w)[NL], int t8, int i) __attribute__((always_inline)) -> uint32_t {
+    const uint32_t tb = (uint32_t)(t8 & 3);
+    if constexpr (BITS == 4) {
+      const uint32_t sel = BF ? (0x0c0c0c00u | tb) : (0x0c000c00u | tb | (tb << 16));
+      const uint32_t pb = __builtin_amdgcn_perm(0u, t8 < 4 ? w[i].x : w[i].y, sel);
+      if (BF) return (((pb << 12) | pb) & mask) | cexp;
+      const uint32_t v = (pb & mask) | cexp;
+      const half2_t d = __builtin_bit_cast(half2_t, v) * unscale + __builtin_bit_cast(half2_t, zc[t8]);
+      return __builtin_bit_cast(uint32_t, d);
+    } else {
+      const uint32_t wa = t8 < 4 ? w[2 * i].x : w[2 * i].y, wb = t8 < 4 ? w[2 * i + 1].x : w[2 * i + 1].y;
+      if constexpr (BF) {
+        typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
+        typedef float f2_t __attribute__((ext_vector_type(2)));
+        const float fa = (float)((wa >> (8 * tb)) & 0xFFu) - zi8[t8];
+        const float fb = (float)((wb >> (8 * tb)) & 0xFFu) - zi8[t8];
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f2_t{fa, fb}, bf2_t));
+      } else {
+        const uint32_t pb = __builtin_amdgcn_perm(wb, wa, 0x0c000c00u | ((4u + tb) << 16) | tb);
+        const half2_t d = __builtin_bit_cast(half2_t, pb | cexp) + __builtin_bit_cast(half2_t, zc[t8]);
+        return __builtin_bit_cast(uint32_t, d);
+      }
+    }
+  };
+  constexpr bool PIPE = TIED && !GROUPED && !RAGGED;     // (the ragged form has no registers left for it)
+  uint32_t bcarry[4] = {0u, 0u, 0u, 0u};         // tile 0 of the k-step about to be multiplied
+  auto shifted = [&](int slot, uint2 (&w)[NL]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < NL; ++i) w[i] = RAGGED ? rg_shr_bytes(wr[slot][i], wshift) : wr[slot][i];
+  };
+  auto step_pipe = [&](int slot, int next_slot) __attribute__((always_inline)) {
+    uint2 w[NL];
+    shifted(slot, w);
+    uint32_t bc[4] = {bcarry[0], bcarry[1], bcarry[2], bcarry[3]};
+#pragma unroll
+    for (int t8 = 0; t8 < 8; ++t8) {
+      const uint4 b = make_uint4(bc[0], bc[1], bc[2], bc[3]);
+      uint32_t nx[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        Act<TX>::mma_acc(acc[rb][t8], aq[slot][rb], b);
+        if (t8 < 7 && (rb & 1)) nx[rb >> 1] = dq_reg(w, t8 + 1, rb >> 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) bc[i] = nx[i];
+    }
+    uint2 wn[NL];
+    shifted(next_slot, wn);
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      Act<TX>::mma_accv(acc[rb][8], aq[slot][rb], ones);
+      if (rb & 1) bcarry[rb >> 1] = dq_reg(wn, 0, rb >> 1);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
   const std::integral_constant<bool, false> plain{};
   const std::integral_constant<bool, true> tail{};
   int s0 = 0;
+  if constexpr (PIPE) {
+    uint2 w0[NL];
+    shifted(0, w0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) bcarry[i] = dq_reg(w0, 0, i);
+  }
   for (; s0 + RING <= iters_full; s0 += RING) {
 #pragma unroll
     for (int u = 0; u < RING; ++u) {
-      compute(u, plain);
+      if constexpr (PIPE) step_pipe(u, (u + 1) % RING);
+      else compute(u, plain);
       // (16-row tiles: nothing is fetched for k-steps past this wavefront's last; wave-uniform.  64-row tiles keep
       // one basic block per k-step for the instruction order below, and re-read their last k-step instead)
-      if (SCHED != 0 || s0 + u + RING < iters) load_step(u, s0 + u + RING);
+      if (SCHED != 0 || PIPE || s0 + u + RING < iters) load_step(u, s0 + u + RING);
       // One wavefront per SIMD issues in order: an MFMA occupies the matrix pipe for four passes, during
       // which the wavefront can issue only what stands behind it in program order and does not depend on it.
       // So the dequantisation of the next tile goes between the MFMAs of this one: one MFMA, then a few
@@ -240,7 +319,10 @@ __global__ __launch_bounds__(256, (RB == 1 ? 2 : 1)) void qmm_fwd_reg_kernel(con
   // at most RING - 1 full k-steps left, all of them loaded; then the ragged one
 #pragma unroll
   for (int u = 0; u < RING - 1; ++u)
-    if (s0 + u < iters_full) compute(u, plain);
+    if (s0 + u < iters_full) {
+      if constexpr (PIPE) step_pipe(u, u + 1);
+      else compute(u, plain);
+    }
   if (has_tail) {
     const int slot = iters_full - s0;            // 0 .. RING - 1
 #pragma unroll
@@ -248,104 +330,114 @@ __global__ __launch_bounds__(256, (RB == 1 ? 2 : 1)) void qmm_fwd_reg_kernel(con
       if (u == slot) compute(u, tail);
   }
 
+  if constexpr (TIED) mma_drain();
   // scale and zero point of this lane's channels, in flight while the tiles are summed
   float sc[8], zf[8];
   if constexpr (!GROUPED) {
     rg_params8(scale, zs_dtype, col, C, sc);
     rg_params8(zero, zs_dtype, col, C, zf);
   }
-  floatx4 sum[RG_NT];
-  const int tile = ty * gridDim.x + tx;
   // acc64 (16-row tiles only): every split finishes its own outputs and adds them to the cells
   const bool atom = RB == 1 && acc64 != nullptr && S > 1;
-  if (!rg_reduce<RB>(acc, sum, rg_lds, &s_flag, part, counters, tile, split, atom ? 1 : S)) return;
-  // sum[t8][r] = sum_k x[m][k] (code - zi)[k][col + t8] (bf16, 4-bit: code + 128), sum[8][r] = sum_k x[m][k],
-  // m = m0 + 16 rb + 4 g + r
-  if (!col_ok && !atom) return;
-  const int rb = wk;                             // rg_reduce returned true: wk < RB
+  // One pass of the reduction per four row blocks (a 128-row tile: two passes, each with its own arrival
+  // counter and partial tiles, as if it were two 64-row tiles).
+  auto finish = [&](auto hc) __attribute__((always_inline)) {
+    constexpr int H = decltype(hc)::value;
+    floatx4 sum[RG_NT];
+    const int tile = (ty * NH + H) * gridDim.x + tx;
+    if (!rg_reduce<RBT, RB, H * RBT>(acc, sum, rg_lds, &s_flag, part, counters, tile, split, atom ? 1 : S)) return;
+    // sum[t8][r] = sum_k x[m][k] (code - zi)[k][col + t8] (bf16, 4-bit: code + 128), sum[8][r] = sum_k x[m][k],
+    // m = m0 + 16 (H RBT + rb) + 4 g + r
+    if (!col_ok && !atom) return;
+    const int rb = H * RBT + wk;                   // rg_reduce returned true: wk < RBT
+    // (first use of the parameters: after the reduction's waits)
+    float sca[8], zfa[8];
 #pragma unroll
-  for (int t8 = 0; t8 < 8; ++t8) {
-    if (GROUPED) {
-      sc[t8] = 1.f;
-      zf[t8] = 0.f;
-    } else {
-      zf[t8] = (BF && BITS == 4) ? 128.f + zf[t8] : zf[t8] - fminf(fmaxf(rintf(zf[t8]), -512.f), 512.f);
+    for (int t8 = 0; t8 < 8; ++t8) {
+      sca[t8] = GROUPED ? 1.f : sc[t8];
+      zfa[t8] = GROUPED ? 0.f
+                        : ((BF && BITS == 4) ? 128.f + zf[t8] : zf[t8] - fminf(fmaxf(rintf(zf[t8]), -512.f), 512.f));
     }
-  }
-  if constexpr (RB == 1) {
-    if (atom) {
-      // This wavefront's finished values go through the LDS (the other wavefronts are done with it) so that
-      // consecutive lanes hold consecutive channels: the memory side takes an atomic per 64-byte segment,
-      // not per lane.  Then two passes per eight rows, so that a lane's atomics are in flight together.  The
-      // word that comes back tells the last of the S contributions that it is the last, and gives it the
-      // complete sum: it rounds, stores the output and zeroes the cell.  Integer addition is exact and
-      // commutative: the result does not depend on the order of arrival.
-      float *tr = rg_lds;                                  // [16 rows][128 channels]
+    if constexpr (RB == 1) {
+      if (atom) {
+        // This wavefront's finished values go through the LDS (the other wavefronts are done with it) so that
+        // consecutive lanes hold consecutive channels: the memory side takes an atomic per 64-byte segment,
+        // not per lane.  Then two passes per eight rows, so that a lane's atomics are in flight together.  The
+        // word that comes back tells the last of the S contributions that it is the last, and gives it the
+        // complete sum: it rounds, stores the output and zeroes the cell.  Integer addition is exact and
+        // commutative: the result does not depend on the order of arrival.
+        float *tr = rg_lds;                                  // [16 rows][128 channels]
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float rs = sum[8][r];
-        float pv[8];
+        for (int r = 0; r < 4; ++r) {
+          const float rs = sum[8][r];
+          float pv[8];
 #pragma unroll
-        for (int t8 = 0; t8 < 8; ++t8) pv[t8] = sc[t8] * (sum[t8][r] - zf[t8] * rs);
-        float *dst = tr + (4 * g + r) * RG_BN + 8 * l16;
-        *reinterpret_cast<float4 *>(dst) = make_float4(pv[0], pv[1], pv[2], pv[3]);
-        *reinterpret_cast<float4 *>(dst + 4) = make_float4(pv[4], pv[5], pv[6], pv[7]);
-      }
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // one wavefront: its LDS accesses complete in order
-#pragma unroll
-      for (int mh = 0; mh < 2; ++mh) {
-        if (8 * mh >= M - m0) break;
-        unsigned long long old[16], word[16];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int mr = 8 * mh + (i >> 1), c = 64 * (i & 1) + lane;
-          old[i] = word[i] = 0ull;
-          if (m0 + mr >= M || nbase + c >= C) continue;
-          const float pv = tr[mr * RG_BN + c];
-          const bool ok = fabsf(pv) <= 65536.f;                       // false for NaN, too
-          const long long fx = ok ? __float2ll_rn(pv * (float)(1 << QD_FRAC)) : QD_POISON;
-          word[i] = ((unsigned long long)fx << 8) + 1ull;
-          old[i] = atomicAdd(acc64 + (int64_t)(m0 + mr) * C + nbase + c, word[i]);
+          for (int t8 = 0; t8 < 8; ++t8) pv[t8] = sca[t8] * (sum[t8][r] - zfa[t8] * rs);
+          float *dst = tr + (4 * g + r) * RG_BN + 8 * l16;
+          *reinterpret_cast<float4 *>(dst) = make_float4(pv[0], pv[1], pv[2], pv[3]);
+          *reinterpret_cast<float4 *>(dst + 4) = make_float4(pv[4], pv[5], pv[6], pv[7]);
         }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // one wavefront: its LDS accesses complete in order
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int mr = 8 * mh + (i >> 1), c = 64 * (i & 1) + lane;
-          const unsigned long long total = old[i] + word[i];
-          if ((int)(total & 255ull) != S) continue;                   // (also the lanes that added nothing: 0 != S)
-          const long long fsum = (long long)total >> 8;
-          const bool fine = fsum <= (1LL << 49) && fsum >= -(1LL << 49);
-          const float res = fine ? (float)fsum * (1.f / (float)(1 << QD_FRAC)) : __builtin_nanf("");
-          out[(int64_t)(m0 + mr) * C + nbase + c] = Act<TX>::out(res);
-          __hip_atomic_store(acc64 + (int64_t)(m0 + mr) * C + nbase + c, 0ull, __ATOMIC_RELAXED,
-                             __HIP_MEMORY_SCOPE_AGENT);
+        for (int mh = 0; mh < 2; ++mh) {
+          if (8 * mh >= M - m0) break;
+          unsigned long long old[16], word[16];
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int mr = 8 * mh + (i >> 1), c = 64 * (i & 1) + lane;
+            old[i] = word[i] = 0ull;
+            if (m0 + mr >= M || nbase + c >= C) continue;
+            const float pv = tr[mr * RG_BN + c];
+            const bool ok = fabsf(pv) <= 65536.f;                       // false for NaN, too
+            const long long fx = ok ? __float2ll_rn(pv * (float)(1 << QD_FRAC)) : QD_POISON;
+            word[i] = ((unsigned long long)fx << 8) + 1ull;
+            old[i] = atomicAdd(acc64 + (int64_t)(m0 + mr) * C + nbase + c, word[i]);
+          }
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int mr = 8 * mh + (i >> 1), c = 64 * (i & 1) + lane;
+            const unsigned long long total = old[i] + word[i];
+            if ((int)(total & 255ull) != S) continue;                   // (also the lanes that added nothing: 0 != S)
+            const long long fsum = (long long)total >> 8;
+            const bool fine = fsum <= (1LL << 49) && fsum >= -(1LL << 49);
+            const float res = fine ? (float)fsum * (1.f / (float)(1 << QD_FRAC)) : __builtin_nanf("");
+            out[(int64_t)(m0 + mr) * C + nbase + c] = Act<TX>::out(res);
+            __hip_atomic_store(acc64 + (int64_t)(m0 + mr) * C + nbase + c, 0ull, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+          }
         }
+        return;
       }
-      return;
     }
-  }
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int m = m0 + 16 * rb + 4 * g + r;
-    if (m >= M) continue;
-    const float rs = sum[8][r];
-    TX o[8];
+    for (int r = 0; r < 4; ++r) {
+      const int m = m0 + 16 * rb + 4 * g + r;
+      if (m >= M) continue;
+      const float rs = sum[8][r];
+      TX o[8];
 #pragma unroll
-    for (int t8 = 0; t8 < 8; ++t8) o[t8] = Act<TX>::out(sc[t8] * (sum[t8][r] - zf[t8] * rs));
-    TX *dst = out + (int64_t)m * C + col;
-    if (RAGGED) {
+      for (int t8 = 0; t8 < 8; ++t8) o[t8] = Act<TX>::out(sca[t8] * (sum[t8][r] - zfa[t8] * rs));
+      TX *dst = out + (int64_t)m * C + col;
+      if (RAGGED) {
 #pragma unroll
-      for (int t8 = 0; t8 < 8; ++t8)
-        if (col + t8 < C) dst[t8] = o[t8];
-    } else {
-      *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(o);
+        for (int t8 = 0; t8 < 8; ++t8)
+          if (col + t8 < C) dst[t8] = o[t8];
+      } else {
+        *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(o);
+      }
     }
+  };
+  finish(std::integral_constant<int, 0>{});
+  if constexpr (NH == 2) {
+    __syncthreads();                                 // the first pass's sums have been read
+    finish(std::integral_constant<int, 1>{});
   }
 }
 
 template <int BITS, int RB, int RING, bool RAGGED, typename TX, bool GROUPED>
 int launch_inst(hipStream_t st, const RegPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
                 int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *wsp, int group_size) {
-  constexpr size_t lds = (size_t)4 * RB * RG_NT * RG_TILE_FLOATS * sizeof(float);
+  constexpr size_t lds = (size_t)4 * (RB > 4 ? 4 : RB) * RG_NT * RG_TILE_FLOATS * sizeof(float);
   auto kern = qmm_fwd_reg_kernel<BITS, RB, RING, RAGGED, TX, GROUPED>;
   if (lds > 64 * 1024 && !gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), (int)lds)) return GPTQ_HIP_ELAUNCH;
   const int64_t K = BITS == 4 ? 2 * R : R;
@@ -378,6 +470,10 @@ int launch_bx(hipStream_t st, const RegPlan &p, const void *x, int64_t M, const 
   return launch_inst<BITS, RB, RING, RAGGED, TX, GROUPED>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size)
   if (group_size > 0) {
     // the group's parameters ride in the ring: shorter rings
+    if (p.rb == 8) {
+      if (p.ragged) GPTQ_REG(8, 2, true, true);
+      GPTQ_REG(8, 2, false, true);
+    }
     if (p.rb == 4) {
       if (p.ragged) GPTQ_REG(4, 2, true, true);
       GPTQ_REG(4, 2, false, true);
@@ -385,7 +481,12 @@ int launch_bx(hipStream_t st, const RegPlan &p, const void *x, int64_t M, const 
     if (p.ragged) GPTQ_REG(1, 3, true, true);
     GPTQ_REG(1, 3, false, true);
   }
-  // a ring of three k-steps for 64-row tiles (registers), of six for the 16-row tiles of the decode case
+  // a ring of two k-steps for 128-row tiles, of three for 64-row tiles (registers), of six for the 16-row tiles
+  // of the decode case
+  if (p.rb == 8) {
+    if (p.ragged) GPTQ_REG(8, 2, true, false);
+    GPTQ_REG(8, 3, false, false);
+  }
   if (p.rb == 4) {
     if (p.ragged) GPTQ_REG(4, 3, true, false);
     GPTQ_REG(4, 3, false, false);
@@ -404,17 +505,20 @@ RegPlan reg_fwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned) {
   const int64_t K = bits == 4 ? 2 * R : R;
   if ((bits != 4 && bits != 8) || M < 1 || C < 8 || K < 8 || R >= (1LL << 30) || C >= (1LL << 30)) return p;
   p.bits = bits;
-  p.rb = M <= 16 ? 1 : 4;
+  // 128-row tiles (a weight tile is dequantised once for twice the rows; their reduction takes two passes) where
+  // they alone fill most of the chip, 64-row tiles otherwise
+  p.rb = M <= 16 ? 1 : ((M > 64 && ceil_div64(C, RG_BN) * ceil_div64(M, 128) >= 160) ? 8 : 4);
   p.ragged = !aligned || C % 8 != 0 || K % 8 != 0;
   const int64_t tiles_x = ceil_div64(C, RG_BN);
-  if (tiles_x > QMM_MAX_COUNTERS) return p;
+  const int64_t nh = p.rb == 8 ? 2 : 1;          // arrival counters per tile (a 128-row tile is reduced in two passes)
+  if (tiles_x * nh > QMM_MAX_COUNTERS) return p;
   int64_t tiles_y = ceil_div64(M, 16 * p.rb);
-  if (tiles_y > QMM_MAX_COUNTERS / tiles_x) tiles_y = QMM_MAX_COUNTERS / tiles_x;    // further rows: further launches
+  if (tiles_y > QMM_MAX_COUNTERS / (tiles_x * nh)) tiles_y = QMM_MAX_COUNTERS / (tiles_x * nh);    // further rows: further launches
   p.tiles = tiles_x * tiles_y;
   const int64_t T = ceil_div64(K, 32);
-  // workgroups wanted: one per CU for 64-row tiles (their registers allow no more), two for 16-row tiles;
-  // every wavefront of a split keeps at least four k-steps
-  const int64_t want = p.rb == 4 ? 256 : 512;
+  // workgroups wanted: one per CU for 64- and 128-row tiles (their registers allow no more), two for 16-row
+  // tiles; every wavefront of a split keeps at least four k-steps
+  const int64_t want = p.rb == 1 ? 512 : 256;
   int64_t S = 1;
   if (p.tiles < want) {
     S = want / p.tiles;

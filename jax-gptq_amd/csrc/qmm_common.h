@@ -9,6 +9,7 @@ typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 // 16-bit activation types of the MFMA kernels
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 template <typename TX> struct Act;
 template <> struct Act<__half> {
   static constexpr bool BF = false;
@@ -17,6 +18,20 @@ template <> struct Act<__half> {
   static __device__ __forceinline__ floatx4 mma(const uint4 &a, const uint4 &b, floatx4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
                                                   __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+  }
+  // The same MFMA with the accumulator tied in place: `acc` in accumulation registers, `accv` in vector
+  // registers.  For kernels whose accumulators fill the accumulation file: the compiler's own form of the
+  // instruction may write a different register than it reads, which then costs a copy per tile and k-step.
+  // (Inline asm is outside the compiler's hazard handling.  An MFMA must not read an operand register within two
+  // wait states of the vector instruction that wrote it, hence the s_nop in front; callers keep the reads of
+  // the result away from the last MFMA, see mma_drain.)
+  static __device__ __forceinline__ void mma_acc(floatx4 &c, const uint4 &a, const uint4 &b) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0"
+                 : "+a"(c) : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)));
+  }
+  static __device__ __forceinline__ void mma_accv(floatx4 &c, const uint4 &a, const uint4 &b) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0"
+                 : "+v"(c) : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)));
   }
   static __device__ __forceinline__ __half out(float v) { return __float2half_rn(v); }
 };
@@ -29,8 +44,19 @@ template <> struct Act<__hip_bfloat16> {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, a),
                                                    __builtin_bit_cast(bf8_t, b), c, 0, 0, 0);
   }
+  static __device__ __forceinline__ void mma_acc(floatx4 &c, const uint4 &a, const uint4 &b) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                 : "+a"(c) : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)));
+  }
+  static __device__ __forceinline__ void mma_accv(floatx4 &c, const uint4 &a, const uint4 &b) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                 : "+v"(c) : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)));
+  }
   static __device__ __forceinline__ __hip_bfloat16 out(float v) { return __float2bfloat16(v); }
 };
+// After the last mma_acc / mma_accv and before anything reads their accumulators: an MFMA's result is
+// written several passes after its issue, and nothing but wait states keeps a read from overtaking it.
+__device__ __forceinline__ void mma_drain() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 
 // Workspace layout (only touched when the K range is split over S > 1 workgroups):
 //   [counters: QMM_COUNTER_BYTES, one int32 per (m-chunk, strip), zero between calls; the

@@ -143,8 +143,10 @@ __device__ __forceinline__ floatx4 rg_load_part_issue(const float *p) {
 //   scope, executed at the memory side); the last workgroup of the tile reads all S partials with
 //   agent-scope loads and adds them in split order, so the result does not depend on the arrival order,
 //   and leaves the counter at zero for the next call.
-template <int RB>
-__device__ __forceinline__ bool rg_reduce(floatx4 (&acc)[RB][RG_NT], floatx4 (&sum)[RG_NT], float *lds,
+// (NRB, R0: the wavefront holds NRB row blocks, of which this call sums the RB blocks R0 .. R0 + RB - 1; a
+// 128-row tile goes through as two calls of four row blocks, with a barrier between them.)
+template <int RB, int NRB = RB, int R0 = 0>
+__device__ __forceinline__ bool rg_reduce(floatx4 (&acc)[NRB][RG_NT], floatx4 (&sum)[RG_NT], float *lds,
                                           int *s_flag, float *part, int32_t *counters, int tile, int split,
                                           int S) {
   const int tid = threadIdx.x, lane = tid & 63, wk = tid >> 6;
@@ -152,7 +154,7 @@ __device__ __forceinline__ bool rg_reduce(floatx4 (&acc)[RB][RG_NT], floatx4 (&s
   for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
     for (int t = 0; t < RG_NT; ++t)
-      *reinterpret_cast<floatx4 *>(lds + (((wk * RB + rb) * RG_NT + t) * 64 + lane) * 4) = acc[rb][t];
+      *reinterpret_cast<floatx4 *>(lds + (((wk * RB + rb) * RG_NT + t) * 64 + lane) * 4) = acc[R0 + rb][t];
   __syncthreads();
   const bool owner = wk < RB;
   const int rb_own = owner ? wk : 0;
