@@ -27,15 +27,40 @@ def _case(rng):
     return bits, M, K, N, tr, xdt, zs, group, int(rng.integers(0, 2))
 
 
+def _wide_case(rng):
+    """More than 64 rows against 160 or more column tiles of 128 channels: the shapes that run on 128-row tiles
+    (aligned, ragged and grouped instantiations; k-steps that end inside a 32-wide step)."""
+    bits = int(rng.choice([4, 8]))
+    M = int(rng.choice([65, 128, 129, 200, 257]))
+    K = int(rng.choice([32, 40, 64, 72, 96, 160, 200]))
+    N = int(rng.choice([20480, 20488, 20490, 24001, 50257]))
+    xdt = str(rng.choice(["float16", "bfloat16", "float32"]))
+    zs = str(rng.choice(["float32", "float16", "bfloat16"]))
+    group = 0
+    if rng.random() < 0.3:
+        cands = [g for g in (32, 64, 96) if K % g == 0]
+        if cands:
+            group = int(rng.choice(cands))
+    return bits, M, K, N, False, xdt, zs, group, int(rng.integers(0, 2))
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_qmatmul_random_cases_with_many_column_tiles(seed):
+    _run_cases(np.random.default_rng(2000 + seed), _wide_case, 14)
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_qmatmul_random_cases(seed):
+    _run_cases(np.random.default_rng(1000 + seed), _case, 25)
+
+
+def _run_cases(rng, make_case, count):
     import torch
     import jax_gptq_amd.gptq as G
     from jax_gptq_amd.op import quantized_matmul
-    rng = np.random.default_rng(1000 + seed)
     failures = []
-    for it in range(25):
-        bits, M, K, N, tr, xdt, zs, group, off = _case(rng)
+    for it in range(count):
+        bits, M, K, N, tr, xdt, zs, group, off = make_case(rng)
         top = 16 if bits == 4 else 256
         codes = rng.integers(0, top, (K, N)).astype(np.uint8)
         tdt = getattr(torch, zs)
