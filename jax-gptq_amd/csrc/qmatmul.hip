@@ -687,6 +687,16 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
   float *xs = red + (size_t)NW * MR * QSTRIP;   // [wave][2][16]
   if (g == 0) { xs[wave * 32 + l16] = se; xs[wave * 32 + 16 + l16] = so; }
   __syncthreads();
+  // the activation sums over the wavefronts, once per workgroup (read per output they were 2 NW broadcast
+  // reads for each of a thread's outputs: most of the LDS instructions of this phase)
+  float *xt = xs + NW * 32;                     // [2][16]
+  if (tid < 32) {
+    float a = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) a += xs[w * 32 + tid];
+    xt[tid] = a;
+  }
+  __syncthreads();
   // Two passes over this thread's outputs, so that its atomics are in flight together: a pass that used each
   // returned word at once would pay one round trip to the memory side per output.
   unsigned long long old[IT], word[IT];
@@ -698,13 +708,10 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
     live[it] = idx < ITEMS && m < mvalid && n < C;
     old[it] = word[it] = 0ull;
     if (!live[it]) continue;
-    float v = 0.f, e = 0.f, o = 0.f;
+    float v = 0.f;
+    const float e = xt[m], o = xt[16 + m];
 #pragma unroll
-    for (int w = 0; w < NW; ++w) {
-      v += red[(w * MR + m) * QSTRIP + qtile_pos(c)];
-      e += xs[w * 32 + m];
-      o += xs[w * 32 + 16 + m];
-    }
+    for (int w = 0; w < NW; ++w) v += red[(w * MR + m) * QSTRIP + qtile_pos(c)];
     const float r = BF ? (v - 128.f * (e + o)) - pz[it] * (e + o)
                        : (v - 1024.f * (e + o)) - pz[it] * (e + 16.f * o);
     const float pv = psc[it] * r;
@@ -885,7 +892,7 @@ DecPlan dec_plan(int64_t M, int64_t R, int64_t C) {
       p.total_bytes = p.S > 1 ? QMM_HEAD_BYTES + p.x1_bytes + p.part_bytes : 0;
     }
   }
-  p.lds_bytes = ((size_t)p.nw * p.mr * QSTRIP + (size_t)p.nw * 32) * sizeof(float);
+  p.lds_bytes = ((size_t)p.nw * p.mr * QSTRIP + (size_t)p.nw * 32 + 32) * sizeof(float);
   p.use = true;
   return p;
 }
