@@ -541,13 +541,26 @@ __global__ __launch_bounds__(256, 2) void qmm_fwd_stream_kernel(
 //    qmm_reduce_and_store (ATOM = false).
 constexpr int QD_MAX_SPLITS = 32;
 
-template <int NW, int KS, int MR, bool ATOM, bool LOOP, typename TZ, typename TX>
+//  * X32 (fp16 arithmetic, ATOM only): activations and result are fp32 in memory.  What the separate
+//    conversion kernels do around the other paths happens in here: the power of two that brings a row's
+//    largest finite magnitude into [2, 4) is either found by every workgroup itself (rowexp_in == nullptr:
+//    it reads the whole row, 16 KB of L2-resident data per row at K = 4096, which pays for one or two
+//    rows) or comes from x32_rowexp_kernel; the scaled activations of the workgroup's k range are rounded
+//    to fp16 as they are consumed, and the workgroup that completes an output rounds it to fp16, widens it
+//    and scales it back: the same arithmetic, bit for bit, without staging buffers and with one launch
+//    (M = 1: 16.8 -> 9.8 us) or two (more rows) instead of three.
+template <int NW, int KS, int MR, bool ATOM, bool LOOP, typename TZ, typename TX, bool X32 = false>
 __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
-    const TX *x, int M, int K, const uint8_t *pk, int R, int C, const TZ *zero, const TZ *scale,
-    TX *out, QmmWs ws, int S, int rows_per_split) {
+    const std::conditional_t<X32, float, TX> *x, int M, int K, const uint8_t *pk, int R, int C, const TZ *zero,
+    const TZ *scale, std::conditional_t<X32, float, TX> *out, QmmWs ws, int S, int rows_per_split,
+    const int32_t *rowexp_in) {
   constexpr bool BF = Act<TX>::BF;
+  static_assert(!X32 || (ATOM && !BF), "fp32 rows: fp16 arithmetic and the atomic sum only");
+  typedef std::conditional_t<X32, float, TX> XT;
   extern __shared__ float red[];   // [NW][MR][256] partial tiles, then [NW][2][16] x sums
   __shared__ int s_last;
+  __shared__ float s_rowmax[X32 ? NW : 1][16];
+  __shared__ int s_rowexp[16];
   // every kernel argument in registers before the first address is formed (left to itself the compiler
   // fetches them one by one where they are first used, and waits for each)
   asm volatile("" ::"s"(x), "s"(pk), "s"(zero), "s"(scale), "s"(out), "s"(ws.acc64), "s"(ws.counters), "s"(ws.part),
@@ -569,14 +582,15 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
   // k-step enters with zero activations.  LOOP: a ring of KS k-steps that is refilled as it is consumed,
   // for matrices beyond what the chip holds in flight; otherwise all KS k-steps of the range are issued
   // at once, and a wavefront skips the k-steps that lie past its range altogether.
-  struct Step { uint4 d[4]; uint4 pr; };
+  struct Step { uint4 d[4]; uint4 pr; uint4 pr2; };      // pr2: the second half of an fp32 chunk (X32)
   const bool m_ok = l16 < mvalid;
-  const TX *xr = x + (int64_t)(m0 + (m_ok ? l16 : 0)) * K;
+  const XT *xr = x + (int64_t)(m0 + (m_ok ? l16 : 0)) * K;
   const int col0 = min(strip * QSTRIP + 16 * l16, C - 16);
   const uint8_t *wp = pk + col0;
   auto issue = [&](Step &st, int t) __attribute__((always_inline)) {
     const int rbase = r_begin + (t * NW + wave) * 16 + 4 * g;
     st.pr = *reinterpret_cast<const uint4 *>(xr + 2 * min(rbase, R - 4));
+    if (X32) st.pr2 = *reinterpret_cast<const uint4 *>(xr + 2 * min(rbase, R - 4) + 4);
     const uint8_t *row = wp + (int64_t)min(rbase, R - 4) * C;       // R % 4 == 0: four rows inside the matrix
 #pragma unroll
     for (int i = 0; i < 4; ++i) st.d[i] = *reinterpret_cast<const uint4 *>(row + (int64_t)i * C);
@@ -588,8 +602,21 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
 #pragma unroll
   for (int t = 0; t < 16; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
   float se = 0.f, so = 0.f;
+  int xe = 0;                                     // X32: exponent of this lane's row scale
   auto consume = [&](Step &st, int t) __attribute__((always_inline)) {
     uint4 pr = st.pr;
+    if constexpr (X32) {
+      // eight fp32 activations -> fp16 of the scaled row, round to nearest even
+      const uint32_t f[8] = {st.pr.x, st.pr.y, st.pr.z, st.pr.w, st.pr2.x, st.pr2.y, st.pr2.z, st.pr2.w};
+      uint32_t h[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const __half a = __float2half_rn(ldexpf(__builtin_bit_cast(float, f[2 * i]), -xe));
+        const __half b = __float2half_rn(ldexpf(__builtin_bit_cast(float, f[2 * i + 1]), -xe));
+        h[i] = (uint32_t)__builtin_bit_cast(uint16_t, a) | ((uint32_t)__builtin_bit_cast(uint16_t, b) << 16);
+      }
+      pr = make_uint4(h[0], h[1], h[2], h[3]);
+    }
     {
       const bool ok = m_ok && t < nsteps && r_begin + (t * NW + wave) * 16 + 4 * g < r_end;
       pr.x = ok ? pr.x : 0u;
@@ -638,6 +665,47 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
       psc[it] = to_f32(scale[n]);
     }
   }
+  if constexpr (X32) {
+    // the scale of every row of this workgroup: largest finite magnitude over all of K (K % 8 == 0, rows 32-byte
+    // aligned), under the weight loads
+    if (rowexp_in == nullptr) {
+      for (int m = 0; m < mvalid; ++m) {
+        const float *row = x + (int64_t)(m0 + m) * K;
+        float amax = 0.f;
+        for (int k = tid * 4; k < K; k += NT * 4) {
+          const float4 v = *reinterpret_cast<const float4 *>(row + k);
+          const float a4[4] = {fabsf(v.x), fabsf(v.y), fabsf(v.z), fabsf(v.w)};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) amax = (a4[i] <= 3.4028235e38f && a4[i] > amax) ? a4[i] : amax;   // not NaN, not infinity
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+        if (lane == 0) s_rowmax[wave][m] = amax;
+      }
+    }
+    __syncthreads();
+    if (tid < 16) {
+      if (rowexp_in != nullptr) {
+        s_rowexp[tid] = tid < mvalid ? rowexp_in[m0 + tid] : 0;
+      } else {
+        float a = 0.f;
+        if (tid < mvalid) {
+#pragma unroll
+          for (int w = 0; w < NW; ++w) a = fmaxf(a, s_rowmax[w][tid]);
+        }
+        int ex = 0;
+        (void)frexpf(a, &ex);                      // 2^(ex-1) <= a < 2^ex
+        s_rowexp[tid] = a > 0.f ? ex - 2 : 0;      // largest magnitude of the scaled row in [2, 4)
+      }
+    }
+    __syncthreads();
+    xe = s_rowexp[l16];
+  }
+  // rounds a finished output to the 16-bit type; fp32 rows: widened again and scaled back (exact)
+  auto store_out = [&](int m, int n, float v) __attribute__((always_inline)) {
+    if constexpr (X32) out[(int64_t)(m0 + m) * C + n] = ldexpf(__half2float(__float2half_rn(v)), s_rowexp[m]);
+    else out[(int64_t)(m0 + m) * C + n] = Act<TX>::out(v);
+  };
   // (without this the scheduler sinks the parameter loads below the wait for the weights, and their latency
   // is paid after the last k-step instead of under it)
   __builtin_amdgcn_sched_barrier(0);
@@ -679,7 +747,7 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
             make_float4(acc[4 * q][r], acc[4 * q + 1][r], acc[4 * q + 2][r], acc[4 * q + 3][r]);
     }
   }
-  if (!ATOM) {
+  if constexpr (!ATOM) {
     qmm_reduce_and_store<IT>(red, &s_last, NW, MR, mvalid, strip, split, m0, M, C, S, zero, scale, out, ws,
                              se, so);
     return;
@@ -716,7 +784,7 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
                        : (v - 1024.f * (e + o)) - pz[it] * (e + 16.f * o);
     const float pv = psc[it] * r;
     if (S == 1) {
-      out[(int64_t)(m0 + m) * C + n] = Act<TX>::out(pv);
+      store_out(m, n, pv);
       live[it] = false;
       continue;
     }
@@ -734,7 +802,7 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
     const long long sum = (long long)total >> 8;
     const bool fine = sum <= (1LL << 49) && sum >= -(1LL << 49);
     const float res = fine ? (float)sum * (1.f / (float)(1 << QD_FRAC)) : __builtin_nanf("");
-    out[(int64_t)(m0 + m) * C + n] = Act<TX>::out(res);
+    store_out(m, n, res);
     __hip_atomic_store(ws.acc64 + (int64_t)(m0 + m) * C + n, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
@@ -897,18 +965,46 @@ DecPlan dec_plan(int64_t M, int64_t R, int64_t C) {
   return p;
 }
 
-template <int NW, int KS, int MR, bool ATOM, bool LOOP, typename TZ, typename TX>
+template <int NW, int KS, int MR, bool ATOM, bool LOOP, typename TZ, typename TX, bool X32 = false>
 int launch_dec_inst(hipStream_t st, const DecPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
-                    int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
-  auto kern = qmm_fwd_dec_kernel<NW, KS, MR, ATOM, LOOP, TZ, TX>;
+                    int64_t C, const void *zero, const void *scale, void *out, void *wsp,
+                    const int32_t *rowexp = nullptr) {
+  typedef std::conditional_t<X32, float, TX> XT;
+  auto kern = qmm_fwd_dec_kernel<NW, KS, MR, ATOM, LOOP, TZ, TX, X32>;
   if (p.lds_bytes > 48 * 1024 && !gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), (int)p.lds_bytes))
     return GPTQ_HIP_ELAUNCH;
   const QmmWs ws = qmm_ws(wsp, p.x1_bytes);
   hipLaunchKernelGGL(kern, dim3((unsigned)p.strips, (unsigned)p.S, 1), dim3(NW * 64), p.lds_bytes, st,
-                     (const TX *)x, (int)M, (int)(2 * R), pk, (int)R, (int)C, (const TZ *)zero,
-                     (const TZ *)scale, (TX *)out, ws, p.S, p.rows);
+                     (const XT *)x, (int)M, (int)(2 * R), pk, (int)R, (int)C, (const TZ *)zero,
+                     (const TZ *)scale, (XT *)out, ws, p.S, p.rows, rowexp);
   GPTQ_CHECK_LAUNCH();
   return GPTQ_HIP_OK;
+}
+
+// fp32 rows in, fp32 rows out, fp16 arithmetic (plans with the atomic sum only); rowexp: the rows' scale
+// exponents from x32_rowexp_kernel, or nullptr (the kernel finds them itself: one or two rows)
+template <typename TZ>
+int launch_dec_x32(hipStream_t st, const DecPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
+                   int64_t C, const void *zero, const void *scale, void *out, void *wsp, const int32_t *rowexp) {
+#define GPTQ_DEC32(NW, KS, MR, LOOP) \
+  return launch_dec_inst<NW, KS, MR, true, LOOP, TZ, __half, true>(st, p, x, M, pk, R, C, zero, scale, out, wsp, \
+                                                                   rowexp)
+  if (!p.atom) return GPTQ_HIP_EINVAL;
+  if (p.mr == 16) {
+    if (p.loop) GPTQ_DEC32(8, 4, 16, true);
+    GPTQ_DEC32(8, 4, 16, false);
+  }
+  if (p.mr == 1) {
+    if (p.loop) GPTQ_DEC32(16, 2, 1, true);
+    if (p.nw == 16) GPTQ_DEC32(16, 2, 1, false);
+    if (p.ks == 1) GPTQ_DEC32(8, 1, 1, false);
+    GPTQ_DEC32(8, 2, 1, false);
+  }
+  if (p.loop) GPTQ_DEC32(16, 2, 4, true);
+  if (p.nw == 16) GPTQ_DEC32(16, 2, 4, false);
+  if (p.ks == 1) GPTQ_DEC32(8, 1, 4, false);
+  GPTQ_DEC32(8, 2, 4, false);
+#undef GPTQ_DEC32
 }
 
 template <typename TZ, typename TX>
@@ -1735,6 +1831,26 @@ __global__ __launch_bounds__(256) void x32_to_f16_rows_kernel(const float *x, in
   if (threadIdx.x == 0) rowexp[m] = e;
 }
 
+// only the exponent of a row's scale (for the decode kernel that converts in place)
+__global__ __launch_bounds__(256) void x32_rowexp_kernel(const float *x, int64_t kin, int32_t *rowexp) {
+  const float *xr = x + (int64_t)blockIdx.x * kin;
+  __shared__ float smax[4];
+  float amax = 0.f;
+  for (int64_t k = threadIdx.x; k < kin; k += 256) {
+    const float a = fabsf(xr[k]);
+    amax = (a <= 3.4028235e38f && a > amax) ? a : amax;   // NaN and infinity do not set the scale
+  }
+  for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+  if ((threadIdx.x & 63) == 0) smax[threadIdx.x >> 6] = amax;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    amax = fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3]));
+    int ex = 0;
+    (void)frexpf(amax, &ex);
+    rowexp[blockIdx.x] = amax > 0.f ? ex - 2 : 0;
+  }
+}
+
 __global__ __launch_bounds__(256) void f16_rows_to_f32_kernel(const __half *o16, int64_t nout,
                                                               const int32_t *rowexp, float *out) {
   const int64_t m = blockIdx.y;
@@ -1833,6 +1949,28 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
       int32_t *rowexp = reinterpret_cast<int32_t *>(base + fp.exp_off);
       const int64_t Kl = bits == 4 ? 2 * R : R;
       const int64_t kin = transpose_b ? C : Kl, nout = transpose_b ? Kl : C;
+      // up to 16 rows on the decode kernel's shapes: converted inside that kernel (no staging, one launch)
+      if (bits == 4 && !transpose_b && group_size == 0 && M <= 16 && R % 4 == 0 && C % 16 == 0 &&
+          ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(packed)) & 15) == 0 &&
+          (reinterpret_cast<uintptr_t>(out) & 3) == 0) {
+        const DecPlan dp = dec_plan(M, R, C);
+        if (dp.use && dp.atom && (dp.total_bytes == 0 || (ws && ws_bytes >= dp.total_bytes))) {
+          const int32_t *re = nullptr;
+          if (M > 2) {            // beyond two rows every workgroup's own pass over the rows costs more than a launch
+            hipLaunchKernelGGL(x32_rowexp_kernel, dim3((unsigned)M), dim3(256), 0, st,
+                               reinterpret_cast<const float *>(x), kin, rowexp);
+            GPTQ_CHECK_LAUNCH();
+            re = rowexp;
+          }
+          switch (zs_dtype) {
+            case GPTQ_HIP_F32: return launch_dec_x32<float>(st, dp, x, M, packed, R, C, zero, scale, out, ws, re);
+            case GPTQ_HIP_F16: return launch_dec_x32<__half>(st, dp, x, M, packed, R, C, zero, scale, out, ws, re);
+            case GPTQ_HIP_BF16:
+              return launch_dec_x32<__hip_bfloat16>(st, dp, x, M, packed, R, C, zero, scale, out, ws, re);
+            default: return GPTQ_HIP_EDTYPE;
+          }
+        }
+      }
       for (int64_t r0 = 0; r0 < M; r0 += fp.mc) {
         const int64_t mm = M - r0 < fp.mc ? M - r0 : fp.mc;
         hipLaunchKernelGGL(x32_to_f16_rows_kernel, dim3((unsigned)mm), dim3(256), 0, st,
