@@ -2000,8 +2000,8 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
     return reg_fwd_launch(st, rp, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, out, ws, (int)group_size);
   };
   if (bits == 4 && !transpose_b && group_size == 0) {
-    // few rows against a whole matrix (16 < M <= 256): the register-operand kernel, unless its tiles are too
-    // few to fill the chip even when split (the tiled kernel below splits finer)
+    // more than 16 rows: the register-operand kernel, unless its tiles are too few to fill the chip even when
+    // split (the tiled kernel below splits finer)
     if (rp.use && !rp.ragged && M > 16 && rp.tiles * rp.S >= 64) return run_reg_fwd();
     // GEMM-shaped work goes to the tiled kernel (split-K when the output tiles alone do not fill
     // the chip); small M goes through the decode kernel or the 16-row chunked kernels.

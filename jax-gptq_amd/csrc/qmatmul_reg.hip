@@ -1,12 +1,12 @@
 // Packed-weight matmul, forward, with both MFMA operands built in registers:
 //   out[M, C] = x[M, K] @ ((code - zero) * scale),  codes packed as 4-bit pairs (K = 2 R) or bytes (K = R).
-// Serves what the tuned 4-bit kernels of qmatmul.hip do not: 8-bit codes (any M), shapes whose rows are
-// not 8- or 16-byte multiples (C % 8 != 0, e.g. a vocabulary-sized C; K % 8 != 0; unaligned operands), and
-// for 4-bit codes the range 16 < M <= 256, where the work is the weights' and the output tiles are few.
+// Serves every forward product of more than 16 rows, and below that what the 4-bit decode kernel of
+// qmatmul.hip does not take: 8-bit codes and shapes whose rows are not 8- or 16-byte multiples (C % 8 != 0,
+// e.g. a vocabulary-sized C; K % 8 != 0; unaligned operands).
 //
-// A workgroup owns a (16 RB) x 128 output tile over a range of k-steps (all of K unless the contraction is
-// split over S workgroups) and its four wavefronts split those k-steps among them (k-step t of 32 k goes to
-// wavefront t % 4): nothing is staged in LDS and the k loop has no barrier.
+// A workgroup owns a (16 RB) x 128 output tile (RB = 1, 4 or 8 row blocks) over a range of k-steps (all of K
+// unless the contraction is split over S workgroups) and its four wavefronts split those k-steps among them
+// (k-step t of 32 k goes to wavefront t % 4): nothing is staged in LDS and the k loop has no barrier.
 //   B: lane (l16, g) loads 8 bytes = 8 channels of each packed row that holds its 8 k of the k-step
 //      (4-bit: rows 4g .. 4g+3, 8-bit: rows 8g .. 8g+7); the MFMA tile t8 takes byte t8 of every row.
 //      4-bit, fp16: byte permute, and-or under the exponent of 1024, one packed fma that rescales the high
