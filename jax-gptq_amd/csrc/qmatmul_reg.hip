@@ -39,10 +39,11 @@ __global__ __launch_bounds__(256, (RB == 1 ? 2 : 1)) void qmm_fwd_reg_kernel(con
                                                           unsigned long long *acc64) {
   constexpr bool BF = Act<TX>::BF && !GROUPED;      // grouped: the fp16 form of the dequantisation for both types
   // vector instructions between two MFMAs of the main loop (0: compiler's order)
-  constexpr int SCHED = RB == 4 ? 4 : 0;
-  // 128-row tiles: 256 accumulation registers hold the 8 x 8 product tiles, the row-sum tiles live in vector
-  // registers, and every MFMA accumulates in place (Act::mma_acc)
-  constexpr bool TIED = RB == 8;
+  constexpr int SCHED = (RB == 4 && (GROUPED || RAGGED)) ? 4 : 0;
+  // 64- and 128-row tiles: every MFMA accumulates in place (Act::mma_acc; the compiler's own form may write
+  // another register than it reads, and it rotates accumulators through copies).  128-row tiles: the 256
+  // accumulation registers hold the 8 x 8 product tiles, the row-sum tiles live in vector registers.
+  constexpr bool TIED = RB >= 4;
   constexpr int RBT = RB > 4 ? 4 : RB;           // row blocks per pass of the final reduction (LDS: 36 KB each)
   constexpr int NH = RB / RBT;                   // passes
   constexpr int NL = BITS == 4 ? 4 : 8;          // packed rows per lane and k-step
@@ -225,10 +226,11 @@ __global__ __launch_bounds__(256, (RB == 1 ? 2 : 1)) void qmm_fwd_reg_kernel(con
       }
     }
   };
-  // ---- 128-row tiles, per-channel parameters: the k-step in software-pipelined form.  The in-place MFMAs are
-  // inline asm, which the scheduler does not move; so the source order is the issue order: after every second
-  // MFMA of a tile the three vector instructions that build one operand register of the NEXT tile, and under the
-  // row-sum tile's MFMAs the first tile of the next k-step, whose weights are in the other ring slot.
+  // ---- 64- and 128-row tiles, per-channel parameters: the k-step in software-pipelined form.  The in-place MFMAs
+  // are inline asm, which the scheduler does not move; so the source order is the issue order: after every MFMA
+  // (128-row tiles: every second one) of a tile the three vector instructions that build one operand register of
+  // the NEXT tile, and under the row-sum tile's MFMAs the first tile of the next k-step, whose weights are in
+  // the next ring slot.
   auto dq_reg = [&](const uint2 (&w)[NL], int t8, int i) __attribute__((always_inline)) -> uint32_t {
     const uint32_t tb = (uint32_t)(t8 & 3);
     if constexpr (BITS == 4) {
@@ -270,7 +272,7 @@ __global__ __launch_bounds__(256, (RB == 1 ? 2 : 1)) void qmm_fwd_reg_kernel(con
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         Act<TX>::mma_acc(acc[rb][t8], aq[slot][rb], b);
-        if (t8 < 7 && (rb & 1)) nx[rb >> 1] = dq_reg(w, t8 + 1, rb >> 1);
+        if (t8 < 7 && (RB == 4 || (rb & 1))) nx[RB == 4 ? rb : rb >> 1] = dq_reg(w, t8 + 1, RB == 4 ? rb : rb >> 1);
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
@@ -281,7 +283,7 @@ __global__ __launch_bounds__(256, (RB == 1 ? 2 : 1)) void qmm_fwd_reg_kernel(con
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
       Act<TX>::mma_accv(acc[rb][8], aq[slot][rb], ones);
-      if (rb & 1) bcarry[rb >> 1] = dq_reg(wn, 0, rb >> 1);
+      if (RB == 4 || (rb & 1)) bcarry[RB == 4 ? rb : rb >> 1] = dq_reg(wn, 0, RB == 4 ? rb : rb >> 1);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
