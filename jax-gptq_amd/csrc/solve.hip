@@ -22,12 +22,26 @@
 // bit-identical to a CPU evaluation of gptq.py:136-147.
 #include "common.h"
 #include "gemm_f32.h"
+#include <type_traits>
+#include <utility>
 
 namespace {
 
 constexpr int SOLVE_CH = 64;               // channels per workgroup (one per lane)
 constexpr int SOLVE_NW = 8;                // wavefronts per workgroup (4: 45 us per block, 8: 40, 16: 52)
 constexpr int SOLVE_TPB = SOLVE_CH * SOLVE_NW;
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <int I> using ic = std::integral_constant<int, I>;
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+  (f(ic<I>{}), ...);
+}
+// f(ic<0>), f(ic<1>), ..., f(ic<N - 1>): a loop whose index is a constant expression in the body
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 template <int SB, typename TQ>
 __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
@@ -35,58 +49,328 @@ __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
     const float *zero, float maxq, TQ *Qb, uint8_t *cb, float *Err) {
   // Wb, Qb, cb: first row of the block in W, Q, codes; Lb: the block's diagonal corner of L
 #pragma clang fp contract(off)
-  extern __shared__ float smem[];
-  float *Ln = smem;                 // Ln[j * bs + i] = Lb[j][i]
-  float *Wl = smem + bs * bs;       // Wl[j * SOLVE_CH + lane] = W[block row j][channel]
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  float *Ln = smem;                         // Ln[j * bs + i] = Lb[j][i]
+  float *Wl = Ln + bs * bs;                 // Wl[j * SOLVE_CH + lane] = W[block row j][channel]
+  float *Es = Wl + bs * SOLVE_CH;           // [2][SB][SOLVE_CH] errors of a sub-block (two sub-blocks alternate)
+  float *Qs = Es + 2 * SB * SOLVE_CH;       // the same for the codes
+  float *QHs = Qs + 2 * SB * SOLVE_CH;      // and for the dequantised values
+  float *R1s = QHs + 2 * SB * SOLVE_CH;     // [bs] refined reciprocals of L's diagonal (NaN: outside the fast form's range)
   const int tid = threadIdx.x;
   const int lane = tid & (SOLVE_CH - 1);
   const int wave = tid / SOLVE_CH;
-  const int64_t n = (int64_t)blockIdx.x * SOLVE_CH + lane;
+  const int64_t n0 = (int64_t)blockIdx.x * SOLVE_CH;
+  const int64_t n = n0 + lane;
   const bool live = n < N;
   const int64_t nl = live ? n : N - 1;   // lanes past the edge shadow the last channel, store nothing
 
-  // ---- stage L's corner and the W tile; loads are unconditional (clamped) and batched so
-  //      that a wavefront has 16 of them in flight before it waits
-  {
-    const int total = bs * bs;
-    for (int base = 0; base < total; base += SOLVE_TPB * 16) {
-      float v[16];
+  // ---- staging of rows [row_lo, row_hi) of L's corner and of the W tile by threads t = 0 .. nthr - 1.  Loads are
+  //      unconditional (clamped) and go out in batches before the first wait; 16-byte loads where the shapes allow.
+  const bool vec = (bs & 3) == 0 && (ldl & 3) == 0 && (reinterpret_cast<uintptr_t>(Lb) & 15) == 0 && (N & 3) == 0 &&
+                   n0 + SOLVE_CH <= N && (reinterpret_cast<uintptr_t>(Wb) & 15) == 0;
+  // d -> the reciprocal as the compiler's division sequence refines it; NaN where the fast form of the chain
+  // may not be used for the row
+  auto diag_recip = [](float d) __attribute__((always_inline)) -> float {
+    const float r0c = __builtin_amdgcn_rcpf(d);
+    const float e0 = __builtin_fmaf(-d, r0c, 1.0f);
+    const float r1 = __builtin_fmaf(e0, r0c, r0c);
+    return (fabsf(d) >= 0x1p-40f && fabsf(d) <= 0x1p40f) ? r1 : __builtin_nanf("");
+  };
+  auto stage = [&](int row_lo, int row_hi, int t, int nthr) __attribute__((always_inline)) {
+    const int rows = row_hi - row_lo;
+    if (t < 0 || rows <= 0) return;
+    if (vec) {
+      const int q4 = bs >> 2, total4 = rows * q4;
+      if (nthr % q4 == 0) {
+        // a thread keeps its group of four columns and walks down the rows (no division per load)
+        const int j0 = t / q4, i4 = t - j0 * q4, jstep = nthr / q4;
+        for (int jb = j0; jb < rows; jb += jstep * 8) {
+          f32x4 v[8];
 #pragma unroll
-      for (int u = 0; u < 16; ++u) {
-        const int idx = min(base + u * SOLVE_TPB + tid, total - 1);
-        const int j = idx / bs, i = idx - j * bs;
-        v[u] = Lb[(int64_t)j * ldl + i];
+          for (int u = 0; u < 8; ++u) {
+            const int j = min(jb + u * jstep, rows - 1);
+            v[u] = *reinterpret_cast<const f32x4 *>(Lb + (int64_t)(row_lo + j) * ldl + 4 * i4);
+          }
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const int row = row_lo + jb + u * jstep;
+            if (row < row_hi) {
+              *reinterpret_cast<f32x4 *>(Ln + row * bs + 4 * i4) = v[u];
+              if ((row >> 2) == i4) {
+                const int r = row & 3;
+                R1s[row] = diag_recip(r == 0 ? v[u][0] : (r == 1 ? v[u][1] : (r == 2 ? v[u][2] : v[u][3])));
+              }
+            }
+          }
+        }
+      } else {
+        for (int base = 0; base < total4; base += nthr * 8) {
+          f32x4 v[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const int idx = min(base + u * nthr + t, total4 - 1);
+            const int j = idx / q4, i4 = idx - j * q4;
+            v[u] = *reinterpret_cast<const f32x4 *>(Lb + (int64_t)(row_lo + j) * ldl + 4 * i4);
+          }
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const int idx = base + u * nthr + t;
+            if (idx < total4) {
+              *reinterpret_cast<f32x4 *>(Ln + row_lo * bs + 4 * idx) = v[u];
+              const int j = idx / q4, i4 = idx - j * q4, row = row_lo + j;
+              if ((row >> 2) == i4) {
+                const int r = row & 3;
+                R1s[row] = diag_recip(r == 0 ? v[u][0] : (r == 1 ? v[u][1] : (r == 2 ? v[u][2] : v[u][3])));
+              }
+            }
+          }
+        }
       }
+      const int totalw = rows * (SOLVE_CH / 4);
+      for (int base = 0; base < totalw; base += nthr * 4) {
+        f32x4 v[4];
 #pragma unroll
-      for (int u = 0; u < 16; ++u) {
-        const int idx = base + u * SOLVE_TPB + tid;
-        if (idx < total) Ln[idx] = v[u];
+        for (int u = 0; u < 4; ++u) {
+          const int idx = min(base + u * nthr + t, totalw - 1);
+          const int j = idx / (SOLVE_CH / 4), c4 = idx - j * (SOLVE_CH / 4);
+          v[u] = *reinterpret_cast<const f32x4 *>(Wb + (int64_t)(row_lo + j) * N + n0 + 4 * c4);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int idx = base + u * nthr + t;
+          if (idx < totalw) *reinterpret_cast<f32x4 *>(Wl + row_lo * SOLVE_CH + 4 * idx) = v[u];
+        }
+      }
+    } else {
+      const int total = rows * bs;
+      for (int base = 0; base < total; base += nthr * 16) {
+        float v[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+          const int idx = min(base + u * nthr + t, total - 1);
+          const int j = idx / bs, i = idx - j * bs;
+          v[u] = Lb[(int64_t)(row_lo + j) * ldl + i];
+        }
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+          const int idx = base + u * nthr + t;
+          if (idx < total) {
+            Ln[row_lo * bs + idx] = v[u];
+            const int j = idx / bs, i = idx - j * bs;
+            if (i == row_lo + j) R1s[i] = diag_recip(v[u]);
+          }
+        }
+      }
+      const int totalw = rows * SOLVE_CH;
+      for (int base = 0; base < totalw; base += nthr * 16) {
+        float v[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+          const int idx = min(base + u * nthr + t, totalw - 1);
+          const int j = idx / SOLVE_CH, c = idx - j * SOLVE_CH;
+          const int64_t nc = n0 + c < N ? n0 + c : N - 1;
+          v[u] = Wb[(int64_t)(row_lo + j) * N + nc];
+        }
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+          const int idx = base + u * nthr + t;
+          if (idx < totalw) Wl[row_lo * SOLVE_CH + idx] = v[u];
+        }
       }
     }
-    const float *src = Wb + nl;
-    for (int j0 = wave; j0 < bs; j0 += SOLVE_NW * 16) {
-      float v[16];
-#pragma unroll
-      for (int u = 0; u < 16; ++u) v[u] = src[(int64_t)min(j0 + SOLVE_NW * u, bs - 1) * N];
-#pragma unroll
-      for (int u = 0; u < 16; ++u) {
-        const int j = j0 + SOLVE_NW * u;
-        if (j < bs) Wl[j * SOLVE_CH + lane] = v[u];
-      }
-    }
-  }
-  const float sc = scale[nl], z = zero[nl];
+  };
+  // rows [row_lo, row_hi) of the tile receive the errors e of the sub-block whose first row (= first column
+  // of L) is lcol; the rows are dealt round-robin to UW wavefronts, NB rows at a time (a row is a chain of SB
+  // dependent subtractions)
   float *wcol = Wl + lane;
-  __syncthreads();
-
-  for (int r0 = 0; r0 < bs; r0 += SB) {
-    float w[SB], e[SB];
+  auto update_rows = [&](int row_lo, int row_hi, const float (&e)[SB], int lcol, int widx, auto nbc, auto nwc)
+                         __attribute__((always_inline)) {
+    constexpr int NB = decltype(nbc)::value, UW = decltype(nwc)::value;
+    for (int j = row_lo + widx; j < row_hi; j += UW * NB) {
+      float x[NB], l[NB][SB];
 #pragma unroll
-    for (int t = 0; t < SB; ++t) w[t] = wcol[(r0 + t) * SOLVE_CH];
-    const float *ld = Ln + r0 * bs + r0;  // diagonal sub-block
+      for (int v = 0; v < NB; ++v) {
+        const int jj = min(j + UW * v, row_hi - 1);
+        x[v] = wcol[jj * SOLVE_CH];
+        const float *lr = Ln + jj * bs + lcol;
+        if constexpr (SB % 4 == 0) {
+#pragma unroll
+          for (int c = 0; c < SB / 4; ++c) {
+            const f32x4 q = *reinterpret_cast<const f32x4 *>(lr + 4 * c);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) l[v][4 * c + i] = q[i];
+          }
+        } else {
+#pragma unroll
+          for (int u = 0; u < SB; ++u) l[v][u] = lr[u];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < SB; ++u) {
+#pragma unroll
+        for (int v = 0; v < NB; ++v) {
+          const float upd = l[v][u] * e[u];
+          x[v] = x[v] - upd;
+        }
+      }
+#pragma unroll
+      for (int v = 0; v < NB; ++v)
+        if (j + UW * v < row_hi) wcol[(j + UW * v) * SOLVE_CH] = x[v];
+    }
+  };
+  // results of sub-block sb (in its LDS buffers) to memory, rows dealt over NWV wavefronts
+  auto store_sub = [&](int sb, int widx, auto nwc) __attribute__((always_inline)) {
+    constexpr int NWV = decltype(nwc)::value;
+    if (!live) return;
+    const int off = (sb & 1) * SB * SOLVE_CH + lane;
 #pragma unroll
     for (int t = 0; t < SB; ++t) {
-      float x = w[t];
+      if ((t % NWV) == widx) {
+        const int64_t o = (int64_t)(sb * SB + t) * N + n;
+        if (Qb) Qb[o] = from_f32<TQ>(QHs[off + t * SOLVE_CH]);
+        if (cb) cb[o] = (uint8_t)Qs[off + t * SOLVE_CH];
+        Err[o] = Es[off + t * SOLVE_CH];
+      }
+    }
+  };
+
+  stage(0, SB, tid, SOLVE_TPB);
+  const float sc = scale[nl], z = zero[nl];
+  const float rs = 1.0f / sc;
+  // the clamp of the code, moved to the integer before the zero point is added: exact for an integral zero point
+  const float klo = -z, khi = maxq - z;
+  const bool z_plain = !(z == rintf(z) && fabsf(z) <= 0x1p22f);
+  __syncthreads();
+
+  // ---- The chain of a sub-block (first wavefront): row t needs the error of row t - 1, and one wavefront issues
+  // an instruction every five to six cycles, so what counts is the number of instructions.  The fast form has
+  // 12 dependent ones per row (the two IEEE divisions of the plain form alone have 20):
+  //  * rint(x / sc) is taken from x * (1 / sc).  The product lies within 2^-22 |x / sc| of the rounded
+  //    quotient, so both round to the same integer unless the product is that close to a half-integer;
+  //  * the code is clamped as an integer before the zero point is added (see klo, khi);
+  //  * (x - qh) / d is the sequence the compiler emits for a division (reciprocal refined once, quotient
+  //    refined twice with exact remainders), with the part that depends only on d taken out of the chain.
+  //    The emitted form first rescales operands whose exponents are extreme (v_div_scale) and patches
+  //    special values afterwards (v_div_fixup); with 2^-40 <= |a|, |d| <= 2^40 neither does anything, and
+  //    the results are the same bit for bit.
+  // A lane that leaves these ranges anywhere in the sub-block (or meets a NaN, which reaches the last error)
+  // makes the wavefront evaluate the sub-block again with the plain divisions.
+  // What does not depend on the errors is out of the chain: the refined reciprocals of L's diagonal are computed
+  // by the threads that stage it, and the sub-block's triangle of L is read into registers between two chains.  The chain is
+  // right-looking (an error goes into all later rows of the sub-block as soon as it exists; every element still
+  // receives its updates in the order u = 0, 1, ...), and the source fixes the instruction order: between two
+  // dependent instructions of row t stand the updates that the error of row t - 1 owes to rows t + 1 ..., and
+  // that row's bookkeeping.
+  constexpr int TRI = SB * (SB + 1) / 2;
+  float lt[TRI], r1[SB];
+  auto prologue = [&](int r0) __attribute__((always_inline)) {
+    const float *ld = Ln + r0 * bs + r0;  // diagonal sub-block
+    if constexpr (SB % 4 == 0) {
+#pragma unroll
+      for (int t = 0; t < SB; ++t)
+#pragma unroll
+        for (int c = 0; c <= t / 4; ++c) {
+          const f32x4 v = *reinterpret_cast<const f32x4 *>(ld + t * bs + 4 * c);
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (4 * c + i <= t) lt[t * (t + 1) / 2 + 4 * c + i] = v[i];
+        }
+    } else {
+#pragma unroll
+      for (int t = 0; t < SB; ++t)
+#pragma unroll
+        for (int u = 0; u <= t; ++u) lt[t * (t + 1) / 2 + u] = ld[t * bs + u];
+    }
+#pragma unroll
+    for (int t = 0; t < SB; ++t) r1[t] = R1s[r0 + t];
+  };
+  auto chain_fast = [&](int r0, int boff) __attribute__((always_inline)) -> bool {
+    float xs[SB], e[SB], tmp[SB];
+    float qa_s[SB], k_s[SB], kc_s[SB], qh_s[SB], a_s[SB];
+    float fmax_acc = 0.f, qmax_acc = 0.f, amin_acc = 1.0f, amax_acc = 1.0f;
+#pragma unroll
+    for (int t = 0; t < SB; ++t) xs[t] = wcol[(r0 + t) * SOLVE_CH];
+    // the i-th instruction that the error of row te owes to the rows te + 2, ... (multiply, then subtract)
+    auto upd_op = [&](int te, int i) __attribute__((always_inline)) {
+      const int t2 = te + 2 + (i >> 1);
+      if ((i & 1) == 0) tmp[i >> 1] = lt[t2 * (t2 + 1) / 2 + te] * e[te];
+      else xs[t2] = xs[t2] - tmp[i >> 1];
+    };
+    constexpr int NBK = 7;
+    auto bk_op = [&](int te, int j) __attribute__((always_inline)) {
+      if (j == 0) fmax_acc = fmaxf(fmax_acc, fabsf(qa_s[te] - k_s[te]));
+      if (j == 1) qmax_acc = fmaxf(qmax_acc, fabsf(qa_s[te]));
+      if (j == 2) amin_acc = fminf(amin_acc, fabsf(a_s[te]));
+      if (j == 3) amax_acc = fmaxf(amax_acc, fabsf(a_s[te]));
+      if (j == 4) Es[boff + te * SOLVE_CH] = e[te];
+      if (j == 5) Qs[boff + te * SOLVE_CH] = kc_s[te] + z;
+      if (j == 6) QHs[boff + te * SOLVE_CH] = qh_s[te];
+    };
+    static_for<SB>([&](auto tc) __attribute__((always_inline)) {
+      constexpr int t = decltype(tc)::value;
+      constexpr int te = t - 1;
+      constexpr int P = t >= 1 ? 2 * (SB - 1 - t) : 0;
+      constexpr int B = t >= 1 ? NBK : 0;
+      constexpr int G = 12;
+      constexpr int per = (P + B + G - 1) / G;
+      // gap g of the row: the next `per` owed instructions, then a fence for the scheduler
+      auto fill = [&](auto gc) __attribute__((always_inline)) {
+        static_for<per>([&](auto cc) __attribute__((always_inline)) {
+          constexpr int done = decltype(gc)::value * per + decltype(cc)::value;
+          if constexpr (done < P) upd_op(te, done);
+          else if constexpr (done < P + B) bk_op(te, done - P);
+        });
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      const float d = lt[t * (t + 1) / 2 + t];
+      float x = xs[t];
+      if constexpr (t >= 1) {
+        const float upd = lt[t * (t + 1) / 2 + te] * e[te];
+        fill(ic<0>{});
+        x = x - upd;
+        fill(ic<1>{});
+      }
+      const float qa = x * rs;
+      fill(ic<2>{});
+      const float k = rintf(qa);
+      fill(ic<3>{});
+      const float kc = __builtin_amdgcn_fmed3f(k, klo, khi);
+      fill(ic<4>{});
+      const float qh = sc * kc;
+      fill(ic<5>{});
+      const float a = x - qh;
+      fill(ic<6>{});
+      const float q0 = a * r1[t];
+      fill(ic<7>{});
+      const float rem0 = __builtin_fmaf(-d, q0, a);
+      fill(ic<8>{});
+      const float q1 = __builtin_fmaf(rem0, r1[t], q0);
+      fill(ic<9>{});
+      const float rem1 = __builtin_fmaf(-d, q1, a);
+      fill(ic<10>{});
+      e[t] = __builtin_fmaf(rem1, r1[t], q1);
+      fill(ic<11>{});
+      qa_s[t] = qa;
+      k_s[t] = k;
+      kc_s[t] = kc;
+      qh_s[t] = qh;
+      a_s[t] = a;
+    });
+#pragma unroll
+    for (int j = 0; j < NBK; ++j) bk_op(SB - 1, j);
+    bool redo = z_plain;
+    redo |= !(fmax_acc <= 0.5f - 0x1p-21f * fmaxf(qmax_acc, 1.0f));
+    redo |= !(amin_acc >= 0x1p-40f && amax_acc <= 0x1p40f);
+    redo |= !(e[SB - 1] == e[SB - 1]);
+    return redo;
+  };
+  // the plain form (gptq.py:136-147 as written)
+  auto chain_plain = [&](int r0, int boff) __attribute__((always_inline)) {
+    const float *ld = Ln + r0 * bs + r0;
+    float e[SB];
+#pragma unroll
+    for (int t = 0; t < SB; ++t) {
+      float x = wcol[(r0 + t) * SOLVE_CH];
 #pragma unroll
       for (int u = 0; u < t; ++u) {
         const float upd = ld[t * bs + u] * e[u];
@@ -96,27 +380,62 @@ __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
       q = fminf(fmaxf(q, 0.f), maxq);
       const float qh = sc * (q - z);
       e[t] = (x - qh) / ld[t * bs + t];
-      if (live && (t % SOLVE_NW) == wave) {   // the stores of a sub-block are dealt over the wavefronts
-        const int64_t o = (int64_t)(r0 + t) * N + n;
-        if (Qb) Qb[o] = from_f32<TQ>(qh);
-        if (cb) cb[o] = (uint8_t)q;
-        Err[o] = e[t];
-      }
+      Es[boff + t * SOLVE_CH] = e[t];
+      Qs[boff + t * SOLVE_CH] = q;
+      QHs[boff + t * SOLVE_CH] = qh;
     }
-    // rows of this block below the sub-block, round-robin over the wavefronts
-#pragma unroll 2
-    for (int j = r0 + SB + wave; j < bs; j += SOLVE_NW) {
-      float x = wcol[j * SOLVE_CH];
-      const float *lr = Ln + j * bs + r0;
+  };
+
+  // The block is walked in sub-blocks of SB rows.  The first wavefront evaluates the sub-block's chain;
+  // meanwhile the others bring the rows below the sub-block up to date with the errors of the previous
+  // sub-block and write that sub-block's results out (first sub-block: they stage the rest of the tile).  Then
+  // all put the new errors into the rows of the next sub-block, and the first wavefront reads that sub-block's
+  // triangle.  Two barriers per sub-block.
+  // (The first wavefront runs a loop of its own, with the same barriers: the triangle's 150 registers are then
+  // live in that loop only.)
+  const int nsb = bs / SB;
+  constexpr int NBA = (SB + SOLVE_NW - 1) / SOLVE_NW;      // rows per wavefront between two chains
+  if (wave == 0) {
+    prologue(0);
+    for (int s = 0; s < nsb; ++s) {
+      const int r0 = s * SB;
+      const int boff = (s & 1) * SB * SOLVE_CH + lane;
+      if (__builtin_amdgcn_ballot_w64(chain_fast(r0, boff)) != 0ull) chain_plain(r0, boff);
+      __syncthreads();
+      if (s + 1 < nsb) {
+        float e[SB];
 #pragma unroll
-      for (int u = 0; u < SB; ++u) {
-        const float upd = lr[u] * e[u];
-        x = x - upd;
+        for (int t = 0; t < SB; ++t) e[t] = Es[boff + t * SOLVE_CH];
+        update_rows(r0 + SB, r0 + 2 * SB, e, r0, 0, ic<NBA>{}, ic<SOLVE_NW>{});
+        prologue(r0 + SB);
+        __syncthreads();
       }
-      wcol[j * SOLVE_CH] = x;
     }
-    __syncthreads();
+  } else {
+    for (int s = 0; s < nsb; ++s) {
+      const int r0 = s * SB;
+      const int boff = (s & 1) * SB * SOLVE_CH + lane;
+      if (s == 0) {
+        stage(SB, bs, tid - SOLVE_CH, SOLVE_TPB - SOLVE_CH);
+      } else {
+        float e[SB];
+        const int poff = ((s - 1) & 1) * SB * SOLVE_CH + lane;
+#pragma unroll
+        for (int t = 0; t < SB; ++t) e[t] = Es[poff + t * SOLVE_CH];
+        update_rows(r0 + SB, bs, e, r0 - SB, wave - 1, ic<4>{}, ic<SOLVE_NW - 1>{});
+        store_sub(s - 1, wave - 1, std::integral_constant<int, SOLVE_NW - 1>{});
+      }
+      __syncthreads();
+      if (s + 1 < nsb) {
+        float e[SB];
+#pragma unroll
+        for (int t = 0; t < SB; ++t) e[t] = Es[boff + t * SOLVE_CH];
+        update_rows(r0 + SB, r0 + 2 * SB, e, r0, wave, ic<NBA>{}, ic<SOLVE_NW>{});
+        __syncthreads();
+      }
+    }
   }
+  store_sub(nsb - 1, wave, std::integral_constant<int, SOLVE_NW>{});
 }
 
 template <int SB>
@@ -124,9 +443,9 @@ int launch_block(hipStream_t st, const float *W, int64_t N, const float *L, int6
                  const float *scale, const float *zero, float maxq, void *Q, int q_dtype,
                  uint8_t *codes, float *Err) {
   const dim3 grid((unsigned)ceil_div64(N, SOLVE_CH)), block(SOLVE_TPB);
-  const size_t lds = ((size_t)bs * bs + (size_t)bs * SOLVE_CH) * sizeof(float);
+  const size_t lds = ((size_t)bs * bs + (size_t)bs * SOLVE_CH + (size_t)6 * SB * SOLVE_CH + (size_t)bs) * sizeof(float);
   if (lds > 64 * 1024) {
-    // up to 96 KB of the 160 KB LDS of a CU; the limit has to be raised per kernel
+    // up to 120 KB of the 160 KB LDS of a CU; the limit has to be raised per kernel
     const void *fn = q_dtype == GPTQ_HIP_F32
                          ? reinterpret_cast<const void *>(block_quant_kernel<SB, float>)
                          : (q_dtype == GPTQ_HIP_F16
