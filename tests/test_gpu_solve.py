@@ -45,6 +45,56 @@ def test_process_block_bit_exact(G, bs):
         assert np.array_equal(to_np(e), e_ref)
 
 
+@pytest.mark.parametrize("N", [256, 197])
+@pytest.mark.parametrize("diag", ["plain", "tiny", "huge", "mixed"])
+def test_process_block_bit_exact_outside_the_fast_range(G, N, diag):
+    """The kernel's chain uses reciprocal forms of the two divisions where they are proven to give the bits of
+    the division, and falls back to the divisions elsewhere: ties of the rounding, weights on the grid (zero
+    error), extreme and denormal scales, fractional zero points, extreme diagonals of L, infinities and
+    NaNs all have to come out as the CPU evaluation has them.  (One known difference is left out of the
+    comparison: where the value to be quantised is a NaN, numpy's clip returns NaN and the kernel's
+    fmin(fmax(., 0), maxq) returns a number; the errors are NaN in both, as long as the NaN does not come from a
+    zero scale, which is therefore not among the cases.)"""
+    rng = np.random.default_rng(700 + N + len(diag))
+    bs, K = 32, 64
+    L = np.tril(0.1 * rng.standard_normal((K, K))).astype(np.float32)
+    d = rng.uniform(0.5, 2.0, K).astype(np.float32)
+    if diag == "tiny":
+        d *= np.float32(1e-15)
+    elif diag == "huge":
+        d *= np.float32(1e15)
+    elif diag == "mixed":
+        d[3::7] *= np.float32(1e-14)
+        d[5::11] *= np.float32(1e14)
+    L[np.arange(K), np.arange(K)] = d
+    scale = np.full(N, 2.0 ** -6, np.float32)
+    scale[1::8] = rng.uniform(0.001, 0.02, scale[1::8].shape).astype(np.float32)
+    scale[2::16] = np.float32(1e-30)
+    scale[3::16] = np.float32(1e30)
+    scale[4::32] = np.float32(1e-40)          # denormal
+    zero = rng.integers(0, 16, N).astype(np.float32)
+    zero[6::16] += np.float32(0.5)
+    zero[7::32] = np.float32(3e7)
+    k = rng.integers(-3, 19, (K, N)).astype(np.float32)
+    W = (scale[None, :] * (k - zero[None, :])).astype(np.float32)          # on the grid: zero error
+    half = rng.random((K, N)) < 0.3
+    W[half] += (0.5 * scale[None, :] * np.ones((K, 1), np.float32))[half]  # ties of the rounding
+    noise = rng.random((K, N)) < 0.4
+    W[noise] += (0.3 * scale[None, :] * rng.standard_normal((K, N)).astype(np.float32))[noise]
+    W[5, 9::40] = np.inf
+    W[17, 11::40] = np.nan
+    W[40, 13::40] = -np.inf
+    p = {"scale": scale, "zero": zero, "maxq": 15}
+    with np.errstate(all="ignore"):
+        for start in (0, K - bs):
+            q_ref, e_ref = O.process_block(W, L, start, p, bs)
+            q, e = G._process_block(W, L, start, p, bs)
+            q, e = to_np(q), to_np(e)
+            assert np.array_equal(e, e_ref, equal_nan=True)
+            known = ~np.isnan(q_ref)
+            assert np.array_equal(q[known], q_ref[known])
+
+
 def _check_against_oracle(G, W, xs, X_all, **kw):
     Q, p = G.gptq(W, xs, **kw)
     Qr, pr = O.gptq(W, xs, **kw)
