@@ -80,6 +80,15 @@ __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
     const int rows = row_hi - row_lo;
     if (t < 0 || rows <= 0) return;
     if (vec) {
+      // the first batch of the W tile goes out before the loads of L and is stored after them
+      const int totalw = rows * (SOLVE_CH / 4);
+      f32x4 wv[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int idx = min(u * nthr + t, totalw - 1);
+        const int j = idx / (SOLVE_CH / 4), c4 = idx - j * (SOLVE_CH / 4);
+        wv[u] = *reinterpret_cast<const f32x4 *>(Wb + (int64_t)(row_lo + j) * N + n0 + 4 * c4);
+      }
       const int q4 = bs >> 2, total4 = rows * q4;
       if (nthr % q4 == 0) {
         // a thread keeps its group of four columns and walks down the rows (no division per load)
@@ -88,13 +97,14 @@ __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
           f32x4 v[8];
 #pragma unroll
           for (int u = 0; u < 8; ++u) {
+            // (right of the diagonal nothing is needed: those threads re-read the diagonal's group)
             const int j = min(jb + u * jstep, rows - 1);
-            v[u] = *reinterpret_cast<const f32x4 *>(Lb + (int64_t)(row_lo + j) * ldl + 4 * i4);
+            v[u] = *reinterpret_cast<const f32x4 *>(Lb + (int64_t)(row_lo + j) * ldl + 4 * min(i4, (row_lo + j) >> 2));
           }
 #pragma unroll
           for (int u = 0; u < 8; ++u) {
             const int row = row_lo + jb + u * jstep;
-            if (row < row_hi) {
+            if (row < row_hi && i4 <= (row >> 2)) {
               *reinterpret_cast<f32x4 *>(Ln + row * bs + 4 * i4) = v[u];
               if ((row >> 2) == i4) {
                 const int r = row & 3;
@@ -126,8 +136,12 @@ __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
           }
         }
       }
-      const int totalw = rows * (SOLVE_CH / 4);
-      for (int base = 0; base < totalw; base += nthr * 4) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int idx = u * nthr + t;
+        if (idx < totalw) *reinterpret_cast<f32x4 *>(Wl + row_lo * SOLVE_CH + 4 * idx) = wv[u];
+      }
+      for (int base = nthr * 4; base < totalw; base += nthr * 4) {
         f32x4 v[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
