@@ -1,22 +1,21 @@
 // Blocked GPTQ column loop: quantise block_size rows with error feedback, then push the
-// accumulated error into the remaining rows with fp32 MFMA GEMMs: after every block into the
-// rest of its 512-row group, after every group into everything below it.
+// accumulated error into the remaining rows with fp32 MFMA GEMMs: inside a 512-row group every
+// block first receives what the group's earlier blocks owe it, and after every group everything
+// below it receives the group's errors in one product.
 //
 // In-block kernel: the N output channels are independent, so one lane owns one channel and a
-// workgroup of eight wavefronts owns 64 channels.  The workgroup first copies its channels of
-// the block's rows and the block's corner of L into LDS (all loads of a wavefront in flight
-// at once), then works out of LDS only.  The block is walked in sub-blocks of SB rows:
-//   * the SB rows of a sub-block and their SB errors live in VGPRs (statically indexed,
-//     fully unrolled triangle).  This part is a sequential chain per channel; all
-//     wavefronts evaluate it redundantly (same instructions, same values), which saves a
-//     broadcast of the errors and costs nothing: the chain is bound by latency, not by issue;
-//   * the rows of the block below the sub-block are then updated in the LDS tile, the rows
-//     dealt round-robin to the wavefronts; one barrier per sub-block.
+// workgroup of eight wavefronts owns 64 channels.  It works out of LDS: its channels of the
+// block's rows, the block's corner of L, the refined reciprocals of L's diagonal.  The block is
+// walked in sub-blocks of SB rows:
+//   * the first wavefront evaluates the sub-block's sequential chain (row t needs the error of
+//     row t - 1) with the sub-block's triangle of L and its rows in VGPRs;
+//   * meanwhile the other wavefronts apply the previous sub-block's errors to the rows below
+//     (rows dealt round-robin) and write that sub-block's results to memory;
+//   * then all wavefronts put the new errors into the rows of the next sub-block.
 // Each lane touches only its own column of the tile (no bank conflicts); L is read with
-// broadcast reads (every lane the same address), the SB factors of one row are consecutive.
-// W itself is not written.
+// broadcast reads (every lane the same address).  W itself is not written.
 //
-// Every floating-point operation is the IEEE operation the reference writes (true
+// Every floating-point result is that of the IEEE operation the reference writes (true
 // division, round-half-even, separate multiply and subtract) and every element receives
 // its updates in the reference's order, so given the same L and W the block result is
 // bit-identical to a CPU evaluation of gptq.py:136-147.
@@ -576,6 +575,13 @@ int solve_impl(hipStream_t st, float *W, int64_t K, int64_t N, const float *L, c
         sc = scale_g + gi * N;
         zr = zero_g + gi * N;
       }
+      if (group_size == 0 && start > gs) {
+        // the block's rows receive what the earlier blocks of this update group owe them, in one product
+        // with k = start - gs (per-channel parameters: nothing reads the rows below the block before their
+        // own turn, so each row of the group is read and written once per group, not once per block above it)
+        const int rc = trailing_update(st, L + start * K + gs, K, Err, W + start * N, N, block_size, start - gs);
+        if (rc) return rc;
+      }
       void *Qb = Q ? (void *)((char *)Q + (size_t)start * N * qsz) : nullptr;
       uint8_t *cb = codes ? codes + start * N : nullptr;
       float *Eb = Err + (start - gs) * N;
@@ -583,8 +589,9 @@ int solve_impl(hipStream_t st, float *W, int64_t K, int64_t N, const float *L, c
                              q_dtype, cb, Eb);
       if (rc) return rc;
       const int64_t end = start + block_size;
-      if (end < ge) {
-        // rows of this group below the block: W[end:ge] -= L[end:ge, start:end] @ Err_block
+      if (group_size > 0 && end < ge) {
+        // grouped parameters are taken from rows that must be current when their group begins, so here every
+        // block updates all rows of the update group below it: W[end:ge] -= L[end:ge, start:end] @ Err_block
         rc = trailing_update(st, L + end * K + start, K, Eb, W + end * N, N, ge - end, block_size);
         if (rc) return rc;
       }
