@@ -105,19 +105,19 @@ __global__ __launch_bounds__(256) void copy_out_kernel(const R *Minv, int64_t Kp
 // standard Cholesky of the index-reversed block: G G^T = J D J, M_bb = J G^T J.  Writes
 // M_bb over A[b,b] (upper part zeroed) and M_bb^-1 = J G^-T J into Minv[b,b].
 //
-// Five wavefronts.  Four factorise: lane r of each keeps row r of G for the 16 columns c = 4 j + w
-// of wavefront w (fully unrolled loops).  The wavefront that owns column k scales it (pivot by
-// v_readlane, reciprocal square root) and publishes it through LDS; after the barrier every
-// factorising wavefront holds the column in one VGPR, from which lane c's entry becomes a scalar
-// operand (v_readlane) of the update of its column c: two instructions per remaining column, at
-// most 16 columns per wavefront and step.  The owner of column k + 1 updates that column first
-// and scales and publishes it before it turns to its other columns, so the chain from one pivot
-// to the next is one LDS round trip, one update and the scaling.  The fifth wavefront follows
-// one step behind and computes row k of X = G^-1 (lane j keeps column j of X) from row k of G,
-// which it reads from LDS with broadcast reads.  One workgroup barrier per step.  The block is on
-// the critical path of the blocked factorisation (nothing else can run while it does), so latency
-// is what counts here.  Entries above the diagonal of G hold garbage while the factorisation
-// runs (masking them would cost a third instruction per element) and are written out as zeros.
+// Five wavefronts.  Four factorise: lane r of each keeps row r of G for 16 columns, dealt in panels of four
+// adjacent columns (panel p belongs to wavefront p mod 4).  What bounds the kernel is the chain from one
+// synchronisation to the next, so there is one per panel, not one per column: the owner of a panel factorises
+// its four columns by itself (pivot by v_readlane, reciprocal square root, the later columns of the panel
+// updated at once) and publishes them through LDS; after the barrier every factorising wavefront holds the four
+// columns in four VGPRs, from which lane c's entries become scalar operands (v_readlane) of the updates of its
+// column c: two instructions per column and pivot, in the order of the pivots.  The owner of the next panel
+// updates that panel first and factorises and publishes it before it turns to its other columns.  The fifth
+// wavefront follows one panel behind and computes four rows of X = G^-1 (lane j keeps column j of X) from the
+// rows of G, which it reads from LDS with broadcast reads.  The block is on the critical path of the blocked
+// factorisation (nothing else can run while it does), so latency is what counts here.  Entries above the
+// diagonal of G hold garbage while the factorisation runs (masking them would cost a third instruction per
+// element) and are written out as zeros.
 static_assert(NB == 64, "the diagonal kernel maps one matrix row to one lane of a wavefront");
 constexpr int GSTR = NB + 4;   // LDS row stride of G: rows stay 16-byte aligned
 
@@ -145,6 +145,7 @@ __device__ __forceinline__ void root_and_inverse(double piv, double &root, doubl
 }
 
 constexpr int DIAG_FW = 4;                       // factorising wavefronts
+constexpr int PW = 4;                            // columns per panel
 constexpr int DIAG_THREADS = (DIAG_FW + 1) * 64;
 
 template <typename R>
@@ -153,7 +154,7 @@ __global__ __launch_bounds__(DIAG_THREADS) void chol_diag_kernel(R *A, R *Minv, 
   __shared__ __attribute__((aligned(16))) R dinv[NB];        // 1 / G[k][k]
   __shared__ __attribute__((aligned(16))) R Gs[NB * GSTR];   // G, row major
   __shared__ __attribute__((aligned(16))) R Xs[NB * (NB + 1)];   // X = G^-1, row major
-  __shared__ __attribute__((aligned(16))) R Lcol[2][NB];     // column k of G, by step parity
+  __shared__ __attribute__((aligned(16))) R Lcol[2][PW][NB]; // the columns of a panel of G, by panel parity
   constexpr int XSTR = NB + 1;
   constexpr int CW = NB / DIAG_FW;                           // columns per factorising wavefront
   const int r = threadIdx.x & 63;
@@ -164,57 +165,70 @@ __global__ __launch_bounds__(DIAG_THREADS) void chol_diag_kernel(R *A, R *Minv, 
   typedef R rowvec __attribute__((ext_vector_type(NB)));
 
   if (wave < DIAG_FW) {
+    // slot j of wavefront w holds column col_of(j) = 16 (j / 4) + 4 w + j % 4
+    auto col_of = [&](int j) __attribute__((always_inline)) { return (PW * DIAG_FW) * (j / PW) + PW * wave + (j % PW); };
     // G[r][c] (c <= r) = D[63-c][63-r]: for fixed c the lanes read one row of D (coalesced)
     colvec g;
 #pragma unroll
     for (int j = 0; j < CW; ++j) {
-      const int c = DIAG_FW * j + wave;
+      const int c = col_of(j);
       g[j] = D[(int64_t)(NB - 1 - c) * ld + (NB - 1 - r)];   // c > r: finite garbage, never used
     }
     bool bad = false;
-    // scales column k (held by this wavefront as g[k / 4]) and publishes it
-    auto scale_and_publish = [&](int k) __attribute__((always_inline)) {
-      const int jk = k / DIAG_FW;
-      const R piv = lane_bcast(g[jk], k);
-      bad = bad || !(piv > R(0));
-      R root, rinv;
-      root_and_inverse(piv, root, rinv);
-      const R l = (r == k) ? root : g[jk] * rinv;
-      g[jk] = l;
-      Lcol[k & 1][r] = l;
-      Gs[r * GSTR + k] = (k <= r) ? l : R(0);
-      if (r == k) dinv[k] = rinv;
+    // G[r][c] -= l[r] l[c] for the column in slot j; pinned to its place: left free, the compiler may defer
+    // every update until the element is needed and keep the operands of all steps alive
+    auto update = [&](int j, R l) __attribute__((always_inline)) {
+      R t = g[j] - l * lane_bcast(l, col_of(j));
+      asm volatile("" : "+v"(t));
+      g[j] = t;
     };
-    if (wave == 0) scale_and_publish(0);
+    // factorises panel p (held by this wavefront in slots 4 (p / 4) ...) and publishes it
+    auto factor_panel = [&](int p) __attribute__((always_inline)) {
+      const int j0 = PW * (p / DIAG_FW);
 #pragma unroll
-    for (int k = 0; k < NB; ++k) {
-      __syncthreads();                        // column k is in LDS
-      const R l = Lcol[k & 1][r];
-      const int owner = k % DIAG_FW, jk = k / DIAG_FW;
-      // G[r][c] -= G[r][k] G[c][k] for this wavefront's column c = 4 j + wave
-      auto update = [&](int j) __attribute__((always_inline)) {
-        R t = g[j] - l * lane_bcast(l, DIAG_FW * j + wave);
-        // Pin the update to this step: left free, the compiler may defer every update until the
-        // element is needed and keep the operands of all steps alive.
-        asm volatile("" : "+v"(t));
-        g[j] = t;
+      for (int q = 0; q < PW; ++q) {
+        const int k = PW * p + q;
+        const R piv = lane_bcast(g[j0 + q], k);
+        bad = bad || !(piv > R(0));
+        R root, rinv;
+        root_and_inverse(piv, root, rinv);
+        const R l = (r == k) ? root : g[j0 + q] * rinv;
+        g[j0 + q] = l;
+        Lcol[p & 1][q][r] = l;
+        Gs[r * GSTR + k] = (k <= r) ? l : R(0);
+        if (r == k) dinv[k] = rinv;
+#pragma unroll
+        for (int q2 = q + 1; q2 < PW; ++q2) update(j0 + q2, l);
+      }
+    };
+    if (wave == 0) factor_panel(0);
+#pragma unroll
+    for (int p = 0; p < NB / PW; ++p) {
+      __syncthreads();                        // panel p is in LDS
+      R l[PW];
+#pragma unroll
+      for (int q = 0; q < PW; ++q) l[q] = Lcol[p & 1][q][r];
+      auto apply = [&](int j) __attribute__((always_inline)) {
+#pragma unroll
+        for (int q = 0; q < PW; ++q) update(j, l[q]);
       };
-      if (k + 1 < NB) {
-        // column k + 1 first, by its owner, which then scales and publishes it
-        const int nown = (k + 1) % DIAG_FW, jn = (k + 1) / DIAG_FW;
+      if (p + 1 < NB / PW) {
+        // the next panel first, by its owner, which then factorises and publishes it
+        const int nown = (p + 1) % DIAG_FW, jn0 = PW * ((p + 1) / DIAG_FW);
         if (wave == nown) {
-          update(jn);
-          scale_and_publish(k + 1);
-        }
 #pragma unroll
-        for (int j = jk; j < CW; ++j) {
-          // columns c > k of this wavefront, except k + 1 (done above by its owner)
-          if (j == jk) {
-            if (wave > owner && !(wave == nown && j == jn)) update(j);
-          } else if (j == jn) {
-            if (wave != nown) update(j);
-          } else {
-            update(j);
+          for (int q = 0; q < PW; ++q) apply(jn0 + q);
+          factor_panel(p + 1);
+        }
+        // the other columns right of the panel
+#pragma unroll
+        for (int j = 0; j < CW; ++j) {
+          const int jp = j / PW;                       // the slot's panel is 4 jp + wave
+          const bool next = (jp == (p + 1) / DIAG_FW);  // ... the next panel, if this wavefront owns it
+          if (jp > p / DIAG_FW) {
+            if (!next || wave != nown) apply(j);
+          } else if (jp == p / DIAG_FW) {
+            if (wave > p % DIAG_FW && !(next && wave == nown)) apply(j);
           }
         }
       }
@@ -224,14 +238,19 @@ __global__ __launch_bounds__(DIAG_THREADS) void chol_diag_kernel(R *A, R *Minv, 
     // ---- X = G^-1, lane j computes column j: x[i] = (delta_ij - sum_{k<i} G[i][k] x[k]) / G[i][i]
     rowvec x;
 #pragma unroll
-    for (int i = 0; i < NB; ++i) {
-      __syncthreads();                       // row i of G (columns 0..i) is complete
-      R acc = (i == r) ? 1 : 0;
+    for (int p = 0; p < NB / PW; ++p) {
+      __syncthreads();                       // rows 4 p .. 4 p + 3 of G are complete
 #pragma unroll
-      for (int k = 0; k < i; ++k) acc -= Gs[i * GSTR + k] * x[k];
-      R xi = acc * dinv[i];   // stays 0 for i < j since every term is 0
-      asm volatile("" : "+v"(xi));         // keeps the row reads of later steps from being hoisted
-      x[i] = xi;
+      for (int q = 0; q < PW; ++q) {
+        const int i = PW * p + q;
+        // four partial sums: one chain of up to 63 dependent instructions otherwise
+        R acc[4] = {(i == r) ? R(1) : R(0), R(0), R(0), R(0)};
+#pragma unroll
+        for (int k = 0; k < i; ++k) acc[k & 3] -= Gs[i * GSTR + k] * x[k];
+        R xi = ((acc[0] + acc[1]) + (acc[2] + acc[3])) * dinv[i];   // stays 0 for i < j: every term is 0
+        asm volatile("" : "+v"(xi));         // keeps the row reads of later steps from being hoisted
+        x[i] = xi;
+      }
     }
 #pragma unroll
     for (int i = 0; i < NB; ++i) Xs[i * XSTR + r] = x[i];
