@@ -57,7 +57,7 @@ __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
   float *R1s = QHs + 2 * SB * SOLVE_CH;     // [bs] refined reciprocals of L's diagonal (NaN: outside the fast form's range)
   const int tid = threadIdx.x;
   const int lane = tid & (SOLVE_CH - 1);
-  const int wave = tid / SOLVE_CH;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / SOLVE_CH);   // wave-uniform: scalar branches on it
   const int64_t n0 = (int64_t)blockIdx.x * SOLVE_CH;
   const int64_t n = n0 + lane;
   const bool live = n < N;
