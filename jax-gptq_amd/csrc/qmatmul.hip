@@ -2043,10 +2043,10 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
     }
   }
   // Transposed, 4-bit: the tiled kernel has no split over the contraction, so while its 64 x 128 output tiles
-  // number fewer than the CUs it runs as long as a full chip's worth of tiles would (122 us for any M <= 448
+  // number no more than the CUs it runs as long as a full chip's worth of tiles would (122 us for any M <= 448
   // on 4096 x 11008); there the register-operand kernel, which splits, takes over (M = 128: 124 -> 38 us,
-  // M = 16: 122 -> 23 us).
-  const bool bwd_tiles_fill = ceil_div64(2 * R, 128) * ceil_div64(M, 64) >= 256 ||
+  // M = 16: 122 -> 23 us; exactly one tile per CU, M = 512: 133 -> 103 us).
+  const bool bwd_tiles_fill = ceil_div64(2 * R, 128) * ceil_div64(M, 64) > 256 ||
                               !(reg_groups_ok && reg_bwd_plan(M, R, C, bits, al).use);
   if (bits == 4 && transpose_b && group_size == 0 && bwd_tiles_fill &&
       bwd_fast_ok(x_dtype, M, R, C, x, packed, zero, scale)) {
