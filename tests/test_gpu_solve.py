@@ -45,6 +45,24 @@ def test_process_block_bit_exact(G, bs):
         assert np.array_equal(to_np(e), e_ref)
 
 
+@pytest.mark.parametrize("bs,K,N", [(32, 96, 256), (48, 144, 260), (96, 192, 64), (112, 224, 128), (128, 384, 192),
+                                    (16, 50, 130), (64, 192, 1024)])
+def test_process_block_bit_exact_more_shapes(G, bs, K, N):
+    """Block sizes with 2 to 8 sub-blocks of 16 rows (and of 4 rows: 50 is not a multiple of 4, so L's rows are
+    not 16-byte aligned), channel counts with full and partial 64-channel tiles, blocks at the start, in the
+    middle and at the end of the matrix."""
+    W, X = _problem(300 + bs + N, K, N, 4 * K + 50, correlated=True)
+    H = O.accumulate_H([X])
+    _, L, bad = O.damp_and_invert(W, H, 0.01)
+    assert not bad
+    p = O.get_col_quantize_params(W)
+    for start in sorted({0, ((K - bs) // 2 // 2) * 2, K - bs}):
+        q_ref, e_ref = O.process_block(W, L, start, p, bs)
+        q, e = G._process_block(W, L, start, p, bs)
+        assert np.array_equal(to_np(q), q_ref)
+        assert np.array_equal(to_np(e), e_ref)
+
+
 @pytest.mark.parametrize("N", [256, 197])
 @pytest.mark.parametrize("diag", ["plain", "tiny", "huge", "mixed"])
 def test_process_block_bit_exact_outside_the_fast_range(G, N, diag):
