@@ -243,11 +243,10 @@ __global__ __launch_bounds__(DIAG_THREADS) void chol_diag_kernel(R *A, R *Minv, 
 #pragma unroll
       for (int q = 0; q < PW; ++q) {
         const int i = PW * p + q;
-        // four partial sums: one chain of up to 63 dependent instructions otherwise
-        R acc[4] = {(i == r) ? R(1) : R(0), R(0), R(0), R(0)};
+        R acc = (i == r) ? R(1) : R(0);
 #pragma unroll
-        for (int k = 0; k < i; ++k) acc[k & 3] -= Gs[i * GSTR + k] * x[k];
-        R xi = ((acc[0] + acc[1]) + (acc[2] + acc[3])) * dinv[i];   // stays 0 for i < j: every term is 0
+        for (int k = 0; k < i; ++k) acc -= Gs[i * GSTR + k] * x[k];
+        R xi = acc * dinv[i];                // stays 0 for i < j: every term is 0
         asm volatile("" : "+v"(xi));         // keeps the row reads of later steps from being hoisted
         x[i] = xi;
       }

@@ -549,13 +549,20 @@ constexpr int QD_MAX_SPLITS = 32;
 //    to fp16 as they are consumed, and the workgroup that completes an output rounds it to fp16, widens it
 //    and scales it back: the same arithmetic, bit for bit, without staging buffers and with one launch
 //    (M = 1: 16.8 -> 9.8 us) or two (more rows) instead of three.
-template <int NW, int KS, int MR, bool ATOM, bool LOOP, typename TZ, typename TX, bool X32 = false>
+//  * BITS = 8 (fp16 activations): a k-step is 32 rows of one code per byte, eight 16-byte rows per lane; two
+//    rows' bytes become {1024 + a, 1024 + b} with a byte permute and an or, the activations enter as they
+//    are, and all offsets leave through one activation sum (the odd-k sum stays zero).
+template <int NW, int KS, int MR, bool ATOM, bool LOOP, typename TZ, typename TX, bool X32 = false, int BITS = 4>
 __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
     const std::conditional_t<X32, float, TX> *x, int M, int K, const uint8_t *pk, int R, int C, const TZ *zero,
     const TZ *scale, std::conditional_t<X32, float, TX> *out, QmmWs ws, int S, int rows_per_split,
     const int32_t *rowexp_in) {
   constexpr bool BF = Act<TX>::BF;
   static_assert(!X32 || (ATOM && !BF), "fp32 rows: fp16 arithmetic and the atomic sum only");
+  static_assert(BITS == 4 || (BITS == 8 && !BF && !X32), "8-bit codes: fp16 activations");
+  constexpr int NR = BITS == 4 ? 4 : 8;          // rows per lane and k-step
+  constexpr int RPS = 4 * NR;                    // rows per k-step of a wavefront
+  constexpr int XK = BITS == 4 ? 2 : 1;          // k per row
   typedef std::conditional_t<X32, float, TX> XT;
   extern __shared__ float red[];   // [NW][MR][256] partial tiles, then [NW][2][16] x sums
   __shared__ int s_last;
@@ -570,8 +577,8 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
   const int mvalid = min(16, M - m0);
   const int g = lane >> 4, l16 = lane & 15;
   const int r_begin = split * rows_per_split, r_end = min(R, r_begin + rows_per_split);
-  // k-step t of this wavefront: packed rows r_begin + (t NW + wave) 16 + [0, 16)
-  const int groups = (r_end - r_begin + 15) >> 4;
+  // k-step t of this wavefront: packed rows r_begin + (t NW + wave) RPS + [0, RPS)
+  const int groups = (r_end - r_begin + RPS - 1) / RPS;
   const int nsteps = groups > wave ? (groups - wave + NW - 1) / NW : 0;
 
   // One k-step of loads: the activations of the lane group's four packed rows (16 bytes = 8 k; range
@@ -582,18 +589,18 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
   // k-step enters with zero activations.  LOOP: a ring of KS k-steps that is refilled as it is consumed,
   // for matrices beyond what the chip holds in flight; otherwise all KS k-steps of the range are issued
   // at once, and a wavefront skips the k-steps that lie past its range altogether.
-  struct Step { uint4 d[4]; uint4 pr; uint4 pr2; };      // pr2: the second half of an fp32 chunk (X32)
+  struct Step { uint4 d[NR]; uint4 pr; uint4 pr2; };     // pr2: the second half of an fp32 chunk (X32)
   const bool m_ok = l16 < mvalid;
   const XT *xr = x + (int64_t)(m0 + (m_ok ? l16 : 0)) * K;
   const int col0 = min(strip * QSTRIP + 16 * l16, C - 16);
   const uint8_t *wp = pk + col0;
   auto issue = [&](Step &st, int t) __attribute__((always_inline)) {
-    const int rbase = r_begin + (t * NW + wave) * 16 + 4 * g;
-    st.pr = *reinterpret_cast<const uint4 *>(xr + 2 * min(rbase, R - 4));
-    if (X32) st.pr2 = *reinterpret_cast<const uint4 *>(xr + 2 * min(rbase, R - 4) + 4);
-    const uint8_t *row = wp + (int64_t)min(rbase, R - 4) * C;       // R % 4 == 0: four rows inside the matrix
+    const int rbase = r_begin + (t * NW + wave) * RPS + NR * g;
+    st.pr = *reinterpret_cast<const uint4 *>(xr + XK * min(rbase, R - NR));
+    if (X32) st.pr2 = *reinterpret_cast<const uint4 *>(xr + XK * min(rbase, R - NR) + 4);
+    const uint8_t *row = wp + (int64_t)min(rbase, R - NR) * C;      // R % NR == 0: the rows are inside the matrix
 #pragma unroll
-    for (int i = 0; i < 4; ++i) st.d[i] = *reinterpret_cast<const uint4 *>(row + (int64_t)i * C);
+    for (int i = 0; i < NR; ++i) st.d[i] = *reinterpret_cast<const uint4 *>(row + (int64_t)i * C);
   };
 
   const DqConst dqk = dq_const<BF>();
@@ -618,11 +625,28 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
       pr = make_uint4(h[0], h[1], h[2], h[3]);
     }
     {
-      const bool ok = m_ok && t < nsteps && r_begin + (t * NW + wave) * 16 + 4 * g < r_end;
+      const bool ok = m_ok && t < nsteps && r_begin + (t * NW + wave) * RPS + NR * g < r_end;
       pr.x = ok ? pr.x : 0u;
       pr.y = ok ? pr.y : 0u;
       pr.z = ok ? pr.z : 0u;
       pr.w = ok ? pr.w : 0u;
+    }
+    if constexpr (BITS == 8) {
+      // the lane's eight k are its eight rows, in order: A as loaded, B register i = rows 2 i, 2 i + 1
+      se += (Act<TX>::lo(pr.x) + Act<TX>::hi(pr.x)) + (Act<TX>::lo(pr.y) + Act<TX>::hi(pr.y));
+      se += (Act<TX>::lo(pr.z) + Act<TX>::hi(pr.z)) + (Act<TX>::lo(pr.w) + Act<TX>::hi(pr.w));
+#pragma unroll
+      for (int tl = 0; tl < 16; ++tl) {
+        const int w = tl >> 2, tb = tl & 3;
+        const uint32_t sel = 0x0c000c00u | ((uint32_t)(4 + tb) << 16) | (uint32_t)tb;
+        uint4 bv;
+        bv.x = __builtin_amdgcn_perm(u4_comp(st.d[1], w), u4_comp(st.d[0], w), sel) | 0x64006400u;
+        bv.y = __builtin_amdgcn_perm(u4_comp(st.d[3], w), u4_comp(st.d[2], w), sel) | 0x64006400u;
+        bv.z = __builtin_amdgcn_perm(u4_comp(st.d[5 % NR], w), u4_comp(st.d[4 % NR], w), sel) | 0x64006400u;
+        bv.w = __builtin_amdgcn_perm(u4_comp(st.d[7 % NR], w), u4_comp(st.d[6 % NR], w), sel) | 0x64006400u;
+        acc[tl] = Act<TX>::mma(pr, bv, acc[tl]);
+      }
+      return;
     }
     uint4 av;
     av.x = __builtin_amdgcn_perm(pr.y, pr.x, 0x05040100u);  // {x[2r0],   x[2r1]}
@@ -897,8 +921,11 @@ struct DecPlan {
   size_t lds_bytes, x1_bytes, part_bytes, total_bytes;
 };
 
-DecPlan dec_plan(int64_t M, int64_t R, int64_t C) {
+DecPlan dec_plan(int64_t M, int64_t R8, int64_t C, int bits = 4) {
   DecPlan p{};
+  // 8-bit codes: planned in k-steps like a 4-bit matrix of half the rows (a k-step carries twice the bytes)
+  if (bits == 8 && R8 % 8 != 0) return p;
+  const int64_t R = bits == 8 ? R8 / 2 : R8;
   if (M < 1 || M > 16 || R % 4 != 0 || C % 16 != 0 || C < 16 || R >= (1LL << 30) || C >= (1LL << 30)) return p;
   p.strips = (int)ceil_div64(C, QSTRIP);
   if (p.strips > QMM_MAX_COUNTERS) return p;
@@ -961,21 +988,27 @@ DecPlan dec_plan(int64_t M, int64_t R, int64_t C) {
     }
   }
   p.lds_bytes = ((size_t)p.nw * p.mr * QSTRIP + (size_t)p.nw * 32 + 32) * sizeof(float);
+  if (bits == 8) {
+    // (the ring-loop forms of the 8-bit instantiation do not fit their register budgets: those matrices stay
+    // with the register-operand kernel)
+    if (p.loop) return DecPlan{};
+    p.rows *= 2;
+  }
   p.use = true;
   return p;
 }
 
-template <int NW, int KS, int MR, bool ATOM, bool LOOP, typename TZ, typename TX, bool X32 = false>
+template <int NW, int KS, int MR, bool ATOM, bool LOOP, typename TZ, typename TX, bool X32 = false, int BITS = 4>
 int launch_dec_inst(hipStream_t st, const DecPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
                     int64_t C, const void *zero, const void *scale, void *out, void *wsp,
                     const int32_t *rowexp = nullptr) {
   typedef std::conditional_t<X32, float, TX> XT;
-  auto kern = qmm_fwd_dec_kernel<NW, KS, MR, ATOM, LOOP, TZ, TX, X32>;
+  auto kern = qmm_fwd_dec_kernel<NW, KS, MR, ATOM, LOOP, TZ, TX, X32, BITS>;
   if (p.lds_bytes > 48 * 1024 && !gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), (int)p.lds_bytes))
     return GPTQ_HIP_ELAUNCH;
   const QmmWs ws = qmm_ws(wsp, p.x1_bytes);
   hipLaunchKernelGGL(kern, dim3((unsigned)p.strips, (unsigned)p.S, 1), dim3(NW * 64), p.lds_bytes, st,
-                     (const XT *)x, (int)M, (int)(2 * R), pk, (int)R, (int)C, (const TZ *)zero,
+                     (const XT *)x, (int)M, (int)(BITS == 4 ? 2 * R : R), pk, (int)R, (int)C, (const TZ *)zero,
                      (const TZ *)scale, (XT *)out, ws, p.S, p.rows, rowexp);
   GPTQ_CHECK_LAUNCH();
   return GPTQ_HIP_OK;
@@ -1029,6 +1062,28 @@ int launch_dec_zx(hipStream_t st, const DecPlan &p, const void *x, int64_t M, co
   if (p.ks == 1) GPTQ_DEC(8, 1, 4, true, false);
   GPTQ_DEC(8, 2, 4, true, false);
 #undef GPTQ_DEC
+}
+
+// 8-bit codes, fp16 activations
+template <typename TZ>
+int launch_dec_z8(hipStream_t st, const DecPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
+                  int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
+#define GPTQ_DEC8(NW, KS, MR, ATOM, LOOP) \
+  return launch_dec_inst<NW, KS, MR, ATOM, LOOP, TZ, __half, false, 8>(st, p, x, M, pk, R, C, zero, scale, out, wsp)
+  if (p.loop) return GPTQ_HIP_EINVAL;
+  if (p.mr == 16) {
+    if (p.atom) GPTQ_DEC8(8, 4, 16, true, false);
+    GPTQ_DEC8(8, 4, 16, false, false);
+  }
+  if (p.mr == 1) {
+    if (p.nw == 16) GPTQ_DEC8(16, 2, 1, true, false);
+    if (p.ks == 1) GPTQ_DEC8(8, 1, 1, true, false);
+    GPTQ_DEC8(8, 2, 1, true, false);
+  }
+  if (p.nw == 16) GPTQ_DEC8(16, 2, 4, true, false);
+  if (p.ks == 1) GPTQ_DEC8(8, 1, 4, true, false);
+  GPTQ_DEC8(8, 2, 4, true, false);
+#undef GPTQ_DEC8
 }
 
 template <typename TZ>
@@ -1881,7 +1936,11 @@ size_t ws16_bytes(int64_t M, int64_t R, int64_t C, int transpose_b, int bits) {
   }
   const RegPlan rp = reg_fwd_plan(M, R, C, bits, true);
   size_t need = rp.use ? rp.total_bytes : 0;
-  if (bits != 4) return need;
+  if (bits != 4) {
+    const DecPlan d8 = dec_plan(M, R, C, 8);
+    if (d8.use && d8.total_bytes > need) need = d8.total_bytes;
+    return need;
+  }
   // which kernel runs also depends on pointer alignment: enough for any of them
   const size_t cand[4] = {fwd_plan(M, R, C, false).total_bytes, gemm_plan(M, R, C).total_bytes,
                           fwd_plan(M, R, C, true).total_bytes, 0};
@@ -1999,6 +2058,19 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
     if (rp.total_bytes && (!ws || ws_bytes < rp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
     return reg_fwd_launch(st, rp, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, out, ws, (int)group_size);
   };
+  if (bits == 8 && !transpose_b && group_size == 0 && x_dtype == GPTQ_HIP_F16 && M <= 16 &&
+      fwd_fast_ok(x_dtype, M, R, C, x, packed) && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    // up to 16 fp16 rows against 8-bit codes: the decode kernel
+    const DecPlan dp = dec_plan(M, R, C, 8);
+    if (dp.use) {
+      if (dp.total_bytes && (!ws || ws_bytes < dp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+      switch (zs_dtype) {
+        case GPTQ_HIP_F32: return launch_dec_z8<float>(st, dp, x, M, packed, R, C, zero, scale, out, ws);
+        case GPTQ_HIP_F16: return launch_dec_z8<__half>(st, dp, x, M, packed, R, C, zero, scale, out, ws);
+        default: return launch_dec_z8<__hip_bfloat16>(st, dp, x, M, packed, R, C, zero, scale, out, ws);
+      }
+    }
+  }
   if (bits == 4 && !transpose_b && group_size == 0) {
     // more than 16 rows: the register-operand kernel, unless its tiles are too few to fill the chip even when
     // split (the tiled kernel below splits finer)

@@ -1,8 +1,9 @@
 // Packed-weight matmul, forward, with both MFMA operands built in registers:
 //   out[M, C] = x[M, K] @ ((code - zero) * scale),  codes packed as 4-bit pairs (K = 2 R) or bytes (K = R).
-// Serves every forward product of more than 16 rows, and below that what the 4-bit decode kernel of
-// qmatmul.hip does not take: 8-bit codes and shapes whose rows are not 8- or 16-byte multiples (C % 8 != 0,
-// e.g. a vocabulary-sized C; K % 8 != 0; unaligned operands).
+// Serves every forward product of more than 16 rows, and below that what the decode kernel of qmatmul.hip
+// does not take: shapes whose rows are not 8- or 16-byte multiples (C % 8 != 0, e.g. a vocabulary-sized C;
+// K % 8 != 0; unaligned operands), and of the 8-bit products those with bf16 activations or a matrix beyond
+// what the decode kernel keeps in flight.
 //
 // A workgroup owns a (16 RB) x 128 output tile (RB = 1, 4 or 8 row blocks) over a range of k-steps (all of K
 // unless the contraction is split over S workgroups) and its four wavefronts split those k-steps among them

@@ -70,6 +70,22 @@ def test_qmatmul_8bit_fp16(OP, M, N, K, transpose):
     _check(got, x.astype(np.float32), qm, transpose)
 
 
+@pytest.mark.parametrize("K,N", [(64, 256), (256, 512), (1024, 16), (4096, 1024), (2048, 8192), (8192, 2048),
+                                 (520, 272)])
+@pytest.mark.parametrize("M", [1, 2, 4, 5, 8, 9, 16])
+def test_qmatmul_8bit_decode_kernel_instantiations(OP, M, K, N):
+    """Up to 16 fp16 rows against aligned 8-bit matrices run on the decode kernel: one, four or sixteen rows of
+    the tile kept, one to four k-steps per wavefront, 8 or 16 wavefronts, with and without a split over K
+    (atomic sum or partial tiles).  Each case three times on the same workspace (the sum's cells must be left
+    zero), with fractional zero points."""
+    qm = _matrix8(11 * M + K + N, K, N, np.float16, frac=True)
+    rng = np.random.default_rng(M + K)
+    for rep in range(3):
+        x = rng.standard_normal((M, K)).astype(np.float16)
+        got = OP.quantized_matmul(x, qm, transpose_b=False)
+        _check(got, x.astype(np.float32), qm, False)
+
+
 @pytest.mark.parametrize("transpose", [False, True])
 @pytest.mark.parametrize("zs", ["float32", "float16", "bfloat16"])
 @pytest.mark.parametrize("xdt", ["float16", "bfloat16", "float32"])
