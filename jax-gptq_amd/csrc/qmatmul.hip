@@ -518,6 +518,29 @@ __global__ __launch_bounds__(256, 2) void qmm_fwd_stream_kernel(
                            out, ws, se, so);
 }
 
+// 16 bytes from an address of any alignment
+struct __attribute__((packed, aligned(1))) QdU4 { uint32_t x, y, z, w; };
+template <bool UNALIGNED>
+__device__ __forceinline__ uint4 qd_load16(const void *p) {
+  if (UNALIGNED) {
+    QdU4 v;
+    __builtin_memcpy(&v, p, 16);
+    return make_uint4(v.x, v.y, v.z, v.w);
+  }
+  return *reinterpret_cast<const uint4 *>(p);
+}
+// the 16 bytes of v moved down by `bytes` (0 .. 15) places, zeros from above
+__device__ __forceinline__ uint4 qd_shr_bytes16(uint4 v, int bytes) {
+  const int ws = bytes >> 2;
+  const uint32_t bs = (uint32_t)(bytes & 3);
+  const uint32_t w0 = ws == 0 ? v.x : (ws == 1 ? v.y : (ws == 2 ? v.z : v.w));
+  const uint32_t w1 = ws == 0 ? v.y : (ws == 1 ? v.z : (ws == 2 ? v.w : 0u));
+  const uint32_t w2 = ws == 0 ? v.z : (ws == 1 ? v.w : 0u);
+  const uint32_t w3 = ws == 0 ? v.w : 0u;
+  return make_uint4(__builtin_amdgcn_alignbyte(w1, w0, bs), __builtin_amdgcn_alignbyte(w2, w1, bs),
+                    __builtin_amdgcn_alignbyte(w3, w2, bs), __builtin_amdgcn_alignbyte(0u, w3, bs));
+}
+
 // ---------------------------------------------------------------------------- MFMA path, decode
 // M <= 16 on matrices that the chip holds in flight (up to ~50 MB packed).  Same operands and
 // arithmetic as qmm_fwd_mfma_kernel; what differs is everything around the MFMAs, which is where
@@ -552,7 +575,11 @@ constexpr int QD_MAX_SPLITS = 32;
 //  * BITS = 8 (fp16 activations): a k-step is 32 rows of one code per byte, eight 16-byte rows per lane; two
 //    rows' bytes become {1024 + a, 1024 + b} with a byte permute and an or, the activations enter as they
 //    are, and all offsets leave through one activation sum (the odd-k sum stays zero).
-template <int NW, int KS, int MR, bool ATOM, bool LOOP, typename TZ, typename TX, bool X32 = false, int BITS = 4>
+//  * RAGC (ATOM only): rows of any length C >= 16, so rows that start anywhere: unaligned 16-byte loads, and in the
+//    last strip a lane whose 16 channels would reach past the row loads the row's last 16 bytes instead and
+//    shifts them into place (a wave-uniform branch; the other strips run the code of the aligned form).
+template <int NW, int KS, int MR, bool ATOM, bool LOOP, typename TZ, typename TX, bool X32 = false, int BITS = 4,
+          bool RAGC = false>
 __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
     const std::conditional_t<X32, float, TX> *x, int M, int K, const uint8_t *pk, int R, int C, const TZ *zero,
     const TZ *scale, std::conditional_t<X32, float, TX> *out, QmmWs ws, int S, int rows_per_split,
@@ -560,6 +587,7 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
   constexpr bool BF = Act<TX>::BF;
   static_assert(!X32 || (ATOM && !BF), "fp32 rows: fp16 arithmetic and the atomic sum only");
   static_assert(BITS == 4 || (BITS == 8 && !BF && !X32), "8-bit codes: fp16 activations");
+  static_assert(!RAGC || (ATOM && !X32 && BITS == 4), "ragged rows: 4-bit codes, the atomic sum");
   constexpr int NR = BITS == 4 ? 4 : 8;          // rows per lane and k-step
   constexpr int RPS = 4 * NR;                    // rows per k-step of a wavefront
   constexpr int XK = BITS == 4 ? 2 : 1;          // k per row
@@ -594,13 +622,17 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
   const XT *xr = x + (int64_t)(m0 + (m_ok ? l16 : 0)) * K;
   const int col0 = min(strip * QSTRIP + 16 * l16, C - 16);
   const uint8_t *wp = pk + col0;
+  // RAGC: bytes by which this lane's loads start before its first channel (its channels past the row's end, if
+  // any, are never stored); only the last strip has such lanes
+  const int rag_shift = RAGC ? max(0, min(strip * QSTRIP + 16 * l16, C - 1) - col0) : 0;
+  const bool rag_strip = RAGC && strip * QSTRIP + QSTRIP > C;
   auto issue = [&](Step &st, int t) __attribute__((always_inline)) {
     const int rbase = r_begin + (t * NW + wave) * RPS + NR * g;
     st.pr = *reinterpret_cast<const uint4 *>(xr + XK * min(rbase, R - NR));
     if (X32) st.pr2 = *reinterpret_cast<const uint4 *>(xr + XK * min(rbase, R - NR) + 4);
     const uint8_t *row = wp + (int64_t)min(rbase, R - NR) * C;      // R % NR == 0: the rows are inside the matrix
 #pragma unroll
-    for (int i = 0; i < NR; ++i) st.d[i] = *reinterpret_cast<const uint4 *>(row + (int64_t)i * C);
+    for (int i = 0; i < NR; ++i) st.d[i] = qd_load16<RAGC>(row + (int64_t)i * C);
   };
 
   const DqConst dqk = dq_const<BF>();
@@ -612,6 +644,12 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
   int xe = 0;                                     // X32: exponent of this lane's row scale
   auto consume = [&](Step &st, int t) __attribute__((always_inline)) {
     uint4 pr = st.pr;
+    if constexpr (RAGC) {
+      if (rag_strip) {
+#pragma unroll
+        for (int i = 0; i < NR; ++i) st.d[i] = qd_shr_bytes16(st.d[i], rag_shift);
+      }
+    }
     if constexpr (X32) {
       // eight fp32 activations -> fp16 of the scaled row, round to nearest even
       const uint32_t f[8] = {st.pr.x, st.pr.y, st.pr.z, st.pr.w, st.pr2.x, st.pr2.y, st.pr2.z, st.pr2.w};
@@ -921,12 +959,12 @@ struct DecPlan {
   size_t lds_bytes, x1_bytes, part_bytes, total_bytes;
 };
 
-DecPlan dec_plan(int64_t M, int64_t R8, int64_t C, int bits = 4) {
+DecPlan dec_plan(int64_t M, int64_t R8, int64_t C, int bits = 4, bool ragged_c = false) {
   DecPlan p{};
   // 8-bit codes: planned in k-steps like a 4-bit matrix of half the rows (a k-step carries twice the bytes)
   if (bits == 8 && R8 % 8 != 0) return p;
   const int64_t R = bits == 8 ? R8 / 2 : R8;
-  if (M < 1 || M > 16 || R % 4 != 0 || C % 16 != 0 || C < 16 || R >= (1LL << 30) || C >= (1LL << 30)) return p;
+  if (M < 1 || M > 16 || R % 4 != 0 || (C % 16 != 0 && !(ragged_c && bits == 4)) || C < 16 || R >= (1LL << 30) || C >= (1LL << 30)) return p;
   p.strips = (int)ceil_div64(C, QSTRIP);
   if (p.strips > QMM_MAX_COUNTERS) return p;
   p.mr = M == 1 ? 1 : (M <= 4 ? 4 : 16);
@@ -988,6 +1026,7 @@ DecPlan dec_plan(int64_t M, int64_t R8, int64_t C, int bits = 4) {
     }
   }
   p.lds_bytes = ((size_t)p.nw * p.mr * QSTRIP + (size_t)p.nw * 32 + 32) * sizeof(float);
+  if (C % 16 != 0 && !p.atom) return DecPlan{};      // ragged rows: instantiated for the atomic sum only
   if (bits == 8) {
     // (the ring-loop forms of the 8-bit instantiation do not fit their register budgets: those matrices stay
     // with the register-operand kernel)
@@ -998,12 +1037,13 @@ DecPlan dec_plan(int64_t M, int64_t R8, int64_t C, int bits = 4) {
   return p;
 }
 
-template <int NW, int KS, int MR, bool ATOM, bool LOOP, typename TZ, typename TX, bool X32 = false, int BITS = 4>
+template <int NW, int KS, int MR, bool ATOM, bool LOOP, typename TZ, typename TX, bool X32 = false, int BITS = 4,
+          bool RAGC = false>
 int launch_dec_inst(hipStream_t st, const DecPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
                     int64_t C, const void *zero, const void *scale, void *out, void *wsp,
                     const int32_t *rowexp = nullptr) {
   typedef std::conditional_t<X32, float, TX> XT;
-  auto kern = qmm_fwd_dec_kernel<NW, KS, MR, ATOM, LOOP, TZ, TX, X32, BITS>;
+  auto kern = qmm_fwd_dec_kernel<NW, KS, MR, ATOM, LOOP, TZ, TX, X32, BITS, RAGC>;
   if (p.lds_bytes > 48 * 1024 && !gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), (int)p.lds_bytes))
     return GPTQ_HIP_ELAUNCH;
   const QmmWs ws = qmm_ws(wsp, p.x1_bytes);
@@ -1062,6 +1102,37 @@ int launch_dec_zx(hipStream_t st, const DecPlan &p, const void *x, int64_t M, co
   if (p.ks == 1) GPTQ_DEC(8, 1, 4, true, false);
   GPTQ_DEC(8, 2, 4, true, false);
 #undef GPTQ_DEC
+}
+
+// 4-bit codes, rows of any length (plans with the atomic sum)
+template <typename TZ, typename TX>
+int launch_dec_zx_rag(hipStream_t st, const DecPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
+                      int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
+#define GPTQ_DECR(NW, KS, MR, LOOP) \
+  return launch_dec_inst<NW, KS, MR, true, LOOP, TZ, TX, false, 4, true>(st, p, x, M, pk, R, C, zero, scale, out, wsp)
+  if (!p.atom) return GPTQ_HIP_EINVAL;
+  if (p.mr == 16) {
+    if (p.loop) GPTQ_DECR(8, 4, 16, true);
+    GPTQ_DECR(8, 4, 16, false);
+  }
+  if (p.mr == 1) {
+    if (p.loop) GPTQ_DECR(16, 2, 1, true);
+    if (p.nw == 16) GPTQ_DECR(16, 2, 1, false);
+    if (p.ks == 1) GPTQ_DECR(8, 1, 1, false);
+    GPTQ_DECR(8, 2, 1, false);
+  }
+  if (p.loop) GPTQ_DECR(16, 2, 4, true);
+  if (p.nw == 16) GPTQ_DECR(16, 2, 4, false);
+  if (p.ks == 1) GPTQ_DECR(8, 1, 4, false);
+  GPTQ_DECR(8, 2, 4, false);
+#undef GPTQ_DECR
+}
+template <typename TZ>
+int launch_dec_z_rag(hipStream_t st, const DecPlan &p, const void *x, int x_dtype, int64_t M, const uint8_t *pk,
+                     int64_t R, int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
+  if (x_dtype == GPTQ_HIP_BF16)
+    return launch_dec_zx_rag<TZ, __hip_bfloat16>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
+  return launch_dec_zx_rag<TZ, __half>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
 }
 
 // 8-bit codes, fp16 activations
@@ -1947,6 +2018,8 @@ size_t ws16_bytes(int64_t M, int64_t R, int64_t C, int transpose_b, int bits) {
   for (size_t c : cand) need = c > need ? c : need;
   const DecPlan dp = dec_plan(M, R, C);
   if (dp.use && dp.total_bytes > need) need = dp.total_bytes;
+  const DecPlan dr = dec_plan(M, R, C, 4, true);
+  if (dr.use && dr.total_bytes > need) need = dr.total_bytes;
   return need;
 }
 
@@ -2068,6 +2141,21 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
         case GPTQ_HIP_F32: return launch_dec_z8<float>(st, dp, x, M, packed, R, C, zero, scale, out, ws);
         case GPTQ_HIP_F16: return launch_dec_z8<__half>(st, dp, x, M, packed, R, C, zero, scale, out, ws);
         default: return launch_dec_z8<__hip_bfloat16>(st, dp, x, M, packed, R, C, zero, scale, out, ws);
+      }
+    }
+  }
+  if (bits == 4 && !transpose_b && group_size == 0 && M <= 16 && C % 16 != 0 && R % 4 == 0 &&
+      (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 1) == 0) {
+    // up to 16 rows against rows that are no multiple of 16 channels (a vocabulary-sized C): the decode kernel's
+    // form for rows of any length and alignment
+    const DecPlan dp = dec_plan(M, R, C, 4, true);
+    if (dp.use) {
+      if (dp.total_bytes && (!ws || ws_bytes < dp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+      switch (zs_dtype) {
+        case GPTQ_HIP_F32: return launch_dec_z_rag<float>(st, dp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
+        case GPTQ_HIP_F16: return launch_dec_z_rag<__half>(st, dp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
+        default:
+          return launch_dec_z_rag<__hip_bfloat16>(st, dp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
       }
     }
   }

@@ -49,6 +49,22 @@ def test_qmatmul_random_cases_with_many_column_tiles(seed):
     _run_cases(np.random.default_rng(2000 + seed), _wide_case, 14)
 
 
+def _ragged_decode_case(rng):
+    """Up to 16 rows, 4-bit, K a multiple of 8, N no multiple of 16: the decode kernel's form for rows of any
+    length (unaligned row starts; a last strip whose lanes reach past the row), from tiny to vocabulary-sized."""
+    M = int(rng.choice([1, 2, 3, 4, 5, 8, 9, 16]))
+    K = int(rng.choice([8, 64, 128, 256, 520, 768, 1024, 4096]))
+    N = int(rng.choice([17, 31, 100, 255, 257, 300, 909, 1000, 4097, 8193, 50257]))
+    xdt = str(rng.choice(["float16", "bfloat16"]))
+    zs = str(rng.choice(["float32", "float16", "bfloat16"]))
+    return 4, M, K, N, False, xdt, zs, 0, int(rng.integers(0, 2))
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_qmatmul_random_cases_few_rows_ragged_columns(seed):
+    _run_cases(np.random.default_rng(3000 + seed), _ragged_decode_case, 30)
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_qmatmul_random_cases(seed):
     _run_cases(np.random.default_rng(1000 + seed), _case, 25)
