@@ -14,6 +14,7 @@ struct RegPlan {
   bool atom;               // 16-row tiles: the splits add their results to 64-bit fixed-point cells (one returning
                            // atomic per output) instead of writing partial tiles and taking a ticket
   int64_t tiles;           // output tiles of one launch
+  int tail_x;              // 128-row tiles: this many trailing column tiles run on 64-row tiles in a second launch
   size_t part_bytes, total_bytes;
 };
 

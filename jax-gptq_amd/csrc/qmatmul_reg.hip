@@ -37,7 +37,7 @@ __global__ __launch_bounds__(256, (RB == 1 ? 2 : 1)) void qmm_fwd_reg_kernel(con
                                                           int C, const void *zero, const void *scale,
                                                           int zs_dtype, TX *out, float *part, int32_t *counters,
                                                           int S, int steps_per_split, int group_size,
-                                                          unsigned long long *acc64) {
+                                                          unsigned long long *acc64, int tx0) {
   constexpr bool BF = Act<TX>::BF && !GROUPED;      // grouped: the fp16 form of the dequantisation for both types
   // vector instructions between two MFMAs of the main loop (0: compiler's order)
   constexpr int SCHED = (RB == 4 && (GROUPED || RAGGED)) ? 4 : 0;
@@ -54,12 +54,13 @@ __global__ __launch_bounds__(256, (RB == 1 ? 2 : 1)) void qmm_fwd_reg_kernel(con
   // every kernel argument in registers before the first address is formed (left to itself the compiler
   // fetches them in groups where they are first used, and waits for each group)
   asm volatile("" ::"s"(x), "s"(pk), "s"(zero), "s"(scale), "s"(out), "s"(part), "s"(counters), "s"(M), "s"(K),
-               "s"(R), "s"(C), "s"(zs_dtype), "s"(S), "s"(steps_per_split), "s"(group_size), "s"(acc64));
+               "s"(R), "s"(C), "s"(zs_dtype), "s"(S), "s"(steps_per_split), "s"(group_size), "s"(acc64), "s"(tx0));
   const int tid = threadIdx.x, lane = tid & 63, wk = tid >> 6;
   const int g = lane >> 4, l16 = lane & 15;
   int tx, ty;
   qmm_tile_coords(tx, ty);
-  const int m0 = ty * (16 * RB), nbase = tx * RG_BN, split = blockIdx.z;
+  // (tx0: first column tile of this launch, where the columns are dealt over two launches)
+  const int m0 = ty * (16 * RB), nbase = (tx + tx0) * RG_BN, split = blockIdx.z;
   const int T = (K + 31) >> 5;
   // this workgroup's k-steps [t_begin, t_end); wavefront wk takes t_begin + wk, + 4, ...
   const int t_begin = split * steps_per_split, t_end = min(T, t_begin + steps_per_split);
@@ -439,7 +440,8 @@ __global__ __launch_bounds__(256, (RB == 1 ? 2 : 1)) void qmm_fwd_reg_kernel(con
 
 template <int BITS, int RB, int RING, bool RAGGED, typename TX, bool GROUPED>
 int launch_inst(hipStream_t st, const RegPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
-                int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *wsp, int group_size) {
+                int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *wsp, int group_size,
+                int64_t tx0 = 0, int64_t ntx = -1) {
   constexpr size_t lds = (size_t)4 * (RB > 4 ? 4 : RB) * RG_NT * RG_TILE_FLOATS * sizeof(float);
   auto kern = qmm_fwd_reg_kernel<BITS, RB, RING, RAGGED, TX, GROUPED>;
   if (lds > 64 * 1024 && !gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), (int)lds)) return GPTQ_HIP_ELAUNCH;
@@ -448,19 +450,22 @@ int launch_inst(hipStream_t st, const RegPlan &p, const void *x, int64_t M, cons
   float *part = reinterpret_cast<float *>(reinterpret_cast<char *>(wsp) + QMM_HEAD_BYTES);
   unsigned long long *acc64 =
       p.atom ? reinterpret_cast<unsigned long long *>(reinterpret_cast<char *>(wsp) + QMM_COUNTER_BYTES) : nullptr;
-  const int64_t tiles_x = ceil_div64(C, RG_BN);
+  // column tiles [tx0, tx0 + ntx) (all of them unless the plan deals the columns over two launches)
+  const int64_t tiles_all = ceil_div64(C, RG_BN);
+  const int64_t tiles_x = ntx < 0 ? tiles_all : ntx;
   // rows per launch: 32-bit element offsets into x, grid.y, one arrival counter per tile, the partial region
   int64_t rows_max = ((1LL << 31) - 1) / K;
   if (rows_max > 65535LL * 16 * RB) rows_max = 65535LL * 16 * RB;
-  const int64_t tiles_y_max = p.tiles / tiles_x;                       // what the plan sized the workspace for
-  if (rows_max > tiles_y_max * 16 * RB) rows_max = tiles_y_max * 16 * RB;
+  const int64_t tiles_y_max = p.tiles / tiles_all;                     // what the plan sized the workspace for
+  if (p.S > 1 && rows_max > tiles_y_max * 16 * RB) rows_max = tiles_y_max * 16 * RB;
   rows_max -= rows_max % (16 * RB);
   if (rows_max < 16 * RB) return GPTQ_HIP_EINVAL;
   for (int64_t r0 = 0; r0 < M; r0 += rows_max) {
     const int64_t rows = M - r0 < rows_max ? M - r0 : rows_max;
     const dim3 grid((unsigned)tiles_x, (unsigned)ceil_div64(rows, 16 * RB), (unsigned)p.S);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (const TX *)x + r0 * K, (int)rows, (int)K, pk, (int)R,
-                       (int)C, zero, scale, zs_dtype, (TX *)out + r0 * C, part, counters, p.S, p.steps, group_size, acc64);
+                       (int)C, zero, scale, zs_dtype, (TX *)out + r0 * C, part, counters, p.S, p.steps, group_size, acc64,
+                       (int)tx0);
     GPTQ_CHECK_LAUNCH();
   }
   return GPTQ_HIP_OK;
@@ -486,6 +491,20 @@ int launch_bx(hipStream_t st, const RegPlan &p, const void *x, int64_t M, const 
   }
   // a ring of two k-steps for 128-row tiles, of three for 64-row tiles (registers), of six for the 16-row tiles
   // of the decode case
+  if (p.rb == 8 && p.tail_x > 0) {
+    // 128-row tiles on the columns that fill whole rounds of workgroups, 64-row tiles on the rest
+    const int64_t main_x = ceil_div64(C, RG_BN) - p.tail_x;
+    const int rc = p.ragged ? launch_inst<BITS, 8, 2, true, TX, false>(st, p, x, M, pk, R, C, zero, scale, zs_dtype,
+                                                                         out, ws, group_size, 0, main_x)
+                            : launch_inst<BITS, 8, 3, false, TX, false>(st, p, x, M, pk, R, C, zero, scale, zs_dtype,
+                                                                          out, ws, group_size, 0, main_x);
+    if (rc) return rc;
+    if (p.ragged)
+      return launch_inst<BITS, 4, 3, true, TX, false>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws,
+                                                      group_size, main_x, p.tail_x);
+    return launch_inst<BITS, 4, 3, false, TX, false>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws,
+                                                     group_size, main_x, p.tail_x);
+  }
   if (p.rb == 8) {
     if (p.ragged) GPTQ_REG(8, 2, true, false);
     GPTQ_REG(8, 3, false, false);
@@ -530,6 +549,18 @@ RegPlan reg_fwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned) {
   }
   p.steps = (int)ceil_div64(T, S);
   p.S = (int)ceil_div64(T, p.steps);
+  // 128-row tiles whose last round of workgroups would be at most half full (one workgroup per CU): the
+  // columns that fill whole rounds keep them, the remaining column tiles run on 64-row tiles in a second
+  // launch, one partial round of half-sized tiles (M = 2048 on 4096 x 11008: 80 + 6 column tiles, 5 rounds +
+  // 192 workgroups instead of 5.4 -> 6 rounds).  Rounds have to be long for the second launch to pay.
+  p.tail_x = 0;
+  if (p.rb == 8 && p.S == 1 && T >= 64) {
+    const int64_t all = tiles_x * tiles_y, full = all / 256, rem = all % 256;
+    if (full >= 1 && rem > 0 && rem <= 128) {
+      const int64_t main_x = full * 256 / tiles_y, tail = tiles_x - main_x;
+      if (main_x >= 1 && tail >= 1 && tail * tiles_y * 2 <= 256) p.tail_x = (int)tail;
+    }
+  }
   // 16-row tiles (one launch, M <= 16): the atomic sum where the cells hold the output and the atomics are few
   // (the memory side retires them at a limited rate: 900000 of them cost what the ticket path costs on
   // 4096 x 11008 and 4 us more on 7168 x 28672)
