@@ -27,7 +27,7 @@
 namespace {
 
 constexpr int SOLVE_CH = 64;               // channels per workgroup (one per lane)
-constexpr int SOLVE_NW = 8;                // wavefronts per workgroup (4: 45 us per block, 8: 40, 16: 52)
+constexpr int SOLVE_NW = 8;                // wavefronts per workgroup: one runs the chains, seven update and store
 constexpr int SOLVE_TPB = SOLVE_CH * SOLVE_NW;
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
@@ -49,7 +49,7 @@ __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
   // Wb, Qb, cb: first row of the block in W, Q, codes; Lb: the block's diagonal corner of L
 #pragma clang fp contract(off)
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  float *Ln = smem;                         // Ln[j * bs + i] = Lb[j][i]
+  float *Ln = smem;                         // Ln[j * bs + i] = Lb[j][i] for i <= j (nothing right of the diagonal is read)
   float *Wl = Ln + bs * bs;                 // Wl[j * SOLVE_CH + lane] = W[block row j][channel]
   float *Es = Wl + bs * SOLVE_CH;           // [2][SB][SOLVE_CH] errors of a sub-block (two sub-blocks alternate)
   float *Qs = Es + 2 * SB * SOLVE_CH;       // the same for the codes
