@@ -2059,9 +2059,12 @@ bool aligned16(const void *a, const void *b) {
 
 // group_size = 0: zero / scale [C]; group_size > 0: zero / scale [K / group_size, C] (register-operand kernels,
 // whose k-steps of 32 and tiles of 128 output columns must not straddle a group, or the plain kernels)
+// out32 / rowexp / wrote32 (the recursive call for fp32 rows): where the product runs on register-operand tiles of
+// more than 16 rows it stores the fp32 result itself (RegPlan::out32) and sets *wrote32
 int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed, int64_t R, int64_t C,
                  const void *zero, const void *scale, int zs_dtype, int bits, int64_t group_size, int transpose_b,
-                 void *out, void *ws, size_t ws_bytes) {
+                 void *out, void *ws, size_t ws_bytes, float *out32 = nullptr, const int32_t *rowexp = nullptr,
+                 bool *wrote32 = nullptr) {
   if (M < 0 || R <= 0 || C <= 0 || (bits != 4 && bits != 8)) return GPTQ_HIP_EINVAL;
   if (group_size < 0 || group_size % 2 != 0 || (group_size > 0 && (bits == 4 ? 2 * R : R) % group_size != 0) ||
       group_size > (1LL << 30))
@@ -2108,9 +2111,15 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
         hipLaunchKernelGGL(x32_to_f16_rows_kernel, dim3((unsigned)mm), dim3(256), 0, st,
                            reinterpret_cast<const float *>(x) + r0 * kin, kin, x16, rowexp);
         GPTQ_CHECK_LAUNCH();
+        bool wrote = false;
         const int rc = qmatmul_impl(stream, x16, GPTQ_HIP_F16, mm, packed, R, C, zero, scale, zs_dtype, bits,
-                                    group_size, transpose_b, o16, ws, fp.inner);
+                                    group_size, transpose_b, o16, ws, fp.inner,
+                                    (transpose_b || (reinterpret_cast<uintptr_t>(out) & 15) != 0)
+                                        ? nullptr
+                                        : reinterpret_cast<float *>(out) + r0 * nout,
+                                    rowexp, &wrote);
         if (rc) return rc;
+        if (wrote) continue;                  // the product's tiles stored the fp32 rows themselves
         unsigned gx = (unsigned)ceil_div64(nout, 1024);
         if (gx > 64) gx = 64;
         hipLaunchKernelGGL(f16_rows_to_f32_kernel, dim3(gx, (unsigned)mm), dim3(256), 0, st, o16, nout,
@@ -2129,7 +2138,13 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
   const RegPlan rp = (transpose_b || !reg_groups_ok) ? RegPlan{} : reg_fwd_plan(M, R, C, bits, al);
   auto run_reg_fwd = [&]() -> int {
     if (rp.total_bytes && (!ws || ws_bytes < rp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
-    return reg_fwd_launch(st, rp, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, out, ws, (int)group_size);
+    RegPlan q = rp;
+    if (out32 && rowexp && wrote32 && rp.rb > 1 && x_dtype == GPTQ_HIP_F16) {
+      q.out32 = out32;
+      q.rowexp = rowexp;
+      *wrote32 = true;
+    }
+    return reg_fwd_launch(st, q, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, out, ws, (int)group_size);
   };
   if (bits == 8 && !transpose_b && group_size == 0 && x_dtype == GPTQ_HIP_F16 && M <= 16 &&
       fwd_fast_ok(x_dtype, M, R, C, x, packed) && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {

@@ -15,6 +15,11 @@ struct RegPlan {
                            // atomic per output) instead of writing partial tiles and taking a ticket
   int64_t tiles;           // output tiles of one launch
   int tail_x;              // 128-row tiles: this many trailing column tiles run on 64-row tiles in a second launch
+  // Not part of the plan proper; set by the caller for a product whose activations were fp32 rows scaled by
+  // 2^-rowexp[m] and rounded to fp16: tiles of more than 16 rows then store ldexp(fp16(result), rowexp[m]) as
+  // fp32 into out32 [M, C] instead of fp16 into `out`.
+  float *out32;
+  const int32_t *rowexp;
   size_t part_bytes, total_bytes;
 };
 

@@ -37,7 +37,8 @@ __global__ __launch_bounds__(256, (RB == 1 ? 2 : 1)) void qmm_fwd_reg_kernel(con
                                                           int C, const void *zero, const void *scale,
                                                           int zs_dtype, TX *out, float *part, int32_t *counters,
                                                           int S, int steps_per_split, int group_size,
-                                                          unsigned long long *acc64, int tx0) {
+                                                          unsigned long long *acc64, int tx0, float *out32,
+                                                          const int32_t *rowexp) {
   constexpr bool BF = Act<TX>::BF && !GROUPED;      // grouped: the fp16 form of the dequantisation for both types
   // vector instructions between two MFMAs of the main loop (0: compiler's order)
   constexpr int SCHED = (RB == 4 && (GROUPED || RAGGED)) ? 4 : 0;
@@ -421,6 +422,23 @@ __global__ __launch_bounds__(256, (RB == 1 ? 2 : 1)) void qmm_fwd_reg_kernel(con
       TX o[8];
 #pragma unroll
       for (int t8 = 0; t8 < 8; ++t8) o[t8] = Act<TX>::out(sca[t8] * (sum[t8][r] - zfa[t8] * rs));
+      if (out32 != nullptr) {
+        // fp32 rows: the fp16 result widened and scaled back by the row's power of two (exact)
+        const int e = rowexp[m];
+        float *d32 = out32 + (int64_t)m * C + col;
+        float f[8];
+#pragma unroll
+        for (int t8 = 0; t8 < 8; ++t8) f[t8] = ldexpf((float)o[t8], e);
+        if (RAGGED) {
+#pragma unroll
+          for (int t8 = 0; t8 < 8; ++t8)
+            if (col + t8 < C) d32[t8] = f[t8];
+        } else {
+          *reinterpret_cast<float4 *>(d32) = make_float4(f[0], f[1], f[2], f[3]);
+          *reinterpret_cast<float4 *>(d32 + 4) = make_float4(f[4], f[5], f[6], f[7]);
+        }
+        continue;
+      }
       TX *dst = out + (int64_t)m * C + col;
       if (RAGGED) {
 #pragma unroll
@@ -465,7 +483,7 @@ int launch_inst(hipStream_t st, const RegPlan &p, const void *x, int64_t M, cons
     const dim3 grid((unsigned)tiles_x, (unsigned)ceil_div64(rows, 16 * RB), (unsigned)p.S);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (const TX *)x + r0 * K, (int)rows, (int)K, pk, (int)R,
                        (int)C, zero, scale, zs_dtype, (TX *)out + r0 * C, part, counters, p.S, p.steps, group_size, acc64,
-                       (int)tx0);
+                       (int)tx0, (RB > 1 && p.out32) ? p.out32 + r0 * C : nullptr, p.rowexp ? p.rowexp + r0 : nullptr);
     GPTQ_CHECK_LAUNCH();
   }
   return GPTQ_HIP_OK;
