@@ -1941,10 +1941,31 @@ __global__ __launch_bounds__(256) void x32_to_f16_rows_kernel(const float *x, in
   const float *xr = x + m * kin;
   __half *dst = x16 + m * kin;
   __shared__ float smax[4];
+  constexpr int VR = 16;                       // 16-byte loads per thread that the one-pass form keeps in registers
+  // rows of up to 16384 elements, 16-byte aligned: read once, all loads in flight together
+  const bool one_pass = (kin & 3) == 0 && kin <= 256 * 4 * VR && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+  float4 v[VR];
   float amax = 0.f;
-  for (int64_t k = threadIdx.x; k < kin; k += 256) {
-    const float a = fabsf(xr[k]);
+  auto see = [&](float f) __attribute__((always_inline)) {
+    const float a = fabsf(f);
     amax = (a <= 3.4028235e38f && a > amax) ? a : amax;   // NaN and infinity do not set the scale
+  };
+  if (one_pass) {
+    const int64_t last = kin - 4;
+#pragma unroll
+    for (int i = 0; i < VR; ++i) {
+      const int64_t k = (int64_t)(i * 256 + threadIdx.x) * 4;
+      v[i] = *reinterpret_cast<const float4 *>(xr + (k < kin ? k : last));
+    }
+#pragma unroll
+    for (int i = 0; i < VR; ++i) {
+      see(v[i].x);
+      see(v[i].y);
+      see(v[i].z);
+      see(v[i].w);
+    }
+  } else {
+    for (int64_t k = threadIdx.x; k < kin; k += 256) see(xr[k]);
   }
   for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
   if ((threadIdx.x & 63) == 0) smax[threadIdx.x >> 6] = amax;
@@ -1953,7 +1974,19 @@ __global__ __launch_bounds__(256) void x32_to_f16_rows_kernel(const float *x, in
   int ex = 0;
   (void)frexpf(amax, &ex);                    // 2^(ex-1) <= amax < 2^ex
   const int e = amax > 0.f ? ex - 2 : 0;      // largest magnitude of the scaled row in [2, 4)
-  for (int64_t k = threadIdx.x; k < kin; k += 256) dst[k] = __float2half_rn(ldexpf(xr[k], -e));
+  if (one_pass) {
+#pragma unroll
+    for (int i = 0; i < VR; ++i) {
+      const int64_t k = (int64_t)(i * 256 + threadIdx.x) * 4;
+      if (k < kin) {
+        const __half h[4] = {__float2half_rn(ldexpf(v[i].x, -e)), __float2half_rn(ldexpf(v[i].y, -e)),
+                             __float2half_rn(ldexpf(v[i].z, -e)), __float2half_rn(ldexpf(v[i].w, -e))};
+        *reinterpret_cast<uint2 *>(dst + k) = *reinterpret_cast<const uint2 *>(h);
+      }
+    }
+  } else {
+    for (int64_t k = threadIdx.x; k < kin; k += 256) dst[k] = __float2half_rn(ldexpf(xr[k], -e));
+  }
   if (threadIdx.x == 0) rowexp[m] = e;
 }
 
