@@ -1995,9 +1995,29 @@ __global__ __launch_bounds__(256) void x32_rowexp_kernel(const float *x, int64_t
   const float *xr = x + (int64_t)blockIdx.x * kin;
   __shared__ float smax[4];
   float amax = 0.f;
-  for (int64_t k = threadIdx.x; k < kin; k += 256) {
-    const float a = fabsf(xr[k]);
+  auto see = [&](float f) __attribute__((always_inline)) {
+    const float a = fabsf(f);
     amax = (a <= 3.4028235e38f && a > amax) ? a : amax;   // NaN and infinity do not set the scale
+  };
+  if ((kin & 3) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    // 16-byte loads, four of a thread in flight together
+    for (int64_t k0 = (int64_t)threadIdx.x * 4; k0 < kin; k0 += 4 * 1024) {
+      float4 v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int64_t k = k0 + i * 1024;
+        v[i] = *reinterpret_cast<const float4 *>(xr + (k < kin ? k : kin - 4));
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        see(v[i].x);
+        see(v[i].y);
+        see(v[i].z);
+        see(v[i].w);
+      }
+    }
+  } else {
+    for (int64_t k = threadIdx.x; k < kin; k += 256) see(xr[k]);
   }
   for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
   if ((threadIdx.x & 63) == 0) smax[threadIdx.x >> 6] = amax;
