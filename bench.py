@@ -195,13 +195,17 @@ def bench_qmatmul(reps=240):
                  (2048, 1, "float16")]
         if K == K_IN and bits == 4:
             cases += [(1, 0, "bfloat16"), (16, 0, "bfloat16"), (2048, 1, "bfloat16")]
+            # fp32 rows in and out (what a JAX caller of the reference passes by default): rounded to fp16
+            # precision on the way in, as the reference's dot rounds them to TF32
+            cases += [(1, 0, "float32"), (128, 0, "float32")]
         if K * N >= (1 << 27):
             cases = [(1, 0, "float16"), (16, 0, "float16")]
         if N % 16:
             cases = [(1, 0, "float16"), (16, 0, "float16"), (512, 0, "float16"), (512, 1, "float16")]
         for (M, tr, xdt) in cases:
             tdt = getattr(torch, xdt)
-            xcode = _native.F16 if xdt == "float16" else _native.BF16
+            xcode = {"float16": _native.F16, "bfloat16": _native.BF16, "float32": _native.F32}[xdt]
+            esz = 4 if xdt == "float32" else 2
             x = torch.randn((M, N if tr else K), generator=g, device="cuda").to(tdt)
             y = torch.empty((M, K if tr else N), dtype=tdt, device="cuda")
             ws = torch.zeros(max(lib.gptq_hip_qmatmul_bits_workspace_bytes(M, R, N, tr, xcode, bits), 256),
@@ -230,7 +234,7 @@ def bench_qmatmul(reps=240):
             e1.record()
             torch.cuda.synchronize()
             us_cached = e0.elapsed_time(e1) * 1e3 / reps
-            nbytes = R * N + 2 * N * 2 + M * K * 2 + M * N * 2
+            nbytes = R * N + 2 * N * 2 + M * K * esz + M * N * esz
             out.append({"M": M, "K": K, "N": N, "bits": bits, "transpose_b": tr, "x_dtype": xdt, "us": round(us, 2),
                         "us_cache_resident": round(us_cached, 2),
                         "algorithmic_bytes": nbytes,
