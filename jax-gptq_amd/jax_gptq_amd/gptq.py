@@ -25,8 +25,14 @@ _DT_H = {torch.float32: N.F32, torch.float64: N.F64}       # element types of H 
 _DT_X64 = {**_DT, torch.float64: N.F64}                    # batches of the fp64 Hessian
 
 
+_HAVE_GPU = None       # torch.cuda.is_available(), asked once (it reads the environment on every call)
+
+
 def _device():
-    if not torch.cuda.is_available():
+    global _HAVE_GPU
+    if _HAVE_GPU is None:
+        _HAVE_GPU = bool(torch.cuda.is_available())
+    if not _HAVE_GPU:
         raise RuntimeError("jax_gptq_amd needs a ROCm GPU (gfx950); there is no CPU path")
     return torch.device("cuda", torch.cuda.current_device())
 
@@ -35,6 +41,11 @@ def _dev(x, dtype=None):
     """Array-like -> contiguous tensor on the current GPU."""
     if isinstance(x, torch.Tensor):
         t = x
+        # the common case of the per-call operators: already in place
+        if t.is_cuda and t.device.index == torch.cuda.current_device():
+            if dtype is not None and t.dtype != dtype:
+                t = t.to(dtype)
+            return t if t.is_contiguous() else t.contiguous()
     else:
         t = torch.from_numpy(np.ascontiguousarray(np.asarray(x)))
     t = t.to(_device())

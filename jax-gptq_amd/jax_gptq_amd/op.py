@@ -8,6 +8,8 @@ backward pass is the same operator with ``transpose_b`` flipped.
 """
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from . import _native as N
@@ -20,8 +22,8 @@ from .gptq import _DT, _float_dev, _dev, _ptr, _stream, _ws
 _WS_CACHE = {}
 
 
-def _qmm_workspace(nbytes, device):
-    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+def _qmm_workspace(nbytes, device, stream_handle):
+    key = (device.index, stream_handle)
     ws = _WS_CACHE.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.zeros(max(int(nbytes), 256), dtype=torch.uint8, device=device)
@@ -51,17 +53,19 @@ def _quantized_matmul_raw(x, int_weight, zero, scale, transpose_b, bits=4, group
     if zero.dtype != scale.dtype:
         scale = scale.to(zero.dtype)
     out = torch.empty((M, out_n), dtype=x.dtype, device=x.device)
+    handle = torch.cuda.current_stream(x.device).cuda_stream      # asked once per call
+    stream = ctypes.c_void_p(handle)
     ws = _qmm_workspace(lib.gptq_hip_qmatmul_bits_workspace_bytes(M, R, C, int(transpose_b), _DT[x.dtype], bits),
-                        x.device)
+                        x.device, handle)
     if group_size:
         zero, scale = zero.contiguous(), scale.contiguous()
         if tuple(zero.shape) != (Kw // group_size, C) or tuple(scale.shape) != (Kw // group_size, C):
             raise ValueError("grouped zero/scale must be [K / group_size, N]")
-        N.check(lib.gptq_hip_qmatmul_grouped(_stream(), _ptr(x), _DT[x.dtype], M, _ptr(int_weight), R, C,
+        N.check(lib.gptq_hip_qmatmul_grouped(stream, _ptr(x), _DT[x.dtype], M, _ptr(int_weight), R, C,
                                              _ptr(zero), _ptr(scale), _DT[zero.dtype], group_size, bits,
                                              int(transpose_b), _ptr(out), _ptr(ws), ws.numel()), "qmatmul")
     else:
-        N.check(lib.gptq_hip_qmatmul_bits(_stream(), _ptr(x), _DT[x.dtype], M, _ptr(int_weight), R, C,
+        N.check(lib.gptq_hip_qmatmul_bits(stream, _ptr(x), _DT[x.dtype], M, _ptr(int_weight), R, C,
                                           _ptr(zero), _ptr(scale), _DT[zero.dtype], bits, int(transpose_b),
                                           _ptr(out), _ptr(ws), ws.numel()), "qmatmul")
     if leading_dims is not None:
