@@ -2055,8 +2055,9 @@ namespace {
 size_t ws16_bytes(int64_t M, int64_t R, int64_t C, int transpose_b, int bits) {
   if (M <= 0 || R <= 0 || C <= 0) return 0;
   if (transpose_b) {
-    const RegBwdPlan bp = reg_bwd_plan(M, R, C, bits, true);
-    return bp.use ? bp.total_bytes : 0;
+    const RegBwdPlan bp = reg_bwd_plan(M, R, C, bits, true), bp8 = reg_bwd_plan(M, R, C, bits, true, 8);
+    const size_t a = bp.use ? bp.total_bytes : 0, b = bp8.use ? bp8.total_bytes : 0;
+    return a > b ? a : b;
   }
   const RegPlan rp = reg_fwd_plan(M, R, C, bits, true);
   size_t need = rp.use ? rp.total_bytes : 0;
@@ -2274,6 +2275,17 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
   // number no more than the CUs it runs as long as a full chip's worth of tiles would (122 us for any M <= 448
   // on 4096 x 11008); there the register-operand kernel, which splits, takes over (M = 128: 124 -> 38 us,
   // M = 16: 122 -> 23 us; exactly one tile per CU, M = 512: 133 -> 103 us).
+  // fp16 activations, more than 64 rows: 128-row tiles of the register-operand kernel (a dequantised operand
+  // serves twice the rows; 4096 x 11008 at M = 2048: 335 -> 268 us, 8-bit: 512 -> 347 us) unless their last round
+  // of 256 workgroups would leave much of the chip idle (11008 x 4096 at M = 512: 344 tiles)
+  if (transpose_b && reg_groups_ok && x_dtype == GPTQ_HIP_F16 && M > 64) {
+    const RegBwdPlan bp8 = reg_bwd_plan(M, R, C, bits, al, 8);
+    const int64_t rounds = bp8.use ? (bp8.tiles + 255) / 256 : 0;
+    if (bp8.use && (bp8.tiles <= 256 || bp8.tiles * 5 >= rounds * 256 * 4)) {
+      if (bp8.total_bytes && (!ws || ws_bytes < bp8.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+      return reg_bwd_launch(st, bp8, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, out, ws, (int)group_size);
+    }
+  }
   const bool bwd_tiles_fill = ceil_div64(2 * R, 128) * ceil_div64(M, 64) > 256 ||
                               !(reg_groups_ok && reg_bwd_plan(M, R, C, bits, al).use);
   if (bits == 4 && transpose_b && group_size == 0 && bwd_tiles_fill &&

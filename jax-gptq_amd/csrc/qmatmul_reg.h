@@ -33,13 +33,14 @@ int reg_fwd_launch(hipStream_t st, const RegPlan &p, const void *x, int x_dtype,
 // Transposed product out[M, K] = x[M, C] @ dequant(packed[R, C])^T.
 struct RegBwdPlan {
   bool use;
-  int bits;
+  int bits, rb;            // rb: 16-row blocks per output tile (4, or 8 for fp16 activations where 128-row tiles fill the chip)
   bool ragged;
   int S, steps;
   int64_t tiles;
   size_t part_bytes, total_bytes;
 };
-RegBwdPlan reg_bwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned);
+// rb = 8: 128-row tiles (fp16 activations only; the launch falls back to 64-row tiles for bf16)
+RegBwdPlan reg_bwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned, int rb = 4);
 // group_size > 0: a multiple of 128 (the 128 output columns of a tile share one group)
 int reg_bwd_launch(hipStream_t st, const RegBwdPlan &p, const void *x, int x_dtype, int64_t M, const uint8_t *pk,
                    int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws,

@@ -1,10 +1,11 @@
 // Packed-weight matmul, transposed form (the VJP of the forward product), both MFMA operands built in registers:
 //   out[M, K] = x[M, C] @ ((code - zero) * scale)^T,  codes packed as 4-bit pairs (K = 2 R) or bytes (K = R).
-// Serves what qmm_bwd_gemm_kernel does not: 8-bit codes and shapes whose rows are not multiples of 16
-// channels or that are not 16-byte aligned.
+// Serves fp16 activations of more than 64 rows (128-row tiles), and what qmm_bwd_gemm_kernel does not: 8-bit
+// codes, shapes whose rows are not multiples of 16 channels or that are not 16-byte aligned, and products whose
+// output tiles are too few to fill the chip without a split over the contraction.
 //
 // The contraction runs along the channels, the contiguous axis of the packed matrix.  A workgroup owns a
-// 64 x 128 output tile (128 output columns = 64 packed rows of nibble pairs or 128 rows of bytes) over a range
+// 64 x 128 or 128 x 128 output tile (128 output columns = 64 packed rows of nibble pairs or 128 rows of bytes) over a range
 // of k-steps of 32 channels; its four wavefronts take the k-steps t % 4 == wavefront; no staging of the
 // operands in LDS, no barrier in the k loop.
 //   B: lane (l16, g) loads the 8 bytes = channels 32 t + 8 g .. + 7 of packed row j0 + 16 jg + l16 for every
@@ -25,18 +26,24 @@ namespace {
 
 using namespace qmm;
 
-constexpr int RGB_RB = 4;
+constexpr int RGB_RB = 4;                      // row blocks per pass of the final reduction (and per 64-row tile)
 constexpr int RGB_RING = 3;
 constexpr int RGB_LDS_BYTES = 4 * RGB_RB * RG_NT * RG_TILE_FLOATS * 4;     // 144 KB: the reduction buffer
 constexpr int RGB_MAX_STEPS = RGB_LDS_BYTES / 8 / 32;                      // k-steps whose constants fit (8 B / channel)
 
-template <int BITS, bool RAGGED, typename TX>
+// RB = 4: 64-row tiles.  RB = 8 (fp16 activations): 128-row tiles, a dequantised operand serves twice the rows;
+// the 8 x 8 product tiles fill the 256 accumulation registers and every MFMA accumulates in place
+// (Act::mma_acc, read only after mma_drain), the reduction runs in two passes of four row blocks.
+template <int BITS, bool RAGGED, typename TX, int RB = RGB_RB>
 __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, const uint8_t *pk, int R, int C,
                                                           const void *zero, const void *scale, int zs_dtype,
                                                           TX *out, float *part, int32_t *counters, int S,
                                                           int steps_per_split, int group_size) {
   constexpr bool BF = Act<TX>::BF;
-  constexpr int RB = RGB_RB, RING = RGB_RING;
+  constexpr int RING = RB == 8 ? 2 : RGB_RING;
+  constexpr bool TIED = RB == 8;
+  constexpr int RBT = RGB_RB, NH = RB / RBT;      // row blocks per pass of the final reduction, passes
+  static_assert(RB == 4 || (RB == 8 && !BF), "128-row tiles: fp16 activations (bf16 needs a ninth tile)");
   constexpr int NG = BITS == 4 ? 4 : 8;          // groups of 16 packed rows: 8 MFMA tiles either way
   constexpr int NJ = 16 * NG;
   extern __shared__ __attribute__((aligned(16))) float rg_lds[];
@@ -176,12 +183,20 @@ __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, co
           const uint4 bh = make_uint4(hi4[0], hi4[1], hi4[2], hi4[3]);
 #pragma unroll
           for (int rb = 0; rb < RB; ++rb) {
-            acc[rb][2 * jg] = Act<TX>::mma(a[rb], bl, acc[rb][2 * jg]);
-            acc[rb][2 * jg + 1] = Act<TX>::mma(a[rb], bh, acc[rb][2 * jg + 1]);
+            if constexpr (TIED) {
+              Act<TX>::mma_acc(acc[rb][2 * jg], a[rb], bl);
+              Act<TX>::mma_acc(acc[rb][2 * jg + 1], a[rb], bh);
+            } else {
+              acc[rb][2 * jg] = Act<TX>::mma(a[rb], bl, acc[rb][2 * jg]);
+              acc[rb][2 * jg + 1] = Act<TX>::mma(a[rb], bh, acc[rb][2 * jg + 1]);
+            }
           }
         } else {
 #pragma unroll
-          for (int rb = 0; rb < RB; ++rb) acc[rb][jg] = Act<TX>::mma(a[rb], bl, acc[rb][jg]);
+          for (int rb = 0; rb < RB; ++rb) {
+            if constexpr (TIED) Act<TX>::mma_acc(acc[rb][jg], a[rb], bl);
+            else acc[rb][jg] = Act<TX>::mma(a[rb], bl, acc[rb][jg]);
+          }
         }
       }
     } else {
@@ -261,55 +276,67 @@ __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, co
       if (u == slot) compute(u, iters_full, tail);
   }
 
+  if constexpr (TIED) mma_drain();
   __syncthreads();                                                   // every wavefront is done with the tables
-  floatx4 sum[RG_NT];
-  const int tile = ty * gridDim.x + tx;
-  if (!rg_reduce<RB>(acc, sum, rg_lds, &s_flag, part, counters, tile, split, S)) return;
-  const int rb = wk;
   const int64_t KO = BITS == 4 ? 2 * (int64_t)R : R;
+  // one pass of the reduction per four row blocks (a 128-row tile: two passes, each with its own arrival counter
+  // and partial tiles, as if it were two 64-row tiles)
+  auto finish = [&](auto hc) __attribute__((always_inline)) {
+    constexpr int H = decltype(hc)::value;
+    floatx4 sum[RG_NT];
+    const int tile = (ty * NH + H) * gridDim.x + tx;
+    if (!rg_reduce<RBT, RB, H * RBT>(acc, sum, rg_lds, &s_flag, part, counters, tile, split, S)) return;
+    const int rb = H * RBT + wk;
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int m = m0 + 16 * rb + 4 * g + r;
-    float t = 0.f;
-    if (BF) {
-      t = sum[8][r];
-      t += __shfl_xor(t, 8);                  // columns < 8: the integer part's term, the others: the fraction's
-    }
-    if (m >= M) continue;
-    TX *orow = out + (int64_t)m * KO;
+    for (int r = 0; r < 4; ++r) {
+      const int m = m0 + 16 * rb + 4 * g + r;
+      float t = 0.f;
+      if (BF) {
+        t = sum[8][r];
+        t += __shfl_xor(t, 8);                  // columns < 8: the integer part's term, the others: the fraction's
+      }
+      if (m >= M) continue;
+      TX *orow = out + (int64_t)m * KO;
 #pragma unroll
-    for (int jg = 0; jg < NG; ++jg) {
-      const int j = j0 + 16 * jg + l16;
-      if (j >= R) continue;
-      if constexpr (BITS == 4) {
-        TX o2[2] = {Act<TX>::out(sum[2 * jg][r] - t), Act<TX>::out(sum[2 * jg + 1][r] - t)};
-        *reinterpret_cast<uint32_t *>(orow + 2 * j) = *reinterpret_cast<const uint32_t *>(o2);
-      } else {
-        orow[j] = Act<TX>::out(sum[jg][r] - t);
+      for (int jg = 0; jg < NG; ++jg) {
+        const int j = j0 + 16 * jg + l16;
+        if (j >= R) continue;
+        if constexpr (BITS == 4) {
+          TX o2[2] = {Act<TX>::out(sum[2 * jg][r] - t), Act<TX>::out(sum[2 * jg + 1][r] - t)};
+          *reinterpret_cast<uint32_t *>(orow + 2 * j) = *reinterpret_cast<const uint32_t *>(o2);
+        } else {
+          orow[j] = Act<TX>::out(sum[jg][r] - t);
+        }
       }
     }
+  };
+  finish(std::integral_constant<int, 0>{});
+  if constexpr (NH == 2) {
+    __syncthreads();                                                 // the first pass's sums have been read
+    finish(std::integral_constant<int, 1>{});
   }
 }
 
-template <int BITS, bool RAGGED, typename TX>
+template <int BITS, bool RAGGED, typename TX, int RB = RGB_RB>
 int launch_inst(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
                 int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *wsp, int group_size) {
   constexpr int NJ = BITS == 4 ? 64 : 128;
-  auto kern = qmm_bwd_reg_kernel<BITS, RAGGED, TX>;
+  auto kern = qmm_bwd_reg_kernel<BITS, RAGGED, TX, RB>;
   if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), RGB_LDS_BYTES)) return GPTQ_HIP_ELAUNCH;
   const int64_t KO = BITS == 4 ? 2 * R : R;
   int32_t *counters = reinterpret_cast<int32_t *>(wsp);
   float *part = reinterpret_cast<float *>(reinterpret_cast<char *>(wsp) + QMM_HEAD_BYTES);
   const int64_t tiles_x = ceil_div64(R, NJ);
+  constexpr int TR = 16 * RB;                    // rows of a tile
   int64_t rows_max = ((1LL << 31) - 1) / C;
-  if (rows_max > 65535LL * 64) rows_max = 65535LL * 64;
+  if (rows_max > 65535LL * TR) rows_max = 65535LL * TR;
   const int64_t tiles_y_max = p.tiles / tiles_x;
-  if (rows_max > tiles_y_max * 64) rows_max = tiles_y_max * 64;
-  rows_max -= rows_max % 64;
-  if (rows_max < 64) return GPTQ_HIP_EINVAL;
+  if (rows_max > tiles_y_max * TR) rows_max = tiles_y_max * TR;
+  rows_max -= rows_max % TR;
+  if (rows_max < TR) return GPTQ_HIP_EINVAL;
   for (int64_t r0 = 0; r0 < M; r0 += rows_max) {
     const int64_t rows = M - r0 < rows_max ? M - r0 : rows_max;
-    const dim3 grid((unsigned)tiles_x, (unsigned)ceil_div64(rows, 64), (unsigned)p.S);
+    const dim3 grid((unsigned)tiles_x, (unsigned)ceil_div64(rows, TR), (unsigned)p.S);
     hipLaunchKernelGGL(kern, grid, dim3(256), RGB_LDS_BYTES, st, (const TX *)x + r0 * C, (int)rows, pk, (int)R,
                        (int)C, zero, scale, zs_dtype, (TX *)out + r0 * KO, part, counters, p.S, p.steps, group_size);
     GPTQ_CHECK_LAUNCH();
@@ -320,6 +347,13 @@ int launch_inst(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, c
 template <int BITS, typename TX>
 int launch_bx(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
               int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws, int group_size) {
+  if constexpr (!Act<TX>::BF) {
+    if (p.rb == 8) {
+      if (p.ragged)
+        return launch_inst<BITS, true, TX, 8>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
+      return launch_inst<BITS, false, TX, 8>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
+    }
+  }
   if (p.ragged) return launch_inst<BITS, true, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
   return launch_inst<BITS, false, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
 }
@@ -328,15 +362,18 @@ int launch_bx(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, con
 
 namespace qmm {
 
-RegBwdPlan reg_bwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned) {
+RegBwdPlan reg_bwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned, int rb) {
   RegBwdPlan p{};
   if ((bits != 4 && bits != 8) || M < 1 || C < 8 || R < 1 || R >= (1LL << 30) || C >= (1LL << 30)) return p;
   p.bits = bits;
   p.ragged = !aligned || C % 8 != 0;
   const int64_t tiles_x = ceil_div64(R, bits == 4 ? 64 : 128);
   if (tiles_x > QMM_MAX_COUNTERS) return p;
-  int64_t tiles_y = ceil_div64(M, 64);
-  if (tiles_y > QMM_MAX_COUNTERS / tiles_x) tiles_y = QMM_MAX_COUNTERS / tiles_x;
+  if (rb != 4 && rb != 8) return p;
+  p.rb = rb;
+  const int64_t nh = p.rb / 4;                   // arrival counters per tile
+  int64_t tiles_y = ceil_div64(M, 16 * p.rb);
+  if (tiles_y > QMM_MAX_COUNTERS / (tiles_x * nh)) tiles_y = QMM_MAX_COUNTERS / (tiles_x * nh);
   p.tiles = tiles_x * tiles_y;
   const int64_t T = ceil_div64(C, 32);
   int64_t S = 1;
@@ -349,7 +386,7 @@ RegBwdPlan reg_bwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned)
   if (S < s_min) S = s_min;
   p.steps = (int)ceil_div64(T, S);
   p.S = (int)ceil_div64(T, p.steps);
-  p.part_bytes = p.S > 1 ? (size_t)p.tiles * p.S * RGB_RB * RG_NT * RG_TILE_FLOATS * sizeof(float) : 0;
+  p.part_bytes = p.S > 1 ? (size_t)p.tiles * p.S * p.rb * RG_NT * RG_TILE_FLOATS * sizeof(float) : 0;
   p.total_bytes = p.S > 1 ? QMM_HEAD_BYTES + p.part_bytes : 0;
   p.use = true;
   return p;
