@@ -2281,7 +2281,7 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
   if (transpose_b && reg_groups_ok && x_dtype == GPTQ_HIP_F16 && M > 64) {
     const RegBwdPlan bp8 = reg_bwd_plan(M, R, C, bits, al, 8);
     const int64_t rounds = bp8.use ? (bp8.tiles + 255) / 256 : 0;
-    if (bp8.use && (bp8.tiles <= 256 || bp8.tiles * 5 >= rounds * 256 * 4)) {
+    if (bp8.use && (bp8.tiles <= 256 || bp8.tail_x > 0 || bp8.tiles * 5 >= rounds * 256 * 4)) {
       if (bp8.total_bytes && (!ws || ws_bytes < bp8.total_bytes)) return GPTQ_HIP_EWORKSPACE;
       return reg_bwd_launch(st, bp8, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, out, ws, (int)group_size);
     }

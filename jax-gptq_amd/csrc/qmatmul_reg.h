@@ -34,6 +34,7 @@ int reg_fwd_launch(hipStream_t st, const RegPlan &p, const void *x, int x_dtype,
 struct RegBwdPlan {
   bool use;
   int bits, rb;            // rb: 16-row blocks per output tile (4, or 8 for fp16 activations where 128-row tiles fill the chip)
+  int tail_x;              // 128-row tiles: this many trailing column tiles run on 64-row tiles in a second launch
   bool ragged;
   int S, steps;
   int64_t tiles;

@@ -38,7 +38,7 @@ template <int BITS, bool RAGGED, typename TX, int RB = RGB_RB>
 __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, const uint8_t *pk, int R, int C,
                                                           const void *zero, const void *scale, int zs_dtype,
                                                           TX *out, float *part, int32_t *counters, int S,
-                                                          int steps_per_split, int group_size) {
+                                                          int steps_per_split, int group_size, int tx0) {
   constexpr bool BF = Act<TX>::BF;
   constexpr int RING = RB == 8 ? 2 : RGB_RING;
   constexpr bool TIED = RB == 8;
@@ -52,7 +52,8 @@ __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, co
   const int g = lane >> 4, l16 = lane & 15;
   int tx, ty;
   qmm_tile_coords(tx, ty);
-  const int j0 = tx * NJ, m0 = ty * (16 * RB), split = blockIdx.z;
+  // (tx0: first column tile of this launch, where the columns are dealt over two launches)
+  const int j0 = (tx + tx0) * NJ, m0 = ty * (16 * RB), split = blockIdx.z;
   const int T = (C + 31) >> 5;
   const int t_begin = split * steps_per_split, t_end = min(T, t_begin + steps_per_split);
   const int range = max(0, t_end - t_begin);
@@ -319,26 +320,30 @@ __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, co
 
 template <int BITS, bool RAGGED, typename TX, int RB = RGB_RB>
 int launch_inst(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
-                int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *wsp, int group_size) {
+                int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *wsp, int group_size,
+                int64_t tx0 = 0, int64_t ntx = -1) {
   constexpr int NJ = BITS == 4 ? 64 : 128;
   auto kern = qmm_bwd_reg_kernel<BITS, RAGGED, TX, RB>;
   if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), RGB_LDS_BYTES)) return GPTQ_HIP_ELAUNCH;
   const int64_t KO = BITS == 4 ? 2 * R : R;
   int32_t *counters = reinterpret_cast<int32_t *>(wsp);
   float *part = reinterpret_cast<float *>(reinterpret_cast<char *>(wsp) + QMM_HEAD_BYTES);
-  const int64_t tiles_x = ceil_div64(R, NJ);
+  // column tiles [tx0, tx0 + ntx) (all of them unless the plan deals the columns over two launches)
+  const int64_t tiles_all = ceil_div64(R, NJ);
+  const int64_t tiles_x = ntx < 0 ? tiles_all : ntx;
   constexpr int TR = 16 * RB;                    // rows of a tile
   int64_t rows_max = ((1LL << 31) - 1) / C;
   if (rows_max > 65535LL * TR) rows_max = 65535LL * TR;
-  const int64_t tiles_y_max = p.tiles / tiles_x;
-  if (rows_max > tiles_y_max * TR) rows_max = tiles_y_max * TR;
+  const int64_t tiles_y_max = p.tiles / tiles_all;
+  if (p.S > 1 && rows_max > tiles_y_max * TR) rows_max = tiles_y_max * TR;
   rows_max -= rows_max % TR;
   if (rows_max < TR) return GPTQ_HIP_EINVAL;
   for (int64_t r0 = 0; r0 < M; r0 += rows_max) {
     const int64_t rows = M - r0 < rows_max ? M - r0 : rows_max;
     const dim3 grid((unsigned)tiles_x, (unsigned)ceil_div64(rows, TR), (unsigned)p.S);
     hipLaunchKernelGGL(kern, grid, dim3(256), RGB_LDS_BYTES, st, (const TX *)x + r0 * C, (int)rows, pk, (int)R,
-                       (int)C, zero, scale, zs_dtype, (TX *)out + r0 * KO, part, counters, p.S, p.steps, group_size);
+                       (int)C, zero, scale, zs_dtype, (TX *)out + r0 * KO, part, counters, p.S, p.steps, group_size,
+                       (int)tx0);
     GPTQ_CHECK_LAUNCH();
   }
   return GPTQ_HIP_OK;
@@ -348,6 +353,20 @@ template <int BITS, typename TX>
 int launch_bx(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
               int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws, int group_size) {
   if constexpr (!Act<TX>::BF) {
+    if (p.rb == 8 && p.tail_x > 0) {
+      // 128-row tiles on the columns that fill whole rounds of workgroups, 64-row tiles on the rest
+      const int64_t main_x = ceil_div64(R, BITS == 4 ? 64 : 128) - p.tail_x;
+      const int rc = p.ragged ? launch_inst<BITS, true, TX, 8>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws,
+                                                               group_size, 0, main_x)
+                              : launch_inst<BITS, false, TX, 8>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws,
+                                                                group_size, 0, main_x);
+      if (rc) return rc;
+      if (p.ragged)
+        return launch_inst<BITS, true, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size, main_x,
+                                           p.tail_x);
+      return launch_inst<BITS, false, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size, main_x,
+                                          p.tail_x);
+    }
     if (p.rb == 8) {
       if (p.ragged)
         return launch_inst<BITS, true, TX, 8>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
@@ -386,6 +405,16 @@ RegBwdPlan reg_bwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned,
   if (S < s_min) S = s_min;
   p.steps = (int)ceil_div64(T, S);
   p.S = (int)ceil_div64(T, p.steps);
+  // 128-row tiles whose last round of workgroups would be at most half full: the trailing column tiles run on
+  // 64-row tiles in a second launch (as in the forward kernel's plan)
+  p.tail_x = 0;
+  if (p.rb == 8 && p.S == 1 && T >= 64) {
+    const int64_t all = tiles_x * tiles_y, full = all / 256, rem = all % 256;
+    if (full >= 1 && rem > 0 && rem <= 128) {
+      const int64_t main_x = full * 256 / tiles_y, tail = tiles_x - main_x;
+      if (main_x >= 1 && tail >= 1 && tail * tiles_y * 2 <= 256) p.tail_x = (int)tail;
+    }
+  }
   p.part_bytes = p.S > 1 ? (size_t)p.tiles * p.S * p.rb * RG_NT * RG_TILE_FLOATS * sizeof(float) : 0;
   p.total_bytes = p.S > 1 ? QMM_HEAD_BYTES + p.part_bytes : 0;
   p.use = true;
