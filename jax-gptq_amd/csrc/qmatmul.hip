@@ -2275,10 +2275,10 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
   // number no more than the CUs it runs as long as a full chip's worth of tiles would (122 us for any M <= 448
   // on 4096 x 11008); there the register-operand kernel, which splits, takes over (M = 128: 124 -> 38 us,
   // M = 16: 122 -> 23 us; exactly one tile per CU, M = 512: 133 -> 103 us).
-  // fp16 activations, more than 64 rows: 128-row tiles of the register-operand kernel (a dequantised operand
+  // more than 64 rows: 128-row tiles of the register-operand kernel (a dequantised operand
   // serves twice the rows; 4096 x 11008 at M = 2048: 335 -> 268 us, 8-bit: 512 -> 347 us) unless their last round
   // of 256 workgroups would leave much of the chip idle (11008 x 4096 at M = 512: 344 tiles)
-  if (transpose_b && reg_groups_ok && x_dtype == GPTQ_HIP_F16 && M > 64) {
+  if (transpose_b && reg_groups_ok && M > 64) {
     const RegBwdPlan bp8 = reg_bwd_plan(M, R, C, bits, al, 8);
     const int64_t rounds = bp8.use ? (bp8.tiles + 255) / 256 : 0;
     if (bp8.use && (bp8.tiles <= 256 || bp8.tail_x > 0 || bp8.tiles * 5 >= rounds * 256 * 4)) {

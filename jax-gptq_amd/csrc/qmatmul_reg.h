@@ -40,7 +40,7 @@ struct RegBwdPlan {
   int64_t tiles;
   size_t part_bytes, total_bytes;
 };
-// rb = 8: 128-row tiles (fp16 activations only; the launch falls back to 64-row tiles for bf16)
+// rb = 8: 128-row tiles
 RegBwdPlan reg_bwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned, int rb = 4);
 // group_size > 0: a multiple of 128 (the 128 output columns of a tile share one group)
 int reg_bwd_launch(hipStream_t st, const RegBwdPlan &p, const void *x, int x_dtype, int64_t M, const uint8_t *pk,

@@ -31,9 +31,10 @@ constexpr int RGB_RING = 3;
 constexpr int RGB_LDS_BYTES = 4 * RGB_RB * RG_NT * RG_TILE_FLOATS * 4;     // 144 KB: the reduction buffer
 constexpr int RGB_MAX_STEPS = RGB_LDS_BYTES / 8 / 32;                      // k-steps whose constants fit (8 B / channel)
 
-// RB = 4: 64-row tiles.  RB = 8 (fp16 activations): 128-row tiles, a dequantised operand serves twice the rows;
+// RB = 4: 64-row tiles.  RB = 8: 128-row tiles, a dequantised operand serves twice the rows;
 // the 8 x 8 product tiles fill the 256 accumulation registers and every MFMA accumulates in place
-// (Act::mma_acc, read only after mma_drain), the reduction runs in two passes of four row blocks.
+// (Act::mma_acc, read only after mma_drain; bf16's ninth tiles in vector registers), the reduction runs in two
+// passes of four row blocks.
 template <int BITS, bool RAGGED, typename TX, int RB = RGB_RB>
 __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, const uint8_t *pk, int R, int C,
                                                           const void *zero, const void *scale, int zs_dtype,
@@ -43,7 +44,7 @@ __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, co
   constexpr int RING = RB == 8 ? 2 : RGB_RING;
   constexpr bool TIED = RB == 8;
   constexpr int RBT = RGB_RB, NH = RB / RBT;      // row blocks per pass of the final reduction, passes
-  static_assert(RB == 4 || (RB == 8 && !BF), "128-row tiles: fp16 activations (bf16 needs a ninth tile)");
+  static_assert(RB == 4 || RB == 8, "64- or 128-row tiles");
   constexpr int NG = BITS == 4 ? 4 : 8;          // groups of 16 packed rows: 8 MFMA tiles either way
   constexpr int NJ = 16 * NG;
   extern __shared__ __attribute__((aligned(16))) float rg_lds[];
@@ -224,7 +225,8 @@ __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, co
           o[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f2_t{Act<TX>::lo(aw[i]) * sf[2 * i],
                                                                            Act<TX>::hi(aw[i]) * sf[2 * i + 1]}, bf2_t));
         a[rb] = make_uint4(o[0], o[1], o[2], o[3]);
-        acc[rb][8] = Act<TX>::mma(a[rb], bz, acc[rb][8]);
+        if constexpr (TIED) Act<TX>::mma_accv(acc[rb][8], a[rb], bz);      // (the ninth tiles live in vector registers)
+        else acc[rb][8] = Act<TX>::mma(a[rb], bz, acc[rb][8]);
       }
 #pragma unroll
       for (int jg = 0; jg < NG; ++jg) {
@@ -247,12 +249,20 @@ __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, co
           const uint4 bh = make_uint4(hi4[0], hi4[1], hi4[2], hi4[3]);
 #pragma unroll
           for (int rb = 0; rb < RB; ++rb) {
-            acc[rb][2 * jg] = Act<TX>::mma(a[rb], bl, acc[rb][2 * jg]);
-            acc[rb][2 * jg + 1] = Act<TX>::mma(a[rb], bh, acc[rb][2 * jg + 1]);
+            if constexpr (TIED) {
+              Act<TX>::mma_acc(acc[rb][2 * jg], a[rb], bl);
+              Act<TX>::mma_acc(acc[rb][2 * jg + 1], a[rb], bh);
+            } else {
+              acc[rb][2 * jg] = Act<TX>::mma(a[rb], bl, acc[rb][2 * jg]);
+              acc[rb][2 * jg + 1] = Act<TX>::mma(a[rb], bh, acc[rb][2 * jg + 1]);
+            }
           }
         } else {
 #pragma unroll
-          for (int rb = 0; rb < RB; ++rb) acc[rb][jg] = Act<TX>::mma(a[rb], bl, acc[rb][jg]);
+          for (int rb = 0; rb < RB; ++rb) {
+            if constexpr (TIED) Act<TX>::mma_acc(acc[rb][jg], a[rb], bl);
+            else acc[rb][jg] = Act<TX>::mma(a[rb], bl, acc[rb][jg]);
+          }
         }
       }
     }
@@ -352,7 +362,7 @@ int launch_inst(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, c
 template <int BITS, typename TX>
 int launch_bx(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
               int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws, int group_size) {
-  if constexpr (!Act<TX>::BF) {
+  {
     if (p.rb == 8 && p.tail_x > 0) {
       // 128-row tiles on the columns that fill whole rounds of workgroups, 64-row tiles on the rest
       const int64_t main_x = ceil_div64(R, BITS == 4 ? 64 : 128) - p.tail_x;
