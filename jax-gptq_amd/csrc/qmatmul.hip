@@ -2168,7 +2168,7 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
         bool wrote = false;
         const int rc = qmatmul_impl(stream, x16, GPTQ_HIP_F16, mm, packed, R, C, zero, scale, zs_dtype, bits,
                                     group_size, transpose_b, o16, ws, fp.inner,
-                                    (transpose_b || (reinterpret_cast<uintptr_t>(out) & 15) != 0)
+                                    (reinterpret_cast<uintptr_t>(out) & 15) != 0
                                         ? nullptr
                                         : reinterpret_cast<float *>(out) + r0 * nout,
                                     rowexp, &wrote);
@@ -2283,7 +2283,13 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
     const int64_t rounds = bp8.use ? (bp8.tiles + 255) / 256 : 0;
     if (bp8.use && (bp8.tiles <= 256 || bp8.tail_x > 0 || bp8.tiles * 5 >= rounds * 256 * 4)) {
       if (bp8.total_bytes && (!ws || ws_bytes < bp8.total_bytes)) return GPTQ_HIP_EWORKSPACE;
-      return reg_bwd_launch(st, bp8, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, out, ws, (int)group_size);
+      RegBwdPlan q = bp8;
+      if (out32 && rowexp && wrote32 && x_dtype == GPTQ_HIP_F16) {
+        q.out32 = out32;
+        q.rowexp = rowexp;
+        *wrote32 = true;
+      }
+      return reg_bwd_launch(st, q, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, out, ws, (int)group_size);
     }
   }
   const bool bwd_tiles_fill = ceil_div64(2 * R, 128) * ceil_div64(M, 64) > 256 ||
@@ -2302,7 +2308,13 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
     const RegBwdPlan bp = reg_bwd_plan(M, R, C, bits, al);
     if (bp.use) {
       if (bp.total_bytes && (!ws || ws_bytes < bp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
-      return reg_bwd_launch(st, bp, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, out, ws, (int)group_size);
+      RegBwdPlan q = bp;
+      if (out32 && rowexp && wrote32 && x_dtype == GPTQ_HIP_F16) {
+        q.out32 = out32;
+        q.rowexp = rowexp;
+        *wrote32 = true;
+      }
+      return reg_bwd_launch(st, q, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, out, ws, (int)group_size);
     }
   }
   return bits == 4

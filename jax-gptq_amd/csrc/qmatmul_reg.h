@@ -33,8 +33,11 @@ int reg_fwd_launch(hipStream_t st, const RegPlan &p, const void *x, int x_dtype,
 // Transposed product out[M, K] = x[M, C] @ dequant(packed[R, C])^T.
 struct RegBwdPlan {
   bool use;
-  int bits, rb;            // rb: 16-row blocks per output tile (4, or 8 for fp16 activations where 128-row tiles fill the chip)
+  int bits, rb;            // rb: 16-row blocks per output tile (4, or 8: 128-row tiles)
   int tail_x;              // 128-row tiles: this many trailing column tiles run on 64-row tiles in a second launch
+  // set by the caller for fp32 rows (see RegPlan): the tiles store ldexp(fp16(result), rowexp[m]) as fp32
+  float *out32;
+  const int32_t *rowexp;
   bool ragged;
   int S, steps;
   int64_t tiles;

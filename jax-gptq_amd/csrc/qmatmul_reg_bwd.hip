@@ -39,7 +39,8 @@ template <int BITS, bool RAGGED, typename TX, int RB = RGB_RB>
 __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, const uint8_t *pk, int R, int C,
                                                           const void *zero, const void *scale, int zs_dtype,
                                                           TX *out, float *part, int32_t *counters, int S,
-                                                          int steps_per_split, int group_size, int tx0) {
+                                                          int steps_per_split, int group_size, int tx0, float *out32,
+                                                          const int32_t *rowexp) {
   constexpr bool BF = Act<TX>::BF;
   constexpr int RING = RB == 8 ? 2 : RGB_RING;
   constexpr bool TIED = RB == 8;
@@ -307,6 +308,24 @@ __global__ __launch_bounds__(256) void qmm_bwd_reg_kernel(const TX *x, int M, co
         t += __shfl_xor(t, 8);                  // columns < 8: the integer part's term, the others: the fraction's
       }
       if (m >= M) continue;
+      if (out32 != nullptr) {
+        // fp32 rows: the fp16 result widened and scaled back by the row's power of two (exact)
+        const int e = rowexp[m];
+        float *orow32 = out32 + (int64_t)m * KO;
+#pragma unroll
+        for (int jg = 0; jg < NG; ++jg) {
+          const int j = j0 + 16 * jg + l16;
+          if (j >= R) continue;
+          if constexpr (BITS == 4) {
+            const float2 o2 = make_float2(ldexpf((float)Act<TX>::out(sum[2 * jg][r] - t), e),
+                                          ldexpf((float)Act<TX>::out(sum[2 * jg + 1][r] - t), e));
+            *reinterpret_cast<float2 *>(orow32 + 2 * j) = o2;
+          } else {
+            orow32[j] = ldexpf((float)Act<TX>::out(sum[jg][r] - t), e);
+          }
+        }
+        continue;
+      }
       TX *orow = out + (int64_t)m * KO;
 #pragma unroll
       for (int jg = 0; jg < NG; ++jg) {
@@ -353,7 +372,7 @@ int launch_inst(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, c
     const dim3 grid((unsigned)tiles_x, (unsigned)ceil_div64(rows, TR), (unsigned)p.S);
     hipLaunchKernelGGL(kern, grid, dim3(256), RGB_LDS_BYTES, st, (const TX *)x + r0 * C, (int)rows, pk, (int)R,
                        (int)C, zero, scale, zs_dtype, (TX *)out + r0 * KO, part, counters, p.S, p.steps, group_size,
-                       (int)tx0);
+                       (int)tx0, p.out32 ? p.out32 + r0 * KO : nullptr, p.rowexp ? p.rowexp + r0 : nullptr);
     GPTQ_CHECK_LAUNCH();
   }
   return GPTQ_HIP_OK;
