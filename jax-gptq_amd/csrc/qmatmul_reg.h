@@ -30,6 +30,14 @@ int reg_fwd_launch(hipStream_t st, const RegPlan &p, const void *x, int x_dtype,
                    int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws,
                    int group_size);
 
+// 128 x 512 tiles for many rows (qmatmul_wide.hip; 4-bit codes, per-channel parameters, aligned operands):
+// number of leading 512-channel tiles they take (0: none), and the launch over those tiles.  out32 / rowexp as
+// in RegPlan.
+int64_t wide_fwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned);
+int wide_fwd_launch(hipStream_t st, const void *x, int x_dtype, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
+                    const void *zero, const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32,
+                    const int32_t *rowexp);
+
 // Transposed product out[M, K] = x[M, C] @ dequant(packed[R, C])^T.
 struct RegBwdPlan {
   bool use;

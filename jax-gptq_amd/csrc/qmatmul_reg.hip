@@ -489,6 +489,17 @@ int launch_inst(hipStream_t st, const RegPlan &p, const void *x, int64_t M, cons
   return GPTQ_HIP_OK;
 }
 
+// 128-row tiles whose last round of workgroups would be at most half full (one workgroup per CU): this many
+// trailing column tiles go to 64-row tiles in a launch of their own, one partial round of half-sized tiles, and
+// the columns in front of them fill whole rounds.  Rounds have to be long (T k-steps) for the second launch to pay.
+int64_t deal_tail(int64_t tiles_x, int64_t tiles_y, int64_t T) {
+  if (T < 64) return 0;
+  const int64_t all = tiles_x * tiles_y, full = all / 256, rem = all % 256;
+  if (full < 1 || rem == 0 || rem > 128) return 0;
+  const int64_t main_x = full * 256 / tiles_y, tail = tiles_x - main_x;
+  return (main_x >= 1 && tail >= 1 && tail * tiles_y * 2 <= 256) ? tail : 0;
+}
+
 template <int BITS, typename TX>
 int launch_bx(hipStream_t st, const RegPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
               const void *zero, const void *scale, int zs_dtype, void *out, void *ws, int group_size) {
@@ -509,23 +520,40 @@ int launch_bx(hipStream_t st, const RegPlan &p, const void *x, int64_t M, const 
   }
   // a ring of two k-steps for 128-row tiles, of three for 64-row tiles (registers), of six for the 16-row tiles
   // of the decode case
-  if (p.rb == 8 && p.tail_x > 0) {
-    // 128-row tiles on the columns that fill whole rounds of workgroups, 64-row tiles on the rest
-    const int64_t main_x = ceil_div64(C, RG_BN) - p.tail_x;
-    const int rc = p.ragged ? launch_inst<BITS, 8, 2, true, TX, false>(st, p, x, M, pk, R, C, zero, scale, zs_dtype,
-                                                                         out, ws, group_size, 0, main_x)
-                            : launch_inst<BITS, 8, 3, false, TX, false>(st, p, x, M, pk, R, C, zero, scale, zs_dtype,
-                                                                          out, ws, group_size, 0, main_x);
-    if (rc) return rc;
+  if (p.rb == 8) {
+    const int64_t tiles_all = ceil_div64(C, RG_BN), tiles_y = ceil_div64(M, 128), K = BITS == 4 ? 2 * R : R;
+    // 128 x 512 tiles (qmatmul_wide.hip) on the leading columns that fill whole rounds of workgroups
+    int64_t first = 0;
+    if constexpr (BITS == 4) {
+      if (!p.ragged && p.S == 1) {
+        const int64_t wide_x = wide_fwd_tiles(M, R, C, true);
+        if (wide_x > 0) {
+          const int rc = wide_fwd_launch(st, x, Act<TX>::BF ? GPTQ_HIP_BF16 : GPTQ_HIP_F16, M, pk, R, C, zero, scale,
+                                         zs_dtype, out, wide_x, p.out32, p.rowexp);
+          if (rc) return rc;
+          first = 4 * wide_x;
+        }
+      }
+    }
+    const int64_t rest = tiles_all - first;
+    if (rest == 0) return GPTQ_HIP_OK;
+    // of the rest: 128-row tiles on the columns that fill whole rounds, 64-row tiles on the remaining ones
+    int64_t tail = first == 0 ? p.tail_x : deal_tail(rest, tiles_y, ceil_div64(K, 32));
+    if (first > 0 && rest * tiles_y <= 128) tail = rest;
+    const int64_t main_x = rest - tail;
+    if (main_x > 0) {
+      const int rc = p.ragged ? launch_inst<BITS, 8, 2, true, TX, false>(st, p, x, M, pk, R, C, zero, scale, zs_dtype,
+                                                                           out, ws, group_size, first, main_x)
+                              : launch_inst<BITS, 8, 3, false, TX, false>(st, p, x, M, pk, R, C, zero, scale, zs_dtype,
+                                                                            out, ws, group_size, first, main_x);
+      if (rc) return rc;
+    }
+    if (tail == 0) return GPTQ_HIP_OK;
     if (p.ragged)
       return launch_inst<BITS, 4, 3, true, TX, false>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws,
-                                                      group_size, main_x, p.tail_x);
+                                                      group_size, first + main_x, tail);
     return launch_inst<BITS, 4, 3, false, TX, false>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws,
-                                                     group_size, main_x, p.tail_x);
-  }
-  if (p.rb == 8) {
-    if (p.ragged) GPTQ_REG(8, 2, true, false);
-    GPTQ_REG(8, 3, false, false);
+                                                     group_size, first + main_x, tail);
   }
   if (p.rb == 4) {
     if (p.ragged) GPTQ_REG(4, 3, true, false);
@@ -571,14 +599,7 @@ RegPlan reg_fwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned) {
   // columns that fill whole rounds keep them, the remaining column tiles run on 64-row tiles in a second
   // launch, one partial round of half-sized tiles (M = 2048 on 4096 x 11008: 80 + 6 column tiles, 5 rounds +
   // 192 workgroups instead of 5.4 -> 6 rounds).  Rounds have to be long for the second launch to pay.
-  p.tail_x = 0;
-  if (p.rb == 8 && p.S == 1 && T >= 64) {
-    const int64_t all = tiles_x * tiles_y, full = all / 256, rem = all % 256;
-    if (full >= 1 && rem > 0 && rem <= 128) {
-      const int64_t main_x = full * 256 / tiles_y, tail = tiles_x - main_x;
-      if (main_x >= 1 && tail >= 1 && tail * tiles_y * 2 <= 256) p.tail_x = (int)tail;
-    }
-  }
+  p.tail_x = (p.rb == 8 && p.S == 1) ? (int)deal_tail(tiles_x, tiles_y, T) : 0;
   // 16-row tiles (one launch, M <= 16): the atomic sum where the cells hold the output and the atomics are few
   // (the memory side retires them at a limited rate: 900000 of them cost what the ticket path costs on
   // 4096 x 11008 and 4 us more on 7168 x 28672)

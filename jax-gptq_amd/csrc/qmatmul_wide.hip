@@ -1,0 +1,276 @@
+// Packed-weight matmul, forward, 4-bit codes, many rows: out[M, C] = x[M, K] @ ((code - zero) * scale) on
+// 128 x 512 output tiles whose four wavefronts stand side by side.
+//
+// Each wavefront owns a 128 x 128 output tile over ALL of K (8 x 8 product tiles in the 256 accumulation
+// registers) and builds its weight operands in registers from its own 128 channels, exactly as the 128-row tiles
+// of qmatmul_reg.hip do.  What differs is the activations: the four wavefronts need the same 128 rows, so a
+// stage of 64 k (16 KB) is fetched once per workgroup, 16 bytes per thread and piece, and laid into LDS in
+// operand order ([k-step][row block][lane]: a wavefront's operand register quad is one conflict-free 16-byte
+// read).  Per k-step a CU takes in 8 KB of activations + 4 x 2 KB of packed weights for 4 x 72 MFMAs, where
+// the K-split tiles take 4 x 10 KB; the wavefronts' tiles are complete when the loop ends, so there is no
+// reduction over wavefronts either.
+//
+// One barrier per stage, two LDS slots.  Stage s, first k-step: the operand quads of the second k-step are
+// read from LDS while the first is multiplied; then stage s + 1's pieces (fetched two stages earlier into
+// registers) are written to the other slot and stage s + 3's fetched; barrier; second k-step, under which the
+// first operand quads of stage s + 1 are read.  Weights are fetched two stages (less one k-step) ahead.
+//
+// Shapes: K % 64 == 0, C % 8 == 0, 16-byte aligned operands, per-channel parameters; the launch covers whole
+// 512-channel tiles only (the dispatcher gives the remaining columns to the other kernels).  Rows past M are
+// read from row M - 1 and not stored.
+#include "qmatmul_reg.h"
+#include "qmm_reg_common.h"
+#include <type_traits>
+
+namespace {
+
+using namespace qmm;
+
+template <int NWV, typename TX>
+__global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, int M, int K, const uint8_t *pk, int C,
+                                                                   const void *zero, const void *scale,
+                                                                   int zs_dtype, TX *out, int c0, float *out32,
+                                                                   const int32_t *rowexp) {
+  constexpr bool BF = Act<TX>::BF;
+  static_assert(NWV == 4, "the row sums are dealt to four wavefronts");
+  constexpr int NT = 64 * NWV;
+  constexpr int CH = 1024 / NT;                  // 16-byte pieces of a stage per thread
+  constexpr int RB = 8;
+  __shared__ u32x4_t a_lds[2 * 2 * RB * 64];       // [slot][k-step of the stage][row block][lane]
+  asm volatile("" ::"s"(x), "s"(pk), "s"(zero), "s"(scale), "s"(out), "s"(M), "s"(K), "s"(C), "s"(zs_dtype),
+               "s"(c0), "s"(out32), "s"(rowexp));
+  const int tid = threadIdx.x, lane = tid & 63, wk = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = lane >> 4, l16 = lane & 15;
+  int tx, ty;
+  qmm_tile_coords(tx, ty);
+  const int m0 = ty * 128, nbase = c0 + (tx * NWV + wk) * 128;
+  const int NS = K >> 6;
+  const int col = nbase + 8 * l16;
+
+  // this thread's pieces of a stage: row (tid >> 3) + (NT / 8) i of the tile, k 8 (tid & 7) .. + 7 of the stage
+  const int kc = tid & 7;
+  int xoff[CH];
+#pragma unroll
+  for (int i = 0; i < CH; ++i) xoff[i] = min(m0 + (tid >> 3) + (NT / 8) * i, M - 1) * K + 8 * kc;      // M K < 2^31
+  // piece i lands at [kc >> 2][(tid >> 7) + (NT / 128) i][16 (kc & 3) + ((tid >> 3) & 15)]
+  const int dst0 = ((kc >> 2) * RB + (tid >> 7)) * 64 + 16 * (kc & 3) + ((tid >> 3) & 15);
+  const uint8_t *wp = pk + (int64_t)(4 * g) * C + col;
+
+  u32x4_t stg[2][CH];
+  uint2 wr[2][2][4];
+  u32x4_t aq[2][RB];
+  u32x4_t aqr[2][2];                             // row blocks 2 wk, 2 wk + 1 once more, for the row sums
+  auto load_a = [&](int p, int s) __attribute__((always_inline)) {
+    const int so = 64 * min(s, NS - 1);
+#pragma unroll
+    for (int i = 0; i < CH; ++i) stg[p][i] = *reinterpret_cast<const u32x4_t *>(x + xoff[i] + so);
+  };
+  auto write_a = [&](int p, int slot) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < CH; ++i) a_lds[slot * (2 * RB * 64) + dst0 + (NT / 128) * 64 * i] = stg[p][i];
+  };
+  auto load_w = [&](int p, int h, int s) __attribute__((always_inline)) {
+    const uint8_t *q = wp + (int64_t)(32 * min(s, NS - 1) + 16 * h) * C;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) wr[p][h][i] = *reinterpret_cast<const uint2 *>(q + (int64_t)i * C);
+  };
+  auto read_a = [&](int q, int slot, int h) __attribute__((always_inline)) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) aq[q][rb] = a_lds[((slot * 2 + h) * RB + rb) * 64 + lane];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) aqr[q][j] = a_lds[((slot * 2 + h) * RB + 2 * wk + j) * 64 + lane];
+  };
+
+  uint32_t zraw0[8];
+  rg_params8_raw(zero, zs_dtype, 0, col, C, zraw0);
+  __builtin_amdgcn_sched_barrier(0);
+  load_a(1, 0);
+  load_w(0, 0, 0);
+  load_w(0, 1, 0);
+  load_a(0, 1);
+  load_w(1, 0, 1);
+  load_w(1, 1, 1);
+  __builtin_amdgcn_sched_barrier(0);
+
+  uint32_t zc[8];
+#pragma unroll
+  for (int t8 = 0; t8 < 8; ++t8) {
+    const float zi = fminf(fmaxf(rintf(rg_raw_to_f32(zraw0[t8], zs_dtype)), -512.f), 512.f);
+    zc[t8] = BF ? 0u : __builtin_bit_cast(uint32_t, half2_t{(_Float16)(-(1024.f + zi)), (_Float16)(-(64.f + zi))});
+  }
+  uint32_t mask = BF ? 0x000F000Fu : 0x00F0000Fu, cexp = BF ? 0x43004300u : 0x64006400u;
+  asm volatile("" : "+s"(mask));
+  asm volatile("" : "+v"(cexp));
+  const half2_t unscale = half2_t{(_Float16)1.f, (_Float16)0.0625f};
+  const uint32_t one2 = BF ? 0x3F803F80u : 0x3C003C00u;
+  uint4 ones = make_uint4(one2, one2, one2, one2);
+  asm volatile("" : "+v"(ones.x), "+v"(ones.y), "+v"(ones.z), "+v"(ones.w));      // kept in registers: not rebuilt in front of an MFMA
+
+  floatx4 acc[RB][8];
+#pragma unroll
+  for (int i = 0; i < RB; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  // operand register i of tile t8 (channel 8 l16 + t8): codes of packed row i of the lane's four, see qmatmul_reg.hip
+  auto dq_reg = [&](const uint2 (&w)[4], int t8, int i) __attribute__((always_inline)) -> uint32_t {
+    const uint32_t tb = (uint32_t)(t8 & 3);
+    const uint32_t sel = BF ? (0x0c0c0c00u | tb) : (0x0c000c00u | tb | (tb << 16));
+    const uint32_t pb = __builtin_amdgcn_perm(0u, t8 < 4 ? w[i].x : w[i].y, sel);
+    if (BF) return (((pb << 12) | pb) & mask) | cexp;                  // {128 + lo, 128 + hi}
+    const uint32_t v = (pb & mask) | cexp;                             // {1024 + lo, 1024 + 16 hi}
+    const half2_t d = __builtin_bit_cast(half2_t, v) * unscale + __builtin_bit_cast(half2_t, zc[t8]);
+    return __builtin_bit_cast(uint32_t, d);
+  };
+  // One k-step: the in-place MFMAs are inline asm, which the scheduler does not move, so the source order is the
+  // issue order: after every second MFMA of a tile the three vector instructions of one operand register of the
+  // next tile (under the last tile: of the first tile of the next k-step).  The vector instructions stand after
+  // the even row blocks' MFMAs, so every MFMA that reads a freshly built operand has at least one other MFMA
+  // between itself and the instruction that wrote it: the MFMAs need no wait states in front of them.
+  // Row sums (the ninth tile): wavefront wk accumulates those of row blocks 2 wk and 2 wk + 1 only (operand quads
+  // ar, read from LDS a second time so that no register is indexed with wk); the wavefronts exchange them through
+  // LDS when the loop is done.
+  uint32_t bcarry[4];
+  floatx4 rsum[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
+  auto step_pipe = [&](const u32x4_t (&a)[RB], const u32x4_t (&ar)[2], const uint2 (&w)[4], const uint2 (&wn)[4]) __attribute__((always_inline)) {
+    uint32_t bc[4] = {bcarry[0], bcarry[1], bcarry[2], bcarry[3]};
+#pragma unroll
+    for (int t8 = 0; t8 < 8; ++t8) {
+      const uint4 b = make_uint4(bc[0], bc[1], bc[2], bc[3]);
+      uint32_t nx[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        Act<TX>::mma_acc_nw(acc[rb][t8], __builtin_bit_cast(uint4, a[rb]), b);
+        if (!(rb & 1)) nx[rb >> 1] = t8 < 7 ? dq_reg(w, t8 + 1, rb >> 1) : dq_reg(wn, 0, rb >> 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) bc[i] = nx[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) bcarry[i] = bc[i];
+    Act<TX>::mma_accv_nw(rsum[0], __builtin_bit_cast(uint4, ar[0]), ones);
+    Act<TX>::mma_accv_nw(rsum[1], __builtin_bit_cast(uint4, ar[1]), ones);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  write_a(1, 0);
+  load_a(1, 2);
+  __syncthreads();
+  read_a(0, 0, 0);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) bcarry[i] = dq_reg(wr[0][0], 0, i);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // stage s with ring position cur = s & 1 (a compile-time constant: registers are indexed with it)
+  auto stage = [&](auto curc, int s) __attribute__((always_inline)) {
+    constexpr int cur = decltype(curc)::value;
+    read_a(1, cur, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    step_pipe(aq[0], aqr[0], wr[cur][0], wr[cur][1]);
+    load_w(cur, 0, s + 2);
+    write_a(cur, cur ^ 1);
+    load_a(cur, s + 3);
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    read_a(0, cur ^ 1, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    step_pipe(aq[1], aqr[1], wr[cur][1], wr[cur ^ 1][0]);
+    load_w(cur, 1, s + 2);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  int s = 0;
+  for (; s + 2 <= NS; s += 2) {
+    stage(std::integral_constant<int, 0>{}, s);
+    stage(std::integral_constant<int, 1>{}, s + 1);
+  }
+  if (s < NS) stage(std::integral_constant<int, 0>{}, s);
+
+  mma_drain();
+  float sc[8], zf[8];
+  rg_params8(scale, zs_dtype, col, C, sc);
+  rg_params8(zero, zs_dtype, col, C, zf);
+  // the row sums change hands through the LDS of the activations, once every wavefront has left the loop
+  floatx4 *rs_lds = reinterpret_cast<floatx4 *>(a_lds);                 // [row block][lane]
+  __syncthreads();
+  rs_lds[(2 * wk) * 64 + lane] = rsum[0];
+  rs_lds[(2 * wk + 1) * 64 + lane] = rsum[1];
+  __syncthreads();
+  float zfa[8];
+#pragma unroll
+  for (int t8 = 0; t8 < 8; ++t8)
+    zfa[t8] = BF ? 128.f + zf[t8] : zf[t8] - fminf(fmaxf(rintf(zf[t8]), -512.f), 512.f);
+  // acc[rb][t8][r] = sum_k x[m][k] (code - zi)[k][col + t8] (bf16: code + 128), rs_lds[rb][lane][r] = sum_k x[m][k],
+  // m = m0 + 16 rb + 4 g + r
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const floatx4 rs4 = rs_lds[rb * 64 + lane];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = m0 + 16 * rb + 4 * g + r;
+      if (m >= M) continue;
+      const float rs = rs4[r];
+      TX o[8];
+#pragma unroll
+      for (int t8 = 0; t8 < 8; ++t8) o[t8] = Act<TX>::out(sc[t8] * (acc[rb][t8][r] - zfa[t8] * rs));
+      if (out32 != nullptr) {
+        // fp32 rows: the fp16 result widened and scaled back by the row's power of two (exact)
+        const int e = rowexp[m];
+        float *d32 = out32 + (int64_t)m * C + col;
+        float f[8];
+#pragma unroll
+        for (int t8 = 0; t8 < 8; ++t8) f[t8] = ldexpf((float)o[t8], e);
+        *reinterpret_cast<float4 *>(d32) = make_float4(f[0], f[1], f[2], f[3]);
+        *reinterpret_cast<float4 *>(d32 + 4) = make_float4(f[4], f[5], f[6], f[7]);
+        continue;
+      }
+      *reinterpret_cast<uint4 *>(out + (int64_t)m * C + col) = *reinterpret_cast<const uint4 *>(o);
+    }
+  }
+}
+
+template <typename TX>
+int launch_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
+                const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32, const int32_t *rowexp) {
+  const int64_t K = 2 * R;
+  int64_t rows_max = ((1LL << 31) - 1) / K;
+  if (rows_max > 65535LL * 128) rows_max = 65535LL * 128;
+  rows_max -= rows_max % 128;
+  if (rows_max < 128) return GPTQ_HIP_EINVAL;
+  for (int64_t r0 = 0; r0 < M; r0 += rows_max) {
+    const int64_t rows = M - r0 < rows_max ? M - r0 : rows_max;
+    const dim3 grid((unsigned)wide_x, (unsigned)ceil_div64(rows, 128), 1);
+    hipLaunchKernelGGL((qmm_fwd_wide_kernel<4, TX>), grid, dim3(256), 0, st, (const TX *)x + r0 * K, (int)rows, (int)K,
+                       pk, (int)C, zero, scale, zs_dtype, (TX *)out + r0 * C, 0, out32 ? out32 + r0 * C : nullptr,
+                       rowexp ? rowexp + r0 : nullptr);
+    GPTQ_CHECK_LAUNCH();
+  }
+  return GPTQ_HIP_OK;
+}
+
+}  // namespace
+
+namespace qmm {
+
+int64_t wide_fwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned) {
+  const int64_t K = 2 * R;
+  if (!aligned || K % 64 != 0 || K < 512 || C % 8 != 0 || M < 256) return 0;
+  const int64_t tiles_y = ceil_div64(M, 128), full_x = C / 512;
+  const int64_t wgs = full_x * tiles_y;
+  // whole rounds of 256 workgroups (one per CU); a single round that is at least 7/8 full is taken as it is
+  if (wgs >= 256) return (wgs / 256) * 256 / tiles_y;
+  return wgs >= 224 ? full_x : 0;
+}
+
+int wide_fwd_launch(hipStream_t st, const void *x, int x_dtype, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
+                    const void *zero, const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32,
+                    const int32_t *rowexp) {
+  if (zs_dtype != GPTQ_HIP_F32 && zs_dtype != GPTQ_HIP_F16 && zs_dtype != GPTQ_HIP_BF16) return GPTQ_HIP_EDTYPE;
+  if (wide_x < 1 || wide_x * 512 > C) return GPTQ_HIP_EINVAL;
+  if (x_dtype == GPTQ_HIP_BF16)
+    return launch_wide<__hip_bfloat16>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp);
+  if (x_dtype != GPTQ_HIP_F16) return GPTQ_HIP_EDTYPE;
+  return launch_wide<__half>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp);
+}
+
+}  // namespace qmm

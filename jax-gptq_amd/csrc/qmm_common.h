@@ -33,6 +33,16 @@ template <> struct Act<__half> {
     asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0"
                  : "+v"(c) : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)));
   }
+  // The same two without the wait states: for a caller whose source order guarantees that the instruction in
+  // front of the MFMA is not a vector instruction that writes one of its operands (e.g. another MFMA).
+  static __device__ __forceinline__ void mma_acc_nw(floatx4 &c, const uint4 &a, const uint4 &b) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0"
+                 : "+a"(c) : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)));
+  }
+  static __device__ __forceinline__ void mma_accv_nw(floatx4 &c, const uint4 &a, const uint4 &b) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0"
+                 : "+v"(c) : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)));
+  }
   static __device__ __forceinline__ __half out(float v) { return __float2half_rn(v); }
 };
 template <> struct Act<__hip_bfloat16> {
@@ -50,6 +60,16 @@ template <> struct Act<__hip_bfloat16> {
   }
   static __device__ __forceinline__ void mma_accv(floatx4 &c, const uint4 &a, const uint4 &b) {
     asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                 : "+v"(c) : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)));
+  }
+  // The same two without the wait states: for a caller whose source order guarantees that the instruction in
+  // front of the MFMA is not a vector instruction that writes one of its operands (e.g. another MFMA).
+  static __device__ __forceinline__ void mma_acc_nw(floatx4 &c, const uint4 &a, const uint4 &b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                 : "+a"(c) : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)));
+  }
+  static __device__ __forceinline__ void mma_accv_nw(floatx4 &c, const uint4 &a, const uint4 &b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
                  : "+v"(c) : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)));
   }
   static __device__ __forceinline__ __hip_bfloat16 out(float v) { return __float2bfloat16(v); }

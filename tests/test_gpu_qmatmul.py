@@ -168,6 +168,35 @@ def test_qmatmul_bf16_x_mfma_path(OP, M, N, K, zs):
     assert np.all(err <= 1e-2 + 2.0 ** -8 * np.abs(ref)), err.max()
 
 
+@pytest.mark.parametrize("xdt,zs", [("float16", "float32"), ("float16", "float16"), ("bfloat16", "float32"),
+                                    ("bfloat16", "bfloat16"), ("float32", "float32")])
+@pytest.mark.parametrize("M,N,K", [(3500, 4480, 512), (2048, 11008, 1024), (4096, 4096, 576)])
+def test_qmatmul_many_rows_128x512_tiles(OP, M, N, K, xdt, zs):
+    """Forward products of many rows: the leading columns that fill whole rounds of workgroups run on
+    128 x 512 tiles whose wavefronts share the activations through LDS, the rest on the 128- and 64-row
+    tiles (4480 = 8 x 512 + 384 columns; 11008: 16 tiles + 22 x 128 columns; M = 3500 leaves a ragged
+    last row tile; K = 576 has an odd number of 64-k stages).  Fractional zero points exercise the row
+    sums that the wavefronts exchange; fp32 rows the scaled fp32 store."""
+    import torch
+    import jax_gptq_amd.gptq as G
+    rng = np.random.default_rng(M + N + K)
+    codes = rng.integers(0, 16, (K, N)).astype(np.uint8)
+    tdt = getattr(torch, zs)
+    scale = torch.from_numpy(rng.uniform(0.001, 0.01, N).astype(np.float32)).to(tdt)
+    zero = torch.from_numpy(rng.uniform(0.0, 15.0, N).astype(np.float32)).to(tdt)
+    qm = G.QuantizedMatrix(torch.from_numpy(O.pack_colwise(codes)).cuda(), zero.cuda(), scale.cuda())
+    rowscale = np.array([1.0, 1e-3, 3e4])[np.arange(M) % 3][:, None] if xdt == "float32" else np.ones((M, 1))
+    x = torch.from_numpy((rng.standard_normal((M, K)) * rowscale).astype(np.float32)).to(getattr(torch, xdt))
+    got = OP.quantized_matmul(x, qm)
+    assert got.dtype == getattr(torch, xdt) and tuple(got.shape) == (M, N)
+    dense = (codes.astype(np.float64) - zero.double().numpy()[None]) * scale.double().numpy()[None]
+    ref = x.double().numpy() @ dense
+    err = np.abs(to_np(got).astype(np.float64) - ref)
+    rel = 2.0 ** -8 if xdt == "bfloat16" else RTOL
+    tol = (ATOL + rel * np.abs(ref / rowscale)) * rowscale
+    assert np.all(err <= tol), float((err / tol).max())
+
+
 @pytest.mark.parametrize("zs", ["float32", "float16", "bfloat16"])
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 11008), (16, 11008, 4096), (128, 4096, 1024), (70, 2304, 768),
                                    (5, 48, 96), (200, 5120, 256), (300, 1008, 514), (2048, 4096, 512)])
