@@ -130,7 +130,8 @@ __global__ __launch_bounds__(256, (RB == 1 ? 2 : 1)) void qmm_fwd_reg_kernel(con
   asm volatile("" : "+v"(cexp));
   const half2_t unscale = half2_t{(_Float16)1.f, (_Float16)0.0625f};
   const uint32_t one2 = BF ? 0x3F803F80u : 0x3C003C00u;
-  const uint4 ones = make_uint4(one2, one2, one2, one2);
+  uint4 ones = make_uint4(one2, one2, one2, one2);
+  asm volatile("" : "+v"(ones.x), "+v"(ones.y), "+v"(ones.z), "+v"(ones.w));      // kept in registers: not rebuilt in front of an MFMA
 
   floatx4 acc[RB][RG_NT];
 #pragma unroll
@@ -264,18 +265,33 @@ __global__ __launch_bounds__(256, (RB == 1 ? 2 : 1)) void qmm_fwd_reg_kernel(con
 #pragma unroll
     for (int i = 0; i < NL; ++i) w[i] = RAGGED ? rg_shr_bytes(wr[slot][i], wshift) : wr[slot][i];
   };
+  // 128-row tiles: the vector instructions stand after the MFMAs of the even row blocks, so an MFMA that reads a
+  // freshly built operand always has another MFMA between itself and the instruction that wrote it (the odd row
+  // blocks' MFMAs count as a use of what was just built, which keeps the compiler from sinking it further), and
+  // the MFMAs go without wait states.  Where that use cannot be expressed (the first tile of the next k-step, built
+  // under the row-sum MFMAs) and at the head of the k-step the wait states stay.
+  auto pipe_mma = [&](floatx4 &c, const uint4 &a, const uint4 &b) __attribute__((always_inline)) {
+    if constexpr (RB == 8) Act<TX>::mma_acc_nw(c, a, b);
+    else Act<TX>::mma_acc(c, a, b);
+  };
+  auto pipe_mmav = [&](floatx4 &c, const uint4 &a, const uint4 &b) __attribute__((always_inline)) {
+    if constexpr (RB == 8) Act<TX>::mma_accv_nw(c, a, b);
+    else Act<TX>::mma_accv(c, a, b);
+  };
   auto step_pipe = [&](int slot, int next_slot) __attribute__((always_inline)) {
     uint2 w[NL];
     shifted(slot, w);
     uint32_t bc[4] = {bcarry[0], bcarry[1], bcarry[2], bcarry[3]};
+    if constexpr (RB == 8) asm volatile("s_nop 1");
 #pragma unroll
     for (int t8 = 0; t8 < 8; ++t8) {
       const uint4 b = make_uint4(bc[0], bc[1], bc[2], bc[3]);
       uint32_t nx[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
-        Act<TX>::mma_acc(acc[rb][t8], aq[slot][rb], b);
-        if (t8 < 7 && (RB == 4 || (rb & 1))) nx[RB == 4 ? rb : rb >> 1] = dq_reg(w, t8 + 1, RB == 4 ? rb : rb >> 1);
+        if (RB == 8 && (rb & 1) && t8 < 7) Act<TX>::mma_acc_nw_after(acc[rb][t8], aq[slot][rb], b, nx[rb >> 1]);
+        else pipe_mma(acc[rb][t8], aq[slot][rb], b);
+        if (t8 < 7 && (RB == 4 || !(rb & 1))) nx[RB == 4 ? rb : rb >> 1] = dq_reg(w, t8 + 1, RB == 4 ? rb : rb >> 1);
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
@@ -285,8 +301,9 @@ __global__ __launch_bounds__(256, (RB == 1 ? 2 : 1)) void qmm_fwd_reg_kernel(con
     shifted(next_slot, wn);
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
-      Act<TX>::mma_accv(acc[rb][8], aq[slot][rb], ones);
-      if (RB == 4 || (rb & 1)) bcarry[RB == 4 ? rb : rb >> 1] = dq_reg(wn, 0, RB == 4 ? rb : rb >> 1);
+      if (RB == 8 && (rb & 1)) Act<TX>::mma_accv(acc[rb][8], aq[slot][rb], ones);      // (with wait states: see bcarry)
+      else pipe_mmav(acc[rb][8], aq[slot][rb], ones);
+      if (RB == 4 || !(rb & 1)) bcarry[RB == 4 ? rb : rb >> 1] = dq_reg(wn, 0, RB == 4 ? rb : rb >> 1);
       __builtin_amdgcn_sched_barrier(0);
     }
   };

@@ -125,8 +125,9 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
   // One k-step: the in-place MFMAs are inline asm, which the scheduler does not move, so the source order is the
   // issue order: after every second MFMA of a tile the three vector instructions of one operand register of the
   // next tile (under the last tile: of the first tile of the next k-step).  The vector instructions stand after
-  // the even row blocks' MFMAs, so every MFMA that reads a freshly built operand has at least one other MFMA
-  // between itself and the instruction that wrote it: the MFMAs need no wait states in front of them.
+  // the even row blocks' MFMAs and the odd ones count as a use of what was just built, so every MFMA that reads a
+  // freshly built operand has at least one other MFMA between itself and the instruction that wrote it: the
+  // MFMAs need no wait states in front of them.
   // Row sums (the ninth tile): wavefront wk accumulates those of row blocks 2 wk and 2 wk + 1 only (operand quads
   // ar, read from LDS a second time so that no register is indexed with wk); the wavefronts exchange them through
   // LDS when the loop is done.
@@ -140,7 +141,8 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
       uint32_t nx[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
-        Act<TX>::mma_acc_nw(acc[rb][t8], __builtin_bit_cast(uint4, a[rb]), b);
+        if (rb & 1) Act<TX>::mma_acc_nw_after(acc[rb][t8], __builtin_bit_cast(uint4, a[rb]), b, nx[rb >> 1]);
+        else Act<TX>::mma_acc_nw(acc[rb][t8], __builtin_bit_cast(uint4, a[rb]), b);
         if (!(rb & 1)) nx[rb >> 1] = t8 < 7 ? dq_reg(w, t8 + 1, rb >> 1) : dq_reg(wn, 0, rb >> 1);
         __builtin_amdgcn_sched_barrier(0);
       }

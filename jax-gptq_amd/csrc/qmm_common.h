@@ -43,6 +43,13 @@ template <> struct Act<__half> {
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0"
                  : "+v"(c) : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)));
   }
+  // mma_acc_nw that also counts as a use of `dep` (which the instruction does not read): whatever computes
+  // `dep` is thereby placed in front of this MFMA, so the MFMA that really reads it, further down, has this one
+  // between itself and the write.  (The compiler is otherwise free to sink a computation down to its first use.)
+  static __device__ __forceinline__ void mma_acc_nw_after(floatx4 &c, const uint4 &a, const uint4 &b, uint32_t dep) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0"
+                 : "+a"(c) : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)), "v"(dep));
+  }
   static __device__ __forceinline__ __half out(float v) { return __float2half_rn(v); }
 };
 template <> struct Act<__hip_bfloat16> {
@@ -71,6 +78,13 @@ template <> struct Act<__hip_bfloat16> {
   static __device__ __forceinline__ void mma_accv_nw(floatx4 &c, const uint4 &a, const uint4 &b) {
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
                  : "+v"(c) : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)));
+  }
+  // mma_acc_nw that also counts as a use of `dep` (which the instruction does not read): whatever computes
+  // `dep` is thereby placed in front of this MFMA, so the MFMA that really reads it, further down, has this one
+  // between itself and the write.  (The compiler is otherwise free to sink a computation down to its first use.)
+  static __device__ __forceinline__ void mma_acc_nw_after(floatx4 &c, const uint4 &a, const uint4 &b, uint32_t dep) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                 : "+a"(c) : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)), "v"(dep));
   }
   static __device__ __forceinline__ __hip_bfloat16 out(float v) { return __float2bfloat16(v); }
 };
