@@ -38,6 +38,11 @@ int wide_fwd_launch(hipStream_t st, const void *x, int x_dtype, int64_t M, const
                     const void *zero, const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32,
                     const int32_t *rowexp);
 
+// The same for the transposed product (fp16 rows): leading tiles of 512 output columns = 256 packed rows.
+int64_t wide_bwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned);
+int wide_bwd_launch(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
+                    const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32, const int32_t *rowexp);
+
 // Transposed product out[M, K] = x[M, C] @ dequant(packed[R, C])^T.
 struct RegBwdPlan {
   bool use;

@@ -378,29 +378,53 @@ int launch_inst(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, c
   return GPTQ_HIP_OK;
 }
 
+// 128-row tiles whose last round of workgroups would be at most half full: this many trailing column tiles run on
+// 64-row tiles in a second launch (as in the forward kernel's plan)
+int64_t bwd_deal_tail(int64_t tiles_x, int64_t tiles_y, int64_t T) {
+  if (T < 64) return 0;
+  const int64_t all = tiles_x * tiles_y, full = all / 256, rem = all % 256;
+  if (full < 1 || rem == 0 || rem > 128) return 0;
+  const int64_t main_x = full * 256 / tiles_y, tail = tiles_x - main_x;
+  return (main_x >= 1 && tail >= 1 && tail * tiles_y * 2 <= 256) ? tail : 0;
+}
+
 template <int BITS, typename TX>
 int launch_bx(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
               int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws, int group_size) {
-  {
-    if (p.rb == 8 && p.tail_x > 0) {
-      // 128-row tiles on the columns that fill whole rounds of workgroups, 64-row tiles on the rest
-      const int64_t main_x = ceil_div64(R, BITS == 4 ? 64 : 128) - p.tail_x;
+  if (p.rb == 8) {
+    const int64_t tiles_all = ceil_div64(R, BITS == 4 ? 64 : 128), tiles_y = ceil_div64(M, 128);
+    // 128 x 512 tiles (qmatmul_wide.hip) on the leading output columns that fill whole rounds of workgroups
+    int64_t first = 0;
+    if constexpr (BITS == 4 && !Act<TX>::BF) {
+      // (also where this kernel's own tiles need a split because the constants of all channels do not fit its LDS)
+      if (!p.ragged && group_size == 0) {
+        const int64_t wide_x = wide_bwd_tiles(M, R, C, true);
+        if (wide_x > 0) {
+          const int rc = wide_bwd_launch(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, p.out32, p.rowexp);
+          if (rc) return rc;
+          first = 4 * wide_x;
+        }
+      }
+    }
+    const int64_t rest = tiles_all - first;
+    if (rest == 0) return GPTQ_HIP_OK;
+    // of the rest: 128-row tiles on the columns that fill whole rounds of workgroups, 64-row tiles on the others
+    int64_t tail = first == 0 ? p.tail_x : (p.S == 1 ? bwd_deal_tail(rest, tiles_y, ceil_div64(C, 32)) : 0);
+    if (first > 0 && p.S == 1 && rest * tiles_y <= 128) tail = rest;
+    const int64_t main_x = rest - tail;
+    if (main_x > 0) {
       const int rc = p.ragged ? launch_inst<BITS, true, TX, 8>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws,
-                                                               group_size, 0, main_x)
+                                                               group_size, first, main_x)
                               : launch_inst<BITS, false, TX, 8>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws,
-                                                                group_size, 0, main_x);
+                                                                group_size, first, main_x);
       if (rc) return rc;
-      if (p.ragged)
-        return launch_inst<BITS, true, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size, main_x,
-                                           p.tail_x);
-      return launch_inst<BITS, false, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size, main_x,
-                                          p.tail_x);
     }
-    if (p.rb == 8) {
-      if (p.ragged)
-        return launch_inst<BITS, true, TX, 8>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
-      return launch_inst<BITS, false, TX, 8>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
-    }
+    if (tail == 0) return GPTQ_HIP_OK;
+    if (p.ragged)
+      return launch_inst<BITS, true, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size,
+                                         first + main_x, tail);
+    return launch_inst<BITS, false, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size,
+                                        first + main_x, tail);
   }
   if (p.ragged) return launch_inst<BITS, true, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
   return launch_inst<BITS, false, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
@@ -434,16 +458,7 @@ RegBwdPlan reg_bwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned,
   if (S < s_min) S = s_min;
   p.steps = (int)ceil_div64(T, S);
   p.S = (int)ceil_div64(T, p.steps);
-  // 128-row tiles whose last round of workgroups would be at most half full: the trailing column tiles run on
-  // 64-row tiles in a second launch (as in the forward kernel's plan)
-  p.tail_x = 0;
-  if (p.rb == 8 && p.S == 1 && T >= 64) {
-    const int64_t all = tiles_x * tiles_y, full = all / 256, rem = all % 256;
-    if (full >= 1 && rem > 0 && rem <= 128) {
-      const int64_t main_x = full * 256 / tiles_y, tail = tiles_x - main_x;
-      if (main_x >= 1 && tail >= 1 && tail * tiles_y * 2 <= 256) p.tail_x = (int)tail;
-    }
-  }
+  p.tail_x = (p.rb == 8 && p.S == 1) ? (int)bwd_deal_tail(tiles_x, tiles_y, T) : 0;
   p.part_bytes = p.S > 1 ? (size_t)p.tiles * p.S * p.rb * RG_NT * RG_TILE_FLOATS * sizeof(float) : 0;
   p.total_bytes = p.S > 1 ? QMM_HEAD_BYTES + p.part_bytes : 0;
   p.use = true;

@@ -231,6 +231,173 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
   }
 }
 
+// The transposed product on the same tiling: out[M, K] = x[M, C] @ ((code - zero) * scale)^T, fp16 rows.  A
+// wavefront owns 128 rows x 128 output columns (64 packed rows) over all channels; the contraction runs along the
+// channels, in stages of 64, whose activations the four wavefronts share through LDS as above; the weight operand
+// is built as in qmatmul_reg_bwd.hip (lane (l16, g): 8 channels of packed row j0 + 16 jg + l16; scale and
+// -zero * scale of all channels converted once into LDS).  C % 64 == 0, whole 512-column tiles only.
+template <typename TX>
+__global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M, const uint8_t *pk, int R, int C,
+                                                               const void *zero, const void *scale, int zs_dtype,
+                                                               TX *out, float *out32, const int32_t *rowexp) {
+  static_assert(!Act<TX>::BF, "fp16 rows");
+  constexpr int RB = 8, NG = 4;
+  extern __shared__ __attribute__((aligned(16))) float wide_lds[];     // halves sc[C], halves nzs[C], then the stages
+  _Float16 *tab_s = reinterpret_cast<_Float16 *>(wide_lds);
+  _Float16 *tab_nz = tab_s + C;
+  u32x4_t *a_lds = reinterpret_cast<u32x4_t *>(wide_lds + C);          // [slot][k-step of the stage][row block][lane]
+  const int tid = threadIdx.x, lane = tid & 63, wk = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = lane >> 4, l16 = lane & 15;
+  int tx, ty;
+  qmm_tile_coords(tx, ty);
+  const int m0 = ty * 128, j0 = (tx * 4 + wk) * 64;
+  const int NS = C >> 6;
+
+  const int kc = tid & 7;
+  int xoff[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) xoff[i] = min(m0 + (tid >> 3) + 32 * i, M - 1) * C + 8 * kc;            // M C < 2^31
+  const int dst0 = ((kc >> 2) * RB + (tid >> 7)) * 64 + 16 * (kc & 3) + ((tid >> 3) & 15);
+  const uint8_t *wpj[NG];
+#pragma unroll
+  for (int jg = 0; jg < NG; ++jg) wpj[jg] = pk + (int64_t)(j0 + 16 * jg + l16) * C + 8 * g;
+
+  u32x4_t stg[2][4];
+  uint2 wr[2][2][NG];
+  u32x4_t aq[2][RB];
+  auto load_a = [&](int p, int s) __attribute__((always_inline)) {
+    const int so = 64 * min(s, NS - 1);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) stg[p][i] = *reinterpret_cast<const u32x4_t *>(x + xoff[i] + so);
+  };
+  auto write_a = [&](int p, int slot) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a_lds[slot * (2 * RB * 64) + dst0 + 2 * 64 * i] = stg[p][i];
+  };
+  auto load_w = [&](int p, int h, int s) __attribute__((always_inline)) {
+    const int c = 64 * min(s, NS - 1) + 32 * h;
+#pragma unroll
+    for (int jg = 0; jg < NG; ++jg) wr[p][h][jg] = *reinterpret_cast<const uint2 *>(wpj[jg] + c);
+  };
+  auto read_a = [&](int q, int slot, int h) __attribute__((always_inline)) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) aq[q][rb] = a_lds[((slot * 2 + h) * RB + rb) * 64 + lane];
+  };
+
+  load_a(1, 0);
+  load_w(0, 0, 0);
+  load_w(0, 1, 0);
+  load_a(0, 1);
+  load_w(1, 0, 1);
+  load_w(1, 1, 1);
+  __builtin_amdgcn_sched_barrier(0);
+  // per-channel constants of all channels
+  for (int c = tid; c < C; c += 256) {
+    const float z = rg_param(zero, zs_dtype, c), sc = rg_param(scale, zs_dtype, c);
+    tab_s[c] = (_Float16)sc;
+    tab_nz[c] = (_Float16)(-z * sc);
+  }
+
+  floatx4 acc[RB][8];
+#pragma unroll
+  for (int i = 0; i < RB; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const half2_t k1024 = half2_t{(_Float16)1024.f, (_Float16)1024.f};
+  const half2_t k16th = half2_t{(_Float16)0.0625f, (_Float16)0.0625f}, k64 = half2_t{(_Float16)64.f, (_Float16)64.f};
+  uint32_t c64 = 0x64646464u;
+  asm volatile("" : "+v"(c64));
+
+  // one k-step of 32 channels starting at channel c0 (of which this lane's operand registers hold 8 g .. 8 g + 7)
+  auto compute = [&](const u32x4_t (&a)[RB], const uint2 (&w)[NG], int c0) __attribute__((always_inline)) {
+    const int ti = c0 + 8 * g;
+    const uint4 s4 = *reinterpret_cast<const uint4 *>(tab_s + ti);
+    const uint4 n4 = *reinterpret_cast<const uint4 *>(tab_nz + ti);
+    const uint32_t sw[4] = {s4.x, s4.y, s4.z, s4.w}, nw[4] = {n4.x, n4.y, n4.z, n4.w};
+#pragma unroll
+    for (int jg = 0; jg < NG; ++jg) {
+      uint32_t lo4[4], hi4[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t word = i < 2 ? w[jg].x : w[jg].y;
+        const uint32_t sel = (i & 1) ? 0x04030402u : 0x04010400u;            // bytes (2e, 2e+1) under 0x64
+        const half2_t sc = __builtin_bit_cast(half2_t, sw[i]), nz = __builtin_bit_cast(half2_t, nw[i]);
+        const half2_t cl = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(c64, word & 0x0F0F0F0Fu, sel)) - k1024;
+        const half2_t ch = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(c64, word & 0xF0F0F0F0u, sel)) * k16th - k64;
+        lo4[i] = __builtin_bit_cast(uint32_t, cl * sc + nz);
+        hi4[i] = __builtin_bit_cast(uint32_t, ch * sc + nz);
+      }
+      const uint4 bl = make_uint4(lo4[0], lo4[1], lo4[2], lo4[3]), bh = make_uint4(hi4[0], hi4[1], hi4[2], hi4[3]);
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        Act<TX>::mma_acc(acc[rb][2 * jg], __builtin_bit_cast(uint4, a[rb]), bl);
+        Act<TX>::mma_acc(acc[rb][2 * jg + 1], __builtin_bit_cast(uint4, a[rb]), bh);
+      }
+    }
+  };
+
+  write_a(1, 0);
+  load_a(1, 2);
+  __syncthreads();                                                   // stage 0 and the tables are in LDS
+  read_a(0, 0, 0);
+  __builtin_amdgcn_sched_barrier(0);
+
+  auto stage = [&](auto curc, int s) __attribute__((always_inline)) {
+    constexpr int cur = decltype(curc)::value;
+    read_a(1, cur, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    compute(aq[0], wr[cur][0], 64 * s);
+    __builtin_amdgcn_sched_barrier(0);
+    load_w(cur, 0, s + 2);
+    write_a(cur, cur ^ 1);
+    load_a(cur, s + 3);
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    read_a(0, cur ^ 1, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    compute(aq[1], wr[cur][1], 64 * s + 32);
+    __builtin_amdgcn_sched_barrier(0);
+    load_w(cur, 1, s + 2);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  int s = 0;
+  for (; s + 2 <= NS; s += 2) {
+    stage(std::integral_constant<int, 0>{}, s);
+    stage(std::integral_constant<int, 1>{}, s + 1);
+  }
+  if (s < NS) stage(std::integral_constant<int, 0>{}, s);
+
+  mma_drain();
+  // acc[rb][2 jg + e][r] = out[m0 + 16 rb + 4 g + r][2 (j0 + 16 jg + l16) + e]
+  const int64_t KO = 2 * (int64_t)R;
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = m0 + 16 * rb + 4 * g + r;
+      if (m >= M) continue;
+      if (out32 != nullptr) {
+        const int e = rowexp[m];
+        float *orow32 = out32 + (int64_t)m * KO;
+#pragma unroll
+        for (int jg = 0; jg < NG; ++jg) {
+          const int j = j0 + 16 * jg + l16;
+          *reinterpret_cast<float2 *>(orow32 + 2 * j) = make_float2(ldexpf((float)Act<TX>::out(acc[rb][2 * jg][r]), e),
+                                                                    ldexpf((float)Act<TX>::out(acc[rb][2 * jg + 1][r]), e));
+        }
+        continue;
+      }
+      TX *orow = out + (int64_t)m * KO;
+#pragma unroll
+      for (int jg = 0; jg < NG; ++jg) {
+        const int j = j0 + 16 * jg + l16;
+        TX o2[2] = {Act<TX>::out(acc[rb][2 * jg][r]), Act<TX>::out(acc[rb][2 * jg + 1][r])};
+        *reinterpret_cast<uint32_t *>(orow + 2 * j) = *reinterpret_cast<const uint32_t *>(o2);
+      }
+    }
+  }
+}
+
 template <typename TX>
 int launch_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
                 const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32, const int32_t *rowexp) {
@@ -244,6 +411,27 @@ int launch_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int
     const dim3 grid((unsigned)wide_x, (unsigned)ceil_div64(rows, 128), 1);
     hipLaunchKernelGGL((qmm_fwd_wide_kernel<4, TX>), grid, dim3(256), 0, st, (const TX *)x + r0 * K, (int)rows, (int)K,
                        pk, (int)C, zero, scale, zs_dtype, (TX *)out + r0 * C, 0, out32 ? out32 + r0 * C : nullptr,
+                       rowexp ? rowexp + r0 : nullptr);
+    GPTQ_CHECK_LAUNCH();
+  }
+  return GPTQ_HIP_OK;
+}
+
+int launch_bwd_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
+                    const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32, const int32_t *rowexp) {
+  auto kern = qmm_bwd_wide_kernel<__half>;
+  const int lds = (int)(4 * C + 2 * 2 * 8 * 64 * 16);
+  if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), lds)) return GPTQ_HIP_ELAUNCH;
+  const int64_t KO = 2 * R;
+  int64_t rows_max = ((1LL << 31) - 1) / C;
+  if (rows_max > 65535LL * 128) rows_max = 65535LL * 128;
+  rows_max -= rows_max % 128;
+  if (rows_max < 128) return GPTQ_HIP_EINVAL;
+  for (int64_t r0 = 0; r0 < M; r0 += rows_max) {
+    const int64_t rows = M - r0 < rows_max ? M - r0 : rows_max;
+    const dim3 grid((unsigned)wide_x, (unsigned)ceil_div64(rows, 128), 1);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (const __half *)x + r0 * C, (int)rows, pk, (int)R, (int)C, zero,
+                       scale, zs_dtype, (__half *)out + r0 * KO, out32 ? out32 + r0 * KO : nullptr,
                        rowexp ? rowexp + r0 : nullptr);
     GPTQ_CHECK_LAUNCH();
   }
@@ -273,6 +461,22 @@ int wide_fwd_launch(hipStream_t st, const void *x, int x_dtype, int64_t M, const
     return launch_wide<__hip_bfloat16>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp);
   if (x_dtype != GPTQ_HIP_F16) return GPTQ_HIP_EDTYPE;
   return launch_wide<__half>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp);
+}
+
+int64_t wide_bwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned) {
+  // (the constants of all channels and the stages share the LDS: 4 C + 32 KB)
+  if (!aligned || C % 64 != 0 || C < 512 || C > 30720 || M < 256) return 0;
+  const int64_t tiles_y = ceil_div64(M, 128), full_x = R / 256;
+  const int64_t wgs = full_x * tiles_y;
+  if (wgs >= 256) return (wgs / 256) * 256 / tiles_y;
+  return wgs >= 224 ? full_x : 0;
+}
+
+int wide_bwd_launch(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
+                    const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32, const int32_t *rowexp) {
+  if (zs_dtype != GPTQ_HIP_F32 && zs_dtype != GPTQ_HIP_F16 && zs_dtype != GPTQ_HIP_BF16) return GPTQ_HIP_EDTYPE;
+  if (wide_x < 1 || wide_x * 256 > R) return GPTQ_HIP_EINVAL;
+  return launch_bwd_wide(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp);
 }
 
 }  // namespace qmm

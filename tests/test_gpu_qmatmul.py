@@ -197,6 +197,32 @@ def test_qmatmul_many_rows_128x512_tiles(OP, M, N, K, xdt, zs):
     assert np.all(err <= tol), float((err / tol).max())
 
 
+@pytest.mark.parametrize("xdt,zs", [("float16", "float32"), ("float16", "float16"), ("float32", "bfloat16")])
+@pytest.mark.parametrize("M,N,K", [(3500, 512, 4480), (2048, 1024, 11008), (4096, 576, 4096), (1800, 20480, 8192)])
+def test_qmatmul_many_rows_128x512_tiles_transposed(OP, M, N, K, xdt, zs):
+    """The transposed product of many fp16 (or fp32) rows on the same tiling: 512 output columns per
+    workgroup, contraction along the channels in stages of 64 (N = 576: an odd number of stages;
+    N = 20480 channels: more than the other kernel's LDS holds constants for, so its tiles split the
+    contraction while these do not)."""
+    import torch
+    import jax_gptq_amd.gptq as G
+    rng = np.random.default_rng(M + N + K)
+    codes = rng.integers(0, 16, (K, N)).astype(np.uint8)
+    tdt = getattr(torch, zs)
+    scale = torch.from_numpy(rng.uniform(0.001, 0.01, N).astype(np.float32)).to(tdt)
+    zero = torch.from_numpy(rng.uniform(0.0, 15.0, N).astype(np.float32)).to(tdt)
+    qm = G.QuantizedMatrix(torch.from_numpy(O.pack_colwise(codes)).cuda(), zero.cuda(), scale.cuda())
+    rowscale = np.array([1.0, 1e-3, 3e4])[np.arange(M) % 3][:, None] if xdt == "float32" else np.ones((M, 1))
+    x = torch.from_numpy((0.05 * rng.standard_normal((M, N)) * rowscale).astype(np.float32)).to(getattr(torch, xdt))
+    got = OP.quantized_matmul(x, qm, transpose_b=True)
+    assert got.dtype == getattr(torch, xdt) and tuple(got.shape) == (M, K)
+    dense = (codes.astype(np.float64) - zero.double().numpy()[None]) * scale.double().numpy()[None]
+    ref = x.double().numpy() @ dense.T
+    err = np.abs(to_np(got).astype(np.float64) - ref)
+    tol = (ATOL + RTOL * np.abs(ref / rowscale)) * rowscale
+    assert np.all(err <= tol), float((err / tol).max())
+
+
 @pytest.mark.parametrize("zs", ["float32", "float16", "bfloat16"])
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 11008), (16, 11008, 4096), (128, 4096, 1024), (70, 2304, 768),
                                    (5, 48, 96), (200, 5120, 256), (300, 1008, 514), (2048, 4096, 512)])
