@@ -199,7 +199,7 @@ def bench_qmatmul(reps=240):
             # precision on the way in, as the reference's dot rounds them to TF32
             cases += [(1, 0, "float32"), (128, 0, "float32")]
         if K * N >= (1 << 27):
-            cases = [(1, 0, "float16"), (16, 0, "float16")]
+            cases = [(1, 0, "float16"), (16, 0, "float16"), (2048, 0, "float16"), (2048, 1, "float16")]
         if N % 16:
             cases = [(1, 0, "float16"), (16, 0, "float16"), (512, 0, "float16"), (512, 1, "float16")]
         for (M, tr, xdt) in cases:
