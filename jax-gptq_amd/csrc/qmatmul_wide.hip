@@ -308,45 +308,87 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   uint32_t c64 = 0x64646464u;
   asm volatile("" : "+v"(c64));
 
-  // one k-step of 32 channels starting at channel c0 (of which this lane's operand registers hold 8 g .. 8 g + 7)
-  auto compute = [&](const u32x4_t (&a)[RB], const uint2 (&w)[NG], int c0) __attribute__((always_inline)) {
-    const int ti = c0 + 8 * g;
-    const uint4 s4 = *reinterpret_cast<const uint4 *>(tab_s + ti);
-    const uint4 n4 = *reinterpret_cast<const uint4 *>(tab_nz + ti);
+  // operand registers of a pair of output columns (low / high nibbles) from word `word` of a packed row: codes of the
+  // two channels that `sel` picks, times their scale, minus zero * scale
+  auto build_lo = [&](uint32_t word, uint32_t sel, uint32_t scw, uint32_t nzw) __attribute__((always_inline)) -> uint32_t {
+    const half2_t cl = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(c64, word & 0x0F0F0F0Fu, sel)) - k1024;
+    return __builtin_bit_cast(uint32_t, cl * __builtin_bit_cast(half2_t, scw) + __builtin_bit_cast(half2_t, nzw));
+  };
+  auto build_hi = [&](uint32_t word, uint32_t sel, uint32_t scw, uint32_t nzw) __attribute__((always_inline)) -> uint32_t {
+    const half2_t ch = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(c64, word & 0xF0F0F0F0u, sel)) * k16th - k64;
+    return __builtin_bit_cast(uint32_t, ch * __builtin_bit_cast(half2_t, scw) + __builtin_bit_cast(half2_t, nzw));
+  };
+  // One k-step of 32 channels starting at channel c0 (of which this lane's operand registers hold 8 g .. 8 g + 7),
+  // software-pipelined: under the 16 MFMAs of a group of 16 packed rows the operand registers of the next group are
+  // built (of the next k-step's first group under the last), four vector instructions behind every second MFMA,
+  // and the MFMA after them counts as a use of the fresh register; so the MFMAs go without wait states, as in the
+  // forward kernel.  carry_l / carry_h: the operand registers of the group about to be multiplied.
+  uint32_t carry_l[4], carry_h[4];
+  auto compute = [&](const u32x4_t (&a)[RB], const uint2 (&w)[NG], const uint2 &wnext, int c0, int c0n)
+                     __attribute__((always_inline)) {
+    const int ti = c0 + 8 * g, tin = min(c0n, C - 32) + 8 * g;
+    const uint4 s4 = *reinterpret_cast<const uint4 *>(tab_s + ti), n4 = *reinterpret_cast<const uint4 *>(tab_nz + ti);
+    const uint4 s4n = *reinterpret_cast<const uint4 *>(tab_s + tin), n4n = *reinterpret_cast<const uint4 *>(tab_nz + tin);
     const uint32_t sw[4] = {s4.x, s4.y, s4.z, s4.w}, nw[4] = {n4.x, n4.y, n4.z, n4.w};
+    const uint32_t swn[4] = {s4n.x, s4n.y, s4n.z, s4n.w}, nwn[4] = {n4n.x, n4n.y, n4n.z, n4n.w};
+    uint32_t bl[4] = {carry_l[0], carry_l[1], carry_l[2], carry_l[3]};
+    uint32_t bh[4] = {carry_h[0], carry_h[1], carry_h[2], carry_h[3]};
 #pragma unroll
     for (int jg = 0; jg < NG; ++jg) {
-      uint32_t lo4[4], hi4[4];
+      const uint4 Bl = make_uint4(bl[0], bl[1], bl[2], bl[3]), Bh = make_uint4(bh[0], bh[1], bh[2], bh[3]);
+      const uint2 wsrc = jg + 1 < NG ? w[jg + 1 < NG ? jg + 1 : 0] : wnext;
+      uint32_t nl[4] = {0u, 0u, 0u, 0u}, nh[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int n = 0; n < 16; ++n) {
+        const int rb = n >> 1, i = n >> 2;
+        const bool hi_piece = (n >> 1) & 1;
+        if (!(n & 1)) {
+          Act<TX>::mma_acc_nw(acc[rb][2 * jg], __builtin_bit_cast(uint4, a[rb]), Bl);
+          const uint32_t word = i < 2 ? wsrc.x : wsrc.y;
+          const uint32_t sel = (i & 1) ? 0x04030402u : 0x04010400u;          // bytes (2e, 2e+1) under 0x64
+          const uint32_t scw = jg + 1 < NG ? sw[i] : swn[i], nzw = jg + 1 < NG ? nw[i] : nwn[i];
+          if (hi_piece) nh[i] = build_hi(word, sel, scw, nzw);
+          else nl[i] = build_lo(word, sel, scw, nzw);
+        } else {
+          Act<TX>::mma_acc_nw_after(acc[rb][2 * jg + 1], __builtin_bit_cast(uint4, a[rb]), Bh, hi_piece ? nh[i] : nl[i]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const uint32_t word = i < 2 ? w[jg].x : w[jg].y;
-        const uint32_t sel = (i & 1) ? 0x04030402u : 0x04010400u;            // bytes (2e, 2e+1) under 0x64
-        const half2_t sc = __builtin_bit_cast(half2_t, sw[i]), nz = __builtin_bit_cast(half2_t, nw[i]);
-        const half2_t cl = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(c64, word & 0x0F0F0F0Fu, sel)) - k1024;
-        const half2_t ch = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(c64, word & 0xF0F0F0F0u, sel)) * k16th - k64;
-        lo4[i] = __builtin_bit_cast(uint32_t, cl * sc + nz);
-        hi4[i] = __builtin_bit_cast(uint32_t, ch * sc + nz);
+        bl[i] = nl[i];
+        bh[i] = nh[i];
       }
-      const uint4 bl = make_uint4(lo4[0], lo4[1], lo4[2], lo4[3]), bh = make_uint4(hi4[0], hi4[1], hi4[2], hi4[3]);
+    }
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        Act<TX>::mma_acc(acc[rb][2 * jg], __builtin_bit_cast(uint4, a[rb]), bl);
-        Act<TX>::mma_acc(acc[rb][2 * jg + 1], __builtin_bit_cast(uint4, a[rb]), bh);
-      }
+    for (int i = 0; i < 4; ++i) {
+      carry_l[i] = bl[i];
+      carry_h[i] = bh[i];
     }
   };
 
   write_a(1, 0);
   load_a(1, 2);
   __syncthreads();                                                   // stage 0 and the tables are in LDS
-  read_a(0, 0, 0);
+  {
+    const uint4 s4 = *reinterpret_cast<const uint4 *>(tab_s + 8 * g), n4 = *reinterpret_cast<const uint4 *>(tab_nz + 8 * g);
+    const uint32_t sw[4] = {s4.x, s4.y, s4.z, s4.w}, nw[4] = {n4.x, n4.y, n4.z, n4.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t word = i < 2 ? wr[0][0][0].x : wr[0][0][0].y, sel = (i & 1) ? 0x04030402u : 0x04010400u;
+      carry_l[i] = build_lo(word, sel, sw[i], nw[i]);
+      carry_h[i] = build_hi(word, sel, sw[i], nw[i]);
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  read_a(0, 0, 0);                                                   // (LDS reads between the build and the first MFMA)
   __builtin_amdgcn_sched_barrier(0);
 
   auto stage = [&](auto curc, int s) __attribute__((always_inline)) {
     constexpr int cur = decltype(curc)::value;
     read_a(1, cur, 1);
     __builtin_amdgcn_sched_barrier(0);
-    compute(aq[0], wr[cur][0], 64 * s);
+    compute(aq[0], wr[cur][0], wr[cur][1][0], 64 * s, 64 * s + 32);
     __builtin_amdgcn_sched_barrier(0);
     load_w(cur, 0, s + 2);
     write_a(cur, cur ^ 1);
@@ -355,7 +397,7 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
     __syncthreads();
     read_a(0, cur ^ 1, 0);
     __builtin_amdgcn_sched_barrier(0);
-    compute(aq[1], wr[cur][1], 64 * s + 32);
+    compute(aq[1], wr[cur][1], wr[cur ^ 1][0][0], 64 * s + 32, 64 * s + 64);
     __builtin_amdgcn_sched_barrier(0);
     load_w(cur, 1, s + 2);
     __builtin_amdgcn_sched_barrier(0);
