@@ -332,7 +332,8 @@ def test_qmatmul_after_gptq_matches_dense(OP):
         assert np.mean(np.abs(ret - expected)) < 3e-2        # reference test_kernel.py:41
 
 
-@pytest.mark.parametrize("M,xdt", [(1, "float16"), (16, "bfloat16"), (200, "float16"), (3, "float32")])
+@pytest.mark.parametrize("M,xdt", [(1, "float16"), (16, "bfloat16"), (200, "float16"), (3, "float32"),
+                                   (2048, "float16")])      # (2048 rows: three launches, 128 x 512 tiles first)
 def test_qmatmul_in_a_captured_graph(OP, M, xdt):
     """A decode loop would capture the matmul in a HIP graph: the call only enqueues kernels (no
     memset, no allocation of its own, split-K counters left at zero by every launch), so a graph
