@@ -53,7 +53,9 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
 #pragma unroll
   for (int i = 0; i < CH; ++i) xoff[i] = min(m0 + (tid >> 3) + (NT / 8) * i, M - 1) * K + 8 * kc;      // M K < 2^31
   // piece i lands at [kc >> 2][(tid >> 7) + (NT / 128) i][16 (kc & 3) + ((tid >> 3) & 15)]
-  const int dst0 = ((kc >> 2) * RB + (tid >> 7)) * 64 + 16 * (kc & 3) + ((tid >> 3) & 15);
+  // (the lane index within a block is XORed with 4 g ^ 2 h: the eight lanes that write one row's 128 bytes would
+  //  otherwise hit the same banks; the reads, which XOR the same value, stay conflict free)
+  const int dst0 = ((kc >> 2) * RB + (tid >> 7)) * 64 + 16 * (kc & 3) + (((tid >> 3) & 15) ^ (4 * (kc & 3)) ^ (2 * (kc >> 2)));
   const uint8_t *wp = pk + (int64_t)(4 * g) * C + col;
 
   u32x4_t stg[2][CH];
@@ -75,10 +77,11 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
     for (int i = 0; i < 4; ++i) wr[p][h][i] = *reinterpret_cast<const uint2 *>(q + (int64_t)i * C);
   };
   auto read_a = [&](int q, int slot, int h) __attribute__((always_inline)) {
+    const int sl = lane ^ (4 * g) ^ (2 * h);
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) aq[q][rb] = a_lds[((slot * 2 + h) * RB + rb) * 64 + lane];
+    for (int rb = 0; rb < RB; ++rb) aq[q][rb] = a_lds[((slot * 2 + h) * RB + rb) * 64 + sl];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) aqr[q][j] = a_lds[((slot * 2 + h) * RB + 2 * wk + j) * 64 + lane];
+    for (int j = 0; j < 2; ++j) aqr[q][j] = a_lds[((slot * 2 + h) * RB + 2 * wk + j) * 64 + sl];
   };
 
   uint32_t zraw0[8];
@@ -257,7 +260,7 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   int xoff[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) xoff[i] = min(m0 + (tid >> 3) + 32 * i, M - 1) * C + 8 * kc;            // M C < 2^31
-  const int dst0 = ((kc >> 2) * RB + (tid >> 7)) * 64 + 16 * (kc & 3) + ((tid >> 3) & 15);
+  const int dst0 = ((kc >> 2) * RB + (tid >> 7)) * 64 + 16 * (kc & 3) + (((tid >> 3) & 15) ^ (4 * (kc & 3)) ^ (2 * (kc >> 2)));
   const uint8_t *wpj[NG];
 #pragma unroll
   for (int jg = 0; jg < NG; ++jg) wpj[jg] = pk + (int64_t)(j0 + 16 * jg + l16) * C + 8 * g;
@@ -280,8 +283,9 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
     for (int jg = 0; jg < NG; ++jg) wr[p][h][jg] = *reinterpret_cast<const uint2 *>(wpj[jg] + c);
   };
   auto read_a = [&](int q, int slot, int h) __attribute__((always_inline)) {
+    const int sl = lane ^ (4 * g) ^ (2 * h);                         // (bank swizzle, as in the forward kernel)
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) aq[q][rb] = a_lds[((slot * 2 + h) * RB + rb) * 64 + lane];
+    for (int rb = 0; rb < RB; ++rb) aq[q][rb] = a_lds[((slot * 2 + h) * RB + rb) * 64 + sl];
   };
 
   load_a(1, 0);
