@@ -31,11 +31,12 @@ int reg_fwd_launch(hipStream_t st, const RegPlan &p, const void *x, int x_dtype,
                    int group_size);
 
 // 128 x 512 tiles for many rows (qmatmul_wide.hip; 4-bit codes, per-channel parameters, aligned operands):
-// number of leading 512-channel tiles they take (0: none), and the launch over those tiles.  out32 / rowexp as
-// in RegPlan.
-int64_t wide_fwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned);
+// number of leading 512-channel tiles they take (0: none; *half: tiles of 256 channels, four wavefronts of 64 x 128,
+// for shapes whose 512-channel tiles are under one round), and the launch over those tiles.  out32 / rowexp as in
+// RegPlan.
+int64_t wide_fwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half);
 int wide_fwd_launch(hipStream_t st, const void *x, int x_dtype, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
-                    const void *zero, const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32,
+                    const void *zero, const void *scale, int zs_dtype, void *out, int64_t wide_x, bool half, float *out32,
                     const int32_t *rowexp);
 
 // The same for the transposed product (fp16 rows): leading tiles of 512 output columns = 256 packed rows.

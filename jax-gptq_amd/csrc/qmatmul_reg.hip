@@ -543,12 +543,13 @@ int launch_bx(hipStream_t st, const RegPlan &p, const void *x, int64_t M, const 
     int64_t first = 0;
     if constexpr (BITS == 4) {
       if (!p.ragged && p.S == 1) {
-        const int64_t wide_x = wide_fwd_tiles(M, R, C, true);
+        bool half = false;
+        const int64_t wide_x = wide_fwd_tiles(M, R, C, true, &half);
         if (wide_x > 0) {
           const int rc = wide_fwd_launch(st, x, Act<TX>::BF ? GPTQ_HIP_BF16 : GPTQ_HIP_F16, M, pk, R, C, zero, scale,
-                                         zs_dtype, out, wide_x, p.out32, p.rowexp);
+                                         zs_dtype, out, wide_x, half, p.out32, p.rowexp);
           if (rc) return rc;
-          first = 4 * wide_x;
+          first = (half ? 2 : 4) * wide_x;
         }
       }
     }

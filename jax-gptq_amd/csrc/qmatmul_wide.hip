@@ -26,7 +26,10 @@ namespace {
 
 using namespace qmm;
 
-template <int NWV, typename TX>
+// HALF: a 128 x 256 tile, the four wavefronts as two row halves x two column halves of 64 x 128 each (for shapes
+// whose 128 x 512 tiles are under one round of workgroups): the two wavefronts of a column half build the same
+// weight operands, the two of a row half share their row sums.
+template <int NWV, typename TX, bool HALF = false>
 __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, int M, int K, const uint8_t *pk, int C,
                                                                    const void *zero, const void *scale,
                                                                    int zs_dtype, TX *out, int c0, float *out32,
@@ -35,15 +38,17 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
   static_assert(NWV == 4, "the row sums are dealt to four wavefronts");
   constexpr int NT = 64 * NWV;
   constexpr int CH = 1024 / NT;                  // 16-byte pieces of a stage per thread
-  constexpr int RB = 8;
-  __shared__ u32x4_t a_lds[2 * 2 * RB * 64];       // [slot][k-step of the stage][row block][lane]
+  constexpr int RB = HALF ? 4 : 8;               // row blocks of a wavefront
+  constexpr int TB = 8;                          // row blocks of the workgroup's tile
+  __shared__ u32x4_t a_lds[2 * 2 * TB * 64];       // [slot][k-step of the stage][row block][lane]
   asm volatile("" ::"s"(x), "s"(pk), "s"(zero), "s"(scale), "s"(out), "s"(M), "s"(K), "s"(C), "s"(zs_dtype),
                "s"(c0), "s"(out32), "s"(rowexp));
   const int tid = threadIdx.x, lane = tid & 63, wk = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 4, l16 = lane & 15;
   int tx, ty;
   qmm_tile_coords(tx, ty);
-  const int m0 = ty * 128, nbase = c0 + (tx * NWV + wk) * 128;
+  const int rb0 = HALF ? 4 * (wk >> 1) : 0;      // first row block of this wavefront
+  const int m0 = ty * 128, nbase = c0 + (HALF ? tx * 2 + (wk & 1) : tx * NWV + wk) * 128;
   const int NS = K >> 6;
   const int col = nbase + 8 * l16;
 
@@ -55,7 +60,7 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
   // piece i lands at [kc >> 2][(tid >> 7) + (NT / 128) i][16 (kc & 3) + ((tid >> 3) & 15)]
   // (the lane index within a block is XORed with 4 g ^ 2 h: the eight lanes that write one row's 128 bytes would
   //  otherwise hit the same banks; the reads, which XOR the same value, stay conflict free)
-  const int dst0 = ((kc >> 2) * RB + (tid >> 7)) * 64 + 16 * (kc & 3) + (((tid >> 3) & 15) ^ (4 * (kc & 3)) ^ (2 * (kc >> 2)));
+  const int dst0 = ((kc >> 2) * TB + (tid >> 7)) * 64 + 16 * (kc & 3) + (((tid >> 3) & 15) ^ (4 * (kc & 3)) ^ (2 * (kc >> 2)));
   const uint8_t *wp = pk + (int64_t)(4 * g) * C + col;
 
   u32x4_t stg[2][CH];
@@ -69,7 +74,7 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
   };
   auto write_a = [&](int p, int slot) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < CH; ++i) a_lds[slot * (2 * RB * 64) + dst0 + (NT / 128) * 64 * i] = stg[p][i];
+    for (int i = 0; i < CH; ++i) a_lds[slot * (2 * TB * 64) + dst0 + (NT / 128) * 64 * i] = stg[p][i];
   };
   auto load_w = [&](int p, int h, int s) __attribute__((always_inline)) {
     const uint8_t *q = wp + (int64_t)(32 * min(s, NS - 1) + 16 * h) * C;
@@ -79,9 +84,9 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
   auto read_a = [&](int q, int slot, int h) __attribute__((always_inline)) {
     const int sl = lane ^ (4 * g) ^ (2 * h);
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) aq[q][rb] = a_lds[((slot * 2 + h) * RB + rb) * 64 + sl];
+    for (int rb = 0; rb < RB; ++rb) aq[q][rb] = a_lds[((slot * 2 + h) * TB + rb0 + rb) * 64 + sl];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) aqr[q][j] = a_lds[((slot * 2 + h) * RB + 2 * wk + j) * 64 + sl];
+    for (int j = 0; j < 2; ++j) aqr[q][j] = a_lds[((slot * 2 + h) * TB + 2 * wk + j) * 64 + sl];
   };
 
   uint32_t zraw0[8];
@@ -142,11 +147,28 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
     for (int t8 = 0; t8 < 8; ++t8) {
       const uint4 b = make_uint4(bc[0], bc[1], bc[2], bc[3]);
       uint32_t nx[4] = {0u, 0u, 0u, 0u};
+      auto dq_next = [&](int i) __attribute__((always_inline)) { nx[i] = t8 < 7 ? dq_reg(w, t8 + 1, i) : dq_reg(wn, 0, i); };
+      if constexpr (!HALF) {
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        if (rb & 1) Act<TX>::mma_acc_nw_after(acc[rb][t8], __builtin_bit_cast(uint4, a[rb]), b, nx[rb >> 1]);
-        else Act<TX>::mma_acc_nw(acc[rb][t8], __builtin_bit_cast(uint4, a[rb]), b);
-        if (!(rb & 1)) nx[rb >> 1] = t8 < 7 ? dq_reg(w, t8 + 1, rb >> 1) : dq_reg(wn, 0, rb >> 1);
+        for (int rb = 0; rb < RB; ++rb) {
+          if (rb & 1) Act<TX>::mma_acc_nw_after(acc[rb][t8], __builtin_bit_cast(uint4, a[rb]), b, nx[rb >> 1]);
+          else Act<TX>::mma_acc_nw(acc[rb][t8], __builtin_bit_cast(uint4, a[rb]), b);
+          if (!(rb & 1)) dq_next(rb >> 1);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+        // four MFMAs per tile: all four operand registers of the next tile are built before the last of them
+        Act<TX>::mma_acc_nw(acc[0][t8], __builtin_bit_cast(uint4, a[0]), b);
+        dq_next(0);
+        dq_next(1);
+        __builtin_amdgcn_sched_barrier(0);
+        Act<TX>::mma_acc_nw_after2(acc[1][t8], __builtin_bit_cast(uint4, a[1]), b, nx[0], nx[1]);
+        dq_next(2);
+        __builtin_amdgcn_sched_barrier(0);
+        Act<TX>::mma_acc_nw_after(acc[2][t8], __builtin_bit_cast(uint4, a[2]), b, nx[2]);
+        dq_next(3);
+        __builtin_amdgcn_sched_barrier(0);
+        Act<TX>::mma_acc_nw_after(acc[3][t8], __builtin_bit_cast(uint4, a[3]), b, nx[3]);
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
@@ -209,10 +231,10 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
   // m = m0 + 16 rb + 4 g + r
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    const floatx4 rs4 = rs_lds[rb * 64 + lane];
+    const floatx4 rs4 = rs_lds[(rb0 + rb) * 64 + lane];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int m = m0 + 16 * rb + 4 * g + r;
+      const int m = m0 + 16 * (rb0 + rb) + 4 * g + r;
       if (m >= M) continue;
       const float rs = rs4[r];
       TX o[8];
@@ -446,7 +468,8 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
 
 template <typename TX>
 int launch_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
-                const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32, const int32_t *rowexp) {
+                const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32, const int32_t *rowexp,
+                bool half) {
   const int64_t K = 2 * R;
   int64_t rows_max = ((1LL << 31) - 1) / K;
   if (rows_max > 65535LL * 128) rows_max = 65535LL * 128;
@@ -455,9 +478,14 @@ int launch_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int
   for (int64_t r0 = 0; r0 < M; r0 += rows_max) {
     const int64_t rows = M - r0 < rows_max ? M - r0 : rows_max;
     const dim3 grid((unsigned)wide_x, (unsigned)ceil_div64(rows, 128), 1);
-    hipLaunchKernelGGL((qmm_fwd_wide_kernel<4, TX>), grid, dim3(256), 0, st, (const TX *)x + r0 * K, (int)rows, (int)K,
-                       pk, (int)C, zero, scale, zs_dtype, (TX *)out + r0 * C, 0, out32 ? out32 + r0 * C : nullptr,
-                       rowexp ? rowexp + r0 : nullptr);
+    if (half)
+      hipLaunchKernelGGL((qmm_fwd_wide_kernel<4, TX, true>), grid, dim3(256), 0, st, (const TX *)x + r0 * K, (int)rows,
+                         (int)K, pk, (int)C, zero, scale, zs_dtype, (TX *)out + r0 * C, 0,
+                         out32 ? out32 + r0 * C : nullptr, rowexp ? rowexp + r0 : nullptr);
+    else
+      hipLaunchKernelGGL((qmm_fwd_wide_kernel<4, TX>), grid, dim3(256), 0, st, (const TX *)x + r0 * K, (int)rows,
+                         (int)K, pk, (int)C, zero, scale, zs_dtype, (TX *)out + r0 * C, 0,
+                         out32 ? out32 + r0 * C : nullptr, rowexp ? rowexp + r0 : nullptr);
     GPTQ_CHECK_LAUNCH();
   }
   return GPTQ_HIP_OK;
@@ -488,34 +516,40 @@ int launch_bwd_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk,
 
 namespace qmm {
 
-int64_t wide_fwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned) {
-  const int64_t K = 2 * R;
-  if (!aligned || K % 64 != 0 || K < 512 || C % 8 != 0 || M < 256) return 0;
-  const int64_t tiles_y = ceil_div64(M, 128), full_x = C / 512;
+// whole rounds of 256 workgroups (one per CU); a single round that is at least 7/8 full is taken as it is
+static int64_t wide_rounds(int64_t full_x, int64_t tiles_y) {
   const int64_t wgs = full_x * tiles_y;
-  // whole rounds of 256 workgroups (one per CU); a single round that is at least 7/8 full is taken as it is
   if (wgs >= 256) return (wgs / 256) * 256 / tiles_y;
   return wgs >= 224 ? full_x : 0;
 }
 
+int64_t wide_fwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half) {
+  const int64_t K = 2 * R;
+  *half = false;
+  if (!aligned || K % 64 != 0 || K < 512 || C % 8 != 0 || M < 256) return 0;
+  const int64_t tiles_y = ceil_div64(M, 128);
+  const int64_t n = wide_rounds(C / 512, tiles_y);
+  if (n > 0) return n;
+  // 128 x 256 tiles of four 64 x 128 wavefronts where the 512-channel tiles are under a round
+  *half = true;
+  return wide_rounds(C / 256, tiles_y);
+}
+
 int wide_fwd_launch(hipStream_t st, const void *x, int x_dtype, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
-                    const void *zero, const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32,
+                    const void *zero, const void *scale, int zs_dtype, void *out, int64_t wide_x, bool half, float *out32,
                     const int32_t *rowexp) {
   if (zs_dtype != GPTQ_HIP_F32 && zs_dtype != GPTQ_HIP_F16 && zs_dtype != GPTQ_HIP_BF16) return GPTQ_HIP_EDTYPE;
-  if (wide_x < 1 || wide_x * 512 > C) return GPTQ_HIP_EINVAL;
+  if (wide_x < 1 || wide_x * (half ? 256 : 512) > C) return GPTQ_HIP_EINVAL;
   if (x_dtype == GPTQ_HIP_BF16)
-    return launch_wide<__hip_bfloat16>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp);
+    return launch_wide<__hip_bfloat16>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half);
   if (x_dtype != GPTQ_HIP_F16) return GPTQ_HIP_EDTYPE;
-  return launch_wide<__half>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp);
+  return launch_wide<__half>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half);
 }
 
 int64_t wide_bwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned) {
   // (the constants of all channels and the stages share the LDS: 4 C + 32 KB)
   if (!aligned || C % 64 != 0 || C < 512 || C > 30720 || M < 256) return 0;
-  const int64_t tiles_y = ceil_div64(M, 128), full_x = R / 256;
-  const int64_t wgs = full_x * tiles_y;
-  if (wgs >= 256) return (wgs / 256) * 256 / tiles_y;
-  return wgs >= 224 ? full_x : 0;
+  return wide_rounds(R / 256, ceil_div64(M, 128));
 }
 
 int wide_bwd_launch(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,

@@ -50,6 +50,12 @@ template <> struct Act<__half> {
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0"
                  : "+a"(c) : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)), "v"(dep));
   }
+  static __device__ __forceinline__ void mma_acc_nw_after2(floatx4 &c, const uint4 &a, const uint4 &b, uint32_t dep0,
+                                                           uint32_t dep1) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0"
+                 : "+a"(c)
+                 : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)), "v"(dep0), "v"(dep1));
+  }
   static __device__ __forceinline__ __half out(float v) { return __float2half_rn(v); }
 };
 template <> struct Act<__hip_bfloat16> {
@@ -85,6 +91,12 @@ template <> struct Act<__hip_bfloat16> {
   static __device__ __forceinline__ void mma_acc_nw_after(floatx4 &c, const uint4 &a, const uint4 &b, uint32_t dep) {
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
                  : "+a"(c) : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)), "v"(dep));
+  }
+  static __device__ __forceinline__ void mma_acc_nw_after2(floatx4 &c, const uint4 &a, const uint4 &b, uint32_t dep0,
+                                                           uint32_t dep1) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                 : "+a"(c)
+                 : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)), "v"(dep0), "v"(dep1));
   }
   static __device__ __forceinline__ __hip_bfloat16 out(float v) { return __float2bfloat16(v); }
 };

@@ -170,13 +170,15 @@ def test_qmatmul_bf16_x_mfma_path(OP, M, N, K, zs):
 
 @pytest.mark.parametrize("xdt,zs", [("float16", "float32"), ("float16", "float16"), ("bfloat16", "float32"),
                                     ("bfloat16", "bfloat16"), ("float32", "float32")])
-@pytest.mark.parametrize("M,N,K", [(3500, 4480, 512), (2048, 11008, 1024), (4096, 4096, 576)])
+@pytest.mark.parametrize("M,N,K", [(3500, 4480, 512), (2048, 11008, 1024), (4096, 4096, 576), (2000, 4224, 1088)])
 def test_qmatmul_many_rows_128x512_tiles(OP, M, N, K, xdt, zs):
     """Forward products of many rows: the leading columns that fill whole rounds of workgroups run on
     128 x 512 tiles whose wavefronts share the activations through LDS, the rest on the 128- and 64-row
     tiles (4480 = 8 x 512 + 384 columns; 11008: 16 tiles + 22 x 128 columns; M = 3500 leaves a ragged
-    last row tile; K = 576 has an odd number of 64-k stages).  Fractional zero points exercise the row
-    sums that the wavefronts exchange; fp32 rows the scaled fp32 store."""
+    last row tile; K = 576 has an odd number of 64-k stages; 2000 x 4224: the 512-channel tiles are
+    under one round of workgroups, so 128 x 256 tiles of four 64 x 128 wavefronts take 16 x 256 columns).
+    Fractional zero points exercise the row sums that the wavefronts exchange; fp32 rows the scaled
+    fp32 store."""
     import torch
     import jax_gptq_amd.gptq as G
     rng = np.random.default_rng(M + N + K)
