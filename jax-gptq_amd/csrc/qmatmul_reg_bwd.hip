@@ -398,11 +398,12 @@ int launch_bx(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, con
     if constexpr (BITS == 4 && !Act<TX>::BF) {
       // (also where this kernel's own tiles need a split because the constants of all channels do not fit its LDS)
       if (!p.ragged && group_size == 0) {
-        const int64_t wide_x = wide_bwd_tiles(M, R, C, true);
+        bool half = false;
+        const int64_t wide_x = wide_bwd_tiles(M, R, C, true, &half);
         if (wide_x > 0) {
-          const int rc = wide_bwd_launch(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, p.out32, p.rowexp);
+          const int rc = wide_bwd_launch(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, half, p.out32, p.rowexp);
           if (rc) return rc;
-          first = 4 * wide_x;
+          first = (half ? 2 : 4) * wide_x;
         }
       }
     }

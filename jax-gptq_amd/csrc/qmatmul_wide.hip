@@ -261,12 +261,13 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
 // channels, in stages of 64, whose activations the four wavefronts share through LDS as above; the weight operand
 // is built as in qmatmul_reg_bwd.hip (lane (l16, g): 8 channels of packed row j0 + 16 jg + l16; scale and
 // -zero * scale of all channels converted once into LDS).  C % 64 == 0, whole 512-column tiles only.
-template <typename TX>
+template <typename TX, bool HALF = false>
 __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M, const uint8_t *pk, int R, int C,
                                                                const void *zero, const void *scale, int zs_dtype,
                                                                TX *out, float *out32, const int32_t *rowexp) {
   static_assert(!Act<TX>::BF, "fp16 rows");
-  constexpr int RB = 8, NG = 4;
+  // (HALF: 128 rows x 256 output columns, the four wavefronts as two row halves x two column halves, as forward)
+  constexpr int RB = HALF ? 4 : 8, TB = 8, NG = 4;
   extern __shared__ __attribute__((aligned(16))) float wide_lds[];     // halves sc[C], halves nzs[C], then the stages
   _Float16 *tab_s = reinterpret_cast<_Float16 *>(wide_lds);
   _Float16 *tab_nz = tab_s + C;
@@ -275,14 +276,15 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   const int g = lane >> 4, l16 = lane & 15;
   int tx, ty;
   qmm_tile_coords(tx, ty);
-  const int m0 = ty * 128, j0 = (tx * 4 + wk) * 64;
+  const int rb0 = HALF ? 4 * (wk >> 1) : 0;
+  const int m0 = ty * 128, j0 = (HALF ? tx * 2 + (wk & 1) : tx * 4 + wk) * 64;
   const int NS = C >> 6;
 
   const int kc = tid & 7;
   int xoff[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) xoff[i] = min(m0 + (tid >> 3) + 32 * i, M - 1) * C + 8 * kc;            // M C < 2^31
-  const int dst0 = ((kc >> 2) * RB + (tid >> 7)) * 64 + 16 * (kc & 3) + (((tid >> 3) & 15) ^ (4 * (kc & 3)) ^ (2 * (kc >> 2)));
+  const int dst0 = ((kc >> 2) * TB + (tid >> 7)) * 64 + 16 * (kc & 3) + (((tid >> 3) & 15) ^ (4 * (kc & 3)) ^ (2 * (kc >> 2)));
   const uint8_t *wpj[NG];
 #pragma unroll
   for (int jg = 0; jg < NG; ++jg) wpj[jg] = pk + (int64_t)(j0 + 16 * jg + l16) * C + 8 * g;
@@ -297,7 +299,7 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   };
   auto write_a = [&](int p, int slot) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) a_lds[slot * (2 * RB * 64) + dst0 + 2 * 64 * i] = stg[p][i];
+    for (int i = 0; i < 4; ++i) a_lds[slot * (2 * TB * 64) + dst0 + 2 * 64 * i] = stg[p][i];
   };
   auto load_w = [&](int p, int h, int s) __attribute__((always_inline)) {
     const int c = 64 * min(s, NS - 1) + 32 * h;
@@ -307,7 +309,7 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   auto read_a = [&](int q, int slot, int h) __attribute__((always_inline)) {
     const int sl = lane ^ (4 * g) ^ (2 * h);                         // (bank swizzle, as in the forward kernel)
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) aq[q][rb] = a_lds[((slot * 2 + h) * RB + rb) * 64 + sl];
+    for (int rb = 0; rb < RB; ++rb) aq[q][rb] = a_lds[((slot * 2 + h) * TB + rb0 + rb) * 64 + sl];
   };
 
   load_a(1, 0);
@@ -364,20 +366,52 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
       const uint4 Bl = make_uint4(bl[0], bl[1], bl[2], bl[3]), Bh = make_uint4(bh[0], bh[1], bh[2], bh[3]);
       const uint2 wsrc = jg + 1 < NG ? w[jg + 1 < NG ? jg + 1 : 0] : wnext;
       uint32_t nl[4] = {0u, 0u, 0u, 0u}, nh[4] = {0u, 0u, 0u, 0u};
+      auto piece = [&](int pc) __attribute__((always_inline)) {      // piece pc = 2 i + (0: low, 1: high nibbles)
+        const int i = pc >> 1;
+        const uint32_t word = i < 2 ? wsrc.x : wsrc.y;
+        const uint32_t sel = (i & 1) ? 0x04030402u : 0x04010400u;            // bytes (2e, 2e+1) under 0x64
+        const uint32_t scw = jg + 1 < NG ? sw[i] : swn[i], nzw = jg + 1 < NG ? nw[i] : nwn[i];
+        if (pc & 1) nh[i] = build_hi(word, sel, scw, nzw);
+        else nl[i] = build_lo(word, sel, scw, nzw);
+      };
+      if constexpr (!HALF) {
 #pragma unroll
-      for (int n = 0; n < 16; ++n) {
-        const int rb = n >> 1, i = n >> 2;
-        const bool hi_piece = (n >> 1) & 1;
-        if (!(n & 1)) {
-          Act<TX>::mma_acc_nw(acc[rb][2 * jg], __builtin_bit_cast(uint4, a[rb]), Bl);
-          const uint32_t word = i < 2 ? wsrc.x : wsrc.y;
-          const uint32_t sel = (i & 1) ? 0x04030402u : 0x04010400u;          // bytes (2e, 2e+1) under 0x64
-          const uint32_t scw = jg + 1 < NG ? sw[i] : swn[i], nzw = jg + 1 < NG ? nw[i] : nwn[i];
-          if (hi_piece) nh[i] = build_hi(word, sel, scw, nzw);
-          else nl[i] = build_lo(word, sel, scw, nzw);
-        } else {
-          Act<TX>::mma_acc_nw_after(acc[rb][2 * jg + 1], __builtin_bit_cast(uint4, a[rb]), Bh, hi_piece ? nh[i] : nl[i]);
+        for (int n = 0; n < 16; ++n) {
+          const int rb = n >> 1, i = n >> 2;
+          const bool hi_piece = (n >> 1) & 1;
+          if (!(n & 1)) {
+            Act<TX>::mma_acc_nw(acc[rb][2 * jg], __builtin_bit_cast(uint4, a[rb]), Bl);
+            piece(n >> 1);
+          } else {
+            Act<TX>::mma_acc_nw_after(acc[rb][2 * jg + 1], __builtin_bit_cast(uint4, a[rb]), Bh, hi_piece ? nh[i] : nl[i]);
+          }
+          __builtin_amdgcn_sched_barrier(0);
         }
+      } else {
+        // eight MFMAs per group: two pieces behind the first, one behind each of the next six, none behind the last
+        Act<TX>::mma_acc_nw(acc[0][2 * jg], __builtin_bit_cast(uint4, a[0]), Bl);
+        piece(0);
+        piece(1);
+        __builtin_amdgcn_sched_barrier(0);
+        Act<TX>::mma_acc_nw_after2(acc[0][2 * jg + 1], __builtin_bit_cast(uint4, a[0]), Bh, nl[0], nh[0]);
+        piece(2);
+        __builtin_amdgcn_sched_barrier(0);
+        Act<TX>::mma_acc_nw_after(acc[1][2 * jg], __builtin_bit_cast(uint4, a[1]), Bl, nl[1]);
+        piece(3);
+        __builtin_amdgcn_sched_barrier(0);
+        Act<TX>::mma_acc_nw_after(acc[1][2 * jg + 1], __builtin_bit_cast(uint4, a[1]), Bh, nh[1]);
+        piece(4);
+        __builtin_amdgcn_sched_barrier(0);
+        Act<TX>::mma_acc_nw_after(acc[2][2 * jg], __builtin_bit_cast(uint4, a[2]), Bl, nl[2]);
+        piece(5);
+        __builtin_amdgcn_sched_barrier(0);
+        Act<TX>::mma_acc_nw_after(acc[2][2 * jg + 1], __builtin_bit_cast(uint4, a[2]), Bh, nh[2]);
+        piece(6);
+        __builtin_amdgcn_sched_barrier(0);
+        Act<TX>::mma_acc_nw_after(acc[3][2 * jg], __builtin_bit_cast(uint4, a[3]), Bl, nl[3]);
+        piece(7);
+        __builtin_amdgcn_sched_barrier(0);
+        Act<TX>::mma_acc_nw_after(acc[3][2 * jg + 1], __builtin_bit_cast(uint4, a[3]), Bh, nh[3]);
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
@@ -442,7 +476,7 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int m = m0 + 16 * rb + 4 * g + r;
+      const int m = m0 + 16 * (rb0 + rb) + 4 * g + r;
       if (m >= M) continue;
       if (out32 != nullptr) {
         const int e = rowexp[m];
@@ -492,8 +526,9 @@ int launch_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int
 }
 
 int launch_bwd_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
-                    const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32, const int32_t *rowexp) {
-  auto kern = qmm_bwd_wide_kernel<__half>;
+                    const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32, const int32_t *rowexp,
+                    bool half) {
+  auto kern = half ? qmm_bwd_wide_kernel<__half, true> : qmm_bwd_wide_kernel<__half, false>;
   const int lds = (int)(4 * C + 2 * 2 * 8 * 64 * 16);
   if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), lds)) return GPTQ_HIP_ELAUNCH;
   const int64_t KO = 2 * R;
@@ -546,17 +581,23 @@ int wide_fwd_launch(hipStream_t st, const void *x, int x_dtype, int64_t M, const
   return launch_wide<__half>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half);
 }
 
-int64_t wide_bwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned) {
+int64_t wide_bwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half) {
+  *half = false;
   // (the constants of all channels and the stages share the LDS: 4 C + 32 KB)
   if (!aligned || C % 64 != 0 || C < 512 || C > 30720 || M < 256) return 0;
-  return wide_rounds(R / 256, ceil_div64(M, 128));
+  const int64_t tiles_y = ceil_div64(M, 128);
+  const int64_t n = wide_rounds(R / 256, tiles_y);
+  if (n > 0) return n;
+  *half = true;
+  return wide_rounds(R / 128, tiles_y);
 }
 
 int wide_bwd_launch(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
-                    const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32, const int32_t *rowexp) {
+                    const void *scale, int zs_dtype, void *out, int64_t wide_x, bool half, float *out32,
+                    const int32_t *rowexp) {
   if (zs_dtype != GPTQ_HIP_F32 && zs_dtype != GPTQ_HIP_F16 && zs_dtype != GPTQ_HIP_BF16) return GPTQ_HIP_EDTYPE;
-  if (wide_x < 1 || wide_x * 256 > R) return GPTQ_HIP_EINVAL;
-  return launch_bwd_wide(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp);
+  if (wide_x < 1 || wide_x * (half ? 128 : 256) > R) return GPTQ_HIP_EINVAL;
+  return launch_bwd_wide(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half);
 }
 
 }  // namespace qmm

@@ -200,7 +200,8 @@ def test_qmatmul_many_rows_128x512_tiles(OP, M, N, K, xdt, zs):
 
 
 @pytest.mark.parametrize("xdt,zs", [("float16", "float32"), ("float16", "float16"), ("float32", "bfloat16")])
-@pytest.mark.parametrize("M,N,K", [(3500, 512, 4480), (2048, 1024, 11008), (4096, 576, 4096), (1800, 20480, 8192)])
+@pytest.mark.parametrize("M,N,K", [(3500, 512, 4480), (2048, 1024, 11008), (4096, 576, 4096), (1800, 20480, 8192),
+                                   (2000, 1088, 4224)])      # (4224 output columns: 128 x 256 tiles, as forward)
 def test_qmatmul_many_rows_128x512_tiles_transposed(OP, M, N, K, xdt, zs):
     """The transposed product of many fp16 (or fp32) rows on the same tiling: 512 output columns per
     workgroup, contraction along the channels in stages of 64 (N = 576: an odd number of stages;
