@@ -67,6 +67,7 @@ def build(force=False, verbose=True):
 
 
 JAX_SHIM = os.path.join(OUT_DIR, "libgptq_hip_jax.so")
+JAX_SHIM_ERROR = None       # compiler log of a failed shim build
 
 
 def jax_ffi_include_dir():
@@ -93,7 +94,17 @@ def build_jax_ffi(verbose=True):
     cmd = [_hipcc(), "-O2", "-fPIC", "-std=c++17", "-shared", "-x", "hip", "--offload-arch=gfx950",
            "-I", inc, os.path.join(CSRC, "jax_ffi.cc"), "-o", JAX_SHIM,
            "-L", OUT_DIR, "-l:libgptq_hip.so", "-Wl,-rpath,$ORIGIN"]
-    subprocess.check_call(cmd)
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+    if p.returncode != 0:
+        # the shim is optional and has never been compiled against a real jaxlib: a failure here must
+        # not take the mandatory library down with it
+        global JAX_SHIM_ERROR
+        JAX_SHIM_ERROR = p.stdout.decode(errors="replace")
+        sys.stderr.write("[build] the XLA FFI shim did not compile (the ctypes library is unaffected):\n"
+                         + JAX_SHIM_ERROR + "\n")
+        if os.path.exists(JAX_SHIM):
+            os.remove(JAX_SHIM)
+        return None
     if verbose:
         print(f"[build] wrote {JAX_SHIM}")
     return JAX_SHIM

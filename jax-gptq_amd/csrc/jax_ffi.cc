@@ -17,6 +17,7 @@
 // for every XLA_FFI_DEFINE_HANDLER_SYMBOL below (jax_gptq_amd/jax_frontend.py does this).
 #include <cstdint>
 #include <optional>
+#include <string>
 #include <vector>
 
 #include <hip/hip_runtime.h>

@@ -502,10 +502,17 @@ def gptq(W, xs, block_size=128, actorder=False, damping=0.01, use_fp64=False, H=
     keep = H is not None or shared is not None      # somebody else still needs H as accumulated
     if H is None:
         H = accumulate_H(xs, use_fp64=use_fp64, split_fp16=split_fp16 and not use_fp64)
+    if not isinstance(H, torch.Tensor):
+        H = _dev(H)
     if H.dim() != 2 or H.shape[0] != H.shape[1] or H.dtype != (torch.float64 if use_fp64 else torch.float32):
         raise ValueError("H must be the square matrix accumulate_H(xs, use_fp64) returns")
     if H.shape[0] != K:
         raise ValueError(f"calibration feature dim {H.shape[0]} != K={K}")
+    # a caller's H may be a strided view (a corner of a larger matrix) or live elsewhere: the kernels
+    # take a dense [K, K] matrix on the current device
+    H = _dev(H)
+    if H.data_ptr() % 16:
+        H = H.clone()           # a dense view that starts mid-allocation: the kernels load 16 bytes at a time
     if shared is not None:
         shared["H"] = H
 

@@ -126,6 +126,15 @@ def test_products_on_the_same_activations_share_one_hessian(T, J, monkeypatch):
     assert T.equal(H, H0) and T.equal(Q1, Q2)
     with pytest.raises(ValueError):
         G.gptq(originals["q"].clone(), xs, block_size=64, H=H[:, :-1])
+    # a Hessian handed over as a strided view (the corner of a larger matrix), and one that starts
+    # in the middle of an allocation, are the same matrix to gptq
+    big = T.zeros((300, 300), dtype=H.dtype, device=H.device)
+    big[:256, :256] = H
+    Q3, _ = G.gptq(originals["q"].clone(), xs, block_size=64, H=big[:256, :256])
+    flat = T.zeros(256 * 256 + 1, dtype=H.dtype, device=H.device)
+    flat[1:] = H.reshape(-1)
+    Q4, _ = G.gptq(originals["q"].clone(), xs, block_size=64, H=flat[1:].view(256, 256))
+    assert T.equal(Q3, Q1) and T.equal(Q4, Q1)
 
 
 def test_transform(T, J):
