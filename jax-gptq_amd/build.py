@@ -13,7 +13,7 @@ CSRC = os.path.join(HERE, "csrc")
 OUT_DIR = os.path.join(HERE, "jax_gptq_amd")
 LIB = os.path.join(OUT_DIR, "libgptq_hip.so")
 SOURCES = ["api.hip", "codec.hip", "gemm_f32.hip", "gemm_f64.hip", "hessian.hip", "cholinv.hip", "solve.hip",
-           "qmatmul.hip", "qmatmul_reg.hip", "qmatmul_reg_bwd.hip", "qmatmul_wide.hip"]
+           "qmatmul.hip", "qmatmul_mid.hip", "qmatmul_reg.hip", "qmatmul_reg_bwd.hip", "qmatmul_wide.hip"]
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-result"]

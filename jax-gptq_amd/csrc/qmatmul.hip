@@ -2072,6 +2072,8 @@ size_t ws16_bytes(int64_t M, int64_t R, int64_t C, int transpose_b, int bits) {
   for (size_t c : cand) need = c > need ? c : need;
   const DecPlan dp = dec_plan(M, R, C);
   if (dp.use && dp.total_bytes > need) need = dp.total_bytes;
+  const MidPlan mp = mid_fwd_plan(M, R, C, true);
+  if (mp.use && mp.total_bytes > need) need = mp.total_bytes;
   const DecPlan dr = dec_plan(M, R, C, 4, true);
   if (dr.use && dr.total_bytes > need) need = dr.total_bytes;
   return need;
@@ -2226,6 +2228,19 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
         default:
           return launch_dec_z_rag<__hip_bfloat16>(st, dp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
       }
+    }
+  }
+  if (bits == 4 && !transpose_b && group_size == 0 && x_dtype == GPTQ_HIP_F16) {
+    // 17 .. 256 fp16 rows: tall, narrow tiles whose eight wavefronts split the contraction (qmatmul_mid.hip)
+    MidPlan mp = mid_fwd_plan(M, R, C, al && (reinterpret_cast<uintptr_t>(packed) & 15) == 0);
+    if (mp.use) {
+      if (mp.total_bytes && (!ws || ws_bytes < mp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+      if (out32 && rowexp && wrote32) {
+        mp.out32 = out32;
+        mp.rowexp = rowexp;
+        *wrote32 = true;
+      }
+      return mid_fwd_launch(st, mp, x, M, packed, R, C, zero, scale, zs_dtype, out, ws);
     }
   }
   if (bits == 4 && !transpose_b && group_size == 0) {

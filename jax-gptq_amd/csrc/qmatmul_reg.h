@@ -30,6 +30,22 @@ int reg_fwd_launch(hipStream_t st, const RegPlan &p, const void *x, int x_dtype,
                    int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws,
                    int group_size);
 
+// Tall, narrow tiles for a few dozen rows (qmatmul_mid.hip; 4-bit codes, per-channel parameters, 16-byte aligned
+// operands, fp16 activations, K % 256 == 0, C % 16 == 0; `use` is false where the other tiles are faster): a workgroup
+// of eight wavefronts owns 16 rb rows x 16 nb channels over one of S ranges of `steps` k-steps.  out32 / rowexp as in
+// RegPlan.
+struct MidPlan {
+  bool use;
+  int rb, nb, S, steps;
+  int64_t tiles_x, tiles_y;
+  float *out32;
+  const int32_t *rowexp;
+  size_t part_bytes, total_bytes;
+};
+MidPlan mid_fwd_plan(int64_t M, int64_t R, int64_t C, bool aligned);
+int mid_fwd_launch(hipStream_t st, const MidPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
+                   const void *zero, const void *scale, int zs_dtype, void *out, void *ws);
+
 // 128 x 512 tiles for many rows (qmatmul_wide.hip; 4-bit codes, per-channel parameters, aligned operands):
 // number of leading 512-channel tiles they take (0: none; *half: tiles of 256 channels, four wavefronts of 64 x 128,
 // for shapes whose 512-channel tiles are under one round), and the launch over those tiles.  out32 / rowexp as in

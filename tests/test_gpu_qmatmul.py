@@ -199,6 +199,42 @@ def test_qmatmul_many_rows_128x512_tiles(OP, M, N, K, xdt, zs):
     assert np.all(err <= tol), float((err / tol).max())
 
 
+@pytest.mark.parametrize("xdt,zs", [("float16", "float32"), ("float16", "float16"), ("float16", "bfloat16"),
+                                    ("float32", "float32")])
+@pytest.mark.parametrize("M,N,K", [(17, 11008, 4096), (32, 11008, 4096), (33, 4096, 11008), (64, 11008, 4096),
+                                   (50, 80, 2304), (128, 4096, 4096), (100, 1104, 1024), (256, 3072, 768),
+                                   (40, 64, 256)])
+def test_qmatmul_few_dozen_rows_tall_narrow_tiles(OP, M, N, K, xdt, zs):
+    """17 to a few dozen fp16 rows (up to 128 / 256 on small matrices), K a multiple of 256, C of 16: 32- or 64-row
+    tiles of 64 channels whose eight wavefronts split the contraction and share the activations through LDS
+    (4096 x 11008: 172 workgroups over all of K; 11008 x 4096 and 4096 x 4096: 64 column tiles x 4 splits, partial
+    tiles through the workspace; 80 and 1104 channels: a last tile of 16 channels; M = 33, 50, 100: ragged row
+    tiles; 2304 = 9 stages and 256 = 1 stage: the loop's remainder).  The weight operands are formed as
+    (code - zero) 2^-9 in fp16, so a fractional zero point costs fp16's relative precision and no more; fp32 rows
+    of very different magnitudes go through the scaled fp16 staging and the tiles' own fp32 store."""
+    import torch
+    import jax_gptq_amd.gptq as G
+    rng = np.random.default_rng(M + N + K)
+    codes = rng.integers(0, 16, (K, N)).astype(np.uint8)
+    tdt = getattr(torch, zs)
+    scale = torch.from_numpy(rng.uniform(0.001, 0.01, N).astype(np.float32)).to(tdt)
+    zero = torch.from_numpy(rng.uniform(0.0, 15.0, N).astype(np.float32)).to(tdt)      # fractional, too
+    qm = G.QuantizedMatrix(torch.from_numpy(O.pack_colwise(codes)).cuda(), zero.cuda(), scale.cuda())
+    rowscale = np.array([1.0, 1e-3, 3e4])[np.arange(M) % 3][:, None] if xdt == "float32" else np.ones((M, 1))
+    x = torch.from_numpy((rng.standard_normal((M, K)) * rowscale).astype(np.float32)).to(getattr(torch, xdt))
+    dense = (codes.astype(np.float64) - zero.double().numpy()[None]) * scale.double().numpy()[None]
+    ref = x.double().numpy() @ dense
+    tol = (ATOL + RTOL * np.abs(ref / rowscale)) * rowscale
+    first = None
+    for rep in range(3):            # the split sums leave their counters as they found them
+        got = OP.quantized_matmul(x, qm)
+        assert got.dtype == getattr(torch, xdt) and tuple(got.shape) == (M, N)
+        err = np.abs(to_np(got).astype(np.float64) - ref)
+        assert np.all(err <= tol), float((err / tol).max())
+        first = got.clone() if first is None else first
+        assert torch.equal(got, first)          # and are summed in split order: the same bits every time
+
+
 @pytest.mark.parametrize("xdt,zs", [("float16", "float32"), ("float16", "float16"), ("float32", "bfloat16")])
 @pytest.mark.parametrize("M,N,K", [(3500, 512, 4480), (2048, 1024, 11008), (4096, 576, 4096), (1800, 20480, 8192),
                                    (2000, 1088, 4224)])      # (4224 output columns: 128 x 256 tiles, as forward)
