@@ -23,7 +23,9 @@ SHAPES = [
     (28672, 7168, 128),  # 30 GB of calibration rows resident
 ]
 # the large-layer configuration also names 8-bit codes (one per byte; not in the reference)
-SHAPES = [s + (4,) for s in SHAPES] + [(7168, 28672, 128, 8), (28672, 7168, 16, 8)]
+SHAPES = [s + (4,) for s in SHAPES] + [(7168, 28672, 128, 8), (28672, 7168, 16, 8), (28672, 7168, 128, 8)]
+# the attention projections of the Llama-7B-shaped block (q / k / v / o) as a layer of their own at the full set
+SHAPES.append((4096, 4096, 128, 4))
 
 
 @pytest.mark.parametrize("K,N,nb,bits", SHAPES)
