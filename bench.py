@@ -193,6 +193,8 @@ def bench_qmatmul(reps=240):
         # forward at the decode / small-batch sizes, and the transposed (VJP) product at 2048 rows
         cases = [(1, 0, "float16"), (16, 0, "float16"), (128, 0, "float16"), (2048, 0, "float16"),
                  (2048, 1, "float16")]
+        if bits == 4 and K * N == K_IN * N_OUT:
+            cases[2:2] = [(32, 0, "float16"), (64, 0, "float16")]
         if K == K_IN and bits == 4:
             cases += [(1, 0, "bfloat16"), (16, 0, "bfloat16"), (2048, 1, "bfloat16")]
             # fp32 rows in and out (what a JAX caller of the reference passes by default): rounded to fp16
@@ -235,7 +237,10 @@ def bench_qmatmul(reps=240):
             torch.cuda.synchronize()
             us_cached = e0.elapsed_time(e1) * 1e3 / reps
             nbytes = R * N + 2 * N * 2 + M * K * esz + M * N * esz
+            plan = _native.qmatmul_plan(M, R, N, transpose_b=tr, x_dtype=xcode, zs_dtype=_native.F16, bits=bits)
             out.append({"M": M, "K": K, "N": N, "bits": bits, "transpose_b": tr, "x_dtype": xdt, "us": round(us, 2),
+                        "kernel": plan["kernel"] + (" + " + plan["rest"] if plan["rest"] else ""),
+                        "splits": plan["splits"],
                         "us_cache_resident": round(us_cached, 2),
                         "algorithmic_bytes": nbytes,
                         "GBps": round(nbytes / us * 1e-3, 1),

@@ -223,6 +223,42 @@ int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const 
                      int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype,
                      int transpose_b, void *out, void *ws, size_t ws_bytes);
 
+/* ---- which kernel a product runs on (host only: nothing is launched, no device is touched) ----------
+ * No counterpart in the reference, whose Triton kernel picks its tiles by autotuning at run time
+ * (kernel.py:4-16).  gptq_hip_qmatmul_plan_query fills *plan with what gptq_hip_qmatmul /
+ * gptq_hip_qmatmul_bits / gptq_hip_qmatmul_grouped would run for these arguments when they are given the
+ * workspace their size query names: `kernel` takes the product or its leading columns, `kernel_rest` (0 if none) the
+ * remaining columns, `splits` workgroups share one output tile's contraction, `workgroups` is the first kernel's
+ * grid (0 where it is not planned ahead), `fp32_rows` says how fp32 activations travel (0: as they are, 1: scaled
+ * and rounded to fp16 rows in the workspace by a kernel of their own, 2: inside the product's kernel).  `aligned`:
+ * all operands 16-byte aligned (1) or only to their element size (0).  For tests that keep every kernel family
+ * reachable, benchmarks that name the kernel they time, and callers that want to know. */
+enum {
+  GPTQ_HIP_QMM_SIMPLE = 1,        /* one thread per output */
+  GPTQ_HIP_QMM_DECODE = 2,        /* up to 16 rows: 256-channel strips, all loads in flight at once */
+  GPTQ_HIP_QMM_DECODE_RAGGED = 3, /* the same for rows of any length */
+  GPTQ_HIP_QMM_CHUNKED = 4,       /* up to 16 rows per chunk, activations only 4-byte aligned */
+  GPTQ_HIP_QMM_MID = 6,           /* 17 to a few dozen rows: tall, narrow tiles */
+  GPTQ_HIP_QMM_REG16 = 7,         /* register-operand tiles of 16, 64, 128 rows x 128 channels */
+  GPTQ_HIP_QMM_REG64 = 8,
+  GPTQ_HIP_QMM_REG128 = 9,
+  GPTQ_HIP_QMM_WIDE = 10,         /* 128 x 512 tiles, activations shared through LDS */
+  GPTQ_HIP_QMM_WIDE_HALF = 11,    /* 128 x 256 */
+  GPTQ_HIP_QMM_BWD_SIMPLE = 21,   /* transposed product */
+  GPTQ_HIP_QMM_BWD_REG64 = 22,
+  GPTQ_HIP_QMM_BWD_REG128 = 23,
+  GPTQ_HIP_QMM_BWD_WIDE = 24,
+  GPTQ_HIP_QMM_BWD_WIDE_HALF = 25,
+  GPTQ_HIP_QMM_BWD_GEMM = 26      /* weights dequantised into LDS */
+};
+typedef struct gptq_hip_qmatmul_plan {
+  int kernel, kernel_rest, splits, fp32_rows;
+  int64_t workgroups;
+} gptq_hip_qmatmul_plan;
+int gptq_hip_qmatmul_plan_query(int64_t M, int64_t R, int64_t C, int transpose_b, int x_dtype, int zs_dtype, int bits,
+                                int64_t group_size, int aligned, gptq_hip_qmatmul_plan *plan);
+const char *gptq_hip_qmatmul_kernel_name(int kernel);
+
 /* ---- the same product for 8-bit codes -----------------------------------------------------------
  * No counterpart in the reference, whose packing and kernels are fixed at 4 bits (gptq.py:241,253,
  * kernel.py:92-104); for the 8-bit codes gptq() can produce here (bits = 8).  bits = 4: exactly

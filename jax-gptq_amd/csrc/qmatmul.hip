@@ -393,131 +393,6 @@ __global__ __launch_bounds__(SPW == 2 ? 1024 : 512) void qmm_fwd_mfma_kernel(
                                            zero, scale, out, ws, se, so);
 }
 
-// ---------------------------------------------------------------------------- MFMA path, streaming
-// The same arithmetic for matrices that are several times larger than what the chip holds in
-// flight.  Above, a workgroup issues all its loads, waits, computes and reduces; its lifetime is
-// a chain of latencies, and with more workgroups than slots the chip runs them in rounds of
-// that lifetime (2.7 TB/s on a 103 MB matrix).  Here a workgroup (4 wavefronts) owns a strip and
-// a long row range and walks it in k-steps of 16 packed rows per wavefront, QS_RING k-steps of
-// loads in flight per wavefront in a register ring: a finished k-step is refilled at once with
-// the loads of k-step t + QS_RING.  The accumulators of all 16 tiles stay in registers, the
-// reduction across wavefronts and splits runs once at the end.  Steps past the end of the
-// range load clamped (valid) addresses and enter with zero activations.
-constexpr int QS_RING = 4;
-constexpr int QS_NW = 4;
-
-template <typename TZ, typename TX>
-__global__ __launch_bounds__(256, 2) void qmm_fwd_stream_kernel(
-    const TX *x, int M, int K, const uint8_t *pk, int R, int C, const TZ *zero,
-    const TZ *scale, TX *out, QmmWs ws, int S, int rows_per_split) {
-  constexpr bool BF = Act<TX>::BF;
-  extern __shared__ float red[];
-  __shared__ int s_last;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int strip = blockIdx.x, split = blockIdx.y, m0 = blockIdx.z * 16;
-  const int mvalid = min(16, M - m0);
-  const int mrows = mvalid <= 4 ? 4 : 16;
-  const int g = lane >> 4, l16 = lane & 15;
-  const int r_begin = split * rows_per_split, r_end = min(R, r_begin + rows_per_split);
-  // k-step t of this wavefront: packed rows r_begin + (t * QS_NW + wave) * 16 + [0, 16)
-  const int groups = (r_end - r_begin + 15) >> 4;                       // 16-row groups of the range
-  const int nsteps = groups > wave ? (groups - wave + QS_NW - 1) / QS_NW : 0;
-
-  const bool m_ok = l16 < mvalid;
-  const TX *xr = x + (int64_t)(m0 + (m_ok ? l16 : 0)) * K;
-  const int col0 = min(strip * QSTRIP + 16 * l16, C - 16);             // C % 16 == 0, C >= 16
-  const uint8_t *wp = pk + col0;
-
-  // Lane group g owns the packed rows 4g .. 4g+3 of a k-step, i.e. 8 consecutive k: its
-  // activations are one 16-byte load (R % 4 == 0 and x 16-byte aligned are preconditions; range
-  // boundaries are multiples of 4 rows, so a group of 4 rows is inside the range or outside).
-  struct Step { uint4 d[4]; uint4 pr; };
-  auto issue = [&](Step &st, int t) __attribute__((always_inline)) {
-    const int rbase = r_begin + (t * QS_NW + wave) * 16 + 4 * g;
-    st.pr = *reinterpret_cast<const uint4 *>(xr + 2 * min(rbase, R - 4));
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int row = min(rbase + i, R - 1);
-      st.d[i] = *reinterpret_cast<const uint4 *>(wp + (int64_t)row * C);
-    }
-  };
-
-  floatx4 acc[16];
-#pragma unroll
-  for (int t = 0; t < 16; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-  float se = 0.f, so = 0.f;
-  const half2_t sixteenth = half2_t{(_Float16)0.0625f, (_Float16)0.0625f};
-  const DqConst dqk = dq_const<BF>();
-
-  auto consume = [&](Step &st, int t) __attribute__((always_inline)) {
-    const int rbase = r_begin + (t * QS_NW + wave) * 16 + 4 * g;
-    const bool ok = m_ok && t < nsteps && rbase < r_end;
-    uint32_t pr[4];
-    pr[0] = ok ? st.pr.x : 0u;
-    pr[1] = ok ? st.pr.y : 0u;
-    pr[2] = ok ? st.pr.z : 0u;
-    pr[3] = ok ? st.pr.w : 0u;
-    uint4 av;
-    av.x = __builtin_amdgcn_perm(pr[1], pr[0], 0x05040100u);
-    av.z = __builtin_amdgcn_perm(pr[3], pr[2], 0x05040100u);
-    uint32_t o0 = __builtin_amdgcn_perm(pr[1], pr[0], 0x07060302u);
-    uint32_t o1 = __builtin_amdgcn_perm(pr[3], pr[2], 0x07060302u);
-    if (!BF) {
-      o0 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, o0) * sixteenth);
-      o1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, o1) * sixteenth);
-    }
-    av.y = o0;
-    av.w = o1;
-    se += (Act<TX>::lo(av.x) + Act<TX>::hi(av.x)) + (Act<TX>::lo(av.z) + Act<TX>::hi(av.z));
-    so += (Act<TX>::lo(o0) + Act<TX>::hi(o0)) + (Act<TX>::lo(o1) + Act<TX>::hi(o1));
-#pragma unroll
-    for (int tl = 0; tl < 16; ++tl) {
-      const int w = tl >> 2, tb = tl & 3;
-      const uint32_t sel = 0x0c000c00u | ((uint32_t)(4 + tb) << 16) | (uint32_t)tb;
-      uint4 bv;
-      dequant_pair<BF>(dqk, u4_comp(st.d[0], w), u4_comp(st.d[1], w), sel, bv.x, bv.y);
-      dequant_pair<BF>(dqk, u4_comp(st.d[2], w), u4_comp(st.d[3], w), sel, bv.z, bv.w);
-      acc[tl] = Act<TX>::mma(av, bv, acc[tl]);
-    }
-  };
-
-  Step ring[QS_RING];
-#pragma unroll
-  for (int u = 0; u < QS_RING; ++u) issue(ring[u], u);
-  int t0 = 0;
-  for (; t0 + QS_RING <= nsteps; t0 += QS_RING) {
-#pragma unroll
-    for (int u = 0; u < QS_RING; ++u) {
-      consume(ring[u], t0 + u);
-      issue(ring[u], t0 + u + QS_RING);
-    }
-  }
-  // at most QS_RING - 1 k-steps left, all of them loaded
-#pragma unroll
-  for (int u = 0; u < QS_RING - 1; ++u)
-    if (t0 + u < nsteps) consume(ring[u], t0 + u);
-
-  se += __shfl_xor(se, 16);
-  se += __shfl_xor(se, 32);
-  so += __shfl_xor(so, 16);
-  so += __shfl_xor(so, 32);
-  // acc[tl][r] = tile[m = 4g + r][channel 16 * l16 + tl]
-  float *slot = red + (size_t)wave * mrows * QSTRIP;
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int m = 4 * g + r;
-    if (m < mrows) {
-      float *dst = slot + m * QSTRIP;
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        *reinterpret_cast<float4 *>(dst + qtile_chunk(l16, q)) =
-            make_float4(acc[4 * q][r], acc[4 * q + 1][r], acc[4 * q + 2][r], acc[4 * q + 3][r]);
-    }
-  }
-  qmm_reduce_and_store<16>(red, &s_last, QS_NW, mrows, mvalid, strip, split, m0, M, C, S, zero, scale,
-                           out, ws, se, so);
-}
-
 // 16 bytes from an address of any alignment
 struct __attribute__((packed, aligned(1))) QdU4 { uint32_t x, y, z, w; };
 template <bool UNALIGNED>
@@ -871,12 +746,10 @@ __global__ __launch_bounds__(NW * 64) void qmm_fwd_dec_kernel(
 
 struct FwdPlan {
   int nw, spw, S, strips, mch;
-  bool stream;             // qmm_fwd_stream_kernel: rows_per_split packed rows per workgroup
-  int rows_per_split;
   size_t lds_bytes, counter_bytes, x1_bytes, part_bytes, total_bytes;
 };
 
-FwdPlan fwd_plan(int64_t M, int64_t R, int64_t C, bool allow_stream) {
+FwdPlan fwd_plan(int64_t M, int64_t R, int64_t C) {
   FwdPlan p;
   p.strips = (int)ceil_div64(C, QSTRIP);
   p.mch = (int)ceil_div64(M, 16);
@@ -885,22 +758,6 @@ FwdPlan fwd_plan(int64_t M, int64_t R, int64_t C, bool allow_stream) {
   if (M <= 4) { p.nw = 16; p.spw = 2; }
   else { p.nw = 8; p.spw = 4; }
   p.S = (int)ceil_div64(R, (int64_t)p.nw * p.spw * 16);
-  p.stream = false;
-  p.rows_per_split = 0;
-  if (M <= 16 && allow_stream && R % 4 == 0 && C >= 16) {
-    // two 4-wavefront workgroups per CU; streaming pays once a wavefront has >= 8 k-steps
-    // (measured: even at 65 MB of packed weights, 20 - 35 % faster from 80 MB on)
-    int64_t S = 512 / p.strips;
-    if (S < 1) S = 1;
-    const int64_t rows = round_up64(ceil_div64(R, S), QS_NW * 16);
-    if (rows >= 8 * QS_NW * 16) {
-      p.stream = true;
-      p.rows_per_split = (int)rows;
-      p.S = (int)ceil_div64(R, rows);
-      p.nw = QS_NW;
-      p.spw = 1;
-    }
-  }
   const int mrows = (M <= 4) ? 4 : 16;
   p.lds_bytes = ((size_t)p.nw * mrows * QSTRIP + (size_t)p.nw * 32) * sizeof(float);
   p.counter_bytes = QMM_HEAD_BYTES;
@@ -933,22 +790,6 @@ int launch_fwd_mfma(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, 
                        p.S);
     GPTQ_CHECK_LAUNCH();
   }
-  return GPTQ_HIP_OK;
-}
-
-template <typename TZ, typename TX>
-int launch_fwd_stream(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, const uint8_t *pk,
-                      int64_t R, int64_t C, const void *zero, const void *scale, void *out, void *wsp) {
-  const QmmWs ws = qmm_ws(wsp, p.x1_bytes);
-  auto kern = qmm_fwd_stream_kernel<TZ, TX>;
-  if (p.strips > QMM_MAX_COUNTERS || p.mch != 1 || C < 16) return GPTQ_HIP_EINVAL;
-  if (p.lds_bytes > 48 * 1024 && !gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), (int)p.lds_bytes))
-    return GPTQ_HIP_ELAUNCH;
-  const dim3 grid((unsigned)p.strips, (unsigned)p.S, 1);
-  hipLaunchKernelGGL(kern, grid, dim3(QS_NW * 64), p.lds_bytes, st, (const TX *)x, (int)M,
-                     (int)(2 * R), pk, (int)R, (int)C, (const TZ *)zero, (const TZ *)scale, (TX *)out,
-                     ws, p.S, p.rows_per_split);
-  GPTQ_CHECK_LAUNCH();
   return GPTQ_HIP_OK;
 }
 
@@ -1169,7 +1010,6 @@ template <typename TZ, typename TX>
 int launch_fwd_mfma_zx(hipStream_t st, const FwdPlan &p, const void *x, int64_t M, const uint8_t *pk,
                        int64_t R, int64_t C, const void *zero, const void *scale, void *out,
                        void *wsp) {
-  if (p.stream) return launch_fwd_stream<TZ, TX>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
   if (p.spw == 2) return launch_fwd_mfma<2, TZ, TX, false>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
   // the m-chunks of one call start 16 rows (32 R bytes) apart: aligned together with x when R % 4 == 0
   if ((reinterpret_cast<uintptr_t>(x) & 15) == 0 && R % 4 == 0)
@@ -1186,365 +1026,15 @@ int launch_fwd_mfma_z(hipStream_t st, const FwdPlan &p, const void *x, int x_dty
   return launch_fwd_mfma_zx<TZ, __half>(st, p, x, M, pk, R, C, zero, scale, out, wsp);
 }
 
-// ---------------------------------------------------------------------------- large M
-// Forward, fp16 activations, M > 32: a tiled GEMM that dequantises on the way into LDS.
-// Workgroup tile BM = 64 or 128 (M) x BN (N) x 64 (k) per stage, 4 wavefronts as 2 x 2, accumulators of
-// v_mfma_f32_16x16x32_f16 in registers for the whole K loop (no split-K, no partials).
-//   A = activations: staged in their natural [m][k] layout (k contiguous = the operand order)
-//   B = weights: every thread loads 16 packed bytes (16 channels of one packed row), turns
-//       each byte into the fp16 pair {code_lo - zi, code_hi - zi}, zi = rint(zero) (0x6400 trick:
-//       1024 + code_lo and 1024 + 16 code_hi by masking in place, then one packed fma with
-//       {1, 1/16} and {-(1024 + zi), -(64 + zi)}, exact) and stores it at Bs[channel][2*row],
-//       so that the operand fetch is again one 16-byte read of 8 consecutive k.  The fraction
-//       zero - zi (0 for the zero points GPTQ produces) is applied exactly in the epilogue
-//       through the row sums of the activations, which the staging threads keep in fp32.
-// Row pitch 72 halves and a skew of 8 words per 16-channel group keep both the transposing
-// stores and the operand reads free of bank conflicts.  scale is applied in the epilogue.
+// ---------------------------------------------------------------------------- tiled kernel, LDS layout
+// 64 x 128 x 64 tiles of the transposed kernel below: row pitch 72 halves and a skew of 8 words per 16-channel group
+// keep both the transposing stores and the operand reads free of bank conflicts.
 constexpr int GBM = 64, GBK = 64;
 constexpr int GPITCH = GBK + 8;                 // halves per LDS row
 constexpr int GGROUP = 16 * GPITCH + 16;        // halves per 16-row group (16 = the 8-word skew)
 
 __device__ __forceinline__ int g_off(int row, int k) {   // LDS offset (halves) of element [row][k]
   return (row >> 4) * GGROUP + (row & 15) * GPITCH + k;
-}
-
-// bf16 activations: the weights enter as 128 + code (bit operations only, exact in bf16) and
-// the whole 128 + zero is removed in the epilogue through the same row sums.
-template <int BM, int BN, typename TZ, typename TX, bool SPLIT>
-__global__ __launch_bounds__(256, 2) void qmm_fwd_gemm_kernel(const TX *x, int M, int K,
-                                                           const uint8_t *pk, int R, int C,
-                                                           const TZ *zero, const TZ *scale,
-                                                           TX *out, QmmWs ws, int S) {
-  constexpr bool BF = Act<TX>::BF;
-  __shared__ int s_last;
-  constexpr int A_HALVES = (BM / 16) * GGROUP;
-  constexpr int B_HALVES = (BN / 16) * GGROUP;
-  constexpr int TM = BM / 32;                   // 16-wide MFMA tiles per wavefront along M
-  constexpr int TN = BN / 32;                   // ... and along N
-  constexpr int B_THREADS = 2 * BN;             // threads that stage weights: 32 rows x BN/16 segments
-  constexpr int TPR = 256 / BM;                 // threads that stage one activation row
-  constexpr int AL = 64 / TPR / 8;              // 16-byte loads per thread and stage
-  extern __shared__ __attribute__((aligned(16))) _Float16 qgemm_lds[];
-  _Float16 (*As)[A_HALVES] = reinterpret_cast<_Float16 (*)[A_HALVES]>(qgemm_lds);
-  _Float16 (*Bs)[B_HALVES] = reinterpret_cast<_Float16 (*)[B_HALVES]>(qgemm_lds + 2 * A_HALVES);
-  float *rowsum = reinterpret_cast<float *>(qgemm_lds + 2 * A_HALVES + 2 * B_HALVES);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1, g = lane >> 4, l16 = lane & 15;
-  int tx, ty;
-  qmm_tile_coords(tx, ty);
-  const int n0 = tx * BN, m0 = ty * BM;
-  // split-K: this workgroup multiplies the stages [kbeg, kend) of the contraction axis
-  const int split = SPLIT ? blockIdx.z : 0;
-  const int sps = ((K + GBK - 1) / GBK + S - 1) / S;
-  const int kbeg = SPLIT ? split * sps * GBK : 0, kend = SPLIT ? min(K, kbeg + sps * GBK) : K;
-
-  // A staging: TPR threads per row, 8 * AL consecutive halves each
-  const int a_row = tid / TPR, a_k = (tid % TPR) * (8 * AL);
-  const bool a_ok = (m0 + a_row) < M;
-  const TX *a_src = x + (int64_t)(m0 + a_row) * K + a_k;
-  // B staging: thread -> packed row tid / (BN/16), 16 channels at (tid % (BN/16)) * 16
-  const int b_row = tid / (BN / 16), b_c = (tid % (BN / 16)) * 16;
-  const bool b_thread = tid < B_THREADS;
-  const bool b_ok = b_thread && (n0 + b_c) < C;
-  const uint8_t *b_src = pk + (int64_t)b_row * C + n0 + b_c;
-  float xsum = 0.f;     // sum over k of this thread's share of activation row a_row
-  // -(1024 + rint(zero)) per staged channel, as fp16 pairs
-  uint32_t zc[16];
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    // unconditional clamped loads: sixteen loads in flight instead of sixteen latencies in a row
-    const float zl = to_f32(zero[min(n0 + b_c + i, C - 1)]);
-    const float z = (b_ok && !BF) ? rintf(zl) : 0.f;
-    // low nibble arrives as 1024 + code, high nibble as (1024 + 16 code) / 16 = 64 + code
-    zc[i] = __builtin_bit_cast(uint32_t, half2_t{(_Float16)(-(1024.f + z)), (_Float16)(-(64.f + z))});
-  }
-
-  // Register ring of four stages (named variables, so that they are sure to live in VGPRs):
-  // the loads of stage s + 4 are issued while stage s is being multiplied, so about four
-  // stage times hide the memory latency even with one workgroup per CU.
-  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-  struct Stage { u32x4 a[AL]; u32x4 b; };
-  // Loads are unconditional (out-of-range lanes read a clamped, valid address and are zeroed
-  // when the stage is written to LDS): a load inside a branch would make the compiler wait
-  // for it at the join and defeat the prefetch.  K % 8 == 0 is guaranteed by the dispatcher.
-  auto load_stage = [&](int k0, Stage &st) __attribute__((always_inline)) {
-#pragma unroll
-    for (int l = 0; l < AL; ++l) {
-      const bool ok = a_ok && (k0 + a_k + 8 * (l + 1) <= kend);
-      st.a[l] = *reinterpret_cast<const u32x4 *>(ok ? a_src + k0 + 8 * l : x);
-    }
-    const bool okb = b_ok && ((k0 >> 1) + b_row < R) && (!SPLIT || k0 + 2 * b_row < kend);
-    st.b = *reinterpret_cast<const u32x4 *>(okb ? b_src + (int64_t)(k0 >> 1) * C : pk);
-  };
-  auto store_stage = [&](int buf, int k0, const Stage &st) __attribute__((always_inline)) {
-    const u32x4 zero4 = {0u, 0u, 0u, 0u};
-    const half2_t ones = half2_t{(_Float16)1.f, (_Float16)1.f};
-#pragma unroll
-    for (int l = 0; l < AL; ++l) {
-      const bool ok = a_ok && (k0 + a_k + 8 * (l + 1) <= kend);
-      const u32x4 va = ok ? st.a[l] : zero4;
-      *reinterpret_cast<u32x4 *>(&As[buf][g_off(a_row, a_k + 8 * l)]) = va;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const uint32_t w0 = va[i];
-        if (BF) xsum += Act<TX>::lo(w0) + Act<TX>::hi(w0);
-        else xsum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, w0), ones, xsum, false);
-      }
-    }
-    if (b_thread) {
-      const bool okb = b_ok && ((k0 >> 1) + b_row < R) && (!SPLIT || k0 + 2 * b_row < kend);
-      const u32x4 pbm = okb ? st.b : zero4;
-      const uint32_t w[4] = {pbm[0], pbm[1], pbm[2], pbm[3]};
-      const half2_t unscale = half2_t{(_Float16)1.f, (_Float16)0.0625f};
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        uint32_t v;
-        if (BF) {
-          const uint32_t b = (w[i >> 2] >> (8 * (i & 3))) & 0xFFu;
-          v = ((b | (b << 12)) & 0x000F000Fu) | 0x43004300u;                   // bf16 {128+lo, 128+hi}
-        } else {
-          // three operations per byte: the byte into both halves, both nibbles masked in place
-          // under the exponent of 1024 (fp16 {1024 + lo, 1024 + 16 hi}), one packed fma that
-          // rescales the high half and subtracts offset and zero point (all values are small
-          // integers, so this is exact)
-          const uint32_t sel = 0x0c000c00u | (uint32_t)(i & 3) | ((uint32_t)(i & 3) << 16);
-          const uint32_t pb = __builtin_amdgcn_perm(0u, w[i >> 2], sel);
-          v = (pb & 0x00F0000Fu) | 0x64006400u;
-          const half2_t d = __builtin_bit_cast(half2_t, v) * unscale + __builtin_bit_cast(half2_t, zc[i]);
-          v = __builtin_bit_cast(uint32_t, d);
-        }
-        *reinterpret_cast<uint32_t *>(&Bs[buf][g_off(b_c + i, 2 * b_row)]) = v;
-      }
-    }
-  };
-
-  floatx4 acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-  Stage s0, s1, s2, s3;
-  load_stage(kbeg, s0);
-  load_stage(kbeg + GBK, s1);
-  load_stage(kbeg + 2 * GBK, s2);
-  load_stage(kbeg + 3 * GBK, s3);
-  int buf = 0;
-  store_stage(0, kbeg, s0);
-  __syncthreads();
-  // one stage: refill the ring slot that was just consumed, multiply the stage in LDS, write
-  // the next stage to the other LDS buffer
-  // (Every path into the loop head is a point where the compiler merges the states of the
-  // outstanding loads: an early exit inside the unrolled group made it drain the ring there.
-  // Hence full groups of four without exits, and a tail that issues no loads.)
-  auto step = [&](int k0, Stage &refill, const Stage &next, bool do_load, bool has_next)
-                  __attribute__((always_inline)) {
-    if (do_load) load_stage(k0 + 4 * GBK, refill);
-#pragma unroll
-    for (int ks = 0; ks < GBK; ks += 32) {
-      uint4 a[TM], b[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        a[i] = *reinterpret_cast<const uint4 *>(&As[buf][g_off(wm * (BM / 2) + i * 16 + l16, ks + 8 * g)]);
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        b[j] = *reinterpret_cast<const uint4 *>(
-            &Bs[buf][g_off(wn * (BN / 2) + j * 16 + l16, ks + 8 * g)]);
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = Act<TX>::mma(a[i], b[j], acc[i][j]);
-    }
-    if (has_next) store_stage(buf ^ 1, k0 + GBK, next);
-    __syncthreads();
-    buf ^= 1;
-  };
-  if constexpr (BM == 64) {
-    const int nst = (kend - kbeg + GBK - 1) / GBK;
-    int si = 0, kb = kbeg;
-    for (; si + 4 < nst; si += 4, kb += 4 * GBK) {
-      step(kb, s0, s1, true, true);
-      step(kb + GBK, s1, s2, true, true);
-      step(kb + 2 * GBK, s2, s3, true, true);
-      step(kb + 3 * GBK, s3, s0, true, true);
-    }
-    for (; si < nst; ++si, kb += GBK) {      // at most four stages, all of them loaded
-      step(kb, s0, s1, false, si + 1 < nst);
-      s0 = s1;
-      s1 = s2;
-      s2 = s3;
-    }
-  } else {
-    // 128-row tiles: the exit-free form needs ~50 more registers and drops this instantiation
-    // to one wavefront per SIMD (measured 395 us against 283 at M = 2048); here the ring is
-    // drained at the head of every group of four stages instead.
-    auto stepx = [&](int k0, Stage &refill, const Stage &next) __attribute__((always_inline)) {
-      if (k0 >= kend) return;
-      step(k0, refill, next, true, k0 + GBK < kend);
-    };
-    for (int kb = kbeg; kb < kend; kb += 4 * GBK) {
-      stepx(kb, s0, s1);
-      stepx(kb + GBK, s1, s2);
-      stepx(kb + 2 * GBK, s2, s3);
-      stepx(kb + 3 * GBK, s3, s0);
-    }
-  }
-
-  // the staging threads of a row are neighbouring lanes
-  xsum += __shfl_xor(xsum, 1);
-  if (TPR == 4) xsum += __shfl_xor(xsum, 2);
-  if ((tid % TPR) == 0) rowsum[a_row] = xsum;
-  __syncthreads();
-  if (SPLIT) {
-    // Partial tile and partial row sums to the workspace (agent-scope write-through stores), an
-    // arrival ticket per output tile; the last workgroup of a tile adds the S partials in split
-    // order, so the result does not depend on the arrival order, and leaves the counter at zero.
-    const int tile = ty * gridDim.x + tx;
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int n = n0 + wn * (BN / 2) + j * 16 + l16;
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int m = m0 + wm * (BM / 2) + i * 16 + 4 * g + r;
-          if (n < C && m < M)
-            __hip_atomic_store(&ws.part[((int64_t)split * M + m) * C + n], acc[i][j][r],
-                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
-    float *xp = ws.x1part + ((int64_t)tile * S) * BM;
-    if (tid < BM)
-      __hip_atomic_store(&xp[split * BM + tid], rowsum[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    if (tid == 0) {
-      int32_t *ctr = ws.counters + tile;
-      const int ticket = atomicAdd(ctr, 1);
-      s_last = (ticket == S - 1);
-      if (ticket == S - 1) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    if (!s_last) return;
-    if (tid < BM) {
-      float a = 0.f;
-      for (int sp = 0; sp < S; ++sp)
-        a += __hip_atomic_load(&xp[sp * BM + tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      rowsum[tid] = a;
-    }
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
-    for (int sp = 0; sp < S; ++sp) {
-      floatx4 pv[TM][TN];
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int n = min(n0 + wn * (BN / 2) + j * 16 + l16, C - 1);
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int m = min(m0 + wm * (BM / 2) + i * 16 + 4 * g + r, M - 1);
-            pv[i][j][r] = __hip_atomic_load(&ws.part[((int64_t)sp * M + m) * C + n], __ATOMIC_RELAXED,
-                                            __HIP_MEMORY_SCOPE_AGENT);
-          }
-      }
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] += pv[i][j];
-    }
-    __syncthreads();
-  }
-  // acc[i][j][r] = out[m0 + wm*32 + i*16 + 4g + r][n0 + wn*BN/2 + j*16 + l16]
-#pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int n = n0 + wn * (BN / 2) + j * 16 + l16;
-    if (n >= C) continue;
-    const float sc = to_f32(scale[n]);
-    const float z = to_f32(zero[n]);
-    const float zf = BF ? 128.f + z : z - rintf(z);
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int ml = wm * (BM / 2) + i * 16 + 4 * g + r;
-        if (m0 + ml < M)
-          out[(int64_t)(m0 + ml) * C + n] = Act<TX>::out(sc * (acc[i][j][r] - zf * rowsum[ml]));
-      }
-  }
-}
-
-// Tiled kernel plan: S = 1 when the 64 x 128 output tiles alone fill the chip, else split-K
-// over S workgroups per tile (partials and arrival counters in the workspace, as above).
-struct GemmPlan {
-  bool use;
-  int bm;            // rows per output tile: 128 from M = 256 on (the dequantisation of a weight stage
-                     // is shared by twice as many rows; measured slower than 64 at M = 128), else 64
-  int S;
-  int64_t tiles;
-  size_t x1_bytes, part_bytes, total_bytes;
-};
-
-GemmPlan gemm_plan(int64_t M, int64_t R, int64_t C) {
-  GemmPlan p;
-  p.bm = M >= 256 ? 128 : 64;
-  p.tiles = ceil_div64(C, 128) * ceil_div64(M, p.bm);
-  const int64_t stages = ceil_div64(2 * R, GBK);
-  int64_t S = 1;
-  if (p.tiles < 384) {
-    // about two (64-row tiles) or one (128-row tiles) workgroups per CU; every further split adds
-    // an M x C fp32 partial that is written and read once more
-    S = ((p.bm == 64 ? 512 : 256) + p.tiles - 1) / p.tiles;
-    if (S > 8) S = 8;
-    while (S > 1 && stages / S < 8) --S;          // at least 8 stages per workgroup
-    // every split must own at least one stage
-    while (S > 1 && (S - 1) * ceil_div64(stages, S) >= stages) --S;
-  }
-  p.S = (int)S;
-  p.use = M > 32 && (2 * R) % 8 == 0 && p.tiles * S >= 160 && p.tiles <= QMM_MAX_COUNTERS &&
-          ceil_div64(M, p.bm) <= 65535;
-  p.x1_bytes = S > 1 ? (size_t)round_up64(p.tiles * S * p.bm * (int64_t)sizeof(float), 256) : 0;
-  p.part_bytes = S > 1 ? (size_t)S * M * C * sizeof(float) : 0;
-  p.total_bytes = S > 1 ? QMM_HEAD_BYTES + p.x1_bytes + p.part_bytes : 0;
-  return p;
-}
-
-template <int BM, typename TZ, typename TX, bool SPLIT>
-int launch_fwd_gemm_inst(hipStream_t st, const GemmPlan &p, const void *x, int64_t M, const uint8_t *pk,
-                         int64_t R, int64_t C, const void *zero, const void *scale, void *out,
-                         const QmmWs &ws) {
-  constexpr size_t lds = (size_t)(2 * (BM / 16) * GGROUP + 2 * (128 / 16) * GGROUP) * sizeof(_Float16) +
-                         BM * sizeof(float);
-  auto kern = qmm_fwd_gemm_kernel<BM, 128, TZ, TX, SPLIT>;
-  if (lds > 64 * 1024 && !gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), (int)lds)) return GPTQ_HIP_ELAUNCH;
-  const dim3 grid((unsigned)ceil_div64(C, 128), (unsigned)ceil_div64(M, BM), (unsigned)p.S);
-  hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (const TX *)x, (int)M, (int)(2 * R), pk, (int)R,
-                     (int)C, (const TZ *)zero, (const TZ *)scale, (TX *)out, ws, p.S);
-  GPTQ_CHECK_LAUNCH();
-  return GPTQ_HIP_OK;
-}
-
-template <typename TZ, typename TX>
-int launch_fwd_gemm_x(hipStream_t st, const GemmPlan &p, const void *x, int64_t M, const uint8_t *pk,
-                      int64_t R, int64_t C, const void *zero, const void *scale, void *out,
-                      const QmmWs &ws) {
-  if (p.bm == 128) {
-    if (p.S > 1) return launch_fwd_gemm_inst<128, TZ, TX, true>(st, p, x, M, pk, R, C, zero, scale, out, ws);
-    return launch_fwd_gemm_inst<128, TZ, TX, false>(st, p, x, M, pk, R, C, zero, scale, out, ws);
-  }
-  if (p.S > 1) return launch_fwd_gemm_inst<64, TZ, TX, true>(st, p, x, M, pk, R, C, zero, scale, out, ws);
-  return launch_fwd_gemm_inst<64, TZ, TX, false>(st, p, x, M, pk, R, C, zero, scale, out, ws);
-}
-
-template <typename TZ>
-int launch_fwd_gemm(hipStream_t st, const GemmPlan &p, const void *x, int x_dtype, int64_t M,
-                    const uint8_t *pk, int64_t R, int64_t C, const void *zero, const void *scale,
-                    void *out, void *wsp) {
-  const QmmWs ws = qmm_ws(wsp, p.x1_bytes);
-  if (x_dtype == GPTQ_HIP_BF16)
-    return launch_fwd_gemm_x<TZ, __hip_bfloat16>(st, p, x, M, pk, R, C, zero, scale, out, ws);
-  return launch_fwd_gemm_x<TZ, __half>(st, p, x, M, pk, R, C, zero, scale, out, ws);
 }
 
 // ---------------------------------------------------------------------------- transposed
@@ -2067,9 +1557,8 @@ size_t ws16_bytes(int64_t M, int64_t R, int64_t C, int transpose_b, int bits) {
     return need;
   }
   // which kernel runs also depends on pointer alignment: enough for any of them
-  const size_t cand[4] = {fwd_plan(M, R, C, false).total_bytes, gemm_plan(M, R, C).total_bytes,
-                          fwd_plan(M, R, C, true).total_bytes, 0};
-  for (size_t c : cand) need = c > need ? c : need;
+  const size_t chunked = fwd_plan(M, R, C).total_bytes;
+  need = chunked > need ? chunked : need;
   const DecPlan dp = dec_plan(M, R, C);
   if (dp.use && dp.total_bytes > need) need = dp.total_bytes;
   const MidPlan mp = mid_fwd_plan(M, R, C, true);
@@ -2120,7 +1609,17 @@ bool aligned16(const void *a, const void *b) {
 int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed, int64_t R, int64_t C,
                  const void *zero, const void *scale, int zs_dtype, int bits, int64_t group_size, int transpose_b,
                  void *out, void *ws, size_t ws_bytes, float *out32 = nullptr, const int32_t *rowexp = nullptr,
-                 bool *wrote32 = nullptr) {
+                 bool *wrote32 = nullptr, gptq_hip_qmatmul_plan *plan = nullptr) {
+  // plan != nullptr: nothing is launched; the pointers are only looked at for their alignment, and *plan says
+  // which kernel the same call would run (`planned` in front of every launch).
+  auto planned = [&](int kernel, int rest, int64_t splits, int64_t workgroups) -> bool {
+    if (!plan) return false;
+    plan->kernel = kernel;
+    plan->kernel_rest = rest;
+    plan->splits = (int)splits;
+    plan->workgroups = workgroups;
+    return true;
+  };
   if (M < 0 || R <= 0 || C <= 0 || (bits != 4 && bits != 8)) return GPTQ_HIP_EINVAL;
   if (group_size < 0 || group_size % 2 != 0 || (group_size > 0 && (bits == 4 ? 2 * R : R) % group_size != 0) ||
       group_size > (1LL << 30))
@@ -2146,6 +1645,10 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
           (reinterpret_cast<uintptr_t>(out) & 3) == 0) {
         const DecPlan dp = dec_plan(M, R, C);
         if (dp.use && dp.atom && (dp.total_bytes == 0 || (ws && ws_bytes >= dp.total_bytes))) {
+          if (planned(GPTQ_HIP_QMM_DECODE, 0, dp.S, (int64_t)dp.strips * dp.S)) {
+            plan->fp32_rows = 2;
+            return GPTQ_HIP_OK;
+          }
           const int32_t *re = nullptr;
           if (M > 2) {            // beyond two rows every workgroup's own pass over the rows costs more than a launch
             hipLaunchKernelGGL(x32_rowexp_kernel, dim3((unsigned)M), dim3(256), 0, st,
@@ -2161,6 +1664,14 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
             default: return GPTQ_HIP_EDTYPE;
           }
         }
+      }
+      if (plan) {
+        // the kernel of the (first) chunk of rows, on the aligned staging buffers
+        const int64_t mm = M < fp.mc ? M : fp.mc;
+        const int rc = qmatmul_impl(stream, x16, GPTQ_HIP_F16, mm, packed, R, C, zero, scale, zs_dtype, bits, group_size,
+                                    transpose_b, o16, ws, fp.inner, nullptr, nullptr, nullptr, plan);
+        plan->fp32_rows = 1;
+        return rc;
       }
       for (int64_t r0 = 0; r0 < M; r0 += fp.mc) {
         const int64_t mm = M - r0 < fp.mc ? M - r0 : fp.mc;
@@ -2184,6 +1695,7 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
       }
       return GPTQ_HIP_OK;
     }
+    if (planned(transpose_b ? GPTQ_HIP_QMM_BWD_SIMPLE : GPTQ_HIP_QMM_SIMPLE, 0, 1, 0)) return GPTQ_HIP_OK;
     return bits == 4
                ? dispatch_simple<4>(st, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out, group_size)
                : dispatch_simple<8>(st, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out, group_size);
@@ -2194,6 +1706,19 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
   const RegPlan rp = (transpose_b || !reg_groups_ok) ? RegPlan{} : reg_fwd_plan(M, R, C, bits, al);
   auto run_reg_fwd = [&]() -> int {
     if (rp.total_bytes && (!ws || ws_bytes < rp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+    if (plan) {
+      const RegParts parts = reg_fwd_parts(rp, M, R, C, x_dtype == GPTQ_HIP_BF16, (int)group_size);
+      const int own = rp.rb == 8 ? GPTQ_HIP_QMM_REG128 : (rp.rb == 4 ? GPTQ_HIP_QMM_REG64 : GPTQ_HIP_QMM_REG16);
+      const int64_t ty = ceil_div64(M, 16 * rp.rb);
+      if (parts.wide_x > 0)
+        planned(parts.half ? GPTQ_HIP_QMM_WIDE_HALF : GPTQ_HIP_QMM_WIDE,
+                parts.main_x > 0 ? GPTQ_HIP_QMM_REG128 : (parts.tail > 0 ? GPTQ_HIP_QMM_REG64 : 0), 1,
+                parts.wide_x * ceil_div64(M, 128));
+      else
+        planned(parts.main_x > 0 ? own : GPTQ_HIP_QMM_REG64, (parts.main_x > 0 && parts.tail > 0) ? GPTQ_HIP_QMM_REG64 : 0,
+                rp.S, (parts.main_x > 0 ? parts.main_x : parts.tail) * ty * rp.S);
+      return GPTQ_HIP_OK;
+    }
     RegPlan q = rp;
     if (out32 && rowexp && wrote32 && rp.rb > 1 && x_dtype == GPTQ_HIP_F16) {
       q.out32 = out32;
@@ -2208,6 +1733,7 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
     const DecPlan dp = dec_plan(M, R, C, 8);
     if (dp.use) {
       if (dp.total_bytes && (!ws || ws_bytes < dp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+      if (planned(GPTQ_HIP_QMM_DECODE, 0, dp.S, (int64_t)dp.strips * dp.S)) return GPTQ_HIP_OK;
       switch (zs_dtype) {
         case GPTQ_HIP_F32: return launch_dec_z8<float>(st, dp, x, M, packed, R, C, zero, scale, out, ws);
         case GPTQ_HIP_F16: return launch_dec_z8<__half>(st, dp, x, M, packed, R, C, zero, scale, out, ws);
@@ -2222,6 +1748,7 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
     const DecPlan dp = dec_plan(M, R, C, 4, true);
     if (dp.use) {
       if (dp.total_bytes && (!ws || ws_bytes < dp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+      if (planned(GPTQ_HIP_QMM_DECODE_RAGGED, 0, dp.S, (int64_t)dp.strips * dp.S)) return GPTQ_HIP_OK;
       switch (zs_dtype) {
         case GPTQ_HIP_F32: return launch_dec_z_rag<float>(st, dp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
         case GPTQ_HIP_F16: return launch_dec_z_rag<__half>(st, dp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
@@ -2235,6 +1762,7 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
     MidPlan mp = mid_fwd_plan(M, R, C, al && (reinterpret_cast<uintptr_t>(packed) & 15) == 0);
     if (mp.use) {
       if (mp.total_bytes && (!ws || ws_bytes < mp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+      if (planned(GPTQ_HIP_QMM_MID, 0, mp.S, mp.tiles_x * mp.tiles_y * mp.S)) return GPTQ_HIP_OK;
       if (out32 && rowexp && wrote32) {
         mp.out32 = out32;
         mp.rowexp = rowexp;
@@ -2244,27 +1772,14 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
     }
   }
   if (bits == 4 && !transpose_b && group_size == 0) {
-    // more than 16 rows: the register-operand kernel, unless its tiles are too few to fill the chip even when
-    // split (the tiled kernel below splits finer)
+    // more than 16 rows: the register-operand kernel, unless its tiles are too few to fill a quarter of the chip
+    // even when split (small matrices: the chunked kernel below, 16 rows at a time)
     if (rp.use && !rp.ragged && M > 16 && rp.tiles * rp.S >= 64) return run_reg_fwd();
-    // GEMM-shaped work goes to the tiled kernel (split-K when the output tiles alone do not fill
-    // the chip); small M goes through the decode kernel or the 16-row chunked kernels.
-    const GemmPlan gp = gemm_plan(M, R, C);
-    if (fwd_fast_ok(x_dtype, M, R, C, x, packed) && gp.use && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
-      if (gp.total_bytes && (!ws || ws_bytes < gp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
-      switch (zs_dtype) {
-        case GPTQ_HIP_F32:
-          return launch_fwd_gemm<float>(st, gp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
-        case GPTQ_HIP_F16:
-          return launch_fwd_gemm<__half>(st, gp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
-        default:
-          return launch_fwd_gemm<__hip_bfloat16>(st, gp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
-      }
-    }
     if (fwd_fast_ok(x_dtype, M, R, C, x, packed) && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
       const DecPlan dp = dec_plan(M, R, C);
       if (dp.use) {
         if (dp.total_bytes && (!ws || ws_bytes < dp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+        if (planned(GPTQ_HIP_QMM_DECODE, 0, dp.S, (int64_t)dp.strips * dp.S)) return GPTQ_HIP_OK;
         switch (zs_dtype) {
           case GPTQ_HIP_F32: return launch_dec_z<float>(st, dp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
           case GPTQ_HIP_F16: return launch_dec_z<__half>(st, dp, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
@@ -2274,8 +1789,9 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
       }
     }
     if (fwd_fast_ok(x_dtype, M, R, C, x, packed)) {
-      const FwdPlan p = fwd_plan(M, R, C, (reinterpret_cast<uintptr_t>(x) & 15) == 0);
+      const FwdPlan p = fwd_plan(M, R, C);
       if (p.total_bytes && (!ws || ws_bytes < p.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+      if (planned(GPTQ_HIP_QMM_CHUNKED, 0, p.S, (int64_t)p.strips * p.S * p.mch)) return GPTQ_HIP_OK;
       switch (zs_dtype) {
         case GPTQ_HIP_F32:
           return launch_fwd_mfma_z<float>(st, p, x, x_dtype, M, packed, R, C, zero, scale, out, ws);
@@ -2293,11 +1809,28 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
   // more than 64 rows: 128-row tiles of the register-operand kernel (a dequantised operand
   // serves twice the rows; 4096 x 11008 at M = 2048: 335 -> 268 us, 8-bit: 512 -> 347 us) unless their last round
   // of 256 workgroups would leave much of the chip idle (11008 x 4096 at M = 512: 344 tiles)
+  auto plan_reg_bwd = [&](const RegBwdPlan &bp) {
+    const RegParts parts = reg_bwd_parts(bp, M, R, C, x_dtype == GPTQ_HIP_BF16, (int)group_size);
+    const int own = bp.rb == 8 ? GPTQ_HIP_QMM_BWD_REG128 : GPTQ_HIP_QMM_BWD_REG64;
+    const int64_t ty = ceil_div64(M, 16 * bp.rb);
+    if (parts.wide_x > 0)
+      planned(parts.half ? GPTQ_HIP_QMM_BWD_WIDE_HALF : GPTQ_HIP_QMM_BWD_WIDE,
+              parts.main_x > 0 ? GPTQ_HIP_QMM_BWD_REG128 : (parts.tail > 0 ? GPTQ_HIP_QMM_BWD_REG64 : 0), 1,
+              parts.wide_x * ceil_div64(M, 128));
+    else
+      planned(parts.main_x > 0 ? own : GPTQ_HIP_QMM_BWD_REG64,
+              (parts.main_x > 0 && parts.tail > 0) ? GPTQ_HIP_QMM_BWD_REG64 : 0, bp.S,
+              (parts.main_x > 0 ? parts.main_x : parts.tail) * ty * bp.S);
+  };
   if (transpose_b && reg_groups_ok && M > 64) {
     const RegBwdPlan bp8 = reg_bwd_plan(M, R, C, bits, al, 8);
     const int64_t rounds = bp8.use ? (bp8.tiles + 255) / 256 : 0;
     if (bp8.use && (bp8.tiles <= 256 || bp8.tail_x > 0 || bp8.tiles * 5 >= rounds * 256 * 4)) {
       if (bp8.total_bytes && (!ws || ws_bytes < bp8.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+      if (plan) {
+        plan_reg_bwd(bp8);
+        return GPTQ_HIP_OK;
+      }
       RegBwdPlan q = bp8;
       if (out32 && rowexp && wrote32 && x_dtype == GPTQ_HIP_F16) {
         q.out32 = out32;
@@ -2311,6 +1844,7 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
                               !(reg_groups_ok && reg_bwd_plan(M, R, C, bits, al).use);
   if (bits == 4 && transpose_b && group_size == 0 && bwd_tiles_fill &&
       bwd_fast_ok(x_dtype, M, R, C, x, packed, zero, scale)) {
+    if (planned(GPTQ_HIP_QMM_BWD_GEMM, 0, 1, ceil_div64(2 * R, 128) * ceil_div64(M, 64))) return GPTQ_HIP_OK;
     switch (zs_dtype) {
       case GPTQ_HIP_F32: return launch_bwd_gemm<float>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
       case GPTQ_HIP_F16: return launch_bwd_gemm<__half>(st, x, x_dtype, M, packed, R, C, zero, scale, out);
@@ -2323,6 +1857,10 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
     const RegBwdPlan bp = reg_bwd_plan(M, R, C, bits, al);
     if (bp.use) {
       if (bp.total_bytes && (!ws || ws_bytes < bp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
+      if (plan) {
+        plan_reg_bwd(bp);
+        return GPTQ_HIP_OK;
+      }
       RegBwdPlan q = bp;
       if (out32 && rowexp && wrote32 && x_dtype == GPTQ_HIP_F16) {
         q.out32 = out32;
@@ -2332,6 +1870,7 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
       return reg_bwd_launch(st, q, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, out, ws, (int)group_size);
     }
   }
+  if (planned(transpose_b ? GPTQ_HIP_QMM_BWD_SIMPLE : GPTQ_HIP_QMM_SIMPLE, 0, 1, 0)) return GPTQ_HIP_OK;
   return bits == 4
              ? dispatch_simple<4>(st, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out, group_size)
              : dispatch_simple<8>(st, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out, group_size);
@@ -2340,6 +1879,40 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
 }  // namespace
 
 extern "C" {
+
+int gptq_hip_qmatmul_plan_query(int64_t M, int64_t R, int64_t C, int transpose_b, int x_dtype, int zs_dtype, int bits,
+                                int64_t group_size, int aligned, gptq_hip_qmatmul_plan *plan) {
+  if (!plan || M < 1) return GPTQ_HIP_EINVAL;
+  *plan = gptq_hip_qmatmul_plan{};
+  // never dereferenced: qmatmul_impl only looks at the alignment of the pointers when it is given a plan
+  const uintptr_t base = aligned ? 0x10000u : 0x10002u;
+  void *fake = reinterpret_cast<void *>(base);
+  void *fake_ws = reinterpret_cast<void *>((uintptr_t)0x20000u);
+  return qmatmul_impl(nullptr, fake, x_dtype, M, reinterpret_cast<const uint8_t *>(aligned ? base : base - 1), R, C, fake,
+                      fake, zs_dtype, bits, group_size, transpose_b, fake, fake_ws, ~(size_t)0, nullptr, nullptr, nullptr, plan);
+}
+
+const char *gptq_hip_qmatmul_kernel_name(int kernel) {
+  switch (kernel) {
+    case GPTQ_HIP_QMM_SIMPLE: return "qmm_fwd_simple";
+    case GPTQ_HIP_QMM_DECODE: return "qmm_fwd_dec_kernel";
+    case GPTQ_HIP_QMM_DECODE_RAGGED: return "qmm_fwd_dec_kernel (rows of any length)";
+    case GPTQ_HIP_QMM_CHUNKED: return "qmm_fwd_mfma_kernel";
+    case GPTQ_HIP_QMM_MID: return "qmm_fwd_mid_kernel";
+    case GPTQ_HIP_QMM_REG16: return "qmm_fwd_reg_kernel (16-row tiles)";
+    case GPTQ_HIP_QMM_REG64: return "qmm_fwd_reg_kernel (64-row tiles)";
+    case GPTQ_HIP_QMM_REG128: return "qmm_fwd_reg_kernel (128-row tiles)";
+    case GPTQ_HIP_QMM_WIDE: return "qmm_fwd_wide_kernel (128 x 512)";
+    case GPTQ_HIP_QMM_WIDE_HALF: return "qmm_fwd_wide_kernel (128 x 256)";
+    case GPTQ_HIP_QMM_BWD_SIMPLE: return "qmm_bwd_simple";
+    case GPTQ_HIP_QMM_BWD_REG64: return "qmm_bwd_reg_kernel (64-row tiles)";
+    case GPTQ_HIP_QMM_BWD_REG128: return "qmm_bwd_reg_kernel (128-row tiles)";
+    case GPTQ_HIP_QMM_BWD_WIDE: return "qmm_bwd_wide_kernel (128 x 512)";
+    case GPTQ_HIP_QMM_BWD_WIDE_HALF: return "qmm_bwd_wide_kernel (128 x 256)";
+    case GPTQ_HIP_QMM_BWD_GEMM: return "qmm_bwd_gemm_kernel";
+    default: return "none";
+  }
+}
 
 size_t gptq_hip_qmatmul_workspace_bytes(int64_t M, int64_t R, int64_t C, int transpose_b) {
   return ws16_bytes(M, R, C, transpose_b, 4);

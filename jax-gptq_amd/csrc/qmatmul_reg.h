@@ -24,6 +24,16 @@ struct RegPlan {
 };
 
 RegPlan reg_fwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned);
+// How a product on 128-row tiles (rb = 8) is dealt over launches: the leading wide_x tiles of 512 (half: 256)
+// channels or output columns on the 128 x 512 tiles of qmatmul_wide.hip = `first` column tiles of 128, then main_x
+// column tiles on 128-row tiles, then `tail` column tiles on 64-row tiles.  The launch functions and the plan
+// query both go by this.
+struct RegParts {
+  int64_t wide_x;
+  bool half;
+  int64_t first, main_x, tail;
+};
+RegParts reg_fwd_parts(const RegPlan &p, int64_t M, int64_t R, int64_t C, bool bf16, int group_size);
 // x / out element type x_dtype (F16 or BF16), zero / scale element type zs_dtype (F32, F16, BF16).
 // group_size = 0: zero / scale [C]; group_size > 0 (a multiple of 32): zero / scale [K / group_size, C].
 int reg_fwd_launch(hipStream_t st, const RegPlan &p, const void *x, int x_dtype, int64_t M, const uint8_t *pk,
@@ -77,6 +87,7 @@ struct RegBwdPlan {
 };
 // rb = 8: 128-row tiles
 RegBwdPlan reg_bwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned, int rb = 4);
+RegParts reg_bwd_parts(const RegBwdPlan &p, int64_t M, int64_t R, int64_t C, bool bf16, int group_size);
 // group_size > 0: a multiple of 128 (the 128 output columns of a tile share one group)
 int reg_bwd_launch(hipStream_t st, const RegBwdPlan &p, const void *x, int x_dtype, int64_t M, const uint8_t *pk,
                    int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws,

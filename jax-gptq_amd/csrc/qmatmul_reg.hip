@@ -538,40 +538,25 @@ int launch_bx(hipStream_t st, const RegPlan &p, const void *x, int64_t M, const 
   // a ring of two k-steps for 128-row tiles, of three for 64-row tiles (registers), of six for the 16-row tiles
   // of the decode case
   if (p.rb == 8) {
-    const int64_t tiles_all = ceil_div64(C, RG_BN), tiles_y = ceil_div64(M, 128), K = BITS == 4 ? 2 * R : R;
-    // 128 x 512 tiles (qmatmul_wide.hip) on the leading columns that fill whole rounds of workgroups
-    int64_t first = 0;
-    if constexpr (BITS == 4) {
-      if (!p.ragged && p.S == 1) {
-        bool half = false;
-        const int64_t wide_x = wide_fwd_tiles(M, R, C, true, &half);
-        if (wide_x > 0) {
-          const int rc = wide_fwd_launch(st, x, Act<TX>::BF ? GPTQ_HIP_BF16 : GPTQ_HIP_F16, M, pk, R, C, zero, scale,
-                                         zs_dtype, out, wide_x, half, p.out32, p.rowexp);
-          if (rc) return rc;
-          first = (half ? 2 : 4) * wide_x;
-        }
-      }
-    }
-    const int64_t rest = tiles_all - first;
-    if (rest == 0) return GPTQ_HIP_OK;
-    // of the rest: 128-row tiles on the columns that fill whole rounds, 64-row tiles on the remaining ones
-    int64_t tail = first == 0 ? p.tail_x : deal_tail(rest, tiles_y, ceil_div64(K, 32));
-    if (first > 0 && rest * tiles_y <= 128) tail = rest;
-    const int64_t main_x = rest - tail;
-    if (main_x > 0) {
-      const int rc = p.ragged ? launch_inst<BITS, 8, 2, true, TX, false>(st, p, x, M, pk, R, C, zero, scale, zs_dtype,
-                                                                           out, ws, group_size, first, main_x)
-                              : launch_inst<BITS, 8, 3, false, TX, false>(st, p, x, M, pk, R, C, zero, scale, zs_dtype,
-                                                                            out, ws, group_size, first, main_x);
+    const RegParts q = reg_fwd_parts(p, M, R, C, Act<TX>::BF, group_size);
+    if (q.wide_x > 0) {
+      const int rc = wide_fwd_launch(st, x, Act<TX>::BF ? GPTQ_HIP_BF16 : GPTQ_HIP_F16, M, pk, R, C, zero, scale,
+                                     zs_dtype, out, q.wide_x, q.half, p.out32, p.rowexp);
       if (rc) return rc;
     }
-    if (tail == 0) return GPTQ_HIP_OK;
+    if (q.main_x > 0) {
+      const int rc = p.ragged ? launch_inst<BITS, 8, 2, true, TX, false>(st, p, x, M, pk, R, C, zero, scale, zs_dtype,
+                                                                           out, ws, group_size, q.first, q.main_x)
+                              : launch_inst<BITS, 8, 3, false, TX, false>(st, p, x, M, pk, R, C, zero, scale, zs_dtype,
+                                                                            out, ws, group_size, q.first, q.main_x);
+      if (rc) return rc;
+    }
+    if (q.tail == 0) return GPTQ_HIP_OK;
     if (p.ragged)
       return launch_inst<BITS, 4, 3, true, TX, false>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws,
-                                                      group_size, first + main_x, tail);
+                                                      group_size, q.first + q.main_x, q.tail);
     return launch_inst<BITS, 4, 3, false, TX, false>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws,
-                                                     group_size, first + main_x, tail);
+                                                     group_size, q.first + q.main_x, q.tail);
   }
   if (p.rb == 4) {
     if (p.ragged) GPTQ_REG(4, 3, true, false);
@@ -585,6 +570,29 @@ int launch_bx(hipStream_t st, const RegPlan &p, const void *x, int64_t M, const 
 }  // namespace
 
 namespace qmm {
+
+RegParts reg_fwd_parts(const RegPlan &p, int64_t M, int64_t R, int64_t C, bool bf16, int group_size) {
+  (void)bf16;
+  RegParts q{};
+  const int64_t tiles_all = ceil_div64(C, RG_BN);
+  if (p.rb != 8 || group_size > 0) {
+    q.main_x = tiles_all;
+    return q;
+  }
+  const int64_t tiles_y = ceil_div64(M, 128), K = p.bits == 4 ? 2 * R : R;
+  // 128 x 512 tiles (qmatmul_wide.hip) on the leading columns that fill whole rounds of workgroups
+  if (p.bits == 4 && !p.ragged && p.S == 1) {
+    q.wide_x = wide_fwd_tiles(M, R, C, true, &q.half);
+    if (q.wide_x > 0) q.first = (q.half ? 2 : 4) * q.wide_x;
+  }
+  const int64_t rest = tiles_all - q.first;
+  if (rest == 0) return q;
+  // of the rest: 128-row tiles on the columns that fill whole rounds, 64-row tiles on the remaining ones
+  q.tail = q.first == 0 ? p.tail_x : deal_tail(rest, tiles_y, ceil_div64(K, 32));
+  if (q.first > 0 && rest * tiles_y <= 128) q.tail = rest;
+  q.main_x = rest - q.tail;
+  return q;
+}
 
 RegPlan reg_fwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned) {
   RegPlan p{};

@@ -392,40 +392,24 @@ template <int BITS, typename TX>
 int launch_bx(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R,
               int64_t C, const void *zero, const void *scale, int zs_dtype, void *out, void *ws, int group_size) {
   if (p.rb == 8) {
-    const int64_t tiles_all = ceil_div64(R, BITS == 4 ? 64 : 128), tiles_y = ceil_div64(M, 128);
-    // 128 x 512 tiles (qmatmul_wide.hip) on the leading output columns that fill whole rounds of workgroups
-    int64_t first = 0;
-    if constexpr (BITS == 4 && !Act<TX>::BF) {
-      // (also where this kernel's own tiles need a split because the constants of all channels do not fit its LDS)
-      if (!p.ragged && group_size == 0) {
-        bool half = false;
-        const int64_t wide_x = wide_bwd_tiles(M, R, C, true, &half);
-        if (wide_x > 0) {
-          const int rc = wide_bwd_launch(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, half, p.out32, p.rowexp);
-          if (rc) return rc;
-          first = (half ? 2 : 4) * wide_x;
-        }
-      }
-    }
-    const int64_t rest = tiles_all - first;
-    if (rest == 0) return GPTQ_HIP_OK;
-    // of the rest: 128-row tiles on the columns that fill whole rounds of workgroups, 64-row tiles on the others
-    int64_t tail = first == 0 ? p.tail_x : (p.S == 1 ? bwd_deal_tail(rest, tiles_y, ceil_div64(C, 32)) : 0);
-    if (first > 0 && p.S == 1 && rest * tiles_y <= 128) tail = rest;
-    const int64_t main_x = rest - tail;
-    if (main_x > 0) {
-      const int rc = p.ragged ? launch_inst<BITS, true, TX, 8>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws,
-                                                               group_size, first, main_x)
-                              : launch_inst<BITS, false, TX, 8>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws,
-                                                                group_size, first, main_x);
+    const RegParts q = reg_bwd_parts(p, M, R, C, Act<TX>::BF, group_size);
+    if (q.wide_x > 0) {
+      const int rc = wide_bwd_launch(st, x, M, pk, R, C, zero, scale, zs_dtype, out, q.wide_x, q.half, p.out32, p.rowexp);
       if (rc) return rc;
     }
-    if (tail == 0) return GPTQ_HIP_OK;
+    if (q.main_x > 0) {
+      const int rc = p.ragged ? launch_inst<BITS, true, TX, 8>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws,
+                                                               group_size, q.first, q.main_x)
+                              : launch_inst<BITS, false, TX, 8>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws,
+                                                                group_size, q.first, q.main_x);
+      if (rc) return rc;
+    }
+    if (q.tail == 0) return GPTQ_HIP_OK;
     if (p.ragged)
       return launch_inst<BITS, true, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size,
-                                         first + main_x, tail);
+                                         q.first + q.main_x, q.tail);
     return launch_inst<BITS, false, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size,
-                                        first + main_x, tail);
+                                        q.first + q.main_x, q.tail);
   }
   if (p.ragged) return launch_inst<BITS, true, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
   return launch_inst<BITS, false, TX>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws, group_size);
@@ -434,6 +418,29 @@ int launch_bx(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, con
 }  // namespace
 
 namespace qmm {
+
+RegParts reg_bwd_parts(const RegBwdPlan &p, int64_t M, int64_t R, int64_t C, bool bf16, int group_size) {
+  RegParts q{};
+  const int64_t tiles_all = ceil_div64(R, p.bits == 4 ? 64 : 128);
+  if (p.rb != 8) {
+    q.main_x = tiles_all;
+    return q;
+  }
+  const int64_t tiles_y = ceil_div64(M, 128);
+  // 128 x 512 tiles (qmatmul_wide.hip) on the leading output columns that fill whole rounds of workgroups
+  // (also where this kernel's own tiles need a split because the constants of all channels do not fit its LDS)
+  if (p.bits == 4 && !bf16 && !p.ragged && group_size == 0) {
+    q.wide_x = wide_bwd_tiles(M, R, C, true, &q.half);
+    if (q.wide_x > 0) q.first = (q.half ? 2 : 4) * q.wide_x;
+  }
+  const int64_t rest = tiles_all - q.first;
+  if (rest == 0) return q;
+  // of the rest: 128-row tiles on the columns that fill whole rounds of workgroups, 64-row tiles on the others
+  q.tail = q.first == 0 ? p.tail_x : (p.S == 1 ? bwd_deal_tail(rest, tiles_y, ceil_div64(C, 32)) : 0);
+  if (q.first > 0 && p.S == 1 && rest * tiles_y <= 128) q.tail = rest;
+  q.main_x = rest - q.tail;
+  return q;
+}
 
 RegBwdPlan reg_bwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned, int rb) {
   RegBwdPlan p{};

@@ -60,7 +60,28 @@ SIGNATURES = {
     "gptq_hip_qmatmul_grouped": (_i32, [_vp, _vp, _i32, _i64, _vp, _i64, _i64, _vp, _vp, _i32, _i64, _i32, _i32, _vp,
                                         _vp, _sz]),
     "gptq_hip_qmatmul_static": (_i32, [_vp, _vp, _i32, _i64, _vp, _i64, _i64, _vp, _vp, _i32, _i32, _vp]),
+    "gptq_hip_qmatmul_plan_query": (_i32, [_i64, _i64, _i64, _i32, _i32, _i32, _i32, _i64, _i32, _vp]),
+    "gptq_hip_qmatmul_kernel_name": (ctypes.c_char_p, [_i32]),
 }
+
+
+class QmatmulPlan(ctypes.Structure):
+    """gptq_hip_qmatmul_plan of include/gptq_hip.h."""
+    _fields_ = [("kernel", ctypes.c_int), ("kernel_rest", ctypes.c_int), ("splits", ctypes.c_int),
+                ("fp32_rows", ctypes.c_int), ("workgroups", ctypes.c_int64)]
+
+
+def qmatmul_plan(M, R, C, transpose_b=0, x_dtype=F16, zs_dtype=F16, bits=4, group_size=0, aligned=1):
+    """Which kernel(s) the packed matmul runs for these arguments (host only): a dict with the kernels' names,
+    the splits of the contraction, the first kernel's workgroups and how fp32 rows travel."""
+    lib = load()
+    plan = QmatmulPlan()
+    check(lib.gptq_hip_qmatmul_plan_query(M, R, C, transpose_b, x_dtype, zs_dtype, bits, group_size, aligned,
+                                          ctypes.byref(plan)), "qmatmul_plan_query")
+    return {"kernel_id": plan.kernel, "kernel": lib.gptq_hip_qmatmul_kernel_name(plan.kernel).decode(),
+            "rest": lib.gptq_hip_qmatmul_kernel_name(plan.kernel_rest).decode() if plan.kernel_rest else None,
+            "rest_id": plan.kernel_rest, "splits": plan.splits, "workgroups": plan.workgroups,
+            "fp32_rows": plan.fp32_rows}
 
 _lib = None
 
