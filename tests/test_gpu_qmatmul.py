@@ -219,6 +219,8 @@ def test_qmatmul_few_dozen_rows_tall_narrow_tiles(OP, M, N, K, xdt, zs):
     tdt = getattr(torch, zs)
     scale = torch.from_numpy(rng.uniform(0.001, 0.01, N).astype(np.float32)).to(tdt)
     zero = torch.from_numpy(rng.uniform(0.0, 15.0, N).astype(np.float32)).to(tdt)      # fractional, too
+    if xdt == "float32":
+        zero = zero.round()     # (the rounding of fp32 rows to fp16 uses up the tolerance at K = 11008 by itself)
     qm = G.QuantizedMatrix(torch.from_numpy(O.pack_colwise(codes)).cuda(), zero.cuda(), scale.cuda())
     rowscale = np.array([1.0, 1e-3, 3e4])[np.arange(M) % 3][:, None] if xdt == "float32" else np.ones((M, 1))
     x = torch.from_numpy((rng.standard_normal((M, K)) * rowscale).astype(np.float32)).to(getattr(torch, xdt))
