@@ -309,8 +309,11 @@ int gptq_hip_qmatmul_grouped(void *stream, const void *x, int x_dtype, int64_t M
  * exceeds GPTQ_HIP_QMATMUL_STATIC_BYTES is refused with GPTQ_HIP_ETOOBIG and nothing is enqueued.
  * All calls on one GPU share the one array: calls that may overlap in time on a GPU (different
  * streams, different threads) race on it; serialise them or use gptq_hip_qmatmul with a workspace
- * per stream.  The first call on a device looks up the array's address and clears its arrival
- * counters with a small kernel on `stream`. */
+ * per stream.  Nothing is cleared at run time (the array is zero when the library is loaded and every
+ * product leaves its counters at zero), so a call enqueues the product's kernels and nothing else.  The FIRST
+ * call on a device for a given kind of product makes host-side runtime calls that do not belong under stream
+ * capture (it looks up the array's address; kernels that need more than 64 KB of LDS have their limit raised
+ * once): make one eager call of the same shape before capturing, as a warm-up. */
 #define GPTQ_HIP_QMATMUL_STATIC_BYTES ((size_t)32 << 20)
 int gptq_hip_qmatmul_static(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,
                             int64_t R, int64_t C, const void *zero, const void *scale, int zs_dtype,

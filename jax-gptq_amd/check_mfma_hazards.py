@@ -7,8 +7,8 @@ script compiles the files to assembly and verifies it on every MFMA of every ins
     python jax-gptq_amd/check_mfma_hazards.py        # exit status 0: no hazard
 
 An instruction in between counts one wait state, `s_nop n` n + 1, an MFMA two (its issue takes a pass of four
-cycles).  Branch targets are ignored: the scan walks the listing in order, which is the fall-through path; the
-kernels' loop heads start with LDS reads or an explicit `s_nop`.
+cycles).  Every way into an MFMA is followed: the fall-through path and, through labels, the instructions in front
+of the branches to them (a loop's back edge).
 """
 import os
 import re
@@ -32,27 +32,63 @@ def _regs(tok):
 
 
 def scan(asm_text):
-    """Returns (number of MFMAs, list of (writer, mfma) pairs that are too close)."""
-    lines = [l.strip() for l in asm_text.splitlines()]
-    lines = [l for l in lines if l and not l.startswith(";") and not l.startswith(".") and not l.endswith(":")]
+    """Returns (number of MFMAs, list of (writer, mfma) pairs that are too close).
+
+    The two wait states in front of an MFMA are looked for along every path into it: the fall-through path
+    and, where a label lies within them, the instructions in front of every branch to that label (a loop's
+    back edge puts the end of the body in front of its head)."""
+    raw = [l.strip() for l in asm_text.splitlines()]
+    lines, labels = [], {}
+    for l in raw:
+        if not l or l.startswith(";") or l.startswith("//"):
+            continue
+        l = l.split(";")[0].strip()
+        if l.endswith(":"):
+            labels.setdefault(l[:-1], len(lines))          # the label stands in front of instruction len(lines)
+            continue
+        if l.startswith("."):
+            continue
+        lines.append(l)
+    jumps = {}                                             # instruction index of a label -> branches to it
+    for i, l in enumerate(lines):
+        if l.startswith("s_cbranch") or l.startswith("s_branch"):
+            t = l.split()[-1]
+            if t in labels:
+                jumps.setdefault(labels[t], []).append(i)
     found, n = [], 0
+
+    def walk(j, states, src, mfma, seen):
+        # instruction j and those in front of it, until two wait states are counted
+        while j >= 0 and states < 2:
+            if j + 1 in jumps:                             # a label in front of instruction j + 1: its other ways in
+                for b in jumps[j + 1]:
+                    if (b, states) not in seen:
+                        seen.add((b, states))
+                        walk(b, states, src, mfma, seen)
+            p = lines[j]
+            if p.startswith("s_branch"):                   # nothing falls through an unconditional branch
+                return
+            if p.startswith("s_nop"):
+                states += int(p.split()[1]) + 1
+            else:
+                if p.startswith("v_") and not p.startswith("v_mfma"):
+                    if _regs(p.split(None, 1)[1].split(",")[0].strip()) & src:
+                        found.append((p, mfma))
+                states += 2 if p.startswith("v_mfma") else 1
+            j -= 1
+
     for i, l in enumerate(lines):
         if not l.startswith("v_mfma"):
             continue
         n += 1
         ops = [t.strip() for t in l.split(None, 1)[1].split(",")]
         src = _regs(ops[1]) | _regs(ops[2])
-        states, j = 0, i - 1
-        while j >= 0 and states < 2:
-            p = lines[j]
-            if p.startswith("s_nop"):
-                states += int(p.split()[1]) + 1
-            else:
-                if p.startswith("v_") and not p.startswith("v_mfma"):
-                    if _regs(p.split(None, 1)[1].split(",")[0].strip()) & src:
-                        found.append((p, l))
-                states += 2 if p.startswith("v_mfma") else 1
-            j -= 1
+        seen = set()
+        if i in jumps:                                     # the MFMA is itself a branch target
+            for b in jumps[i]:
+                seen.add((b, 0))
+                walk(b, 0, src, l, seen)
+        walk(i - 1, 0, src, l, seen)
     return n, found
 
 

@@ -1973,14 +1973,10 @@ constexpr int QMM_STATIC_MAX_DEVICES = 64;
 std::mutex g_static_mutex;
 void *g_static_ptr[QMM_STATIC_MAX_DEVICES] = {};
 
-__global__ __launch_bounds__(256) void qmm_static_clear_kernel(uint32_t *p, int n) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i < n) p[i] = 0u;
-}
-
-// Address of the current device's copy of the array; on the first call on a device also clears the
-// arrival counters at its start (a fill kernel on the caller's stream, ahead of the product).
-int qmm_static_base(hipStream_t st, void **base) {
+// Address of the current device's copy of the array (looked up once per device).  Nothing has to be cleared: the
+// array is zero when the library is loaded, and every product leaves the arrival counters and the 64-bit cells at
+// its head as it found them.
+int qmm_static_base(void **base) {
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= QMM_STATIC_MAX_DEVICES) return GPTQ_HIP_EINVAL;
   std::lock_guard<std::mutex> lock(g_static_mutex);
@@ -1990,10 +1986,6 @@ int qmm_static_base(hipStream_t st, void **base) {
       (void)hipGetLastError();
       return GPTQ_HIP_ELAUNCH;
     }
-    const int words = QMM_HEAD_BYTES / 4;
-    hipLaunchKernelGGL(qmm_static_clear_kernel, dim3((words + 255) / 256), dim3(256), 0, st,
-                       reinterpret_cast<uint32_t *>(ptr), words);
-    GPTQ_CHECK_LAUNCH();
     g_static_ptr[dev] = ptr;
   }
   *base = g_static_ptr[dev];
@@ -2012,7 +2004,7 @@ int gptq_hip_qmatmul_static(void *stream, const void *x, int x_dtype, int64_t M,
   if (gptq_hip_qmatmul_workspace_bytes_x(M, R, C, transpose_b, x_dtype) > QMM_STATIC_BYTES)
     return GPTQ_HIP_ETOOBIG;
   void *base = nullptr;
-  const int rc = qmm_static_base(as_stream(stream), &base);
+  const int rc = qmm_static_base(&base);
   if (rc) return rc;
   return gptq_hip_qmatmul(stream, x, x_dtype, M, packed, R, C, zero, scale, zs_dtype, transpose_b, out,
                           base, QMM_STATIC_BYTES);

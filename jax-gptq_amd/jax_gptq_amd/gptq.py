@@ -217,6 +217,48 @@ def quant_matrix_shape(quantized_matrix, bits=None):
 _MAX_BATCHES_PER_CALL = 1024
 
 
+_METADATA = frozenset(("shape", "dtype", "device", "ndim", "is_cuda", "requires_grad", "layout", "names", "grad_fn"))
+_METADATA_CALLS = frozenset(("dim", "size", "stride", "is_contiguous", "numel", "element_size", "nelement",
+                             "storage_offset", "is_floating_point", "ndimension", "get_device"))
+
+
+class _UpperH(torch.Tensor):
+    """The Hessian state between two ``_accumulate_H_step`` calls.  The kernel adds a batch to the upper tiles
+    only; completing the lower triangle costs a pass over the whole matrix, as much as a fifth of a 2048-row batch
+    at K = 4096, so it is put off until something other than the next step looks at the values: any torch
+    function (and ``data_ptr``) completes it first.  Shape and type queries do not."""
+
+    @staticmethod
+    def wrap(t):
+        r = t.as_subclass(_UpperH)
+        r._pending = True
+        return r
+
+    def _complete(self):
+        if getattr(self, "_pending", False):
+            self._pending = False
+            with torch._C.DisableTorchFunctionSubclass():
+                N.check(N.load().gptq_hip_hessian_finalize(_stream(), ctypes.c_void_p(self.data_ptr()),
+                                                           _DT_H[self.dtype], self.shape[0], 1.0), "hessian_finalize")
+
+    @classmethod
+    def __torch_function__(cls, func, types, args=(), kwargs=None):
+        kwargs = kwargs or {}
+        name = getattr(func, "__name__", "")
+        meta = (name in _METADATA_CALLS or
+                (name == "__get__" and getattr(getattr(func, "__self__", None), "__name__", "") in _METADATA))
+        if not meta:
+            for a in list(args) + list(kwargs.values()):
+                if isinstance(a, _UpperH):
+                    a._complete()
+                elif isinstance(a, (list, tuple)):
+                    for b in a:
+                        if isinstance(b, _UpperH):
+                            b._complete()
+        with torch._C.DisableTorchFunctionSubclass():
+            return func(*args, **kwargs)
+
+
 def _accumulate_H_step(H, running_mean, n_samples, batch):
     """One batch of the Hessian accumulation (reference ``gptq.py:57-74``).
 
@@ -224,10 +266,10 @@ def _accumulate_H_step(H, running_mean, n_samples, batch):
     raw second-moment sum ``sum_b X_b^T X_b`` as a full symmetric matrix and ``running_mean`` stays
     zero, so that the reference's closing formula ``H / n + outer(mean, mean)`` (``gptq.py:100-101``)
     yields ``sum X^T X / n``, the matrix ``accumulate_H`` returns.  The kernel adds to the upper
-    tiles; the mirror into the lower triangle is redone after every step, so ``H`` is a valid
-    state whenever the caller looks at it.
+    tiles; the mirror into the lower triangle is made when the caller looks at ``H`` (see ``_UpperH``), not after
+    every step, so ``H`` is a valid state whenever the caller looks at it and a chain of steps pays for one mirror.
     """
-    lib = N.load()
+    N.load()
     batch = _float_dev(batch, keep_fp64=(H.dtype == torch.float64))
     if batch.dim() > 2:
         batch = batch.reshape(-1, batch.shape[-1])
@@ -236,9 +278,11 @@ def _accumulate_H_step(H, running_mean, n_samples, batch):
     if batch.shape[-1] != H.shape[0]:
         raise ValueError("the batch and H disagree on the feature dimension")
     if batch.shape[0] > 0:
-        _hessian_accumulate(H, [batch.contiguous()])
-        N.check(lib.gptq_hip_hessian_finalize(_stream(), _ptr(H), _DT_H[H.dtype], H.shape[0], 1.0),
-                "hessian_finalize")
+        with torch._C.DisableTorchFunctionSubclass():       # (taking H's address must not complete it)
+            _hessian_accumulate(H, [batch.contiguous()])
+        if not isinstance(H, _UpperH):
+            H = _UpperH.wrap(H)
+        H._pending = True
     return H, running_mean, n_samples + batch.shape[0]
 
 

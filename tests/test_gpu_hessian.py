@@ -268,6 +268,49 @@ def test_accumulate_H_step_chain_equals_accumulate_H(G, rows, K, nb, dt):
         assert float((L1 - L2).abs().max()) < 1e-3 * float(L2.abs().max())
 
 
+def test_accumulate_H_step_completes_the_lower_triangle_when_it_is_looked_at(G):
+    """A chain of steps pays for ONE mirror into the lower triangle: the state a step returns completes itself when
+    anything but the next step looks at its values (a torch function, the address handed to a kernel), and shape
+    or type queries do not count as looking."""
+    import torch
+    K, rows = 1024, 256
+    g = torch.Generator(device="cuda").manual_seed(3)
+    xs = [torch.randn((rows, K), device="cuda", generator=g) for _ in range(4)]
+    ref = sum(x.double().T @ x.double() for x in xs)
+
+    def chain():
+        H = torch.zeros((K, K), device="cuda")
+        m, n = torch.zeros(K, device="cuda"), 0
+        for x in xs:
+            H, m, n = G._accumulate_H_step(H, m, n, x)
+        return H, n
+
+    H, n = chain()
+    assert n == 4 * rows and tuple(H.shape) == (K, K) and H.dtype == torch.float32 and H.dim() == 2 and H.is_cuda
+    assert H._pending                                   # nothing above looked at the values
+    full = H.clone()                                    # a torch function: completes first
+    assert not H._pending and type(full) is torch.Tensor
+    assert torch.equal(full, full.T)
+    assert float((full.double() - ref).abs().max()) < 2e-5 * float(ref.abs().max())
+    # the address (what the library's own entry points take) completes as well
+    H2, _ = chain()
+    assert H2._pending
+    H2.data_ptr()
+    assert not H2._pending
+    torch.cuda.synchronize()
+    assert torch.equal(H2.clone(), full)
+    # a further step after a look, and the closing formula and solve on a state nobody looked at
+    H3, n3 = chain()
+    Q1, _ = G.gptq(torch.randn((K, 64), device="cuda", generator=g) * 0.02, None, H=H3 / n3)
+    H4, _ = chain()
+    H4.sum()
+    H4, _, n4 = G._accumulate_H_step(H4, torch.zeros(K, device="cuda"), n, xs[0])
+    assert H4._pending and n4 == 5 * rows
+    ref5 = ref + xs[0].double().T @ xs[0].double()
+    assert float((H4.double() - ref5).abs().max()) < 2e-5 * float(ref5.abs().max())
+    assert torch.equal(H4.clone(), H4.clone().T)
+
+
 def test_accumulate_H_step_takes_3d_and_empty_batches(G):
     import torch
     rng = np.random.default_rng(5)

@@ -38,6 +38,26 @@ def test_scanner_accepts_wait_states_and_mfmas_between(checker):
     assert n == 1 and found == []
 
 
+def test_scanner_follows_a_loop_back_edge(checker):
+    """A vector write of an operand register at the end of a loop body, an MFMA at the loop's head: the two are
+    adjacent across the back edge only."""
+    loop = ["s_mov_b32 s0, 0", ".LBB0_1:", MFMA, "s_add_i32 s0, s0, 1", "s_cmp_lt_i32 s0, 8",
+            "v_pk_fma_f16 v21, v1, s0, v2", "s_cbranch_scc1 .LBB0_1", "s_endpgm"]
+    n, found = checker.scan("\n".join(loop))
+    assert n == 1 and len(found) == 1
+    # wait states at the head of the loop, or an MFMA as the last instruction of the body, clear it
+    ok1 = loop[:2] + ["s_nop 1"] + loop[2:]
+    other = "v_mfma_f32_16x16x32_f16 a[4:7], v[30:33], v[40:43], a[4:7]"
+    ok2 = loop[:6] + [other] + loop[6:]
+    for listing in (ok1, ok2):
+        n, found = checker.scan("\n".join(listing))
+        assert found == [], listing
+    # nothing falls through an unconditional branch: the write in front of it reaches the label's code only
+    skip = ["v_pk_fma_f16 v21, v1, s0, v2", "s_branch .LBB0_2", ".LBB0_3:", MFMA, ".LBB0_2:", "s_endpgm"]
+    n, found = checker.scan("\n".join(skip))
+    assert n == 1 and found == []
+
+
 @pytest.mark.timeout(600)
 def test_compiled_kernels_have_no_operand_hazard(checker):
     assert checker.check(verbose=False) == 0

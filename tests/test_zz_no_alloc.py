@@ -103,3 +103,37 @@ def test_static_entry_refuses_what_does_not_fit():
     # and the entry point still works afterwards
     q = _problem(4, 2, 256, 128, torch.float16, False)
     assert torch.equal(_run(lib, N, q, static=True), _run(lib, N, q, static=False))
+
+
+@pytest.mark.parametrize("M,K,Nc,dt", [(1, 4096, 11008, "float16"), (16, 4096, 11008, "float16"),
+                                        (64, 4096, 4096, "float16"), (4, 4096, 4096, "float32")])
+def test_static_entry_in_a_captured_graph(M, K, Nc, dt):
+    """What the entry point is for: after one eager call of the same shape (the warm-up the header asks for) the call
+    is captured into a HIP graph; every replay, with eager work and new input contents in between, gives bit for bit
+    what gptq_hip_qmatmul gives for the input contents of that moment."""
+    import torch
+    from jax_gptq_amd import _native as N
+    from jax_gptq_amd.gptq import _DT, _ptr
+    import ctypes
+    lib = N.load()
+    p = _problem(21, M, K, Nc, getattr(torch, dt), False)
+    _run(lib, N, p, static=True)                          # warm-up, eager
+    out = torch.full((M, Nc), float("nan"), dtype=p["x"].dtype, device=p["x"].device)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rc = lib.gptq_hip_qmatmul_static(st, _ptr(p["x"]), _DT[p["x"].dtype], M, _ptr(p["packed"]), p["R"], p["C"],
+                                         _ptr(p["zero"]), _ptr(p["scale"]), _DT[p["zero"].dtype], 0, _ptr(out))
+    assert rc == 0
+    g = torch.Generator(device="cuda").manual_seed(5)
+    for rep in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        expect = _run(lib, N, p, static=False)
+        assert torch.equal(out, expect), rep
+        # eager work on the same array and new input contents between the replays
+        _run(lib, N, p, static=True)
+        p["x"].copy_(torch.randn(p["x"].shape, device="cuda", generator=g).to(p["x"].dtype))
+        torch.cuda.synchronize()
