@@ -216,7 +216,14 @@ int gptq_hip_dequant_bits(void *stream, const uint8_t *packed, int64_t outer, in
  * plain kernels (several launches where M exceeds a grid dimension).
  * The workspace begins with arrival counters of the split-K reduction: it must be
  * ZERO-FILLED before its first use; every call leaves the counters zero again, so one
- * buffer can serve any sequence of calls that do not overlap in time. */
+ * buffer can serve any sequence of calls that do not overlap in time.
+ * Range of the split sums: where up to 16 rows (forward) are summed over S > 1 workgroups through the workspace's
+ * 64-bit cells, a workgroup's PARTIAL result enters as a fixed-point number (2^-28 steps): a partial that is
+ * not finite or beyond +-65536 poisons its cell, and that output is NaN.  The reference accumulates in fp32 and
+ * casts to fp16 (kernel.py:111, op.py:43), so it yields +-inf for a result beyond the fp16 range and a finite value
+ * where partial sums of that size cancel; here both cases give NaN.  Results within the fp16 range whose partial sums
+ * stay within +-65536 (every product of fp16-range activations with 4-bit weights of sensible scale) are summed
+ * exactly, in an order-independent way. */
 size_t gptq_hip_qmatmul_workspace_bytes(int64_t M, int64_t R, int64_t C, int transpose_b);
 size_t gptq_hip_qmatmul_workspace_bytes_x(int64_t M, int64_t R, int64_t C, int transpose_b, int x_dtype);
 int gptq_hip_qmatmul(void *stream, const void *x, int x_dtype, int64_t M, const uint8_t *packed,

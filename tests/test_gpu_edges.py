@@ -101,3 +101,36 @@ def test_pack_unpack_maximum_codes_and_odd_axis_error(G):
     with pytest.raises(ValueError):
         G.pack_colwise(np.zeros((5, 4), np.uint8))
     assert to_np(G.pack_colwise(np.zeros((0, 4), np.uint8))).shape == (0, 4)
+
+
+def test_qmatmul_split_sum_range():
+    """The decode path sums the splits of the contraction in 64-bit fixed-point cells: a PARTIAL result beyond
+    +-65536 poisons its cell and the output is NaN, also where the partial sums would cancel (the reference's fp32
+    accumulation would give the finite sum there, and +-inf where the result itself leaves the fp16 range).  Partials
+    just inside the range are summed exactly."""
+    import torch
+    import jax_gptq_amd.gptq as G
+    from jax_gptq_amd.op import quantized_matmul
+    from jax_gptq_amd import _native as N
+    K, C = 4096, 512
+    plan = N.qmatmul_plan(1, K // 2, C)
+    assert plan["kernel"] == "qmm_fwd_dec_kernel" and plan["splits"] > 1
+    pk = torch.full((K // 2, C), 0x88, dtype=torch.uint8, device="cuda")          # every code 8
+    zero = torch.zeros(C, device="cuda")
+    scale = torch.ones(C, device="cuda")
+    qm = G.QuantizedMatrix(pk, zero, scale)
+    # first half of the contraction +v, second half -v: a split's partial is +-8 v times its K / S columns, the sum 0
+    half = K // 2
+    for v, poisoned in ((4.0, False), (64.0, True)):
+        x = torch.cat([torch.full((1, half), v), torch.full((1, half), -v)], dim=1).to(torch.float16).cuda()
+        y = quantized_matmul(x, qm).float()
+        if poisoned:
+            assert 8 * v * (K // plan["splits"]) > 65536 * 0.9
+            assert bool(torch.isnan(y).all())
+        else:
+            assert 8 * v * (K // plan["splits"]) < 65536
+            assert bool((y == 0).all())
+    # a further call on the same (cached) workspace finds clean cells
+    x = torch.ones((1, K), dtype=torch.float16, device="cuda") / 64
+    y = quantized_matmul(x, qm).float()
+    assert bool((y == 8.0 * K / 64).all())
