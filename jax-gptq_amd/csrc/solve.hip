@@ -300,7 +300,9 @@ __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
   auto chain_fast = [&](int r0, int boff) __attribute__((always_inline)) -> bool {
     float xs[SB], e[SB], tmp[SB];
     float qa_s[SB], k_s[SB], kc_s[SB], qh_s[SB], a_s[SB];
-    float fmax_acc = 0.f, qmax_acc = 0.f, amin_acc = 1.0f, amax_acc = 1.0f;
+    int ex_s[SB];
+    float fmax_acc = 0.f, qmax_acc = 0.f, amax_acc = 1.0f;
+    int emin_acc = 0;                  // smallest binary exponent of the non-zero a (frexp's: a = m 2^e, 0.5 <= m < 1)
 #pragma unroll
     for (int t = 0; t < SB; ++t) xs[t] = wcol[(r0 + t) * SOLVE_CH];
     // the i-th instruction that the error of row te owes to the rows te + 2, ... (multiply, then subtract)
@@ -309,15 +311,18 @@ __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
       if ((i & 1) == 0) tmp[i >> 1] = lt[t2 * (t2 + 1) / 2 + te] * e[te];
       else xs[t2] = xs[t2] - tmp[i >> 1];
     };
-    constexpr int NBK = 7;
+    constexpr int NBK = 8;
     auto bk_op = [&](int te, int j) __attribute__((always_inline)) {
       if (j == 0) fmax_acc = fmaxf(fmax_acc, fabsf(qa_s[te] - k_s[te]));
       if (j == 1) qmax_acc = fmaxf(qmax_acc, fabsf(qa_s[te]));
-      if (j == 2) amin_acc = fminf(amin_acc, fabsf(a_s[te]));
-      if (j == 3) amax_acc = fmaxf(amax_acc, fabsf(a_s[te]));
-      if (j == 4) Es[boff + te * SOLVE_CH] = e[te];
-      if (j == 5) Qs[boff + te * SOLVE_CH] = kc_s[te] + z;
-      if (j == 6) QHs[boff + te * SOLVE_CH] = qh_s[te];
+      // (an exact zero has exponent 0 here: it needs none of what the plain division adds, the fast form gives
+      // the same zero; rows of dead features and weights that sit on the grid produce them)
+      if (j == 2) ex_s[te] = __builtin_amdgcn_frexp_expf(a_s[te]);
+      if (j == 3) emin_acc = min(emin_acc, ex_s[te]);
+      if (j == 4) amax_acc = fmaxf(amax_acc, fabsf(a_s[te]));
+      if (j == 5) Es[boff + te * SOLVE_CH] = e[te];
+      if (j == 6) Qs[boff + te * SOLVE_CH] = kc_s[te] + z;
+      if (j == 7) QHs[boff + te * SOLVE_CH] = qh_s[te];
     };
     static_for<SB>([&](auto tc) __attribute__((always_inline)) {
       constexpr int t = decltype(tc)::value;
@@ -373,7 +378,7 @@ __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
     for (int j = 0; j < NBK; ++j) bk_op(SB - 1, j);
     bool redo = z_plain;
     redo |= !(fmax_acc <= 0.5f - 0x1p-21f * fmaxf(qmax_acc, 1.0f));
-    redo |= !(amin_acc >= 0x1p-40f && amax_acc <= 0x1p40f);
+    redo |= !(emin_acc >= -39 && amax_acc <= 0x1p40f);
     redo |= !(e[SB - 1] == e[SB - 1]);
     return redo;
   };
