@@ -358,6 +358,9 @@ def main():
                     help="--section hessian only: fp32 rows as pairs of fp16 numbers (accumulate_H(split_fp16=True))")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-qmatmul", action="store_true", help="skip the int4 matmul section")
+    ap.add_argument("--no-streamed", action="store_true",
+                    help="skip the one-call-per-batch Hessian section (a kernel trace of the run then holds "
+                         "syrk32d_kernel's one-launch-per-layer calls only)")
     ap.add_argument("--section", default="all", choices=["all", "hessian", "factor", "solve", "qmatmul", "copy"],
                     help="profiling aid: run only one part (hessian: X^T X over the 128 batches; factor: damping + "
                          "Cholesky factor of the inverse of a K = 4096 Hessian; solve: the blocked column loop of the "
@@ -516,7 +519,7 @@ def main():
                                       "frac": m1["hbm_frac"], "traffic": qmatmul_traffic_bytes()}
         # the practical ceiling: a kernel that only reads, at the same sizes
         result["hbm_read_ceiling"] = bench_read_ceiling()
-    if args.section == "all":
+    if args.section == "all" and not args.no_streamed:
         result["hessian_streamed"] = bench_hessian_streamed(G, xs)
     if not args.no_cpu:
         packed_gpu, params_gpu = one_layer(G, W, xs)
