@@ -1018,6 +1018,15 @@ constexpr int D32_OP = D32_BK * D32_ROW;
 constexpr int D32_SLAB = 2 * D32_OP;
 constexpr int D32_LDS_BYTES = D32_NBUF * D32_SLAB;
 
+//
+// PIECES: the short call (one batch per call, the reference's streaming use, gptq.py:97-98).  With row slices
+// the 136 tiles of K = 4096 times RS never come close to a multiple of the 256 CUs unless RS is large, and every
+// workgroup pays its pipeline fill and 256 KB of partial tile.  Here the (tile, slab) pairs of the call, tile
+// major, are cut into gridDim.x equal runs, one per workgroup: a workgroup works through the end of one tile,
+// whole tiles (added to H directly) and the beginning of another, so it writes at most two partial tiles
+// (slots 2 w and 2 w + 1 of the workspace), which syrk_reduce_pieces_kernel sums in workgroup order.
+// p.chunk holds the slabs per tile (rows of the call / 16).
+template <bool PIECES>
 __global__ __launch_bounds__(256) void syrk32d_kernel(SyrkArgs p) {
   extern __shared__ __attribute__((aligned(16))) char lds32d[];
   typedef __attribute__((address_space(3))) char lds_char;
@@ -1030,17 +1039,42 @@ __global__ __launch_bounds__(256) void syrk32d_kernel(SyrkArgs p) {
       item = ((q >> 5) * 8u + xcd) * 32u + (q & 31u);
     }
   }
-  const int rs = (int)item / ntiles, t = (int)item - rs * ntiles;
-  int ti, tj;
-  tile_decode(t, p.T, ti, tj);
-  const int m0 = ti * W16_TB, n0 = tj * W16_TB, K = p.K;
+  const int K = p.K;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
+  // PIECES: this workgroup's run [u0, u1) of the tile-major (tile, slab) pairs
+  int64_t u0 = 0, u1 = 0;
+  if (PIECES) {
+    const int64_t U = (int64_t)ntiles * p.chunk;
+    u0 = (int64_t)item * U / gridDim.x;
+    u1 = (int64_t)(item + 1) * U / gridDim.x;
+    if (u0 >= u1) return;
+  }
+  bool first_piece = true;
+  do {
+  int rs = 0, t, piece_rows = p.chunk;
+  int64_t g0;
+  bool whole = false;
+  if (PIECES) {
+    t = (int)(u0 / p.chunk);
+    const int s0 = (int)(u0 - (int64_t)t * p.chunk);
+    const int n = (int)min((int64_t)(p.chunk - s0), u1 - u0);
+    g0 = (int64_t)s0 * D32_BK;
+    piece_rows = n * D32_BK;
+    whole = n == p.chunk;
+    u0 += n;
+  } else {
+    rs = (int)item / ntiles;
+    t = (int)item - rs * ntiles;
+    g0 = (int64_t)rs * p.chunk;
+  }
+  int ti, tj;
+  tile_decode(t, p.T, ti, tj);
+  const int m0 = ti * W16_TB, n0 = tj * W16_TB;
 
-  // slice [g0, g0 + chunk) of the concatenated batches: first slab (b, kt), number of slabs
+  // rows [g0, g0 + piece_rows) of the concatenated batches: first slab (b, kt), number of slabs
   int b = 0, kt = 0, nslabs = 0;
   {
-    const int64_t g0 = (int64_t)rs * p.chunk;
     int64_t base = 0;
     bool started = false;
     int rem = 0;
@@ -1050,7 +1084,7 @@ __global__ __launch_bounds__(256) void syrk32d_kernel(SyrkArgs p) {
         started = true;
         b = bb;
         kt = (int)(g0 - base);
-        rem = p.chunk;
+        rem = piece_rows;
       }
       if (started && rem > 0) {
         const int from = (bb == b) ? kt : 0;
@@ -1172,31 +1206,105 @@ __global__ __launch_bounds__(256) void syrk32d_kernel(SyrkArgs p) {
     mfma_all(prev);          // last k pair of the last slab
   }
 
-  if (p.RS == 1) {
+  // (PIECES: the element offsets below do not change from piece to piece; left visible, the compiler computes
+  // all 512 of them in front of the loop and parks them in scratch memory, and a kernel with that much scratch
+  // pays for its allocation at every launch)
+  int e_col = wn * 128 + l32, e_row = wm * 128 + 4 * lhi;
+  if (PIECES) asm volatile("" : "+v"(e_col), "+v"(e_row));
+  if (PIECES ? whole : p.RS == 1) {
 #pragma unroll
     for (int ii = 0; ii < 4; ++ii)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int col = n0 + wn * 128 + j * 32 + l32;
+        const int col = n0 + e_col + j * 32;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int row = m0 + wm * 128 + ii * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+          const int row = m0 + e_row + ii * 32 + 8 * (r >> 2) + (r & 3);
           p.H[(int64_t)row * K + col] += acc[ii][j][r];
         }
       }
+  } else if (PIECES) {
+    // a partial tile is the workgroup's first piece (slot 2 w) or, whole tiles in between, its last.  It is
+    // stored in register order (16 bytes per lane, 1 KB per store instruction: float4 number
+    // ((wave * 16 + ii * 4 + j) * 4 + r / 4) * 64 + lane), which is the order syrk_reduce_pieces_kernel sums in.
+    float4 *dst = reinterpret_cast<float4 *>(p.ws + (int64_t)(2 * item + (first_piece ? 0 : 1)) * (W16_TB * W16_TB)) +
+                  wave * 4096 + lane;
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq)
+          dst[((ii * 4 + j) * 4 + rq) * 64] =
+              make_float4(acc[ii][j][4 * rq], acc[ii][j][4 * rq + 1], acc[ii][j][4 * rq + 2], acc[ii][j][4 * rq + 3]);
   } else {
     float *dst = p.ws + ((int64_t)rs * ntiles + t) * (W16_TB * W16_TB);
 #pragma unroll
     for (int ii = 0; ii < 4; ++ii)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int col = wn * 128 + j * 32 + l32;
+        const int col = e_col + j * 32;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int row = wm * 128 + ii * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+          const int row = e_row + ii * 32 + 8 * (r >> 2) + (r & 3);
           dst[row * W16_TB + col] = acc[ii][j][r];
         }
       }
+  }
+  if (!PIECES) break;
+  first_piece = false;
+  __syncthreads();           // the next piece's loads reuse the slab buffers
+  } while (u0 < u1);
+}
+
+// PIECES form of the reduction: the partial tiles of tile t lie in the slots of the workgroups whose runs cut it
+// (see syrk32d_kernel); H tile += their sum in workgroup order.  A tile that one workgroup covered alone has
+// been added already.  G workgroups, S slabs per tile.
+__global__ __launch_bounds__(256) void syrk_reduce_pieces_kernel(float *H, const float *ws, int K, int T, int S, int G) {
+  constexpr int TB = W16_TB, RED_PARTS = TB * TB / 4096;
+  const int ntiles = T * (T + 1) / 2;
+  const int t = blockIdx.x / RED_PARTS, part = blockIdx.x % RED_PARTS;
+  const int64_t U = (int64_t)ntiles * S, lo = (int64_t)t * S, hi = lo + S;
+  // first workgroup whose run [w U / G, (w + 1) U / G) reaches into [lo, hi)
+  int w = (int)(lo * G / U);
+  while (w > 0 && (int64_t)w * U / G > lo) --w;
+  while ((int64_t)(w + 1) * U / G <= lo) ++w;
+  if ((int64_t)w * U / G <= lo && (int64_t)(w + 1) * U / G >= hi) return;     // whole tile, one workgroup
+  int ti, tj;
+  tile_decode(t, T, ti, tj);
+  const int m0 = ti * TB, n0 = tj * TB;
+  // float4 number e of a partial tile holds rows r .. r + 3 of one column (the kernel's register order)
+  float4 s[4], h[4];
+  int e[4];
+  float *hp[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    e[u] = part * 1024 + u * 256 + threadIdx.x;
+    s[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    const int lane = e[u] & 63, rq = (e[u] >> 6) & 3, j = (e[u] >> 8) & 3, ii = (e[u] >> 10) & 3, wv = e[u] >> 12;
+    const int row = (wv >> 1) * 128 + ii * 32 + 8 * rq + 4 * (lane >> 5), col = (wv & 1) * 128 + j * 32 + (lane & 31);
+    hp[u] = H + (int64_t)(m0 + row) * K + n0 + col;
+    h[u] = make_float4(hp[u][0], hp[u][K], hp[u][2 * (int64_t)K], hp[u][3 * (int64_t)K]);
+  }
+  for (; w < G && (int64_t)w * U / G < hi; ++w) {
+    const int64_t a = (int64_t)w * U / G;
+    if ((int64_t)(w + 1) * U / G <= a) continue;      // an empty run wrote nothing
+    const bool first = a >= lo;                       // the run starts inside this tile: its first piece
+    const float4 *src = reinterpret_cast<const float4 *>(ws) + (int64_t)(2 * w + (first ? 0 : 1)) * (TB * TB / 4);
+    float4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = src[e[u]];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      s[u].x += v[u].x; s[u].y += v[u].y; s[u].z += v[u].z; s[u].w += v[u].w;
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    hp[u][0] = h[u].x + s[u].x;
+    hp[u][K] = h[u].y + s[u].y;
+    hp[u][2 * (int64_t)K] = h[u].z + s[u].z;
+    hp[u][3 * (int64_t)K] = h[u].w + s[u].w;
   }
 }
 
@@ -1307,6 +1415,24 @@ int pick_rs_call(int64_t K, int64_t total_rows, int slab_rows, double us_per_row
   return best;
 }
 constexpr double H_US_PER_ROW_F32 = 0.228, H_US_PER_ROW_16 = 0.0305;
+
+// The (tile, slab) runs of syrk32d_kernel<true>: G workgroups (one round), two partial-tile slots each.  A run is
+// one chain of MFMA accumulations, so the call may not be longer than H_CHAIN_ROWS rows (see
+// gptq_hip_hessian_accumulate); runs shorter than eight slabs are not worth their pipeline fill.
+struct PiecesPlan { bool use; int G; size_t ws_bytes; };
+PiecesPlan pieces_plan(int64_t K, int64_t total_rows) {
+  PiecesPlan pp{false, 0, 0};
+  if (!use_wide16(K) || K % W16_TB != 0 || total_rows <= 0 || total_rows % D32_BK != 0 || total_rows > H_CHAIN_ROWS)
+    return pp;
+  const int64_t T = K / W16_TB, nt = T * (T + 1) / 2, U = nt * (total_rows / D32_BK);
+  int64_t G = U / 8;
+  if (G > 256) G = 256;
+  if (G < 1) return pp;
+  pp.use = true;
+  pp.G = (int)G;
+  pp.ws_bytes = (size_t)(2 * G) * W16_TB * W16_TB * sizeof(float);
+  return pp;
+}
 
 // ---------------------------------------------------------------------------- fp32 rows on the 16-bit matrix cores
 // Opt-in path for fp32 calibration rows: x = (hi + lo) * 2^e with hi = fp16(x 2^-e), lo =
@@ -1450,6 +1576,8 @@ size_t gptq_hip_hessian_accumulate_workspace_bytes(int64_t K, int h_dtype) {
     const int64_t Tw = ceil_div64(K, W16_TB), nw = Tw * (Tw + 1) / 2;
     const size_t wide = rw == 1 ? 0 : (size_t)rw * nw * W16_TB * W16_TB * sizeof(float);
     if (wide > need) need = wide;
+    const size_t pieces = (size_t)512 * W16_TB * W16_TB * sizeof(float);     // pieces_plan: two slots x 256 workgroups
+    if (pieces > need) need = pieces;
   }
   return need;
 }
@@ -1618,9 +1746,27 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
       const int64_t chunk = round_up64(ceil_div64(total_rows, w.RS), D32_BK);
       if (chunk > 2147483647LL) return GPTQ_HIP_EINVAL;
       w.chunk = (int)chunk;
-      if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(syrk32d_kernel), D32_LDS_BYTES))
+      // a short call: equal runs of (tile, slab) pairs over one round of workgroups instead of row slices,
+      // where the model says so (time of a run + what the two partial tiles per workgroup cost)
+      const PiecesPlan pp = pieces_plan(K, total_rows);
+      if (pp.use && ws && ws_bytes >= pp.ws_bytes) {
+        const double sliced = (double)ceil_div64(nt * w.RS, 256) * (H_US_PER_ROW_F32 * (double)chunk + 30.0);
+        const double pieces = H_US_PER_ROW_F32 * (double)total_rows * (double)nt / (double)pp.G + 50.0;
+        if (pieces < 0.9 * sliced) {
+          if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(syrk32d_kernel<true>), D32_LDS_BYTES))
+            return GPTQ_HIP_ELAUNCH;
+          w.chunk = (int)slabs;
+          hipLaunchKernelGGL(syrk32d_kernel<true>, dim3((unsigned)pp.G), block, D32_LDS_BYTES, st, w);
+          GPTQ_CHECK_LAUNCH();
+          hipLaunchKernelGGL(syrk_reduce_pieces_kernel, dim3((unsigned)(nt * (W16_TB * W16_TB / 4096))), dim3(256), 0, st, H,
+                             w.ws, (int)K, w.T, (int)slabs, pp.G);
+          GPTQ_CHECK_LAUNCH();
+          continue;
+        }
+      }
+      if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(syrk32d_kernel<false>), D32_LDS_BYTES))
         return GPTQ_HIP_ELAUNCH;
-      hipLaunchKernelGGL(syrk32d_kernel, dim3((unsigned)(nt * w.RS)), block, D32_LDS_BYTES, st, w);
+      hipLaunchKernelGGL(syrk32d_kernel<false>, dim3((unsigned)(nt * w.RS)), block, D32_LDS_BYTES, st, w);
       GPTQ_CHECK_LAUNCH();
       if (w.RS > 1) {
         hipLaunchKernelGGL(syrk_reduce_kernel<W16_TB>, dim3((unsigned)(nt * (W16_TB * W16_TB / 4096))), dim3(256), 0, st, H, w.ws,

@@ -230,6 +230,36 @@ def test_accumulate_H_fp32_wide_tile_kernel(G, rows, K, nb):
     assert np.abs(H2 - ref2).max() < TOL * max(1.0, np.abs(ref2).max())
 
 
+@pytest.mark.parametrize("rows,K,nb", [(2048, 4096, 1), (2048, 6144, 1), (16, 1024, 1), (32, 1024, 1), (160, 2048, 3),
+                                       (1024, 1024, 2), (2048, 11008, 1), (4096, 4096, 2), (2064, 4096, 1)])
+def test_accumulate_H_short_calls_in_equal_runs_of_tile_slabs(G, rows, K, nb):
+    """A short call (the reference's one call per batch, gptq.py:97-98) is dealt to one round of workgroups as
+    equal runs of (tile, 16-row slab) pairs: a run ends one tile, covers whole tiles and begins another.  Cases:
+    136 tiles on 256 workgroups (every tile cut), 300 and 946 tiles (whole tiles inside the runs), fewer pairs than
+    workgroups (one workgroup per few tiles), several batches per call, rows that are no multiple of the runs.
+    Against the closed form in double, symmetric, the same bits on a second call, and a second call ADDS."""
+    import torch
+    rng = np.random.default_rng(rows + K + nb)
+    xs = [rng.standard_normal((rows, K)).astype(np.float32) for _ in range(nb)]
+    for x in xs:
+        x[:, 5] = 0.0
+    dev = [torch.from_numpy(x).cuda() for x in xs]
+    H = to_np(G.accumulate_H(dev))
+    ref = _closed_form(xs)
+    assert H.shape == (K, K) and np.array_equal(H, H.T)
+    assert np.abs(H - ref).max() < TOL * max(1.0, np.abs(ref).max())
+    assert np.all(H[5] == 0) and np.all(H[:, 5] == 0)
+    assert np.array_equal(H, to_np(G.accumulate_H(dev)))
+    # two steps of the chain over the same rows: twice the sums over twice the rows
+    Hs = torch.zeros((K, K), dtype=torch.float32, device="cuda")
+    mean = torch.zeros((K,), dtype=torch.float32, device="cuda")
+    Hs, mean, n = G._accumulate_H_step(Hs, mean, 0, dev[0])
+    Hs, mean, n = G._accumulate_H_step(Hs, mean, n, dev[0])
+    assert n == 2 * rows
+    ref1 = _closed_form(xs[:1])
+    assert np.abs(to_np(Hs) / n - ref1).max() < TOL * max(1.0, np.abs(ref1).max())
+
+
 @pytest.mark.parametrize("rows,K,nb,dt", [(64, 384, 5, "float32"), (37, 200, 4, "float32"), (256, 1024, 6, "float32"),
                                           (2048, 4096, 3, "float32"), (96, 1280, 4, "float16"),
                                           (50, 520, 3, "bfloat16")])
