@@ -94,7 +94,8 @@ int gptq_hip_hessian_accumulate_split16(void *stream, const void *const *x_ptrs,
  * passing the whole calibration set at once is the fast path; one batch per call
  * reproduces the reference's streaming use.  The running mean of the reference cancels
  * algebraically (H = sum X^T X / n), so none is kept.
- * ws: gptq_hip_hessian_accumulate_workspace_bytes(K, h_dtype) bytes (0 for large K and for fp64).
+ * ws: gptq_hip_hessian_accumulate_workspace_bytes(K, h_dtype) bytes (0 for fp64; partial tiles of the row slices
+ * of a long call or of the equal runs of (tile, row slab) pairs that a call of up to 32768 fp32 rows is cut into).
  * gptq_hip_hessian_finalize multiplies by 1/n_samples and mirrors the upper
  * triangle into the lower one, giving the full symmetric H the reference returns.
  * Limits: K <= 46000 (one launch's table of tiles), a call's batches at most 2^31 rows in all;

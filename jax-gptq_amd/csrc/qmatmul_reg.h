@@ -31,6 +31,7 @@ RegPlan reg_fwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned);
 struct RegParts {
   int64_t wide_x;
   bool half;
+  int64_t wide2_x;         // 8-bit codes: 256-channel tiles behind the whole rounds of 512-channel ones (part of `first`)
   int64_t first, main_x, tail;
 };
 RegParts reg_fwd_parts(const RegPlan &p, int64_t M, int64_t R, int64_t C, bool bf16, int group_size);
@@ -56,14 +57,15 @@ MidPlan mid_fwd_plan(int64_t M, int64_t R, int64_t C, bool aligned);
 int mid_fwd_launch(hipStream_t st, const MidPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
                    const void *zero, const void *scale, int zs_dtype, void *out, void *ws);
 
-// 128 x 512 tiles for many rows (qmatmul_wide.hip; 4-bit codes, per-channel parameters, aligned operands):
+// 128 x 512 tiles for many rows (qmatmul_wide.hip; 4-bit codes, or 8-bit codes with fp16 rows; per-channel
+// parameters, aligned operands):
 // number of leading 512-channel tiles they take (0: none; *half: tiles of 256 channels, four wavefronts of 64 x 128,
 // for shapes whose 512-channel tiles are under one round), and the launch over those tiles.  out32 / rowexp as in
 // RegPlan.
-int64_t wide_fwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half);
+int64_t wide_fwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half, int bits = 4);
 int wide_fwd_launch(hipStream_t st, const void *x, int x_dtype, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
                     const void *zero, const void *scale, int zs_dtype, void *out, int64_t wide_x, bool half, float *out32,
-                    const int32_t *rowexp);
+                    const int32_t *rowexp, int bits = 4, int64_t c0 = 0);
 
 // The same for the transposed product (fp16 rows): leading tiles of 512 output columns = 256 packed rows (*half: of 256
 // output columns = 128 packed rows).

@@ -541,7 +541,12 @@ int launch_bx(hipStream_t st, const RegPlan &p, const void *x, int64_t M, const 
     const RegParts q = reg_fwd_parts(p, M, R, C, Act<TX>::BF, group_size);
     if (q.wide_x > 0) {
       const int rc = wide_fwd_launch(st, x, Act<TX>::BF ? GPTQ_HIP_BF16 : GPTQ_HIP_F16, M, pk, R, C, zero, scale,
-                                     zs_dtype, out, q.wide_x, q.half, p.out32, p.rowexp);
+                                     zs_dtype, out, q.wide_x, q.half, p.out32, p.rowexp, BITS);
+      if (rc) return rc;
+    }
+    if (q.wide2_x > 0) {
+      const int rc = wide_fwd_launch(st, x, GPTQ_HIP_F16, M, pk, R, C, zero, scale, zs_dtype, out, q.wide2_x, true,
+                                     p.out32, p.rowexp, BITS, 512 * q.wide_x);
       if (rc) return rc;
     }
     if (q.main_x > 0) {
@@ -572,7 +577,6 @@ int launch_bx(hipStream_t st, const RegPlan &p, const void *x, int64_t M, const 
 namespace qmm {
 
 RegParts reg_fwd_parts(const RegPlan &p, int64_t M, int64_t R, int64_t C, bool bf16, int group_size) {
-  (void)bf16;
   RegParts q{};
   const int64_t tiles_all = ceil_div64(C, RG_BN);
   if (p.rb != 8 || group_size > 0) {
@@ -581,9 +585,18 @@ RegParts reg_fwd_parts(const RegPlan &p, int64_t M, int64_t R, int64_t C, bool b
   }
   const int64_t tiles_y = ceil_div64(M, 128), K = p.bits == 4 ? 2 * R : R;
   // 128 x 512 tiles (qmatmul_wide.hip) on the leading columns that fill whole rounds of workgroups
-  if (p.bits == 4 && !p.ragged && p.S == 1) {
-    q.wide_x = wide_fwd_tiles(M, R, C, true, &q.half);
+  if ((p.bits == 4 || !bf16) && !p.ragged && p.S == 1) {
+    q.wide_x = wide_fwd_tiles(M, R, C, true, &q.half, p.bits);
     if (q.wide_x > 0) q.first = (q.half ? 2 : 4) * q.wide_x;
+    // 8-bit codes: the 128-row tiles run them at 60 % of the wide tiles' rate, so what is left behind whole rounds of
+    // 512-channel tiles goes to 256-channel tiles if those fill half a round or more
+    if (p.bits == 8 && q.wide_x > 0 && !q.half) {
+      const int64_t n2 = (C - 512 * q.wide_x) / 256;
+      if (n2 * tiles_y >= 128 && n2 * tiles_y <= 256) {
+        q.wide2_x = n2;
+        q.first += 2 * n2;
+      }
+    }
   }
   const int64_t rest = tiles_all - q.first;
   if (rest == 0) return q;

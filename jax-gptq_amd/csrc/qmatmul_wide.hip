@@ -29,13 +29,20 @@ using namespace qmm;
 // HALF: a 128 x 256 tile, the four wavefronts as two row halves x two column halves of 64 x 128 each (for shapes
 // whose 128 x 512 tiles are under one round of workgroups): the two wavefronts of a column half build the same
 // weight operands, the two of a row half share their row sums.
-template <int NWV, typename TX, bool HALF = false>
+//
+// BITS = 8 (one code per byte, K = R, fp16 rows): a lane loads 8 bytes of each of its eight rows of a k-step; the
+// bytes of two rows that a byte permute pairs ARE fp16 subnormals {a 2^-24, b 2^-24}, and one packed fma with
+// 2^15 and -rint(zero) 2^-9 yields (code - rint(zero)) 2^-9 exactly: two vector instructions per operand register
+// (three for 4-bit codes); the epilogue multiplies the sums by 512.
+template <int NWV, typename TX, bool HALF = false, int BITS = 4>
 __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, int M, int K, const uint8_t *pk, int C,
                                                                    const void *zero, const void *scale,
                                                                    int zs_dtype, TX *out, int c0, float *out32,
                                                                    const int32_t *rowexp) {
   constexpr bool BF = Act<TX>::BF;
   static_assert(NWV == 4, "the row sums are dealt to four wavefronts");
+  static_assert(BITS == 4 || (BITS == 8 && !BF), "8-bit codes: fp16 rows");
+  constexpr int NRW = BITS == 8 ? 8 : 4;         // packed rows of a lane per k-step
   constexpr int NT = 64 * NWV;
   constexpr int CH = 1024 / NT;                  // 16-byte pieces of a stage per thread
   constexpr int RB = HALF ? 4 : 8;               // row blocks of a wavefront
@@ -61,10 +68,10 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
   // (the lane index within a block is XORed with 4 g ^ 2 h: the eight lanes that write one row's 128 bytes would
   //  otherwise hit the same banks; the reads, which XOR the same value, stay conflict free)
   const int dst0 = ((kc >> 2) * TB + (tid >> 7)) * 64 + 16 * (kc & 3) + (((tid >> 3) & 15) ^ (4 * (kc & 3)) ^ (2 * (kc >> 2)));
-  const uint8_t *wp = pk + (int64_t)(4 * g) * C + col;
+  const uint8_t *wp = pk + (int64_t)(NRW * g) * C + col;
 
   u32x4_t stg[2][CH];
-  uint2 wr[2][2][4];
+  uint2 wr[2][2][NRW];
   u32x4_t aq[2][RB];
   u32x4_t aqr[2][2];                             // row blocks 2 wk, 2 wk + 1 once more, for the row sums
   auto load_a = [&](int p, int s) __attribute__((always_inline)) {
@@ -77,9 +84,9 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
     for (int i = 0; i < CH; ++i) a_lds[slot * (2 * TB * 64) + dst0 + (NT / 128) * 64 * i] = stg[p][i];
   };
   auto load_w = [&](int p, int h, int s) __attribute__((always_inline)) {
-    const uint8_t *q = wp + (int64_t)(32 * min(s, NS - 1) + 16 * h) * C;
+    const uint8_t *q = wp + (int64_t)(8 * NRW * min(s, NS - 1) + 4 * NRW * h) * C;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) wr[p][h][i] = *reinterpret_cast<const uint2 *>(q + (int64_t)i * C);
+    for (int i = 0; i < NRW; ++i) wr[p][h][i] = *reinterpret_cast<const uint2 *>(q + (int64_t)i * C);
   };
   auto read_a = [&](int q, int slot, int h) __attribute__((always_inline)) {
     const int sl = lane ^ (4 * g) ^ (2 * h);
@@ -104,12 +111,13 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
 #pragma unroll
   for (int t8 = 0; t8 < 8; ++t8) {
     const float zi = fminf(fmaxf(rintf(rg_raw_to_f32(zraw0[t8], zs_dtype)), -512.f), 512.f);
-    zc[t8] = BF ? 0u : __builtin_bit_cast(uint32_t, half2_t{(_Float16)(-(1024.f + zi)), (_Float16)(-(64.f + zi))});
+    if (BITS == 8) zc[t8] = __builtin_bit_cast(uint32_t, half2_t{(_Float16)(-zi * 0x1p-9f), (_Float16)(-zi * 0x1p-9f)});
+    else zc[t8] = BF ? 0u : __builtin_bit_cast(uint32_t, half2_t{(_Float16)(-(1024.f + zi)), (_Float16)(-(64.f + zi))});
   }
   uint32_t mask = BF ? 0x000F000Fu : 0x00F0000Fu, cexp = BF ? 0x43004300u : 0x64006400u;
   asm volatile("" : "+s"(mask));
   asm volatile("" : "+v"(cexp));
-  const half2_t unscale = half2_t{(_Float16)1.f, (_Float16)0.0625f};
+  const half2_t unscale = BITS == 8 ? half2_t{(_Float16)32768.f, (_Float16)32768.f} : half2_t{(_Float16)1.f, (_Float16)0.0625f};
   const uint32_t one2 = BF ? 0x3F803F80u : 0x3C003C00u;
   uint4 ones = make_uint4(one2, one2, one2, one2);
   asm volatile("" : "+v"(ones.x), "+v"(ones.y), "+v"(ones.z), "+v"(ones.w));      // kept in registers: not rebuilt in front of an MFMA
@@ -121,8 +129,16 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
     for (int j = 0; j < 8; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   // operand register i of tile t8 (channel 8 l16 + t8): codes of packed row i of the lane's four, see qmatmul_reg.hip
-  auto dq_reg = [&](const uint2 (&w)[4], int t8, int i) __attribute__((always_inline)) -> uint32_t {
+  auto dq_reg = [&](const uint2 (&w)[NRW], int t8, int i) __attribute__((always_inline)) -> uint32_t {
     const uint32_t tb = (uint32_t)(t8 & 3);
+    if constexpr (BITS == 8) {
+      // byte t8 of rows 2 i (even k, low half) and 2 i + 1 (odd k): {a 2^-24, b 2^-24} -> (code - zi) 2^-9
+      const uint32_t sel8 = 0x0c000c00u | tb | ((4u + tb) << 16);
+      const uint32_t pb = t8 < 4 ? __builtin_amdgcn_perm(w[2 * i + 1].x, w[2 * i].x, sel8)
+                                 : __builtin_amdgcn_perm(w[2 * i + 1].y, w[2 * i].y, sel8);
+      const half2_t d = __builtin_bit_cast(half2_t, pb) * unscale + __builtin_bit_cast(half2_t, zc[t8]);
+      return __builtin_bit_cast(uint32_t, d);
+    }
     const uint32_t sel = BF ? (0x0c0c0c00u | tb) : (0x0c000c00u | tb | (tb << 16));
     const uint32_t pb = __builtin_amdgcn_perm(0u, t8 < 4 ? w[i].x : w[i].y, sel);
     if (BF) return (((pb << 12) | pb) & mask) | cexp;                  // {128 + lo, 128 + hi}
@@ -141,7 +157,7 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
   // LDS when the loop is done.
   uint32_t bcarry[4];
   floatx4 rsum[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
-  auto step_pipe = [&](const u32x4_t (&a)[RB], const u32x4_t (&ar)[2], const uint2 (&w)[4], const uint2 (&wn)[4]) __attribute__((always_inline)) {
+  auto step_pipe = [&](const u32x4_t (&a)[RB], const u32x4_t (&ar)[2], const uint2 (&w)[NRW], const uint2 (&wn)[NRW]) __attribute__((always_inline)) {
     uint32_t bc[4] = {bcarry[0], bcarry[1], bcarry[2], bcarry[3]};
 #pragma unroll
     for (int t8 = 0; t8 < 8; ++t8) {
@@ -239,7 +255,8 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
       const float rs = rs4[r];
       TX o[8];
 #pragma unroll
-      for (int t8 = 0; t8 < 8; ++t8) o[t8] = Act<TX>::out(sc[t8] * (acc[rb][t8][r] - zfa[t8] * rs));
+      for (int t8 = 0; t8 < 8; ++t8)
+        o[t8] = Act<TX>::out(sc[t8] * ((BITS == 8 ? 512.f * acc[rb][t8][r] : acc[rb][t8][r]) - zfa[t8] * rs));
       if (out32 != nullptr) {
         // fp32 rows: the fp16 result widened and scaled back by the row's power of two (exact)
         const int e = rowexp[m];
@@ -500,11 +517,11 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   }
 }
 
-template <typename TX>
+template <typename TX, int BITS = 4>
 int launch_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
                 const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32, const int32_t *rowexp,
-                bool half) {
-  const int64_t K = 2 * R;
+                bool half, int64_t c0) {
+  const int64_t K = BITS == 8 ? R : 2 * R;
   int64_t rows_max = ((1LL << 31) - 1) / K;
   if (rows_max > 65535LL * 128) rows_max = 65535LL * 128;
   rows_max -= rows_max % 128;
@@ -513,12 +530,12 @@ int launch_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int
     const int64_t rows = M - r0 < rows_max ? M - r0 : rows_max;
     const dim3 grid((unsigned)wide_x, (unsigned)ceil_div64(rows, 128), 1);
     if (half)
-      hipLaunchKernelGGL((qmm_fwd_wide_kernel<4, TX, true>), grid, dim3(256), 0, st, (const TX *)x + r0 * K, (int)rows,
-                         (int)K, pk, (int)C, zero, scale, zs_dtype, (TX *)out + r0 * C, 0,
+      hipLaunchKernelGGL((qmm_fwd_wide_kernel<4, TX, true, BITS>), grid, dim3(256), 0, st, (const TX *)x + r0 * K, (int)rows,
+                         (int)K, pk, (int)C, zero, scale, zs_dtype, (TX *)out + r0 * C, (int)c0,
                          out32 ? out32 + r0 * C : nullptr, rowexp ? rowexp + r0 : nullptr);
     else
-      hipLaunchKernelGGL((qmm_fwd_wide_kernel<4, TX>), grid, dim3(256), 0, st, (const TX *)x + r0 * K, (int)rows,
-                         (int)K, pk, (int)C, zero, scale, zs_dtype, (TX *)out + r0 * C, 0,
+      hipLaunchKernelGGL((qmm_fwd_wide_kernel<4, TX, false, BITS>), grid, dim3(256), 0, st, (const TX *)x + r0 * K, (int)rows,
+                         (int)K, pk, (int)C, zero, scale, zs_dtype, (TX *)out + r0 * C, (int)c0,
                          out32 ? out32 + r0 * C : nullptr, rowexp ? rowexp + r0 : nullptr);
     GPTQ_CHECK_LAUNCH();
   }
@@ -558,8 +575,8 @@ static int64_t wide_rounds(int64_t full_x, int64_t tiles_y) {
   return wgs >= 224 ? full_x : 0;
 }
 
-int64_t wide_fwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half) {
-  const int64_t K = 2 * R;
+int64_t wide_fwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half, int bits) {
+  const int64_t K = bits == 8 ? R : 2 * R;
   *half = false;
   if (!aligned || K % 64 != 0 || K < 512 || C % 8 != 0 || M < 256) return 0;
   const int64_t tiles_y = ceil_div64(M, 128);
@@ -572,13 +589,17 @@ int64_t wide_fwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half
 
 int wide_fwd_launch(hipStream_t st, const void *x, int x_dtype, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
                     const void *zero, const void *scale, int zs_dtype, void *out, int64_t wide_x, bool half, float *out32,
-                    const int32_t *rowexp) {
+                    const int32_t *rowexp, int bits, int64_t c0) {
   if (zs_dtype != GPTQ_HIP_F32 && zs_dtype != GPTQ_HIP_F16 && zs_dtype != GPTQ_HIP_BF16) return GPTQ_HIP_EDTYPE;
-  if (wide_x < 1 || wide_x * (half ? 256 : 512) > C) return GPTQ_HIP_EINVAL;
+  if (wide_x < 1 || c0 < 0 || c0 % 128 != 0 || c0 + wide_x * (half ? 256 : 512) > C) return GPTQ_HIP_EINVAL;
+  if (bits == 8) {
+    if (x_dtype != GPTQ_HIP_F16) return GPTQ_HIP_EDTYPE;
+    return launch_wide<__half, 8>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half, c0);
+  }
   if (x_dtype == GPTQ_HIP_BF16)
-    return launch_wide<__hip_bfloat16>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half);
+    return launch_wide<__hip_bfloat16>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half, c0);
   if (x_dtype != GPTQ_HIP_F16) return GPTQ_HIP_EDTYPE;
-  return launch_wide<__half>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half);
+  return launch_wide<__half>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half, c0);
 }
 
 int64_t wide_bwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half) {

@@ -53,7 +53,10 @@ def test_workspace_queries_are_pure_host_functions():
     assert lib.gptq_hip_damp_invert_workspace_bytes(4096, _native.F32) >= 3 * kp * kp * 4
     assert lib.gptq_hip_damp_invert_workspace_bytes(4096, _native.F64) >= 3 * kp * kp * 8
     assert lib.gptq_hip_damp_invert_workspace_bytes(100, _native.F32) >= 3 * 128 * 128 * 4
-    assert lib.gptq_hip_hessian_accumulate_workspace_bytes(28672, _native.F32) == 0
+    # K = 28672: so many tiles that no row slices are needed; what is left is the two partial-tile slots for each of
+    # the 256 workgroups of a short call
+    assert lib.gptq_hip_hessian_accumulate_workspace_bytes(28672, _native.F32) == 512 * 256 * 256 * 4
+    assert lib.gptq_hip_hessian_accumulate_workspace_bytes(768, _native.F32) > 0
     assert lib.gptq_hip_hessian_accumulate_workspace_bytes(256, _native.F64) == 0
     assert lib.gptq_hip_solve_workspace_bytes(4096, 11008, 128) == 512 * 11008 * 4      # error rows of a 512-row group
     assert lib.gptq_hip_solve_workspace_bytes(4096, 11008, 129) == 0
