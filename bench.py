@@ -200,6 +200,8 @@ def bench_qmatmul(reps=240):
             # fp32 rows in and out (what a JAX caller of the reference passes by default): rounded to fp16
             # precision on the way in, as the reference's dot rounds them to TF32
             cases += [(1, 0, "float32"), (128, 0, "float32")]
+        if K == N_OUT and bits == 4:
+            cases += [(2048, 1, "bfloat16")]
         if K * N >= (1 << 27):
             cases = [(1, 0, "float16"), (16, 0, "float16"), (2048, 0, "float16"), (2048, 1, "float16")]
         if N % 16:

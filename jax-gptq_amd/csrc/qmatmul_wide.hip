@@ -278,17 +278,30 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
 // channels, in stages of 64, whose activations the four wavefronts share through LDS as above; the weight operand
 // is built as in qmatmul_reg_bwd.hip (lane (l16, g): 8 channels of packed row j0 + 16 jg + l16; scale and
 // -zero * scale of all channels converted once into LDS).  C % 64 == 0, whole 512-column tiles only.
+//
+// bf16 rows: (code - zero) * scale rounded to bf16 would lose precision, so, as in qmatmul_reg_bwd.hip, the scale
+// goes to the other operand, once per workgroup on the way into LDS: A = bf16(x * scale), B = 128 + code (a byte
+// permute under 0x43: 1.75 vector instructions per operand register against fp16's four), and the term
+// t[m] = sum_c A (128 + zero) comes from a ninth MFMA tile whose B operand holds 128 + rint(zero) in its first eight
+// columns and zero - rint(zero) in the others; wavefront wk accumulates it for row blocks 2 wk and 2 wk + 1 only
+// and the four exchange it through LDS at the end, as the forward kernel's row sums.  Tables: scale in fp32 and
+// the offset pair, 8 C bytes (C <= 16384).
 template <typename TX, bool HALF = false>
 __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M, const uint8_t *pk, int R, int C,
                                                                const void *zero, const void *scale, int zs_dtype,
                                                                TX *out, float *out32, const int32_t *rowexp) {
-  static_assert(!Act<TX>::BF, "fp16 rows");
+  constexpr bool BF = Act<TX>::BF;
   // (HALF: 128 rows x 256 output columns, the four wavefronts as two row halves x two column halves, as forward)
   constexpr int RB = HALF ? 4 : 8, TB = 8, NG = 4;
-  extern __shared__ __attribute__((aligned(16))) float wide_lds[];     // halves sc[C], halves nzs[C], then the stages
+  // fp16: halves sc[C], halves nzs[C]; bf16: floats sf[C], words {128 + rint z | z - rint z}[C]; then the stages
+  extern __shared__ __attribute__((aligned(16))) float wide_lds[];
   _Float16 *tab_s = reinterpret_cast<_Float16 *>(wide_lds);
   _Float16 *tab_nz = tab_s + C;
-  u32x4_t *a_lds = reinterpret_cast<u32x4_t *>(wide_lds + C);          // [slot][k-step of the stage][row block][lane]
+  float *tab_sf = wide_lds;
+  uint32_t *tab_zt = reinterpret_cast<uint32_t *>(wide_lds + C);
+  u32x4_t *a_lds = reinterpret_cast<u32x4_t *>(wide_lds + (BF ? 2 : 1) * C);   // [slot][k-step of the stage][row block][lane]
+  typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
+  typedef float f2_t __attribute__((ext_vector_type(2)));
   const int tid = threadIdx.x, lane = tid & 63, wk = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 4, l16 = lane & 15;
   int tx, ty;
@@ -309,6 +322,7 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   u32x4_t stg[2][4];
   uint2 wr[2][2][NG];
   u32x4_t aq[2][RB];
+  u32x4_t aqr[2][2];                             // bf16: row blocks 2 wk, 2 wk + 1 once more, for the ninth tile
   auto load_a = [&](int p, int s) __attribute__((always_inline)) {
     const int so = 64 * min(s, NS - 1);
 #pragma unroll
@@ -317,6 +331,18 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   auto write_a = [&](int p, int slot) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) a_lds[slot * (2 * TB * 64) + dst0 + 2 * 64 * i] = stg[p][i];
+  };
+  // bf16 rows: the pieces of stage s in stg[p] times their channels' scale, rounded to bf16 (register e of piece i
+  // is unit 4 i + e; the units of a stage are spread over the MFMAs of the k-step in front of its write_a)
+  auto scales_of = [&](int s, float (&sf)[8]) __attribute__((always_inline)) {
+    const float *sp = tab_sf + 64 * min(s, NS - 1) + 8 * kc;
+    const float4 f0 = *reinterpret_cast<const float4 *>(sp), f1 = *reinterpret_cast<const float4 *>(sp + 4);
+    sf[0] = f0.x; sf[1] = f0.y; sf[2] = f0.z; sf[3] = f0.w; sf[4] = f1.x; sf[5] = f1.y; sf[6] = f1.z; sf[7] = f1.w;
+  };
+  auto scale_unit = [&](int p, int u, const float (&sf)[8]) __attribute__((always_inline)) {
+    const int i = u >> 2, e = u & 3;
+    stg[p][i][e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f2_t{Act<TX>::lo(stg[p][i][e]) * sf[2 * e],
+                                                                             Act<TX>::hi(stg[p][i][e]) * sf[2 * e + 1]}, bf2_t));
   };
   auto load_w = [&](int p, int h, int s) __attribute__((always_inline)) {
     const int c = 64 * min(s, NS - 1) + 32 * h;
@@ -327,6 +353,10 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
     const int sl = lane ^ (4 * g) ^ (2 * h);                         // (bank swizzle, as in the forward kernel)
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) aq[q][rb] = a_lds[((slot * 2 + h) * TB + rb0 + rb) * 64 + sl];
+    if constexpr (BF) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) aqr[q][j] = a_lds[((slot * 2 + h) * TB + 2 * wk + j) * 64 + sl];
+    }
   };
 
   load_a(1, 0);
@@ -339,8 +369,14 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   // per-channel constants of all channels
   for (int c = tid; c < C; c += 256) {
     const float z = rg_param(zero, zs_dtype, c), sc = rg_param(scale, zs_dtype, c);
-    tab_s[c] = (_Float16)sc;
-    tab_nz[c] = (_Float16)(-z * sc);
+    if constexpr (BF) {
+      const float zi = fminf(fmaxf(rintf(z), -128.f), 128.f);       // 128 + zi: an integer bf16 holds exactly
+      tab_sf[c] = sc;
+      tab_zt[c] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f2_t{128.f + zi, z - zi}, bf2_t));
+    } else {
+      tab_s[c] = (_Float16)sc;
+      tab_nz[c] = (_Float16)(-z * sc);
+    }
   }
 
   floatx4 acc[RB][8];
@@ -350,16 +386,19 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
     for (int j = 0; j < 8; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
   const half2_t k1024 = half2_t{(_Float16)1024.f, (_Float16)1024.f};
   const half2_t k16th = half2_t{(_Float16)0.0625f, (_Float16)0.0625f}, k64 = half2_t{(_Float16)64.f, (_Float16)64.f};
-  uint32_t c64 = 0x64646464u;
-  asm volatile("" : "+v"(c64));
+  uint32_t c64 = 0x64646464u, c43 = 0x43434343u;
+  asm volatile("" : "+v"(c64), "+v"(c43));
+  floatx4 rsum[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
 
   // operand registers of a pair of output columns (low / high nibbles) from word `word` of a packed row: codes of the
   // two channels that `sel` picks, times their scale, minus zero * scale
   auto build_lo = [&](uint32_t word, uint32_t sel, uint32_t scw, uint32_t nzw) __attribute__((always_inline)) -> uint32_t {
+    if constexpr (BF) return __builtin_amdgcn_perm(c43, word & 0x0F0F0F0Fu, sel);      // {128 + code, 128 + code}
     const half2_t cl = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(c64, word & 0x0F0F0F0Fu, sel)) - k1024;
     return __builtin_bit_cast(uint32_t, cl * __builtin_bit_cast(half2_t, scw) + __builtin_bit_cast(half2_t, nzw));
   };
   auto build_hi = [&](uint32_t word, uint32_t sel, uint32_t scw, uint32_t nzw) __attribute__((always_inline)) -> uint32_t {
+    if constexpr (BF) return __builtin_amdgcn_perm(c43, (word >> 4) & 0x0F0F0F0Fu, sel);
     const half2_t ch = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(c64, word & 0xF0F0F0F0u, sel)) * k16th - k64;
     return __builtin_bit_cast(uint32_t, ch * __builtin_bit_cast(half2_t, scw) + __builtin_bit_cast(half2_t, nzw));
   };
@@ -369,13 +408,32 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   // and the MFMA after them counts as a use of the fresh register; so the MFMAs go without wait states, as in the
   // forward kernel.  carry_l / carry_h: the operand registers of the group about to be multiplied.
   uint32_t carry_l[4], carry_h[4];
-  auto compute = [&](const u32x4_t (&a)[RB], const uint2 (&w)[NG], const uint2 &wnext, int c0, int c0n)
-                     __attribute__((always_inline)) {
+  // scp: (bf16 rows) -1, or the stg slot whose pieces, those of stage sst, are scaled under this k-step's MFMAs
+  auto compute = [&](const u32x4_t (&a)[RB], const u32x4_t (&ar)[2], const uint2 (&w)[NG], const uint2 &wnext, int c0,
+                     int c0n, auto scp, int sst) __attribute__((always_inline)) {
+    constexpr int SCP = BF ? decltype(scp)::value : -1;
+    float sf[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if constexpr (SCP >= 0) scales_of(sst, sf);
     const int ti = c0 + 8 * g, tin = min(c0n, C - 32) + 8 * g;
-    const uint4 s4 = *reinterpret_cast<const uint4 *>(tab_s + ti), n4 = *reinterpret_cast<const uint4 *>(tab_nz + ti);
-    const uint4 s4n = *reinterpret_cast<const uint4 *>(tab_s + tin), n4n = *reinterpret_cast<const uint4 *>(tab_nz + tin);
-    const uint32_t sw[4] = {s4.x, s4.y, s4.z, s4.w}, nw[4] = {n4.x, n4.y, n4.z, n4.w};
-    const uint32_t swn[4] = {s4n.x, s4n.y, s4n.z, s4n.w}, nwn[4] = {n4n.x, n4n.y, n4n.z, n4n.w};
+    uint32_t sw[4] = {0u, 0u, 0u, 0u}, nw[4] = {0u, 0u, 0u, 0u}, swn[4] = {0u, 0u, 0u, 0u}, nwn[4] = {0u, 0u, 0u, 0u};
+    uint4 bz = make_uint4(0u, 0u, 0u, 0u);
+    if constexpr (BF) {
+      // the ninth tile's B operand of this k-step: columns < 8 the integer parts, the others the fractions
+      const uint4 z0 = *reinterpret_cast<const uint4 *>(tab_zt + ti), z1 = *reinterpret_cast<const uint4 *>(tab_zt + ti + 4);
+      const uint32_t zsel = l16 < 8 ? 0x05040100u : 0x07060302u;
+      bz = make_uint4(__builtin_amdgcn_perm(z0.y, z0.x, zsel), __builtin_amdgcn_perm(z0.w, z0.z, zsel),
+                      __builtin_amdgcn_perm(z1.y, z1.x, zsel), __builtin_amdgcn_perm(z1.w, z1.z, zsel));
+      // a use here, in front of the k-step's MFMAs: left to the compiler the four permutes sink down to their
+      // first use, the ninth tile's MFMA at the end, which must not follow them directly
+      asm volatile("" ::"v"(bz.x), "v"(bz.y), "v"(bz.z), "v"(bz.w));
+    } else {
+      const uint4 s4 = *reinterpret_cast<const uint4 *>(tab_s + ti), n4 = *reinterpret_cast<const uint4 *>(tab_nz + ti);
+      const uint4 s4n = *reinterpret_cast<const uint4 *>(tab_s + tin), n4n = *reinterpret_cast<const uint4 *>(tab_nz + tin);
+      sw[0] = s4.x; sw[1] = s4.y; sw[2] = s4.z; sw[3] = s4.w;
+      nw[0] = n4.x; nw[1] = n4.y; nw[2] = n4.z; nw[3] = n4.w;
+      swn[0] = s4n.x; swn[1] = s4n.y; swn[2] = s4n.z; swn[3] = s4n.w;
+      nwn[0] = n4n.x; nwn[1] = n4n.y; nwn[2] = n4n.z; nwn[3] = n4n.w;
+    }
     uint32_t bl[4] = {carry_l[0], carry_l[1], carry_l[2], carry_l[3]};
     uint32_t bh[4] = {carry_h[0], carry_h[1], carry_h[2], carry_h[3]};
 #pragma unroll
@@ -401,6 +459,8 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
             piece(n >> 1);
           } else {
             Act<TX>::mma_acc_nw_after(acc[rb][2 * jg + 1], __builtin_bit_cast(uint4, a[rb]), Bh, hi_piece ? nh[i] : nl[i]);
+            if constexpr (SCP >= 0)
+              if ((n & 3) == 1) scale_unit(SCP, 4 * jg + (n >> 2), sf);
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -412,23 +472,27 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
         __builtin_amdgcn_sched_barrier(0);
         Act<TX>::mma_acc_nw_after2(acc[0][2 * jg + 1], __builtin_bit_cast(uint4, a[0]), Bh, nl[0], nh[0]);
         piece(2);
+        if constexpr (SCP >= 0) scale_unit(SCP, 4 * jg, sf);
         __builtin_amdgcn_sched_barrier(0);
         Act<TX>::mma_acc_nw_after(acc[1][2 * jg], __builtin_bit_cast(uint4, a[1]), Bl, nl[1]);
         piece(3);
         __builtin_amdgcn_sched_barrier(0);
         Act<TX>::mma_acc_nw_after(acc[1][2 * jg + 1], __builtin_bit_cast(uint4, a[1]), Bh, nh[1]);
         piece(4);
+        if constexpr (SCP >= 0) scale_unit(SCP, 4 * jg + 1, sf);
         __builtin_amdgcn_sched_barrier(0);
         Act<TX>::mma_acc_nw_after(acc[2][2 * jg], __builtin_bit_cast(uint4, a[2]), Bl, nl[2]);
         piece(5);
         __builtin_amdgcn_sched_barrier(0);
         Act<TX>::mma_acc_nw_after(acc[2][2 * jg + 1], __builtin_bit_cast(uint4, a[2]), Bh, nh[2]);
         piece(6);
+        if constexpr (SCP >= 0) scale_unit(SCP, 4 * jg + 2, sf);
         __builtin_amdgcn_sched_barrier(0);
         Act<TX>::mma_acc_nw_after(acc[3][2 * jg], __builtin_bit_cast(uint4, a[3]), Bl, nl[3]);
         piece(7);
         __builtin_amdgcn_sched_barrier(0);
         Act<TX>::mma_acc_nw_after(acc[3][2 * jg + 1], __builtin_bit_cast(uint4, a[3]), Bh, nh[3]);
+        if constexpr (SCP >= 0) scale_unit(SCP, 4 * jg + 3, sf);
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
@@ -442,14 +506,30 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
       carry_l[i] = bl[i];
       carry_h[i] = bh[i];
     }
+    if constexpr (BF) {
+      Act<TX>::mma_accv_nw(rsum[0], __builtin_bit_cast(uint4, ar[0]), bz);
+      Act<TX>::mma_accv_nw(rsum[1], __builtin_bit_cast(uint4, ar[1]), bz);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
 
+  if constexpr (BF) {
+    __syncthreads();                                                 // the scales are in LDS
+    float sf[8];
+    scales_of(0, sf);
+#pragma unroll
+    for (int u = 0; u < 16; ++u) scale_unit(1, u, sf);
+  }
   write_a(1, 0);
   load_a(1, 2);
   __syncthreads();                                                   // stage 0 and the tables are in LDS
   {
-    const uint4 s4 = *reinterpret_cast<const uint4 *>(tab_s + 8 * g), n4 = *reinterpret_cast<const uint4 *>(tab_nz + 8 * g);
-    const uint32_t sw[4] = {s4.x, s4.y, s4.z, s4.w}, nw[4] = {n4.x, n4.y, n4.z, n4.w};
+    uint32_t sw[4] = {0u, 0u, 0u, 0u}, nw[4] = {0u, 0u, 0u, 0u};
+    if constexpr (!BF) {
+      const uint4 s4 = *reinterpret_cast<const uint4 *>(tab_s + 8 * g), n4 = *reinterpret_cast<const uint4 *>(tab_nz + 8 * g);
+      sw[0] = s4.x; sw[1] = s4.y; sw[2] = s4.z; sw[3] = s4.w;
+      nw[0] = n4.x; nw[1] = n4.y; nw[2] = n4.z; nw[3] = n4.w;
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const uint32_t word = i < 2 ? wr[0][0][0].x : wr[0][0][0].y, sel = (i & 1) ? 0x04030402u : 0x04010400u;
@@ -465,7 +545,7 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
     constexpr int cur = decltype(curc)::value;
     read_a(1, cur, 1);
     __builtin_amdgcn_sched_barrier(0);
-    compute(aq[0], wr[cur][0], wr[cur][1][0], 64 * s, 64 * s + 32);
+    compute(aq[0], aqr[0], wr[cur][0], wr[cur][1][0], 64 * s, 64 * s + 32, std::integral_constant<int, cur>{}, s + 1);
     __builtin_amdgcn_sched_barrier(0);
     load_w(cur, 0, s + 2);
     write_a(cur, cur ^ 1);
@@ -474,7 +554,7 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
     __syncthreads();
     read_a(0, cur ^ 1, 0);
     __builtin_amdgcn_sched_barrier(0);
-    compute(aq[1], wr[cur][1], wr[cur ^ 1][0][0], 64 * s + 32, 64 * s + 64);
+    compute(aq[1], aqr[1], wr[cur][1], wr[cur ^ 1][0][0], 64 * s + 32, 64 * s + 64, std::integral_constant<int, -1>{}, 0);
     __builtin_amdgcn_sched_barrier(0);
     load_w(cur, 1, s + 2);
     __builtin_amdgcn_sched_barrier(0);
@@ -487,10 +567,23 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   if (s < NS) stage(std::integral_constant<int, 0>{}, s);
 
   mma_drain();
-  // acc[rb][2 jg + e][r] = out[m0 + 16 rb + 4 g + r][2 (j0 + 16 jg + l16) + e]
+  // acc[rb][2 jg + e][r] = out[m0 + 16 rb + 4 g + r][2 (j0 + 16 jg + l16) + e]  (bf16: plus t[m], see above)
   const int64_t KO = 2 * (int64_t)R;
+  floatx4 *rs_lds = reinterpret_cast<floatx4 *>(a_lds);                 // [row block][lane]
+  if constexpr (BF) {
+    __syncthreads();                                                   // every wavefront has left the loop
+    rs_lds[(2 * wk) * 64 + lane] = rsum[0];
+    rs_lds[(2 * wk + 1) * 64 + lane] = rsum[1];
+    __syncthreads();
+  }
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
+    floatx4 t4 = floatx4{0.f, 0.f, 0.f, 0.f};
+    if constexpr (BF) {
+      t4 = rs_lds[(rb0 + rb) * 64 + lane];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) t4[r] += __shfl_xor(t4[r], 8);      // integer parts' term + fractions' term
+    }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int m = m0 + 16 * (rb0 + rb) + 4 * g + r;
@@ -510,7 +603,7 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
 #pragma unroll
       for (int jg = 0; jg < NG; ++jg) {
         const int j = j0 + 16 * jg + l16;
-        TX o2[2] = {Act<TX>::out(acc[rb][2 * jg][r]), Act<TX>::out(acc[rb][2 * jg + 1][r])};
+        TX o2[2] = {Act<TX>::out(acc[rb][2 * jg][r] - t4[r]), Act<TX>::out(acc[rb][2 * jg + 1][r] - t4[r])};
         *reinterpret_cast<uint32_t *>(orow + 2 * j) = *reinterpret_cast<const uint32_t *>(o2);
       }
     }
@@ -542,11 +635,13 @@ int launch_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int
   return GPTQ_HIP_OK;
 }
 
+template <typename TX>
 int launch_bwd_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
                     const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32, const int32_t *rowexp,
                     bool half) {
-  auto kern = half ? qmm_bwd_wide_kernel<__half, true> : qmm_bwd_wide_kernel<__half, false>;
-  const int lds = (int)(4 * C + 2 * 2 * 8 * 64 * 16);
+  if (Act<TX>::BF && half) return GPTQ_HIP_EINVAL;                    // (not dispatched, see wide_bwd_tiles)
+  auto kern = (!Act<TX>::BF && half) ? qmm_bwd_wide_kernel<TX, !Act<TX>::BF> : qmm_bwd_wide_kernel<TX, false>;
+  const int lds = (int)((Act<TX>::BF ? 8 : 4) * C + 2 * 2 * 8 * 64 * 16);
   if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), lds)) return GPTQ_HIP_ELAUNCH;
   const int64_t KO = 2 * R;
   int64_t rows_max = ((1LL << 31) - 1) / C;
@@ -556,8 +651,8 @@ int launch_bwd_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk,
   for (int64_t r0 = 0; r0 < M; r0 += rows_max) {
     const int64_t rows = M - r0 < rows_max ? M - r0 : rows_max;
     const dim3 grid((unsigned)wide_x, (unsigned)ceil_div64(rows, 128), 1);
-    hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (const __half *)x + r0 * C, (int)rows, pk, (int)R, (int)C, zero,
-                       scale, zs_dtype, (__half *)out + r0 * KO, out32 ? out32 + r0 * KO : nullptr,
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (const TX *)x + r0 * C, (int)rows, pk, (int)R, (int)C, zero,
+                       scale, zs_dtype, (TX *)out + r0 * KO, out32 ? out32 + r0 * KO : nullptr,
                        rowexp ? rowexp + r0 : nullptr);
     GPTQ_CHECK_LAUNCH();
   }
@@ -602,23 +697,30 @@ int wide_fwd_launch(hipStream_t st, const void *x, int x_dtype, int64_t M, const
   return launch_wide<__half>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half, c0);
 }
 
-int64_t wide_bwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half) {
+int64_t wide_bwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half, bool bf16) {
   *half = false;
-  // (the constants of all channels and the stages share the LDS: 4 C + 32 KB)
-  if (!aligned || C % 64 != 0 || C < 512 || C > 30720 || M < 256) return 0;
+  // (the constants of all channels and the stages share the LDS: 4 C + 32 KB; bf16 rows: 8 C + 32 KB)
+  if (!aligned || C % 64 != 0 || C < 512 || C > (bf16 ? 16384 : 30720) || M < 256) return 0;
   const int64_t tiles_y = ceil_div64(M, 128);
   const int64_t n = wide_rounds(R / 256, tiles_y);
   if (n > 0) return n;
+  // (bf16 rows: the 128 x 256 form, whose wavefronts have half the MFMAs to hide the scaling of the rows behind,
+  // measured slower than the 128-row tiles: 284 against 273 us at M = 2048 on 4096 x 11008)
+  if (bf16) return 0;
   *half = true;
   return wide_rounds(R / 128, tiles_y);
 }
 
 int wide_bwd_launch(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
                     const void *scale, int zs_dtype, void *out, int64_t wide_x, bool half, float *out32,
-                    const int32_t *rowexp) {
+                    const int32_t *rowexp, bool bf16) {
   if (zs_dtype != GPTQ_HIP_F32 && zs_dtype != GPTQ_HIP_F16 && zs_dtype != GPTQ_HIP_BF16) return GPTQ_HIP_EDTYPE;
   if (wide_x < 1 || wide_x * (half ? 128 : 256) > R) return GPTQ_HIP_EINVAL;
-  return launch_bwd_wide(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half);
+  if (bf16) {
+    if (out32 || C > 16384) return GPTQ_HIP_EINVAL;
+    return launch_bwd_wide<__hip_bfloat16>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, nullptr, nullptr, half);
+  }
+  return launch_bwd_wide<__half>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half);
 }
 
 }  // namespace qmm

@@ -237,14 +237,17 @@ def test_qmatmul_few_dozen_rows_tall_narrow_tiles(OP, M, N, K, xdt, zs):
         assert torch.equal(got, first)          # and are summed in split order: the same bits every time
 
 
-@pytest.mark.parametrize("xdt,zs", [("float16", "float32"), ("float16", "float16"), ("float32", "bfloat16")])
+@pytest.mark.parametrize("xdt,zs", [("float16", "float32"), ("float16", "float16"), ("float32", "bfloat16"),
+                                    ("bfloat16", "float32"), ("bfloat16", "bfloat16")])
 @pytest.mark.parametrize("M,N,K", [(3500, 512, 4480), (2048, 1024, 11008), (4096, 576, 4096), (1800, 20480, 8192),
                                    (2000, 1088, 4224)])      # (4224 output columns: 128 x 256 tiles, as forward)
 def test_qmatmul_many_rows_128x512_tiles_transposed(OP, M, N, K, xdt, zs):
     """The transposed product of many fp16 (or fp32) rows on the same tiling: 512 output columns per
     workgroup, contraction along the channels in stages of 64 (N = 576: an odd number of stages;
     N = 20480 channels: more than the other kernel's LDS holds constants for, so its tiles split the
-    contraction while these do not)."""
+    contraction while these do not).  bf16 rows (up to 16384 channels): the scale multiplies the rows on their
+    way into LDS, the weights enter as 128 + code and the term in 128 + zero leaves through a ninth tile that the
+    wavefronts share out (fractional zero points included); 20480 channels stay on the 128-row tiles."""
     import torch
     import jax_gptq_amd.gptq as G
     rng = np.random.default_rng(M + N + K)
@@ -260,7 +263,8 @@ def test_qmatmul_many_rows_128x512_tiles_transposed(OP, M, N, K, xdt, zs):
     dense = (codes.astype(np.float64) - zero.double().numpy()[None]) * scale.double().numpy()[None]
     ref = x.double().numpy() @ dense.T
     err = np.abs(to_np(got).astype(np.float64) - ref)
-    tol = (ATOL + RTOL * np.abs(ref / rowscale)) * rowscale
+    rel = 2.0 ** -8 if xdt == "bfloat16" else RTOL
+    tol = (ATOL + rel * np.abs(ref / rowscale)) * rowscale
     assert np.all(err <= tol), float((err / tol).max())
 
 
