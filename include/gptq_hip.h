@@ -156,6 +156,14 @@ int gptq_hip_process_block(void *stream, const float *Wblock, int64_t N, const f
                            int maxq, void *Qblock, int q_dtype, uint8_t *codes_block,
                            float *errors);
 
+/* The lazy batch update that follows a block (or a group of blocks): replaces
+ *   W = W.at[end:, :].add(-(Hinv[end:, start:end] @ errors))        (gptq.py:204-205).
+ * Wbelow points at W[end][0] ([rows, N], updated in place), Lpanel at L[end][start] (row stride ldl),
+ * errors is [k, N] fp32 as gptq_hip_process_block writes them (k = end - start rows, or the rows of several
+ * consecutive blocks).  fp32 MFMA product, k summed in ascending order within a workgroup's tile. */
+int gptq_hip_lazy_update(void *stream, float *Wbelow, int64_t N, const float *Lpanel, int64_t ldl, const float *errors,
+                         int64_t rows, int64_t k);
+
 /* ---- activation order ---------------------------------------------------------------
  * Replaces the gathers of _permute / _unpermute (gptq.py:170-180); the argsort itself
  * stays with the caller.  out[i, :] = in[perm[i], :] for rows; the symmetric form

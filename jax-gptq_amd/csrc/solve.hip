@@ -552,6 +552,15 @@ int gptq_hip_process_block(void *stream, const float *Wblock, int64_t N, const f
                        Qblock, q_dtype, codes_block, errors);
 }
 
+int gptq_hip_lazy_update(void *stream, float *Wbelow, int64_t N, const float *Lpanel, int64_t ldl, const float *errors,
+                         int64_t rows, int64_t k) {
+  if (rows < 0 || k < 0 || N <= 0 || rows > 2147483647LL || k > 2147483647LL || N > 2147483647LL)
+    return GPTQ_HIP_EINVAL;
+  if (rows == 0 || k == 0) return GPTQ_HIP_OK;
+  if (!Wbelow || !Lpanel || !errors || ldl < k) return GPTQ_HIP_EINVAL;
+  return trailing_update(as_stream(stream), Lpanel, ldl, errors, Wbelow, N, rows, k);
+}
+
 }  // extern "C"
 
 namespace {

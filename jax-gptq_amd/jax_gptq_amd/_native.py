@@ -39,6 +39,7 @@ SIGNATURES = {
     "gptq_hip_solve_workspace_bytes": (_sz, [_i64, _i64, _i32]),
     "gptq_hip_solve": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _i32, _i32, _vp, _i32, _vp, _vp, _sz]),
     "gptq_hip_process_block": (_i32, [_vp, _vp, _i64, _vp, _i64, _i32, _vp, _vp, _i32, _vp, _i32, _vp, _vp]),
+    "gptq_hip_lazy_update": (_i32, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _i64]),
     "gptq_hip_gather_rows": (_i32, [_vp, _vp, _vp, _i32, _i64, _i64, _vp]),
     "gptq_hip_gather_sym": (_i32, [_vp, _vp, _vp, _i32, _i64, _vp]),
     "gptq_hip_pack_int4": (_i32, [_vp, _vp, _i32, _i64, _i64, _i64, _vp]),

@@ -474,6 +474,24 @@ def _process_block(W, Hinv, start, quantize_params, block_size):
     return q, err
 
 
+def _lazy_update(W, Hinv, errors, start, end):
+    """The lazy batch update behind a block or a run of blocks (reference ``gptq.py:204-205``):
+    ``W[end:] -= Hinv[end:, start:end] @ errors`` in place, ``errors`` ``[end - start, N]`` fp32; returns ``W``."""
+    lib = N.load()
+    K, Nc = W.shape
+    if not (0 <= start <= end <= K) or tuple(errors.shape) != (end - start, Nc):
+        raise ValueError("block out of range")
+    if W.dtype != torch.float32 or Hinv.dtype != torch.float32 or errors.dtype != torch.float32 \
+            or not (W.is_contiguous() and Hinv.is_contiguous() and errors.is_contiguous()):
+        raise ValueError("fp32, contiguous operands")
+    if end < K and end > start:
+        below, panel = W[end:], Hinv[end:, start:]
+        N.check(lib.gptq_hip_lazy_update(_stream(), ctypes.c_void_p(below.data_ptr()), Nc,
+                                         ctypes.c_void_p(panel.data_ptr()), Hinv.shape[1], _ptr(errors),
+                                         K - end, end - start), "lazy_update")
+    return W
+
+
 def _solve(W, L, params, block_size, out_dtype, want_codes=False):
     lib = N.load()
     K, Nc = W.shape

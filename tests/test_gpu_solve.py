@@ -241,3 +241,31 @@ def test_gptq_other_code_widths(G, bits):
             G.pack_matrix(Q, p)
     with pytest.raises(ValueError):
         G.gptq(W, [X], bits=9)
+
+
+@pytest.mark.parametrize("K,N,start,k", [(4096, 11008, 0, 512), (4096, 11008, 2560, 512), (4096, 11008, 3072, 512),
+                                         (2048, 8192, 0, 512), (1024, 768, 0, 128), (1536, 4096, 512, 256),
+                                         (4096, 4352, 1024, 512), (1000, 520, 128, 128), (11008, 4096, 512, 512)])
+def test_lazy_update_against_double(K, N, start, k):
+    """The lazy batch update W[end:] -= L[end:, start:end] @ errors (gptq.py:204-205) at the shapes of the column
+    loop, against the product in double: the k = 512 updates of the benchmark layer (3584, 1024 and 512 rows
+    below the group), k = 128 and 256 inside a group, shapes that are no multiple of the tiles.  fp32 products
+    summed in fp32: 1e-5 sqrt(k) of the largest magnitude; the same bits on a second evaluation."""
+    import torch
+    import jax_gptq_amd.gptq as G
+    g = torch.Generator(device="cuda").manual_seed(K + N + start)
+    W = torch.randn((K, N), generator=g, device="cuda")
+    L = torch.tril(torch.randn((K, K), generator=g, device="cuda"))
+    E = torch.randn((k, N), generator=g, device="cuda")
+    end = start + k
+    ref = W.double()
+    ref[end:] -= L[end:, start:end].double() @ E.double()
+    W0 = W.clone()
+    got = G._lazy_update(W, L, E, start, end)
+    assert got.data_ptr() == W.data_ptr()
+    assert torch.equal(got[:end], W0[:end])
+    err = float((got.double() - ref).abs().max())
+    assert err <= 1e-5 * float(ref.abs().max()) * (k ** 0.5), err
+    # the same bits on a second evaluation
+    W2 = G._lazy_update(W0.clone(), L, E, start, end)
+    assert torch.equal(W2, got)
