@@ -1824,7 +1824,8 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
               (parts.main_x > 0 ? parts.main_x : parts.tail) * ty * bp.S);
   };
   if (transpose_b && reg_groups_ok && M > 64) {
-    const RegBwdPlan bp8 = reg_bwd_plan(M, R, C, bits, al, 8);
+    RegBwdPlan bp8 = reg_bwd_plan(M, R, C, bits, al, 8);
+    bp8.no_wide = (reinterpret_cast<uintptr_t>(packed) & 15) != 0;
     const int64_t rounds = bp8.use ? (bp8.tiles + 255) / 256 : 0;
     if (bp8.use && (bp8.tiles <= 256 || bp8.tail_x > 0 || bp8.tiles * 5 >= rounds * 256 * 4)) {
       if (bp8.total_bytes && (!ws || ws_bytes < bp8.total_bytes)) return GPTQ_HIP_EWORKSPACE;

@@ -67,12 +67,13 @@ int wide_fwd_launch(hipStream_t st, const void *x, int x_dtype, int64_t M, const
                     const void *zero, const void *scale, int zs_dtype, void *out, int64_t wide_x, bool half, float *out32,
                     const int32_t *rowexp, int bits = 4, int64_t c0 = 0);
 
-// The same for the transposed product (fp16 rows; bf16 rows up to 16384 channels): leading tiles of 512 output columns = 256 packed rows (*half: of 256
+// The same for the transposed product (fp16 rows; bf16 rows up to 16384 channels; 8-bit codes with fp16 rows:
+// tiles of 512 / 256 output columns = as many packed rows): leading tiles of 512 output columns = 256 packed rows (*half: of 256
 // output columns = 128 packed rows).
-int64_t wide_bwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half, bool bf16 = false);
+int64_t wide_bwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half, bool bf16 = false, int bits = 4);
 int wide_bwd_launch(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
                     const void *scale, int zs_dtype, void *out, int64_t wide_x, bool half, float *out32,
-                    const int32_t *rowexp, bool bf16 = false);
+                    const int32_t *rowexp, bool bf16 = false, int bits = 4);
 
 // Transposed product out[M, K] = x[M, C] @ dequant(packed[R, C])^T.
 struct RegBwdPlan {
@@ -83,6 +84,7 @@ struct RegBwdPlan {
   float *out32;
   const int32_t *rowexp;
   bool ragged;
+  bool no_wide;            // set by the caller when the packed matrix is not 16-byte aligned (the 128 x 512 tiles load 16 bytes)
   int S, steps;
   int64_t tiles;
   size_t part_bytes, total_bytes;

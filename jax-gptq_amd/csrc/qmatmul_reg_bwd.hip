@@ -395,7 +395,7 @@ int launch_bx(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, con
     const RegParts q = reg_bwd_parts(p, M, R, C, Act<TX>::BF, group_size);
     if (q.wide_x > 0) {
       const int rc = wide_bwd_launch(st, x, M, pk, R, C, zero, scale, zs_dtype, out, q.wide_x, q.half, p.out32, p.rowexp,
-                                     Act<TX>::BF);
+                                     Act<TX>::BF, BITS);
       if (rc) return rc;
     }
     if (q.main_x > 0) {
@@ -430,8 +430,8 @@ RegParts reg_bwd_parts(const RegBwdPlan &p, int64_t M, int64_t R, int64_t C, boo
   const int64_t tiles_y = ceil_div64(M, 128);
   // 128 x 512 tiles (qmatmul_wide.hip) on the leading output columns that fill whole rounds of workgroups
   // (also where this kernel's own tiles need a split because the constants of all channels do not fit its LDS)
-  if (p.bits == 4 && !p.ragged && group_size == 0) {
-    q.wide_x = wide_bwd_tiles(M, R, C, true, &q.half, bf16);
+  if ((p.bits == 4 || !bf16) && !p.ragged && !p.no_wide && group_size == 0) {
+    q.wide_x = wide_bwd_tiles(M, R, C, true, &q.half, bf16, p.bits);
     if (q.wide_x > 0) q.first = (q.half ? 2 : 4) * q.wide_x;
   }
   const int64_t rest = tiles_all - q.first;

@@ -286,13 +286,20 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
 // columns and zero - rint(zero) in the others; wavefront wk accumulates it for row blocks 2 wk and 2 wk + 1 only
 // and the four exchange it through LDS at the end, as the forward kernel's row sums.  Tables: scale in fp32 and
 // the offset pair, 8 C bytes (C <= 16384).
-template <typename TX, bool HALF = false>
+//
+// BITS = 8 (one code per byte, fp16 rows): a packed row is one output column, a wavefront's 128 columns are eight
+// groups of 16 rows with one product tile each; the bytes of two channels that a permute pairs are fp16 subnormals
+// {a 2^-24, b 2^-24}, and one packed fma with the channels' scale 2^15 and -zero scale 2^-9 (the tables hold
+// them in that form) yields (code - zero) scale 2^-9: two vector instructions per operand register; the epilogue
+// multiplies by 512.
+template <typename TX, bool HALF = false, int BITS = 4>
 __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M, const uint8_t *pk, int R, int C,
                                                                const void *zero, const void *scale, int zs_dtype,
                                                                TX *out, float *out32, const int32_t *rowexp) {
   constexpr bool BF = Act<TX>::BF;
   // (HALF: 128 rows x 256 output columns, the four wavefronts as two row halves x two column halves, as forward)
-  constexpr int RB = HALF ? 4 : 8, TB = 8, NG = 4;
+  static_assert(BITS == 4 || (BITS == 8 && !BF), "8-bit codes: fp16 rows");
+  constexpr int RB = HALF ? 4 : 8, TB = 8, NG = BITS == 8 ? 8 : 4;
   // fp16: halves sc[C], halves nzs[C]; bf16: floats sf[C], words {128 + rint z | z - rint z}[C]; then the stages
   extern __shared__ __attribute__((aligned(16))) float wide_lds[];
   _Float16 *tab_s = reinterpret_cast<_Float16 *>(wide_lds);
@@ -307,20 +314,25 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   int tx, ty;
   qmm_tile_coords(tx, ty);
   const int rb0 = HALF ? 4 * (wk >> 1) : 0;
-  const int m0 = ty * 128, j0 = (HALF ? tx * 2 + (wk & 1) : tx * 4 + wk) * 64;
+  const int m0 = ty * 128, j0 = (HALF ? tx * 2 + (wk & 1) : tx * 4 + wk) * (16 * NG);
   const int NS = C >> 6;
 
   const int kc = tid & 7;
   int xoff[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) xoff[i] = min(m0 + (tid >> 3) + 32 * i, M - 1) * C + 8 * kc;            // M C < 2^31
-  const int dst0 = ((kc >> 2) * TB + (tid >> 7)) * 64 + 16 * (kc & 3) + (((tid >> 3) & 15) ^ (4 * (kc & 3)) ^ (2 * (kc >> 2)));
+  // Which eight channels of a stage lane group g multiplies in k-step h is free as long as both operands agree:
+  // here they are 16 g + 8 h .. + 7, so that a lane's weights of BOTH k-steps are 16 contiguous bytes of a packed row,
+  // one load per row and stage (the address unit's cost is per instruction, and these loads touch sixteen rows
+  // each).  Chunk kc of the activations (channels 8 kc .. + 7) therefore belongs to k-step kc & 1, lane group kc >> 1.
+  const int kg = kc >> 1, kh = kc & 1;
+  const int dst0 = (kh * TB + (tid >> 7)) * 64 + 16 * kg + (((tid >> 3) & 15) ^ (4 * kg) ^ (2 * kh));
   const uint8_t *wpj[NG];
 #pragma unroll
-  for (int jg = 0; jg < NG; ++jg) wpj[jg] = pk + (int64_t)(j0 + 16 * jg + l16) * C + 8 * g;
+  for (int jg = 0; jg < NG; ++jg) wpj[jg] = pk + (int64_t)(j0 + 16 * jg + l16) * C + 16 * g;
 
   u32x4_t stg[2][4];
-  uint2 wr[2][2][NG];
+  uint4 wr[2][NG];
   u32x4_t aq[2][RB];
   u32x4_t aqr[2][2];                             // bf16: row blocks 2 wk, 2 wk + 1 once more, for the ninth tile
   auto load_a = [&](int p, int s) __attribute__((always_inline)) {
@@ -344,10 +356,15 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
     stg[p][i][e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f2_t{Act<TX>::lo(stg[p][i][e]) * sf[2 * e],
                                                                              Act<TX>::hi(stg[p][i][e]) * sf[2 * e + 1]}, bf2_t));
   };
-  auto load_w = [&](int p, int h, int s) __attribute__((always_inline)) {
-    const int c = 64 * min(s, NS - 1) + 32 * h;
+  auto load_w = [&](int p, int s) __attribute__((always_inline)) {
+    const int c = 64 * min(s, NS - 1);
 #pragma unroll
-    for (int jg = 0; jg < NG; ++jg) wr[p][h][jg] = *reinterpret_cast<const uint2 *>(wpj[jg] + c);
+    for (int jg = 0; jg < NG; ++jg) wr[p][jg] = *reinterpret_cast<const uint4 *>(wpj[jg] + c);
+  };
+  // the weights of k-step h of the stage in slot p
+  auto half_w = [&](int p, int h, uint2 (&w)[NG]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int jg = 0; jg < NG; ++jg) w[jg] = h ? make_uint2(wr[p][jg].z, wr[p][jg].w) : make_uint2(wr[p][jg].x, wr[p][jg].y);
   };
   auto read_a = [&](int q, int slot, int h) __attribute__((always_inline)) {
     const int sl = lane ^ (4 * g) ^ (2 * h);                         // (bank swizzle, as in the forward kernel)
@@ -360,11 +377,9 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   };
 
   load_a(1, 0);
-  load_w(0, 0, 0);
-  load_w(0, 1, 0);
+  load_w(0, 0);
   load_a(0, 1);
-  load_w(1, 0, 1);
-  load_w(1, 1, 1);
+  load_w(1, 1);
   __builtin_amdgcn_sched_barrier(0);
   // per-channel constants of all channels
   for (int c = tid; c < C; c += 256) {
@@ -373,6 +388,9 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
       const float zi = fminf(fmaxf(rintf(z), -128.f), 128.f);       // 128 + zi: an integer bf16 holds exactly
       tab_sf[c] = sc;
       tab_zt[c] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f2_t{128.f + zi, z - zi}, bf2_t));
+    } else if constexpr (BITS == 8) {
+      tab_s[c] = (_Float16)(sc * 32768.f);
+      tab_nz[c] = (_Float16)(-z * sc * 0x1p-9f);
     } else {
       tab_s[c] = (_Float16)sc;
       tab_nz[c] = (_Float16)(-z * sc);
@@ -394,6 +412,11 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   // two channels that `sel` picks, times their scale, minus zero * scale
   auto build_lo = [&](uint32_t word, uint32_t sel, uint32_t scw, uint32_t nzw) __attribute__((always_inline)) -> uint32_t {
     if constexpr (BF) return __builtin_amdgcn_perm(c43, word & 0x0F0F0F0Fu, sel);      // {128 + code, 128 + code}
+    if constexpr (BITS == 8) {
+      // sel pairs bytes (2 e, 2 e + 1) under zero bytes: {a 2^-24, b 2^-24} as fp16 subnormals
+      const half2_t v = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, word, sel | 0x0c000c00u));
+      return __builtin_bit_cast(uint32_t, v * __builtin_bit_cast(half2_t, scw) + __builtin_bit_cast(half2_t, nzw));
+    }
     const half2_t cl = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(c64, word & 0x0F0F0F0Fu, sel)) - k1024;
     return __builtin_bit_cast(uint32_t, cl * __builtin_bit_cast(half2_t, scw) + __builtin_bit_cast(half2_t, nzw));
   };
@@ -414,7 +437,7 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
     constexpr int SCP = BF ? decltype(scp)::value : -1;
     float sf[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if constexpr (SCP >= 0) scales_of(sst, sf);
-    const int ti = c0 + 8 * g, tin = min(c0n, C - 32) + 8 * g;
+    const int ti = c0 + 16 * g, tin = c0n + 16 * g;
     uint32_t sw[4] = {0u, 0u, 0u, 0u}, nw[4] = {0u, 0u, 0u, 0u}, swn[4] = {0u, 0u, 0u, 0u}, nwn[4] = {0u, 0u, 0u, 0u};
     uint4 bz = make_uint4(0u, 0u, 0u, 0u);
     if constexpr (BF) {
@@ -449,7 +472,37 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
         if (pc & 1) nh[i] = build_hi(word, sel, scw, nzw);
         else nl[i] = build_lo(word, sel, scw, nzw);
       };
-      if constexpr (!HALF) {
+      if constexpr (BITS == 8) {
+        // one product tile per group of 16 packed rows: RB MFMAs, the four operand registers of the next group
+        // behind them (as the forward kernel's k-step)
+        auto piece8 = [&](int i) __attribute__((always_inline)) {
+          const uint32_t word = i < 2 ? wsrc.x : wsrc.y;
+          const uint32_t sel = (i & 1) ? 0x04030402u : 0x04010400u;
+          nl[i] = build_lo(word, sel, jg + 1 < NG ? sw[i] : swn[i], jg + 1 < NG ? nw[i] : nwn[i]);
+        };
+        if constexpr (!HALF) {
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) {
+            if (rb & 1) Act<TX>::mma_acc_nw_after(acc[rb][jg], __builtin_bit_cast(uint4, a[rb]), Bl, nl[rb >> 1]);
+            else Act<TX>::mma_acc_nw(acc[rb][jg], __builtin_bit_cast(uint4, a[rb]), Bl);
+            if (!(rb & 1)) piece8(rb >> 1);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        } else {
+          Act<TX>::mma_acc_nw(acc[0][jg], __builtin_bit_cast(uint4, a[0]), Bl);
+          piece8(0);
+          piece8(1);
+          __builtin_amdgcn_sched_barrier(0);
+          Act<TX>::mma_acc_nw_after2(acc[1][jg], __builtin_bit_cast(uint4, a[1]), Bl, nl[0], nl[1]);
+          piece8(2);
+          __builtin_amdgcn_sched_barrier(0);
+          Act<TX>::mma_acc_nw_after(acc[2][jg], __builtin_bit_cast(uint4, a[2]), Bl, nl[2]);
+          piece8(3);
+          __builtin_amdgcn_sched_barrier(0);
+          Act<TX>::mma_acc_nw_after(acc[3][jg], __builtin_bit_cast(uint4, a[3]), Bl, nl[3]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else if constexpr (!HALF) {
 #pragma unroll
         for (int n = 0; n < 16; ++n) {
           const int rb = n >> 1, i = n >> 2;
@@ -526,15 +579,15 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   {
     uint32_t sw[4] = {0u, 0u, 0u, 0u}, nw[4] = {0u, 0u, 0u, 0u};
     if constexpr (!BF) {
-      const uint4 s4 = *reinterpret_cast<const uint4 *>(tab_s + 8 * g), n4 = *reinterpret_cast<const uint4 *>(tab_nz + 8 * g);
+      const uint4 s4 = *reinterpret_cast<const uint4 *>(tab_s + 16 * g), n4 = *reinterpret_cast<const uint4 *>(tab_nz + 16 * g);
       sw[0] = s4.x; sw[1] = s4.y; sw[2] = s4.z; sw[3] = s4.w;
       nw[0] = n4.x; nw[1] = n4.y; nw[2] = n4.z; nw[3] = n4.w;
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const uint32_t word = i < 2 ? wr[0][0][0].x : wr[0][0][0].y, sel = (i & 1) ? 0x04030402u : 0x04010400u;
+      const uint32_t word = i < 2 ? wr[0][0].x : wr[0][0].y, sel = (i & 1) ? 0x04030402u : 0x04010400u;
       carry_l[i] = build_lo(word, sel, sw[i], nw[i]);
-      carry_h[i] = build_hi(word, sel, sw[i], nw[i]);
+      carry_h[i] = BITS == 8 ? 0u : build_hi(word, sel, sw[i], nw[i]);
     }
   }
   __builtin_amdgcn_sched_barrier(0);
@@ -545,18 +598,21 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
     constexpr int cur = decltype(curc)::value;
     read_a(1, cur, 1);
     __builtin_amdgcn_sched_barrier(0);
-    compute(aq[0], aqr[0], wr[cur][0], wr[cur][1][0], 64 * s, 64 * s + 32, std::integral_constant<int, cur>{}, s + 1);
+    uint2 w0[NG], w1[NG];
+    half_w(cur, 0, w0);
+    half_w(cur, 1, w1);
+    compute(aq[0], aqr[0], w0, w1[0], 64 * s, 64 * s + 8, std::integral_constant<int, cur>{}, s + 1);
     __builtin_amdgcn_sched_barrier(0);
-    load_w(cur, 0, s + 2);
     write_a(cur, cur ^ 1);
     load_a(cur, s + 3);
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
     read_a(0, cur ^ 1, 0);
     __builtin_amdgcn_sched_barrier(0);
-    compute(aq[1], aqr[1], wr[cur][1], wr[cur ^ 1][0][0], 64 * s + 32, 64 * s + 64, std::integral_constant<int, -1>{}, 0);
+    compute(aq[1], aqr[1], w1, make_uint2(wr[cur ^ 1][0].x, wr[cur ^ 1][0].y), 64 * s + 8, min(64 * s + 64, C - 64),
+            std::integral_constant<int, -1>{}, 0);
     __builtin_amdgcn_sched_barrier(0);
-    load_w(cur, 1, s + 2);
+    load_w(cur, s + 2);
     __builtin_amdgcn_sched_barrier(0);
   };
   int s = 0;
@@ -568,7 +624,7 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
 
   mma_drain();
   // acc[rb][2 jg + e][r] = out[m0 + 16 rb + 4 g + r][2 (j0 + 16 jg + l16) + e]  (bf16: plus t[m], see above)
-  const int64_t KO = 2 * (int64_t)R;
+  const int64_t KO = BITS == 8 ? (int64_t)R : 2 * (int64_t)R;
   floatx4 *rs_lds = reinterpret_cast<floatx4 *>(a_lds);                 // [row block][lane]
   if constexpr (BF) {
     __syncthreads();                                                   // every wavefront has left the loop
@@ -591,6 +647,12 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
       if (out32 != nullptr) {
         const int e = rowexp[m];
         float *orow32 = out32 + (int64_t)m * KO;
+        if constexpr (BITS == 8) {
+#pragma unroll
+          for (int jg = 0; jg < NG; ++jg)
+            orow32[j0 + 16 * jg + l16] = ldexpf((float)Act<TX>::out(512.f * acc[rb][jg][r]), e);
+          continue;
+        }
 #pragma unroll
         for (int jg = 0; jg < NG; ++jg) {
           const int j = j0 + 16 * jg + l16;
@@ -600,6 +662,11 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
         continue;
       }
       TX *orow = out + (int64_t)m * KO;
+      if constexpr (BITS == 8) {
+#pragma unroll
+        for (int jg = 0; jg < NG; ++jg) orow[j0 + 16 * jg + l16] = Act<TX>::out(512.f * acc[rb][jg][r]);
+        continue;
+      }
 #pragma unroll
       for (int jg = 0; jg < NG; ++jg) {
         const int j = j0 + 16 * jg + l16;
@@ -635,15 +702,15 @@ int launch_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int
   return GPTQ_HIP_OK;
 }
 
-template <typename TX>
+template <typename TX, int BITS = 4>
 int launch_bwd_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
                     const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32, const int32_t *rowexp,
                     bool half) {
   if (Act<TX>::BF && half) return GPTQ_HIP_EINVAL;                    // (not dispatched, see wide_bwd_tiles)
-  auto kern = (!Act<TX>::BF && half) ? qmm_bwd_wide_kernel<TX, !Act<TX>::BF> : qmm_bwd_wide_kernel<TX, false>;
+  auto kern = (!Act<TX>::BF && half) ? qmm_bwd_wide_kernel<TX, !Act<TX>::BF, BITS> : qmm_bwd_wide_kernel<TX, false, BITS>;
   const int lds = (int)((Act<TX>::BF ? 8 : 4) * C + 2 * 2 * 8 * 64 * 16);
   if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), lds)) return GPTQ_HIP_ELAUNCH;
-  const int64_t KO = 2 * R;
+  const int64_t KO = BITS == 8 ? R : 2 * R;
   int64_t rows_max = ((1LL << 31) - 1) / C;
   if (rows_max > 65535LL * 128) rows_max = 65535LL * 128;
   rows_max -= rows_max % 128;
@@ -697,25 +764,31 @@ int wide_fwd_launch(hipStream_t st, const void *x, int x_dtype, int64_t M, const
   return launch_wide<__half>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half, c0);
 }
 
-int64_t wide_bwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half, bool bf16) {
+int64_t wide_bwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half, bool bf16, int bits) {
   *half = false;
+  const int64_t rows512 = bits == 8 ? 512 : 256;       // packed rows of 512 output columns
   // (the constants of all channels and the stages share the LDS: 4 C + 32 KB; bf16 rows: 8 C + 32 KB)
   if (!aligned || C % 64 != 0 || C < 512 || C > (bf16 ? 16384 : 30720) || M < 256) return 0;
   const int64_t tiles_y = ceil_div64(M, 128);
-  const int64_t n = wide_rounds(R / 256, tiles_y);
+  if (bits == 8 && bf16) return 0;
+  const int64_t n = wide_rounds(R / rows512, tiles_y);
   if (n > 0) return n;
   // (bf16 rows: the 128 x 256 form, whose wavefronts have half the MFMAs to hide the scaling of the rows behind,
   // measured slower than the 128-row tiles: 284 against 273 us at M = 2048 on 4096 x 11008)
   if (bf16) return 0;
   *half = true;
-  return wide_rounds(R / 128, tiles_y);
+  return wide_rounds(R / (rows512 / 2), tiles_y);
 }
 
 int wide_bwd_launch(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
                     const void *scale, int zs_dtype, void *out, int64_t wide_x, bool half, float *out32,
-                    const int32_t *rowexp, bool bf16) {
+                    const int32_t *rowexp, bool bf16, int bits) {
   if (zs_dtype != GPTQ_HIP_F32 && zs_dtype != GPTQ_HIP_F16 && zs_dtype != GPTQ_HIP_BF16) return GPTQ_HIP_EDTYPE;
-  if (wide_x < 1 || wide_x * (half ? 128 : 256) > R) return GPTQ_HIP_EINVAL;
+  if (wide_x < 1 || wide_x * (half ? 128 : 256) * (bits == 8 ? 2 : 1) > R) return GPTQ_HIP_EINVAL;
+  if (bits == 8) {
+    if (bf16) return GPTQ_HIP_EDTYPE;
+    return launch_bwd_wide<__half, 8>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half);
+  }
   if (bf16) {
     if (out32 || C > 16384) return GPTQ_HIP_EINVAL;
     return launch_bwd_wide<__hip_bfloat16>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, nullptr, nullptr, half);

@@ -241,6 +241,35 @@ def test_qmatmul_8bit_many_rows_128x512_tiles(OP, M, N, K, xdt, zs):
     assert np.all(err <= tol), float((err / tol).max())
 
 
+@pytest.mark.parametrize("xdt,zs", [("float16", "float32"), ("float16", "float16"), ("float32", "bfloat16"),
+                                    ("bfloat16", "float32")])
+@pytest.mark.parametrize("M,N,K", [(3500, 512, 4480), (2048, 1024, 11008), (4096, 576, 4096), (1800, 20480, 4096),
+                                   (2000, 1088, 4224)])
+def test_qmatmul_8bit_many_rows_128x512_tiles_transposed(OP, M, N, K, xdt, zs):
+    """The transposed product of many fp16 (or fp32) rows against 8-bit codes on the 128 x 512 tiles: a packed row
+    is one output column, 512 of them per workgroup, the contraction along the channels in stages of 64 (an odd
+    number of stages, 20480 channels, 128 x 256 tiles where the wide ones are under a round, columns left over for
+    the 128-row tiles); bf16 rows stay on the 128-row tiles."""
+    import torch
+    import jax_gptq_amd.gptq as G
+    rng = np.random.default_rng(M + N + K)
+    codes = rng.integers(0, 256, (K, N)).astype(np.uint8)
+    tdt = getattr(torch, zs)
+    scale = torch.from_numpy(rng.uniform(0.0001, 0.001, N).astype(np.float32)).to(tdt)
+    zero = torch.from_numpy(rng.uniform(0.0, 255.0, N).astype(np.float32)).to(tdt)
+    qm = G.QuantizedMatrix(torch.from_numpy(codes).cuda(), zero.cuda(), scale.cuda(), bits=8)
+    rowscale = np.array([1.0, 1e-3, 3e4])[np.arange(M) % 3][:, None] if xdt == "float32" else np.ones((M, 1))
+    x = torch.from_numpy((0.05 * rng.standard_normal((M, N)) * rowscale).astype(np.float32)).to(getattr(torch, xdt))
+    got = OP.quantized_matmul(x, qm, transpose_b=True)
+    assert got.dtype == getattr(torch, xdt) and tuple(got.shape) == (M, K)
+    dense = (codes.astype(np.float64) - zero.double().numpy()[None]) * scale.double().numpy()[None]
+    ref = x.double().numpy() @ dense.T
+    err = np.abs(to_np(got).astype(np.float64) - ref)
+    rel = 2.0 ** -8 if xdt == "bfloat16" else RTOL
+    tol = (ATOL + rel * np.abs(ref / rowscale)) * rowscale
+    assert np.all(err <= tol), float((err / tol).max())
+
+
 @pytest.mark.parametrize("xdt", ["float16", "bfloat16"])
 @pytest.mark.parametrize("M,N,K", [(17, 1024, 4096), (64, 11008, 512), (100, 2048, 1000), (200, 4096, 1064),
                                    (256, 1152, 2048), (33, 8192, 8192)])
