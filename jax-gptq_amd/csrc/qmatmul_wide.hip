@@ -706,8 +706,7 @@ template <typename TX, int BITS = 4>
 int launch_bwd_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
                     const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32, const int32_t *rowexp,
                     bool half) {
-  if (Act<TX>::BF && half) return GPTQ_HIP_EINVAL;                    // (not dispatched, see wide_bwd_tiles)
-  auto kern = (!Act<TX>::BF && half) ? qmm_bwd_wide_kernel<TX, !Act<TX>::BF, BITS> : qmm_bwd_wide_kernel<TX, false, BITS>;
+  auto kern = half ? qmm_bwd_wide_kernel<TX, true, BITS> : qmm_bwd_wide_kernel<TX, false, BITS>;
   const int lds = (int)((Act<TX>::BF ? 8 : 4) * C + 2 * 2 * 8 * 64 * 16);
   if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), lds)) return GPTQ_HIP_ELAUNCH;
   const int64_t KO = BITS == 8 ? R : 2 * R;
@@ -773,9 +772,6 @@ int64_t wide_bwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half
   if (bits == 8 && bf16) return 0;
   const int64_t n = wide_rounds(R / rows512, tiles_y);
   if (n > 0) return n;
-  // (bf16 rows: the 128 x 256 form, whose wavefronts have half the MFMAs to hide the scaling of the rows behind,
-  // measured slower than the 128-row tiles: 284 against 273 us at M = 2048 on 4096 x 11008)
-  if (bf16) return 0;
   *half = true;
   return wide_rounds(R / (rows512 / 2), tiles_y);
 }

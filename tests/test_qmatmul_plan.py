@@ -24,7 +24,7 @@ CASES = [
     (2048, 11008, 4096, 1, "F16", 4, 1), (2048, 4096, 11008, 1, "F16", 4, 1), (2048, 11008, 4096, 1, "BF16", 4, 1),
     (1, 11008, 4096, 0, "F32", 4, 1), (128, 11008, 4096, 0, "F32", 4, 1),
     (1, 28672, 7168, 0, "F16", 4, 1), (16, 28672, 7168, 0, "F16", 4, 1), (2048, 28672, 7168, 0, "F16", 4, 1),
-    (2048, 28672, 7168, 1, "F16", 4, 1),
+    (2048, 28672, 7168, 1, "F16", 4, 1), (2048, 28672, 7168, 1, "BF16", 4, 1), (2048, 11008, 4096, 0, "F16", 8, 1),
     (1, 11008, 4096, 0, "F16", 8, 1), (128, 11008, 4096, 0, "F16", 8, 1), (2048, 11008, 4096, 1, "F16", 8, 1),
     (1, 50257, 768, 0, "F16", 4, 1), (512, 50257, 768, 0, "F16", 4, 1), (512, 50257, 768, 1, "F16", 4, 1),
     # the tall, narrow tiles, the 128 x 512 / 128 x 256 tiles and their transposed forms
@@ -71,7 +71,13 @@ def test_headline_cases_run_on_the_kernels_the_design_names(N):
     big = _plan(N, 2048, 11008, 4096, 0, "F16", 4, 1)
     assert big["kernel"].startswith("qmm_fwd_wide_kernel") and big["rest"].startswith("qmm_fwd_reg_kernel")
     assert _plan(N, 2048, 11008, 4096, 1, "F16", 4, 1)["kernel"].startswith("qmm_bwd_wide_kernel")
-    assert _plan(N, 2048, 11008, 4096, 1, "BF16", 4, 1)["kernel"].startswith("qmm_bwd_reg_kernel (128")
+    assert _plan(N, 2048, 11008, 4096, 1, "BF16", 4, 1)["kernel"].startswith("qmm_bwd_wide_kernel")
+    # bf16 rows: the constants of more than 16384 channels do not fit beside the stages
+    assert _plan(N, 2048, 28672, 7168, 1, "BF16", 4, 1)["kernel"].startswith("qmm_bwd_reg_kernel (128")
+    # 8-bit codes with many fp16 rows, both directions (bf16 rows stay on the 128-row tiles)
+    assert _plan(N, 2048, 11008, 4096, 0, "F16", 8, 1)["kernel"].startswith("qmm_fwd_wide_kernel")
+    assert _plan(N, 2048, 11008, 4096, 1, "F16", 8, 1)["kernel"].startswith("qmm_bwd_wide_kernel")
+    assert _plan(N, 2048, 11008, 4096, 0, "BF16", 8, 1)["kernel"].startswith("qmm_fwd_reg_kernel (128")
     # fp32 rows: converted inside the decode kernel up to 16 rows, staged as fp16 rows beyond
     assert _plan(N, 1, 11008, 4096, 0, "F32", 4, 1)["fp32_rows"] == 2
     assert _plan(N, 128, 11008, 4096, 0, "F32", 4, 1)["fp32_rows"] == 1
