@@ -180,7 +180,7 @@ def bench_qmatmul(reps=240):
     g.manual_seed(1)
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     # the two Llama-7B MLP shapes of the benchmark layer, then the OPT-30B fc1 shape (103 MB packed:
-    # decode matmuls of that size run the streaming kernel)
+    # decode matmuls of that size run the decode kernel's ring-loop form)
     # (K, N, bits): the last two are what the register-operand kernels serve: 8-bit codes (one per byte)
     # and a vocabulary-sized N that is not a multiple of 16 channels
     for (K, N, bits) in ((4096, 11008, 4), (11008, 4096, 4), (7168, 28672, 4), (4096, 11008, 8), (768, 50257, 4)):

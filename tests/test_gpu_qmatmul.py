@@ -304,7 +304,7 @@ def test_qmatmul_bf16_x_transposed_mfma_path(OP, M, N, K, zs):
                                             (5, 28672, 7168, "bfloat16", "bfloat16"),
                                             (2, 32000, 5120, "float16", "float16")])
 def test_qmatmul_streaming_kernel_large_matrices(OP, M, N, K, xdt, zs):
-    """M <= 16 on matrices of 80 MB and more runs the streaming kernel (long row range per
+    """M <= 16 on matrices of 80 MB and more runs the decode kernel's ring-loop form (long row range per
     workgroup, register ring of loads); (3, 29936, 9000) has a ragged last k-step, a partial
     last strip and fractional zero points.  Reference: fp32 dense product by torch on the
     device (the host evaluation of these sizes takes minutes)."""
