@@ -1758,13 +1758,13 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
       }
     }
   }
-  if (bits == 4 && !transpose_b && group_size == 0 && x_dtype == GPTQ_HIP_F16) {
-    // 17 .. 256 fp16 rows: tall, narrow tiles whose eight wavefronts split the contraction (qmatmul_mid.hip)
-    MidPlan mp = mid_fwd_plan(M, R, C, al && (reinterpret_cast<uintptr_t>(packed) & 15) == 0);
+  if (bits == 4 && !transpose_b && group_size == 0) {
+    // 17 .. 256 rows: tall, narrow tiles whose eight wavefronts split the contraction (qmatmul_mid.hip)
+    MidPlan mp = mid_fwd_plan(M, R, C, al && (reinterpret_cast<uintptr_t>(packed) & 15) == 0, x_dtype == GPTQ_HIP_BF16);
     if (mp.use) {
       if (mp.total_bytes && (!ws || ws_bytes < mp.total_bytes)) return GPTQ_HIP_EWORKSPACE;
       if (planned(GPTQ_HIP_QMM_MID, 0, mp.S, mp.tiles_x * mp.tiles_y * mp.S)) return GPTQ_HIP_OK;
-      if (out32 && rowexp && wrote32) {
+      if (out32 && rowexp && wrote32 && x_dtype == GPTQ_HIP_F16) {
         mp.out32 = out32;
         mp.rowexp = rowexp;
         *wrote32 = true;

@@ -31,7 +31,12 @@
 // 44 MB at M = 32 on 4096 x 11008, twice the weights), which is why the dispatcher takes it up to 64 rows
 // (128 on small matrices) and leaves more rows to the 64 x 128 and 128 x 128 tiles.
 //
-// Shapes: K % 256 == 0 (whole stages), C % 16 == 0, operands 16-byte aligned, per-channel parameters, fp16
+// bf16 activations: the operand registers are 128 + code (a byte permute and an or under 0x4300: exact in bf16),
+// the term (128 + zero) sum_k x[m][k] leaves in the epilogue; the row sums come from one more MFMA per row block and
+// k-step against a vector of ones (the matrix pipe is mostly idle here) and are summed over the wavefronts with
+// the tiles.  A split applies the term to its own partial sums before it hands them over (it is linear in them).
+//
+// Shapes: K % 256 == 0 (whole stages), C % 16 == 0, operands 16-byte aligned, per-channel parameters, fp16 or bf16
 // activations (fp32 rows through the fp16 staging of the dispatcher: out32 / rowexp).
 #include "qmatmul_reg.h"
 #include "qmm_reg_common.h"
@@ -71,12 +76,13 @@ constexpr int mid_rbt(int nb, int rb) {
   return r;
 }
 
-template <int RB, int WR, int KS>
-__global__ __launch_bounds__(MID_TPB) void qmm_fwd_mid_kernel(const __half *x, int M, int K, const uint8_t *pk, int R,
+template <typename TX, int RB, int WR, int KS>
+__global__ __launch_bounds__(MID_TPB) void qmm_fwd_mid_kernel(const TX *x, int M, int K, const uint8_t *pk, int R,
                                                              int C, const void *zero, const void *scale, int zs_dtype,
-                                                             __half *out, float *part, int32_t *counters, int S,
+                                                             TX *out, float *part, int32_t *counters, int S,
                                                              int steps_per_split, int tiles_x, int tiles_y, float *out32,
                                                              const int32_t *rowexp) {
+  constexpr bool BF = Act<TX>::BF;
   constexpr int NB = 4;                          // 16-channel blocks per tile
   constexpr int ROWS = 16 * RB;
   constexpr int BUF = ROWS * MID_PITCH;          // one stage
@@ -157,6 +163,11 @@ __global__ __launch_bounds__(MID_TPB) void qmm_fwd_mid_kernel(const __half *x, i
     zneg[t] = __builtin_bit_cast(uint32_t, half2_t{h, h});
   }
   const half2_t mul = half2_t{(_Float16)32768.f, (_Float16)2048.f};
+  uint32_t c43 = 0x43004300u, one2 = 0x3F803F80u;
+  asm volatile("" : "+v"(c43), "+v"(one2));
+  floatx4 rsacc[RB];                             // bf16: sum_k x[m][k] of this wavefront's k-steps (every column alike)
+#pragma unroll
+  for (int i = 0; i < RB; ++i) rsacc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   floatx4 acc[RB][NB];
 #pragma unroll
@@ -201,7 +212,7 @@ __global__ __launch_bounds__(MID_TPB) void qmm_fwd_mid_kernel(const __half *x, i
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       mlo[i] = wv[i] & 0x0F0F0F0Fu;
-      mhi[i] = wv[i] & 0xF0F0F0F0u;
+      mhi[i] = BF ? (wv[i] >> 4) & 0x0F0F0F0Fu : wv[i] & 0xF0F0F0F0u;
     }
 #pragma unroll
     for (int t = 0; t < NB; ++t) {
@@ -209,14 +220,23 @@ __global__ __launch_bounds__(MID_TPB) void qmm_fwd_mid_kernel(const __half *x, i
       uint32_t b4[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const uint32_t pb = __builtin_amdgcn_perm(mhi[i], mlo[i], sel);     // {lo, 16 hi} as fp16 subnormals
-        const half2_t d = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, pb), mul,
-                                                    __builtin_bit_cast(half2_t, zneg[t]));
-        b4[i] = __builtin_bit_cast(uint32_t, d);
+        const uint32_t pb = __builtin_amdgcn_perm(mhi[i], mlo[i], sel);     // fp16: {lo, 16 hi} as subnormals
+        if constexpr (BF) {
+          b4[i] = pb | c43;                                                   // {128 + lo, 128 + hi}
+        } else {
+          const half2_t d = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, pb), mul,
+                                                      __builtin_bit_cast(half2_t, zneg[t]));
+          b4[i] = __builtin_bit_cast(uint32_t, d);
+        }
       }
       const uint4 b = make_uint4(b4[0], b4[1], b4[2], b4[3]);
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) acc[rb][t] = Act<__half>::mma(a[sub % AS][rb], b, acc[rb][t]);
+      for (int rb = 0; rb < RB; ++rb) acc[rb][t] = Act<TX>::mma(a[sub % AS][rb], b, acc[rb][t]);
+    }
+    if constexpr (BF) {
+      const uint4 ones = make_uint4(one2, one2, one2, one2);
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) rsacc[rb] = Act<TX>::mma(a[sub % AS][rb], ones, rsacc[rb]);
     }
     __builtin_amdgcn_sched_barrier(0);
     store_x(sub, (buf ^ 1) * BUFK + sub * BUF);
@@ -240,20 +260,37 @@ __global__ __launch_bounds__(MID_TPB) void qmm_fwd_mid_kernel(const __half *x, i
   __syncthreads();                       // (the last stages may have ended without one)
   // ---- sum over the eight wavefronts (and the S workgroups of a split tile); wavefront q < RBT finishes row
   // block q of the pass
-  float sc[NB];
+  float sc[NB], zoff[NB];
 #pragma unroll
-  for (int t = 0; t < NB; ++t) sc[t] = rg_raw_to_f32(sraw[t], zs_dtype) * 512.f;
+  for (int t = 0; t < NB; ++t) {
+    sc[t] = rg_raw_to_f32(sraw[t], zs_dtype) * (BF ? 1.f : 512.f);
+    zoff[t] = 128.f + rg_raw_to_f32(zraw[t], zs_dtype);
+  }
   float *red = reinterpret_cast<float *>(mid_lds);      // [wavefront][row block of the pass][tile][lane][4]
   auto finish = [&](auto pc) __attribute__((always_inline)) {
     constexpr int P = decltype(pc)::value;
+    const bool owner = w < RBT;
+    const int rbo = owner ? w : 0;
+    floatx4 rs = floatx4{0.f, 0.f, 0.f, 0.f};
+    if constexpr (BF) {
+      // the row sums first, through the same buffer
+#pragma unroll
+      for (int rb = 0; rb < RBT; ++rb)
+        *reinterpret_cast<floatx4 *>(red + ((w * RBT + rb) * 64 + lane) * 4) = rsacc[P * RBT + rb];
+      __syncthreads();
+      if (owner) {
+#pragma unroll
+        for (int q = 0; q < MID_WAVES; ++q)
+          rs += *reinterpret_cast<const floatx4 *>(red + ((q * RBT + rbo) * 64 + lane) * 4);
+      }
+      __syncthreads();
+    }
 #pragma unroll
     for (int rb = 0; rb < RBT; ++rb)
 #pragma unroll
       for (int t = 0; t < NB; ++t)
         *reinterpret_cast<floatx4 *>(red + (((w * RBT + rb) * NB + t) * 64 + lane) * 4) = acc[P * RBT + rb][t];
     __syncthreads();
-    const bool owner = w < RBT;
-    const int rbo = owner ? w : 0;
     floatx4 sum[NB];
 #pragma unroll
     for (int t = 0; t < NB; ++t) {
@@ -264,6 +301,13 @@ __global__ __launch_bounds__(MID_TPB) void qmm_fwd_mid_kernel(const __half *x, i
           v += *reinterpret_cast<const floatx4 *>(red + (((q * RBT + rbo) * NB + t) * 64 + lane) * 4);
       }
       sum[t] = v;
+    }
+    if constexpr (BF) {
+      // sum_k x (128 + code) - (128 + zero) sum_k x, on this workgroup's range of k
+#pragma unroll
+      for (int t = 0; t < NB; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sum[t][r] -= zoff[t] * rs[r];
     }
     if (S > 1) {
       const int tile = ((ty * NP + P) * tiles_x + tx);
@@ -312,15 +356,29 @@ __global__ __launch_bounds__(MID_TPB) void qmm_fwd_mid_kernel(const __half *x, i
       if (P + 1 < NP) __syncthreads();                         // red is free for the next pass
       if (!owner) return;
     }
-    // sum[t][r] = 2^-9 sum_k x[m][k] (code - zero)[k][col + t], m = m0 + 16 (P RBT + rbo) + 4 g + r
+    // sum[t][r] = (fp16: 2^-9) sum_k x[m][k] (code - zero)[k][col + t], m = m0 + 16 (P RBT + rbo) + 4 g + r
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int m = m0 + 16 * (P * RBT + rbo) + 4 * g + r;
       if (m >= M) continue;
+      const bool whole = c0 + 16 * NB <= C;                    // (uniform) every channel of the tile exists
+      if constexpr (BF) {
+        TX ob[NB];
+#pragma unroll
+        for (int t = 0; t < NB; ++t) ob[t] = Act<TX>::out(sc[t] * sum[t][r]);
+        TX *dstb = out + (int64_t)m * C + col;
+        if (whole) {
+          *reinterpret_cast<uint2 *>(dstb) = *reinterpret_cast<const uint2 *>(ob);
+        } else {
+#pragma unroll
+          for (int t = 0; t < NB; ++t)
+            if (col + t < C) dstb[t] = ob[t];
+        }
+        continue;
+      }
       _Float16 o[NB];
 #pragma unroll
       for (int t = 0; t < NB; ++t) o[t] = (_Float16)(sc[t] * sum[t][r]);
-      const bool whole = c0 + 16 * NB <= C;                    // (uniform) every channel of the tile exists
       if (out32 != nullptr) {
         // fp32 rows: the fp16 result widened and scaled back by the row's power of two (exact)
         const int e = rowexp[m];
@@ -335,7 +393,7 @@ __global__ __launch_bounds__(MID_TPB) void qmm_fwd_mid_kernel(const __half *x, i
         }
         continue;
       }
-      __half *dst = out + (int64_t)m * C + col;
+      __half *dst = reinterpret_cast<__half *>(out) + (int64_t)m * C + col;
       if (whole) {
         // (col % 4 == 0, C % 16 == 0, out 16-byte aligned)
         *reinterpret_cast<uint2 *>(dst) = make_uint2(__builtin_bit_cast(uint32_t, half2_t{o[0], o[1]}),
@@ -351,7 +409,7 @@ __global__ __launch_bounds__(MID_TPB) void qmm_fwd_mid_kernel(const __half *x, i
   if constexpr (NP == 2) finish(std::integral_constant<int, 1>{});
 }
 
-template <int RB>
+template <typename TX, int RB>
 int mid_launch_inst(hipStream_t st, const MidPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
                     const void *zero, const void *scale, int zs_dtype, void *out, void *wsp) {
   // ring of weight k-steps (what the registers allow) and stages between two barriers (what the LDS holds twice)
@@ -361,13 +419,13 @@ int mid_launch_inst(hipStream_t st, const MidPlan &p, const void *x, int64_t M, 
   constexpr size_t stage_bytes = (size_t)2 * KS * 16 * RB * MID_PITCH + (size_t)MID_WAVES * 1024;
   constexpr size_t red_bytes = (size_t)MID_WAVES * RBT * 4 * RG_TILE_FLOATS * sizeof(float);
   constexpr size_t lds = stage_bytes > red_bytes ? stage_bytes : red_bytes;
-  auto kern = qmm_fwd_mid_kernel<RB, WR, KS>;
+  auto kern = qmm_fwd_mid_kernel<TX, RB, WR, KS>;
   if (lds > 64 * 1024 && !gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), (int)lds)) return GPTQ_HIP_ELAUNCH;
   int32_t *counters = reinterpret_cast<int32_t *>(wsp);
   float *part = reinterpret_cast<float *>(reinterpret_cast<char *>(wsp) + QMM_HEAD_BYTES);
   const dim3 grid((unsigned)(p.tiles_x * p.tiles_y * p.S));
-  hipLaunchKernelGGL(kern, grid, dim3(MID_TPB), lds, st, (const __half *)x, (int)M, (int)(2 * R), pk, (int)R, (int)C, zero,
-                     scale, zs_dtype, (__half *)out, part, counters, p.S, p.steps, (int)p.tiles_x, (int)p.tiles_y, p.out32, p.rowexp);
+  hipLaunchKernelGGL(kern, grid, dim3(MID_TPB), lds, st, (const TX *)x, (int)M, (int)(2 * R), pk, (int)R, (int)C, zero,
+                     scale, zs_dtype, (TX *)out, part, counters, p.S, p.steps, (int)p.tiles_x, (int)p.tiles_y, p.out32, p.rowexp);
   GPTQ_CHECK_LAUNCH();
   return GPTQ_HIP_OK;
 }
@@ -376,8 +434,9 @@ int mid_launch_inst(hipStream_t st, const MidPlan &p, const void *x, int64_t M, 
 
 namespace qmm {
 
-MidPlan mid_fwd_plan(int64_t M, int64_t R, int64_t C, bool aligned) {
+MidPlan mid_fwd_plan(int64_t M, int64_t R, int64_t C, bool aligned, bool bf16) {
   MidPlan p{};
+  p.bf16 = bf16;
   const int64_t K = 2 * R;
   if (!aligned || M < 17 || M > 256 || K % MID_STAGE_K != 0 || C % 16 != 0 || C < 64 || M * K >= (1LL << 31) ||
       R >= (1LL << 30) || C >= (1LL << 30))
@@ -418,8 +477,14 @@ int mid_fwd_launch(hipStream_t st, const MidPlan &p, const void *x, int64_t M, c
                    const void *zero, const void *scale, int zs_dtype, void *out, void *ws) {
   if (zs_dtype != GPTQ_HIP_F32 && zs_dtype != GPTQ_HIP_F16 && zs_dtype != GPTQ_HIP_BF16) return GPTQ_HIP_EDTYPE;
   if (p.nb != 4) return GPTQ_HIP_EINVAL;
-  if (p.rb == 2) return mid_launch_inst<2>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
-  if (p.rb == 4) return mid_launch_inst<4>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+  if (p.bf16) {
+    if (p.out32) return GPTQ_HIP_EINVAL;
+    if (p.rb == 2) return mid_launch_inst<__hip_bfloat16, 2>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+    if (p.rb == 4) return mid_launch_inst<__hip_bfloat16, 4>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+    return GPTQ_HIP_EINVAL;
+  }
+  if (p.rb == 2) return mid_launch_inst<__half, 2>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
+  if (p.rb == 4) return mid_launch_inst<__half, 4>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws);
   return GPTQ_HIP_EINVAL;
 }
 

@@ -46,14 +46,14 @@ int reg_fwd_launch(hipStream_t st, const RegPlan &p, const void *x, int x_dtype,
 // of eight wavefronts owns 16 rb rows x 16 nb channels over one of S ranges of `steps` k-steps.  out32 / rowexp as in
 // RegPlan.
 struct MidPlan {
-  bool use;
+  bool use, bf16;
   int rb, nb, S, steps;
   int64_t tiles_x, tiles_y;
   float *out32;
   const int32_t *rowexp;
   size_t part_bytes, total_bytes;
 };
-MidPlan mid_fwd_plan(int64_t M, int64_t R, int64_t C, bool aligned);
+MidPlan mid_fwd_plan(int64_t M, int64_t R, int64_t C, bool aligned, bool bf16 = false);
 int mid_fwd_launch(hipStream_t st, const MidPlan &p, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C,
                    const void *zero, const void *scale, int zs_dtype, void *out, void *ws);
 

@@ -200,7 +200,7 @@ def test_qmatmul_many_rows_128x512_tiles(OP, M, N, K, xdt, zs):
 
 
 @pytest.mark.parametrize("xdt,zs", [("float16", "float32"), ("float16", "float16"), ("float16", "bfloat16"),
-                                    ("float32", "float32")])
+                                    ("float32", "float32"), ("bfloat16", "float32"), ("bfloat16", "bfloat16")])
 @pytest.mark.parametrize("M,N,K", [(17, 11008, 4096), (32, 11008, 4096), (33, 4096, 11008), (64, 11008, 4096),
                                    (50, 80, 2304), (128, 4096, 4096), (100, 1104, 1024), (256, 3072, 768),
                                    (40, 64, 256)])
@@ -211,7 +211,9 @@ def test_qmatmul_few_dozen_rows_tall_narrow_tiles(OP, M, N, K, xdt, zs):
     tiles through the workspace; 80 and 1104 channels: a last tile of 16 channels; M = 33, 50, 100: ragged row
     tiles; 2304 = 9 stages and 256 = 1 stage: the loop's remainder).  The weight operands are formed as
     (code - zero) 2^-9 in fp16, so a fractional zero point costs fp16's relative precision and no more; fp32 rows
-    of very different magnitudes go through the scaled fp16 staging and the tiles' own fp32 store."""
+    of very different magnitudes go through the scaled fp16 staging and the tiles' own fp32 store; bf16 rows multiply
+    128 + code and the term in 128 + zero leaves through row sums that one more MFMA per row block accumulates
+    (two passes of the final reduction for 64-row tiles; a split applies the term to its own partial sums)."""
     import torch
     import jax_gptq_amd.gptq as G
     rng = np.random.default_rng(M + N + K)
@@ -226,7 +228,7 @@ def test_qmatmul_few_dozen_rows_tall_narrow_tiles(OP, M, N, K, xdt, zs):
     x = torch.from_numpy((rng.standard_normal((M, K)) * rowscale).astype(np.float32)).to(getattr(torch, xdt))
     dense = (codes.astype(np.float64) - zero.double().numpy()[None]) * scale.double().numpy()[None]
     ref = x.double().numpy() @ dense
-    tol = (ATOL + RTOL * np.abs(ref / rowscale)) * rowscale
+    tol = (ATOL + (2.0 ** -8 if xdt == "bfloat16" else RTOL) * np.abs(ref / rowscale)) * rowscale
     first = None
     for rep in range(3):            # the split sums leave their counters as they found them
         got = OP.quantized_matmul(x, qm)

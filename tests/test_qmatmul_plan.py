@@ -67,6 +67,7 @@ def test_headline_cases_run_on_the_kernels_the_design_names(N):
     for M in (17, 32, 64):
         for (Nc, K) in ((11008, 4096), (4096, 11008)):
             assert _plan(N, M, Nc, K, 0, "F16", 4, 1)["kernel"] == "qmm_fwd_mid_kernel", (M, Nc, K)
+    assert _plan(N, 64, 11008, 4096, 0, "BF16", 4, 1)["kernel"] == "qmm_fwd_mid_kernel"
     assert _plan(N, 128, 11008, 4096, 0, "F16", 4, 1)["kernel"].startswith("qmm_fwd_reg_kernel")
     big = _plan(N, 2048, 11008, 4096, 0, "F16", 4, 1)
     assert big["kernel"].startswith("qmm_fwd_wide_kernel") and big["rest"].startswith("qmm_fwd_reg_kernel")
