@@ -15,6 +15,7 @@
 // float is the default path, double the reference's use_fp64 option (gptq.py:182-197).
 #include "common.h"
 #include "gemm_f32.h"
+#include "tile_io.h"
 
 namespace {
 
@@ -148,21 +149,19 @@ constexpr int DIAG_FW = 4;                       // factorising wavefronts
 constexpr int PW = 4;                            // columns per panel
 constexpr int DIAG_THREADS = (DIAG_FW + 1) * 64;
 
-template <typename R>
-__global__ __launch_bounds__(DIAG_THREADS) void chol_diag_kernel(R *A, R *Minv, int64_t ld, int b,
-                                                                 int32_t *status) {
-  __shared__ __attribute__((aligned(16))) R dinv[NB];        // 1 / G[k][k]
-  __shared__ __attribute__((aligned(16))) R Gs[NB * GSTR];   // G, row major
-  __shared__ __attribute__((aligned(16))) R Xs[NB * (NB + 1)];   // X = G^-1, row major
-  __shared__ __attribute__((aligned(16))) R Lcol[2][PW][NB]; // the columns of a panel of G, by panel parity
+// The block's work.  src (row stride lds): the block D, in global memory or (ALIAS) in the LDS array that Gs
+// overwrites once every lane holds its part; Mout (may be null) / Dinv: where M_bb and its inverse go, row stride
+// ld.  dinv [NB], Gs [NB * GSTR], Xs [NB * (NB + 1)], Lcol [2 * PW * NB]: LDS.  All five wavefronts call it.
+template <typename R, bool ALIAS>
+__device__ __forceinline__ void chol_diag_block(const R *src, int64_t lds, R *Mout, R *Dinv, int64_t ld, int b,
+                                                int32_t *status, R *dinv, R *Gs, R *Xs, R *Lcol) {
   constexpr int XSTR = NB + 1;
   constexpr int CW = NB / DIAG_FW;                           // columns per factorising wavefront
   const int r = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-  R *D = A + (int64_t)b * NB * ld + (int64_t)b * NB;
-  R *Dinv = Minv + (int64_t)b * NB * ld + (int64_t)b * NB;
   typedef R colvec __attribute__((ext_vector_type(CW)));    // vector values, never an alloca
   typedef R rowvec __attribute__((ext_vector_type(NB)));
+  auto lcol = [&](int par, int q) __attribute__((always_inline)) -> R * { return Lcol + (par * PW + q) * NB; };
 
   if (wave < DIAG_FW) {
     // slot j of wavefront w holds column col_of(j) = 16 (j / 4) + 4 w + j % 4
@@ -172,8 +171,9 @@ __global__ __launch_bounds__(DIAG_THREADS) void chol_diag_kernel(R *A, R *Minv, 
 #pragma unroll
     for (int j = 0; j < CW; ++j) {
       const int c = col_of(j);
-      g[j] = D[(int64_t)(NB - 1 - c) * ld + (NB - 1 - r)];   // c > r: finite garbage, never used
+      g[j] = src[(int64_t)(NB - 1 - c) * lds + (NB - 1 - r)];   // c > r: finite garbage, never used
     }
+    if (ALIAS) __syncthreads();               // every lane has its part of the block: Gs may overwrite it
     bool bad = false;
     // G[r][c] -= l[r] l[c] for the column in slot j; pinned to its place: left free, the compiler may defer
     // every update until the element is needed and keep the operands of all steps alive
@@ -194,7 +194,7 @@ __global__ __launch_bounds__(DIAG_THREADS) void chol_diag_kernel(R *A, R *Minv, 
         root_and_inverse(piv, root, rinv);
         const R l = (r == k) ? root : g[j0 + q] * rinv;
         g[j0 + q] = l;
-        Lcol[p & 1][q][r] = l;
+        lcol(p & 1, q)[r] = l;
         Gs[r * GSTR + k] = (k <= r) ? l : R(0);
         if (r == k) dinv[k] = rinv;
 #pragma unroll
@@ -207,7 +207,7 @@ __global__ __launch_bounds__(DIAG_THREADS) void chol_diag_kernel(R *A, R *Minv, 
       __syncthreads();                        // panel p is in LDS
       R l[PW];
 #pragma unroll
-      for (int q = 0; q < PW; ++q) l[q] = Lcol[p & 1][q][r];
+      for (int q = 0; q < PW; ++q) l[q] = lcol(p & 1, q)[r];
       auto apply = [&](int j) __attribute__((always_inline)) {
 #pragma unroll
         for (int q = 0; q < PW; ++q) update(j, l[q]);
@@ -235,6 +235,7 @@ __global__ __launch_bounds__(DIAG_THREADS) void chol_diag_kernel(R *A, R *Minv, 
     }
     if (__any(bad) && r == 0) atomicMax(status, b + 1);
   } else {
+    if (ALIAS) __syncthreads();
     // ---- X = G^-1, lane j computes column j: x[i] = (delta_ij - sum_{k<i} G[i][k] x[k]) / G[i][i]
     rowvec x;
 #pragma unroll
@@ -256,17 +257,144 @@ __global__ __launch_bounds__(DIAG_THREADS) void chol_diag_kernel(R *A, R *Minv, 
   }
   __syncthreads();
   // M_bb[i][j] = G[63-j][63-i], Minv_bb[i][j] = X[63-j][63-i]  (i >= j), zero above; wavefronts 0-1
-  // write M_bb (half of the rows each), 2-3 the inverse
+  // write M_bb (half of the rows each), 2-3 the inverse (all four the inverse where M_bb is not wanted)
   if (wave < 4) {
-    const int half = wave & 1;
-    if (wave < 2) {
-      for (int i = half * (NB / 2); i < (half + 1) * (NB / 2); ++i)
-        D[(int64_t)i * ld + r] = (i >= r) ? Gs[(NB - 1 - r) * GSTR + (NB - 1 - i)] : R(0);
-    } else {
-      for (int i = half * (NB / 2); i < (half + 1) * (NB / 2); ++i)
+    if (Mout == nullptr) {
+      for (int i = wave * (NB / 4); i < (wave + 1) * (NB / 4); ++i)
         Dinv[(int64_t)i * ld + r] = (i >= r) ? Xs[(NB - 1 - r) * XSTR + (NB - 1 - i)] : R(0);
+    } else {
+      const int half = wave & 1;
+      if (wave < 2) {
+        for (int i = half * (NB / 2); i < (half + 1) * (NB / 2); ++i)
+          Mout[(int64_t)i * ld + r] = (i >= r) ? Gs[(NB - 1 - r) * GSTR + (NB - 1 - i)] : R(0);
+      } else {
+        for (int i = half * (NB / 2); i < (half + 1) * (NB / 2); ++i)
+          Dinv[(int64_t)i * ld + r] = (i >= r) ? Xs[(NB - 1 - r) * XSTR + (NB - 1 - i)] : R(0);
+      }
     }
   }
+}
+
+template <typename R>
+__global__ __launch_bounds__(DIAG_THREADS) void chol_diag_kernel(R *A, R *Minv, int64_t ld, int b,
+                                                                 int32_t *status) {
+  __shared__ __attribute__((aligned(16))) R dinv[NB];        // 1 / G[k][k]
+  __shared__ __attribute__((aligned(16))) R Gs[NB * GSTR];   // G, row major
+  __shared__ __attribute__((aligned(16))) R Xs[NB * (NB + 1)];   // X = G^-1, row major
+  __shared__ __attribute__((aligned(16))) R Lcol[2 * PW * NB];   // the columns of a panel of G, by panel parity
+  R *D = A + (int64_t)b * NB * ld + (int64_t)b * NB;
+  R *Dinv = Minv + (int64_t)b * NB * ld + (int64_t)b * NB;
+  chol_diag_block<R, false>(D, ld, D, Dinv, ld, b, status, dinv, Gs, Xs, Lcol);
+}
+
+// ---------------------------------------------------------------- one launch per step of the factorisation (fp32)
+// Block b is factorised and its inverse is in Minv[b, b].  What the chain of three launches did per step (solve the
+// block's panel, update everything above and to the left of it, factorise block b - 1) is one launch here: a
+// workgroup owns the 64 x 64 tile (i, j), j <= i < b, of the trailing matrix, and
+//   * solves the panel pieces it needs itself, P_i = Minv_bb^T H[b, i], P_j = Minv_bb^T H[b, j] (each piece is
+//     solved by every workgroup of its tile row and column: 2.1 Mflop, against a launch and its latency); the
+//     unsolved panel stays where it is in A, the tiles on the diagonal write their piece to Minv[b, i], which is
+//     where the merging step reads it;
+//   * updates its tile, A[i, j] -= P_i^T P_j;
+//   * the workgroup of tile (b - 1, b - 1), the first to be dispatched, keeps the updated tile in LDS and
+//     factorises it on the spot (chol_diag_block).
+// Every product is the MFMA sequence of gemm_f32_tn_k64_kernel on the same operands, so the factor is bit for
+// bit the one of the three-launch chain.  52 KB of LDS: three workgroups per CU.
+constexpr int STEP_LD = GSTR;
+constexpr int STEP_MAT = NB * STEP_LD;
+constexpr int STEP_LDS_BYTES = 3 * STEP_MAT * (int)sizeof(float);
+static_assert(NB * (NB + 1) <= STEP_MAT && 2 * PW * NB + NB <= STEP_MAT, "the block's arrays fit the operand buffers");
+
+// SOLVED: the panel has been solved by a launch of its own and lies in Minv[b, :]; the workgroups only update and
+// factorise (late steps have up to 2016 tiles, whose redundant solves take longer than that launch).
+template <bool SOLVED>
+__global__ __launch_bounds__(DIAG_THREADS) void chol_step_kernel(float *A, float *Minv, int64_t ld, int b,
+                                                                 int32_t *status) {
+  extern __shared__ __attribute__((aligned(16))) float step_lds[];
+  float *Dv = step_lds, *Hm = step_lds + STEP_MAT, *Hn = step_lds + 2 * STEP_MAT;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // tile (i, j), j <= i, the last one first
+  const int t = b * (b + 1) / 2 - 1 - (int)blockIdx.x;
+  int i = (int)((sqrtf(8.f * (float)t + 1.f) - 1.f) * 0.5f);
+  while ((i + 1) * (i + 2) / 2 <= t) ++i;
+  while (i * (i + 1) / 2 > t) --i;
+  const int j = t - i * (i + 1) / 2;
+  const bool on_diag = i == j;
+  const bool factor = blockIdx.x == 0;            // tile (b - 1, b - 1)
+  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
+  float *C = A + (int64_t)i * NB * ld + (int64_t)j * NB;
+  float cv[16];
+  if (wave < 4) {
+    const float *Dsrc = Minv + (int64_t)b * NB * ld + (int64_t)b * NB;
+    const float *Hrow = (SOLVED ? Minv : A) + (int64_t)b * NB * ld;
+    const int r = tid >> 4, c4 = (tid & 15) * 4;
+    float4 rd[4], rm[4], rn[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (!SOLVED) rd[q] = *reinterpret_cast<const float4 *>(Dsrc + (int64_t)(r + 16 * q) * ld + c4);
+      rm[q] = *reinterpret_cast<const float4 *>(Hrow + (int64_t)(r + 16 * q) * ld + i * NB + c4);
+      rn[q] = *reinterpret_cast<const float4 *>(Hrow + (int64_t)(r + 16 * q) * ld + j * NB + c4);
+    }
+#pragma unroll
+    for (int q = 0; q < 16; ++q)
+      cv[q] = C[(int64_t)(wm * 32 + 8 * (q >> 2) + 4 * lhi + (q & 3)) * ld + wn * 32 + l32];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (!SOLVED) *reinterpret_cast<float4 *>(&Dv[(r + 16 * q) * STEP_LD + c4]) = rd[q];
+      *reinterpret_cast<float4 *>(&Hm[(r + 16 * q) * STEP_LD + c4]) = rm[q];
+      *reinterpret_cast<float4 *>(&Hn[(r + 16 * q) * STEP_LD + c4]) = rn[q];
+    }
+  }
+  __syncthreads();
+  floatx16 pm, pn;
+#pragma unroll
+  for (int q = 0; q < 16; ++q) pm[q] = pn[q] = 0.f;
+  if (!SOLVED && wave < 4) {
+#pragma unroll 8
+    for (int kk = 0; kk < NB; kk += 2) {
+      const int krow = kk + lhi;
+      const float a = Dv[krow * STEP_LD + wm * 32 + l32];
+      pm = __builtin_amdgcn_mfma_f32_32x32x2f32(a, Hm[krow * STEP_LD + wn * 32 + l32], pm, 0, 0, 0);
+      if (!on_diag) pn = __builtin_amdgcn_mfma_f32_32x32x2f32(a, Hn[krow * STEP_LD + wn * 32 + l32], pn, 0, 0, 0);
+    }
+  }
+  if (!SOLVED) __syncthreads();                   // the unsolved pieces have been read
+  if (!SOLVED && wave < 4) {
+    float *Pout = Minv + (int64_t)b * NB * ld + (int64_t)i * NB;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      const int row = wm * 32 + 8 * (q >> 2) + 4 * lhi + (q & 3), col = wn * 32 + l32;
+      Hm[row * STEP_LD + col] = pm[q];
+      if (on_diag) Pout[(int64_t)row * ld + col] = pm[q];
+      else Hn[row * STEP_LD + col] = pn[q];
+    }
+  }
+  if (!SOLVED) __syncthreads();
+  if (wave < 4) {
+    const float *Pn = on_diag ? Hm : Hn;
+    floatx16 acc;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) acc[q] = 0.f;
+#pragma unroll 8
+    for (int kk = 0; kk < NB; kk += 2) {
+      const int krow = kk + lhi;
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(Hm[krow * STEP_LD + wm * 32 + l32], Pn[krow * STEP_LD + wn * 32 + l32],
+                                                 acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      const int row = wm * 32 + 8 * (q >> 2) + 4 * lhi + (q & 3), col = wn * 32 + l32;
+      const float v = cv[q] - acc[q];
+      if (factor) Dv[row * STEP_LD + col] = v;
+      else C[(int64_t)row * ld + col] = v;
+    }
+  }
+  if (!factor) return;
+  __syncthreads();                                // the updated block is in Dv; the solved pieces have been read
+  __builtin_amdgcn_s_setprio(3);
+  float *Dinv = Minv + (int64_t)(b - 1) * NB * ld + (int64_t)(b - 1) * NB;
+  chol_diag_block<float, true>(Dv, STEP_LD, nullptr, Dinv, ld, b - 1, status, Hn + 2 * PW * NB, Dv, Hm, Hn);
 }
 
 template <typename R>
@@ -326,7 +454,47 @@ int damp_invert(hipStream_t st, R *H, float *W, int64_t K, int64_t N, int64_t ld
   // (K = 28672: 352 ms with one level, 194 ms with two); below K = 6144 the trailing matrix stays
   // in the caches and one level (OUTER = 1) has fewer, larger launches.
   const int OUTER = Kp >= 6144 ? 8 : 1;
-  for (int b1 = nblk; b1 > 0;) {
+  // fp32, one level: one launch per step; the solved panels go to Minv, where the merging step finds them
+  const bool fused = sizeof(R) == 4 && OUTER == 1;
+  if constexpr (sizeof(R) == 4) {
+    if (fused) {
+      if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(chol_step_kernel<false>), STEP_LDS_BYTES) ||
+          !gptq_raise_lds_limit(reinterpret_cast<const void *>(chol_step_kernel<true>), STEP_LDS_BYTES))
+        return GPTQ_HIP_ELAUNCH;
+      // from 32 blocks on (528 tiles) the panel is solved by a launch of its own (5 us): the tiles' redundant solves
+      // would take longer
+      constexpr int bsplit = 32;
+      hipLaunchKernelGGL(chol_diag_kernel<R>, dim3(1), dim3(DIAG_THREADS), 0, st, p.A, p.Minv, Kp, nblk - 1, status);
+      GPTQ_CHECK_LAUNCH();
+      for (int b = nblk - 1; b > 0; --b) {
+        const dim3 grid((unsigned)(b * (b + 1) / 2));
+        if (b >= bsplit) {
+          // Minv[b, 0:b] <- Minv_bb^T A[b, 0:b]
+          GemmArgs g;
+          g.A = p.Minv + (int64_t)b * NB * Kp + (int64_t)b * NB;
+          g.B = p.A + (int64_t)b * NB * Kp;
+          g.C = p.Minv + (int64_t)b * NB * Kp;
+          g.lda = g.ldb = g.ldc = Kp;
+          g.m = NB;
+          g.n = b * NB;
+          g.k = NB;
+          g.alpha = 1.f;
+          g.beta = 0.f;
+          g.a_kmajor = 1;
+          g.in_dtype = DT;
+          const int rc = gptq_gemm(st, g, (R *)nullptr);
+          if (rc) return rc;
+          hipLaunchKernelGGL(chol_step_kernel<true>, grid, dim3(DIAG_THREADS), STEP_LDS_BYTES, st,
+                             reinterpret_cast<float *>(p.A), reinterpret_cast<float *>(p.Minv), Kp, b, status);
+        } else {
+          hipLaunchKernelGGL(chol_step_kernel<false>, grid, dim3(DIAG_THREADS), STEP_LDS_BYTES, st,
+                             reinterpret_cast<float *>(p.A), reinterpret_cast<float *>(p.Minv), Kp, b, status);
+        }
+        GPTQ_CHECK_LAUNCH();
+      }
+    }
+  }
+  for (int b1 = fused ? 0 : nblk; b1 > 0;) {
     const int b0 = ((b1 - 1) / OUTER) * OUTER;      // outer block = diagonal blocks [b0, b1)
     for (int b = b1 - 1; b >= b0; --b) {
       hipLaunchKernelGGL(chol_diag_kernel<R>, dim3(1), dim3(DIAG_THREADS), 0, st, p.A, p.Minv, Kp, b, status);
@@ -417,7 +585,7 @@ int damp_invert(hipStream_t st, R *H, float *W, int64_t K, int64_t N, int64_t ld
     };
     // T = C * Ainv
     GemmArgs g;
-    g.A = p.A + s * Kp;             // C of pair 0: rows [s, 2s), cols [0, s)
+    g.A = (fused ? p.Minv : p.A) + s * Kp;   // C of pair 0: rows [s, 2s), cols [0, s)
     g.B = p.Minv;                   // Ainv of pair 0
     g.C = p.T + s * Kp;
     g.lda = g.ldb = g.ldc = Kp;

@@ -23,7 +23,7 @@ def _spd(seed, K, n, scale_cols=False):
     return (x.T @ x / n).astype(np.float32)
 
 
-@pytest.mark.parametrize("K", [128, 256, 300, 37, 640, 1024])
+@pytest.mark.parametrize("K", [128, 256, 300, 37, 640, 1024, 2240])     # 2240: 35 diagonal blocks, both forms of the step kernel
 def test_cholesky_inv_matches_lapack(G, K):
     H = _spd(K, K, 4 * K, scale_cols=True)
     H += 0.01 * np.mean(np.diag(H)) * np.eye(K, dtype=np.float32)
