@@ -10,9 +10,12 @@
 // H^-1 = M^-1 M^-T = L L^T with L lower triangular and a positive diagonal, which is the
 // unique Cholesky factor the reference computes.
 //
-// All O(K^3) work runs on the MFMA GEMM; only the NB x NB diagonal blocks are factorised
-// and inverted by a single wavefront.  Everything is templated on the scalar type R:
-// float is the default path, double the reference's use_fp64 option (gptq.py:182-197).
+// All O(K^3) work runs on MFMAs; only the NB x NB diagonal blocks are factorised and
+// inverted with vector instructions, by five wavefronts.  Everything is templated on the
+// scalar type R: float is the default path, double the reference's use_fp64 option
+// (gptq.py:182-197).  In fp32 a step of the factorisation (solve the block's panel, update
+// what lies above and left of it, factorise the next diagonal block) is one launch
+// (chol_step_kernel), or two where the panel is long; fp64 keeps three launches per step.
 #include "common.h"
 #include "gemm_f32.h"
 #include "tile_io.h"
@@ -454,10 +457,27 @@ int damp_invert(hipStream_t st, R *H, float *W, int64_t K, int64_t N, int64_t ld
   // (K = 28672: 352 ms with one level, 194 ms with two); below K = 6144 the trailing matrix stays
   // in the caches and one level (OUTER = 1) has fewer, larger launches.
   const int OUTER = Kp >= 6144 ? 8 : 1;
-  // fp32, one level: one launch per step; the solved panels go to Minv, where the merging step finds them
-  const bool fused = sizeof(R) == 4 && OUTER == 1;
+  // fp32: one launch per step, or two; the solved panels go to Minv, where the outer updates and the merging step
+  // find them
+  const bool fused = sizeof(R) == 4;
+  auto solve_panel = [&](int b) -> int {
+    // Minv[b, 0:b] <- Minv_bb^T A[b, 0:b]
+    GemmArgs g;
+    g.A = p.Minv + (int64_t)b * NB * Kp + (int64_t)b * NB;
+    g.B = p.A + (int64_t)b * NB * Kp;
+    g.C = p.Minv + (int64_t)b * NB * Kp;
+    g.lda = g.ldb = g.ldc = Kp;
+    g.m = NB;
+    g.n = b * NB;
+    g.k = NB;
+    g.alpha = 1.f;
+    g.beta = 0.f;
+    g.a_kmajor = 1;
+    g.in_dtype = DT;
+    return gptq_gemm(st, g, (R *)nullptr);
+  };
   if constexpr (sizeof(R) == 4) {
-    if (fused) {
+    if (fused && OUTER == 1) {
       if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(chol_step_kernel<false>), STEP_LDS_BYTES) ||
           !gptq_raise_lds_limit(reinterpret_cast<const void *>(chol_step_kernel<true>), STEP_LDS_BYTES))
         return GPTQ_HIP_ELAUNCH;
@@ -469,20 +489,7 @@ int damp_invert(hipStream_t st, R *H, float *W, int64_t K, int64_t N, int64_t ld
       for (int b = nblk - 1; b > 0; --b) {
         const dim3 grid((unsigned)(b * (b + 1) / 2));
         if (b >= bsplit) {
-          // Minv[b, 0:b] <- Minv_bb^T A[b, 0:b]
-          GemmArgs g;
-          g.A = p.Minv + (int64_t)b * NB * Kp + (int64_t)b * NB;
-          g.B = p.A + (int64_t)b * NB * Kp;
-          g.C = p.Minv + (int64_t)b * NB * Kp;
-          g.lda = g.ldb = g.ldc = Kp;
-          g.m = NB;
-          g.n = b * NB;
-          g.k = NB;
-          g.alpha = 1.f;
-          g.beta = 0.f;
-          g.a_kmajor = 1;
-          g.in_dtype = DT;
-          const int rc = gptq_gemm(st, g, (R *)nullptr);
+          const int rc = solve_panel(b);
           if (rc) return rc;
           hipLaunchKernelGGL(chol_step_kernel<true>, grid, dim3(DIAG_THREADS), STEP_LDS_BYTES, st,
                              reinterpret_cast<float *>(p.A), reinterpret_cast<float *>(p.Minv), Kp, b, status);
@@ -491,6 +498,45 @@ int damp_invert(hipStream_t st, R *H, float *W, int64_t K, int64_t N, int64_t ld
                              reinterpret_cast<float *>(p.A), reinterpret_cast<float *>(p.Minv), Kp, b, status);
         }
         GPTQ_CHECK_LAUNCH();
+      }
+    } else if (fused) {
+      // two levels: inside an outer block the workgroups update the tiles of its rows only (tiles (i, j), b0 <= i < b,
+      // j <= i: the last b (b + 1) / 2 - b0 (b0 + 1) / 2 of the enumeration); the outer block's first diagonal block
+      // stands alone, behind the update with k = OUTER * NB
+      if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(chol_step_kernel<true>), STEP_LDS_BYTES))
+        return GPTQ_HIP_ELAUNCH;
+      for (int b1 = nblk; b1 > 0;) {
+        const int b0 = ((b1 - 1) / OUTER) * OUTER;
+        hipLaunchKernelGGL(chol_diag_kernel<R>, dim3(1), dim3(DIAG_THREADS), 0, st, p.A, p.Minv, Kp, b1 - 1, status);
+        GPTQ_CHECK_LAUNCH();
+        for (int b = b1 - 1; b >= b0 && b > 0; --b) {
+          int rc = solve_panel(b);
+          if (rc) return rc;
+          if (b == b0) break;
+          const dim3 grid((unsigned)(b * (b + 1) / 2 - b0 * (b0 + 1) / 2));
+          hipLaunchKernelGGL(chol_step_kernel<true>, grid, dim3(DIAG_THREADS), STEP_LDS_BYTES, st,
+                             reinterpret_cast<float *>(p.A), reinterpret_cast<float *>(p.Minv), Kp, b, status);
+          GPTQ_CHECK_LAUNCH();
+        }
+        if (b0 > 0) {
+          // A[0:b0, 0:b0] -= P^T P, P = the outer block's solved rows, columns 0 .. b0*NB  (lower tiles)
+          const R *outer = p.Minv + (int64_t)b0 * NB * Kp;
+          GemmArgs s;
+          s.A = outer;
+          s.B = outer;
+          s.C = p.A;
+          s.lda = s.ldb = s.ldc = Kp;
+          s.m = s.n = b0 * NB;
+          s.k = (b1 - b0) * NB;
+          s.alpha = -1.f;
+          s.beta = 1.f;
+          s.a_kmajor = 1;
+          s.in_dtype = DT;
+          s.tri = 2;
+          const int rc = gptq_gemm(st, s, (R *)nullptr);
+          if (rc) return rc;
+        }
+        b1 = b0;
       }
     }
   }
