@@ -83,11 +83,11 @@ def test_damp_and_invert_dead_feature_and_damping(G):
     assert np.abs(L - Lr).max() < 1e-3 * np.abs(Lr).max()
 
 
-def test_not_positive_definite_is_flagged(G):
+@pytest.mark.parametrize("K,idx", [(160, 3), (2240, 700)])     # the pivot fails inside a step of either form
+def test_not_positive_definite_is_flagged(G, K, idx):
     import torch
-    K = 160
     H = _spd(5, K, 4 * K)
-    H[3, 3] = -1.0
+    H[idx, idx] = -1.0
     _, _, bad = G._damp_and_invert(torch.zeros((K, 4), device="cuda"), torch.from_numpy(H).cuda(), 0.0)
     assert bad
     with pytest.raises(ValueError):
