@@ -292,14 +292,20 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
 // {a 2^-24, b 2^-24}, and one packed fma with the channels' scale 2^15 and -zero scale 2^-9 (the tables hold
 // them in that form) yields (code - zero) scale 2^-9: two vector instructions per operand register; the epilogue
 // multiplies by 512.
-template <typename TX, bool HALF = false, int BITS = 4>
+template <typename TX, int HALFM = 0, int BITS = 4>
 __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M, const uint8_t *pk, int R, int C,
                                                                const void *zero, const void *scale, int zs_dtype,
                                                                TX *out, float *out32, const int32_t *rowexp) {
   constexpr bool BF = Act<TX>::BF;
-  // (HALF: 128 rows x 256 output columns, the four wavefronts as two row halves x two column halves, as forward)
+  // (HALFM != 0: 128 rows x 256 output columns.  1: the four wavefronts as two row halves x two column halves, as
+  //  forward.  2 (SIDE): the four wavefronts side by side with all 128 rows and 64 columns each: half the groups of
+  //  packed rows per wavefront and everything else as in the full tile, so the operand instructions per MFMA stay
+  //  what they are there, while the activation reads from LDS double.  M = 2048 on 4096 x 11008: 8-bit codes
+  //  239 -> 204 us, 4-bit codes with fp16 rows 221 -> 211 us, with bf16 rows 223 -> 228 us, which therefore keep
+  //  form 1)
   static_assert(BITS == 4 || (BITS == 8 && !BF), "8-bit codes: fp16 rows");
-  constexpr int RB = HALF ? 4 : 8, TB = 8, NG = BITS == 8 ? 8 : 4;
+  constexpr bool HALF = HALFM != 0, SIDE = HALFM == 2;
+  constexpr int RB = (HALF && !SIDE) ? 4 : 8, TB = 8, NG = (BITS == 8 ? 8 : 4) / (SIDE ? 2 : 1);
   // fp16: halves sc[C], halves nzs[C]; bf16: floats sf[C], words {128 + rint z | z - rint z}[C]; then the stages
   extern __shared__ __attribute__((aligned(16))) float wide_lds[];
   _Float16 *tab_s = reinterpret_cast<_Float16 *>(wide_lds);
@@ -313,8 +319,8 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   const int g = lane >> 4, l16 = lane & 15;
   int tx, ty;
   qmm_tile_coords(tx, ty);
-  const int rb0 = HALF ? 4 * (wk >> 1) : 0;
-  const int m0 = ty * 128, j0 = (HALF ? tx * 2 + (wk & 1) : tx * 4 + wk) * (16 * NG);
+  const int rb0 = (HALF && !SIDE) ? 4 * (wk >> 1) : 0;
+  const int m0 = ty * 128, j0 = ((HALF && !SIDE) ? tx * 2 + (wk & 1) : tx * 4 + wk) * (16 * NG);
   const int NS = C >> 6;
 
   const int kc = tid & 7;
@@ -480,7 +486,7 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
           const uint32_t sel = (i & 1) ? 0x04030402u : 0x04010400u;
           nl[i] = build_lo(word, sel, jg + 1 < NG ? sw[i] : swn[i], jg + 1 < NG ? nw[i] : nwn[i]);
         };
-        if constexpr (!HALF) {
+        if constexpr (!HALF || SIDE) {
 #pragma unroll
           for (int rb = 0; rb < RB; ++rb) {
             if (rb & 1) Act<TX>::mma_acc_nw_after(acc[rb][jg], __builtin_bit_cast(uint4, a[rb]), Bl, nl[rb >> 1]);
@@ -502,7 +508,7 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
           Act<TX>::mma_acc_nw_after(acc[3][jg], __builtin_bit_cast(uint4, a[3]), Bl, nl[3]);
           __builtin_amdgcn_sched_barrier(0);
         }
-      } else if constexpr (!HALF) {
+      } else if constexpr (!HALF || SIDE) {
 #pragma unroll
         for (int n = 0; n < 16; ++n) {
           const int rb = n >> 1, i = n >> 2;
@@ -512,8 +518,14 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
             piece(n >> 1);
           } else {
             Act<TX>::mma_acc_nw_after(acc[rb][2 * jg + 1], __builtin_bit_cast(uint4, a[rb]), Bh, hi_piece ? nh[i] : nl[i]);
-            if constexpr (SCP >= 0)
-              if ((n & 3) == 1) scale_unit(SCP, 4 * jg + (n >> 2), sf);
+            // the sixteen units of the stage being scaled, spread over the k-step's groups
+            if constexpr (SCP >= 0) {
+              if constexpr (NG == 4) {
+                if ((n & 3) == 1) scale_unit(SCP, 4 * jg + (n >> 2), sf);
+              } else {
+                scale_unit(SCP, 8 * jg + (n >> 1), sf);
+              }
+            }
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -706,7 +718,8 @@ template <typename TX, int BITS = 4>
 int launch_bwd_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
                     const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32, const int32_t *rowexp,
                     bool half) {
-  auto kern = half ? qmm_bwd_wide_kernel<TX, true, BITS> : qmm_bwd_wide_kernel<TX, false, BITS>;
+  // 128 x 256 tiles: four wavefronts side by side, except for bf16 rows (two by two)
+  auto kern = half ? qmm_bwd_wide_kernel<TX, Act<TX>::BF ? 1 : 2, BITS> : qmm_bwd_wide_kernel<TX, 0, BITS>;
   const int lds = (int)((Act<TX>::BF ? 8 : 4) * C + 2 * 2 * 8 * 64 * 16);
   if (!gptq_raise_lds_limit(reinterpret_cast<const void *>(kern), lds)) return GPTQ_HIP_ELAUNCH;
   const int64_t KO = BITS == 8 ? R : 2 * R;
