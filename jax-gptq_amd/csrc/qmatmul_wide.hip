@@ -26,9 +26,11 @@ namespace {
 
 using namespace qmm;
 
-// HALF: a 128 x 256 tile, the four wavefronts as two row halves x two column halves of 64 x 128 each (for shapes
-// whose 128 x 512 tiles are under one round of workgroups): the two wavefronts of a column half build the same
-// weight operands, the two of a row half share their row sums.
+// HALF: a 128 x 256 tile (for shapes whose 128 x 512 tiles are under one round of workgroups), the four wavefronts
+// side by side with all 128 rows and 64 channels each (a lane loads 4 bytes = 4 channels of each of its rows): the
+// operand instructions per MFMA stay those of the 128 x 512 tile, the activation reads from LDS double.  (As two
+// row halves x two column halves of 64 x 128 each, every operand was built twice: M = 2048 on 11008 x 4096 took
+// 205 us against 186, with bf16 rows 192 against 175, with 8-bit codes 202 against 188.)
 //
 // BITS = 8 (one code per byte, K = R, fp16 rows): a lane loads 8 bytes of each of its eight rows of a k-step; the
 // bytes of two rows that a byte permute pairs ARE fp16 subnormals {a 2^-24, b 2^-24}, and one packed fma with
@@ -45,7 +47,9 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
   constexpr int NRW = BITS == 8 ? 8 : 4;         // packed rows of a lane per k-step
   constexpr int NT = 64 * NWV;
   constexpr int CH = 1024 / NT;                  // 16-byte pieces of a stage per thread
-  constexpr int RB = HALF ? 4 : 8;               // row blocks of a wavefront
+  constexpr int RB = 8;                          // row blocks of a wavefront
+  constexpr int NTL = HALF ? 4 : 8;              // product tiles (16 channels) of a wavefront's row block
+  constexpr int CPL = HALF ? 4 : 8;              // channels of a lane
   constexpr int TB = 8;                          // row blocks of the workgroup's tile
   __shared__ u32x4_t a_lds[2 * 2 * TB * 64];       // [slot][k-step of the stage][row block][lane]
   asm volatile("" ::"s"(x), "s"(pk), "s"(zero), "s"(scale), "s"(out), "s"(M), "s"(K), "s"(C), "s"(zs_dtype),
@@ -54,10 +58,11 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
   const int g = lane >> 4, l16 = lane & 15;
   int tx, ty;
   qmm_tile_coords(tx, ty);
-  const int rb0 = HALF ? 4 * (wk >> 1) : 0;      // first row block of this wavefront
-  const int m0 = ty * 128, nbase = c0 + (HALF ? tx * 2 + (wk & 1) : tx * NWV + wk) * 128;
+  constexpr int rb0 = 0;                         // first row block of this wavefront
+  const int m0 = ty * 128;
+  const int nbase = c0 + (tx * NWV + wk) * (16 * NTL);
   const int NS = K >> 6;
-  const int col = nbase + 8 * l16;
+  const int col = nbase + CPL * l16;
 
   // this thread's pieces of a stage: row (tid >> 3) + (NT / 8) i of the tile, k 8 (tid & 7) .. + 7 of the stage
   const int kc = tid & 7;
@@ -86,7 +91,10 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
   auto load_w = [&](int p, int h, int s) __attribute__((always_inline)) {
     const uint8_t *q = wp + (int64_t)(8 * NRW * min(s, NS - 1) + 4 * NRW * h) * C;
 #pragma unroll
-    for (int i = 0; i < NRW; ++i) wr[p][h][i] = *reinterpret_cast<const uint2 *>(q + (int64_t)i * C);
+    for (int i = 0; i < NRW; ++i) {
+      if constexpr (HALF) wr[p][h][i] = make_uint2(*reinterpret_cast<const uint32_t *>(q + (int64_t)i * C), 0u);
+      else wr[p][h][i] = *reinterpret_cast<const uint2 *>(q + (int64_t)i * C);
+    }
   };
   auto read_a = [&](int q, int slot, int h) __attribute__((always_inline)) {
     const int sl = lane ^ (4 * g) ^ (2 * h);
@@ -160,31 +168,15 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
   auto step_pipe = [&](const u32x4_t (&a)[RB], const u32x4_t (&ar)[2], const uint2 (&w)[NRW], const uint2 (&wn)[NRW]) __attribute__((always_inline)) {
     uint32_t bc[4] = {bcarry[0], bcarry[1], bcarry[2], bcarry[3]};
 #pragma unroll
-    for (int t8 = 0; t8 < 8; ++t8) {
+    for (int t8 = 0; t8 < NTL; ++t8) {
       const uint4 b = make_uint4(bc[0], bc[1], bc[2], bc[3]);
       uint32_t nx[4] = {0u, 0u, 0u, 0u};
-      auto dq_next = [&](int i) __attribute__((always_inline)) { nx[i] = t8 < 7 ? dq_reg(w, t8 + 1, i) : dq_reg(wn, 0, i); };
-      if constexpr (!HALF) {
+      auto dq_next = [&](int i) __attribute__((always_inline)) { nx[i] = t8 < NTL - 1 ? dq_reg(w, t8 + 1, i) : dq_reg(wn, 0, i); };
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-          if (rb & 1) Act<TX>::mma_acc_nw_after(acc[rb][t8], __builtin_bit_cast(uint4, a[rb]), b, nx[rb >> 1]);
-          else Act<TX>::mma_acc_nw(acc[rb][t8], __builtin_bit_cast(uint4, a[rb]), b);
-          if (!(rb & 1)) dq_next(rb >> 1);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      } else {
-        // four MFMAs per tile: all four operand registers of the next tile are built before the last of them
-        Act<TX>::mma_acc_nw(acc[0][t8], __builtin_bit_cast(uint4, a[0]), b);
-        dq_next(0);
-        dq_next(1);
-        __builtin_amdgcn_sched_barrier(0);
-        Act<TX>::mma_acc_nw_after2(acc[1][t8], __builtin_bit_cast(uint4, a[1]), b, nx[0], nx[1]);
-        dq_next(2);
-        __builtin_amdgcn_sched_barrier(0);
-        Act<TX>::mma_acc_nw_after(acc[2][t8], __builtin_bit_cast(uint4, a[2]), b, nx[2]);
-        dq_next(3);
-        __builtin_amdgcn_sched_barrier(0);
-        Act<TX>::mma_acc_nw_after(acc[3][t8], __builtin_bit_cast(uint4, a[3]), b, nx[3]);
+      for (int rb = 0; rb < RB; ++rb) {
+        if (rb & 1) Act<TX>::mma_acc_nw_after(acc[rb][t8], __builtin_bit_cast(uint4, a[rb]), b, nx[rb >> 1]);
+        else Act<TX>::mma_acc_nw(acc[rb][t8], __builtin_bit_cast(uint4, a[rb]), b);
+        if (!(rb & 1)) dq_next(rb >> 1);
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
@@ -255,7 +247,7 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
       const float rs = rs4[r];
       TX o[8];
 #pragma unroll
-      for (int t8 = 0; t8 < 8; ++t8)
+      for (int t8 = 0; t8 < NTL; ++t8)
         o[t8] = Act<TX>::out(sc[t8] * ((BITS == 8 ? 512.f * acc[rb][t8][r] : acc[rb][t8][r]) - zfa[t8] * rs));
       if (out32 != nullptr) {
         // fp32 rows: the fp16 result widened and scaled back by the row's power of two (exact)
@@ -263,12 +255,13 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
         float *d32 = out32 + (int64_t)m * C + col;
         float f[8];
 #pragma unroll
-        for (int t8 = 0; t8 < 8; ++t8) f[t8] = ldexpf((float)o[t8], e);
+        for (int t8 = 0; t8 < NTL; ++t8) f[t8] = ldexpf((float)o[t8], e);
         *reinterpret_cast<float4 *>(d32) = make_float4(f[0], f[1], f[2], f[3]);
-        *reinterpret_cast<float4 *>(d32 + 4) = make_float4(f[4], f[5], f[6], f[7]);
+        if constexpr (!HALF) *reinterpret_cast<float4 *>(d32 + 4) = make_float4(f[4], f[5], f[6], f[7]);
         continue;
       }
-      *reinterpret_cast<uint4 *>(out + (int64_t)m * C + col) = *reinterpret_cast<const uint4 *>(o);
+      if constexpr (HALF) *reinterpret_cast<uint2 *>(out + (int64_t)m * C + col) = *reinterpret_cast<const uint2 *>(o);
+      else *reinterpret_cast<uint4 *>(out + (int64_t)m * C + col) = *reinterpret_cast<const uint4 *>(o);
     }
   }
 }
