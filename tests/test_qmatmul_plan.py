@@ -70,7 +70,11 @@ def test_headline_cases_run_on_the_kernels_the_design_names(N):
     assert _plan(N, 64, 11008, 4096, 0, "BF16", 4, 1)["kernel"] == "qmm_fwd_mid_kernel"
     assert _plan(N, 128, 11008, 4096, 0, "F16", 4, 1)["kernel"].startswith("qmm_fwd_reg_kernel")
     big = _plan(N, 2048, 11008, 4096, 0, "F16", 4, 1)
-    assert big["kernel"].startswith("qmm_fwd_wide_kernel") and big["rest"].startswith("qmm_fwd_reg_kernel")
+    # the leading 8192 channels on 128 x 512 tiles, the 2816 behind them on 128 x 256 tiles
+    assert big["kernel"] == "qmm_fwd_wide_kernel (128 x 512)" and big["rest"] == "qmm_fwd_wide_kernel (128 x 256)"
+    # where those would be more than a round, the 128-row register-operand tiles take the rest
+    big2 = _plan(N, 4096, 11008, 4096, 0, "F16", 4, 1)
+    assert big2["kernel"].startswith("qmm_fwd_wide_kernel") and big2["rest"].startswith("qmm_fwd_reg_kernel")
     assert _plan(N, 2048, 11008, 4096, 1, "F16", 4, 1)["kernel"].startswith("qmm_bwd_wide_kernel")
     assert _plan(N, 2048, 11008, 4096, 1, "BF16", 4, 1)["kernel"].startswith("qmm_bwd_wide_kernel")
     # bf16 rows: the constants of more than 16384 channels do not fit beside the stages
