@@ -1816,7 +1816,8 @@ int qmatmul_impl(void *stream, const void *x, int x_dtype, int64_t M, const uint
     const int64_t ty = ceil_div64(M, 16 * bp.rb);
     if (parts.wide_x > 0)
       planned(parts.half ? GPTQ_HIP_QMM_BWD_WIDE_HALF : GPTQ_HIP_QMM_BWD_WIDE,
-              parts.main_x > 0 ? GPTQ_HIP_QMM_BWD_REG128 : (parts.tail > 0 ? GPTQ_HIP_QMM_BWD_REG64 : 0), 1,
+              parts.wide2_x > 0 ? GPTQ_HIP_QMM_BWD_WIDE_HALF
+                                : (parts.main_x > 0 ? GPTQ_HIP_QMM_BWD_REG128 : (parts.tail > 0 ? GPTQ_HIP_QMM_BWD_REG64 : 0)), 1,
               parts.wide_x * ceil_div64(M, 128));
     else
       planned(parts.main_x > 0 ? own : GPTQ_HIP_QMM_BWD_REG64,

@@ -31,7 +31,7 @@ RegPlan reg_fwd_plan(int64_t M, int64_t R, int64_t C, int bits, bool aligned);
 struct RegParts {
   int64_t wide_x;
   bool half;
-  int64_t wide2_x;         // 8-bit codes: 256-channel tiles behind the whole rounds of 512-channel ones (part of `first`)
+  int64_t wide2_x;         // 256-channel (transposed: 256-column) tiles behind the whole rounds of 512-wide ones (part of `first`)
   int64_t first, main_x, tail;
 };
 RegParts reg_fwd_parts(const RegPlan &p, int64_t M, int64_t R, int64_t C, bool bf16, int group_size);
@@ -73,7 +73,7 @@ int wide_fwd_launch(hipStream_t st, const void *x, int x_dtype, int64_t M, const
 int64_t wide_bwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half, bool bf16 = false, int bits = 4);
 int wide_bwd_launch(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
                     const void *scale, int zs_dtype, void *out, int64_t wide_x, bool half, float *out32,
-                    const int32_t *rowexp, bool bf16 = false, int bits = 4);
+                    const int32_t *rowexp, bool bf16 = false, int bits = 4, int64_t jbase = 0);
 
 // Transposed product out[M, K] = x[M, C] @ dequant(packed[R, C])^T.
 struct RegBwdPlan {

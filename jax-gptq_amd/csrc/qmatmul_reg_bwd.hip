@@ -398,6 +398,11 @@ int launch_bx(hipStream_t st, const RegBwdPlan &p, const void *x, int64_t M, con
                                      Act<TX>::BF, BITS);
       if (rc) return rc;
     }
+    if (q.wide2_x > 0) {
+      const int rc = wide_bwd_launch(st, x, M, pk, R, C, zero, scale, zs_dtype, out, q.wide2_x, true, p.out32, p.rowexp,
+                                     Act<TX>::BF, BITS, (BITS == 8 ? 512 : 256) * q.wide_x);
+      if (rc) return rc;
+    }
     if (q.main_x > 0) {
       const int rc = p.ragged ? launch_inst<BITS, true, TX, 8>(st, p, x, M, pk, R, C, zero, scale, zs_dtype, out, ws,
                                                                group_size, q.first, q.main_x)
@@ -433,6 +438,15 @@ RegParts reg_bwd_parts(const RegBwdPlan &p, int64_t M, int64_t R, int64_t C, boo
   if ((p.bits == 4 || !bf16) && !p.ragged && !p.no_wide && group_size == 0) {
     q.wide_x = wide_bwd_tiles(M, R, C, true, &q.half, bf16, p.bits);
     if (q.wide_x > 0) q.first = (q.half ? 2 : 4) * q.wide_x;
+    // what is left behind whole rounds of 512-column tiles goes to 256-column tiles if those fill half a round or more
+    if (q.wide_x > 0 && !q.half) {
+      const int64_t rows512 = p.bits == 8 ? 512 : 256;
+      const int64_t n2 = (R - rows512 * q.wide_x) / (rows512 / 2);
+      if (n2 * tiles_y >= 128 && n2 * tiles_y <= 256) {
+        q.wide2_x = n2;
+        q.first += 2 * n2;
+      }
+    }
   }
   const int64_t rest = tiles_all - q.first;
   if (rest == 0) return q;

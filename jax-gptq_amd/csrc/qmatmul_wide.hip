@@ -288,7 +288,8 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
 template <typename TX, int HALFM = 0, int BITS = 4>
 __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M, const uint8_t *pk, int R, int C,
                                                                const void *zero, const void *scale, int zs_dtype,
-                                                               TX *out, float *out32, const int32_t *rowexp) {
+                                                               TX *out, float *out32, const int32_t *rowexp, int jbase) {
+  // jbase: first packed row of this launch's tiles (where the output columns are dealt over two launches)
   constexpr bool BF = Act<TX>::BF;
   // (HALFM != 0: 128 rows x 256 output columns.  1: the four wavefronts as two row halves x two column halves, as
   //  forward.  2 (SIDE): the four wavefronts side by side with all 128 rows and 64 columns each: half the groups of
@@ -313,7 +314,7 @@ __global__ __launch_bounds__(256, 1) void qmm_bwd_wide_kernel(const TX *x, int M
   int tx, ty;
   qmm_tile_coords(tx, ty);
   const int rb0 = (HALF && !SIDE) ? 4 * (wk >> 1) : 0;
-  const int m0 = ty * 128, j0 = ((HALF && !SIDE) ? tx * 2 + (wk & 1) : tx * 4 + wk) * (16 * NG);
+  const int m0 = ty * 128, j0 = jbase + ((HALF && !SIDE) ? tx * 2 + (wk & 1) : tx * 4 + wk) * (16 * NG);
   const int NS = C >> 6;
 
   const int kc = tid & 7;
@@ -710,7 +711,7 @@ int launch_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int
 template <typename TX, int BITS = 4>
 int launch_bwd_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
                     const void *scale, int zs_dtype, void *out, int64_t wide_x, float *out32, const int32_t *rowexp,
-                    bool half) {
+                    bool half, int64_t jbase) {
   // 128 x 256 tiles: four wavefronts side by side, except for bf16 rows (two by two)
   auto kern = half ? qmm_bwd_wide_kernel<TX, Act<TX>::BF ? 1 : 2, BITS> : qmm_bwd_wide_kernel<TX, 0, BITS>;
   const int lds = (int)((Act<TX>::BF ? 8 : 4) * C + 2 * 2 * 8 * 64 * 16);
@@ -725,7 +726,7 @@ int launch_bwd_wide(hipStream_t st, const void *x, int64_t M, const uint8_t *pk,
     const dim3 grid((unsigned)wide_x, (unsigned)ceil_div64(rows, 128), 1);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (const TX *)x + r0 * C, (int)rows, pk, (int)R, (int)C, zero,
                        scale, zs_dtype, (TX *)out + r0 * KO, out32 ? out32 + r0 * KO : nullptr,
-                       rowexp ? rowexp + r0 : nullptr);
+                       rowexp ? rowexp + r0 : nullptr, (int)jbase);
     GPTQ_CHECK_LAUNCH();
   }
   return GPTQ_HIP_OK;
@@ -784,18 +785,20 @@ int64_t wide_bwd_tiles(int64_t M, int64_t R, int64_t C, bool aligned, bool *half
 
 int wide_bwd_launch(hipStream_t st, const void *x, int64_t M, const uint8_t *pk, int64_t R, int64_t C, const void *zero,
                     const void *scale, int zs_dtype, void *out, int64_t wide_x, bool half, float *out32,
-                    const int32_t *rowexp, bool bf16, int bits) {
+                    const int32_t *rowexp, bool bf16, int bits, int64_t jbase) {
   if (zs_dtype != GPTQ_HIP_F32 && zs_dtype != GPTQ_HIP_F16 && zs_dtype != GPTQ_HIP_BF16) return GPTQ_HIP_EDTYPE;
-  if (wide_x < 1 || wide_x * (half ? 128 : 256) * (bits == 8 ? 2 : 1) > R) return GPTQ_HIP_EINVAL;
+  if (wide_x < 1 || jbase < 0 || jbase % 64 != 0 || jbase + wide_x * (half ? 128 : 256) * (bits == 8 ? 2 : 1) > R)
+    return GPTQ_HIP_EINVAL;
   if (bits == 8) {
     if (bf16) return GPTQ_HIP_EDTYPE;
-    return launch_bwd_wide<__half, 8>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half);
+    return launch_bwd_wide<__half, 8>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half, jbase);
   }
   if (bf16) {
     if (out32 || C > 16384) return GPTQ_HIP_EINVAL;
-    return launch_bwd_wide<__hip_bfloat16>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, nullptr, nullptr, half);
+    return launch_bwd_wide<__hip_bfloat16>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, nullptr, nullptr, half,
+                                           jbase);
   }
-  return launch_bwd_wide<__half>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half);
+  return launch_bwd_wide<__half>(st, x, M, pk, R, C, zero, scale, zs_dtype, out, wide_x, out32, rowexp, half, jbase);
 }
 
 }  // namespace qmm
