@@ -2,8 +2,17 @@
 // 128 x 512 output tiles whose four wavefronts stand side by side.
 //
 // Each wavefront owns a 128 x 128 output tile over ALL of K (8 x 8 product tiles in the 256 accumulation
-// registers) and builds its weight operands in registers from its own 128 channels, exactly as the 128-row tiles
-// of qmatmul_reg.hip do.  What differs is the activations: the four wavefronts need the same 128 rows, so a
+// registers) and builds its weight operands in registers from its own 128 channels (lane (l16, g): 8 bytes = 8
+// channels of each packed row that holds its 8 k of the k-step; product tile t8 takes byte t8 of every row).
+//
+// fp16 rows: the weight operand is the RAW codes read as fp16 subnormals, which the MFMA multiplies exactly: a
+// byte permute puts byte t8 into both halves of a register and one mask leaves {lo, hi << 4} = {lo 2^-24,
+// 16 hi 2^-24}: two vector instructions per operand register, no conversion.  The 16 goes to the other operand
+// (the activations of odd k are divided by 16 on their way into LDS, the row sums' operand holds 16 for them);
+// 2^24, the scale and the zero point (- zero sum_k x[m][k], the row sums from a ninth tile) wait for the epilogue.
+// bf16 rows: 128 + code (three instructions), the term (128 + zero) sum_k x leaves in the epilogue likewise.
+//
+// The activations: the four wavefronts need the same 128 rows, so a
 // stage of 64 k (16 KB) is fetched once per workgroup, 16 bytes per thread and piece, and laid into LDS in
 // operand order ([k-step][row block][lane]: a wavefront's operand register quad is one conflict-free 16-byte
 // read).  Per k-step a CU takes in 8 KB of activations + 4 x 2 KB of packed weights for 4 x 72 MFMAs, where
@@ -33,9 +42,8 @@ using namespace qmm;
 // 205 us against 186, with bf16 rows 192 against 175, with 8-bit codes 202 against 188.)
 //
 // BITS = 8 (one code per byte, K = R, fp16 rows): a lane loads 8 bytes of each of its eight rows of a k-step; the
-// bytes of two rows that a byte permute pairs ARE fp16 subnormals {a 2^-24, b 2^-24}, and one packed fma with
-// 2^15 and -rint(zero) 2^-9 yields (code - rint(zero)) 2^-9 exactly: two vector instructions per operand register
-// (three for 4-bit codes); the epilogue multiplies the sums by 512.
+// bytes of two rows that a byte permute pairs ARE the operand, fp16 subnormals {a 2^-24, b 2^-24}: one vector
+// instruction per operand register.
 template <int NWV, typename TX, bool HALF = false, int BITS = 4>
 __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, int M, int K, const uint8_t *pk, int C,
                                                                    const void *zero, const void *scale,
@@ -86,7 +94,24 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
   };
   auto write_a = [&](int p, int slot) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < CH; ++i) a_lds[slot * (2 * TB * 64) + dst0 + (NT / 128) * 64 * i] = stg[p][i];
+    for (int i = 0; i < CH; ++i) {
+      if constexpr (!BF && BITS == 4) {
+        // fp16 rows, 4-bit codes: the high nibbles enter the MFMA as 16 code 2^-24, so the activations of odd k
+        // enter divided by 16 (exact down to 2^-10; below that to 2^-25 absolute)
+        // (written as the instruction: the compiler's own packed multiply of the four words by this constant came
+        //  out as one multiply of the second word copied into all four)
+        const uint32_t odd16 = 0x2C003C00u;      // {1, 1/16}
+        const u32x4_t v = stg[p][i];
+        uint32_t e0, e1, e2, e3;
+        asm("v_pk_mul_f16 %0, %1, %2" : "=v"(e0) : "v"(v.x), "s"(odd16));
+        asm("v_pk_mul_f16 %0, %1, %2" : "=v"(e1) : "v"(v.y), "s"(odd16));
+        asm("v_pk_mul_f16 %0, %1, %2" : "=v"(e2) : "v"(v.z), "s"(odd16));
+        asm("v_pk_mul_f16 %0, %1, %2" : "=v"(e3) : "v"(v.w), "s"(odd16));
+        a_lds[slot * (2 * TB * 64) + dst0 + (NT / 128) * 64 * i] = u32x4_t{e0, e1, e2, e3};
+        continue;
+      }
+      a_lds[slot * (2 * TB * 64) + dst0 + (NT / 128) * 64 * i] = stg[p][i];
+    }
   };
   auto load_w = [&](int p, int h, int s) __attribute__((always_inline)) {
     const uint8_t *q = wp + (int64_t)(8 * NRW * min(s, NS - 1) + 4 * NRW * h) * C;
@@ -104,9 +129,6 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
     for (int j = 0; j < 2; ++j) aqr[q][j] = a_lds[((slot * 2 + h) * TB + 2 * wk + j) * 64 + sl];
   };
 
-  uint32_t zraw0[8];
-  rg_params8_raw(zero, zs_dtype, 0, col, C, zraw0);
-  __builtin_amdgcn_sched_barrier(0);
   load_a(1, 0);
   load_w(0, 0, 0);
   load_w(0, 1, 0);
@@ -115,18 +137,11 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
   load_w(1, 1, 1);
   __builtin_amdgcn_sched_barrier(0);
 
-  uint32_t zc[8];
-#pragma unroll
-  for (int t8 = 0; t8 < 8; ++t8) {
-    const float zi = fminf(fmaxf(rintf(rg_raw_to_f32(zraw0[t8], zs_dtype)), -512.f), 512.f);
-    if (BITS == 8) zc[t8] = __builtin_bit_cast(uint32_t, half2_t{(_Float16)(-zi * 0x1p-9f), (_Float16)(-zi * 0x1p-9f)});
-    else zc[t8] = BF ? 0u : __builtin_bit_cast(uint32_t, half2_t{(_Float16)(-(1024.f + zi)), (_Float16)(-(64.f + zi))});
-  }
-  uint32_t mask = BF ? 0x000F000Fu : 0x00F0000Fu, cexp = BF ? 0x43004300u : 0x64006400u;
+  uint32_t mask = BF ? 0x000F000Fu : 0x00F0000Fu, cexp = 0x43004300u;
   asm volatile("" : "+s"(mask));
   asm volatile("" : "+v"(cexp));
-  const half2_t unscale = BITS == 8 ? half2_t{(_Float16)32768.f, (_Float16)32768.f} : half2_t{(_Float16)1.f, (_Float16)0.0625f};
-  const uint32_t one2 = BF ? 0x3F803F80u : 0x3C003C00u;
+  // the row sums' operand: ones (fp16 rows with 4-bit codes: 16 for the odd k, whose activations enter divided by 16)
+  const uint32_t one2 = BF ? 0x3F803F80u : (BITS == 4 ? 0x4C003C00u : 0x3C003C00u);
   uint4 ones = make_uint4(one2, one2, one2, one2);
   asm volatile("" : "+v"(ones.x), "+v"(ones.y), "+v"(ones.z), "+v"(ones.w));      // kept in registers: not rebuilt in front of an MFMA
 
@@ -140,19 +155,15 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
   auto dq_reg = [&](const uint2 (&w)[NRW], int t8, int i) __attribute__((always_inline)) -> uint32_t {
     const uint32_t tb = (uint32_t)(t8 & 3);
     if constexpr (BITS == 8) {
-      // byte t8 of rows 2 i (even k, low half) and 2 i + 1 (odd k): {a 2^-24, b 2^-24} -> (code - zi) 2^-9
+      // byte t8 of rows 2 i (even k, low half) and 2 i + 1 (odd k): the operand as it stands, {a 2^-24, b 2^-24}
       const uint32_t sel8 = 0x0c000c00u | tb | ((4u + tb) << 16);
-      const uint32_t pb = t8 < 4 ? __builtin_amdgcn_perm(w[2 * i + 1].x, w[2 * i].x, sel8)
-                                 : __builtin_amdgcn_perm(w[2 * i + 1].y, w[2 * i].y, sel8);
-      const half2_t d = __builtin_bit_cast(half2_t, pb) * unscale + __builtin_bit_cast(half2_t, zc[t8]);
-      return __builtin_bit_cast(uint32_t, d);
+      return t8 < 4 ? __builtin_amdgcn_perm(w[2 * i + 1].x, w[2 * i].x, sel8)
+                    : __builtin_amdgcn_perm(w[2 * i + 1].y, w[2 * i].y, sel8);
     }
     const uint32_t sel = BF ? (0x0c0c0c00u | tb) : (0x0c000c00u | tb | (tb << 16));
     const uint32_t pb = __builtin_amdgcn_perm(0u, t8 < 4 ? w[i].x : w[i].y, sel);
     if (BF) return (((pb << 12) | pb) & mask) | cexp;                  // {128 + lo, 128 + hi}
-    const uint32_t v = (pb & mask) | cexp;                             // {1024 + lo, 1024 + 16 hi}
-    const half2_t d = __builtin_bit_cast(half2_t, v) * unscale + __builtin_bit_cast(half2_t, zc[t8]);
-    return __builtin_bit_cast(uint32_t, d);
+    return pb & mask;                                                  // {lo 2^-24, 16 hi 2^-24}
   };
   // One k-step: the in-place MFMAs are inline asm, which the scheduler does not move, so the source order is the
   // issue order: after every second MFMA of a tile the three vector instructions of one operand register of the
@@ -233,10 +244,9 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
   __syncthreads();
   float zfa[8];
 #pragma unroll
-  for (int t8 = 0; t8 < 8; ++t8)
-    zfa[t8] = BF ? 128.f + zf[t8] : zf[t8] - fminf(fmaxf(rintf(zf[t8]), -512.f), 512.f);
-  // acc[rb][t8][r] = sum_k x[m][k] (code - zi)[k][col + t8] (bf16: code + 128), rs_lds[rb][lane][r] = sum_k x[m][k],
-  // m = m0 + 16 rb + 4 g + r
+  for (int t8 = 0; t8 < 8; ++t8) zfa[t8] = BF ? 128.f + zf[t8] : zf[t8];
+  // acc[rb][t8][r] = sum_k x[m][k] code[k][col + t8] 2^-24 (bf16: code + 128, unscaled), rs_lds[rb][lane][r] =
+  // sum_k x[m][k], m = m0 + 16 rb + 4 g + r
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const floatx4 rs4 = rs_lds[(rb0 + rb) * 64 + lane];
@@ -248,7 +258,7 @@ __global__ __launch_bounds__(64 * NWV, 1) void qmm_fwd_wide_kernel(const TX *x, 
       TX o[8];
 #pragma unroll
       for (int t8 = 0; t8 < NTL; ++t8)
-        o[t8] = Act<TX>::out(sc[t8] * ((BITS == 8 ? 512.f * acc[rb][t8][r] : acc[rb][t8][r]) - zfa[t8] * rs));
+        o[t8] = Act<TX>::out(sc[t8] * ((BF ? acc[rb][t8][r] : 0x1p24f * acc[rb][t8][r]) - zfa[t8] * rs));
       if (out32 != nullptr) {
         // fp32 rows: the fp16 result widened and scaled back by the row's power of two (exact)
         const int e = rowexp[m];
