@@ -1,6 +1,7 @@
 // Blocked GPTQ column loop: quantise block_size rows with error feedback, then push the
-// accumulated error into the remaining rows with fp32 MFMA GEMMs: inside a 512-row group every
-// block first receives what the group's earlier blocks owe it, and after every group everything
+// accumulated error into the remaining rows with fp32 MFMAs: inside a 512-row group every
+// block first receives what the group's earlier blocks owe it (in the prologue of its own kernel,
+// or, for irregular shapes, in a product launch in front of it), and after every group everything
 // below it receives the group's errors in one product.
 //
 // In-block kernel: the N output channels are independent, so one lane owns one channel and a
@@ -21,6 +22,7 @@
 // bit-identical to a CPU evaluation of gptq.py:136-147.
 #include "common.h"
 #include "gemm_f32.h"
+#include "tile_io.h"
 #include <type_traits>
 #include <utility>
 
@@ -45,8 +47,14 @@ __device__ __forceinline__ void static_for(F &&f) {
 template <int SB, typename TQ>
 __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
     const float *Wb, int64_t N, const float *Lb, int64_t ldl, int bs, const float *scale,
-    const float *zero, float maxq, TQ *Qb, uint8_t *cb, float *Err) {
+    const float *zero, float maxq, TQ *Qb, uint8_t *cb, float *Err, const float *Lprev, const float *Eprev, int kprev) {
   // Wb, Qb, cb: first row of the block in W, Q, codes; Lb: the block's diagonal corner of L
+  // kprev > 0 (bs = 128, whole 64-channel tiles, 16-byte aligned rows; kprev a multiple of 64): the block's rows
+  // first receive what the kprev rows in front of them in their update group owe them,
+  //   W[block] - Lprev[128, kprev] @ Eprev[kprev, N]   (Lprev = L[block rows, group start ..], Eprev: those rows' errors),
+  // which a product launch of its own did before (14 - 24 us each, three per group of four blocks): here every
+  // workgroup forms its 128 x 64 tile of it with fp32 MFMAs, k ascending in one accumulator and the difference
+  // taken once, so the bits are those of that product.
 #pragma clang fp contract(off)
   extern __shared__ __attribute__((aligned(16))) float smem[];
   float *Ln = smem;                         // Ln[j * bs + i] = Lb[j][i] for i <= j (nothing right of the diagonal is read)
@@ -80,11 +88,12 @@ __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
     if (t < 0 || rows <= 0) return;
     if (vec) {
       // the first batch of the W tile goes out before the loads of L and is stored after them
-      const int totalw = rows * (SOLVE_CH / 4);
+      // (kprev > 0: the tile is in LDS already)
+      const int totalw = kprev > 0 ? 0 : rows * (SOLVE_CH / 4);
       f32x4 wv[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int idx = min(u * nthr + t, totalw - 1);
+        const int idx = max(min(u * nthr + t, totalw - 1), 0);
         const int j = idx / (SOLVE_CH / 4), c4 = idx - j * (SOLVE_CH / 4);
         wv[u] = *reinterpret_cast<const f32x4 *>(Wb + (int64_t)(row_lo + j) * N + n0 + 4 * c4);
       }
@@ -174,7 +183,7 @@ __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
           }
         }
       }
-      const int totalw = rows * SOLVE_CH;
+      const int totalw = kprev > 0 ? 0 : rows * SOLVE_CH;
       for (int base = 0; base < totalw; base += nthr * 16) {
         float v[16];
 #pragma unroll
@@ -247,6 +256,65 @@ __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
     }
   };
 
+  if (kprev > 0) {
+    // ---- the tile W[block] - Lprev @ Eprev into Wl.  Wavefront w: rows 32 (w >> 1) .. + 31, channels 32 (w & 1) .. + 31
+    // of the tile, as one 32 x 32 MFMA tile.  k in chunks of 64 through LDS (the regions of L's corner, of the tile
+    // and of the sub-block buffers, all filled afterwards): Lprev's chunk [128][64] with row stride 65, Eprev's
+    // [64][64] with row stride 68, two buffers, one barrier per chunk.
+    constexpr int KC = 64, LDA = KC + 1, LDB = SOLVE_CH + 4, BUF = 128 * LDA + KC * LDB;
+    constexpr int TPR = KC / 4, RPP = SOLVE_TPB / TPR, NPA = 128 / RPP;      // threads per row of Lprev's chunk, rows per pass, passes
+    constexpr int NPB = KC / (SOLVE_TPB / 16);                              // passes over Eprev's chunk (16 threads per row)
+    static_assert(2 * BUF * 4 <= (128 * 128 + 128 * SOLVE_CH + 6 * 16 * SOLVE_CH) * 4, "the chunk buffers fit in front of R1s");
+    const int rblk = wave >> 1, cblk = wave & 1, l32 = lane & 31, lhi = lane >> 5;
+    float cv[16];
+#pragma unroll
+    for (int q = 0; q < 16; ++q)
+      cv[q] = Wb[(int64_t)(32 * rblk + 8 * (q >> 2) + 4 * lhi + (q & 3)) * N + n0 + 32 * cblk + l32];
+    // this thread's pieces of a chunk: Lprev rows (tid / TPR) + RPP i, columns 4 (tid % TPR) .. + 3; Eprev rows
+    // (tid >> 4) + 32 i, channels 4 (tid & 15) .. + 3
+    const float *ap = Lprev + (int64_t)(tid / TPR) * ldl + 4 * (tid % TPR);
+    const float *bp = Eprev + (int64_t)(tid >> 4) * N + n0 + 4 * (tid & 15);
+    f32x4 ra[NPA], rb[NPB];
+    auto load_chunk = [&](int k0) __attribute__((always_inline)) {
+#pragma unroll
+      for (int i = 0; i < NPA; ++i) ra[i] = *reinterpret_cast<const f32x4 *>(ap + (int64_t)(RPP * i) * ldl + k0);
+#pragma unroll
+      for (int i = 0; i < NPB; ++i) rb[i] = *reinterpret_cast<const f32x4 *>(bp + (int64_t)(k0 + 32 * i) * N);
+    };
+    auto store_chunk = [&](float *buf) __attribute__((always_inline)) {
+      float *as = buf + (tid / TPR) * LDA + 4 * (tid % TPR);
+#pragma unroll
+      for (int i = 0; i < NPA; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) as[RPP * i * LDA + e] = ra[i][e];
+#pragma unroll
+      for (int i = 0; i < NPB; ++i)
+        *reinterpret_cast<f32x4 *>(buf + 128 * LDA + ((tid >> 4) + 32 * i) * LDB + 4 * (tid & 15)) = rb[i];
+    };
+    floatx16 acc;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) acc[q] = 0.f;
+    load_chunk(0);
+    store_chunk(smem);
+    __syncthreads();
+    int b = 0;
+    for (int k0 = 0; k0 < kprev; k0 += KC) {
+      const bool more = k0 + KC < kprev;
+      if (more) load_chunk(k0 + KC);
+      const float *as = smem + b * BUF + (32 * rblk + l32) * LDA + lhi;
+      const float *bs_ = smem + b * BUF + 128 * LDA + lhi * LDB + 32 * cblk + l32;
+#pragma unroll
+      for (int kk = 0; kk < KC; kk += 2) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(as[kk], bs_[kk * LDB], acc, 0, 0, 0);
+      if (more) store_chunk(smem + (b ^ 1) * BUF);
+      __syncthreads();
+      b ^= 1;
+    }
+#pragma unroll
+    for (int q = 0; q < 16; ++q)
+      Wl[(32 * rblk + 8 * (q >> 2) + 4 * lhi + (q & 3)) * SOLVE_CH + 32 * cblk + l32] = cv[q] - acc[q];
+    // (the loop's last barrier: every wavefront is done with the chunk buffers, which the staging below overwrites;
+    //  the tile itself is read after the barrier that follows the staging)
+  }
   stage(0, SB, tid, SOLVE_TPB);
   const float sc = scale[nl], z = zero[nl];
   const float rs = 1.0f / sc;
@@ -456,10 +524,16 @@ __global__ __launch_bounds__(SOLVE_TPB) void block_quant_kernel(
   store_sub(nsb - 1, wave, std::integral_constant<int, SOLVE_NW>{});
 }
 
+// Lprev / Eprev / kprev: see the kernel (kprev = 0: none)
+bool fused_update_ok(const float *W, int64_t N, const float *L, int64_t ldl, int bs, int64_t kprev) {
+  return bs == 128 && kprev > 0 && kprev % 64 == 0 && N % SOLVE_CH == 0 && (ldl & 3) == 0 &&
+         (reinterpret_cast<uintptr_t>(L) & 15) == 0 && (reinterpret_cast<uintptr_t>(W) & 15) == 0;
+}
+
 template <int SB>
 int launch_block(hipStream_t st, const float *W, int64_t N, const float *L, int64_t ldl, int bs,
                  const float *scale, const float *zero, float maxq, void *Q, int q_dtype,
-                 uint8_t *codes, float *Err) {
+                 uint8_t *codes, float *Err, const float *Lprev = nullptr, const float *Eprev = nullptr, int kprev = 0) {
   const dim3 grid((unsigned)ceil_div64(N, SOLVE_CH)), block(SOLVE_TPB);
   const size_t lds = ((size_t)bs * bs + (size_t)bs * SOLVE_CH + (size_t)6 * SB * SOLVE_CH + (size_t)bs) * sizeof(float);
   if (lds > 64 * 1024) {
@@ -474,15 +548,15 @@ int launch_block(hipStream_t st, const float *W, int64_t N, const float *L, int6
   switch (q_dtype) {
     case GPTQ_HIP_F32:
       hipLaunchKernelGGL((block_quant_kernel<SB, float>), grid, block, lds, st, W, N, L, ldl,
-                         bs, scale, zero, maxq, (float *)Q, codes, Err);
+                         bs, scale, zero, maxq, (float *)Q, codes, Err, Lprev, Eprev, kprev);
       break;
     case GPTQ_HIP_F16:
       hipLaunchKernelGGL((block_quant_kernel<SB, __half>), grid, block, lds, st, W, N, L, ldl,
-                         bs, scale, zero, maxq, (__half *)Q, codes, Err);
+                         bs, scale, zero, maxq, (__half *)Q, codes, Err, Lprev, Eprev, kprev);
       break;
     case GPTQ_HIP_BF16:
       hipLaunchKernelGGL((block_quant_kernel<SB, __hip_bfloat16>), grid, block, lds, st, W, N, L,
-                         ldl, bs, scale, zero, maxq, (__hip_bfloat16 *)Q, codes, Err);
+                         ldl, bs, scale, zero, maxq, (__hip_bfloat16 *)Q, codes, Err, Lprev, Eprev, kprev);
       break;
     default:
       return GPTQ_HIP_EDTYPE;
@@ -521,9 +595,9 @@ int trailing_update(hipStream_t st, const float *A, int64_t lda, const float *B,
 
 int process_block(hipStream_t st, const float *Wb, int64_t N, const float *Lb, int64_t ldl, int bs,
                   const float *scale, const float *zero, int maxq, void *Qb, int q_dtype,
-                  uint8_t *cb, float *Err) {
+                  uint8_t *cb, float *Err, const float *Lprev = nullptr, const float *Eprev = nullptr, int kprev = 0) {
 #define GPTQ_SB_CASE(SB) \
-  return launch_block<SB>(st, Wb, N, Lb, ldl, bs, scale, zero, (float)maxq, Qb, q_dtype, cb, Err)
+  return launch_block<SB>(st, Wb, N, Lb, ldl, bs, scale, zero, (float)maxq, Qb, q_dtype, cb, Err, Lprev, Eprev, kprev)
   if (bs % 16 == 0) GPTQ_SB_CASE(16);
   if (bs % 8 == 0) GPTQ_SB_CASE(8);
   if (bs % 4 == 0) GPTQ_SB_CASE(4);
@@ -589,10 +663,12 @@ int solve_impl(hipStream_t st, float *W, int64_t K, int64_t N, const float *L, c
         sc = scale_g + gi * N;
         zr = zero_g + gi * N;
       }
-      if (group_size == 0 && start > gs) {
-        // the block's rows receive what the earlier blocks of this update group owe them, in one product
-        // with k = start - gs (per-channel parameters: nothing reads the rows below the block before their
-        // own turn, so each row of the group is read and written once per group, not once per block above it)
+      // the block's rows receive what the earlier blocks of this update group owe them, in one product
+      // with k = start - gs (per-channel parameters: nothing reads the rows below the block before their
+      // own turn, so each row of the group is read and written once per group, not once per block above it):
+      // inside the block's own kernel where the shapes allow, else in a launch of its own
+      const bool fuse = group_size == 0 && start > gs && fused_update_ok(W + start * N, N, L, K, block_size, start - gs);
+      if (group_size == 0 && start > gs && !fuse) {
         const int rc = trailing_update(st, L + start * K + gs, K, Err, W + start * N, N, block_size, start - gs);
         if (rc) return rc;
       }
@@ -600,7 +676,8 @@ int solve_impl(hipStream_t st, float *W, int64_t K, int64_t N, const float *L, c
       uint8_t *cb = codes ? codes + start * N : nullptr;
       float *Eb = Err + (start - gs) * N;
       int rc = process_block(st, W + start * N, N, L + start * K + start, K, block_size, sc, zr, maxq, Qb,
-                             q_dtype, cb, Eb);
+                             q_dtype, cb, Eb, fuse ? L + start * K + gs : nullptr, fuse ? Err : nullptr,
+                             fuse ? (int)(start - gs) : 0);
       if (rc) return rc;
       const int64_t end = start + block_size;
       if (group_size > 0 && end < ge) {
