@@ -746,7 +746,7 @@ __device__ __forceinline__ void load_to_lds_16(const void *src, uint32_t dst) {
                : "memory", "m0");
 }
 
-template <typename T, typename ARGS>
+template <typename T, typename ARGS, bool PIECES = false>
 __global__ __launch_bounds__(256) void syrk16d_kernel(ARGS p) {
   extern __shared__ __attribute__((aligned(16))) char lds16d[];
   typedef typename Mfma16<T>::v8 v8;
@@ -762,17 +762,44 @@ __global__ __launch_bounds__(256) void syrk16d_kernel(ARGS p) {
       item = ((q >> 5) * 8u + xcd) * 32u + (q & 31u);
     }
   }
-  const int rs = (int)item / ntiles, t = (int)item - rs * ntiles;
-  int ti, tj;
-  tile_decode(t, p.T, ti, tj);
-  const int m0 = ti * W16_TB, n0 = tj * W16_TB, K = p.K;
+  static_assert(!(PIECES && ARGS::DUAL), "runs of (tile, slab) pairs: plain batches only");
+  const int K = p.K;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lhi = lane >> 5;
+  // PIECES: this workgroup's run [u0, u1) of the tile-major (tile, slab) pairs (see syrk32d_kernel); p.chunk
+  // holds the slabs per tile (rows of the call / 32)
+  int64_t u0 = 0, u1 = 0;
+  if (PIECES) {
+    const int64_t U = (int64_t)ntiles * p.chunk;
+    u0 = (int64_t)item * U / gridDim.x;
+    u1 = (int64_t)(item + 1) * U / gridDim.x;
+    if (u0 >= u1) return;
+  }
+  bool first_piece = true;
+  do {
+  int rs = 0, t, piece_rows = p.chunk;
+  int64_t g0;
+  bool whole = false;
+  if (PIECES) {
+    t = (int)(u0 / p.chunk);
+    const int s0 = (int)(u0 - (int64_t)t * p.chunk);
+    const int n = (int)min((int64_t)(p.chunk - s0), u1 - u0);
+    g0 = (int64_t)s0 * D16_BK;
+    piece_rows = n * D16_BK;
+    whole = n == p.chunk;
+    u0 += n;
+  } else {
+    rs = (int)item / ntiles;
+    t = (int)item - rs * ntiles;
+    g0 = (int64_t)rs * p.chunk;
+  }
+  int ti, tj;
+  tile_decode(t, p.T, ti, tj);
+  const int m0 = ti * W16_TB, n0 = tj * W16_TB;
 
-  // slice [g0, g0 + chunk) of the concatenated batches: first slab (b, kt), number of slabs
+  // rows [g0, g0 + piece_rows) of the concatenated batches: first slab (b, kt), number of slabs
   int b = 0, kt = 0, nslabs = 0;
   {
-    const int64_t g0 = (int64_t)rs * p.chunk;
     int64_t base = 0;
     bool started = false;
     int rem = 0;
@@ -782,7 +809,7 @@ __global__ __launch_bounds__(256) void syrk16d_kernel(ARGS p) {
         started = true;
         b = bb;
         kt = (int)(g0 - base);
-        rem = p.chunk;
+        rem = piece_rows;
       }
       if (started && rem > 0) {
         const int from = (bb == b) ? kt : 0;
@@ -960,18 +987,35 @@ __global__ __launch_bounds__(256) void syrk16d_kernel(ARGS p) {
     unit = *p.factor;
     accum = p.accum != 0;
   }
-  if (p.RS == 1) {
+  // (PIECES: offsets that do not change from piece to piece are hidden from the compiler, which would otherwise
+  // compute all 512 of them in front of the loop and park them in scratch memory)
+  int e_col = wn * 128 + l32, e_row = wm * 128 + 4 * lhi;
+  if (PIECES) asm volatile("" : "+v"(e_col), "+v"(e_row));
+  if (PIECES ? whole : p.RS == 1) {
 #pragma unroll
     for (int ii = 0; ii < 4; ++ii)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int col = n0 + wn * 128 + j * 32 + l32;
+        const int col = n0 + e_col + j * 32;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int row = m0 + wm * 128 + ii * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+          const int row = m0 + e_row + ii * 32 + 8 * (r >> 2) + (r & 3);
           p.H[(int64_t)row * K + col] += ARGS::DUAL ? acc[ii][j][r] * unit : acc[ii][j][r];
         }
       }
+  } else if (PIECES) {
+    // partial tile in register order, slot 2 w (the run's first piece) or 2 w + 1 (its last), as syrk32d_kernel
+    // stores it and syrk_reduce_pieces_kernel sums it
+    float4 *dst = reinterpret_cast<float4 *>(p.ws + (int64_t)(2 * item + (first_piece ? 0 : 1)) * (W16_TB * W16_TB)) +
+                  wave * 4096 + lane;
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq)
+          dst[((ii * 4 + j) * 4 + rq) * 64] =
+              make_float4(acc[ii][j][4 * rq], acc[ii][j][4 * rq + 1], acc[ii][j][4 * rq + 2], acc[ii][j][4 * rq + 3]);
   } else {
     float *dst = p.ws + ((int64_t)rs * ntiles + t) * (W16_TB * W16_TB);
 #pragma unroll
@@ -993,6 +1037,10 @@ __global__ __launch_bounds__(256) void syrk16d_kernel(ARGS p) {
         }
       }
   }
+  if (!PIECES) break;
+  first_piece = false;
+  __syncthreads();           // the next piece's loads reuse the slab buffers
+  } while (u0 < u1);
 }
 
 // ---------------------------------------------------------------------------- fp32 inputs, loads straight into LDS
@@ -1416,15 +1464,16 @@ int pick_rs_call(int64_t K, int64_t total_rows, int slab_rows, double us_per_row
 }
 constexpr double H_US_PER_ROW_F32 = 0.228, H_US_PER_ROW_16 = 0.0305;
 
-// The (tile, slab) runs of syrk32d_kernel<true>: G workgroups (one round), two partial-tile slots each.  A run is
-// one chain of MFMA accumulations, so the call may not be longer than H_CHAIN_ROWS rows (see
-// gptq_hip_hessian_accumulate); runs shorter than eight slabs are not worth their pipeline fill.
+// The (tile, slab) runs of syrk32d_kernel<true> and of syrk16d_kernel<.., true> (slabs of slab_rows rows): G
+// workgroups (one round), two partial-tile slots each.  A run is one chain of MFMA accumulations, so the call may
+// not be longer than H_CHAIN_ROWS rows (see gptq_hip_hessian_accumulate); runs shorter than eight slabs are not
+// worth their pipeline fill.
 struct PiecesPlan { bool use; int G; size_t ws_bytes; };
-PiecesPlan pieces_plan(int64_t K, int64_t total_rows) {
+PiecesPlan pieces_plan(int64_t K, int64_t total_rows, int slab_rows) {
   PiecesPlan pp{false, 0, 0};
-  if (!use_wide16(K) || K % W16_TB != 0 || total_rows <= 0 || total_rows % D32_BK != 0 || total_rows > H_CHAIN_ROWS)
+  if (!use_wide16(K) || K % W16_TB != 0 || total_rows <= 0 || total_rows % slab_rows != 0 || total_rows > H_CHAIN_ROWS)
     return pp;
-  const int64_t T = K / W16_TB, nt = T * (T + 1) / 2, U = nt * (total_rows / D32_BK);
+  const int64_t T = K / W16_TB, nt = T * (T + 1) / 2, U = nt * (total_rows / slab_rows);
   int64_t G = U / 8;
   if (G > 256) G = 256;
   if (G < 1) return pp;
@@ -1685,6 +1734,30 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
       bool regular = (K % W16_TB == 0);
       for (int i = 0; i < w.nb; ++i) regular = regular && (w.rows[i] % D16_BK == 0);
       const bool f16 = x_dtype == GPTQ_HIP_F16;
+      // a short call: equal runs of (tile, slab) pairs over one round of workgroups, as for fp32 batches below.
+      // Measured against the row slices (512 .. 4096 rows per call): 10 - 50 % faster up to K = 4608 (171 tiles,
+      // where no number of slices fills the rounds), slower from K = 5120 on: no two workgroups of a run
+      // partition are at the same rows at the same time, every one streams its own pair of panels, and at the
+      // rate of these matrix instructions the reads of X then bound the kernel.  (Fewer runs than tiles: a very
+      // short call, one workgroup per tile is better.)
+      const PiecesPlan pp = (regular && nt <= 171) ? pieces_plan(K, total_rows, D16_BK) : PiecesPlan{false, 0, 0};
+      if (pp.use && pp.G >= nt && ws && ws_bytes >= pp.ws_bytes) {
+        const void *pfn = f16 ? reinterpret_cast<const void *>(syrk16d_kernel<__half, SyrkArgs, true>)
+                              : reinterpret_cast<const void *>(syrk16d_kernel<__hip_bfloat16, SyrkArgs, true>);
+        if (!gptq_raise_lds_limit(pfn, D16_LDS_BYTES)) return GPTQ_HIP_ELAUNCH;
+        const int64_t s32 = total_rows / D16_BK;
+        w.chunk = (int)s32;
+        if (f16)
+          hipLaunchKernelGGL((syrk16d_kernel<__half, SyrkArgs, true>), dim3((unsigned)pp.G), block, D16_LDS_BYTES, st, w);
+        else
+          hipLaunchKernelGGL((syrk16d_kernel<__hip_bfloat16, SyrkArgs, true>), dim3((unsigned)pp.G), block, D16_LDS_BYTES,
+                             st, w);
+        GPTQ_CHECK_LAUNCH();
+        hipLaunchKernelGGL(syrk_reduce_pieces_kernel, dim3((unsigned)(nt * (W16_TB * W16_TB / 4096))), dim3(256), 0, st, H,
+                           w.ws, (int)K, w.T, (int)s32, pp.G);
+        GPTQ_CHECK_LAUNCH();
+        continue;
+      }
       const void *fn = regular ? (f16 ? reinterpret_cast<const void *>(syrk16d_kernel<__half, SyrkArgs>)
                                       : reinterpret_cast<const void *>(syrk16d_kernel<__hip_bfloat16, SyrkArgs>))
                                : (f16 ? reinterpret_cast<const void *>(syrk16w_kernel<__half>)
@@ -1748,7 +1821,7 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
       w.chunk = (int)chunk;
       // a short call: equal runs of (tile, slab) pairs over one round of workgroups instead of row slices,
       // where the model says so (time of a run + what the two partial tiles per workgroup cost)
-      const PiecesPlan pp = pieces_plan(K, total_rows);
+      const PiecesPlan pp = pieces_plan(K, total_rows, D32_BK);
       if (pp.use && ws && ws_bytes >= pp.ws_bytes) {
         const double sliced = (double)ceil_div64(nt * w.RS, 256) * (H_US_PER_ROW_F32 * (double)chunk + 30.0);
         const double pieces = H_US_PER_ROW_F32 * (double)total_rows * (double)nt / (double)pp.G + 50.0;

@@ -260,6 +260,37 @@ def test_accumulate_H_short_calls_in_equal_runs_of_tile_slabs(G, rows, K, nb):
     assert np.abs(to_np(Hs) / n - ref1).max() < TOL * max(1.0, np.abs(ref1).max())
 
 
+@pytest.mark.parametrize("rows,K,nb,dt", [(2048, 4096, 1, "float16"), (2048, 4096, 1, "bfloat16"), (2048, 6144, 1, "float16"),
+                                          (32, 1024, 1, "float16"), (64, 1024, 1, "bfloat16"), (160, 2048, 3, "float16"),
+                                          (1024, 1024, 2, "bfloat16"), (2048, 11008, 1, "float16"),
+                                          (4096, 4096, 2, "float16"), (2080, 4096, 1, "bfloat16"), (512, 4096, 1, "float16")])
+def test_accumulate_H_short_16bit_calls_in_equal_runs_of_tile_slabs(G, rows, K, nb, dt):
+    """The same partition for fp16 / bf16 batches (32-row slabs): every tile cut, whole tiles inside the runs,
+    fewer pairs than workgroups, several batches per call, slab counts that the runs do not divide.  Products of
+    two 16-bit numbers are exact in fp32, so the bar is the closed form of the widened rows to fp32 summation
+    error; a zero feature gives exact zeros; the same bits on a second call; a second step ADDS."""
+    import torch
+    rng = np.random.default_rng(rows + K + nb)
+    tdt = getattr(torch, dt)
+    dev = [torch.from_numpy(rng.standard_normal((rows, K)).astype(np.float32)).to(tdt).cuda() for _ in range(nb)]
+    for x in dev:
+        x[:, 5] = 0.0
+    xs = [x.float().cpu().numpy() for x in dev]
+    H = to_np(G.accumulate_H(dev))
+    ref = _closed_form(xs)
+    assert H.shape == (K, K) and np.array_equal(H, H.T)
+    assert np.abs(H - ref).max() < TOL * max(1.0, np.abs(ref).max())
+    assert np.all(H[5] == 0) and np.all(H[:, 5] == 0)
+    assert np.array_equal(H, to_np(G.accumulate_H(dev)))
+    Hs = torch.zeros((K, K), dtype=torch.float32, device="cuda")
+    mean = torch.zeros((K,), dtype=torch.float32, device="cuda")
+    Hs, mean, n = G._accumulate_H_step(Hs, mean, 0, dev[0])
+    Hs, mean, n = G._accumulate_H_step(Hs, mean, n, dev[0])
+    assert n == 2 * rows
+    ref1 = _closed_form(xs[:1])
+    assert np.abs(to_np(Hs) / n - ref1).max() < TOL * max(1.0, np.abs(ref1).max())
+
+
 @pytest.mark.parametrize("rows,K,nb,dt", [(64, 384, 5, "float32"), (37, 200, 4, "float32"), (256, 1024, 6, "float32"),
                                           (2048, 4096, 3, "float32"), (96, 1280, 4, "float16"),
                                           (50, 520, 3, "bfloat16")])
