@@ -1169,16 +1169,22 @@ __global__ __launch_bounds__(256) void syrk32d_kernel(SyrkArgs p) {
     load_to_lds_16(src + (int64_t)j * K, dst + j * D32_ROW);
   };
 
-  // operand reads of k pair kp: row 2 kp + lhi, feature (32-feature block) + l32
-  const uint32_t rd_a = (uint32_t)(lhi * D32_ROW + (wm * 128 + l32) * 4);
-  const uint32_t rd_b = (uint32_t)(D32_OP + lhi * D32_ROW + (wn * 128 + l32) * 4);
+  // operand reads of k pair kp: row 2 kp + lhi, features 4 l32 .. 4 l32 + 3 of the wavefront's 128 in ONE 16-byte
+  // read per operand: MFMA block q of an operand is the features 4 i + q (i = 0 .. 31: the MFMA's row / column i),
+  // not 32 q + i - which rows of the tile an accumulator holds is free, and this choice takes 2 LDS reads per
+  // 16 MFMAs instead of 8
+  const uint32_t rd_a = (uint32_t)(lhi * D32_ROW + (wm * 128 + 4 * l32) * 4);
+  const uint32_t rd_b = (uint32_t)(D32_OP + lhi * D32_ROW + (wn * 128 + 4 * l32) * 4);
   struct Ops { float a[4], b[4]; };
   auto read_ops = [&](int buf, int kp, Ops &o) __attribute__((always_inline)) {
     const lds_char *base = (const lds_char *)lds32d + buf * D32_SLAB + kp * 2 * D32_ROW;
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const f32x4 va = *reinterpret_cast<const __attribute__((address_space(3))) f32x4 *>(base + rd_a);
+    const f32x4 vb = *reinterpret_cast<const __attribute__((address_space(3))) f32x4 *>(base + rd_b);
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      o.a[q] = *reinterpret_cast<const __attribute__((address_space(3))) float *>(base + rd_a + q * 128);
-      o.b[q] = *reinterpret_cast<const __attribute__((address_space(3))) float *>(base + rd_b + q * 128);
+      o.a[q] = va[q];
+      o.b[q] = vb[q];
     }
   };
 
@@ -1254,22 +1260,23 @@ __global__ __launch_bounds__(256) void syrk32d_kernel(SyrkArgs p) {
     mfma_all(prev);          // last k pair of the last slab
   }
 
+  // accumulator acc[ii][j][r] is row 4 i + ii, column 4 l32 + j of the wavefront's 128 x 128, i = 8 (r / 4) + 4 lhi
+  // + r % 4: the four j of a lane are adjacent columns, 16 bytes of a row
   // (PIECES: the element offsets below do not change from piece to piece; left visible, the compiler computes
-  // all 512 of them in front of the loop and parks them in scratch memory, and a kernel with that much scratch
+  // them all in front of the loop and parks them in scratch memory, and a kernel with that much scratch
   // pays for its allocation at every launch)
-  int e_col = wn * 128 + l32, e_row = wm * 128 + 4 * lhi;
+  int e_col = wn * 128 + 4 * l32, e_row = wm * 128 + 16 * lhi;
   if (PIECES) asm volatile("" : "+v"(e_col), "+v"(e_row));
   if (PIECES ? whole : p.RS == 1) {
 #pragma unroll
     for (int ii = 0; ii < 4; ++ii)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int col = n0 + e_col + j * 32;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = m0 + e_row + ii * 32 + 8 * (r >> 2) + (r & 3);
-          p.H[(int64_t)row * K + col] += acc[ii][j][r];
-        }
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + e_row + 32 * (r >> 2) + 4 * (r & 3) + ii;
+        float4 *hp = reinterpret_cast<float4 *>(p.H + (int64_t)row * K + n0 + e_col);
+        float4 h = *hp;
+        h.x += acc[ii][0][r]; h.y += acc[ii][1][r]; h.z += acc[ii][2][r]; h.w += acc[ii][3][r];
+        *hp = h;
       }
   } else if (PIECES) {
     // a partial tile is the workgroup's first piece (slot 2 w) or, whole tiles in between, its last.  It is
@@ -1290,13 +1297,10 @@ __global__ __launch_bounds__(256) void syrk32d_kernel(SyrkArgs p) {
 #pragma unroll
     for (int ii = 0; ii < 4; ++ii)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int col = e_col + j * 32;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = e_row + ii * 32 + 8 * (r >> 2) + (r & 3);
-          dst[row * W16_TB + col] = acc[ii][j][r];
-        }
+      for (int r = 0; r < 16; ++r) {
+        const int row = e_row + 32 * (r >> 2) + 4 * (r & 3) + ii;
+        *reinterpret_cast<float4 *>(dst + row * W16_TB + e_col) =
+            make_float4(acc[ii][0][r], acc[ii][1][r], acc[ii][2][r], acc[ii][3][r]);
       }
   }
   if (!PIECES) break;
@@ -1307,7 +1311,9 @@ __global__ __launch_bounds__(256) void syrk32d_kernel(SyrkArgs p) {
 
 // PIECES form of the reduction: the partial tiles of tile t lie in the slots of the workgroups whose runs cut it
 // (see syrk32d_kernel); H tile += their sum in workgroup order.  A tile that one workgroup covered alone has
-// been added already.  G workgroups, S slabs per tile.
+// been added already.  G workgroups, S slabs per tile.  PERM: the accumulators' rows and columns as
+// syrk32d_kernel deals them (a lane's four column blocks are adjacent columns, its rows four apart).
+template <bool PERM>
 __global__ __launch_bounds__(256) void syrk_reduce_pieces_kernel(float *H, const float *ws, int K, int T, int S, int G) {
   constexpr int TB = W16_TB, RED_PARTS = TB * TB / 4096;
   const int ntiles = T * (T + 1) / 2;
@@ -1321,7 +1327,10 @@ __global__ __launch_bounds__(256) void syrk_reduce_pieces_kernel(float *H, const
   int ti, tj;
   tile_decode(t, T, ti, tj);
   const int m0 = ti * TB, n0 = tj * TB;
-  // float4 number e of a partial tile holds rows r .. r + 3 of one column (the kernel's register order)
+  // float4 number e of a partial tile holds the accumulator's registers r .. r + 3 of one lane (the kernel's
+  // register order): e = (((wave * 4 + ii) * 4 + j) * 4 + r / 4) * 64 + lane; a thread's four numbers are j = 0 .. 3.
+  // Plain order: rows row .. row + 3 of column block j.  PERM: column j of the lane's four adjacent columns, rows
+  // row, row + 4, row + 8, row + 12 - the thread reads and writes H in rows of 16 bytes.
   float4 s[4], h[4];
   int e[4];
   float *hp[4];
@@ -1330,9 +1339,16 @@ __global__ __launch_bounds__(256) void syrk_reduce_pieces_kernel(float *H, const
     e[u] = part * 1024 + u * 256 + threadIdx.x;
     s[u] = make_float4(0.f, 0.f, 0.f, 0.f);
     const int lane = e[u] & 63, rq = (e[u] >> 6) & 3, j = (e[u] >> 8) & 3, ii = (e[u] >> 10) & 3, wv = e[u] >> 12;
-    const int row = (wv >> 1) * 128 + ii * 32 + 8 * rq + 4 * (lane >> 5), col = (wv & 1) * 128 + j * 32 + (lane & 31);
-    hp[u] = H + (int64_t)(m0 + row) * K + n0 + col;
-    h[u] = make_float4(hp[u][0], hp[u][K], hp[u][2 * (int64_t)K], hp[u][3 * (int64_t)K]);
+    if (PERM) {
+      // u-th of the thread's four rows, its four columns
+      const int row = (wv >> 1) * 128 + 32 * rq + 16 * (lane >> 5) + 4 * u + ii, col = (wv & 1) * 128 + 4 * (lane & 31);
+      hp[u] = H + (int64_t)(m0 + row) * K + n0 + col;
+      h[u] = *reinterpret_cast<const float4 *>(hp[u]);
+    } else {
+      const int row = (wv >> 1) * 128 + ii * 32 + 8 * rq + 4 * (lane >> 5), col = (wv & 1) * 128 + j * 32 + (lane & 31);
+      hp[u] = H + (int64_t)(m0 + row) * K + n0 + col;
+      h[u] = make_float4(hp[u][0], hp[u][K], hp[u][2 * (int64_t)K], hp[u][3 * (int64_t)K]);
+    }
   }
   for (; w < G && (int64_t)w * U / G < hi; ++w) {
     const int64_t a = (int64_t)w * U / G;
@@ -1346,6 +1362,14 @@ __global__ __launch_bounds__(256) void syrk_reduce_pieces_kernel(float *H, const
     for (int u = 0; u < 4; ++u) {
       s[u].x += v[u].x; s[u].y += v[u].y; s[u].z += v[u].z; s[u].w += v[u].w;
     }
+  }
+  if (PERM) {
+    // s[j] holds column j of rows 0 .. 3 (of the thread's four): transposed on the way out
+    *reinterpret_cast<float4 *>(hp[0]) = make_float4(h[0].x + s[0].x, h[0].y + s[1].x, h[0].z + s[2].x, h[0].w + s[3].x);
+    *reinterpret_cast<float4 *>(hp[1]) = make_float4(h[1].x + s[0].y, h[1].y + s[1].y, h[1].z + s[2].y, h[1].w + s[3].y);
+    *reinterpret_cast<float4 *>(hp[2]) = make_float4(h[2].x + s[0].z, h[2].y + s[1].z, h[2].z + s[2].z, h[2].w + s[3].z);
+    *reinterpret_cast<float4 *>(hp[3]) = make_float4(h[3].x + s[0].w, h[3].y + s[1].w, h[3].z + s[2].w, h[3].w + s[3].w);
+    return;
   }
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
@@ -1753,8 +1777,8 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
           hipLaunchKernelGGL((syrk16d_kernel<__hip_bfloat16, SyrkArgs, true>), dim3((unsigned)pp.G), block, D16_LDS_BYTES,
                              st, w);
         GPTQ_CHECK_LAUNCH();
-        hipLaunchKernelGGL(syrk_reduce_pieces_kernel, dim3((unsigned)(nt * (W16_TB * W16_TB / 4096))), dim3(256), 0, st, H,
-                           w.ws, (int)K, w.T, (int)s32, pp.G);
+        hipLaunchKernelGGL(syrk_reduce_pieces_kernel<false>, dim3((unsigned)(nt * (W16_TB * W16_TB / 4096))), dim3(256), 0,
+                           st, H, w.ws, (int)K, w.T, (int)s32, pp.G);
         GPTQ_CHECK_LAUNCH();
         continue;
       }
@@ -1804,7 +1828,8 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
       continue;
     }
     // fp32 batches, regular shapes from K = 1024 on: 256 x 256 tiles, loads straight into LDS
-    bool wide32 = x_dtype == GPTQ_HIP_F32 && use_wide16(K) && K % W16_TB == 0;
+    bool wide32 = x_dtype == GPTQ_HIP_F32 && use_wide16(K) && K % W16_TB == 0 &&
+                  ((reinterpret_cast<uintptr_t>(H) | reinterpret_cast<uintptr_t>(ws)) & 15) == 0;   // 16-byte accesses
     for (int i = 0; i < a.nb && wide32; ++i)
       wide32 = (a.rows[i] % D32_BK == 0) && ((reinterpret_cast<uintptr_t>(a.ptr[i]) & 15) == 0);
     if (wide32) {
@@ -1831,8 +1856,8 @@ int gptq_hip_hessian_accumulate(void *stream, const void *const *x_ptrs, const i
           w.chunk = (int)slabs;
           hipLaunchKernelGGL(syrk32d_kernel<true>, dim3((unsigned)pp.G), block, D32_LDS_BYTES, st, w);
           GPTQ_CHECK_LAUNCH();
-          hipLaunchKernelGGL(syrk_reduce_pieces_kernel, dim3((unsigned)(nt * (W16_TB * W16_TB / 4096))), dim3(256), 0, st, H,
-                             w.ws, (int)K, w.T, (int)slabs, pp.G);
+          hipLaunchKernelGGL(syrk_reduce_pieces_kernel<true>, dim3((unsigned)(nt * (W16_TB * W16_TB / 4096))), dim3(256), 0,
+                             st, H, w.ws, (int)K, w.T, (int)slabs, pp.G);
           GPTQ_CHECK_LAUNCH();
           continue;
         }
