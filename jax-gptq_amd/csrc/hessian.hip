@@ -1050,11 +1050,12 @@ __global__ __launch_bounds__(256) void syrk16d_kernel(ARGS p) {
 // buffers.  A row of a 256-feature panel is 1 KB, i.e. exactly one global_load_lds_dwordx4 of a
 // wavefront; LDS keeps the rows as they are in memory ([k][feature], 1 KB + 128 B apart so that
 // the two rows of an MFMA's k pair fall on different banks), which is the operand order of this
-// MFMA: lane l reads feature l % 32 of row 2 kp + l / 32 with one ds_read_b32.  Against the
-// 128 x 128-tile kernel at the top of this file: a quarter of the barriers and half of the LDS
-// operand reads per MFMA, no staging registers, no LDS writes.
+// MFMA: lane l reads row 2 kp + l / 32, and - the four MFMA blocks of an operand being the features
+// 4 i + q rather than 32 q + i - its features 4 (l % 32) .. + 3 with one ds_read_b128, the operands of
+// all four blocks.  Against the 128 x 128-tile kernel at the top of this file: a quarter of the
+// barriers and an eighth of the LDS operand reads per MFMA, no staging registers, no LDS writes.
 //
-// Per slab and wavefront: 8 k pairs x 16 MFMAs (64 cycles each), 8 loads, 64 operand reads; the
+// Per slab and wavefront: 8 k pairs x 16 MFMAs (64 cycles each), 8 loads, 16 operand reads; the
 // order is fixed by hand as in syrk16d_kernel: before the MFMAs of k pair kp one load of a later
 // slab and the operand reads of k pair kp + 1 are issued.  The loop is skewed by one k pair: a
 // step starts with the last k pair of the previous slab out of registers, so that the first
